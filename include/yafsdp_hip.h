@@ -1,0 +1,142 @@
+/* C ABI of libyafsdp_hip.so: MI355X (gfx950) kernels for the per-rank buffer
+ * path of YaFSDP-style sharded data parallelism.
+ *
+ * The reference (yandex/YaFSDP) has no FFI layer: this path is a handful of
+ * torch ops inside ya_fsdp/_collectives.py and ya_fsdp/_param_group.py.  Each
+ * entry point below names the reference call sites it replaces.
+ *
+ * Conventions
+ *  - All pointers except the `*_ptrs`, `*_numels`, `*_mode` arrays and out
+ *    parameters are DEVICE pointers owned by the caller.  Nothing here
+ *    allocates or frees caller memory; the only library-owned objects are
+ *    metadata tables (yafsdp_table_create / yafsdp_table_destroy).
+ *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All
+ *    work is enqueued on it; no entry point synchronises the device, except
+ *    yafsdp_table_create / yafsdp_table_destroy (one-time set-up / tear-down).
+ *  - dtype arguments take the yafsdp_dtype values.
+ *  - Return value: 0 on success, a positive hipError_t value if a HIP call
+ *    failed, a negative yafsdp_status otherwise.  yafsdp_error_string() turns
+ *    either into text.
+ *  - Divide factors follow ya_fsdp/_collectives.py:270-272: a factor is applied
+ *    only if it is > 1 (pass 0 for "None").  The factor is rounded to binary32
+ *    and the division is a correctly rounded binary32 division (what torch does
+ *    on the host CPU); results are rounded to nearest even into the dtype of the
+ *    tensor the reference would have materialised at that step.
+ *  - Entry points are re-entrant.  Calls that use the same table from several
+ *    host threads are serialised internally.
+ */
+#ifndef YAFSDP_HIP_H_
+#define YAFSDP_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum yafsdp_dtype { YAFSDP_F32 = 0, YAFSDP_BF16 = 1, YAFSDP_F16 = 2 } yafsdp_dtype;
+
+typedef enum yafsdp_status {
+  YAFSDP_OK = 0,
+  YAFSDP_ERR_INVALID_ARGUMENT = -1,
+  YAFSDP_ERR_UNSUPPORTED_DTYPE = -2,
+  YAFSDP_ERR_MISALIGNED = -3,
+  YAFSDP_ERR_WRONG_DEVICE = -4,
+  YAFSDP_ERR_OUT_OF_MEMORY = -5
+} yafsdp_status;
+
+/* per-tensor mode of yafsdp_gather_in / yafsdp_scatter_out / fragments */
+typedef enum yafsdp_mode { YAFSDP_MODE_SKIP = 0, YAFSDP_MODE_COPY = 1, YAFSDP_MODE_ADD = 2 } yafsdp_mode;
+
+typedef struct yafsdp_table yafsdp_table;
+
+/* ABI version of this header (major * 1000 + minor). */
+int yafsdp_version(void);
+
+/* Text for a return code of any entry point. The pointer stays valid. */
+const char* yafsdp_error_string(int code);
+
+/* dst[i] = cast(src[i]), i < n: `Tensor.copy_` between flat buffers.
+ * Replaces: copy-in  all_gather_input.copy_(padded_sharded_param_data)
+ *           (ya_fsdp/_collectives.py:53-54); the size-1-group all-gather
+ *           all_gather_output.copy_(all_gather_input) (:56-58); the size-1-group
+ *           reduce-scatter output_tensor.copy_(rs_input) (:140-150); and
+ *           padded_sharded_param_grad.copy_(output_tensor) (:185).
+ * Same dtype: a byte copy.  dst and src must not partially overlap. */
+int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, void* stream);
+
+/* buf[i] = round(buf[i] / factor) in place, only if factor > 1.
+ * Replaces: _div_if_needed / tensor.div_ (ya_fsdp/_collectives.py:139, 165,
+ * 270-272). */
+int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream);
+
+/* Fused post-reduce on the rank's chunk of the reduce buffer:
+ *   t = chunk[i];  if (post_factor > 1) t = round_chunk_dtype(t / post_factor);
+ *   shard[i] = round_shard_dtype(accumulate ? shard[i] + t : t)
+ * Replaces: _div_if_needed(output_tensor, postdivide_factor)
+ * (ya_fsdp/_collectives.py:165) followed by padded_sharded_param_grad.copy_ (:185)
+ * or .add_ (:189).  The chunk is not written (it is scratch after this point
+ * in the reference). */
+int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
+                       double post_factor, int accumulate, void* stream);
+
+/* Same as yafsdp_post_reduce but per ragged fragment: fragment f covers
+ * elements [sum(numels[:f]), sum(numels[:f+1])) of both shard and chunk and is
+ * copied (YAFSDP_MODE_COPY), accumulated (YAFSDP_MODE_ADD) or left untouched
+ * (YAFSDP_MODE_SKIP).  `frag_numels` and `frag_mode` are host arrays.
+ * Replaces: the _foreach_copy_ / _foreach_add_ pair over per-parameter
+ * fragments (ya_fsdp/_collectives.py:191-214). */
+int yafsdp_post_reduce_fragments(void* shard, int shard_dtype, const void* chunk, int chunk_dtype,
+                                 int n_fragments, const int64_t* frag_numels, const uint8_t* frag_mode,
+                                 double post_factor, void* stream);
+
+/* Build the device-resident metadata table of one flat buffer: `n_tensors`
+ * tensors laid out back to back, tensor p at elements
+ * [sum(numels[:p]), sum(numels[:p+1])), followed by pad lanes up to
+ * `padded_numel`.  `numels` is a host array.  The table is bound to the current
+ * HIP device and is static for the life of a parameter group (the layout of
+ * ya_fsdp/_param_group.py:245-265, 441-457 never changes after construction). */
+int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_numel, yafsdp_table** out);
+int yafsdp_table_destroy(yafsdp_table* table);
+/* Number of tensors / total elements (without pad) / padded elements. */
+int yafsdp_table_info(const yafsdp_table* table, int* n_tensors, int64_t* total_numel, int64_t* padded_numel);
+
+/* Reduce copy-in: gather the tensors of a table into the flat reduce buffer.
+ * Per tensor p, with `mode` a host array of n_tensors yafsdp_mode bytes (NULL =
+ * all COPY) and `tensor_ptrs` a host array of n_tensors device pointers
+ * (ignored for SKIP tensors and empty tensors):
+ *   COPY  view_p = cast(tensor_p)                 torch._foreach_copy_
+ *         (ya_fsdp/_param_group.py:693-700)
+ *   ADD   view_p = round(view_p + tensor_p)       torch._foreach_add_
+ *         (ya_fsdp/_param_group.py:701-708)
+ *   SKIP  view_p untouched
+ * then, if pre_factor > 1, every element of the padded buffer (SKIP tensors
+ * and pad lanes included) is divided in the same pass:
+ *   flat = round(flat / pre_factor)               _div_if_needed(rs_input, pre)
+ *         (ya_fsdp/_collectives.py:139)
+ * zero_pad != 0 writes 0 to the pad lanes [total, padded) (the reference leaves
+ * them uninitialised).  `flat` must be 16-byte aligned. */
+int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode, int tensor_dtype,
+                     void* flat, int flat_dtype, double pre_factor, int zero_pad, void* stream);
+
+/* Materialising copy-out: tensor_p = cast(flat[offset_p : offset_p + numel_p])
+ * for every tensor whose mode is not SKIP (`mode` NULL = all).  The reference's
+ * own copy-out is zero-copy views (ya_fsdp/_param_group.py:441-457,
+ * ya_fsdp/_param.py:209); this is the `split` + `copy_` form of the same split,
+ * for consumers that need separately allocated parameters.  `flat` must be
+ * 16-byte aligned; pad lanes are never read. */
+int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
+                       const uint8_t* mode, int tensor_dtype, void* stream);
+
+/* Launch-shape knobs (process-wide, for measurement): */
+typedef enum yafsdp_option {
+  YAFSDP_OPT_FLAT_BLOCKS_PER_CU = 0,  /* workgroups per compute unit of the flat kernels' grid */
+  YAFSDP_OPT_TABLE_BLOCKS_PER_CU = 1  /* same for gather-in / scatter-out */
+} yafsdp_option;
+int yafsdp_set_option(int option, int value);
+int yafsdp_get_option(int option, int* value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* YAFSDP_HIP_H_ */

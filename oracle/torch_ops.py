@@ -1,0 +1,150 @@
+"""The reference's torch-op sequence for the per-rank buffer path, on CPU tensors.
+
+TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).  Every function performs
+the same ops, in the same order and with the same in-place-ness, as the cited
+reference lines, so every intermediate rounding is reproduced.  The one
+departure, documented where it occurs: flat buffers start zero-filled so that
+pad lanes (uninitialised ``torch.empty`` memory in the reference,
+ya_fsdp/_param_group.py:53-59, 269-271, 281-283) have a defined value.
+"""
+
+from __future__ import annotations
+
+from typing import Sequence
+
+import torch
+
+
+# --------------------------------------------------------------------------- #
+# unshard side                                                                #
+# --------------------------------------------------------------------------- #
+def copy_in(all_gather_input: torch.Tensor, padded_sharded_param_data: torch.Tensor) -> None:
+    """Copy-in: cast the master shard into the all-gather input
+    (ya_fsdp/_collectives.py:53-54)."""
+    all_gather_input.copy_(padded_sharded_param_data)
+
+
+def all_gather_single_rank(all_gather_output: torch.Tensor, all_gather_input: torch.Tensor) -> None:
+    """The "all-gather" of a size-1 group (ya_fsdp/_collectives.py:56-58)."""
+    all_gather_output.copy_(all_gather_input)
+
+
+def unsharded_views(
+    all_gather_output: torch.Tensor, numels: Sequence[int], sizes: Sequence[Sequence[int]]
+) -> list[torch.Tensor]:
+    """Zero-copy copy-out: unsharded parameters are views into the gathered
+    buffer (ya_fsdp/_param_group.py:441-457, ya_fsdp/_param.py:209)."""
+    numels = list(numels)
+    return [
+        v.view(tuple(sz))
+        for v, sz in zip(all_gather_output[: sum(numels)].split(numels), sizes)
+    ]
+
+
+def copy_out_materialize(
+    all_gather_output: torch.Tensor, numels: Sequence[int], outs: Sequence[torch.Tensor]
+) -> None:
+    """Materialising copy-out: the same split as ``unsharded_views`` followed by
+    a ``copy_`` into separately allocated tensors."""
+    numels = list(numels)
+    for v, o in zip(all_gather_output[: sum(numels)].split(numels), outs):
+        o.view(-1).copy_(v)
+
+
+# --------------------------------------------------------------------------- #
+# reduce side                                                                 #
+# --------------------------------------------------------------------------- #
+def reduce_copy_in(
+    rs_views: Sequence[torch.Tensor], grads: Sequence[torch.Tensor], accumulate: bool
+) -> None:
+    """Flatten unsharded gradients into views of the reduce buffer: first
+    micro-batch ``_foreach_copy_`` (ya_fsdp/_param_group.py:693-700), later ones
+    ``_foreach_add_`` (ya_fsdp/_param_group.py:701-708)."""
+    if len(rs_views) == 0:
+        return
+    if accumulate:
+        torch._foreach_add_(list(rs_views), list(grads))
+    else:
+        torch._foreach_copy_(list(rs_views), list(grads))
+
+
+def div_if_needed(tensor: torch.Tensor, div_factor: float | None) -> None:
+    """ya_fsdp/_collectives.py:270-272 (note ``> 1``, not ``!= 1``)."""
+    if div_factor is not None and div_factor > 1:
+        tensor.div_(div_factor)
+
+
+def get_gradient_divide_factors(
+    world_size: int,
+    reduce_dtype: torch.dtype,
+    factor: float | None,
+    force_sum_reduction_for_comms: bool,
+    has_yccl_handle: bool = False,
+) -> tuple[float | None, float | None, str, float | None]:
+    """ya_fsdp/_collectives.py:221-267 with the process group reduced to its
+    size.  Returns ``(pre, post, op, premul)`` where ``op`` is one of "SUM",
+    "AVG", "PREMUL_SUM" and ``premul`` is the pre-multiplier of "PREMUL_SUM"."""
+    if has_yccl_handle:
+        force_sum_reduction_for_comms = True
+    overflow_risk = reduce_dtype not in (torch.float32, torch.bfloat16)
+    if not overflow_risk and not force_sum_reduction_for_comms:
+        if factor is None:
+            if world_size == 1:
+                return None, None, "SUM", None
+            return None, None, "AVG", None
+        if factor == world_size:
+            return None, None, "AVG", None
+        return None, None, "PREMUL_SUM", 1 / factor
+    if factor is None:
+        factor = float(world_size)
+    if overflow_risk:
+        pre_factor: float | None = 1
+        while factor % pre_factor == 0 and factor / pre_factor > pre_factor:
+            pre_factor *= 2
+        post_factor = factor / pre_factor
+    else:
+        pre_factor, post_factor = None, factor
+    return pre_factor, post_factor, "SUM", None
+
+
+def reduce_scatter_local(
+    padded_sharded_param_grad: torch.Tensor,
+    padded_unsharded_param_grad: torch.Tensor,
+    world_size: int,
+    rank: int,
+    predivide_factor: float | None,
+    postdivide_factor: float | None,
+    mode: str,
+    sharded_numels: Sequence[int] | None = None,
+    fragment_has_sharded_grad: Sequence[bool | None] | None = None,
+) -> torch.Tensor:
+    """ya_fsdp/_collectives.py:124-214 for the branch that goes through the
+    reduce buffer (``reduce_in_sharded`` false), with the inter-GPU collective
+    (ya_fsdp/_collectives.py:152-164) replaced by its one-rank share: the rank's
+    chunk of the reduce buffer *is* the reduce-scatter result.
+
+    ``mode``: "copy" (:185), "add" (:189) or "mixed" (:191-214).  For "mixed",
+    ``fragment_has_sharded_grad[p]`` is True (accumulate), False (copy) or None
+    (parameter produced no gradient: fragment untouched)."""
+    div_if_needed(padded_unsharded_param_grad, predivide_factor)  # :139
+    output_tensor = padded_unsharded_param_grad.chunk(world_size)[rank]  # :127-129
+    div_if_needed(output_tensor, postdivide_factor)  # :165
+    if mode == "copy":
+        padded_sharded_param_grad.copy_(output_tensor)  # :185
+    elif mode == "add":
+        padded_sharded_param_grad.add_(output_tensor)  # :189
+    elif mode == "mixed":
+        assert sharded_numels is not None and fragment_has_sharded_grad is not None
+        sharded_numels = list(sharded_numels)
+        n = sum(sharded_numels)
+        grad_frags = padded_sharded_param_grad[:n].split(sharded_numels)
+        out_frags = output_tensor[:n].split(sharded_numels)
+        copy_idx = [i for i, f in enumerate(fragment_has_sharded_grad) if f is False]
+        add_idx = [i for i, f in enumerate(fragment_has_sharded_grad) if f is True]
+        if copy_idx:
+            torch._foreach_copy_([grad_frags[i] for i in copy_idx], [out_frags[i] for i in copy_idx])
+        if add_idx:
+            torch._foreach_add_([grad_frags[i] for i in add_idx], [out_frags[i] for i in add_idx])
+    else:
+        raise ValueError(mode)
+    return output_tensor

@@ -1,0 +1,58 @@
+"""The C-ABI library loads without a GPU and exports every symbol that
+include/yafsdp_hip.h declares (no compute calls here)."""
+
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "yafsdp_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(yafsdp_[a-z_]+)\s*\(", text)))
+
+
+def test_header_and_binding_agree():
+    from yafsdp_amd import _native
+
+    declared = _declared_functions()
+    assert declared, "no declarations parsed"
+    assert sorted(_native.EXPORTED_SYMBOLS) == declared
+
+
+def test_library_exports_every_symbol():
+    from yafsdp_amd import _native
+
+    for name in _declared_functions():
+        assert hasattr(_native.lib, name), name
+    assert _native.lib.yafsdp_version() == 1000
+    assert _native.error_string(0) == "success"
+    assert "dtype" in _native.error_string(-2)
+
+
+def test_argument_validation_without_gpu():
+    """Entry points reject bad arguments before touching the device."""
+    from yafsdp_amd import _native
+
+    L = _native.lib
+    assert L.yafsdp_flat_copy(None, 9, None, 0, 4, None) == -2
+    assert L.yafsdp_flat_copy(None, 0, None, 0, -1, None) == -1
+    assert L.yafsdp_flat_copy(None, 0, None, 0, 4, None) == -1
+    assert L.yafsdp_flat_copy(None, 0, None, 0, 0, None) == 0
+    assert L.yafsdp_flat_div(None, 0, 0, 8.0, None) == 0
+    assert L.yafsdp_post_reduce(None, 0, None, 5, 0, 0.0, 0, None) == -2
+    assert L.yafsdp_set_option(99, 1) == -1
+    assert L.yafsdp_set_option(0, 0) == -1
+    assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
+    assert L.yafsdp_table_destroy(None) == 0
+
+
+def test_no_product_module_imports_the_oracle():
+    pkg = os.path.join(ROOT, "yafsdp_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cuh", ".h")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
+                assert "libbufpath_ref" not in src, f

@@ -1,0 +1,255 @@
+"""GPU parity: every C-ABI entry point against the oracle (the reference's
+torch-op sequence on CPU) on the same seeded inputs, bit for bit.
+
+Floating-point tolerance: none.  Integer views of the outputs must be equal;
+the single exception is that any NaN matches any NaN (payloads are not defined
+by the reference).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import torch_ops
+from tests.helpers import DTYPES, assert_bits_equal, mixed_values, special_values_f32
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def nat():
+    from yafsdp_amd import _native
+
+    return _native
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+# --------------------------------------------------------------------- casts --
+def test_cast_exhaustive_high_halfword(nat):
+    """Every high half-word of binary32 with low half-words straddling the tie,
+    through the copy-in kernel, against the integer closed form."""
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0, 1, 0x7FFF, 0x8000, 0x8001, 0xFFFF, 0x1234, 0xC000], dtype=np.uint32)
+    bits = (hi[:, None] | lows[None, :]).reshape(-1)
+    x = torch.from_numpy(bits.view(np.float32).copy())
+    for dt in (torch.bfloat16, torch.float16):
+        _say("cast f32 ->", dt)
+        want = torch.empty(x.numel(), dtype=dt)
+        torch_ops.copy_in(want, x)
+        got = torch.empty(x.numel(), dtype=dt, device=DEV)
+        nat.flat_copy(got, x.to(DEV))
+        assert_bits_equal(got, want, f"f32->{dt}")
+    allh = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16)
+    for dt in (torch.bfloat16, torch.float16):
+        src = allh.view(dt)
+        want = torch.empty(65536, dtype=torch.float32)
+        torch_ops.copy_in(want, src)
+        got = torch.empty(65536, dtype=torch.float32, device=DEV)
+        nat.flat_copy(got, src.to(DEV))
+        assert_bits_equal(got, want, f"{dt}->f32")
+
+
+@pytest.mark.parametrize("src_dt", DTYPES)
+@pytest.mark.parametrize("dst_dt", DTYPES)
+def test_flat_copy_sizes_and_alignments(nat, src_dt, dst_dt):
+    g = torch.Generator().manual_seed(100)
+    for n in [0, 1, 7, 8, 9, 63, 1000, 8192, 8192 * 3 + 5, 262_147]:
+        for s_off, d_off in [(0, 0), (1, 0), (0, 3), (5, 7), (8, 4)]:
+            _say("flat_copy", src_dt, dst_dt, n, s_off, d_off)
+            src = mixed_values(g, n + s_off, src_dt)
+            want = torch.full((n + d_off + 8,), 3.0, dtype=dst_dt)
+            torch_ops.copy_in(want[d_off : d_off + n], src[s_off:])
+            got = torch.full((n + d_off + 8,), 3.0, dtype=dst_dt, device=DEV)
+            nat.flat_copy(got[d_off : d_off + n], src.to(DEV)[s_off:])
+            assert_bits_equal(got, want, f"flat_copy n={n} offs=({s_off},{d_off})")
+
+
+def test_flat_copy_same_dtype_is_byte_copy(nat):
+    # NaN payloads and every bit pattern pass through a same-dtype copy
+    allh = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16)
+    for dt in (torch.bfloat16, torch.float16):
+        src = allh.view(dt).to(DEV)
+        dst = torch.zeros_like(src)
+        nat.flat_copy(dst, src)
+        assert torch.equal(dst.view(torch.int16).cpu(), allh)
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("factor", [None, 1.0, 0.5, 2.0, 8.0, 64.0, 256.0, 3.0, 7.0, 1.5, 1000.0, 2.0**100])
+def test_flat_div(nat, dt, factor):
+    g = torch.Generator().manual_seed(101)
+    for n, off in [(4099, 0), (20_000, 3)]:
+        _say("flat_div", dt, factor, n, off)
+        x = mixed_values(g, n + off, dt, std=1e-3)
+        want = x.clone()
+        torch_ops.div_if_needed(want[off:], factor)
+        got = x.to(DEV)
+        nat.flat_div(got[off:], factor)
+        assert_bits_equal(got, want, f"div {dt} {factor}")
+
+
+@pytest.mark.parametrize("shard_dt", DTYPES)
+@pytest.mark.parametrize("chunk_dt", DTYPES)
+@pytest.mark.parametrize("post", [None, 8.0, 3.0])
+@pytest.mark.parametrize("acc", [False, True])
+def test_post_reduce(nat, shard_dt, chunk_dt, post, acc):
+    g = torch.Generator().manual_seed(102)
+    for n, off in [(5, 0), (8192 * 2 + 11, 0), (30_001, 1)]:
+        _say("post_reduce", shard_dt, chunk_dt, post, acc, n, off)
+        chunk = mixed_values(g, n + off, chunk_dt, std=1e-3)
+        shard0 = mixed_values(g, n + off, shard_dt, std=1e-4).flip(0).contiguous()
+        want = shard0.clone()
+        torch_ops.reduce_scatter_local(want[off:], chunk.clone()[off:], 1, 0, None, post, "add" if acc else "copy")
+        got = shard0.to(DEV)
+        nat.post_reduce(got[off:], chunk.to(DEV)[off:], post, acc)
+        assert_bits_equal(got, want, "post_reduce")
+
+
+@pytest.mark.parametrize("shard_dt,chunk_dt", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("post", [None, 8.0])
+def test_post_reduce_fragments(nat, shard_dt, chunk_dt, post):
+    g = torch.Generator().manual_seed(103)
+    numels = [0, 7, 12_001, 0, 33, 1, 9000, 5]
+    has = [None, True, False, False, None, True, True, None]
+    s = sum(numels) + 16
+    chunk = mixed_values(g, s, chunk_dt, 1e-3)
+    shard0 = mixed_values(g, s, shard_dt, 1e-4).flip(0).contiguous()
+    want = shard0.clone()
+    torch_ops.reduce_scatter_local(want, chunk.clone(), 1, 0, None, post, "mixed", numels, has)
+    got = shard0.to(DEV)
+    modes = [0 if h is None else (2 if h else 1) for h in has]
+    nat.post_reduce_fragments(got, chunk.to(DEV), numels, modes, post)
+    assert_bits_equal(got, want, "post_reduce_fragments")
+
+
+# ------------------------------------------------------------- table kernels --
+def _random_numels(rng: np.random.Generator, p: int, max_log2: float, with_empty: bool):
+    n = np.floor(np.exp2(rng.uniform(0, max_log2, size=p))).astype(np.int64) | 1
+    if with_empty and p > 3:
+        n[rng.integers(0, p, size=max(1, p // 10))] = 0
+    return n.tolist()
+
+
+TABLE_CASES = [
+    # (P, max log2 numel, with_empty, pad)
+    (1, 3, False, 0),
+    (3, 4, False, 5),
+    (9, 16, True, 17),
+    (32, 14, True, 0),
+    (33, 14, True, 9),
+    (200, 12, True, 4096),
+    (40, 19, False, 513),
+]
+
+
+@pytest.mark.parametrize("case", TABLE_CASES)
+@pytest.mark.parametrize("grad_dt,rs_dt", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                           (torch.float32, torch.bfloat16), (torch.float16, torch.float16),
+                                           (torch.float32, torch.float32)])
+@pytest.mark.parametrize("pre", [None, 8.0, 3.0])
+def test_gather_in(nat, case, grad_dt, rs_dt, pre):
+    p, max_log2, with_empty, pad = case
+    rng = np.random.default_rng(p * 1000 + pad)
+    g = torch.Generator().manual_seed(104 + p)
+    numels = _random_numels(rng, p, max_log2, with_empty)
+    t = sum(numels)
+    t_pad = t + pad
+    _say("gather_in", case, grad_dt, rs_dt, pre, "T", t)
+    grads = [mixed_values(g, n, grad_dt, 1e-3) for n in numels]
+    modes = rng.integers(0, 3, size=p).tolist() if p > 1 else [1]
+    old = torch.zeros(t_pad + 8, dtype=rs_dt)
+    old[:t] = mixed_values(g, t, rs_dt, 1e-3).flip(0)
+    old[t_pad:] = 5.0  # guard lanes beyond the padded buffer stay untouched
+    # oracle: foreach copy, foreach add, then div over the padded buffer
+    want = old.clone()
+    views = list(want[:t].split(numels))
+    cp = [i for i, m in enumerate(modes) if m == 1]
+    ad = [i for i, m in enumerate(modes) if m == 2]
+    torch_ops.reduce_copy_in([views[i] for i in cp], [grads[i] for i in cp], False)
+    torch_ops.reduce_copy_in([views[i] for i in ad], [grads[i] for i in ad], True)
+    torch_ops.div_if_needed(want[:t_pad], pre)
+    table = nat.TensorTable(numels, t_pad, torch.device(DEV))
+    got = old.to(DEV)
+    dgrads = [x.to(DEV) for x in grads]
+    table.gather_in(dgrads, got, modes, pre, zero_pad=True)
+    assert_bits_equal(got, want, "gather_in")
+    # all-copy call with default modes
+    want2 = old.clone()
+    torch_ops.reduce_copy_in(list(want2[:t].split(numels)), grads, False)
+    got2 = old.to(DEV)
+    table.gather_in(dgrads, got2)
+    assert_bits_equal(got2, want2, "gather_in all copy")
+    table.close()
+
+
+def test_gather_in_pad_not_zeroed_sees_divide(nat):
+    numels = [100, 29]
+    t, t_pad = 129, 160
+    g = torch.Generator().manual_seed(105)
+    old = mixed_values(g, t_pad, torch.bfloat16, 1e-2)
+    grads = [mixed_values(g, n, torch.bfloat16, 1e-3) for n in numels]
+    want = old.clone()
+    torch_ops.reduce_copy_in(list(want[:t].split(numels)), grads, False)
+    torch_ops.div_if_needed(want, 4.0)
+    table = nat.TensorTable(numels, t_pad, torch.device(DEV))
+    got = old.to(DEV)
+    table.gather_in([x.to(DEV) for x in grads], got, None, 4.0, zero_pad=False)
+    assert_bits_equal(got, want, "pad lanes divided like the reference's")
+
+
+@pytest.mark.parametrize("case", TABLE_CASES)
+@pytest.mark.parametrize("flat_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
+                                            (torch.bfloat16, torch.float32), (torch.float32, torch.float16)])
+def test_scatter_out(nat, case, flat_dt, out_dt):
+    p, max_log2, with_empty, pad = case
+    rng = np.random.default_rng(p * 1000 + pad + 1)
+    g = torch.Generator().manual_seed(106 + p)
+    numels = _random_numels(rng, p, max_log2, with_empty)
+    t = sum(numels)
+    _say("scatter_out", case, flat_dt, out_dt, "T", t)
+    flat = mixed_values(g, t + pad, flat_dt)
+    want = [torch.full((n + 2,), 3.0, dtype=out_dt) for n in numels]
+    torch_ops.copy_out_materialize(flat, numels, [w[1 : 1 + n] for w, n in zip(want, numels)])
+    got = [torch.full((n + 2,), 3.0, dtype=out_dt, device=DEV) for n in numels]
+    table = nat.TensorTable(numels, t + pad, torch.device(DEV))
+    table.scatter_out(flat.to(DEV), [x[1 : 1 + n] for x, n in zip(got, numels)])
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert_bits_equal(a, b, f"scatter_out tensor {i}")
+    # skip modes: untouched outputs
+    if p > 1:
+        modes = rng.integers(0, 2, size=p).tolist()
+        got2 = [torch.full((n,), 3.0, dtype=out_dt, device=DEV) for n in numels]
+        table.scatter_out(flat.to(DEV), got2, modes)
+        pos = 0
+        for i, n in enumerate(numels):
+            ref = torch.full((n,), 3.0, dtype=out_dt)
+            if modes[i]:
+                ref.copy_(flat[pos : pos + n])
+            assert_bits_equal(got2[i], ref, f"scatter_out modes tensor {i}")
+            pos += n
+    table.close()
+
+
+def test_errors_are_loud(nat):
+    a = torch.zeros(16, dtype=torch.float32, device=DEV)
+    with pytest.raises(RuntimeError):
+        nat.flat_copy(a, torch.zeros(16))  # CPU tensor: no CPU path
+    with pytest.raises(TypeError):
+        nat.flat_copy(a, torch.zeros(16, dtype=torch.float64, device=DEV))
+    with pytest.raises(ValueError):
+        nat.flat_copy(a, torch.zeros(8, device=DEV))
+    with pytest.raises(NotImplementedError):
+        nat.flat_copy(a.view(4, 4).t(), a.view(4, 4))
+    table = nat.TensorTable([8, 8], 16, torch.device(DEV))
+    with pytest.raises(ValueError):
+        table.gather_in([a[:8]], a.bfloat16())
+    with pytest.raises(RuntimeError, match="aligned"):
+        buf = torch.zeros(32, dtype=torch.bfloat16, device=DEV)
+        table.gather_in([a[:8], a[8:]], buf[1:17])
+    assert "invalid argument" in nat.error_string(-1)
+    assert nat.lib.yafsdp_flat_copy(a.data_ptr(), 7, a.data_ptr(), 0, 4, None) == -2

@@ -1,0 +1,66 @@
+"""Build ``libyafsdp_hip.so`` (gfx950 kernels + C ABI) in-tree with hipcc.
+
+Usage: ``python -m yafsdp_amd._build``.  The library is built next to this file
+so that it travels with the source tree; nothing is installed elsewhere.
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT = os.path.join(HERE, "libyafsdp_hip.so")
+SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip"]
+HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "launch.h", "tuning.h"]
+ARCH = "gfx950"
+
+# -ffp-contract=off: every multiply and add of the path rounds on its own, as
+# the separate torch ops of the reference do.  packed-fp32 ops are disabled
+# for all device code of this library.
+HIPCC_FLAGS = [
+    "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.sep not in cand or os.path.exists(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def _compile(src: str, obj: str) -> None:
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+    if err.strip():
+        print(err)
+
+
+def build(force: bool = True, jobs: int = 4) -> str:
+    """Compile every translation unit and link the shared library."""
+    srcs = [os.path.join(CSRC, s) for s in SOURCES + HEADERS] + [os.path.join(HERE, "..", "include", "yafsdp_hip.h")]
+    if not force and os.path.exists(OUT) and all(os.path.getmtime(OUT) >= os.path.getmtime(s) for s in srcs):
+        return OUT
+    build_dir = os.path.join(HERE, "build")
+    os.makedirs(build_dir, exist_ok=True)
+    objs = [os.path.join(build_dir, s.replace(".hip", ".o")) for s in SOURCES]
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        list(ex.map(_compile, SOURCES, objs))
+    cmd = [_hipcc(), "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", OUT, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr}")
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build())

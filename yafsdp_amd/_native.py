@@ -1,0 +1,281 @@
+"""ctypes binding of ``libyafsdp_hip.so`` (the C ABI in ``include/yafsdp_hip.h``).
+
+There is no CPU or torch fallback: if the library is missing, importing this
+module raises, and every call that fails raises ``RuntimeError`` with the
+library's error text.  Tensors enter as raw device pointers and the stream as
+the ``hipStream_t`` handle of torch's current stream, so work is enqueued
+exactly where the reference's torch ops would have been
+(ya_fsdp/_collectives.py:46, 110-111).
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Sequence
+
+import numpy as np
+import torch  # imported before the library so that both share one HIP runtime
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libyafsdp_hip.so")
+
+DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+MODE_SKIP, MODE_COPY, MODE_ADD = 0, 1, 2
+OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU = 0, 1
+
+# every symbol include/yafsdp_hip.h declares
+EXPORTED_SYMBOLS = (
+    "yafsdp_version",
+    "yafsdp_error_string",
+    "yafsdp_flat_copy",
+    "yafsdp_flat_div",
+    "yafsdp_post_reduce",
+    "yafsdp_post_reduce_fragments",
+    "yafsdp_table_create",
+    "yafsdp_table_destroy",
+    "yafsdp_table_info",
+    "yafsdp_gather_in",
+    "yafsdp_scatter_out",
+    "yafsdp_set_option",
+    "yafsdp_get_option",
+)
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m yafsdp_amd._build` "
+            "(hipcc, gfx950). There is no fallback path."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, i64, dbl, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_double, ctypes.c_int
+    lib.yafsdp_version.restype = i32
+    lib.yafsdp_version.argtypes = []
+    lib.yafsdp_error_string.restype = ctypes.c_char_p
+    lib.yafsdp_error_string.argtypes = [i32]
+    lib.yafsdp_flat_copy.restype = i32
+    lib.yafsdp_flat_copy.argtypes = [vp, i32, vp, i32, i64, vp]
+    lib.yafsdp_flat_div.restype = i32
+    lib.yafsdp_flat_div.argtypes = [vp, i32, i64, dbl, vp]
+    lib.yafsdp_post_reduce.restype = i32
+    lib.yafsdp_post_reduce.argtypes = [vp, i32, vp, i32, i64, dbl, i32, vp]
+    lib.yafsdp_post_reduce_fragments.restype = i32
+    lib.yafsdp_post_reduce_fragments.argtypes = [vp, i32, vp, i32, i32, vp, vp, dbl, vp]
+    lib.yafsdp_table_create.restype = i32
+    lib.yafsdp_table_create.argtypes = [i32, vp, i64, ctypes.POINTER(vp)]
+    lib.yafsdp_table_destroy.restype = i32
+    lib.yafsdp_table_destroy.argtypes = [vp]
+    lib.yafsdp_table_info.restype = i32
+    lib.yafsdp_table_info.argtypes = [vp, ctypes.POINTER(i32), ctypes.POINTER(i64), ctypes.POINTER(i64)]
+    lib.yafsdp_gather_in.restype = i32
+    lib.yafsdp_gather_in.argtypes = [vp, vp, vp, i32, vp, i32, dbl, i32, vp]
+    lib.yafsdp_scatter_out.restype = i32
+    lib.yafsdp_scatter_out.argtypes = [vp, vp, i32, vp, vp, i32, vp]
+    lib.yafsdp_set_option.restype = i32
+    lib.yafsdp_set_option.argtypes = [i32, i32]
+    lib.yafsdp_get_option.restype = i32
+    lib.yafsdp_get_option.argtypes = [i32, ctypes.POINTER(i32)]
+    return lib
+
+
+lib = _load()
+
+
+def error_string(code: int) -> str:
+    return lib.yafsdp_error_string(int(code)).decode()
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        raise RuntimeError(f"{what} failed: {error_string(code)} (code {code})")
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}: the buffer path handles float32, bfloat16, float16") from None
+
+
+def _flat_arg(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.device.type != "cuda":
+        raise RuntimeError(f"{what} must live on the GPU, got {t.device}: this path has no CPU implementation")
+    if not t.is_contiguous():
+        raise NotImplementedError(f"{what} must be contiguous: shape={tuple(t.shape)} stride={t.stride()}")
+    return t
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _factor(f: float | None) -> float:
+    return 0.0 if f is None else float(f)
+
+
+# ------------------------------------------------------------------ flat ops --
+def flat_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """``dst.copy_(src)`` for contiguous tensors of equal numel."""
+    _flat_arg(dst, "dst"), _flat_arg(src, "src")
+    if dst.numel() != src.numel():
+        raise ValueError(f"numel mismatch: {dst.numel()} vs {src.numel()}")
+    with torch.cuda.device(dst.device):
+        _check(
+            lib.yafsdp_flat_copy(dst.data_ptr(), _dt(dst), src.data_ptr(), _dt(src), dst.numel(), _stream(dst)),
+            "yafsdp_flat_copy",
+        )
+
+
+def flat_div(buf: torch.Tensor, factor: float | None) -> None:
+    """``_div_if_needed(buf, factor)``."""
+    _flat_arg(buf, "buf")
+    with torch.cuda.device(buf.device):
+        _check(
+            lib.yafsdp_flat_div(buf.data_ptr(), _dt(buf), buf.numel(), _factor(factor), _stream(buf)),
+            "yafsdp_flat_div",
+        )
+
+
+def post_reduce(shard: torch.Tensor, chunk: torch.Tensor, post_factor: float | None, accumulate: bool) -> None:
+    _flat_arg(shard, "shard"), _flat_arg(chunk, "chunk")
+    if shard.numel() != chunk.numel():
+        raise ValueError(f"numel mismatch: {shard.numel()} vs {chunk.numel()}")
+    with torch.cuda.device(shard.device):
+        _check(
+            lib.yafsdp_post_reduce(
+                shard.data_ptr(), _dt(shard), chunk.data_ptr(), _dt(chunk), shard.numel(),
+                _factor(post_factor), int(bool(accumulate)), _stream(shard),
+            ),
+            "yafsdp_post_reduce",
+        )
+
+
+def post_reduce_fragments(
+    shard: torch.Tensor, chunk: torch.Tensor, frag_numels: Sequence[int], frag_modes: Sequence[int],
+    post_factor: float | None,
+) -> None:
+    _flat_arg(shard, "shard"), _flat_arg(chunk, "chunk")
+    numels = np.ascontiguousarray(frag_numels, dtype=np.int64)
+    modes = np.ascontiguousarray(frag_modes, dtype=np.uint8)
+    if numels.shape != modes.shape:
+        raise ValueError("frag_numels and frag_modes differ in length")
+    if int(numels.sum()) > min(shard.numel(), chunk.numel()):
+        raise ValueError("fragments exceed the shard")
+    with torch.cuda.device(shard.device):
+        _check(
+            lib.yafsdp_post_reduce_fragments(
+                shard.data_ptr(), _dt(shard), chunk.data_ptr(), _dt(chunk), int(numels.size),
+                numels.ctypes.data, modes.ctypes.data, _factor(post_factor), _stream(shard),
+            ),
+            "yafsdp_post_reduce_fragments",
+        )
+
+
+# --------------------------------------------------------------- table ops --
+class TensorTable:
+    """Device-resident metadata of one flat buffer (tensor boundaries and the
+    tile -> tensor map).  Static for the life of a parameter group; the tensor
+    pointers are passed with every call."""
+
+    def __init__(self, numels: Sequence[int], padded_numel: int, device: torch.device):
+        self.numels = [int(n) for n in numels]
+        self.total_numel = sum(self.numels)
+        self.padded_numel = int(padded_numel)
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError(f"TensorTable needs a GPU device, got {device}")
+        arr = np.ascontiguousarray(self.numels, dtype=np.int64)
+        handle = ctypes.c_void_p()
+        with torch.cuda.device(self.device):
+            _check(
+                lib.yafsdp_table_create(len(self.numels), arr.ctypes.data, self.padded_numel, ctypes.byref(handle)),
+                "yafsdp_table_create",
+            )
+        self._handle = handle
+        self._ptrs = np.zeros(max(1, len(self.numels)), dtype=np.uint64)
+        self._modes = np.zeros(max(1, len(self.numels)), dtype=np.uint8)
+
+    def close(self) -> None:
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            lib.yafsdp_table_destroy(h)
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _fill(self, tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None, what: str) -> int:
+        if len(tensors) != len(self.numels):
+            raise ValueError(f"{what}: expected {len(self.numels)} tensors, got {len(tensors)}")
+        dtype = None
+        for p, t in enumerate(tensors):
+            m = MODE_COPY if modes is None else int(modes[p])
+            if t is None:
+                m = MODE_SKIP
+            self._modes[p] = m
+            if m == MODE_SKIP:
+                self._ptrs[p] = 0
+                continue
+            _flat_arg(t, f"{what}[{p}]")
+            if t.device != self.device:
+                raise RuntimeError(f"{what}[{p}] is on {t.device}, table on {self.device}")
+            if t.numel() != self.numels[p]:
+                raise ValueError(f"{what}[{p}]: numel {t.numel()} != {self.numels[p]}")
+            if dtype is None:
+                dtype = t.dtype
+            elif t.dtype != dtype:
+                raise TypeError(f"{what}: tensors of one call share a dtype, got {dtype} and {t.dtype}")
+            self._ptrs[p] = t.data_ptr()
+        return DTYPE_CODE[dtype] if dtype is not None else -1
+
+    def gather_in(
+        self, tensors: Sequence[torch.Tensor | None], flat: torch.Tensor, modes: Sequence[int] | None = None,
+        pre_factor: float | None = None, zero_pad: bool = True,
+    ) -> None:
+        """Reduce copy-in (+ fused pre-divide and pad zero-fill) into ``flat``."""
+        _flat_arg(flat, "flat")
+        if flat.numel() < self.padded_numel:
+            raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.padded_numel}")
+        tdt = self._fill(tensors, modes, "tensors")
+        if tdt < 0:
+            tdt = _dt(flat)
+        with torch.cuda.device(self.device):
+            _check(
+                lib.yafsdp_gather_in(
+                    self._handle, self._ptrs.ctypes.data, self._modes.ctypes.data, tdt, flat.data_ptr(), _dt(flat),
+                    _factor(pre_factor), int(bool(zero_pad)), _stream(flat),
+                ),
+                "yafsdp_gather_in",
+            )
+
+    def scatter_out(
+        self, flat: torch.Tensor, tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None = None
+    ) -> None:
+        """Materialising copy-out of ``flat[:total]`` into ``tensors``."""
+        _flat_arg(flat, "flat")
+        if flat.numel() < self.total_numel:
+            raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.total_numel}")
+        tdt = self._fill(tensors, modes, "tensors")
+        if tdt < 0:
+            return
+        with torch.cuda.device(self.device):
+            _check(
+                lib.yafsdp_scatter_out(
+                    self._handle, flat.data_ptr(), _dt(flat), self._ptrs.ctypes.data, self._modes.ctypes.data, tdt,
+                    _stream(flat),
+                ),
+                "yafsdp_scatter_out",
+            )
+
+
+def set_option(option: int, value: int) -> None:
+    _check(lib.yafsdp_set_option(int(option), int(value)), "yafsdp_set_option")
+
+
+def get_option(option: int) -> int:
+    v = ctypes.c_int()
+    _check(lib.yafsdp_get_option(int(option), ctypes.byref(v)), "yafsdp_get_option")
+    return v.value

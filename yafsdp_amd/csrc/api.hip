@@ -1,0 +1,412 @@
+// C ABI of libyafsdp_hip.so: argument validation, metadata tables, launch
+// shapes.  Declarations and the reference call sites each entry point replaces
+// are in include/yafsdp_hip.h.
+#include <atomic>
+#include <cmath>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "../../include/yafsdp_hip.h"
+#include "launch.h"
+#include "tuning.h"
+
+using namespace yafsdp;
+
+namespace {
+
+std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
+std::atomic<int> g_table_blocks_per_cu{kTableBlocksPerCu};
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_cu_count[kMaxDevices];
+
+int cu_count(int device) {
+  if (device < 0 || device >= kMaxDevices) return 256;
+  int c = g_cu_count[device].load(std::memory_order_relaxed);
+  if (c > 0) return c;
+  int v = 0;
+  if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || v <= 0) v = 256;
+  g_cu_count[device].store(v, std::memory_order_relaxed);
+  return v;
+}
+
+inline bool valid_dtype(int dt) { return dt == DT_F32 || dt == DT_BF16 || dt == DT_F16; }
+inline int item_size(int dt) { return dt == DT_F32 ? 4 : 2; }
+inline bool aligned_to(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// How a divide factor is applied (ya_fsdp/_collectives.py:270-272: only > 1).
+// A power-of-two factor whose reciprocal is a normal binary32 number becomes an
+// exact multiply: x * 2^-k and x / 2^k are the same real number rounded once.
+void scale_plan(double factor, int* scale, float* k) {
+  *scale = SCALE_NONE;
+  *k = 1.0f;
+  if (!(factor > 1.0)) return;
+  const float f = static_cast<float>(factor);
+  if (!(f > 1.0f)) return;  // rounded down to 1: dividing by 1.0f changes nothing
+  int e = 0;
+  const float m = std::frexp(f, &e);
+  if (m == 0.5f && e <= 126 && std::isfinite(f)) {
+    *scale = SCALE_MUL;
+    *k = 1.0f / f;
+  } else {
+    *scale = SCALE_DIV;
+    *k = f;
+  }
+}
+
+int grid_for(int64_t n_tiles, int blocks_per_cu, int device) {
+  int64_t cap = int64_t(cu_count(device)) * (blocks_per_cu > 0 ? blocks_per_cu : 1);
+  int64_t g = n_tiles < cap ? n_tiles : cap;
+  return g < 1 ? 1 : int(g);
+}
+
+int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, float k,
+                hipStream_t stream) {
+  if (n == 0) return YAFSDP_OK;
+  if (!aligned_to(dst, item_size(dst_dt)) || !aligned_to(src, item_size(src_dt))) return YAFSDP_ERR_MISALIGNED;
+  int64_t head = ((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / item_size(dst_dt);
+  if (head > n) head = n;
+  const int64_t units = (n - head) >> 3;
+  const int64_t tile = int64_t(kFlatBlock) * kFlatUnroll;
+  const int64_t n_tiles = (units + tile - 1) / tile;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  const int grid = grid_for(n_tiles, g_flat_blocks_per_cu.load(std::memory_order_relaxed), device);
+  e = launch_flat(src_dt, dst_dt, scale, acc, dst, src, n, int(head), k, grid, stream);
+  return int(e);
+}
+
+}  // namespace
+
+struct yafsdp_table {
+  int device = 0;
+  int32_t n_tensors = 0;
+  int32_t n_tiles = 0;
+  int64_t total = 0;
+  int64_t padded = 0;
+  std::vector<int64_t> offsets;  // host copy, n_tensors + 1
+  int64_t* d_offsets = nullptr;
+  int32_t* d_tile_first = nullptr;
+  // staging ring for the per-call pointer/mode arrays of tables with more than
+  // kKargMax tensors: pinned host slot -> device slot, one event per slot
+  static constexpr int kRing = 4;
+  size_t stage_bytes = 0;
+  char* h_stage[kRing] = {nullptr, nullptr, nullptr, nullptr};
+  char* d_stage[kRing] = {nullptr, nullptr, nullptr, nullptr};
+  hipEvent_t ev[kRing] = {nullptr, nullptr, nullptr, nullptr};
+  bool ev_pending[kRing] = {false, false, false, false};
+  int next = 0;
+  std::mutex mu;
+};
+
+namespace {
+
+void table_free(yafsdp_table* t) {
+  if (t == nullptr) return;
+  if (t->d_offsets) (void)hipFree(t->d_offsets);
+  if (t->d_tile_first) (void)hipFree(t->d_tile_first);
+  for (int i = 0; i < yafsdp_table::kRing; i++) {
+    if (t->ev[i]) (void)hipEventDestroy(t->ev[i]);
+    if (t->h_stage[i]) (void)hipHostFree(t->h_stage[i]);
+    if (t->d_stage[i]) (void)hipFree(t->d_stage[i]);
+  }
+  delete t;
+}
+
+// Fill dyn from host arrays; for big tables stage them through the ring.
+// Returns 0 or an error code; *slot is the ring slot used (-1 if none).
+int prepare_dyn(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int elem_size, DynArgs* dyn, int* slot,
+                hipStream_t stream) {
+  *slot = -1;
+  std::memset(dyn, 0, sizeof(*dyn));
+  const int n = t->n_tensors;
+  for (int p = 0; p < n; p++) {
+    const uint8_t m = mode ? mode[p] : uint8_t(MODE_COPY);
+    if (m > MODE_ADD) return YAFSDP_ERR_INVALID_ARGUMENT;
+    const bool live = m != MODE_SKIP && t->offsets[p + 1] > t->offsets[p];
+    if (live) {
+      if (ptrs[p] == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+      if (!aligned_to(ptrs[p], elem_size)) return YAFSDP_ERR_MISALIGNED;
+    }
+  }
+  if (n <= kKargMax) {
+    for (int p = 0; p < n; p++) {
+      dyn->ptr[p] = ptrs[p];
+      dyn->mode[p] = mode ? mode[p] : uint8_t(MODE_COPY);
+    }
+    return YAFSDP_OK;
+  }
+  const int s = t->next;
+  t->next = (t->next + 1) % yafsdp_table::kRing;
+  if (t->ev_pending[s]) {
+    hipError_t e = hipEventSynchronize(t->ev[s]);
+    if (e != hipSuccess) return int(e);
+    t->ev_pending[s] = false;
+  }
+  char* h = t->h_stage[s];
+  std::memcpy(h, ptrs, size_t(n) * sizeof(void*));
+  uint8_t* hm = reinterpret_cast<uint8_t*>(h + size_t(n) * sizeof(void*));
+  for (int p = 0; p < n; p++) hm[p] = mode ? mode[p] : uint8_t(MODE_COPY);
+  hipError_t e = hipMemcpyAsync(t->d_stage[s], h, t->stage_bytes, hipMemcpyHostToDevice, stream);
+  if (e != hipSuccess) return int(e);
+  dyn->dev_ptr = reinterpret_cast<const void* const*>(t->d_stage[s]);
+  dyn->dev_mode = reinterpret_cast<const uint8_t*>(t->d_stage[s] + size_t(n) * sizeof(void*));
+  *slot = s;
+  return YAFSDP_OK;
+}
+
+int finish_dyn(yafsdp_table* t, int slot, hipStream_t stream) {
+  if (slot < 0) return YAFSDP_OK;
+  hipError_t e = hipEventRecord(t->ev[slot], stream);
+  if (e != hipSuccess) return int(e);
+  t->ev_pending[slot] = true;
+  return YAFSDP_OK;
+}
+
+TableView view_of(const yafsdp_table* t) {
+  TableView tv;
+  tv.offsets = t->d_offsets;
+  tv.tile_first = t->d_tile_first;
+  tv.total = t->total;
+  tv.padded = t->padded;
+  tv.n_tensors = t->n_tensors;
+  tv.n_tiles = t->n_tiles;
+  return tv;
+}
+
+}  // namespace
+
+extern "C" {
+
+int yafsdp_version(void) { return 1000; }
+
+const char* yafsdp_error_string(int code) {
+  switch (code) {
+    case YAFSDP_OK: return "success";
+    case YAFSDP_ERR_INVALID_ARGUMENT: return "yafsdp: invalid argument";
+    case YAFSDP_ERR_UNSUPPORTED_DTYPE: return "yafsdp: unsupported dtype (expected 0=f32, 1=bf16, 2=f16)";
+    case YAFSDP_ERR_MISALIGNED: return "yafsdp: pointer not aligned (element size; 16 bytes for flat table buffers)";
+    case YAFSDP_ERR_WRONG_DEVICE: return "yafsdp: table belongs to another device than the current one";
+    case YAFSDP_ERR_OUT_OF_MEMORY: return "yafsdp: host allocation failed";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+  return "yafsdp: unknown error code";
+}
+
+int yafsdp_set_option(int option, int value) {
+  if (value < 1 || value > 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
+  switch (option) {
+    case YAFSDP_OPT_FLAT_BLOCKS_PER_CU: g_flat_blocks_per_cu.store(value); return YAFSDP_OK;
+    case YAFSDP_OPT_TABLE_BLOCKS_PER_CU: g_table_blocks_per_cu.store(value); return YAFSDP_OK;
+  }
+  return YAFSDP_ERR_INVALID_ARGUMENT;
+}
+
+int yafsdp_get_option(int option, int* value) {
+  if (value == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  switch (option) {
+    case YAFSDP_OPT_FLAT_BLOCKS_PER_CU: *value = g_flat_blocks_per_cu.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_TABLE_BLOCKS_PER_CU: *value = g_table_blocks_per_cu.load(); return YAFSDP_OK;
+  }
+  return YAFSDP_ERR_INVALID_ARGUMENT;
+}
+
+int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, void* stream) {
+  if (!valid_dtype(dst_dtype) || !valid_dtype(src_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && (dst == nullptr || src == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n > 0 && dst == src && dst_dtype == src_dtype) return YAFSDP_OK;  // aliasing self-copy
+  return flat_launch(src_dtype, dst_dtype, SCALE_NONE, false, dst, src, n, 1.0f, static_cast<hipStream_t>(stream));
+}
+
+int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && buf == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  scale_plan(factor, &scale, &k);
+  if (scale == SCALE_NONE) return YAFSDP_OK;
+  return flat_launch(dtype, dtype, scale, false, buf, buf, n, k, static_cast<hipStream_t>(stream));
+}
+
+int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n, double post_factor,
+                       int accumulate, void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && (shard == nullptr || chunk == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  scale_plan(post_factor, &scale, &k);
+  if (shard == chunk) {
+    // the reduction already wrote into the shard: only the divide is left, and
+    // accumulating a buffer into itself is not an operation of this path
+    if (shard_dtype != chunk_dtype || accumulate) return YAFSDP_ERR_INVALID_ARGUMENT;
+    if (scale == SCALE_NONE) return YAFSDP_OK;
+  }
+  return flat_launch(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, chunk, n, k,
+                     static_cast<hipStream_t>(stream));
+}
+
+int yafsdp_post_reduce_fragments(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int n_fragments,
+                                 const int64_t* frag_numels, const uint8_t* frag_mode, double post_factor,
+                                 void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n_fragments < 0 || (n_fragments > 0 && (frag_numels == nullptr || frag_mode == nullptr)))
+    return YAFSDP_ERR_INVALID_ARGUMENT;
+  int64_t total = 0;
+  for (int f = 0; f < n_fragments; f++) {
+    if (frag_numels[f] < 0 || frag_mode[f] > MODE_ADD) return YAFSDP_ERR_INVALID_ARGUMENT;
+    total += frag_numels[f];
+  }
+  if (total > 0 && (shard == nullptr || chunk == nullptr || shard == chunk)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  scale_plan(post_factor, &scale, &k);
+  // merge neighbouring fragments of equal mode into runs: one launch per run
+  int64_t pos = 0;
+  int f = 0;
+  while (f < n_fragments) {
+    const uint8_t m = frag_mode[f];
+    int64_t run = 0;
+    while (f < n_fragments && (frag_mode[f] == m || frag_numels[f] == 0)) run += frag_numels[f++];
+    if (m != MODE_SKIP && run > 0) {
+      char* d = static_cast<char*>(shard) + pos * item_size(shard_dtype);
+      const char* s = static_cast<const char*>(chunk) + pos * item_size(chunk_dtype);
+      int rc = flat_launch(chunk_dtype, shard_dtype, scale, m == MODE_ADD, d, s, run, k,
+                           static_cast<hipStream_t>(stream));
+      if (rc != YAFSDP_OK) return rc;
+    }
+    pos += run;
+  }
+  return YAFSDP_OK;
+}
+
+int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_numel, yafsdp_table** out) {
+  if (out == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  if (n_tensors < 0 || (n_tensors > 0 && numels == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  yafsdp_table* t = new (std::nothrow) yafsdp_table();
+  if (t == nullptr) return YAFSDP_ERR_OUT_OF_MEMORY;
+  int rc = YAFSDP_OK;
+  hipError_t e = hipSuccess;
+  std::vector<int32_t> tile_first;
+  do {
+    t->n_tensors = n_tensors;
+    t->offsets.assign(size_t(n_tensors) + 1, 0);
+    for (int p = 0; p < n_tensors; p++) {
+      if (numels[p] < 0) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+      t->offsets[p + 1] = t->offsets[p] + numels[p];
+    }
+    if (rc != YAFSDP_OK) break;
+    t->total = t->offsets[n_tensors];
+    t->padded = padded_numel;
+    if (padded_numel < t->total) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    const int64_t n_tiles = (padded_numel + kTableTileElems - 1) / kTableTileElems;
+    if (n_tiles > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    t->n_tiles = int32_t(n_tiles);
+    // tile_first[tile]: first tensor whose end lies beyond the tile's first element
+    tile_first.resize(size_t(n_tiles));
+    int p = 0;
+    for (int64_t tile = 0; tile < n_tiles; tile++) {
+      const int64_t t0 = tile * kTableTileElems;
+      while (p < n_tensors && t->offsets[p + 1] <= t0) p++;
+      tile_first[size_t(tile)] = p;
+    }
+    if ((e = hipGetDevice(&t->device)) != hipSuccess) break;
+    if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_offsets), t->offsets.size() * sizeof(int64_t))) != hipSuccess) break;
+    if ((e = hipMemcpy(t->d_offsets, t->offsets.data(), t->offsets.size() * sizeof(int64_t), hipMemcpyHostToDevice)) != hipSuccess) break;
+    if (n_tiles > 0) {
+      if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_tile_first), tile_first.size() * sizeof(int32_t))) != hipSuccess) break;
+      if ((e = hipMemcpy(t->d_tile_first, tile_first.data(), tile_first.size() * sizeof(int32_t), hipMemcpyHostToDevice)) != hipSuccess) break;
+    }
+    if (n_tensors > kKargMax) {
+      t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + 1) + 15) & ~size_t(15);
+      for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
+        if ((e = hipHostMalloc(reinterpret_cast<void**>(&t->h_stage[i]), t->stage_bytes, hipHostMallocDefault)) != hipSuccess) break;
+        if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_stage[i]), t->stage_bytes)) != hipSuccess) break;
+        if ((e = hipEventCreateWithFlags(&t->ev[i], hipEventDisableTiming)) != hipSuccess) break;
+      }
+    }
+  } while (false);
+  if (rc == YAFSDP_OK && e != hipSuccess) rc = int(e);
+  if (rc != YAFSDP_OK) {
+    table_free(t);
+    return rc;
+  }
+  *out = t;
+  return YAFSDP_OK;
+}
+
+int yafsdp_table_destroy(yafsdp_table* table) {
+  if (table == nullptr) return YAFSDP_OK;
+  int rc = YAFSDP_OK;
+  for (int i = 0; i < yafsdp_table::kRing; i++) {
+    if (table->ev_pending[i]) {
+      hipError_t e = hipEventSynchronize(table->ev[i]);
+      if (e != hipSuccess) rc = int(e);
+    }
+  }
+  table_free(table);
+  return rc;
+}
+
+int yafsdp_table_info(const yafsdp_table* table, int* n_tensors, int64_t* total_numel, int64_t* padded_numel) {
+  if (table == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n_tensors) *n_tensors = table->n_tensors;
+  if (total_numel) *total_numel = table->total;
+  if (padded_numel) *padded_numel = table->padded;
+  return YAFSDP_OK;
+}
+
+int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode, int tensor_dtype,
+                     void* flat, int flat_dtype, double pre_factor, int zero_pad, void* stream) {
+  if (table == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!valid_dtype(tensor_dtype) || !valid_dtype(flat_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (table->padded == 0) return YAFSDP_OK;
+  if (flat == nullptr || (table->n_tensors > 0 && tensor_ptrs == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(flat, 16)) return YAFSDP_ERR_MISALIGNED;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
+  int scale;
+  float k;
+  scale_plan(pre_factor, &scale, &k);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  std::lock_guard<std::mutex> lock(table->mu);
+  DynArgs dyn;
+  int slot;
+  int rc = prepare_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype), &dyn, &slot, s);
+  if (rc != YAFSDP_OK) return rc;
+  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  e = launch_gather(tensor_dtype, flat_dtype, scale, view_of(table), dyn, flat, k, zero_pad ? 1 : 0, grid, s);
+  if (e != hipSuccess) return int(e);
+  return finish_dyn(table, slot, s);
+}
+
+int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
+                       const uint8_t* mode, int tensor_dtype, void* stream) {
+  if (table == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!valid_dtype(tensor_dtype) || !valid_dtype(flat_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (table->total == 0) return YAFSDP_OK;
+  if (flat == nullptr || tensor_ptrs == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(flat, 16)) return YAFSDP_ERR_MISALIGNED;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  std::lock_guard<std::mutex> lock(table->mu);
+  DynArgs dyn;
+  int slot;
+  int rc = prepare_dyn(table, const_cast<const void* const*>(tensor_ptrs), mode, item_size(tensor_dtype), &dyn, &slot, s);
+  if (rc != YAFSDP_OK) return rc;
+  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  e = launch_scatter(flat_dtype, tensor_dtype, view_of(table), dyn, flat, grid, s);
+  if (e != hipSuccess) return int(e);
+  return finish_dyn(table, slot, s);
+}
+
+}  // extern "C"

@@ -1,0 +1,208 @@
+// Element types, 8-element vector units and the per-element arithmetic of the
+// buffer path, for gfx950 (wave64).
+//
+// A "unit" is 8 consecutive elements: 16 bytes of a 2-byte dtype (one
+// global_load/store_dwordx4 per lane) or 32 bytes of fp32 (two).  All
+// arithmetic is done in binary32, every materialisation point of the reference
+// rounds once (RNE) to the dtype of the tensor it materialises, and no
+// multiply-add is ever contracted (the translation units are built with
+// -ffp-contract=off as well).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace yafsdp {
+
+enum : int { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
+// how a divide factor is applied: not at all, as an exact multiply by the
+// reciprocal (power-of-two factors only: same bits as a division), or as a
+// correctly rounded binary32 division.
+enum : int { SCALE_NONE = 0, SCALE_MUL = 1, SCALE_DIV = 2 };
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+// 16-byte vectors that may sit at any element-aligned address; gfx950 under
+// the HSA runtime executes dwordx4 accesses at such addresses natively
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+
+struct F32 {
+  typedef float storage;
+  typedef u32x4_a4 vec_unaligned;
+  static constexpr int kId = DT_F32;
+  static constexpr int kSize = 4;
+  static constexpr int kVecs = 2;  // dwordx4 accesses per unit
+};
+struct BF16 {
+  typedef uint16_t storage;
+  typedef u32x4_a2 vec_unaligned;
+  static constexpr int kId = DT_BF16;
+  static constexpr int kSize = 2;
+  static constexpr int kVecs = 1;
+};
+struct F16 {
+  typedef uint16_t storage;
+  typedef u32x4_a2 vec_unaligned;
+  static constexpr int kId = DT_F16;
+  static constexpr int kSize = 2;
+  static constexpr int kVecs = 1;
+};
+
+template <class A, class B>
+struct same_t { static constexpr bool value = false; };
+template <class A>
+struct same_t<A, A> { static constexpr bool value = true; };
+
+template <class T>
+struct Unit { u32x4 v[T::kVecs]; };
+
+// ---- memory -----------------------------------------------------------------
+// `p` only needs element alignment.  NT selects the non-temporal (streaming)
+// cache policy.
+template <class T, bool NT>
+__device__ __forceinline__ Unit<T> load_unit(const void* p) {
+  Unit<T> r;
+  const typename T::vec_unaligned* q = reinterpret_cast<const typename T::vec_unaligned*>(p);
+#pragma unroll
+  for (int i = 0; i < T::kVecs; i++) {
+    if constexpr (NT) r.v[i] = __builtin_nontemporal_load(q + i);
+    else r.v[i] = q[i];
+  }
+  return r;
+}
+
+template <class T, bool NT>
+__device__ __forceinline__ void store_unit(void* p, const Unit<T>& u) {
+  typename T::vec_unaligned* q = reinterpret_cast<typename T::vec_unaligned*>(p);
+#pragma unroll
+  for (int i = 0; i < T::kVecs; i++) {
+    if constexpr (NT) __builtin_nontemporal_store(u.v[i], q + i);
+    else q[i] = u.v[i];
+  }
+}
+
+// ---- scalar conversions -------------------------------------------------------
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+template <class T> __device__ __forceinline__ float to_f32(typename T::storage s);
+template <> __device__ __forceinline__ float to_f32<F32>(float s) { return s; }
+template <> __device__ __forceinline__ float to_f32<BF16>(uint16_t s) { return bits_to_f32(uint32_t(s) << 16); }
+template <> __device__ __forceinline__ float to_f32<F16>(uint16_t s) {
+  return (float)__builtin_bit_cast(_Float16, s);
+}
+
+// round to nearest even (hardware v_cvt_pk_bf16_f32 / v_cvt_f16_f32)
+template <class T> __device__ __forceinline__ typename T::storage from_f32(float f);
+template <> __device__ __forceinline__ float from_f32<F32>(float f) { return f; }
+template <> __device__ __forceinline__ uint16_t from_f32<BF16>(float f) {
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+template <> __device__ __forceinline__ uint16_t from_f32<F16>(float f) {
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+// the value a binary32 number has after being stored as T and read back
+template <class T>
+__device__ __forceinline__ float round_to(float f) {
+  if constexpr (same_t<T, F32>::value) return f;
+  else return to_f32<T>(from_f32<T>(f));
+}
+
+// ---- unit <-> 8 floats --------------------------------------------------------
+template <class T>
+__device__ __forceinline__ void unpack(const Unit<T>& u, float (&f)[8]) {
+  if constexpr (same_t<T, F32>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) { f[i] = bits_to_f32(u.v[0][i]); f[4 + i] = bits_to_f32(u.v[1][i]); }
+  } else if constexpr (same_t<T, BF16>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint32_t w = u.v[0][i];
+      f[2 * i] = bits_to_f32(w << 16);
+      f[2 * i + 1] = bits_to_f32(w & 0xFFFF0000u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t w = u.v[0][i];
+      f[2 * i] = (float)__builtin_bit_cast(_Float16, uint16_t(w & 0xFFFFu));
+      f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, uint16_t(w >> 16));
+    }
+  }
+}
+
+template <class T>
+__device__ __forceinline__ Unit<T> pack(const float (&f)[8]) {
+  Unit<T> u;
+  if constexpr (same_t<T, F32>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) { u.v[0][i] = f32_to_bits(f[i]); u.v[1][i] = f32_to_bits(f[4 + i]); }
+  } else if constexpr (same_t<T, BF16>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      f32x2 x = {f[2 * i], f[2 * i + 1]};
+      u.v[0][i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      f32x2 x = {f[2 * i], f[2 * i + 1]};
+      u.v[0][i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+    }
+  }
+  return u;
+}
+
+// ---- the arithmetic -----------------------------------------------------------
+// Keeps a value opaque to the instruction selector (emits nothing).  Without it
+// a multiply next to an fp16 conversion is selected as v_fma_mix*(a, b, +0),
+// whose +0 addend turns a -0 product into +0.
+__device__ __forceinline__ float opaque(float y) {
+  asm("" : "+v"(y));
+  return y;
+}
+
+template <int SCALE>
+__device__ __forceinline__ float apply_scale(float y, float k) {
+  if constexpr (SCALE == SCALE_MUL) return opaque(__fmul_rn(opaque(y), k));  // k = 1/factor, exact
+  else if constexpr (SCALE == SCALE_DIV) return __fdiv_rn(y, k);             // k = factor
+  else return y;
+}
+
+// Reduce copy-in element (tensor dtype S -> flat reduce buffer dtype D):
+//   view.copy_(grad) or view.add_(grad)   -> rounds to D
+//   buffer.div_(pre)                      -> rounds to D again
+// MODE: 1 copy, 2 add, 0 tensor absent (only the divide touches the element).
+enum : int { MODE_SKIP = 0, MODE_COPY = 1, MODE_ADD = 2 };
+
+template <class S, class D, int SCALE, int MODE>
+__device__ __forceinline__ float gather_elem(float s, float d_old, float k) {
+  float y;
+  if constexpr (MODE == MODE_COPY) y = s;
+  else if constexpr (MODE == MODE_ADD) y = __fadd_rn(d_old, s);
+  else y = d_old;
+  if constexpr (SCALE != SCALE_NONE) {
+    if constexpr (MODE != MODE_SKIP) y = round_to<D>(y);
+    y = apply_scale<SCALE>(y, k);
+  }
+  return y;  // caller rounds to D on store
+}
+
+// Post-reduce element (chunk dtype S -> grad shard dtype D):
+//   chunk.div_(post)                      -> rounds to S
+//   shard.copy_(chunk) or shard.add_(chunk) -> rounds to D
+template <class S, class D, int SCALE, bool ACC>
+__device__ __forceinline__ float post_elem(float s, float d_old, float k) {
+  float y = s;
+  if constexpr (SCALE != SCALE_NONE) {
+    y = apply_scale<SCALE>(y, k);
+    if constexpr (ACC || !same_t<S, D>::value) y = round_to<S>(y);
+  }
+  if constexpr (ACC) y = __fadd_rn(d_old, y);
+  return y;  // caller rounds to D on store
+}
+
+}  // namespace yafsdp

@@ -1,0 +1,96 @@
+// Flat (one contiguous range -> one contiguous range) kernels of the buffer
+// path: copy-in cast, single-rank all-gather/reduce-scatter copies, in-place
+// pre/post divide, and the fused post-reduce (divide + copy/accumulate into the
+// gradient shard).
+//
+// Work partitioning: the range is cut into tiles of BLOCK*U units (a unit is 8
+// elements); a workgroup walks tiles with a grid stride; inside a tile lane l of
+// the workgroup touches units l, l+BLOCK, ... so that every wave64 access is one
+// contiguous 1 KiB (2-byte dtypes) or 2 KiB (fp32) span.  All U loads of a lane
+// are issued before the first store.  The destination is 16-byte aligned for
+// the unit loop (the host peels up to 7 leading elements, handled by workgroup 0
+// together with the tail); the source may sit at any element-aligned address.
+#pragma once
+#include "elem.cuh"
+
+namespace yafsdp {
+
+template <class S, class D, int SCALE, bool ACC>
+__device__ __forceinline__ void flat_scalar(void* dst, const void* src, int64_t i, float k) {
+  typedef typename S::storage s_t;
+  typedef typename D::storage d_t;
+  if constexpr (same_t<S, D>::value && SCALE == SCALE_NONE && !ACC) {
+    reinterpret_cast<d_t*>(dst)[i] = reinterpret_cast<const s_t*>(src)[i];
+  } else {
+    float s = to_f32<S>(reinterpret_cast<const s_t*>(src)[i]);
+    float d_old = 0.f;
+    if constexpr (ACC) d_old = to_f32<D>(reinterpret_cast<const d_t*>(dst)[i]);
+    reinterpret_cast<d_t*>(dst)[i] = from_f32<D>(post_elem<S, D, SCALE, ACC>(s, d_old, k));
+  }
+}
+
+template <class S, class D, int SCALE, bool ACC>
+__device__ __forceinline__ Unit<D> flat_unit(const Unit<S>& s, const Unit<D>& d_old, float k) {
+  if constexpr (same_t<S, D>::value && SCALE == SCALE_NONE && !ACC) {
+    return s;  // byte copy: NaN payloads and all bit patterns pass through
+  } else {
+    float fs[8], fd[8], fy[8];
+    unpack<S>(s, fs);
+    if constexpr (ACC) unpack<D>(d_old, fd);
+#pragma unroll
+    for (int e = 0; e < 8; e++) fy[e] = post_elem<S, D, SCALE, ACC>(fs[e], ACC ? fd[e] : 0.f, k);
+    return pack<D>(fy);
+  }
+}
+
+// dst[i] = op(src[i], dst[i]) for i in [0, n).  `head` leading elements bring
+// dst to a 16-byte boundary.  dst == src is allowed (in-place divide).
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
+__global__ void __launch_bounds__(BLOCK)
+flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
+  const int tid = threadIdx.x;
+  const int64_t n_units = (n - head) >> 3;
+  const int64_t body_end = head + (n_units << 3);
+  if (blockIdx.x == 0) {
+    if (tid < head) flat_scalar<S, D, SCALE, ACC>(dst, src, tid, k);
+    const int tail = int(n - body_end);
+    const int t = BLOCK - 1 - tid;
+    if (t < tail) flat_scalar<S, D, SCALE, ACC>(dst, src, body_end + t, k);
+  }
+  char* dbase = reinterpret_cast<char*>(dst) + int64_t(head) * D::kSize;
+  const char* sbase = reinterpret_cast<const char*>(src) + int64_t(head) * S::kSize;
+  constexpr int64_t kTile = int64_t(BLOCK) * U;
+  const int64_t n_tiles = (n_units + kTile - 1) / kTile;
+  for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const int64_t u0 = tile * kTile + tid;
+    Unit<S> s[U];
+    Unit<D> d[U];
+    if (tile * kTile + kTile <= n_units) {
+#pragma unroll
+      for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(sbase + (u0 + int64_t(j) * BLOCK) * (8 * S::kSize));
+      if constexpr (ACC) {
+#pragma unroll
+        for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dbase + (u0 + int64_t(j) * BLOCK) * (8 * D::kSize));
+      }
+#pragma unroll
+      for (int j = 0; j < U; j++)
+        store_unit<D, NTS>(dbase + (u0 + int64_t(j) * BLOCK) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
+    } else {
+#pragma unroll
+      for (int j = 0; j < U; j++) {
+        const int64_t u = u0 + int64_t(j) * BLOCK;
+        if (u < n_units) {
+          s[j] = load_unit<S, NTL>(sbase + u * (8 * S::kSize));
+          if constexpr (ACC) d[j] = load_unit<D, NTL>(dbase + u * (8 * D::kSize));
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < U; j++) {
+        const int64_t u = u0 + int64_t(j) * BLOCK;
+        if (u < n_units) store_unit<D, NTS>(dbase + u * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
+      }
+    }
+  }
+}
+
+}  // namespace yafsdp

@@ -1,0 +1,19 @@
+// Internal launcher interface between the C ABI (api.hip) and the translation
+// units that instantiate the kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "table_kernels.cuh"
+
+namespace yafsdp {
+
+// dst[i] = post_elem(src[i], dst[i]); scale is SCALE_NONE / SCALE_MUL / SCALE_DIV
+hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,
+                       float k, int grid, hipStream_t stream);
+hipError_t launch_gather(int tensor_dt, int flat_dt, int scale, const TableView& tv, const DynArgs& dyn, void* flat,
+                         float k, int pad_zero, int grid, hipStream_t stream);
+hipError_t launch_scatter(int flat_dt, int tensor_dt, const TableView& tv, const DynArgs& dyn, const void* flat,
+                          int grid, hipStream_t stream);
+
+}  // namespace yafsdp
