@@ -1,0 +1,283 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-rank buffer hot path on one MI355X.
+
+One "step" is one pass of the path over one batch of synthetic input, in the
+order a training step runs it for one parameter group:
+
+    copy-in         fp32 master shard [S]          -> bf16 all-gather input [S]
+    copy-out        bf16 gathered buffer [T_pad]   -> P separately allocated tensors
+    reduce copy-in  P bf16 gradients               -> bf16 reduce buffer [T_pad], fused /pre, pad zero-fill
+    post-reduce     rank's bf16 chunk [S]          -> += into the fp32 gradient shard [S]
+
+Default workload: one Llama-3-8B decoder layer at logical world size 8, one
+rank's share.  Inputs are resident in HBM before the timed region starts.
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+
+WORKLOADS = {
+    # name: (shapes in parameter order q,k,v,o,gate,up,down,norm,norm; W; rank; alignment; seed)
+    "llama3-8b-layer-w8": (
+        [(4096, 4096), (1024, 4096), (1024, 4096), (4096, 4096), (14336, 4096), (14336, 4096), (4096, 14336),
+         (4096,), (4096,)], 8, 3, 512, 1002),
+    "llama3-70b-layer-w64": (
+        [(8192, 8192), (1024, 8192), (1024, 8192), (8192, 8192), (28672, 8192), (28672, 8192), (8192, 28672),
+         (8192,), (8192,)], 64, 63, 512, 1003),
+    "tiny-layer-w1": (
+        [(512, 512)] * 4 + [(1376, 512), (1376, 512), (512, 1376), (512,), (512,)], 1, 0, 512, 1001),
+}
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (see profiles/); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def numel_of(shape):
+    n = 1
+    for d in shape:
+        n *= d
+    return n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="llama3-8b-layer-w8", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
+    ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        log(f"bench.py: this build runs on ONE GPU (the logical world size is a layout parameter); "
+            f"--gpus {args.gpus} is not supported.")
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; the buffer path has no CPU implementation to measure.")
+        return 3
+    from yafsdp_amd import _native
+    from yafsdp_amd._layout import make_layout
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    shapes, w, r, align, seed = WORKLOADS[args.workload]
+    numels = [numel_of(s) for s in shapes]
+    lay = make_layout(numels, w, align)
+    t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+    pre = float(w) if w > 1 else None
+    log(f"workload {args.workload}: P={len(numels)} T={t} T_pad={t_pad} S={s} W={w} rank={r} pre-divide={pre}")
+
+    # ---- synthetic inputs, generated on the CPU so that the oracle sees the same bits
+    g = torch.Generator().manual_seed(seed)
+    t0 = time.perf_counter()
+    master = torch.randn(s, generator=g) * 0.02  # fp32 master shard
+    gathered = torch.empty(t_pad, dtype=torch.bfloat16)
+    grads = []
+    pos = 0
+    for n in numels:  # chunked generation keeps the fp32 temporaries small
+        gathered[pos : pos + n] = (torch.randn(n, generator=g) * 0.02).bfloat16()
+        grads.append((torch.randn(n, generator=g) * 1e-3).bfloat16())
+        pos += n
+    gathered[t:] = 0
+    shard0 = torch.randn(s, generator=g) * 1e-4  # existing fp32 gradient shard
+    log(f"inputs generated in {time.perf_counter() - t0:.1f}s")
+
+    d_master = master.to(dev)
+    d_gathered = gathered.to(dev)
+    d_grads = [x.to(dev) for x in grads]
+    d_ag_in = torch.zeros(s, dtype=torch.bfloat16, device=dev)
+    d_outs = [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels]
+    d_rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=dev)
+    d_shard = shard0.to(dev)
+    d_chunk = d_rs[r * s : (r + 1) * s]
+    table = _native.TensorTable(numels, t_pad, dev)
+
+    def op_copy_in():
+        _native.flat_copy(d_ag_in, d_master)
+
+    def op_copy_out():
+        table.scatter_out(d_gathered, d_outs)
+
+    def op_reduce_copy_in():
+        table.gather_in(d_grads, d_rs, None, pre, True)
+
+    def op_post_reduce():
+        _native.post_reduce(d_shard, d_chunk, None, True)
+
+    ops = [
+        ("copy_in", op_copy_in, s * (4 + 2)),
+        ("copy_out", op_copy_out, 2 * t * 2),
+        ("reduce_copy_in", op_reduce_copy_in, t * (2 + 2) + (t_pad - t) * 2),
+        ("post_reduce", op_post_reduce, s * (2 + 4 + 4)),
+    ]
+    bytes_per_step = sum(b for _, _, b in ops)
+
+    def step():
+        for _, fn, _ in ops:
+            fn()
+
+    # ---- parity of one pass against the oracle (same run, same inputs)
+    parity = "skipped"
+    cpu_state = None
+    if not args.no_parity:
+        from oracle import torch_ops
+
+        def cpu_step(st):
+            torch_ops.copy_in(st["ag_in"], master)
+            torch_ops.copy_out_materialize(gathered, numels, st["outs"])
+            torch_ops.reduce_copy_in(st["rs_views"], grads, False)
+            torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
+
+        rs_cpu = torch.zeros(t_pad, dtype=torch.bfloat16)
+        cpu_state = {
+            "ag_in": torch.zeros(s, dtype=torch.bfloat16),
+            "outs": [torch.empty(n, dtype=torch.bfloat16) for n in numels],
+            "rs": rs_cpu,
+            "rs_views": list(rs_cpu[:t].split(numels)),
+            "shard": shard0.clone(),
+        }
+        cpu_step(cpu_state)
+        step()
+        torch.cuda.synchronize()
+
+        def same(a, b):
+            iv = torch.int32 if a.dtype == torch.float32 else torch.int16
+            return torch.equal(a.cpu().view(iv), b.view(iv))
+
+        ok = same(d_ag_in, cpu_state["ag_in"]) and same(d_rs, cpu_state["rs"]) and same(d_shard, cpu_state["shard"])
+        ok = ok and all(same(a, b) for a, b in zip(d_outs, cpu_state["outs"]))
+        parity = "bit-exact" if ok else "MISMATCH"
+        log("parity vs oracle:", parity)
+        if not ok:
+            log("bench.py: GPU results differ from the oracle; refusing to report a throughput.")
+            return 4
+
+    # ---- timed region
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    dom_index = 2  # reduce copy-in: most bytes, fused arithmetic
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ops[0][1]()
+        ops[1][1]()
+        ev[k][0].record()
+        ops[2][1]()
+        ev[k][1].record()
+        ops[3][1]()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = bytes_per_step * args.steps / elapsed / 1e9
+    dom_us = [a.elapsed_time(b) * 1e3 for a, b in ev]
+    dom_avg_us = sum(dom_us) / len(dom_us)
+    dom_bytes = ops[dom_index][2]
+    achieved = dom_bytes / dom_avg_us / 1e3
+
+    # ---- per-kernel table (outside the timed region): each op on its own between events
+    kernels = {}
+    for name, fn, nbytes in ops:
+        times = []
+        for _ in range(20):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            step_others = [f for n2, f, _ in ops if n2 != name]
+            for f in step_others:  # evict: the other ops stream 1-2 GB through the caches
+                f()
+            a.record()
+            fn()
+            b.record()
+            b.synchronize()
+            times.append(a.elapsed_time(b) * 1e3)
+        med = statistics.median(times)
+        kernels[name] = {
+            "bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
+            "GBps": round(nbytes / med / 1e3, 1), "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
+        }
+        log(f"  {name:15s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s "
+            f"({100 * nbytes / med / 1e3 / HBM_PEAK_GBS:.1f}% of peak)")
+
+    # ---- CPU baseline: the oracle (reference torch-op sequence) on the host cores
+    cpu_baseline = None
+    if args.cpu_seconds > 0 and cpu_state is not None:
+        from oracle import torch_ops  # noqa: F811
+
+        reps, spent = 0, 0.0
+        times = []
+        while spent < args.cpu_seconds and reps < 2000:
+            c0 = time.perf_counter()
+            cpu_step(cpu_state)
+            dt = time.perf_counter() - c0
+            times.append(dt)
+            spent += dt
+            reps += 1
+        med = statistics.median(times)
+        cpu_baseline = {
+            "value": round(bytes_per_step / med / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{reps} full passes of the same workload ({args.workload}) with the reference's torch ops "
+                      f"on CPU tensors, median of {reps}, {spent:.1f}s total",
+        }
+        log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads ({reps} passes)")
+
+    out = {
+        "metric": "HBM GB/s + % of peak for copy-in/out+grad-reduce, Llama-3-8B layer @W=8",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": args.workload, "params": len(numels), "total_numel": t, "padded_numel": t_pad,
+            "shard_numel": s, "logical_world_size": w, "rank": r, "shard_alignment": align,
+            "predivide": pre, "bytes_per_step": bytes_per_step,
+            "ops": "copy-in fp32->bf16 [S]; copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
+                   "post-reduce bf16 chunk += fp32 shard [S]",
+        },
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
+        "parity": parity,
+        "roofline": {
+            "bound": "hbm", "kernel": "gather_in_kernel (reduce copy-in)", "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2),
+        },
+        "cpu_baseline": cpu_baseline,
+        "kernels": kernels,
+    }
+    print(json.dumps(out), flush=True)
+    table.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

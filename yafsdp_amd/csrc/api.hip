@@ -84,14 +84,15 @@ int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const vo
 struct yafsdp_table {
   int device = 0;
   int32_t n_tensors = 0;
-  int32_t n_tiles = 0;
   int64_t total = 0;
   int64_t padded = 0;
   std::vector<int64_t> offsets;  // host copy, n_tensors + 1
   int64_t* d_offsets = nullptr;
-  int32_t* d_tile_first = nullptr;
+  // gather-in and scatter-out use different tile sizes: [0] gather, [1] scatter
+  int32_t n_tiles[2] = {0, 0};
+  TileRec* d_tiles[2] = {nullptr, nullptr};  // only for tables with more than kSmallMax tensors
   // staging ring for the per-call pointer/mode arrays of tables with more than
-  // kKargMax tensors: pinned host slot -> device slot, one event per slot
+  // kSmallMax tensors: pinned host slot -> device slot, one event per slot
   static constexpr int kRing = 4;
   size_t stage_bytes = 0;
   char* h_stage[kRing] = {nullptr, nullptr, nullptr, nullptr};
@@ -107,7 +108,8 @@ namespace {
 void table_free(yafsdp_table* t) {
   if (t == nullptr) return;
   if (t->d_offsets) (void)hipFree(t->d_offsets);
-  if (t->d_tile_first) (void)hipFree(t->d_tile_first);
+  for (int i = 0; i < 2; i++)
+    if (t->d_tiles[i]) (void)hipFree(t->d_tiles[i]);
   for (int i = 0; i < yafsdp_table::kRing; i++) {
     if (t->ev[i]) (void)hipEventDestroy(t->ev[i]);
     if (t->h_stage[i]) (void)hipHostFree(t->h_stage[i]);
@@ -116,14 +118,9 @@ void table_free(yafsdp_table* t) {
   delete t;
 }
 
-// Fill dyn from host arrays; for big tables stage them through the ring.
-// Returns 0 or an error code; *slot is the ring slot used (-1 if none).
-int prepare_dyn(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int elem_size, DynArgs* dyn, int* slot,
-                hipStream_t stream) {
-  *slot = -1;
-  std::memset(dyn, 0, sizeof(*dyn));
-  const int n = t->n_tensors;
-  for (int p = 0; p < n; p++) {
+// Validate the per-call host arrays.
+int check_dyn(const yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int elem_size) {
+  for (int p = 0; p < t->n_tensors; p++) {
     const uint8_t m = mode ? mode[p] : uint8_t(MODE_COPY);
     if (m > MODE_ADD) return YAFSDP_ERR_INVALID_ARGUMENT;
     const bool live = m != MODE_SKIP && t->offsets[p + 1] > t->offsets[p];
@@ -132,13 +129,32 @@ int prepare_dyn(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, i
       if (!aligned_to(ptrs[p], elem_size)) return YAFSDP_ERR_MISALIGNED;
     }
   }
-  if (n <= kKargMax) {
-    for (int p = 0; p < n; p++) {
-      dyn->ptr[p] = ptrs[p];
-      dyn->mode[p] = mode ? mode[p] : uint8_t(MODE_COPY);
-    }
-    return YAFSDP_OK;
+  return YAFSDP_OK;
+}
+
+// Small tables: everything travels in the kernel arguments.
+void fill_small(const yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int64_t tile_elems,
+                SmallMeta* m) {
+  std::memset(m, 0, sizeof(*m));
+  const int n = t->n_tensors;
+  m->n_tensors = n;
+  m->modes = 0;
+  for (int i = 0; i <= kSmallMax; i++) {
+    const int64_t o = t->offsets[i <= n ? i : n];
+    m->off[i] = o;
+    m->tile_start[i] = i <= n ? int32_t((o + tile_elems - 1) / tile_elems) : INT32_MAX;
   }
+  for (int p = 0; p < n; p++) {
+    m->ptr[p] = ptrs[p];
+    m->modes |= uint32_t(mode ? mode[p] : uint8_t(MODE_COPY)) << (2 * p);
+  }
+}
+
+// Large tables: stage pointers (8 bytes each) and modes (4 bytes each) through
+// the ring.  Returns 0 or an error code; *slot is the ring slot used.
+int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int which, LargeMeta* m, int* slot,
+                hipStream_t stream) {
+  const int n = t->n_tensors;
   const int s = t->next;
   t->next = (t->next + 1) % yafsdp_table::kRing;
   if (t->ev_pending[s]) {
@@ -148,33 +164,24 @@ int prepare_dyn(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, i
   }
   char* h = t->h_stage[s];
   std::memcpy(h, ptrs, size_t(n) * sizeof(void*));
-  uint8_t* hm = reinterpret_cast<uint8_t*>(h + size_t(n) * sizeof(void*));
-  for (int p = 0; p < n; p++) hm[p] = mode ? mode[p] : uint8_t(MODE_COPY);
+  uint32_t* hm = reinterpret_cast<uint32_t*>(h + size_t(n) * sizeof(void*));
+  for (int p = 0; p < n; p++) hm[p] = mode ? mode[p] : uint32_t(MODE_COPY);
   hipError_t e = hipMemcpyAsync(t->d_stage[s], h, t->stage_bytes, hipMemcpyHostToDevice, stream);
   if (e != hipSuccess) return int(e);
-  dyn->dev_ptr = reinterpret_cast<const void* const*>(t->d_stage[s]);
-  dyn->dev_mode = reinterpret_cast<const uint8_t*>(t->d_stage[s] + size_t(n) * sizeof(void*));
+  m->offsets = t->d_offsets;
+  m->tiles = t->d_tiles[which];
+  m->ptrs = reinterpret_cast<const void* const*>(t->d_stage[s]);
+  m->modes_ = reinterpret_cast<const uint32_t*>(t->d_stage[s] + size_t(n) * sizeof(void*));
+  m->n_tensors = n;
   *slot = s;
   return YAFSDP_OK;
 }
 
-int finish_dyn(yafsdp_table* t, int slot, hipStream_t stream) {
-  if (slot < 0) return YAFSDP_OK;
+int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
   hipError_t e = hipEventRecord(t->ev[slot], stream);
   if (e != hipSuccess) return int(e);
   t->ev_pending[slot] = true;
   return YAFSDP_OK;
-}
-
-TableView view_of(const yafsdp_table* t) {
-  TableView tv;
-  tv.offsets = t->d_offsets;
-  tv.tile_first = t->d_tile_first;
-  tv.total = t->total;
-  tv.padded = t->padded;
-  tv.n_tensors = t->n_tensors;
-  tv.n_tiles = t->n_tiles;
-  return tv;
 }
 
 }  // namespace
@@ -291,7 +298,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
   if (t == nullptr) return YAFSDP_ERR_OUT_OF_MEMORY;
   int rc = YAFSDP_OK;
   hipError_t e = hipSuccess;
-  std::vector<int32_t> tile_first;
+  std::vector<TileRec> tiles;
   do {
     t->n_tensors = n_tensors;
     t->offsets.assign(size_t(n_tensors) + 1, 0);
@@ -303,26 +310,36 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     t->total = t->offsets[n_tensors];
     t->padded = padded_numel;
     if (padded_numel < t->total) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
-    const int64_t n_tiles = (padded_numel + kTableTileElems - 1) / kTableTileElems;
-    if (n_tiles > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
-    t->n_tiles = int32_t(n_tiles);
-    // tile_first[tile]: first tensor whose end lies beyond the tile's first element
-    tile_first.resize(size_t(n_tiles));
-    int p = 0;
-    for (int64_t tile = 0; tile < n_tiles; tile++) {
-      const int64_t t0 = tile * kTableTileElems;
-      while (p < n_tensors && t->offsets[p + 1] <= t0) p++;
-      tile_first[size_t(tile)] = p;
+    const int64_t tile_elems[2] = {kGatherTileElems, kScatterTileElems};
+    for (int w = 0; w < 2; w++) {
+      const int64_t n_tiles = (padded_numel + tile_elems[w] - 1) / tile_elems[w];
+      if (n_tiles > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+      t->n_tiles[w] = int32_t(n_tiles);
     }
+    if (rc != YAFSDP_OK) break;
     if ((e = hipGetDevice(&t->device)) != hipSuccess) break;
     if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_offsets), t->offsets.size() * sizeof(int64_t))) != hipSuccess) break;
     if ((e = hipMemcpy(t->d_offsets, t->offsets.data(), t->offsets.size() * sizeof(int64_t), hipMemcpyHostToDevice)) != hipSuccess) break;
-    if (n_tiles > 0) {
-      if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_tile_first), tile_first.size() * sizeof(int32_t))) != hipSuccess) break;
-      if ((e = hipMemcpy(t->d_tile_first, tile_first.data(), tile_first.size() * sizeof(int32_t), hipMemcpyHostToDevice)) != hipSuccess) break;
+    for (int w = 0; w < 2 && n_tensors > kSmallMax && e == hipSuccess; w++) {
+      // per tile: first tensor whose end lies beyond the tile's first element
+      const int64_t n_tiles = t->n_tiles[w];
+      if (n_tiles == 0) continue;
+      tiles.resize(size_t(n_tiles));
+      int p = 0;
+      for (int64_t tile = 0; tile < n_tiles; tile++) {
+        const int64_t t0 = tile * tile_elems[w];
+        while (p < n_tensors && t->offsets[p + 1] <= t0) p++;
+        TileRec& r = tiles[size_t(tile)];
+        r.first = p;
+        r.full = (p < n_tensors && t->offsets[p + 1] - t0 >= tile_elems[w]) ? 1 : 0;
+        r.delta = p < n_tensors ? t0 - t->offsets[p] : 0;
+      }
+      if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_tiles[w]), tiles.size() * sizeof(TileRec))) != hipSuccess) break;
+      if ((e = hipMemcpy(t->d_tiles[w], tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
     }
-    if (n_tensors > kKargMax) {
-      t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + 1) + 15) & ~size_t(15);
+    if (e != hipSuccess) break;
+    if (n_tensors > kSmallMax) {
+      t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
       for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
         if ((e = hipHostMalloc(reinterpret_cast<void**>(&t->h_stage[i]), t->stage_bytes, hipHostMallocDefault)) != hipSuccess) break;
         if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_stage[i]), t->stage_bytes)) != hipSuccess) break;
@@ -375,15 +392,25 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   float k;
   scale_plan(pre_factor, &scale, &k);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  std::lock_guard<std::mutex> lock(table->mu);
-  DynArgs dyn;
-  int slot;
-  int rc = prepare_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype), &dyn, &slot, s);
+  int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
-  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  e = launch_gather(tensor_dtype, flat_dtype, scale, view_of(table), dyn, flat, k, zero_pad ? 1 : 0, grid, s);
+  const int n_tiles = table->n_tiles[0];
+  const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  if (table->n_tensors <= kSmallMax) {
+    SmallMeta meta;
+    fill_small(table, tensor_ptrs, mode, kGatherTileElems, &meta);
+    return int(launch_gather<SmallMeta>(tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
+                                        zero_pad ? 1 : 0, grid, s));
+  }
+  std::lock_guard<std::mutex> lock(table->mu);
+  LargeMeta meta;
+  int slot = -1;
+  rc = stage_large(table, tensor_ptrs, mode, 0, &meta, &slot, s);
+  if (rc != YAFSDP_OK) return rc;
+  e = launch_gather<LargeMeta>(tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
+                               zero_pad ? 1 : 0, grid, s);
   if (e != hipSuccess) return int(e);
-  return finish_dyn(table, slot, s);
+  return finish_large(table, slot, s);
 }
 
 int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
@@ -398,15 +425,24 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   if (e != hipSuccess) return int(e);
   if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  std::lock_guard<std::mutex> lock(table->mu);
-  DynArgs dyn;
-  int slot;
-  int rc = prepare_dyn(table, const_cast<const void* const*>(tensor_ptrs), mode, item_size(tensor_dtype), &dyn, &slot, s);
+  const void* const* ptrs = const_cast<const void* const*>(tensor_ptrs);
+  int rc = check_dyn(table, ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
-  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  e = launch_scatter(flat_dtype, tensor_dtype, view_of(table), dyn, flat, grid, s);
+  const int n_tiles = table->n_tiles[1];
+  const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  if (table->n_tensors <= kSmallMax) {
+    SmallMeta meta;
+    fill_small(table, ptrs, mode, kScatterTileElems, &meta);
+    return int(launch_scatter<SmallMeta>(flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s));
+  }
+  std::lock_guard<std::mutex> lock(table->mu);
+  LargeMeta meta;
+  int slot = -1;
+  rc = stage_large(table, ptrs, mode, 1, &meta, &slot, s);
+  if (rc != YAFSDP_OK) return rc;
+  e = launch_scatter<LargeMeta>(flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s);
   if (e != hipSuccess) return int(e);
-  return finish_dyn(table, slot, s);
+  return finish_large(table, slot, s);
 }
 
 }  // extern "C"

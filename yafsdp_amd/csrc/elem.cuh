@@ -27,10 +27,14 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 // the HSA runtime executes dwordx4 accesses at such addresses natively
 typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
 typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x2 u32x2_a2 __attribute__((aligned(2)));
 
 struct F32 {
   typedef float storage;
   typedef u32x4_a4 vec_unaligned;
+  typedef u32x4 quad;               // 4 elements
+  typedef u32x4_a4 quad_unaligned;
   static constexpr int kId = DT_F32;
   static constexpr int kSize = 4;
   static constexpr int kVecs = 2;  // dwordx4 accesses per unit
@@ -38,6 +42,8 @@ struct F32 {
 struct BF16 {
   typedef uint16_t storage;
   typedef u32x4_a2 vec_unaligned;
+  typedef u32x2 quad;
+  typedef u32x2_a2 quad_unaligned;
   static constexpr int kId = DT_BF16;
   static constexpr int kSize = 2;
   static constexpr int kVecs = 1;
@@ -45,6 +51,8 @@ struct BF16 {
 struct F16 {
   typedef uint16_t storage;
   typedef u32x4_a2 vec_unaligned;
+  typedef u32x2 quad;
+  typedef u32x2_a2 quad_unaligned;
   static constexpr int kId = DT_F16;
   static constexpr int kSize = 2;
   static constexpr int kVecs = 1;
@@ -154,6 +162,88 @@ __device__ __forceinline__ Unit<T> pack(const float (&f)[8]) {
     }
   }
   return u;
+}
+
+// ---- quads: 4 consecutive elements --------------------------------------------
+// Used when one side of a pair is fp32: lane l of a wave then owns elements
+// 4l..4l+3 and 256+4l..256+4l+3 of a 512-element wave tile, so that every
+// access instruction of the wave covers one contiguous span (64 x 16 bytes of
+// fp32, 64 x 8 bytes of a 2-byte dtype) made of whole cache lines.  With 8
+// consecutive fp32 elements per lane instead, each dwordx4 instruction would
+// touch only every other 16 bytes of the span.
+template <class T>
+struct Quad { typename T::quad v; };
+
+template <class T, bool NT>
+__device__ __forceinline__ Quad<T> load_quad(const void* p) {
+  Quad<T> r;
+  const typename T::quad_unaligned* q = reinterpret_cast<const typename T::quad_unaligned*>(p);
+  if constexpr (NT) r.v = __builtin_nontemporal_load(q);
+  else r.v = *q;
+  return r;
+}
+
+template <class T, bool NT>
+__device__ __forceinline__ void store_quad(void* p, const Quad<T>& u) {
+  typename T::quad_unaligned* q = reinterpret_cast<typename T::quad_unaligned*>(p);
+  if constexpr (NT) __builtin_nontemporal_store(u.v, q);
+  else *q = u.v;
+}
+
+template <class T>
+__device__ __forceinline__ void unpack_quad(const Quad<T>& u, float (&f)[4]) {
+  if constexpr (same_t<T, F32>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) f[i] = bits_to_f32(u.v[i]);
+  } else if constexpr (same_t<T, BF16>::value) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const uint32_t w = u.v[i];
+      f[2 * i] = bits_to_f32(w << 16);
+      f[2 * i + 1] = bits_to_f32(w & 0xFFFF0000u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const uint32_t w = u.v[i];
+      f[2 * i] = (float)__builtin_bit_cast(_Float16, uint16_t(w & 0xFFFFu));
+      f[2 * i + 1] = (float)__builtin_bit_cast(_Float16, uint16_t(w >> 16));
+    }
+  }
+}
+
+template <class T>
+__device__ __forceinline__ Quad<T> pack_quad(const float (&f)[4]) {
+  Quad<T> u;
+  if constexpr (same_t<T, F32>::value) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) u.v[i] = f32_to_bits(f[i]);
+  } else if constexpr (same_t<T, BF16>::value) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      f32x2 x = {f[2 * i], f[2 * i + 1]};
+      u.v[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      f32x2 x = {f[2 * i], f[2 * i + 1]};
+      u.v[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+    }
+  }
+  return u;
+}
+
+// a pair of dtypes takes the quad arrangement when either side is fp32
+template <class S, class D>
+struct wide_pair { static constexpr bool value = (S::kSize == 4 || D::kSize == 4); };
+
+// byte-free element index of quad q (0 .. 2U-1) of this lane inside a tile of
+// BLOCK*U units: wave tiles of 512 elements, two quads per lane per wave tile
+template <int BLOCK>
+__device__ __forceinline__ int quad_elem(int q) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  return ((q >> 1) * (BLOCK / 64) + wave) * 512 + (q & 1) * 256 + lane * 4;
 }
 
 // ---- the arithmetic -----------------------------------------------------------

@@ -4,12 +4,15 @@
 // gradient shard).
 //
 // Work partitioning: the range is cut into tiles of BLOCK*U units (a unit is 8
-// elements); a workgroup walks tiles with a grid stride; inside a tile lane l of
-// the workgroup touches units l, l+BLOCK, ... so that every wave64 access is one
-// contiguous 1 KiB (2-byte dtypes) or 2 KiB (fp32) span.  All U loads of a lane
-// are issued before the first store.  The destination is 16-byte aligned for
-// the unit loop (the host peels up to 7 leading elements, handled by workgroup 0
-// together with the tail); the source may sit at any element-aligned address.
+// elements), one workgroup per tile (grid-stride if the grid is capped).
+//  * pairs of 2-byte dtypes: lane l touches units l, l+BLOCK, ...: every wave64
+//    access is one contiguous 1 KiB span;
+//  * pairs with an fp32 side: quad arrangement (see elem.cuh): every wave64
+//    access is a contiguous 1 KiB (fp32) or 512 B (2-byte) span.
+// All loads of a lane are issued before its first store.  The destination is
+// 16-byte aligned for the tile loop (the host peels up to 7 leading elements,
+// handled by workgroup 0 together with the tail); the source may sit at any
+// element-aligned address.
 #pragma once
 #include "elem.cuh"
 
@@ -43,6 +46,51 @@ __device__ __forceinline__ Unit<D> flat_unit(const Unit<S>& s, const Unit<D>& d_
   }
 }
 
+template <class S, class D, int SCALE, bool ACC>
+__device__ __forceinline__ Quad<D> flat_quad(const Quad<S>& s, const Quad<D>& d_old, float k) {
+  if constexpr (same_t<S, D>::value && SCALE == SCALE_NONE && !ACC) {
+    return s;
+  } else {
+    float fs[4], fd[4], fy[4];
+    unpack_quad<S>(s, fs);
+    if constexpr (ACC) unpack_quad<D>(d_old, fd);
+#pragma unroll
+    for (int e = 0; e < 4; e++) fy[e] = post_elem<S, D, SCALE, ACC>(fs[e], ACC ? fd[e] : 0.f, k);
+    return pack_quad<D>(fy);
+  }
+}
+
+// One full tile (BLOCK*U units) at dst/src; dst 16-byte aligned.
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
+__device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float k) {
+  if constexpr (wide_pair<S, D>::value) {
+    Quad<S> s[2 * U];
+    Quad<D> d[2 * U];
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK>(q) * S::kSize);
+    if constexpr (ACC) {
+#pragma unroll
+      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dst + quad_elem<BLOCK>(q) * D::kSize);
+    }
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++)
+      store_quad<D, NTS>(dst + quad_elem<BLOCK>(q) * D::kSize, flat_quad<S, D, SCALE, ACC>(s[q], d[q], k));
+  } else {
+    const int tid = threadIdx.x;
+    Unit<S> s[U];
+    Unit<D> d[U];
+#pragma unroll
+    for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + (tid + j * BLOCK) * (8 * S::kSize));
+    if constexpr (ACC) {
+#pragma unroll
+      for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dst + (tid + j * BLOCK) * (8 * D::kSize));
+    }
+#pragma unroll
+    for (int j = 0; j < U; j++)
+      store_unit<D, NTS>(dst + (tid + j * BLOCK) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
+  }
+}
+
 // dst[i] = op(src[i], dst[i]) for i in [0, n).  `head` leading elements bring
 // dst to a 16-byte boundary.  dst == src is allowed (in-place divide).
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
@@ -62,32 +110,15 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
   constexpr int64_t kTile = int64_t(BLOCK) * U;
   const int64_t n_tiles = (n_units + kTile - 1) / kTile;
   for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-    const int64_t u0 = tile * kTile + tid;
-    Unit<S> s[U];
-    Unit<D> d[U];
     if (tile * kTile + kTile <= n_units) {
-#pragma unroll
-      for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(sbase + (u0 + int64_t(j) * BLOCK) * (8 * S::kSize));
-      if constexpr (ACC) {
-#pragma unroll
-        for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dbase + (u0 + int64_t(j) * BLOCK) * (8 * D::kSize));
-      }
-#pragma unroll
-      for (int j = 0; j < U; j++)
-        store_unit<D, NTS>(dbase + (u0 + int64_t(j) * BLOCK) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
-    } else {
-#pragma unroll
-      for (int j = 0; j < U; j++) {
-        const int64_t u = u0 + int64_t(j) * BLOCK;
-        if (u < n_units) {
-          s[j] = load_unit<S, NTL>(sbase + u * (8 * S::kSize));
-          if constexpr (ACC) d[j] = load_unit<D, NTL>(dbase + u * (8 * D::kSize));
-        }
-      }
-#pragma unroll
-      for (int j = 0; j < U; j++) {
-        const int64_t u = u0 + int64_t(j) * BLOCK;
-        if (u < n_units) store_unit<D, NTS>(dbase + u * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
+      flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, NTS>(dbase + tile * kTile * (8 * D::kSize),
+                                                           sbase + tile * kTile * (8 * S::kSize), k);
+    } else {  // last, partial tile
+      for (int64_t u = tile * kTile + tid; u < n_units; u += BLOCK) {
+        Unit<S> s = load_unit<S, NTL>(sbase + u * (8 * S::kSize));
+        Unit<D> d;
+        if constexpr (ACC) d = load_unit<D, NTL>(dbase + u * (8 * D::kSize));
+        store_unit<D, NTS>(dbase + u * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s, d, k));
       }
     }
   }

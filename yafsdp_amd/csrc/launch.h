@@ -11,9 +11,13 @@ namespace yafsdp {
 // dst[i] = post_elem(src[i], dst[i]); scale is SCALE_NONE / SCALE_MUL / SCALE_DIV
 hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,
                        float k, int grid, hipStream_t stream);
-hipError_t launch_gather(int tensor_dt, int flat_dt, int scale, const TableView& tv, const DynArgs& dyn, void* flat,
-                         float k, int pad_zero, int grid, hipStream_t stream);
-hipError_t launch_scatter(int flat_dt, int tensor_dt, const TableView& tv, const DynArgs& dyn, const void* flat,
+
+// META is SmallMeta or LargeMeta (explicitly instantiated in gather.hip / scatter.hip)
+template <class META>
+hipError_t launch_gather(int tensor_dt, int flat_dt, int scale, const META& meta, void* flat, int64_t padded,
+                         int n_tiles, float k, int pad_zero, int grid, hipStream_t stream);
+template <class META>
+hipError_t launch_scatter(int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total, int n_tiles,
                           int grid, hipStream_t stream);
 
 }  // namespace yafsdp

@@ -5,34 +5,38 @@
 namespace yafsdp {
 namespace {
 
-template <class S, class D>
-hipError_t go(const TableView& tv, const DynArgs& dyn, const void* flat, int grid, hipStream_t stream) {
-  scatter_out_kernel<S, D, kTableBlock, kTableUnroll, kTableNtLoad, kTableNtStore>
-      <<<dim3(grid), dim3(kTableBlock), 0, stream>>>(tv, dyn, flat);
+template <class META, class S, class D>
+hipError_t go(const META& meta, const void* flat, int64_t total, int n_tiles, int grid, hipStream_t stream) {
+  scatter_out_kernel<META, S, D, kTableBlock, kScatterUnroll, kTableNtLoad, kTableNtStore>
+      <<<dim3(grid), dim3(kTableBlock), 0, stream>>>(meta, flat, total, n_tiles);
   return hipGetLastError();
 }
 
-template <class S>
-hipError_t by_tensor(int tensor_dt, const TableView& tv, const DynArgs& dyn, const void* flat, int grid,
+template <class META, class S>
+hipError_t by_tensor(int tensor_dt, const META& meta, const void* flat, int64_t total, int n_tiles, int grid,
                      hipStream_t stream) {
   switch (tensor_dt) {
-    case DT_F32: return go<S, F32>(tv, dyn, flat, grid, stream);
-    case DT_BF16: return go<S, BF16>(tv, dyn, flat, grid, stream);
-    case DT_F16: return go<S, F16>(tv, dyn, flat, grid, stream);
+    case DT_F32: return go<META, S, F32>(meta, flat, total, n_tiles, grid, stream);
+    case DT_BF16: return go<META, S, BF16>(meta, flat, total, n_tiles, grid, stream);
+    case DT_F16: return go<META, S, F16>(meta, flat, total, n_tiles, grid, stream);
   }
   return hipErrorInvalidValue;
 }
 
 }  // namespace
 
-hipError_t launch_scatter(int flat_dt, int tensor_dt, const TableView& tv, const DynArgs& dyn, const void* flat,
+template <class META>
+hipError_t launch_scatter(int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total, int n_tiles,
                           int grid, hipStream_t stream) {
   switch (flat_dt) {
-    case DT_F32: return by_tensor<F32>(tensor_dt, tv, dyn, flat, grid, stream);
-    case DT_BF16: return by_tensor<BF16>(tensor_dt, tv, dyn, flat, grid, stream);
-    case DT_F16: return by_tensor<F16>(tensor_dt, tv, dyn, flat, grid, stream);
+    case DT_F32: return by_tensor<META, F32>(tensor_dt, meta, flat, total, n_tiles, grid, stream);
+    case DT_BF16: return by_tensor<META, BF16>(tensor_dt, meta, flat, total, n_tiles, grid, stream);
+    case DT_F16: return by_tensor<META, F16>(tensor_dt, meta, flat, total, n_tiles, grid, stream);
   }
   return hipErrorInvalidValue;
 }
+
+template hipError_t launch_scatter<SmallMeta>(int, int, const SmallMeta&, const void*, int64_t, int, int, hipStream_t);
+template hipError_t launch_scatter<LargeMeta>(int, int, const LargeMeta&, const void*, int64_t, int, int, hipStream_t);
 
 }  // namespace yafsdp

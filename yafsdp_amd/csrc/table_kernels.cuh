@@ -3,51 +3,105 @@
 //               absent per tensor, fused pre-divide, pad zero-fill)
 //   scatter-out flat gathered buffer -> P tensors   (materialising copy-out)
 //
-// The flat buffer is cut into tiles of BLOCK*U units (a unit is 8 elements).
-// `tile_first[t]` names the tensor that holds the tile's first element (the
-// first tensor whose end lies beyond it; n_tensors when the tile starts in the
-// pad), so a workgroup finds its work with one table read instead of a search.
-// A tile that lies wholly inside one tensor takes the unrolled path: U
-// dwordx4-wide loads per lane in flight, flat side 16-byte aligned, tensor side
-// at whatever element-aligned address the ragged offset gives.  A tile that
-// crosses tensor boundaries (or the end of the buffer) walks its segments; each
-// segment peels up to 7 elements on either end so that its unit loop is again
-// aligned on the flat side.
+// The flat buffer is cut into tiles of BLOCK*U units (a unit is 8 elements),
+// one workgroup per tile.  A workgroup first learns which tensor holds the
+// tile's first element (the first tensor whose end lies beyond it; n_tensors
+// when the tile starts in the pad), whether the whole tile lies inside that
+// tensor, and the tile's element offset inside it.
+// A tile that lies wholly inside one tensor takes the unrolled path: all loads
+// of a lane in flight before its first store, flat side 16-byte aligned, tensor
+// side at whatever element-aligned address the ragged offset gives.  A tile
+// that crosses tensor boundaries (or the end of the buffer) walks its segments;
+// each segment peels up to 7 elements on either end so that its unit loop is
+// again aligned on the flat side.
 //
-// Tensor base pointers and per-tensor modes change every call (autograd
-// allocates gradients afresh), so they travel outside the static table: in the
-// kernel arguments for up to kKargMax tensors, else through a small device
-// array the host refreshes on the same stream before the launch.
+// Metadata reaches a workgroup through scalar loads only (one tile is one
+// wave-uniform lookup), by one of two routes:
+//  * SmallMeta (up to kSmallMax tensors, e.g. one decoder layer): tensor
+//    pointers, modes, prefix offsets and each tensor's first tile travel in the
+//    kernel arguments; the tile -> tensor search is a handful of scalar compares
+//    and nothing is read from global memory before the data itself.
+//  * LargeMeta: the static part (prefix offsets, one 16-byte record per tile:
+//    first tensor, whole-tile flag, offset inside that tensor) is device
+//    resident and built once per table; the per-call part (tensor pointers and
+//    modes, which change every call because autograd allocates gradients
+//    afresh) is refreshed by the host on the same stream before the launch.
+//    All of it is read through the constant address space, i.e. as scalar loads.
 #pragma once
 #include "flat_kernels.cuh"
 
 namespace yafsdp {
 
-constexpr int kKargMax = 32;
+constexpr int kSmallMax = 16;
 enum : int { MODE_ZERO = 3 };  // internal: fill with zeros (pad lanes)
 
-struct DynArgs {
-  const void* ptr[kKargMax];
-  uint8_t mode[kKargMax];
-  const void* const* dev_ptr;  // non-null when the table has more than kKargMax tensors
-  const uint8_t* dev_mode;
+struct TileRec {
+  int32_t first;  // tensor holding the tile's first element, n_tensors if in the pad
+  int32_t full;   // 1 when the whole tile lies inside tensor `first`
+  int64_t delta;  // tile start minus start of tensor `first` (elements)
 };
 
-struct TableView {
-  const int64_t* offsets;     // n_tensors + 1 prefix offsets (elements), offsets[n_tensors] == total
-  const int32_t* tile_first;  // n_tiles entries
-  int64_t total;              // T
-  int64_t padded;             // T_pad
+struct TileLookup {
+  int first;
+  bool full;
+  int64_t delta;
+};
+
+#define YAFSDP_CONST_AS __attribute__((address_space(4)))
+
+struct SmallMeta {
+  const void* ptr[kSmallMax];
+  int64_t off[kSmallMax + 1];         // prefix offsets; entries past n_tensors repeat the total
+  int32_t tile_start[kSmallMax + 1];  // ceil(off[i] / tile elements); INT32_MAX past n_tensors
+  uint32_t modes;                     // 2 bits per tensor
   int32_t n_tensors;
-  int32_t n_tiles;
+
+  __device__ __forceinline__ TileLookup lookup(int tile, int64_t t0, int64_t tile_elems) const {
+    int p = 0;
+#pragma unroll
+    for (int i = 1; i <= kSmallMax; i++) p += (tile_start[i] <= tile) ? 1 : 0;
+    TileLookup r;
+    r.first = p;
+    const int64_t o0 = off[p];
+    const int64_t o1 = off[p < kSmallMax ? p + 1 : kSmallMax];
+    r.full = p < n_tensors && (o1 - t0 >= tile_elems);
+    r.delta = t0 - o0;
+    return r;
+  }
+  __device__ __forceinline__ const void* tensor(int p) const { return ptr[p]; }
+  __device__ __forceinline__ int mode(int p) const { return int((modes >> (2 * p)) & 3u); }
+  __device__ __forceinline__ int64_t offset(int p) const { return off[p]; }
 };
 
-__device__ __forceinline__ const void* dyn_ptr(const DynArgs& a, int p) {
-  return a.dev_ptr != nullptr ? a.dev_ptr[p] : a.ptr[p];
-}
-__device__ __forceinline__ int dyn_mode(const DynArgs& a, int p) {
-  return a.dev_ptr != nullptr ? a.dev_mode[p] : a.mode[p];
-}
+struct LargeMeta {
+  const int64_t* offsets;    // n_tensors + 1 prefix offsets (elements)
+  const TileRec* tiles;      // n_tiles records
+  const void* const* ptrs;   // n_tensors device pointers (per call)
+  const uint32_t* modes_;    // n_tensors modes (per call)
+  int32_t n_tensors;
+
+  __device__ __forceinline__ TileLookup lookup(int tile, int64_t, int64_t) const {
+    typedef const TileRec YAFSDP_CONST_AS* cptr;
+    const cptr t = (cptr)(uintptr_t)tiles;
+    TileLookup r;
+    r.first = t[tile].first;
+    r.full = t[tile].full != 0;
+    r.delta = t[tile].delta;
+    return r;
+  }
+  __device__ __forceinline__ const void* tensor(int p) const {
+    typedef const void* const YAFSDP_CONST_AS* cptr;
+    return ((cptr)(uintptr_t)ptrs)[p];
+  }
+  __device__ __forceinline__ int mode(int p) const {
+    typedef const uint32_t YAFSDP_CONST_AS* cptr;
+    return int(((cptr)(uintptr_t)modes_)[p]);
+  }
+  __device__ __forceinline__ int64_t offset(int p) const {
+    typedef const int64_t YAFSDP_CONST_AS* cptr;
+    return ((cptr)(uintptr_t)offsets)[p];
+  }
+};
 
 // ------------------------------------------------------------------ gather-in --
 template <class S, class D, int SCALE, int MODE>
@@ -87,10 +141,41 @@ __device__ __forceinline__ Unit<D> gather_unit(const Unit<S>& s, const Unit<D>& 
   }
 }
 
+template <class S, class D, int SCALE, int MODE>
+__device__ __forceinline__ Quad<D> gather_quad(const Quad<S>& s, const Quad<D>& d_old, float k) {
+  if constexpr (MODE == MODE_COPY && same_t<S, D>::value && SCALE == SCALE_NONE) {
+    return s;
+  } else {
+    float fs[4], fd[4], fy[4];
+    if constexpr (MODE != MODE_SKIP) unpack_quad<S>(s, fs);
+    if constexpr (MODE != MODE_COPY) unpack_quad<D>(d_old, fd);
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      fy[e] = gather_elem<S, D, SCALE, MODE>(MODE != MODE_SKIP ? fs[e] : 0.f, MODE != MODE_COPY ? fd[e] : 0.f, k);
+    return pack_quad<D>(fy);
+  }
+}
+
 template <class S, class D, int SCALE, int MODE, int BLOCK, int U, bool NTL, bool NTS>
 __device__ __forceinline__ void gather_full_tile(char* dst, const char* src, float k) {
   constexpr bool kReadSrc = (MODE == MODE_COPY || MODE == MODE_ADD);
   constexpr bool kReadDst = (MODE == MODE_ADD || MODE == MODE_SKIP);
+  if constexpr (wide_pair<S, D>::value) {
+    Quad<S> s[2 * U];
+    Quad<D> d[2 * U];
+    if constexpr (kReadSrc) {
+#pragma unroll
+      for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK>(q) * S::kSize);
+    }
+    if constexpr (kReadDst) {
+#pragma unroll
+      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dst + quad_elem<BLOCK>(q) * D::kSize);
+    }
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++)
+      store_quad<D, NTS>(dst + quad_elem<BLOCK>(q) * D::kSize, gather_quad<S, D, SCALE, MODE>(s[q], d[q], k));
+    return;
+  }
   const int tid = threadIdx.x;
   Unit<S> s[U];
   Unit<D> d[U];
@@ -136,42 +221,39 @@ __device__ __forceinline__ void gather_segment(char* dst, const char* src, int64
 // S: tensor dtype, D: flat buffer dtype.  pad_zero != 0 writes zeros to
 // [total, padded); otherwise pad lanes only see the divide (as in the
 // reference, whose pad content is whatever the buffer held).
-template <class S, class D, int SCALE, int BLOCK, int U, bool NTL, bool NTS>
+template <class META, class S, class D, int SCALE, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
-gather_in_kernel(TableView tv, DynArgs dyn, void* flat, float k, int pad_zero) {
+gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   char* fbase = reinterpret_cast<char*>(flat);
-  for (int tile = blockIdx.x; tile < tv.n_tiles; tile += gridDim.x) {
+  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     const int64_t t0 = int64_t(tile) * kTile;
-    const int64_t t1 = (t0 + kTile < tv.padded) ? t0 + kTile : tv.padded;
-    int p = tv.tile_first[tile];
-    if (p < tv.n_tensors) {
-      const int64_t o0 = tv.offsets[p];
-      const int64_t o1 = tv.offsets[p + 1];
-      if (o1 - t0 >= kTile) {  // the whole tile lies inside tensor p
-        const int mode = dyn_mode(dyn, p);
-        const char* src = reinterpret_cast<const char*>(dyn_ptr(dyn, p)) + (t0 - o0) * S::kSize;
-        char* dst = fbase + t0 * D::kSize;
-        if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, NTS>(dst, src, k);
-        else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, NTS>(dst, src, k);
-        else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, NTS>(dst, src, k);
-        continue;
-      }
+    const int64_t t1 = (t0 + kTile < padded) ? t0 + kTile : padded;
+    const TileLookup rec = meta.lookup(tile, t0, kTile);
+    int p = rec.first;
+    if (rec.full) {  // the whole tile lies inside tensor p
+      const int mode = meta.mode(p);
+      const char* src = reinterpret_cast<const char*>(meta.tensor(p)) + rec.delta * S::kSize;
+      char* dst = fbase + t0 * D::kSize;
+      if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, NTS>(dst, src, k);
+      else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, NTS>(dst, src, k);
+      else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, NTS>(dst, src, k);
+      continue;
     }
     int64_t pos = t0;
     while (pos < t1) {
-      if (p >= tv.n_tensors) {  // pad lanes
+      if (p >= meta.n_tensors) {  // pad lanes
         char* dst = fbase + pos * D::kSize;
         if (pad_zero) gather_segment<S, D, SCALE, MODE_ZERO, BLOCK, NTL, NTS>(dst, nullptr, t1 - pos, pos, k);
         else if (SCALE != SCALE_NONE) gather_segment<S, D, SCALE, MODE_SKIP, BLOCK, NTL, NTS>(dst, nullptr, t1 - pos, pos, k);
         break;
       }
-      const int64_t o1 = tv.offsets[p + 1];
+      const int64_t o1 = meta.offset(p + 1);
       if (o1 <= pos) { ++p; continue; }  // empty tensor
-      const int64_t o0 = tv.offsets[p];
+      const int64_t o0 = meta.offset(p);
       const int64_t e = o1 < t1 ? o1 : t1;
-      const int mode = dyn_mode(dyn, p);
-      const char* src = reinterpret_cast<const char*>(dyn_ptr(dyn, p)) + (pos - o0) * S::kSize;
+      const int mode = meta.mode(p);
+      const char* src = reinterpret_cast<const char*>(meta.tensor(p)) + (pos - o0) * S::kSize;
       char* dst = fbase + pos * D::kSize;
       if (mode == MODE_COPY) gather_segment<S, D, SCALE, MODE_COPY, BLOCK, NTL, NTS>(dst, src, e - pos, pos, k);
       else if (mode == MODE_ADD) gather_segment<S, D, SCALE, MODE_ADD, BLOCK, NTL, NTS>(dst, src, e - pos, pos, k);
@@ -185,6 +267,16 @@ gather_in_kernel(TableView tv, DynArgs dyn, void* flat, float k, int pad_zero) {
 // ---------------------------------------------------------------- scatter-out --
 template <class S, class D, int BLOCK, int U, bool NTL, bool NTS>
 __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
+  if constexpr (wide_pair<S, D>::value) {
+    Quad<S> s[2 * U];
+    Quad<D> unused_q;
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK>(q) * S::kSize);
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++)
+      store_quad<D, NTS>(dst + quad_elem<BLOCK>(q) * D::kSize, flat_quad<S, D, SCALE_NONE, false>(s[q], unused_q, 0.f));
+    return;
+  }
   const int tid = threadIdx.x;
   Unit<S> s[U];
   Unit<D> unused;
@@ -216,35 +308,33 @@ __device__ __forceinline__ void scatter_segment(char* dst, const char* src, int6
 }
 
 // S: flat buffer dtype, D: tensor dtype.  Tensors with mode 0 are not written.
-template <class S, class D, int BLOCK, int U, bool NTL, bool NTS>
+template <class META, class S, class D, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
-scatter_out_kernel(TableView tv, DynArgs dyn, const void* flat) {
+scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   const char* fbase = reinterpret_cast<const char*>(flat);
-  for (int tile = blockIdx.x; tile < tv.n_tiles; tile += gridDim.x) {
+  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     const int64_t t0 = int64_t(tile) * kTile;
-    const int64_t t1 = (t0 + kTile < tv.total) ? t0 + kTile : tv.total;  // pad lanes are never read
-    int p = tv.tile_first[tile];
-    if (p >= tv.n_tensors) continue;
-    {
-      const int64_t o0 = tv.offsets[p];
-      const int64_t o1 = tv.offsets[p + 1];
-      if (o1 - t0 >= kTile) {
-        if (dyn_mode(dyn, p) != MODE_SKIP) {
-          char* dst = reinterpret_cast<char*>(const_cast<void*>(dyn_ptr(dyn, p))) + (t0 - o0) * D::kSize;
-          scatter_full_tile<S, D, BLOCK, U, NTL, NTS>(dst, fbase + t0 * S::kSize);
-        }
-        continue;
+    if (t0 >= total) break;  // pad lanes are never read
+    const int64_t t1 = (t0 + kTile < total) ? t0 + kTile : total;
+    const TileLookup rec = meta.lookup(tile, t0, kTile);
+    int p = rec.first;
+    if (p >= meta.n_tensors) continue;
+    if (rec.full) {
+      if (meta.mode(p) != MODE_SKIP) {
+        char* dst = reinterpret_cast<char*>(const_cast<void*>(meta.tensor(p))) + rec.delta * D::kSize;
+        scatter_full_tile<S, D, BLOCK, U, NTL, NTS>(dst, fbase + t0 * S::kSize);
       }
+      continue;
     }
     int64_t pos = t0;
-    while (pos < t1 && p < tv.n_tensors) {
-      const int64_t o1 = tv.offsets[p + 1];
+    while (pos < t1 && p < meta.n_tensors) {
+      const int64_t o1 = meta.offset(p + 1);
       if (o1 <= pos) { ++p; continue; }
-      const int64_t o0 = tv.offsets[p];
+      const int64_t o0 = meta.offset(p);
       const int64_t e = o1 < t1 ? o1 : t1;
-      if (dyn_mode(dyn, p) != MODE_SKIP) {
-        char* dst = reinterpret_cast<char*>(const_cast<void*>(dyn_ptr(dyn, p))) + (pos - o0) * D::kSize;
+      if (meta.mode(p) != MODE_SKIP) {
+        char* dst = reinterpret_cast<char*>(const_cast<void*>(meta.tensor(p))) + (pos - o0) * D::kSize;
         scatter_segment<S, D, BLOCK, NTL, NTS>(dst, fbase + pos * S::kSize, e - pos, pos);
       }
       pos = e;
