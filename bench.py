@@ -41,9 +41,11 @@ WORKLOADS = {
         [(512, 512)] * 4 + [(1376, 512), (1376, 512), (512, 1376), (512,), (512,)], 1, 0, 512, 1001),
 }
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
-# (see profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch of the dominant kernel (gather_in_kernel), from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
+# (factors 1.99988 and 0.99986): (213037.875 * 1.99988 + 426022.75 * 0.99986) KiB.
+# Summary and commands: profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_461_600}
 
 
 def log(*a):
@@ -65,6 +67,9 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3-8b-layer-w8", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
+                    help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
+                         "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -173,6 +178,13 @@ def main() -> int:
         if not ok:
             log("bench.py: GPU results differ from the oracle; refusing to report a throughput.")
             return 4
+
+    if args.calibrate_copy > 0:
+        d_copy = torch.empty(t_pad, dtype=torch.bfloat16, device=dev)
+        for _ in range(args.calibrate_copy):
+            _native.flat_copy(d_copy, d_gathered)
+        torch.cuda.synchronize()
+        del d_copy
 
     # ---- timed region
     for _ in range(args.warmup):
