@@ -70,6 +70,14 @@ int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, i
  * 270-272). */
 int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream);
 
+/* dst[i] = cast_dst(round_src(src[i] / divisor)), for ANY finite non-zero
+ * divisor (no "> 1" rule): the out-of-place divide of the size-1-group branch
+ * with a custom factor,
+ *   output_tensor.copy_(padded_unsharded_param_grad / gradient_divide_factor)
+ * (ya_fsdp/_collectives.py:141-148).  dst == src with equal dtypes is allowed. */
+int yafsdp_flat_div_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, double divisor,
+                         void* stream);
+
 /* Fused post-reduce on the rank's chunk of the reduce buffer:
  *   t = chunk[i];  if (post_factor > 1) t = round_chunk_dtype(t / post_factor);
  *   shard[i] = round_shard_dtype(accumulate ? shard[i] + t : t)

@@ -1,0 +1,317 @@
+"""Parameter-group level parity on the GPU: layout, views, stream/event
+protocol and the full unshard -> backward -> reduce flow against the
+reference's torch-op sequence (oracle.torch_ops) on CPU, bit for bit."""
+
+import pytest
+import torch
+
+from oracle import torch_ops
+from tests.helpers import assert_bits_equal
+from yafsdp_amd import FSDPMeshInfo, MixedPrecisionPolicy, make_layout
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+TINY_SHAPES = [(512, 512)] * 4 + [(1376, 512), (1376, 512), (512, 1376), (512,), (512,)]
+ODD_SHAPES = [(7, 13), (1,), (129, 3), (5,), (64, 33), (2, 2, 2), (1000,), (3,)]
+
+
+def _params(shapes, dtype, seed, norms_are_ones=True):
+    g = torch.Generator().manual_seed(seed)
+    out = []
+    for s in shapes:
+        if len(s) == 1 and norms_are_ones and s[0] >= 512:
+            out.append(torch.ones(s, dtype=dtype))
+        else:
+            out.append((torch.randn(s, generator=g) * 0.02).to(dtype))
+    return out
+
+
+def _grads(shapes, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(s, generator=g) * 1e-3).to(dtype) for s in shapes]
+
+
+def _make_group(shapes, w, r, align, mp, master_dtype=torch.float32, seed=1):
+    from yafsdp_amd._param_group import YaFSDPParamGroup, init_shared_state
+
+    cpu_params = _params(shapes, master_dtype, seed)
+    dev_params = [p.to(DEV).requires_grad_(True) for p in cpu_params]
+    group = YaFSDPParamGroup(dev_params, FSDPMeshInfo(w, r), DEV, mp, align)
+    init_shared_state([group], DEV)
+    return group, cpu_params
+
+
+class CpuGroup:
+    """The reference's op sequence for one group on CPU tensors (zero-filled
+    buffers so that pad lanes are defined)."""
+
+    def __init__(self, cpu_params, w, r, align, mp):
+        self.w, self.r = w, r
+        self.numels = [p.numel() for p in cpu_params]
+        self.sizes = [tuple(p.shape) for p in cpu_params]
+        self.lay = make_layout(self.numels, w, align)
+        orig = cpu_params[0].dtype
+        self.param_dtype = None if mp.param_dtype in (None, orig) else mp.param_dtype
+        reduce_dtype = None if mp.reduce_dtype == mp.param_dtype else mp.reduce_dtype
+        self.ag_dtype = self.param_dtype or orig
+        self.rs_dtype = reduce_dtype or self.param_dtype or orig
+        t, t_pad, s = self.lay.total_numel, self.lay.padded_unsharded_numel, self.lay.padded_sharded_numel
+        flat = torch.zeros(t_pad, dtype=orig)
+        for v, p in zip(flat[:t].split(self.numels), cpu_params):  # ya_fsdp/_param_group.py:324-326
+            v.copy_(p.view(-1))
+        self.shard = flat.chunk(w)[r].clone()  # :337-339
+        self.grad_shard = torch.zeros(s, dtype=orig)  # :276
+        self.ag_in = self.shard if self.param_dtype is None else torch.zeros(s, dtype=self.ag_dtype)
+        self.ag_out = torch.zeros(t_pad, dtype=self.ag_dtype)
+        self.rs = torch.zeros(t_pad, dtype=self.rs_dtype)
+        self.rs_views = [v.view(sz) for v, sz in zip(self.rs[:t].split(self.numels), self.sizes)]
+
+    def unshard(self, first_of_iteration=True):
+        if first_of_iteration and self.param_dtype is not None:
+            torch_ops.copy_in(self.ag_in, self.shard)
+        if self.w == 1:
+            torch_ops.all_gather_single_rank(self.ag_out, self.ag_in)
+        else:
+            self.ag_out.chunk(self.w)[self.r].copy_(self.ag_in)  # this rank's slot of the all-gather
+        return torch_ops.unsharded_views(self.ag_out, self.numels, self.sizes)
+
+    def accumulate(self, grads, accumulate_flags):
+        cp = [i for i, (g, a) in enumerate(zip(grads, accumulate_flags)) if g is not None and not a]
+        ad = [i for i, (g, a) in enumerate(zip(grads, accumulate_flags)) if g is not None and a]
+        torch_ops.reduce_copy_in([self.rs_views[i] for i in cp], [grads[i] for i in cp], False)
+        torch_ops.reduce_copy_in([self.rs_views[i] for i in ad], [grads[i] for i in ad], True)
+
+    def reduce(self, pre, post, mode, has=None):
+        torch_ops.reduce_scatter_local(
+            self.grad_shard, self.rs, self.w, self.r, pre, post, mode, self.lay.sharded_numels(self.r), has
+        )
+
+
+BF16_MP = MixedPrecisionPolicy(param_dtype=torch.bfloat16)
+
+
+@pytest.mark.parametrize("shapes,w,r,align", [
+    (TINY_SHAPES, 1, 0, 512),   # config 1: tiny Llama-style layer, W=1
+    (TINY_SHAPES, 2, 1, 512),
+    (ODD_SHAPES, 4, 2, 8),      # ragged: shard boundaries inside tensors, pad lanes
+    (ODD_SHAPES, 4, 3, 8),
+    (ODD_SHAPES, 7, 0, 1),
+])
+def test_layout_views_and_unshard(shapes, w, r, align):
+    group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
+    ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
+    assert group.layout.padded_sharded_numel == ref.lay.padded_sharded_numel
+    assert_bits_equal(group._padded_sharded_param_data[None], ref.shard, "master shard")
+    for fp, n, go in zip(group.fsdp_params, ref.lay.sharded_numels(r), ref.lay.global_offsets(r)):
+        assert fp.sharded_numel == n and fp.placement.global_offset == go
+    group.pre_forward()
+    views = ref.unshard()
+    torch.cuda.synchronize()
+    assert group.is_unsharded
+    assert_bits_equal(group._all_gather_input[None], ref.ag_in, "copy-in")
+    assert_bits_equal(group._all_gather_output[None], ref.ag_out, "gathered buffer")
+    for fp, v in zip(group.fsdp_params, views):
+        assert fp.unsharded_param.shape == v.shape
+        # zero-copy: the unsharded parameter aliases the gathered buffer
+        base = group._all_gather_output[None]
+        assert base.data_ptr() <= fp.unsharded_param.data_ptr() < base.data_ptr() + base.numel() * base.element_size()
+        if w == 1:
+            assert_bits_equal(fp.unsharded_param.detach(), v, "unsharded view")
+    # materialising copy-out of the same buffer
+    outs = [torch.empty(s, dtype=torch.bfloat16, device=DEV) for s in shapes]
+    group.copy_out_materialize(outs)
+    want = [torch.empty(s, dtype=torch.bfloat16) for s in shapes]
+    torch_ops.copy_out_materialize(ref.ag_out, ref.numels, want)
+    for a, b in zip(outs, want):
+        assert_bits_equal(a, b, "materialised copy-out")
+    group.post_forward()
+    assert group.is_sharded and group.data_buffer_ctx.owner is None
+
+
+def _run_backward(group, ref, grads_cpu, reduce=True):
+    for fp, g in zip(group.fsdp_params, grads_cpu):
+        fp.unsharded_param.grad = None if g is None else g.to(DEV)
+    flags = [fp.unsharded_accumulated_grad is not None for fp in group.fsdp_params]
+    group.reduce_grads = reduce
+    group.post_backward()
+    ref.accumulate(grads_cpu, flags)
+
+
+@pytest.mark.parametrize("shapes,w,r,align", [(TINY_SHAPES, 1, 0, 512), (ODD_SHAPES, 4, 2, 8), (ODD_SHAPES, 4, 3, 8)])
+@pytest.mark.parametrize("force_sum", [False, True])
+def test_backward_reduce_copy_then_accumulate(shapes, w, r, align, force_sum):
+    group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
+    group.force_sum_reduction_for_comms = force_sum
+    ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
+    # bf16 reduce: (None, None, AVG) -> the division by W happens "inside the collective";
+    # force_sum -> (None, W, SUM).  On one GPU both are a post-divide by W of the rank's chunk.
+    post = float(w) if w > 1 else None
+    for it in range(2):
+        group.pre_forward(); group.post_forward(); group.pre_backward()
+        ref.unshard(first_of_iteration=True)
+        grads = _grads(shapes, torch.bfloat16, 10 + it)
+        _run_backward(group, ref, grads)
+        ref.reduce(None, post, "copy" if it == 0 else "add")
+        group.finalize_backward()
+        torch.cuda.synchronize()
+        if post is None:  # with a post-divide the reference also rewrites its (scratch) chunk in place
+            assert_bits_equal(group._reduce_scatter_input[None], ref.rs, "reduce buffer")
+        assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, f"grad shard after backward {it}")
+        for fp in group.fsdp_params:
+            assert fp.sharded_param.grad is fp.sharded_param_grad
+        assert group.grad_buffer_ctx.owner is None and group._training_state.name == "IDLE"
+
+
+def test_gradient_accumulation_without_sync_uses_add():
+    shapes, w, r, align = ODD_SHAPES, 4, 1, 8
+    group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
+    ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.bfloat16, 20), reduce=False)   # copy, no reduce
+    assert group._post_reduce_event is None
+    group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.bfloat16, 21), reduce=False)   # add, no reduce
+    group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.bfloat16, 22), reduce=True)    # add, then reduce
+    ref.reduce(None, float(w), "copy")
+    group.finalize_backward()
+    torch.cuda.synchronize()
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
+
+
+def test_mixed_params_with_and_without_sharded_grad():
+    shapes, w, r, align = ODD_SHAPES, 2, 0, 8
+    group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
+    ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    g1 = _grads(shapes, torch.bfloat16, 30)
+    g1[1] = None; g1[4] = None                      # two params get no gradient in the first backward
+    _run_backward(group, ref, g1)
+    has = [None if g is None else False for g in g1]
+    ref.reduce(None, float(w), "mixed", has)        # partial first reduction goes through the fragment path
+    group.finalize_backward()
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    ref.unshard()
+    g2 = _grads(shapes, torch.bfloat16, 31)
+    _run_backward(group, ref, g2)
+    has2 = [g is not None for g in g1]              # params that already own a sharded grad accumulate
+    ref.reduce(None, float(w), "mixed", has2)
+    group.finalize_backward()
+    torch.cuda.synchronize()
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
+
+
+def test_fp16_reduce_uses_pre_and_post_divide():
+    shapes, w, r, align = ODD_SHAPES, 8, 5, 8
+    mp = MixedPrecisionPolicy(param_dtype=torch.float16)
+    group, cpu_params = _make_group(shapes, w, r, align, mp)
+    ref = CpuGroup(cpu_params, w, r, align, mp)
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.float16, 40))
+    ref.reduce(4.0, 2.0, "copy")                    # W=8 -> pre 4, post 2 (ya_fsdp/_collectives.py:252-262)
+    group.finalize_backward()
+    torch.cuda.synchronize()
+    # outside this rank's chunk the reduce buffer holds cast + pre-divide only, like the reference's
+    s_, rs_dev = ref.lay.padded_sharded_numel, group._reduce_scatter_input[None]
+    assert_bits_equal(rs_dev[: r * s_], ref.rs[: r * s_], "reduce buffer before the chunk")
+    assert_bits_equal(rs_dev[(r + 1) * s_ :], ref.rs[(r + 1) * s_ :], "reduce buffer after the chunk")
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard fp16 reduce")
+
+
+def test_bf16_masters_fp32_reduce():
+    shapes, w, r, align = ODD_SHAPES, 4, 2, 8
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32)
+    group, cpu_params = _make_group(shapes, w, r, align, mp, master_dtype=torch.bfloat16)
+    assert group.param_dtype is None and group.reduce_dtype == torch.float32   # clamping, ya_fsdp/_param.py:170-183
+    assert group._all_gather_input[None].data_ptr() == group._padded_sharded_param_data[None].data_ptr()
+    ref = CpuGroup(cpu_params, w, r, align, mp)
+    for it in range(2):
+        group.pre_forward(); group.post_forward(); group.pre_backward()
+        _run_backward(group, ref, _grads(shapes, torch.bfloat16, 50 + it))
+        ref.reduce(None, float(w), "copy" if it == 0 else "add")
+        group.finalize_backward()
+    torch.cuda.synchronize()
+    assert group._padded_sharded_param_grad[None].dtype == torch.bfloat16
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "bf16 grad shard, fp32 reduce")
+
+
+def test_fp32_no_mixed_precision_reduces_in_sharded():
+    shapes, w, r, align = ODD_SHAPES, 1, 0, 8
+    mp = MixedPrecisionPolicy()
+    group, cpu_params = _make_group(shapes, w, r, align, mp)
+    ref = CpuGroup(cpu_params, w, r, align, mp)
+    group.gradient_divide_factor = 3.0              # size-1 group with a custom factor: out-of-place divide (:141-148)
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    grads = _grads(shapes, torch.float32, 60)
+    _run_backward(group, ref, grads)
+    ref.grad_shard.copy_(ref.rs / 3.0)
+    group.finalize_backward()
+    torch.cuda.synchronize()
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "fp32 reduce in sharded")
+
+
+def test_buffer_ownership_protocol():
+    from yafsdp_amd._param_group import YaFSDPParamGroup, init_shared_state
+
+    def mk(seed):
+        ps = [p.to(DEV).requires_grad_(True) for p in _params(ODD_SHAPES, torch.float32, seed)]
+        return YaFSDPParamGroup(ps, FSDPMeshInfo(2, 0), DEV, BF16_MP, 8, module_fqn=f"layer{seed}")
+
+    a, b, c = mk(1), mk(2), mk(3)
+    init_shared_state([a, b, c], DEV)               # 2 data buffers round-robin: a and c share one
+    assert a.data_buffer_ctx is c.data_buffer_ctx and a.data_buffer_ctx is not b.data_buffer_ctx
+    assert a.grad_buffer_ctx is b.grad_buffer_ctx is c.grad_buffer_ctx
+    assert a.comm_ctx is b.comm_ctx
+    a.pre_forward()
+    b.pre_forward()                                 # other buffer: fine
+    with pytest.raises(RuntimeError, match="data buffer"):
+        c.pre_forward()                             # ya_fsdp/_param_group.py:567-572
+    a.post_forward()
+    assert a.data_buffer_ctx.release_event is not None
+    c._all_gather_result = None
+    c.pre_forward()                                 # waits on the release event, then owns the buffer
+    assert a.data_buffer_ctx.owner is c and a.data_buffer_ctx.release_event is None
+    # gradient buffer: one for all groups
+    for fp in b.fsdp_params:
+        fp.unsharded_param.grad = torch.zeros_like(fp.unsharded_param)
+    b.grad_buffer_ctx.owner = a
+    with pytest.raises(RuntimeError, match="gradient buffer"):
+        b.post_backward()                           # :660-664
+    b.grad_buffer_ctx.owner = None
+    b.post_backward()
+    assert b.grad_buffer_ctx.owner is None and b.grad_buffer_ctx.release_event is b._post_reduce_event
+    b.finalize_backward(); c.post_forward()
+    torch.cuda.synchronize()
+
+
+def test_copy_in_runs_once_per_iteration():
+    group, cpu_params = _make_group(ODD_SHAPES, 2, 1, 8, BF16_MP)
+    group.pre_forward(); group.post_forward()
+    torch.cuda.synchronize()
+    first = group._all_gather_input[None].clone()
+    with torch.no_grad():
+        group._padded_sharded_param_data[None].add_(1.0)        # an optimizer step
+    group.pre_backward()                                        # same iteration: stale copy is reused (:47-55)
+    torch.cuda.synchronize()
+    assert_bits_equal(group._all_gather_input[None], first.cpu(), "copy-in skipped inside one iteration")
+    group.post_backward(); group.finalize_backward()            # clears the once-per-iteration set (:783)
+    group.pre_forward()
+    torch.cuda.synchronize()
+    assert not torch.equal(group._all_gather_input[None], first)
+
+
+def test_constructor_errors():
+    from yafsdp_amd._param_group import YaFSDPParamGroup
+
+    mi = FSDPMeshInfo(2, 0)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        YaFSDPParamGroup([torch.zeros(4)], mi, torch.device("cpu"))
+    with pytest.raises(NotImplementedError):
+        YaFSDPParamGroup([torch.zeros(4, 4, device=DEV).t()], mi, DEV)
+    with pytest.raises(AssertionError, match="uniform original parameter dtype"):
+        YaFSDPParamGroup([torch.zeros(4, device=DEV), torch.zeros(4, device=DEV, dtype=torch.bfloat16)], mi, DEV)
+    with pytest.raises(ValueError):
+        YaFSDPParamGroup([torch.zeros((), device=DEV)], mi, DEV)
+    with pytest.raises(ValueError):
+        MixedPrecisionPolicy(reduce_dtype=torch.float16, bit32_acc_for_bit16_reduce_scatter=True)

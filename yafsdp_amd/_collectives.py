@@ -1,0 +1,265 @@
+"""Collective + buffer ops of one parameter group: the hot path.
+
+Same function names, positional signatures and return types as
+ya_fsdp/_collectives.py, so that the parameter-group code above it reads the
+same.  Every tensor op of the reference on this path is replaced by one launch
+of a gfx950 kernel through the C ABI (``_native``); there is no torch or CPU
+fallback.
+
+=====================================================  =========================
+reference op                                           here
+=====================================================  =========================
+``all_gather_input.copy_(shard)`` (:53-54)             ``flat_copy``
+``all_gather_output.copy_(all_gather_input)`` (:56-58)  ``flat_copy``
+``_div_if_needed(rs_input, pre)`` (:139)               fused into the reduce
+                                                        copy-in launch, or
+                                                        ``flat_div``
+``output.copy_(rs_input [/ factor])`` (:140-150)       ``flat_copy`` /
+                                                        ``flat_div_copy``
+``_div_if_needed(output, post)`` + ``copy_``/``add_``   ``post_reduce``
+(:165, :185, :189)
+``_foreach_copy_`` + ``_foreach_add_`` (:191-214)       ``post_reduce_fragments``
+=====================================================  =========================
+
+One GPU: ``all_gather_group.size()`` may exceed 1 (logical world size).  The
+inter-GPU exchange (:60-71, :152-164) is then reduced to this rank's share:
+the all-gather writes this rank's slot of the gathered buffer, and the
+reduce-scatter result is this rank's chunk with the division the collective
+would have applied (``ReduceOp.AVG``: by the group size; pre-multiplied sum:
+by the custom factor) applied as a post-divide in the same launch.
+"""
+
+from __future__ import annotations
+
+from typing import TYPE_CHECKING, Any, NamedTuple, Optional, Sequence
+
+import torch
+
+from . import _native
+
+if TYPE_CHECKING:
+    from ._param import YaFSDPParam
+    from ._param_group import YaFSDPParamGroup
+
+MODE_SKIP, MODE_COPY, MODE_ADD = _native.MODE_SKIP, _native.MODE_COPY, _native.MODE_ADD
+
+
+class AllGatherResult(NamedTuple):
+    """ya_fsdp/_collectives.py:20-28."""
+
+    all_gather_event: torch.cuda.Event | None
+    all_gather_work: Any | None
+
+    def wait(self) -> None:
+        if (event := self.all_gather_event) is not None:
+            event.wait()
+        if (work := self.all_gather_work) is not None:
+            work.wait()
+
+
+def all_gather(
+    param_group: "YaFSDPParamGroup",
+    fsdp_params: "list[YaFSDPParam]",
+    padded_sharded_param_data: torch.Tensor,
+    all_gather_input: torch.Tensor,
+    all_gather_output: torch.Tensor,
+    all_gather_group: Any,
+    async_op: bool,
+    all_gather_stream: torch.cuda.Stream,
+    device: torch.device,
+    param_dtype: torch.dtype | None,
+    all_gather_dtype: torch.dtype | None,
+    yccl_handle: Optional[Any],
+) -> AllGatherResult:
+    """ya_fsdp/_collectives.py:31-76."""
+    if yccl_handle is not None:
+        raise NotImplementedError("YCCL handles are not part of this build")
+    with torch.cuda.stream(all_gather_stream):
+        if all_gather_dtype not in param_group._all_gather_input_set_dtypes:
+            for fsdp_param in fsdp_params:
+                fsdp_param.set_all_gather_input()
+            if all_gather_dtype is None and param_dtype is not None:
+                # copy-in: cast the master shard (:53-54); the version counter of
+                # the destination is untouched because no autograd op is involved
+                _native.flat_copy(all_gather_input, padded_sharded_param_data)
+            param_group._all_gather_input_set_dtypes.add(all_gather_dtype)
+        world_size = all_gather_group.size()
+        if world_size == 1:
+            _native.flat_copy(all_gather_output, all_gather_input)  # :56-58
+        else:
+            # this rank's share of all_gather_into_tensor (:60-65)
+            shard_numel = all_gather_input.numel()
+            rank = all_gather_group.rank()
+            _native.flat_copy(all_gather_output[rank * shard_numel : (rank + 1) * shard_numel], all_gather_input)
+        all_gather_work = None
+        all_gather_event = all_gather_stream.record_event()
+    return AllGatherResult(all_gather_event, all_gather_work)
+
+
+def foreach_reduce_copy_in(
+    param_group: "YaFSDPParamGroup",
+    table: "_native.TensorTable",
+    reduce_scatter_input: torch.Tensor,
+    grads: Sequence[torch.Tensor | None],
+    modes: Sequence[int],
+    predivide_factor: float | None,
+) -> None:
+    """The two foreach calls of ya_fsdp/_param_group.py:693-708 as ONE launch:
+    per parameter ``copy`` (first micro-batch), ``add`` (accumulation) or absent,
+    with the pre-divide of ya_fsdp/_collectives.py:139 and the zero-fill of the
+    pad lanes fused in.  Runs on the current (compute) stream, like the
+    reference's foreach calls."""
+    prepared = []
+    for g in grads:
+        if g is not None and not g.is_contiguous():
+            g = g.contiguous()  # the reference's foreach ops accept strided gradients
+        prepared.append(g)
+    table.gather_in(prepared, reduce_scatter_input, modes, predivide_factor, zero_pad=True)
+
+
+def reduce_scatter(
+    fsdp_params: "list[YaFSDPParam]",
+    fsdp_params_with_grad: "list[YaFSDPParam]",
+    padded_sharded_param_grad: torch.Tensor,
+    padded_unsharded_param_grad: torch.Tensor,
+    reduce_scatter_group: Any,
+    reduce_scatter_stream: torch.cuda.Stream,
+    orig_dtype: torch.dtype,
+    param_dtype: torch.dtype | None,
+    reduce_dtype: torch.dtype | None,
+    device: Any,
+    gradient_divide_factor: float | None,
+    force_sum_reduction_for_comms: bool,
+    bit32_acc_for_bit16_reduce_scatter: bool,
+    yccl_handle: Optional[Any],
+    *,
+    predivide_fused: bool = False,
+) -> torch.cuda.Event:
+    """ya_fsdp/_collectives.py:93-218.
+
+    ``predivide_fused``: the caller already applied the pre-divide inside the
+    reduce copy-in launch (``foreach_reduce_copy_in``), so it is skipped here.
+    """
+    if yccl_handle is not None:
+        raise NotImplementedError("YCCL handles are not part of this build")
+    if bit32_acc_for_bit16_reduce_scatter:
+        # the reference passes acc_type= to dist.reduce_scatter_tensor (:157-161),
+        # which only exists in a patched torch; there is no collective here
+        raise NotImplementedError("bit32_acc_for_bit16_reduce_scatter needs an inter-GPU reduce-scatter")
+    reduce_scatter_stream.wait_stream(torch.cuda.current_stream(padded_sharded_param_grad.device))
+    with torch.cuda.stream(reduce_scatter_stream):
+        world_size, rank = reduce_scatter_group.size(), reduce_scatter_group.rank()
+        reduce_in_sharded = (
+            ((reduce_dtype is None and param_dtype is None) or reduce_dtype == orig_dtype)
+            and all(
+                fsdp_param.sharded_param.grad is None
+                for fsdp_param in fsdp_params
+                if fsdp_param.sharded_param.requires_grad
+            )
+            and yccl_handle is None
+        )  # :112-123
+        shard_numel = padded_unsharded_param_grad.numel() // world_size
+        chunk = padded_unsharded_param_grad[rank * shard_numel : (rank + 1) * shard_numel]  # :127-129
+        predivide_factor, postdivide_factor, reduce_scatter_op, premul = _get_gradient_divide_factors(
+            reduce_scatter_group,
+            reduce_dtype or param_dtype or orig_dtype,
+            gradient_divide_factor,
+            force_sum_reduction_for_comms,
+            yccl_handle=yccl_handle,
+        )
+        if not predivide_fused:
+            _div_if_needed(padded_unsharded_param_grad, predivide_factor)  # :139
+        if world_size == 1:
+            custom = (
+                gradient_divide_factor is not None and predivide_factor is None and postdivide_factor is None
+            )  # :141-145
+            output_tensor = padded_sharded_param_grad if reduce_in_sharded else chunk
+            if custom:
+                _native.flat_div_copy(output_tensor, padded_unsharded_param_grad, gradient_divide_factor)  # :146-148
+            elif reduce_in_sharded:
+                _native.flat_copy(output_tensor, padded_unsharded_param_grad)  # :150
+            # else: output aliases the reduce buffer, copy_ onto itself is a no-op (:150)
+            collective_divide = None
+        else:
+            # this rank's share of reduce_scatter_tensor (:152-162): its chunk, divided as the
+            # collective would have (AVG: by the group size; pre-multiplied sum: by the factor)
+            if reduce_scatter_op == "AVG":
+                collective_divide = float(world_size)
+            elif reduce_scatter_op == "PREMUL_SUM":
+                collective_divide = float(gradient_divide_factor)
+            else:
+                collective_divide = None
+            if collective_divide is not None and collective_divide <= 1 and collective_divide != 1:
+                # a pre-multiplier >= 1 is outside the "> 1" rule of the fused divide: apply it on its own
+                _native.flat_div_copy(chunk, chunk, collective_divide)
+                collective_divide = None
+            output_tensor = chunk
+        # post-divide (:165) fused with the copy / accumulate into the gradient shard (:166-214)
+        post = postdivide_factor if collective_divide is None else collective_divide
+        if world_size > 1 and reduce_in_sharded:
+            # the collective would have written straight into the shard (:124-125)
+            _native.post_reduce(padded_sharded_param_grad, chunk, post, False)
+        elif world_size == 1 and reduce_in_sharded:
+            _div_if_needed(padded_sharded_param_grad, post)
+        else:
+            fsdp_params_which_require_grad = [p for p in fsdp_params if p.sharded_param.requires_grad]
+            without_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is None]
+            with_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is not None]
+            if len(without_sharded_grad) == len(fsdp_params_which_require_grad):
+                _native.post_reduce(padded_sharded_param_grad, output_tensor, post, False)  # :185
+            elif len(with_sharded_grad) == len(fsdp_params_which_require_grad):
+                _native.post_reduce(padded_sharded_param_grad, output_tensor, post, True)  # :189
+            else:
+                with_ids = {id(p) for p in with_sharded_grad}
+                without_ids = {id(p) for p in without_sharded_grad}
+                modes = [
+                    MODE_ADD if id(p) in with_ids else (MODE_COPY if id(p) in without_ids else MODE_SKIP)
+                    for p in fsdp_params
+                ]
+                numels = [p.sharded_numel for p in fsdp_params]
+                _native.post_reduce_fragments(padded_sharded_param_grad, output_tensor, numels, modes, post)  # :191-214
+        post_reduce_event = reduce_scatter_stream.record_event()
+        for fsdp_param in fsdp_params_with_grad:
+            fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad  # :216-217
+        return post_reduce_event
+
+
+def _get_gradient_divide_factors(
+    reduce_scatter_group: Any,
+    reduce_dtype: torch.dtype,
+    factor: float | None,
+    force_sum_reduction_for_comms: bool,
+    yccl_handle: Optional[Any] = None,
+) -> tuple[float | None, float | None, str, float | None]:
+    """ya_fsdp/_collectives.py:221-267.  The reduce op is returned by name
+    ("SUM", "AVG", "PREMUL_SUM") with the pre-multiplier as a fourth value,
+    because no NCCL op object is needed on one GPU."""
+    if yccl_handle is not None:
+        force_sum_reduction_for_comms = True
+    overflow_risk = reduce_dtype not in (torch.float32, torch.bfloat16)
+    data_parallel_size = reduce_scatter_group.size()
+    if not overflow_risk and not force_sum_reduction_for_comms:
+        if factor is None:
+            if data_parallel_size == 1:
+                return None, None, "SUM", None
+            return None, None, "AVG", None
+        if factor == reduce_scatter_group.size():
+            return None, None, "AVG", None
+        return None, None, "PREMUL_SUM", 1 / factor
+    if factor is None:
+        factor = float(data_parallel_size)
+    pre_factor: float | None
+    if overflow_risk:
+        pre_factor = 1
+        while factor % pre_factor == 0 and factor / pre_factor > pre_factor:
+            pre_factor *= 2
+        post_factor = factor / pre_factor
+    else:
+        pre_factor, post_factor = None, factor
+    return pre_factor, post_factor, "SUM", None
+
+
+def _div_if_needed(tensor: torch.Tensor, div_factor: float | None) -> None:
+    """ya_fsdp/_collectives.py:270-272."""
+    if div_factor is not None and div_factor > 1:
+        _native.flat_div(tensor, div_factor)

@@ -1,0 +1,69 @@
+"""Shard-group description and training states.
+
+The reference takes its shard world size and rank from a ``DeviceMesh`` and a
+``ProcessGroup`` (ya_fsdp/_common.py:13-35).  This build runs on one GPU: the
+world size is a layout parameter, so the group is a plain ``(size, rank)``
+pair with the two methods of ``ProcessGroup`` the buffer path calls.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from enum import Enum, auto
+
+import torch
+
+
+class LogicalShardGroup:
+    """Stands where ``dist.ProcessGroup`` stands in ya_fsdp/_collectives.py:
+    ``size()`` and ``rank()`` are all the path reads from it.  No inter-GPU
+    exchange is attached: with ``size() > 1`` the all-gather fills only this
+    rank's slot of the gathered buffer and the reduce-scatter result is this
+    rank's chunk of the reduce buffer (peers contribute nothing)."""
+
+    def __init__(self, size: int, rank: int):
+        if size < 1 or not 0 <= rank < size:
+            raise ValueError(f"invalid shard group: size={size} rank={rank}")
+        self._size, self._rank = int(size), int(rank)
+
+    def size(self) -> int:
+        return self._size
+
+    def rank(self) -> int:
+        return self._rank
+
+    def __repr__(self) -> str:
+        return f"LogicalShardGroup(size={self._size}, rank={self._rank})"
+
+
+@dataclass
+class FSDPMeshInfo:
+    """``shard_mesh_size`` / ``shard_mesh_rank`` / ``shard_process_group`` as in
+    ya_fsdp/_common.py:25-34, built from the two integers instead of a mesh."""
+
+    shard_mesh_size: int
+    shard_mesh_rank: int
+
+    def __post_init__(self) -> None:
+        self.shard_process_group = LogicalShardGroup(self.shard_mesh_size, self.shard_mesh_rank)
+
+
+class TrainingState(Enum):
+    """ya_fsdp/_common.py:37-45."""
+
+    FORWARD = auto()
+    PRE_BACKWARD = auto()
+    POST_BACKWARD = auto()
+    IDLE = auto()
+
+
+class ShardedState(Enum):
+    """ya_fsdp/_param.py:33-41 without the post-forward state (no HSDP here)."""
+
+    SHARDED = auto()
+    UNSHARDED = auto()
+
+
+def is_bw() -> bool:
+    """ya_fsdp/_common.py:73-74."""
+    return torch._C._current_graph_task_id() != -1

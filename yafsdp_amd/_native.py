@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "yafsdp_error_string",
     "yafsdp_flat_copy",
     "yafsdp_flat_div",
+    "yafsdp_flat_div_copy",
     "yafsdp_post_reduce",
     "yafsdp_post_reduce_fragments",
     "yafsdp_table_create",
@@ -58,6 +59,8 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_flat_copy.argtypes = [vp, i32, vp, i32, i64, vp]
     lib.yafsdp_flat_div.restype = i32
     lib.yafsdp_flat_div.argtypes = [vp, i32, i64, dbl, vp]
+    lib.yafsdp_flat_div_copy.restype = i32
+    lib.yafsdp_flat_div_copy.argtypes = [vp, i32, vp, i32, i64, dbl, vp]
     lib.yafsdp_post_reduce.restype = i32
     lib.yafsdp_post_reduce.argtypes = [vp, i32, vp, i32, i64, dbl, i32, vp]
     lib.yafsdp_post_reduce_fragments.restype = i32
@@ -134,6 +137,20 @@ def flat_div(buf: torch.Tensor, factor: float | None) -> None:
         _check(
             lib.yafsdp_flat_div(buf.data_ptr(), _dt(buf), buf.numel(), _factor(factor), _stream(buf)),
             "yafsdp_flat_div",
+        )
+
+
+def flat_div_copy(dst: torch.Tensor, src: torch.Tensor, divisor: float) -> None:
+    """``dst.copy_(src / divisor)`` for any finite non-zero divisor."""
+    _flat_arg(dst, "dst"), _flat_arg(src, "src")
+    if dst.numel() != src.numel():
+        raise ValueError(f"numel mismatch: {dst.numel()} vs {src.numel()}")
+    with torch.cuda.device(dst.device):
+        _check(
+            lib.yafsdp_flat_div_copy(
+                dst.data_ptr(), _dt(dst), src.data_ptr(), _dt(src), dst.numel(), float(divisor), _stream(dst)
+            ),
+            "yafsdp_flat_div_copy",
         )
 
 

@@ -1,0 +1,564 @@
+"""Parameter group: flat-buffer layout plus stream/event scheduling around the
+buffer kernels (mirror of ya_fsdp/_param_group.py for the per-rank buffer path).
+
+What is kept from the reference
+  * one flat padded buffer per group, chunked evenly over the (logical) ranks so
+    that shard boundaries fall mid-tensor (ya_fsdp/_param_group.py:245-406); the
+    ragged split is computed in closed form (``_layout``) instead of with
+    per-element index tensors;
+  * shared, pre-allocated byte buffers that unsharded parameters and gradient
+    accumulators are views into (:32-71, :409-457), two data buffers + one
+    gradient buffer per shard group, sized by the largest sharing group
+    (ya_fsdp/_state.py:200-288);
+  * the owner / release-event hand-off of those buffers and the stream choice
+    of unshard / reshard / post_backward / finalize_backward (:550-615, :655-791);
+  * ``torch.profiler.record_function`` range names (:563, :669, :710, :740).
+
+What differs
+  * every tensor op on the path is a kernel launch through ``_collectives`` /
+    ``_native``; the two foreach calls of post_backward are one launch with the
+    pre-divide and the pad zero-fill fused in;
+  * the side stream has the default priority (the reference asks for a
+    high-priority stream, :80-88; mixed stream priorities are avoided on this
+    platform);
+  * module hooks, DTensor wrapping, state-dict hooks and YCCL are outside this
+    build: a group is constructed from a list of tensors.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import logging
+from enum import Enum, auto
+from typing import Any, Generator, Sequence
+
+import torch
+from torch.profiler import record_function
+
+from . import _native
+from ._api import MixedPrecisionPolicy
+from ._collectives import (
+    MODE_ADD,
+    MODE_COPY,
+    MODE_SKIP,
+    AllGatherResult,
+    _get_gradient_divide_factors,
+    all_gather,
+    foreach_reduce_copy_in,
+    reduce_scatter,
+)
+from ._common import FSDPMeshInfo, ShardedState, TrainingState, is_bw
+from ._layout import ShardLayout, make_layout
+from ._param import YaFSDPParam
+
+logger = logging.getLogger("yafsdp_amd")
+
+
+class YaFSDPBufferContext:
+    """ya_fsdp/_param_group.py:32-71."""
+
+    class BufferType(Enum):
+        ALL_GATHER = auto()
+        REDUCE_SCATTER = auto()
+
+    def __init__(self, buffer_type: "YaFSDPBufferContext.BufferType"):
+        self._buffer_type = buffer_type
+        self.buffers: dict[torch.dtype | None, torch.Tensor] = {}
+        self.owner: YaFSDPParamGroup | None = None
+        self.release_event: torch.cuda.Event | None = None
+
+    def lazy_init(self, sizes_by_dtype: "dict[torch.dtype | None, int]", device: torch.device) -> None:
+        # byte buffers allocated as bf16 and re-viewed, as at :53-69; zero-filled
+        # so that pad lanes are defined from the first use on
+        self.buffers = {
+            dtype: torch.zeros(
+                (size_in_bytes + 1) // torch.bfloat16.itemsize, dtype=torch.bfloat16, device=device
+            ).view(torch.uint8)
+            for dtype, size_in_bytes in sizes_by_dtype.items()
+        }
+        self.owner = None
+        self.release_event = None
+
+
+class YaFSDPCommContext:
+    """ya_fsdp/_param_group.py:74-101."""
+
+    def lazy_init(self, device: torch.device) -> None:
+        self.device = device
+        # one side stream serves both the all-gather and the reduce-scatter side (:85-88)
+        self.all_gather_stream = torch.cuda.Stream(device=device)
+        self.reduce_scatter_stream = self.all_gather_stream
+        self.post_forward_order: list[YaFSDPParamGroup] = []
+
+    def get_all_gather_stream(self, async_op: bool, training_state: TrainingState) -> torch.cuda.Stream:
+        if not async_op and training_state in (TrainingState.FORWARD, TrainingState.PRE_BACKWARD):
+            return self.all_gather_stream
+        return torch.cuda.current_stream(self.device)
+
+
+class YaFSDPParamGroup:
+    """One group of parameters sharing flat buffers and collectives."""
+
+    def __init__(
+        self,
+        params: Sequence[torch.Tensor],
+        mesh_info: FSDPMeshInfo,
+        device: torch.device,
+        mp_policy: MixedPrecisionPolicy = MixedPrecisionPolicy(),
+        shard_alignment: int = 8,
+        names: Sequence[str] | None = None,
+        module_fqn: str | None = None,
+    ):
+        device = torch.device(device)
+        if device.type != "cuda":
+            raise RuntimeError(f"the buffer path runs on the GPU only, got device {device}")
+        if mp_policy.all_gather_dtype_to_param_cls:
+            raise NotImplementedError("per-class all-gather dtypes (tensor-subclass extensions) are not part of this build")
+        names = list(names) if names is not None else [f"param{i}" for i in range(len(params))]
+        self.fsdp_params = [YaFSDPParam(p, mesh_info, device, n) for p, n in zip(params, names)]
+        self.mesh_info = mesh_info
+        self.device = device
+        self.mp_policy = mp_policy
+        self.shard_alignment = int(shard_alignment)
+        self._training_state = TrainingState.IDLE
+        self._sharded_state = ShardedState.SHARDED
+        self._module_fqn = module_fqn
+
+        self.comm_ctx = YaFSDPCommContext()
+        self._post_forward_indices: list[int] = []
+        self.reduce_grads: bool = True
+        self.reshard_after_forward: bool = True
+        self.reshard_after_backward: bool = True
+        self.gradient_divide_factor: float | None = None
+        self.force_sum_reduction_for_comms: bool = False
+        self.unshard_async_op: bool = False
+        self.unshard_in_backward: bool = True
+        self._all_gather_result: AllGatherResult | None = None
+        self._post_reduce_event: torch.cuda.Event | None = None
+
+        self._init_mp_dtypes()
+        param_group_requires_grad = any(p.requires_grad for p in self.fsdp_params)
+        self.data_buffer_ctx = YaFSDPBufferContext(YaFSDPBufferContext.BufferType.ALL_GATHER)
+        self.grad_buffer_ctx = (
+            YaFSDPBufferContext(YaFSDPBufferContext.BufferType.REDUCE_SCATTER) if param_group_requires_grad else None
+        )
+        # one all-gather dtype class (key None), kept as dicts like the reference's
+        self._all_gather_dtype_to_fsdp_params: dict[torch.dtype | None, list[YaFSDPParam]] = {None: self.fsdp_params}
+        self._all_gather_input_set_dtypes: set[torch.dtype | None] = set()
+
+        world_size, rank = mesh_info.shard_mesh_size, mesh_info.shard_mesh_rank
+        numels = [p._orig_size.numel() for p in self.fsdp_params]
+        self.layout: ShardLayout = make_layout(numels, world_size, self.shard_alignment)  # :245-265
+        self._unsharded_param_numels = {None: numels}
+        self.padded_unsharded_param_numel = {None: self.layout.padded_unsharded_numel}
+        self._padded_sharded_param_numel = {None: self.layout.padded_sharded_numel}
+        shard = torch.zeros(self.layout.padded_sharded_numel, dtype=self.orig_dtype, device=device)
+        self._padded_sharded_param_data = {None: shard}
+        self._padded_sharded_param_grad = {None: torch.zeros_like(shard) if param_group_requires_grad else None}
+        sharded_numels = self.layout.sharded_numels(rank)  # :354-358, closed form
+        global_offsets = self.layout.global_offsets(rank)  # :359-377
+        per_rank = self.layout.per_rank_sharded_numels()  # :347-353
+        self._sharded_param_numels = {None: sharded_numels}
+        # flatten + shard (:300-339) without the full-size temporary: copy only the
+        # fragment of each parameter that this rank owns
+        pos = 0
+        grad_shard = self._padded_sharded_param_grad[None]
+        with torch.no_grad():
+            for fsdp_param, n, go, sn in zip(self.fsdp_params, sharded_numels, global_offsets, per_rank):
+                frag = shard[pos : pos + n]
+                if n > 0:
+                    _native.flat_copy(frag, fsdp_param.param_data.detach().view(-1)[go : go + n])
+                fsdp_param.init_sharded_param(
+                    frag, grad_shard[pos : pos + n] if grad_shard is not None else None, global_offset=go,
+                    shard_numels=sn,
+                )  # :379-406
+                pos += n
+        self._table: _native.TensorTable | None = None
+
+    # ------------------------------------------------------------ initialisation --
+    def _init_mp_dtypes(self) -> None:
+        """ya_fsdp/_param_group.py:459-485."""
+        for fsdp_param in self.fsdp_params:
+            fsdp_param.init_dtype_attrs(self.mp_policy)
+        trainable = [p for p in self.fsdp_params if p.requires_grad]
+        orig_dtypes = {p.orig_dtype for p in self.fsdp_params}
+        param_dtypes = {p.param_dtype for p in self.fsdp_params}
+        reduce_dtypes = {p.reduce_dtype for p in trainable}
+        if len(orig_dtypes) != 1:
+            raise AssertionError(f"YaFSDP expects uniform original parameter dtype but got {orig_dtypes}")
+        self.orig_dtype = next(iter(orig_dtypes))
+        if len(param_dtypes) != 1:
+            raise AssertionError(f"YaFSDP expects uniform param dtype but got {param_dtypes}")
+        self.param_dtype = next(iter(param_dtypes))
+        if len(trainable) > 0 and len(reduce_dtypes) != 1:
+            raise AssertionError(f"YaFSDP expects uniform reduce dtype but got {reduce_dtypes}")
+        self.reduce_dtype = next(iter(reduce_dtypes)) if len(trainable) > 0 else None
+
+    @property
+    def all_gather_dtype(self) -> torch.dtype:
+        return self.param_dtype or self.orig_dtype
+
+    @property
+    def reduce_scatter_dtype(self) -> torch.dtype:
+        return self.reduce_dtype or self.param_dtype or self.orig_dtype
+
+    def data_buffer_bytes(self) -> int:
+        return self.layout.padded_unsharded_numel * self.all_gather_dtype.itemsize
+
+    def grad_buffer_bytes(self) -> int:
+        return self.layout.padded_unsharded_numel * self.reduce_scatter_dtype.itemsize
+
+    def _init_unsharded_params(self) -> None:
+        """ya_fsdp/_param_group.py:409-457: typed views of the shared byte buffers,
+        split into per-parameter views (the zero-copy copy-out)."""
+        t_pad, total = self.layout.padded_unsharded_numel, self.layout.total_numel
+        numels = self._unsharded_param_numels[None]
+        ag = self.data_buffer_ctx.buffers[None].narrow(0, 0, self.data_buffer_bytes()).view(self.all_gather_dtype)
+        self._all_gather_output = {None: ag}
+        if self.grad_buffer_ctx is not None:
+            rs = self.grad_buffer_ctx.buffers[None].narrow(0, 0, self.grad_buffer_bytes()).view(
+                self.reduce_scatter_dtype
+            )
+        else:
+            rs = None
+        self._reduce_scatter_input = {None: rs}
+        assert ag.numel() == t_pad
+        ag_views = ag[:total].split(numels)
+        rs_views = rs[:total].split(numels) if rs is not None else (None,) * len(numels)
+        for fsdp_param, v, g in zip(self.fsdp_params, ag_views, rs_views):
+            fsdp_param.init_unsharded_param(v, g)
+
+    def lazy_init(self) -> None:
+        """ya_fsdp/_param_group.py:487-547 (idempotent)."""
+        if not hasattr(self.comm_ctx, "all_gather_stream"):
+            self.comm_ctx.lazy_init(self.device)
+        if None not in self.data_buffer_ctx.buffers:
+            raise RuntimeError(
+                "the data buffer of this group is not allocated: call init_shared_state(groups, device) first"
+            )
+        self._init_unsharded_params()
+        shard = self._padded_sharded_param_data[None]
+        sharded_numels = self._sharded_param_numels[None]
+        n_local = sum(sharded_numels)
+        ag_in = shard if self.param_dtype is None else torch.zeros_like(shard, dtype=self.param_dtype)  # :502-508
+        self._all_gather_input = {None: ag_in}
+        for fsdp_param, frag in zip(self.fsdp_params, ag_in[:n_local].split(sharded_numels)):
+            fsdp_param.init_all_gather_input(frag)
+        self._reduce_scatter_output = {}
+        if self.grad_buffer_ctx is not None:
+            rs = self._reduce_scatter_input[None]
+            s = self.layout.padded_sharded_numel
+            r = self.mesh_info.shard_mesh_rank
+            rs_out = rs[r * s : (r + 1) * s]  # chunk(W)[r], :531-535
+            self._reduce_scatter_output[None] = rs_out
+            for fsdp_param, frag in zip(self.fsdp_params, rs_out[:n_local].split(sharded_numels)):
+                fsdp_param.init_reduce_scatter_output(frag)
+        if self._table is None:
+            self._table = _native.TensorTable(
+                self._unsharded_param_numels[None], self.layout.padded_unsharded_numel, self.device
+            )
+
+    # ------------------------------------------------------------------- runtime --
+    @property
+    def _all_gather_process_group(self) -> Any:
+        return self.mesh_info.shard_process_group
+
+    @property
+    def _reduce_scatter_process_group(self) -> Any:
+        return self.mesh_info.shard_process_group
+
+    def unshard(self, async_op: bool = False) -> None:
+        """ya_fsdp/_param_group.py:550-594."""
+        if self._all_gather_result is not None:
+            return
+        if self.is_unsharded:
+            return
+        if not self.unshard_in_backward and self._training_state == TrainingState.PRE_BACKWARD:
+            return
+        logger.debug("%s", self._with_fqn(f"YaFSDP::{self._training_state.name.lower()}_unshard"))
+        with record_function(self._with_fqn("YaFSDP::all_gather")):
+            all_gather_stream = self.comm_ctx.get_all_gather_stream(async_op, self._training_state)
+            data_buffer_ctx = self.data_buffer_ctx
+            if (owner := data_buffer_ctx.owner) is not None and owner is not self:
+                raise RuntimeError(f"{self} tried to acquire its data buffer, but it is in use by {owner}.")
+            if (release_event := data_buffer_ctx.release_event) is not None:
+                all_gather_stream.wait_event(release_event)
+                data_buffer_ctx.release_event = None
+            data_buffer_ctx.owner = self
+            for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+                self._all_gather_result = all_gather(
+                    self,
+                    fsdp_params,
+                    self._padded_sharded_param_data[all_gather_dtype],
+                    self._all_gather_input[all_gather_dtype],
+                    self._all_gather_output[all_gather_dtype],
+                    self._all_gather_process_group,
+                    async_op,
+                    all_gather_stream,
+                    self.device,
+                    self.param_dtype,
+                    all_gather_dtype,
+                    None,
+                )
+
+    def wait_for_unshard(self) -> AllGatherResult | None:
+        """ya_fsdp/_param_group.py:596-602."""
+        if (all_gather_result := self._all_gather_result) is None:
+            return None
+        all_gather_result.wait()
+        self._to_unsharded()
+        self._all_gather_result = None
+        return all_gather_result
+
+    def reshard(self) -> None:
+        """ya_fsdp/_param_group.py:604-615."""
+        if self._training_state == TrainingState.FORWARD and not self.reshard_after_forward:
+            return
+        logger.debug("%s", self._with_fqn(f"YaFSDP::{self._training_state.name.lower()}_reshard"))
+        self._to_sharded()
+        self.data_buffer_ctx.release_event = torch.cuda.current_stream(self.device).record_event()
+        self.data_buffer_ctx.owner = None
+
+    def pre_forward(self) -> None:
+        """ya_fsdp/_param_group.py:617-626 without the autograd hook registration."""
+        with record_function(self._with_fqn("YaFSDP::pre_forward")):
+            self._training_state = TrainingState.FORWARD
+            self.unshard(self.unshard_async_op)
+            self.wait_for_unshard()
+
+    def post_forward(self) -> None:
+        """ya_fsdp/_param_group.py:628-635."""
+        with record_function(self._with_fqn("YaFSDP::post_forward")):
+            if not is_bw():
+                self.reshard()
+                self._record_post_forward()
+            self._training_state = TrainingState.IDLE
+
+    def _record_post_forward(self) -> None:
+        post_forward_index = len(self.comm_ctx.post_forward_order)
+        self.comm_ctx.post_forward_order.append(self)
+        self._post_forward_indices.append(post_forward_index)
+
+    def pre_backward(self, default_prefetch: bool = True) -> None:
+        """ya_fsdp/_param_group.py:644-653."""
+        if self._training_state == TrainingState.PRE_BACKWARD:
+            return
+        with record_function(self._with_fqn("YaFSDP::pre_backward")):
+            self._training_state = TrainingState.PRE_BACKWARD
+            self.unshard(self.unshard_async_op)
+            self.wait_for_unshard()
+            if default_prefetch:
+                self._backward_prefetch()
+
+    def post_backward(self) -> None:
+        """ya_fsdp/_param_group.py:655-771."""
+        self._training_state = TrainingState.POST_BACKWARD
+        current_stream = torch.cuda.current_stream(self.device)
+        if (grad_buffer_ctx := self.grad_buffer_ctx) is not None:
+            if (owner := grad_buffer_ctx.owner) is not None and owner is not self:
+                raise RuntimeError(f"{self} tried to acquire its gradient buffer, but it is in use by {owner}.")
+            if (release_event := grad_buffer_ctx.release_event) is not None:
+                current_stream.wait_event(release_event)
+                grad_buffer_ctx.release_event = None
+            grad_buffer_ctx.owner = self
+        predivide_fused = False
+        with record_function(self._with_fqn("FSDP::post_backward_accumulate")):
+            grads: list[torch.Tensor | None] = []
+            modes: list[int] = []
+            for fsdp_param in self.fsdp_params:
+                has_grad = fsdp_param.requires_grad and fsdp_param.unsharded_param.grad is not None
+                if has_grad and fsdp_param.unsharded_accumulated_grad is None:
+                    grads.append(fsdp_param.unsharded_grad_data)
+                    modes.append(MODE_COPY)  # _foreach_copy_, :693-700
+                    fsdp_param.unsharded_param.grad = None
+                    fsdp_param.unsharded_accumulated_grad = fsdp_param._unsharded_accumulated_grad
+                elif has_grad:
+                    grads.append(fsdp_param.unsharded_grad_data)
+                    modes.append(MODE_ADD)  # _foreach_add_, :701-708
+                    fsdp_param.unsharded_param.grad = None
+                else:
+                    grads.append(None)
+                    modes.append(MODE_SKIP)
+            if any(m != MODE_SKIP for m in modes):
+                assert grad_buffer_ctx is not None and self._table is not None
+                pre = None
+                if self.reduce_grads:
+                    pre, _, _, _ = _get_gradient_divide_factors(
+                        self._reduce_scatter_process_group, self.reduce_scatter_dtype, self.gradient_divide_factor,
+                        self.force_sum_reduction_for_comms,
+                    )
+                    predivide_fused = True
+                foreach_reduce_copy_in(self, self._table, self._reduce_scatter_input[None], grads, modes, pre)
+        fsdp_params_with_grad_per_dtype: dict[torch.dtype | None, list[YaFSDPParam]] = {}
+        with record_function(self._with_fqn("YaFSDP::post_backward_reshard")):
+            if not self.reduce_grads:
+                if self.reshard_after_backward:
+                    self.reshard()
+                return
+            for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+                fsdp_params_with_grad = []
+                for fsdp_param in fsdp_params:
+                    if fsdp_param.unsharded_accumulated_grad is not None:
+                        fsdp_params_with_grad.append(fsdp_param)
+                        fsdp_param.unsharded_accumulated_grad = None
+                fsdp_params_with_grad_per_dtype[all_gather_dtype] = fsdp_params_with_grad
+            if self.reshard_after_backward:
+                self.reshard()
+        if sum(map(len, fsdp_params_with_grad_per_dtype.values())) == 0:
+            if grad_buffer_ctx is not None:
+                grad_buffer_ctx.release_event = current_stream.record_event()
+                grad_buffer_ctx.owner = None
+            return
+        assert grad_buffer_ctx is not None
+        with record_function(self._with_fqn("YaFSDP::post_backward_reduce")):
+            for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+                self._post_reduce_event = reduce_scatter(
+                    fsdp_params,
+                    fsdp_params_with_grad_per_dtype[all_gather_dtype],
+                    self._padded_sharded_param_grad[all_gather_dtype],
+                    self._reduce_scatter_input[all_gather_dtype],
+                    self._reduce_scatter_process_group,
+                    self.comm_ctx.reduce_scatter_stream,
+                    self.orig_dtype,
+                    self.param_dtype,
+                    self.reduce_dtype,
+                    self.device,
+                    self.gradient_divide_factor,
+                    self.force_sum_reduction_for_comms,
+                    self.mp_policy.bit32_acc_for_bit16_reduce_scatter,
+                    None,
+                    predivide_fused=predivide_fused,
+                )
+        grad_buffer_ctx.release_event = self._post_reduce_event
+        grad_buffer_ctx.owner = None
+
+    def finalize_backward(self) -> None:
+        """ya_fsdp/_param_group.py:773-783."""
+        self._wait_for_post_backward()
+        if self._all_gather_result is not None:
+            self._all_gather_result.wait()
+            self._all_gather_result = None
+            self.data_buffer_ctx.owner = None
+        self._post_forward_indices.clear()
+        self._all_gather_input_set_dtypes.clear()
+        self._training_state = TrainingState.IDLE
+
+    def _wait_for_post_backward(self) -> None:
+        """ya_fsdp/_param_group.py:785-791."""
+        if self._post_reduce_event is not None:
+            torch.cuda.current_stream(self.device).wait_event(self._post_reduce_event)
+            self._post_reduce_event = None
+            assert self.grad_buffer_ctx is not None
+            assert self.grad_buffer_ctx.owner is None
+            self.grad_buffer_ctx.release_event = None
+
+    def _backward_prefetch(self) -> None:
+        """ya_fsdp/_param_group.py:793-805."""
+        if not self._post_forward_indices:
+            return
+        curr_index = self._post_forward_indices.pop()
+        if (target_index := curr_index - 1) < 0:
+            return
+        target = self.comm_ctx.post_forward_order[target_index]
+        if target.data_buffer_ctx is not self.data_buffer_ctx:
+            self._prefetch_unshard(target, "backward")
+
+    @staticmethod
+    def _prefetch_unshard(target: "YaFSDPParamGroup", pass_type: str) -> None:
+        """ya_fsdp/_param_group.py:807-827."""
+        if pass_type == "backward":
+            training_state = TrainingState.PRE_BACKWARD
+        elif pass_type == "forward":
+            training_state = TrainingState.FORWARD
+        else:
+            raise ValueError(f"Unknown pass type: {pass_type}")
+        with record_function(f"YaFSDP::{pass_type}_prefetch for {target._module_fqn}"), target.use_training_state(
+            training_state
+        ):
+            target.unshard(target.unshard_async_op)
+
+    # ----------------------------------------------------- materialising copy-out --
+    def copy_out_materialize(self, outs: Sequence[torch.Tensor | None]) -> None:
+        """Copy the gathered flat buffer into separately allocated tensors (one
+        launch).  The group's own unsharded parameters are zero-copy views
+        (``_init_unsharded_params``); this is for consumers that need their own
+        storage.  Runs on the current stream; call after ``wait_for_unshard``."""
+        assert self._table is not None, "lazy_init() first"
+        self._table.scatter_out(self._all_gather_output[None], [o.view(-1) if o is not None else None for o in outs])
+
+    # ------------------------------------------------------------------ utilities --
+    def _to_sharded(self) -> None:
+        if not self.is_sharded:
+            for fsdp_param in self.fsdp_params:
+                fsdp_param.to_sharded()
+            self._sharded_state = ShardedState.SHARDED
+
+    def _to_unsharded(self) -> None:
+        if not self.is_unsharded:
+            for fsdp_param in self.fsdp_params:
+                fsdp_param.to_unsharded()
+            self._sharded_state = ShardedState.UNSHARDED
+
+    @property
+    def is_sharded(self) -> bool:
+        return self._sharded_state == ShardedState.SHARDED
+
+    @property
+    def is_unsharded(self) -> bool:
+        return self._sharded_state == ShardedState.UNSHARDED
+
+    @contextlib.contextmanager
+    def use_training_state(self, training_state: TrainingState) -> Generator[None, Any, None]:
+        old = self._training_state
+        self._training_state = training_state
+        try:
+            yield
+        finally:
+            self._training_state = old
+
+    def _with_fqn(self, label: str) -> str:
+        if self._module_fqn:
+            return f"{label} ({self._module_fqn})"
+        return label
+
+    def __repr__(self) -> str:
+        return f"YaFSDPParamGroup(fqn={self._module_fqn})"
+
+
+def init_shared_state(
+    param_groups: Sequence[YaFSDPParamGroup], device: torch.device, num_data_buffers: int | None = 2,
+    num_grad_buffers: int | None = 1,
+) -> None:
+    """Buffer assignment of ya_fsdp/_state.py:200-288 and :617-678 for groups
+    that share one shard group: one communication context, ``num_data_buffers``
+    data buffers handed out round-robin in group order, ``num_grad_buffers``
+    gradient buffers; each buffer is as large as the largest group using it.
+    ``None`` gives every group its own buffer.  Ends with ``lazy_init`` of each
+    group."""
+    device = torch.device(device)
+    if not param_groups:
+        return
+    comm_ctx = YaFSDPCommContext()
+    comm_ctx.lazy_init(device)
+
+    def assign(groups: Sequence[YaFSDPParamGroup], attr: str, count: int | None, size_of) -> None:
+        if not groups:
+            return
+        n = len(groups) if count is None else min(count, len(groups))
+        ctxs = [getattr(groups[i], attr) for i in range(n)]
+        users: list[list[YaFSDPParamGroup]] = [[] for _ in range(n)]
+        for i, g in enumerate(groups):
+            users[i % n].append(g)
+        for ctx, gs in zip(ctxs, users):
+            ctx.lazy_init({None: max(size_of(g) for g in gs)}, device)
+            for g in gs:
+                setattr(g, attr, ctx)
+
+    assign(list(param_groups), "data_buffer_ctx", num_data_buffers, lambda g: g.data_buffer_bytes())
+    assign(
+        [g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx", num_grad_buffers,
+        lambda g: g.grad_buffer_bytes(),
+    )
+    for g in param_groups:
+        g.comm_ctx = comm_ctx
+        g.lazy_init()

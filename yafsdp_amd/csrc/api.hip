@@ -56,6 +56,22 @@ void scale_plan(double factor, int* scale, float* k) {
   }
 }
 
+// Same for a division that is applied whatever the factor (not the "> 1" rule).
+bool scale_plan_any(double divisor, int* scale, float* k) {
+  const float f = static_cast<float>(divisor);
+  if (!std::isfinite(f) || f == 0.0f) return false;
+  int e = 0;
+  const float m = std::frexp(std::fabs(f), &e);
+  if (m == 0.5f && e <= 126 && e >= -124) {  // +-2^(e-1), reciprocal is a normal number
+    *scale = SCALE_MUL;
+    *k = 1.0f / f;
+  } else {
+    *scale = SCALE_DIV;
+    *k = f;
+  }
+  return true;
+}
+
 int grid_for(int64_t n_tiles, int blocks_per_cu, int device) {
   int64_t cap = int64_t(cu_count(device)) * (blocks_per_cu > 0 ? blocks_per_cu : 1);
   int64_t g = n_tiles < cap ? n_tiles : cap;
@@ -237,6 +253,17 @@ int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream
   scale_plan(factor, &scale, &k);
   if (scale == SCALE_NONE) return YAFSDP_OK;
   return flat_launch(dtype, dtype, scale, false, buf, buf, n, k, static_cast<hipStream_t>(stream));
+}
+
+int yafsdp_flat_div_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, double divisor,
+                         void* stream) {
+  if (!valid_dtype(dst_dtype) || !valid_dtype(src_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && (dst == nullptr || src == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (dst == src && dst_dtype != src_dtype) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  if (!scale_plan_any(divisor, &scale, &k)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  return flat_launch(src_dtype, dst_dtype, scale, false, dst, src, n, k, static_cast<hipStream_t>(stream));
 }
 
 int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n, double post_factor,
