@@ -59,14 +59,191 @@ def numel_of(shape):
     return n
 
 
+def run_full_model(args) -> int:
+    """Full Llama-3-8B per-rank pass at logical W=8 on one GPU: embedding, 32 decoder layers, lm_head and
+    the final norm as 35 parameter groups.  Forward: copy-in + copy-out of group i+1 run on a side stream while a
+    bf16 [4096x4096]x[4096x4096] GEMM stands in for the compute of group i.  Backward (reverse order): two GEMMs
+    per group, then reduce copy-in on the compute stream and post-reduce on the side stream.  Reports the overlap
+    efficiency and per-kernel GB/s (un-overlapped)."""
+    import torch
+
+    from yafsdp_amd import _native
+    from yafsdp_amd._layout import make_layout
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w, r, align = 8, 3, 512
+    layer_shapes = WORKLOADS["llama3-8b-layer-w8"][0]
+    group_shapes = [[(128256, 4096)]] + [layer_shapes] * 32 + [[(128256, 4096)], [(4096,)]]
+    names = ["embed"] + [f"layer{i}" for i in range(32)] + ["lm_head", "norm"]
+    gen = torch.Generator(device=dev).manual_seed(1004)
+
+    def randn(n, std, dtype):
+        out = torch.empty(n, dtype=dtype, device=dev)
+        for i in range(0, n, 1 << 26):
+            m = min(1 << 26, n - i)
+            out[i : i + m] = (torch.randn(m, device=dev, generator=gen) * std).to(dtype)
+        return out
+
+    # per-shape shared resources (synthetic gathered buffers, gradients, output tensors and tables)
+    shape_res = {}
+    groups = []
+    for name, shapes in zip(names, group_shapes):
+        numels = [numel_of(s) for s in shapes]
+        key = tuple(numels)
+        lay = make_layout(numels, w, align)
+        if key not in shape_res:
+            t_pad = lay.padded_unsharded_numel
+            shape_res[key] = {
+                "lay": lay, "table": _native.TensorTable(numels, t_pad, dev),
+                "gathered": [randn(t_pad, 0.02, torch.bfloat16) for _ in range(2)],  # the 2 shared data buffers
+                "outs": [[torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels] for _ in range(2)],
+                "grads": [randn(n, 1e-3, torch.bfloat16) for n in numels],
+                "rs": torch.zeros(t_pad, dtype=torch.bfloat16, device=dev),  # the shared gradient buffer
+            }
+        s_ = lay.padded_sharded_numel
+        groups.append({
+            "name": name, "res": shape_res[key], "lay": lay,
+            "master": randn(s_, 0.02, torch.float32), "ag_in": torch.zeros(s_, dtype=torch.bfloat16, device=dev),
+            "shard": randn(s_, 1e-4, torch.float32),
+        })
+    log(f"{len(groups)} groups, {torch.cuda.memory_allocated() / 1e9:.1f} GB allocated")
+    a = randn(4096 * 4096, 0.02, torch.bfloat16).view(4096, 4096)
+    b = randn(4096 * 4096, 0.02, torch.bfloat16).view(4096, 4096)
+    c = torch.empty(4096, 4096, dtype=torch.bfloat16, device=dev)
+    side = torch.cuda.Stream(device=dev)  # default priority
+    main = torch.cuda.current_stream(dev)
+
+    def unshard(i):  # copy-in + copy-out of group i (current stream)
+        g = groups[i]
+        res = g["res"]
+        _native.flat_copy(g["ag_in"], g["master"])
+        res["table"].scatter_out(res["gathered"][i % 2], res["outs"][i % 2])
+
+    def reduce_in(i):
+        g = groups[i]
+        g["res"]["table"].gather_in(g["res"]["grads"], g["res"]["rs"], None, float(w), True)
+
+    def post(i):
+        g = groups[i]
+        s_ = g["lay"].padded_sharded_numel
+        _native.post_reduce(g["shard"], g["res"]["rs"][r * s_ : (r + 1) * s_], None, True)
+
+    n = len(groups)
+
+    def step(copies=True, gemms=True):
+        # forward
+        ready = [None] * n
+        if copies:
+            with torch.cuda.stream(side):
+                unshard(0)
+                ready[0] = side.record_event()
+        for i in range(n):
+            if copies and i + 1 < n:
+                with torch.cuda.stream(side):  # prefetch the next group while this one computes
+                    unshard(i + 1)
+                    ready[i + 1] = side.record_event()
+            if copies:
+                main.wait_event(ready[i])
+            if gemms:
+                torch.matmul(a, b, out=c)
+        # backward, reverse order
+        freed = None
+        for i in reversed(range(n)):
+            if gemms:
+                torch.matmul(a, b, out=c)
+                torch.matmul(a, b, out=c)
+            if copies:
+                if freed is not None:
+                    main.wait_event(freed)        # the single gradient buffer is released by the previous post-reduce
+                reduce_in(i)                      # compute stream, like the reference's foreach calls
+                done = main.record_event()
+                with torch.cuda.stream(side):     # reduce-scatter stream: waits for the compute stream
+                    side.wait_event(done)
+                    post(i)
+                    freed = side.record_event()
+
+    def timed(copies, gemms, reps):
+        for _ in range(2):
+            step(copies, gemms)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            step(copies, gemms)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    reps = max(1, args.steps // 10)
+    t_gemm = timed(False, True, reps)
+    sweep = {}
+    caps = (4096, 16, 8, 4, 2, 1) if args.sweep_grid_cap else (4096,)
+    for bpc in caps:  # grid cap of the copy kernels in workgroups per compute unit
+        _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, bpc)
+        _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, bpc)
+        tc = timed(True, False, reps)
+        tb = timed(True, True, reps)
+        sweep[bpc] = {"ms_copies_alone": round(tc, 3), "ms_overlapped": round(tb, 3),
+                      "overlap_efficiency": round(max(tc, t_gemm) / tb, 4)}
+        log(f"  grid cap {bpc:5d} workgroups/CU: copies alone {tc:.3f} ms, overlapped {tb:.3f} ms, "
+            f"efficiency {max(tc, t_gemm) / tb:.3f}")
+    best = min(sweep, key=lambda k: sweep[k]["ms_overlapped"])
+    _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, 4096)
+    _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, 4096)
+    t_copy, t_both = sweep[best]["ms_copies_alone"], sweep[best]["ms_overlapped"]
+    eff = max(t_copy, t_gemm) / t_both
+    hidden = (t_copy + t_gemm - t_both) / min(t_copy, t_gemm)
+    bytes_step = 0
+    for g in groups:
+        lay = g["lay"]
+        t_, tp, s_ = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+        bytes_step += s_ * 6 + 4 * t_ + (4 * t_ + 2 * (tp - t_)) + s_ * 10
+    log(f"copies alone {t_copy:.3f} ms ({bytes_step / t_copy / 1e6:.0f} GB/s), gemms alone {t_gemm:.3f} ms, "
+        f"overlapped {t_both:.3f} ms; overlap efficiency {eff:.3f}, hidden fraction {hidden:.3f}")
+    # per-kernel GB/s, un-overlapped, on a decoder layer group
+    kernels = {}
+    li = 5
+    lay = groups[li]["lay"]
+    t_, tp, s_ = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+    per = [("copy_in", lambda: _native.flat_copy(groups[li]["ag_in"], groups[li]["master"]), s_ * 6),
+           ("copy_out", lambda: groups[li]["res"]["table"].scatter_out(groups[li]["res"]["gathered"][1], groups[li]["res"]["outs"][1]), 4 * t_),
+           ("reduce_copy_in", lambda: reduce_in(li), 4 * t_ + 2 * (tp - t_)),
+           ("post_reduce", lambda: post(li), s_ * 10)]
+    for name, fn, nbytes in per:
+        ts = []
+        for _ in range(20):
+            unshard(0)  # 1.3 GB of other traffic in between
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); fn(); e1.record(); e1.synchronize()
+            ts.append(e0.elapsed_time(e1) * 1e3)
+        med = statistics.median(ts)
+        kernels[name] = {"us_median": round(med, 2), "GBps": round(nbytes / med / 1e3, 1)}
+    out = {
+        "metric": "overlap efficiency of the buffer path against a GEMM stand-in, full Llama-3-8B per-rank pass @W=8",
+        "value": round(eff, 4), "unit": "max(copies, gemms) / overlapped", "n_gpus": 1, "steps": reps, "warmup": 2,
+        "ms_per_step": round(t_both, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "llama3-8b-full-w8", "groups": n, "logical_world_size": w, "rank": r,
+                   "gemm": "bf16 4096x4096x4096, 1 per group forward, 2 per group backward"},
+        "ms_copies_alone": round(t_copy, 4), "ms_gemms_alone": round(t_gemm, 4), "ms_overlapped": round(t_both, 4),
+        "hidden_fraction": round(hidden, 4), "grid_cap_sweep": sweep, "grid_cap_used": best, "copy_GBps_alone": round(bytes_step / t_copy / 1e6, 1),
+        "copy_GBps_overlapped_lower_bound": round(bytes_step / t_both / 1e6, 1), "bytes_per_step": bytes_step,
+        "kernels": kernels,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="llama3-8b-layer-w8", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="llama3-8b-layer-w8", choices=sorted(WORKLOADS) + ["llama3-8b-full-w8"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
+    ap.add_argument("--sweep-grid-cap", action="store_true",
+                    help="llama3-8b-full-w8 only: repeat the overlap measurement with the copy kernels' grids capped "
+                         "at 16/8/4/2/1 workgroups per compute unit")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
@@ -82,6 +259,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         log("bench.py: no GPU visible; the buffer path has no CPU implementation to measure.")
         return 3
+    if args.workload == "llama3-8b-full-w8":
+        return run_full_model(args)
     from yafsdp_amd import _native
     from yafsdp_amd._layout import make_layout
 
