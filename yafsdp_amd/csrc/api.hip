@@ -124,8 +124,8 @@ namespace {
 void table_free(yafsdp_table* t) {
   if (t == nullptr) return;
   if (t->d_offsets) (void)hipFree(t->d_offsets);
-  for (int i = 0; i < 2; i++)
-    if (t->d_tiles[i]) (void)hipFree(t->d_tiles[i]);
+  if (t->d_tiles[1] && t->d_tiles[1] != t->d_tiles[0]) (void)hipFree(t->d_tiles[1]);
+  if (t->d_tiles[0]) (void)hipFree(t->d_tiles[0]);
   for (int i = 0; i < yafsdp_table::kRing; i++) {
     if (t->ev[i]) (void)hipEventDestroy(t->ev[i]);
     if (t->h_stage[i]) (void)hipHostFree(t->h_stage[i]);
@@ -351,6 +351,10 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
       // per tile: first tensor whose end lies beyond the tile's first element
       const int64_t n_tiles = t->n_tiles[w];
       if (n_tiles == 0) continue;
+      if (w == 1 && tile_elems[1] == tile_elems[0]) {  // same tile size: one array serves both kernels
+        t->d_tiles[1] = t->d_tiles[0];
+        continue;
+      }
       tiles.resize(size_t(n_tiles));
       int p = 0;
       for (int64_t tile = 0; tile < n_tiles; tile++) {

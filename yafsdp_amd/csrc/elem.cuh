@@ -238,9 +238,17 @@ __device__ __forceinline__ Quad<T> pack_quad(const float (&f)[4]) {
 template <class S, class D>
 struct wide_pair { static constexpr bool value = (S::kSize == 4 || D::kSize == 4); };
 
+// unit index of the j-th unit (0 .. U-1) of this lane inside a tile of BLOCK*U
+// units: lane-strided by BLOCK, so consecutive waves own consecutive 1 KiB
+// spans.  (Giving each wave U consecutive spans instead measured 0-2 % slower.)
+template <int BLOCK, int U>
+__device__ __forceinline__ int unit_index(int j) {
+  return int(threadIdx.x) + j * BLOCK;
+}
+
 // byte-free element index of quad q (0 .. 2U-1) of this lane inside a tile of
 // BLOCK*U units: wave tiles of 512 elements, two quads per lane per wave tile
-template <int BLOCK>
+template <int BLOCK, int U = 1>
 __device__ __forceinline__ int quad_elem(int q) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   return ((q >> 1) * (BLOCK / 64) + wave) * 512 + (q & 1) * 256 + lane * 4;

@@ -67,27 +67,26 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
     Quad<S> s[2 * U];
     Quad<D> d[2 * U];
 #pragma unroll
-    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK>(q) * S::kSize);
+    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK, U>(q) * S::kSize);
     if constexpr (ACC) {
 #pragma unroll
-      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dst + quad_elem<BLOCK>(q) * D::kSize);
+      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dst + quad_elem<BLOCK, U>(q) * D::kSize);
     }
 #pragma unroll
     for (int q = 0; q < 2 * U; q++)
-      store_quad<D, NTS>(dst + quad_elem<BLOCK>(q) * D::kSize, flat_quad<S, D, SCALE, ACC>(s[q], d[q], k));
+      store_quad<D, NTS>(dst + quad_elem<BLOCK, U>(q) * D::kSize, flat_quad<S, D, SCALE, ACC>(s[q], d[q], k));
   } else {
-    const int tid = threadIdx.x;
     Unit<S> s[U];
     Unit<D> d[U];
 #pragma unroll
-    for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + (tid + j * BLOCK) * (8 * S::kSize));
+    for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + unit_index<BLOCK, U>(j) * (8 * S::kSize));
     if constexpr (ACC) {
 #pragma unroll
-      for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dst + (tid + j * BLOCK) * (8 * D::kSize));
+      for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize));
     }
 #pragma unroll
     for (int j = 0; j < U; j++)
-      store_unit<D, NTS>(dst + (tid + j * BLOCK) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
+      store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
   }
 }
 

@@ -165,31 +165,30 @@ __device__ __forceinline__ void gather_full_tile(char* dst, const char* src, flo
     Quad<D> d[2 * U];
     if constexpr (kReadSrc) {
 #pragma unroll
-      for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK>(q) * S::kSize);
+      for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK, U>(q) * S::kSize);
     }
     if constexpr (kReadDst) {
 #pragma unroll
-      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dst + quad_elem<BLOCK>(q) * D::kSize);
+      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dst + quad_elem<BLOCK, U>(q) * D::kSize);
     }
 #pragma unroll
     for (int q = 0; q < 2 * U; q++)
-      store_quad<D, NTS>(dst + quad_elem<BLOCK>(q) * D::kSize, gather_quad<S, D, SCALE, MODE>(s[q], d[q], k));
+      store_quad<D, NTS>(dst + quad_elem<BLOCK, U>(q) * D::kSize, gather_quad<S, D, SCALE, MODE>(s[q], d[q], k));
     return;
   }
-  const int tid = threadIdx.x;
   Unit<S> s[U];
   Unit<D> d[U];
   if constexpr (kReadSrc) {
 #pragma unroll
-    for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + (tid + j * BLOCK) * (8 * S::kSize));
+    for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + unit_index<BLOCK, U>(j) * (8 * S::kSize));
   }
   if constexpr (kReadDst) {
 #pragma unroll
-    for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dst + (tid + j * BLOCK) * (8 * D::kSize));
+    for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize));
   }
 #pragma unroll
   for (int j = 0; j < U; j++)
-    store_unit<D, NTS>(dst + (tid + j * BLOCK) * (8 * D::kSize), gather_unit<S, D, SCALE, MODE>(s[j], d[j], k));
+    store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), gather_unit<S, D, SCALE, MODE>(s[j], d[j], k));
 }
 
 // n elements; dst points at flat element `flat_index`, src at the matching
@@ -271,20 +270,19 @@ __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
     Quad<S> s[2 * U];
     Quad<D> unused_q;
 #pragma unroll
-    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK>(q) * S::kSize);
+    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK, U>(q) * S::kSize);
 #pragma unroll
     for (int q = 0; q < 2 * U; q++)
-      store_quad<D, NTS>(dst + quad_elem<BLOCK>(q) * D::kSize, flat_quad<S, D, SCALE_NONE, false>(s[q], unused_q, 0.f));
+      store_quad<D, NTS>(dst + quad_elem<BLOCK, U>(q) * D::kSize, flat_quad<S, D, SCALE_NONE, false>(s[q], unused_q, 0.f));
     return;
   }
-  const int tid = threadIdx.x;
   Unit<S> s[U];
   Unit<D> unused;
 #pragma unroll
-  for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + (tid + j * BLOCK) * (8 * S::kSize));
+  for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + unit_index<BLOCK, U>(j) * (8 * S::kSize));
 #pragma unroll
   for (int j = 0; j < U; j++)
-    store_unit<D, NTS>(dst + (tid + j * BLOCK) * (8 * D::kSize), flat_unit<S, D, SCALE_NONE, false>(s[j], unused, 0.f));
+    store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE_NONE, false>(s[j], unused, 0.f));
 }
 
 template <class S, class D, int BLOCK, bool NTL, bool NTS>

@@ -11,10 +11,11 @@ constexpr bool kFlatNtStore = true;
 // gather-in / scatter-out: a tile is block * unroll * 8 elements.  Measured with
 // non-zero data and the four kernels of a step running back to back: tiles of
 // 1-2 K elements (2-4 KiB of bf16) in workgroups of one or two waves are the
-// fastest for both kernels; larger workgroups lose 3-10 %.  (All-zero buffers
+// fastest for both kernels (one wave x 2 units ahead by about 1 %); larger
+// workgroups lose 3-10 %.  (All-zero buffers
 // run up to 10 % faster than any other content on this memory system and must
 // not be used for tuning.)
-constexpr int kTableBlock = 128;
+constexpr int kTableBlock = 64;
 constexpr int kGatherUnroll = 2;
 constexpr int kScatterUnroll = 2;
 constexpr bool kTableNtLoad = true;
