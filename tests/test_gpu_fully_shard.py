@@ -1,0 +1,219 @@
+"""``fully_shard`` on one GPU: a wrapped model trains through the buffer
+kernels and its master weights stay bit-identical to a hand-written mixed
+precision loop that performs the same arithmetic with plain torch ops."""
+
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+from yafsdp_amd import MixedPrecisionPolicy, make_layout
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+class Block(nn.Module):
+    def __init__(self, d, h):
+        super().__init__()
+        self.up = nn.Linear(d, h)
+        self.down = nn.Linear(h, d, bias=False)
+
+    def forward(self, x):
+        return x + self.down(torch.relu(self.up(x)))
+
+
+class Net(nn.Module):
+    def __init__(self, d=128, h=256, layers=3):
+        super().__init__()
+        self.blocks = nn.ModuleList([Block(d, h) for _ in range(layers)])
+        self.norm = nn.LayerNorm(d)
+
+    def forward(self, x):
+        for b in self.blocks:
+            x = b(x)
+        return self.norm(x)
+
+
+def _make(seed=0):
+    torch.manual_seed(seed)
+    return Net().to(DEV)
+
+
+def _wrap(model, **kw):
+    from yafsdp_amd import fully_shard
+
+    for b in model.blocks:
+        fully_shard(b, **kw)
+    fully_shard(model.norm, **kw)
+    return fully_shard(model, **kw)  # the root holds no parameters of its own: siblings only
+
+
+def _reference_steps(model0, xs, lr, accumulate_pairs=False):
+    """fp32 masters; bf16 compute copies; bf16 gradients (summed in bf16 over the micro-batches of a step, as
+    the reduce buffer does) upcast into fp32; SGD on the masters."""
+    ref = copy.deepcopy(model0)
+    masters = [p for p in ref.parameters()]
+    opt = torch.optim.SGD(masters, lr=lr)
+    micro = 2 if accumulate_pairs else 1
+    for i in range(0, len(xs), micro):
+        acc = None
+        for x in xs[i : i + micro]:
+            lowp = copy.deepcopy(ref).to(torch.bfloat16)
+            y = lowp(x.to(torch.bfloat16))
+            y.float().pow(2).mean().backward()
+            grads = [p.grad for p in lowp.parameters()]
+            if acc is None:
+                acc = [g.clone() for g in grads]          # view.copy_(grad)
+            else:
+                for a, g in zip(acc, grads):
+                    a.add_(g)                             # view.add_(grad): bf16 result
+        for m, a in zip(masters, acc):
+            m.grad = a.float()                            # shard.copy_(chunk): exact upcast
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    return ref
+
+
+def _gather_full(model):
+    """Full fp32 master values per original parameter name, read back from the flat shards (W=1)."""
+    from yafsdp_amd.fully_shard import YaFSDPModule
+
+    out = {}
+    for mod in model.modules():
+        if isinstance(mod, YaFSDPModule) and (group := mod._get_fsdp_state()._fsdp_param_group) is not None:
+            for fp in group.fsdp_params:
+                out[fp._param_fqn] = fp._sharded_param_data.detach().view(fp._orig_size).clone()
+    return out
+
+
+MP = MixedPrecisionPolicy(param_dtype=torch.bfloat16, cast_forward_inputs=True)
+
+
+def test_training_is_bit_identical_to_manual_mixed_precision():
+    model0 = _make()
+    xs = [torch.randn(16, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(s)) for s in range(4)]
+    ref = _reference_steps(model0, xs, lr=0.05)
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    # the optimizer sees one fp32 1-D shard per original parameter
+    params = list(model.parameters())
+    assert all(p.dtype == torch.float32 and p.dim() == 1 for p in params)
+    assert sum(p.numel() for p in params) == sum(p.numel() for p in model0.parameters())
+    opt = torch.optim.SGD(params, lr=0.05)
+    for x in xs:
+        y = model(x)
+        assert y.dtype == torch.bfloat16
+        y.float().pow(2).mean().backward()
+        assert all(p.grad is not None and p.grad.dtype == torch.float32 for p in params)
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    got = _gather_full(model)
+    want = dict(ref.named_parameters())
+    assert set(got) == set(want)
+    for k in want:
+        assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
+
+
+def test_gradient_accumulation_without_sync():
+    model0 = _make(1)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(10 + s)) for s in range(4)]
+    ref = _reference_steps(model0, xs, lr=0.02, accumulate_pairs=True)
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    params = list(model.parameters())
+    opt = torch.optim.SGD(params, lr=0.02)
+    # unreduced gradients stay in the reduce buffer between micro-batches: one buffer per group
+    model._get_fsdp_state()._lazy_init(allow_no_grad_reduce=True)
+    for i in range(0, 4, 2):
+        model.set_requires_gradient_sync(False)
+        model.set_is_last_backward(False)
+        model(xs[i]).float().pow(2).mean().backward()          # accumulate in the unsharded reduce buffers... 
+        model.set_requires_gradient_sync(True)
+        model.set_is_last_backward(True)
+        model(xs[i + 1]).float().pow(2).mean().backward()      # ...then reduce once
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    got, want = _gather_full(model), dict(ref.named_parameters())
+    assert set(got) == set(want)
+    for k in want:
+        assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
+
+
+def test_module_api_and_states():
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.fully_shard import YaFSDPModule
+
+    model = _wrap(_make(2), mp_policy=MP)
+    assert isinstance(model, YaFSDPModule) and type(model).__name__ == "YaFSDPNet"
+    assert isinstance(model.blocks[0], YaFSDPModule)
+    with pytest.raises(AssertionError, match="deepcopy"):
+        copy.deepcopy(model)
+    with pytest.raises(ValueError, match="containers"):
+        fully_shard(nn.ModuleList([nn.Linear(2, 2)]))
+    with pytest.raises(AssertionError, match="already"):
+        fully_shard(model.blocks[0])
+    x = torch.randn(4, 128, device=DEV)
+    model(x).float().sum().backward()  # the first pass through the root allocates the shared buffers
+    # explicit unshard / reshard
+    blk = model.blocks[1]
+    handle = blk.unshard(async_op=True)
+    handle.wait()
+    assert blk.up.weight.dtype == torch.bfloat16 and blk.up.weight.shape == (256, 128)
+    blk.reshard()
+    assert blk.up.weight.dtype == torch.float32 and blk.up.weight.dim() == 1
+    # the last user of each data buffer keeps its parameters unsharded after forward
+    model(x)
+    groups = [m._get_fsdp_state()._fsdp_param_group for m in [*model.blocks, model.norm]]
+    assert [g.is_unsharded for g in groups] == [False, False, True, True]
+    for m in (model.blocks[2], model.norm):
+        m.reshard()  # a forward without a backward leaves them holding both data buffers
+    model.set_reshard_after_forward(True)
+    model(x)
+    assert all(g.is_sharded for g in groups)
+    with pytest.raises(ValueError):
+        model.set_reshard_after_forward("yes")
+    with pytest.raises(ValueError):
+        model.set_modules_to_forward_prefetch([nn.Linear(2, 2)])
+    model.blocks[0].set_modules_to_forward_prefetch([model.blocks[1]])
+    model.blocks[2].set_modules_to_backward_prefetch([model.blocks[1]])
+    model(x).float().sum().backward()
+    torch.cuda.synchronize()
+    assert all(p.grad is not None for p in model.parameters())
+
+
+def test_nested_groups_must_not_share_a_buffer():
+    from yafsdp_amd import fully_shard
+
+    model = _make(5)
+    for b in model.blocks:
+        fully_shard(b, mp_policy=MP)
+    fully_shard(model, mp_policy=MP)  # the root now owns `norm` and stays unsharded while its children run
+    with pytest.raises(RuntimeError, match="share a (data|grad) buffer"):
+        model(torch.randn(2, 128, device=DEV))  # ya_fsdp/_state.py:375-384
+
+
+def test_lazy_init_requires_root_first():
+    model = _wrap(_make(3), mp_policy=MP)
+    with pytest.raises(RuntimeError, match="root module first"):
+        model.blocks[0](torch.randn(2, 128, device=DEV))
+        model(torch.randn(2, 128, device=DEV))
+
+
+def test_logical_world_size_gives_each_rank_its_ragged_shard():
+    from yafsdp_amd import fully_shard
+
+    model0 = _make(4)
+    full = torch.cat([p.detach().view(-1) for p in model0.blocks[0].parameters()])
+    numels = [p.numel() for p in model0.blocks[0].parameters()]
+    w = 3
+    lay = make_layout(numels, w, 8)
+    pieces = []
+    for r in range(w):
+        blk = copy.deepcopy(model0.blocks[0])
+        fully_shard(blk, mesh=(w, r), mp_policy=MP)
+        sharded = list(blk.parameters())
+        assert [p.numel() for p in sharded] == lay.sharded_numels(r)
+        pieces.append(torch.cat([p.detach() for p in sharded]))
+    assert torch.equal(torch.cat(pieces), full)  # the ranks' fragments tile the flat parameter space

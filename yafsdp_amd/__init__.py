@@ -28,6 +28,9 @@ __all__ = [
     "all_gather",
     "reduce_scatter",
     "AllGatherResult",
+    "fully_shard",
+    "YaFSDPModule",
+    "UnshardHandle",
 ]
 
 _LAZY = {
@@ -38,6 +41,9 @@ _LAZY = {
     "all_gather": "_collectives",
     "reduce_scatter": "_collectives",
     "AllGatherResult": "_collectives",
+    "fully_shard": "fully_shard",
+    "YaFSDPModule": "fully_shard",
+    "UnshardHandle": "fully_shard",
 }
 
 
@@ -45,5 +51,7 @@ def __getattr__(name):
     if name in _LAZY:
         import importlib
 
-        return getattr(importlib.import_module(f"{__name__}.{_LAZY[name]}"), name)
+        value = getattr(importlib.import_module(f"{__name__}.{_LAZY[name]}"), name)
+        globals()[name] = value  # also replaces the submodule of the same name (fully_shard)
+        return value
     raise AttributeError(f"module {__name__!r} has no attribute {name!r}")

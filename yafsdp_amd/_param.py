@@ -5,6 +5,8 @@ what the buffer path touches: no DTensor wrapping, no module attribute swaps).
 
 from __future__ import annotations
 
+from dataclasses import dataclass, field
+
 import torch
 import torch.nn as nn
 
@@ -13,12 +15,27 @@ from ._common import FSDPMeshInfo, ShardedState
 from ._layout import RaggedShard
 
 
+@dataclass
+class ParamModuleInfo:
+    """Where a parameter is registered, so that the sharded / unsharded views
+    can be swapped in with ``setattr`` (ya_fsdp/_param.py:20-31); shared
+    (tied) registrations are listed as well."""
+
+    module: nn.Module
+    param_name: str
+    shared_modules: list[nn.Module] = field(default_factory=list)
+    shared_param_names: list[str] = field(default_factory=list)
+
+
 class YaFSDPParam:
     orig_dtype: torch.dtype
     param_dtype: torch.dtype | None
     reduce_dtype: torch.dtype | None
 
-    def __init__(self, param: torch.Tensor, mesh_info: FSDPMeshInfo, device: torch.device, name: str | None = None):
+    def __init__(
+        self, param: torch.Tensor, mesh_info: FSDPMeshInfo, device: torch.device, name: str | None = None,
+        module_info: ParamModuleInfo | None = None,
+    ):
         if param.device != device:
             raise AssertionError(
                 f"Expects the parameter to already be moved to device {device} but got {param.device}"
@@ -31,6 +48,7 @@ class YaFSDPParam:
             raise ValueError("Change the scalar parameter to a 1D tensor with numel equal to 1.")  # _init.py:156-161
         self.param = param
         self.param_data = param
+        self._module_info = module_info
         self.mesh_info = mesh_info
         self.device = device
         self._param_fqn = name
@@ -68,6 +86,7 @@ class YaFSDPParam:
         self.sharded_param = nn.Parameter(sharded_param_data, requires_grad=self.requires_grad)
         self.sharded_param_grad = sharded_param_grad if self.requires_grad else None
         del self.param, self.param_data  # the group's flat shard now owns the values
+        self._setattr_on_modules(self.sharded_param)
 
     def init_all_gather_input(self, all_gather_input: torch.Tensor) -> None:
         self._all_gather_input = all_gather_input
@@ -93,10 +112,39 @@ class YaFSDPParam:
             raise AssertionError(f"Expects to be in SHARDED, not {self.sharded_state}")
 
     def to_sharded(self) -> None:
+        self._setattr_on_modules(self.sharded_param)
         self.sharded_state = ShardedState.SHARDED
 
     def to_unsharded(self) -> None:
+        self._setattr_on_modules(self.unsharded_param)
         self.sharded_state = ShardedState.UNSHARDED
+
+    def _setattr_on_modules(self, param: nn.Parameter) -> None:
+        """ya_fsdp/_param.py:259-268."""
+        info = self._module_info
+        if info is None:
+            return
+        unsafe_setattr_param(info.module, info.param_name, param)
+        for shared_module, shared_param_name in zip(info.shared_modules, info.shared_param_names):
+            unsafe_setattr_param(shared_module, shared_param_name, param)
+
+    def reset_sharded_param(self) -> None:
+        """Re-sync after ``module._apply`` replaced the registered parameter
+        (ya_fsdp/_param.py:345-357): copy its values back into the flat shard."""
+        info = self._module_info
+        if info is None:
+            return
+        new_param = getattr(info.module, info.param_name)
+        if new_param.data_ptr() != self._sharded_param_data.data_ptr() and self.sharded_numel > 0:
+            from . import _native
+
+            if new_param.device != self._sharded_param_data.device or new_param.numel() != self.sharded_numel:
+                raise NotImplementedError(
+                    "moving a sharded module to another device or changing its parameter sizes is not supported"
+                )
+            _native.flat_copy(self._sharded_param_data, new_param.detach().contiguous().view(-1))
+        self.sharded_param = nn.Parameter(self._sharded_param_data, requires_grad=self.sharded_param.requires_grad)
+        self._setattr_on_modules(self.sharded_param)
 
     @property
     def unsharded_grad_data(self) -> torch.Tensor:
@@ -107,3 +155,12 @@ class YaFSDPParam:
 
     def __repr__(self) -> str:
         return f"YaFSDPParam(fqn={self._param_fqn}, orig_size={self._orig_size})"
+
+
+def unsafe_setattr_param(module: nn.Module, param_name: str, param: nn.Parameter) -> None:
+    """ya_fsdp/_param.py:363-372: skip ``nn.Module.__setattr__`` checks when the
+    module does not override it."""
+    if getattr(module.__setattr__, "__func__", None) is nn.Module.__setattr__:
+        module._parameters[param_name] = param
+    else:
+        setattr(module, param_name, param)

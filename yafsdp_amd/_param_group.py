@@ -21,8 +21,9 @@ What differs
   * the side stream has the default priority (the reference asks for a
     high-priority stream, :80-88; mixed stream priorities are avoided on this
     platform);
-  * module hooks, DTensor wrapping, state-dict hooks and YCCL are outside this
-    build: a group is constructed from a list of tensors.
+  * DTensor wrapping, state-dict hooks and YCCL are outside this build: a group
+    is constructed from a list of tensors (optionally with the modules that own
+    them, so that sharded / unsharded views are swapped in on the modules).
 """
 
 from __future__ import annotations
@@ -49,7 +50,7 @@ from ._collectives import (
 )
 from ._common import FSDPMeshInfo, ShardedState, TrainingState, is_bw
 from ._layout import ShardLayout, make_layout
-from ._param import YaFSDPParam
+from ._param import ParamModuleInfo, YaFSDPParam
 
 logger = logging.getLogger("yafsdp_amd")
 
@@ -108,6 +109,7 @@ class YaFSDPParamGroup:
         shard_alignment: int = 8,
         names: Sequence[str] | None = None,
         module_fqn: str | None = None,
+        modules: tuple = (),
     ):
         device = torch.device(device)
         if device.type != "cuda":
@@ -115,7 +117,9 @@ class YaFSDPParamGroup:
         if mp_policy.all_gather_dtype_to_param_cls:
             raise NotImplementedError("per-class all-gather dtypes (tensor-subclass extensions) are not part of this build")
         names = list(names) if names is not None else [f"param{i}" for i in range(len(params))]
-        self.fsdp_params = [YaFSDPParam(p, mesh_info, device, n) for p, n in zip(params, names)]
+        self.modules = tuple(modules)
+        infos = _get_param_module_infos(list(params), self.modules) if self.modules else [None] * len(params)
+        self.fsdp_params = [YaFSDPParam(p, mesh_info, device, n, mi) for p, n, mi in zip(params, names, infos)]
         self.mesh_info = mesh_info
         self.device = device
         self.mp_policy = mp_policy
@@ -319,20 +323,47 @@ class YaFSDPParamGroup:
         self.data_buffer_ctx.release_event = torch.cuda.current_stream(self.device).record_event()
         self.data_buffer_ctx.owner = None
 
-    def pre_forward(self) -> None:
-        """ya_fsdp/_param_group.py:617-626 without the autograd hook registration."""
+    def pre_forward(self, module: Any = None, args: tuple = (), kwargs: dict | None = None):
+        """ya_fsdp/_param_group.py:617-626.  Called without arguments it only
+        unshards; with the hook arguments it also registers the post-backward
+        hook on the inputs and returns ``(args, kwargs)``."""
+        kwargs = {} if kwargs is None else kwargs
         with record_function(self._with_fqn("YaFSDP::pre_forward")):
             self._training_state = TrainingState.FORWARD
             self.unshard(self.unshard_async_op)
             self.wait_for_unshard()
+            if module is not None:
+                args, kwargs = self._register_post_backward_hook(args, kwargs)
+            return args, kwargs
 
-    def post_forward(self) -> None:
+    def post_forward(self, module: Any = None, input: Any = None, output: Any = None) -> Any:
         """ya_fsdp/_param_group.py:628-635."""
         with record_function(self._with_fqn("YaFSDP::post_forward")):
             if not is_bw():
                 self.reshard()
                 self._record_post_forward()
             self._training_state = TrainingState.IDLE
+            return output
+
+    def _register_post_backward_hook(self, args: tuple, kwargs: dict) -> tuple[tuple, dict]:
+        """ya_fsdp/_param_group.py:859-884: route the inputs that require
+        gradients through an autograd node whose backward runs post_backward."""
+        if not torch.is_grad_enabled():
+            return args, kwargs
+        from torch.utils._pytree import tree_flatten, tree_unflatten
+
+        args_list, args_spec = tree_flatten(args)
+        kwargs_list, kwargs_spec = tree_flatten(kwargs)
+        flat = list(args_list) + list(kwargs_list)
+        idx = [i for i, obj in enumerate(flat) if torch.is_tensor(obj) and obj.requires_grad]
+        if not idx:
+            return args, kwargs
+        outs = RegisterPostBackwardFunction.apply(self, *[flat[i] for i in idx])
+        for i, t in zip(idx, outs):
+            flat[i] = t
+        args = tree_unflatten(flat[: len(args_list)], args_spec)
+        kwargs = tree_unflatten(flat[len(args_list) :], kwargs_spec)
+        return args, kwargs
 
     def _record_post_forward(self) -> None:
         post_forward_index = len(self.comm_ctx.post_forward_order)
@@ -523,6 +554,40 @@ class YaFSDPParamGroup:
 
     def __repr__(self) -> str:
         return f"YaFSDPParamGroup(fqn={self._module_fqn})"
+
+
+def _get_param_module_infos(params: list, modules: tuple) -> list:
+    """ya_fsdp/_param_group.py:942-968."""
+    from torch.distributed.fsdp._common_utils import _named_parameters_with_duplicates
+
+    params_set = {id(p) for p in params}
+    info: dict[int, ParamModuleInfo] = {}
+    for module in modules:
+        for _, submodule in module.named_modules(remove_duplicate=False):
+            for param_name, param in _named_parameters_with_duplicates(submodule, recurse=False):
+                if id(param) in params_set:
+                    if id(param) not in info:
+                        info[id(param)] = ParamModuleInfo(submodule, param_name)
+                    else:
+                        info[id(param)].shared_modules.append(submodule)
+                        info[id(param)].shared_param_names.append(param_name)
+    if len(info) != len(params):
+        raise AssertionError(f"Some parameters are not in the module tree of {modules}")
+    return [info[id(p)] for p in params]
+
+
+class RegisterPostBackwardFunction(torch.autograd.Function):
+    """ya_fsdp/_param_group.py:971-992."""
+
+    @staticmethod
+    def forward(ctx: Any, param_group: YaFSDPParamGroup, *inputs: torch.Tensor):
+        ctx.param_group = param_group
+        return inputs
+
+    @staticmethod
+    def backward(ctx: Any, *grads: torch.Tensor):
+        ctx.param_group.post_backward()
+        return (None, *grads)
 
 
 def init_shared_state(

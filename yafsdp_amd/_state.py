@@ -1,0 +1,330 @@
+"""Per-module state machine of ``fully_shard`` (mirror of ya_fsdp/_state.py):
+forward pre/post hooks, pre-backward tensor hooks, the root post-backward
+callback, lazy initialisation of the shared communication context and buffers.
+All host control flow; the bytes move in ``_param_group`` / ``_collectives``."""
+
+from __future__ import annotations
+
+import functools
+import logging
+from typing import Any
+
+import torch
+import torch.nn as nn
+from torch.autograd import Variable
+from torch.distributed._composable_state import _get_module_state, _insert_module_state, _State
+from torch.distributed.utils import _apply_to_tensors, _to_kwargs
+from torch.utils._pytree import tree_flatten
+
+from ._api import MixedPrecisionPolicy
+from ._common import TrainingState
+from ._param_group import YaFSDPCommContext, YaFSDPParamGroup
+
+logger = logging.getLogger("yafsdp_amd")
+
+
+class YaFSDPStateContext:
+    """ya_fsdp/_state.py:39-53."""
+
+    def __init__(self) -> None:
+        self.all_states: list[YaFSDPState] = []
+        self.iter_forward_root: YaFSDPState | None = None
+        self.post_backward_final_callback_queued: bool = False
+        self.is_last_backward: bool = True
+        self.post_optim_event: torch.cuda.Event | None = None
+
+
+def _cast_fp_tensor(dtype: torch.dtype, x: Any) -> Any:
+    """ya_fsdp/_common.py:63-70."""
+    if not isinstance(x, torch.Tensor) or not torch.is_floating_point(x) or x.dtype == dtype:
+        return x
+    return x.to(dtype)
+
+
+class YaFSDPState(_State):
+    def __init__(self) -> None:
+        super().__init__()
+        self._fsdp_param_group: YaFSDPParamGroup | None = None
+        self._is_root: bool | None = None  # set during lazy init
+        self._state_ctx = YaFSDPStateContext()
+        self._comm_ctx = YaFSDPCommContext()
+        self._training_state: TrainingState = TrainingState.IDLE
+        self._states_to_forward_prefetch: list[YaFSDPState] = []
+        self._states_to_backward_prefetch: list[YaFSDPState] = []
+        self._auto_reshard_after_forward: bool | None = True
+
+    def init(self, modules: tuple, device: torch.device, mp_policy: MixedPrecisionPolicy,
+             auto_reshard_after_forward: bool) -> None:
+        """ya_fsdp/_state.py:72-101 for a single module per call."""
+        if len(modules) != 1:
+            raise NotImplementedError("fully_shard over a list of modules is not part of this build")
+        for module in modules:
+            _insert_module_state(module, self)
+        self._modules = modules
+        self._device = device
+        self._mp_policy = mp_policy
+        self._auto_reshard_after_forward = auto_reshard_after_forward
+        self._pre_forward_hook_handle = modules[0].register_forward_pre_hook(
+            self._pre_forward, prepend=True, with_kwargs=True
+        )
+        self._post_forward_hook_handle = modules[0].register_forward_hook(self._post_forward, prepend=False)
+
+    # ---------------------------------------------------------------- lazy init --
+    def _root_pre_forward(self, module: nn.Module, args: tuple, kwargs: dict) -> tuple[tuple, dict]:
+        """ya_fsdp/_state.py:103-125."""
+        self._lazy_init()
+        if self._state_ctx.iter_forward_root is not None:
+            return args, kwargs
+        self._state_ctx.iter_forward_root = self
+        with torch.profiler.record_function("YaFSDP::root_pre_forward"):
+            if (event := self._state_ctx.post_optim_event) is not None:
+                self._comm_ctx.all_gather_stream.wait_event(event)
+                self._state_ctx.post_optim_event = None
+            else:
+                # wait for the optimizer step before the implicitly prefetched unshards
+                self._comm_ctx.all_gather_stream.wait_stream(torch.cuda.current_stream(self._device))
+            with torch.profiler.record_function("YaFSDP::inputs_to_device"):
+                args_tuple, kwargs_tuple = _to_kwargs(args, kwargs, self._device, False)
+            args, kwargs = args_tuple[0], kwargs_tuple[0]
+        return args, kwargs
+
+    def _lazy_init(self, allow_no_grad_reduce: bool = False) -> None:
+        """ya_fsdp/_state.py:127-175.  ``allow_no_grad_reduce`` gives every group
+        its own gradient buffer, which gradient accumulation without
+        synchronisation needs (the unreduced gradients live in that buffer)."""
+        if self._is_root is not None:
+            return
+        self._is_root = True
+        root_module = self._modules[0]
+        visited_states: set[YaFSDPState] = set()
+        for module_name, module in root_module.named_modules():
+            if (state := _get_module_fsdp_state(module)) is None:
+                continue
+            if module is not root_module:
+                if state not in visited_states and state._is_root is not None:
+                    raise RuntimeError(
+                        "YaFSDP state has already been lazily initialized for "
+                        f"{module_name}\nYaFSDP requires running forward through the root module first"
+                    )
+                state._is_root = False
+            if state not in visited_states:
+                self._state_ctx.all_states.append(state)
+            visited_states.add(state)
+        self._init_fqns()
+        self._init_shared_state(allow_no_grad_reduce)
+        self.validate_shared_state()
+        for state in self._state_ctx.all_states:
+            if state._fsdp_param_group:
+                state._fsdp_param_group.lazy_init()
+
+    def _init_shared_state(self, allow_no_grad_reduce: bool = False) -> None:
+        """ya_fsdp/_state.py:177-288 and :617-678: one communication context;
+        two data buffers handed out round-robin in module order and one gradient
+        buffer, each as large as the largest group that uses it; the last group on
+        each data buffer keeps its parameters unsharded after forward."""
+        self._comm_ctx.lazy_init(self._device)
+        for state in self._state_ctx.all_states:
+            state._state_ctx = self._state_ctx
+            state._comm_ctx = self._comm_ctx
+            if group := state._fsdp_param_group:
+                group.comm_ctx = self._comm_ctx
+        param_groups = [s._fsdp_param_group for s in self._state_ctx.all_states if s._fsdp_param_group is not None]
+        if not param_groups:
+            return
+        no_reshard_after_forward = all(not g.reshard_after_forward for g in param_groups)
+
+        def assign(groups, attr, count, size_of):
+            if not groups:
+                return []
+            n = len(groups) if count is None else min(count, len(groups))
+            ctxs = [getattr(groups[i], attr) for i in range(n)]
+            users = [[] for _ in range(n)]
+            for i, g in enumerate(groups):
+                users[i % n].append(g)
+            for ctx, gs in zip(ctxs, users):
+                ctx.lazy_init({None: max(size_of(g) for g in gs)}, self._device)
+                for g in gs:
+                    setattr(g, attr, ctx)
+            return users
+
+        data_users = assign(param_groups, "data_buffer_ctx", None if no_reshard_after_forward else 2,
+                            lambda g: g.data_buffer_bytes())
+        for state_groups in data_users:
+            last = state_groups[-1]
+            owner_state = next(s for s in self._state_ctx.all_states if s._fsdp_param_group is last)
+            if owner_state._auto_reshard_after_forward:
+                last.reshard_after_forward = False  # ya_fsdp/_state.py:256-260
+        assign([g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx",
+               None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes())
+
+    def validate_shared_state(self) -> None:
+        """ya_fsdp/_state.py:290-414: enough buffers for overlap; at most one
+        group per shared buffer may skip resharding / reducing; and two groups
+        that are unsharded at the same time (a module and one of its
+        descendants) must not share a buffer."""
+        data_users: dict[Any, list[YaFSDPParamGroup]] = {}
+        grad_users: dict[Any, list[YaFSDPParamGroup]] = {}
+        for state in self._state_ctx.all_states:
+            if (group := state._fsdp_param_group) is None:
+                continue
+            data_users.setdefault(group.data_buffer_ctx, []).append(group)
+            if group.grad_buffer_ctx is not None:
+                grad_users.setdefault(group.grad_buffer_ctx, []).append(group)
+        num_groups = sum(map(len, data_users.values()))
+        if len(data_users) < min(2, num_groups):
+            raise ValueError(
+                "num_data_buffers must be no less than min(2, num_param_groups)"
+                f" for correct overlap, but got num_data_buffers={len(data_users)} num_param_groups={num_groups}."
+            )
+        for groups in data_users.values():
+            if len(bad := [g for g in groups if not g.reshard_after_forward]) > 1:
+                raise ValueError(
+                    "Only one parameter group across groups which share a data buffer"
+                    f" is allowed to have no reshard after forward, but got {bad}"
+                )
+            if len(bad := [g for g in groups if not g.reshard_after_backward]) > 1:
+                raise ValueError(
+                    "Only one parameter group across groups which share a data buffer"
+                    f" is allowed to have no reshard after backward, but got {bad}"
+                )
+        for groups in grad_users.values():
+            if len(bad := [g for g in groups if not g.reduce_grads]) > 1:
+                raise ValueError(
+                    "Only one parameter group across groups which share a grad buffer"
+                    f" is allowed to have no grad reduce, but got {bad}"
+                )
+        data_ctx_prefix: dict[Any, str] = {}
+        grad_ctx_prefix: dict[Any, str] = {}
+
+        def validate_buffers(module: nn.Module, prefix: str = "") -> None:
+            state = _get_module_fsdp_state(module)
+            group = state._fsdp_param_group if state is not None else None
+            if group is not None:
+                if group.data_buffer_ctx in data_ctx_prefix:
+                    raise RuntimeError(
+                        f"Param groups of {prefix} and {data_ctx_prefix[group.data_buffer_ctx]} share a"
+                        " data buffer, so they can't be unsharded at the same time."
+                    )
+                data_ctx_prefix[group.data_buffer_ctx] = prefix
+                if group.grad_buffer_ctx is not None:
+                    if group.grad_buffer_ctx in grad_ctx_prefix:
+                        raise RuntimeError(
+                            f"Param groups of {prefix} and {grad_ctx_prefix[group.grad_buffer_ctx]} share a"
+                            " grad buffer, so they can't be unsharded at the same time."
+                        )
+                    grad_ctx_prefix[group.grad_buffer_ctx] = prefix
+            for name, sub in module.named_children():
+                validate_buffers(sub, prefix + ("." if prefix else "") + name)
+            if group is not None:
+                del data_ctx_prefix[group.data_buffer_ctx]
+                if group.grad_buffer_ctx is not None:
+                    del grad_ctx_prefix[group.grad_buffer_ctx]
+
+        validate_buffers(self._modules[0])
+
+    def _init_fqns(self) -> None:
+        """ya_fsdp/_state.py:415-441."""
+        root_module = self._modules[0]
+        param_to_fsdp_param = {}
+        module_to_group = {}
+        for state in self._state_ctx.all_states:
+            if group := state._fsdp_param_group:
+                for fsdp_param in group.fsdp_params:
+                    param_to_fsdp_param[fsdp_param.sharded_param] = fsdp_param
+                for module in group.modules:
+                    module_to_group[module] = group
+        for param_name, param in root_module.named_parameters():
+            if param in param_to_fsdp_param:
+                param_to_fsdp_param[param]._param_fqn = param_name
+        for module_name, module in root_module.named_modules():
+            if module in module_to_group:
+                group = module_to_group[module]
+                group._module_fqn = module_name if group._module_fqn is None else f"{group._module_fqn}, {module_name}"
+
+    # -------------------------------------------------------------------- hooks --
+    def _pre_forward(self, module: nn.Module, args: tuple, kwargs: dict) -> tuple[tuple, dict]:
+        """ya_fsdp/_state.py:443-468."""
+        if self._training_state == TrainingState.PRE_BACKWARD:
+            return args, kwargs
+        self._training_state = TrainingState.FORWARD
+        args, kwargs = self._root_pre_forward(module, args, kwargs)
+        if self._mp_policy.cast_forward_inputs and self._mp_policy.param_dtype:
+            with torch.profiler.record_function("YaFSDP::cast_forward_inputs"):
+                cast_fn = functools.partial(_cast_fp_tensor, self._mp_policy.param_dtype)
+                args, kwargs = _apply_to_tensors(cast_fn, args), _apply_to_tensors(cast_fn, kwargs)
+        if self._fsdp_param_group:
+            args, kwargs = self._fsdp_param_group.pre_forward(module, args, kwargs)
+        for fsdp_state in self._states_to_forward_prefetch:
+            if (target := fsdp_state._fsdp_param_group) is not None:
+                YaFSDPParamGroup._prefetch_unshard(target, "forward")
+        return args, kwargs
+
+    def _post_forward(self, module: nn.Module, input: Any, output: Any) -> Any:
+        """ya_fsdp/_state.py:470-488."""
+        if self._training_state == TrainingState.PRE_BACKWARD:
+            return output
+        if self._fsdp_param_group:
+            output = self._fsdp_param_group.post_forward(module, input, output)
+        output = self._register_pre_backward_hook(output)
+        self._training_state = TrainingState.IDLE
+        if self._state_ctx.iter_forward_root is self:
+            self._state_ctx.iter_forward_root = None
+        if self._mp_policy.output_dtype is not None:
+            with torch.profiler.record_function("YaFSDP::cast_forward_outputs"):
+                output = _apply_to_tensors(functools.partial(_cast_fp_tensor, self._mp_policy.output_dtype), output)
+        return output
+
+    def _pre_backward(self, grad: torch.Tensor) -> torch.Tensor:
+        """ya_fsdp/_state.py:490-499."""
+        self._training_state = TrainingState.PRE_BACKWARD
+        self._register_root_post_backward_final_callback()
+        if self._fsdp_param_group:
+            default_prefetch = len(self._states_to_backward_prefetch) == 0
+            self._fsdp_param_group.pre_backward(default_prefetch)
+        for fsdp_state in self._states_to_backward_prefetch:
+            if (target := fsdp_state._fsdp_param_group) is not None:
+                YaFSDPParamGroup._prefetch_unshard(target, "backward")
+        return grad
+
+    def _root_post_backward_final_callback(self) -> None:
+        """ya_fsdp/_state.py:501-532."""
+        with torch.profiler.record_function("YaFSDP::root_post_backward_callback"):
+            for state in self._state_ctx.all_states:
+                group = state._fsdp_param_group
+                if group and group._training_state != TrainingState.POST_BACKWARD:
+                    # forward inputs did not require gradient: the autograd node did not run
+                    group.post_backward()
+                state._training_state = TrainingState.IDLE
+                if group:
+                    group._training_state = TrainingState.IDLE
+                if self._state_ctx.is_last_backward:
+                    state._finalize_backward()
+            if self._state_ctx.is_last_backward:
+                self._comm_ctx.post_forward_order.clear()
+            self._state_ctx.post_backward_final_callback_queued = False
+
+    def _finalize_backward(self) -> None:
+        if self._fsdp_param_group:
+            self._fsdp_param_group.finalize_backward()
+
+    def _register_pre_backward_hook(self, output: Any) -> Any:
+        """ya_fsdp/_state.py:549-556."""
+        if not torch.is_grad_enabled():
+            return output
+        flat_outputs, _ = tree_flatten(output)
+        for t in flat_outputs:
+            if torch.is_tensor(t) and t.requires_grad:
+                t.register_hook(self._pre_backward)
+        return output
+
+    def _register_root_post_backward_final_callback(self) -> None:
+        """ya_fsdp/_state.py:558-565."""
+        if self._state_ctx.post_backward_final_callback_queued:
+            return
+        self._state_ctx.post_backward_final_callback_queued = True
+        Variable._execution_engine.queue_callback(self._root_post_backward_final_callback)
+
+
+def _get_module_fsdp_state(module: nn.Module) -> YaFSDPState | None:
+    state = _get_module_state(module)
+    return state if isinstance(state, YaFSDPState) else None
