@@ -41,6 +41,18 @@ WORKLOADS = {
         [(512, 512)] * 4 + [(1376, 512), (1376, 512), (512, 1376), (512,), (512,)], 1, 0, 512, 1001),
 }
 
+
+def _ragged_stress_shapes(seed=1005, p=2000):
+    """2,000 tensors with odd element counts, log-uniform in [1, 2^22]; the 70 % drawn as fp32 masters with bf16
+    compute form the group measured here (a group has one master dtype)."""
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    u = torch.rand(p, generator=g, dtype=torch.float64) * 22 * 0.6931471805599453
+    numels = (torch.exp(u).floor().to(torch.int64) | 1).tolist()
+    is_fp32_master = (torch.rand(p, generator=g) < 0.7).tolist()
+    return [(n,) for n, f in zip(numels, is_fp32_master) if f]
+
 # HBM bytes per launch of the dominant kernel (gather_in_kernel), from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
 # (factors 1.99988 and 0.99986): (213037.875 * 1.99988 + 426022.75 * 0.99986) KiB.
@@ -238,7 +250,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="llama3-8b-layer-w8", choices=sorted(WORKLOADS) + ["llama3-8b-full-w8"])
+    ap.add_argument("--workload", default="llama3-8b-layer-w8",
+                    choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
     ap.add_argument("--sweep-grid-cap", action="store_true",
@@ -266,7 +279,10 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    shapes, w, r, align, seed = WORKLOADS[args.workload]
+    if args.workload == "ragged-stress-w256":
+        shapes, w, r, align, seed = _ragged_stress_shapes(), 256, 1, 512, 1005
+    else:
+        shapes, w, r, align, seed = WORKLOADS[args.workload]
     numels = [numel_of(s) for s in shapes]
     lay = make_layout(numels, w, align)
     t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel

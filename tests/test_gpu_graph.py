@@ -1,0 +1,72 @@
+"""A step of the buffer path captured into a HIP graph (tables with at most 16
+tensors pass everything in kernel arguments, so nothing but kernel launches is
+recorded) and replayed several times, with eager work and synchronisations in
+between; every replay must equal the eager result on the same inputs."""
+
+import pytest
+import torch
+
+from tests.helpers import assert_bits_equal
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def test_captured_step_replays_match_eager():
+    from yafsdp_amd import _native, make_layout
+
+    shapes = [(512, 512)] * 2 + [(1376, 512), (512, 1376), (512,), (333,)]
+    numels = [torch.Size(s).numel() for s in shapes]
+    w, r = 4, 2
+    lay = make_layout(numels, w, 8)
+    t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+    g = torch.Generator(device=DEV).manual_seed(77)
+
+    def rnd(n, std, dt):
+        return (torch.randn(n, device=DEV, generator=g) * std).to(dt)
+
+    master, gathered = rnd(s, 0.02, torch.float32), rnd(t_pad, 0.02, torch.bfloat16)
+    grads = [rnd(n, 1e-3, torch.bfloat16) for n in numels]
+    ag_in = torch.zeros(s, dtype=torch.bfloat16, device=DEV)
+    outs = [torch.zeros(n, dtype=torch.bfloat16, device=DEV) for n in numels]
+    rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=DEV)
+    shard = rnd(s, 1e-4, torch.float32)
+    table = _native.TensorTable(numels, t_pad, DEV)
+
+    def step(ag_in_, outs_, rs_, shard_):
+        _native.flat_copy(ag_in_, master)
+        table.scatter_out(gathered, outs_)
+        table.gather_in(grads, rs_, None, float(w), True)
+        _native.post_reduce(shard_, rs_[r * s : (r + 1) * s], None, True)
+
+    # warm up on a side stream, then capture
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(ag_in, outs, rs, shard.clone())
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    shard_graph = shard.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(ag_in, outs, rs, shard_graph)
+    shard_graph.copy_(shard)  # capture does not execute; start both accumulators from the same state
+    shard_eager = shard.clone()
+    for it in range(4):
+        # new inputs in place (same addresses), then eager reference on separate outputs
+        master.add_(0.001 * (it + 1))
+        gathered.mul_(1.0 + 0.125 * it)
+        for gr in grads:
+            gr.mul_(0.5)
+        e_ag, e_outs = torch.zeros_like(ag_in), [torch.zeros_like(o) for o in outs]
+        e_rs = torch.zeros_like(rs)
+        step(e_ag, e_outs, e_rs, shard_eager)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_bits_equal(ag_in, e_ag.cpu(), f"replay {it}: copy-in")
+        for a, b in zip(outs, e_outs):
+            assert_bits_equal(a, b.cpu(), f"replay {it}: copy-out")
+        assert_bits_equal(rs, e_rs.cpu(), f"replay {it}: reduce copy-in")
+        assert_bits_equal(shard_graph, shard_eager.cpu(), f"replay {it}: post-reduce")
+    table.close()

@@ -264,6 +264,13 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
 }
 
 // ---------------------------------------------------------------- scatter-out --
+// One full tile of the flat buffer (src, 16-byte aligned) into a tensor (dst, at
+// whatever element-aligned address the ragged offset gives).  Measured on a
+// 1427-tensor table with odd offsets: these unaligned stores cost 13 % against
+// the aligned case (reads at the same offsets cost 1 %); shifting the tile so
+// that stores are aligned and loads are not gains only 2 %, because what hurts
+// is the cache line shared by two tiles at every tile boundary, not the access
+// width - so the plain form is kept.
 template <class S, class D, int BLOCK, int U, bool NTL, bool NTS>
 __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
   if constexpr (wide_pair<S, D>::value) {
