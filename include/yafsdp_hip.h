@@ -139,7 +139,9 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
 /* Launch-shape knobs (process-wide, for measurement): */
 typedef enum yafsdp_option {
   YAFSDP_OPT_FLAT_BLOCKS_PER_CU = 0,  /* workgroups per compute unit of the flat kernels' grid */
-  YAFSDP_OPT_TABLE_BLOCKS_PER_CU = 1  /* same for gather-in / scatter-out */
+  YAFSDP_OPT_TABLE_BLOCKS_PER_CU = 1, /* same for gather-in / scatter-out */
+  YAFSDP_OPT_TABLE_LARGE_LOG2 = 2     /* 0..62: tables created from now on whose padded size exceeds
+                                         2^value elements run two waves per workgroup instead of one */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);

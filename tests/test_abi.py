@@ -44,6 +44,8 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_post_reduce(None, 0, None, 5, 0, 0.0, 0, None) == -2
     assert L.yafsdp_set_option(99, 1) == -1
     assert L.yafsdp_set_option(0, 0) == -1
+    assert L.yafsdp_set_option(2, 63) == -1
+    assert L.yafsdp_set_option(2, 28) == 0
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
 

@@ -135,6 +135,15 @@ def _random_numels(rng: np.random.Generator, p: int, max_log2: float, with_empty
     return n.tolist()
 
 
+@pytest.fixture(params=["one_wave", "two_waves"])
+def table_workgroup(request, nat):
+    """Run a table test at both workgroup sizes the library picks between by table size."""
+    default = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
+    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default if request.param == "one_wave" else 0)
+    yield request.param
+    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default)
+
+
 TABLE_CASES = [
     # (P, max log2 numel, with_empty, pad)
     (1, 3, False, 0),
@@ -152,7 +161,7 @@ TABLE_CASES = [
                                            (torch.float32, torch.bfloat16), (torch.float16, torch.float16),
                                            (torch.float32, torch.float32)])
 @pytest.mark.parametrize("pre", [None, 8.0, 3.0])
-def test_gather_in(nat, case, grad_dt, rs_dt, pre):
+def test_gather_in(nat, table_workgroup, case, grad_dt, rs_dt, pre):
     p, max_log2, with_empty, pad = case
     rng = np.random.default_rng(p * 1000 + pad)
     g = torch.Generator().manual_seed(104 + p)
@@ -205,7 +214,7 @@ def test_gather_in_pad_not_zeroed_sees_divide(nat):
 @pytest.mark.parametrize("case", TABLE_CASES)
 @pytest.mark.parametrize("flat_dt,out_dt", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
                                             (torch.bfloat16, torch.float32), (torch.float32, torch.float16)])
-def test_scatter_out(nat, case, flat_dt, out_dt):
+def test_scatter_out(nat, table_workgroup, case, flat_dt, out_dt):
     p, max_log2, with_empty, pad = case
     rng = np.random.default_rng(p * 1000 + pad + 1)
     g = torch.Generator().manual_seed(106 + p)

@@ -12,17 +12,19 @@ from __future__ import annotations
 
 import ctypes
 import os
+import threading
 from typing import Sequence
 
 import numpy as np
 import torch  # imported before the library so that both share one HIP runtime
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libyafsdp_hip.so")
+# YAFSDP_HIP_LIBRARY points at a library built elsewhere (same C ABI); default: the in-tree build
+LIB_PATH = os.environ.get("YAFSDP_HIP_LIBRARY") or os.path.join(_HERE, "libyafsdp_hip.so")
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MODE_SKIP, MODE_COPY, MODE_ADD = 0, 1, 2
-OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU = 0, 1
+OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU, OPT_TABLE_LARGE_LOG2 = 0, 1, 2
 
 # every symbol include/yafsdp_hip.h declares
 EXPORTED_SYMBOLS = (
@@ -210,8 +212,11 @@ class TensorTable:
                 "yafsdp_table_create",
             )
         self._handle = handle
+        # per-call pointer / mode arrays; the lock keeps "fill, then launch" atomic when the table is used from
+        # two host threads (the main thread and the autograd engine thread)
         self._ptrs = np.zeros(max(1, len(self.numels)), dtype=np.uint64)
         self._modes = np.zeros(max(1, len(self.numels)), dtype=np.uint8)
+        self._lock = threading.Lock()
 
     def close(self) -> None:
         h, self._handle = getattr(self, "_handle", None), None
@@ -287,10 +292,10 @@ class TensorTable:
         _flat_arg(flat, "flat")
         if flat.numel() < self.padded_numel:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.padded_numel}")
-        tdt = self._fill(tensors, modes, "tensors")
-        if tdt < 0:
-            tdt = _dt(flat)
-        with torch.cuda.device(self.device):
+        with self._lock, torch.cuda.device(self.device):
+            tdt = self._fill(tensors, modes, "tensors")
+            if tdt < 0:
+                tdt = _dt(flat)
             _check(
                 lib.yafsdp_gather_in(
                     self._handle, self._ptrs.ctypes.data, self._modes.ctypes.data, tdt, flat.data_ptr(), _dt(flat),
@@ -306,10 +311,10 @@ class TensorTable:
         _flat_arg(flat, "flat")
         if flat.numel() < self.total_numel:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.total_numel}")
-        tdt = self._fill(tensors, modes, "tensors")
-        if tdt < 0:
-            return
-        with torch.cuda.device(self.device):
+        with self._lock, torch.cuda.device(self.device):
+            tdt = self._fill(tensors, modes, "tensors")
+            if tdt < 0:
+                return
             _check(
                 lib.yafsdp_scatter_out(
                     self._handle, flat.data_ptr(), _dt(flat), self._ptrs.ctypes.data, self._modes.ctypes.data, tdt,

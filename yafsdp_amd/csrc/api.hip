@@ -18,6 +18,7 @@ namespace {
 
 std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
 std::atomic<int> g_table_blocks_per_cu{kTableBlocksPerCu};
+std::atomic<int> g_table_large_log2{kTableLargeThresholdLog2};
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -104,9 +105,10 @@ struct yafsdp_table {
   int64_t padded = 0;
   std::vector<int64_t> offsets;  // host copy, n_tensors + 1
   int64_t* d_offsets = nullptr;
-  // gather-in and scatter-out use different tile sizes: [0] gather, [1] scatter
-  int32_t n_tiles[2] = {0, 0};
-  TileRec* d_tiles[2] = {nullptr, nullptr};  // only for tables with more than kSmallMax tensors
+  int block = kTableBlockSmall;  // workgroup size of the table kernels, chosen from the padded size
+  int64_t tile_elems = 0;        // block * kTableUnroll * 8
+  int32_t n_tiles = 0;
+  TileRec* d_tiles = nullptr;    // only for tables with more than kSmallMax tensors
   // staging ring for the per-call pointer/mode arrays of tables with more than
   // kSmallMax tensors: pinned host slot -> device slot, one event per slot
   static constexpr int kRing = 4;
@@ -124,8 +126,7 @@ namespace {
 void table_free(yafsdp_table* t) {
   if (t == nullptr) return;
   if (t->d_offsets) (void)hipFree(t->d_offsets);
-  if (t->d_tiles[1] && t->d_tiles[1] != t->d_tiles[0]) (void)hipFree(t->d_tiles[1]);
-  if (t->d_tiles[0]) (void)hipFree(t->d_tiles[0]);
+  if (t->d_tiles) (void)hipFree(t->d_tiles);
   for (int i = 0; i < yafsdp_table::kRing; i++) {
     if (t->ev[i]) (void)hipEventDestroy(t->ev[i]);
     if (t->h_stage[i]) (void)hipHostFree(t->h_stage[i]);
@@ -149,8 +150,8 @@ int check_dyn(const yafsdp_table* t, const void* const* ptrs, const uint8_t* mod
 }
 
 // Small tables: everything travels in the kernel arguments.
-void fill_small(const yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int64_t tile_elems,
-                SmallMeta* m) {
+void fill_small(const yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, SmallMeta* m) {
+  const int64_t tile_elems = t->tile_elems;
   std::memset(m, 0, sizeof(*m));
   const int n = t->n_tensors;
   m->n_tensors = n;
@@ -168,7 +169,7 @@ void fill_small(const yafsdp_table* t, const void* const* ptrs, const uint8_t* m
 
 // Large tables: stage pointers (8 bytes each) and modes (4 bytes each) through
 // the ring.  Returns 0 or an error code; *slot is the ring slot used.
-int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, int which, LargeMeta* m, int* slot,
+int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, LargeMeta* m, int* slot,
                 hipStream_t stream) {
   const int n = t->n_tensors;
   const int s = t->next;
@@ -185,7 +186,7 @@ int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, i
   hipError_t e = hipMemcpyAsync(t->d_stage[s], h, t->stage_bytes, hipMemcpyHostToDevice, stream);
   if (e != hipSuccess) return int(e);
   m->offsets = t->d_offsets;
-  m->tiles = t->d_tiles[which];
+  m->tiles = t->d_tiles;
   m->ptrs = reinterpret_cast<const void* const*>(t->d_stage[s]);
   m->modes_ = reinterpret_cast<const uint32_t*>(t->d_stage[s] + size_t(n) * sizeof(void*));
   m->n_tensors = n;
@@ -221,6 +222,11 @@ const char* yafsdp_error_string(int code) {
 }
 
 int yafsdp_set_option(int option, int value) {
+  if (option == YAFSDP_OPT_TABLE_LARGE_LOG2) {
+    if (value < 0 || value > 62) return YAFSDP_ERR_INVALID_ARGUMENT;
+    g_table_large_log2.store(value);
+    return YAFSDP_OK;
+  }
   if (value < 1 || value > 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
   switch (option) {
     case YAFSDP_OPT_FLAT_BLOCKS_PER_CU: g_flat_blocks_per_cu.store(value); return YAFSDP_OK;
@@ -234,6 +240,7 @@ int yafsdp_get_option(int option, int* value) {
   switch (option) {
     case YAFSDP_OPT_FLAT_BLOCKS_PER_CU: *value = g_flat_blocks_per_cu.load(); return YAFSDP_OK;
     case YAFSDP_OPT_TABLE_BLOCKS_PER_CU: *value = g_table_blocks_per_cu.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_TABLE_LARGE_LOG2: *value = g_table_large_log2.load(); return YAFSDP_OK;
   }
   return YAFSDP_ERR_INVALID_ARGUMENT;
 }
@@ -337,38 +344,29 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     t->total = t->offsets[n_tensors];
     t->padded = padded_numel;
     if (padded_numel < t->total) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
-    const int64_t tile_elems[2] = {kGatherTileElems, kScatterTileElems};
-    for (int w = 0; w < 2; w++) {
-      const int64_t n_tiles = (padded_numel + tile_elems[w] - 1) / tile_elems[w];
-      if (n_tiles > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
-      t->n_tiles[w] = int32_t(n_tiles);
-    }
-    if (rc != YAFSDP_OK) break;
+    t->block = table_block_for(padded_numel, g_table_large_log2.load(std::memory_order_relaxed));
+    t->tile_elems = table_tile_elems(t->block);
+    const int64_t n_tiles = (padded_numel + t->tile_elems - 1) / t->tile_elems;
+    if (n_tiles > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    t->n_tiles = int32_t(n_tiles);
     if ((e = hipGetDevice(&t->device)) != hipSuccess) break;
     if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_offsets), t->offsets.size() * sizeof(int64_t))) != hipSuccess) break;
     if ((e = hipMemcpy(t->d_offsets, t->offsets.data(), t->offsets.size() * sizeof(int64_t), hipMemcpyHostToDevice)) != hipSuccess) break;
-    for (int w = 0; w < 2 && n_tensors > kSmallMax && e == hipSuccess; w++) {
+    if (n_tensors > kSmallMax && n_tiles > 0) {
       // per tile: first tensor whose end lies beyond the tile's first element
-      const int64_t n_tiles = t->n_tiles[w];
-      if (n_tiles == 0) continue;
-      if (w == 1 && tile_elems[1] == tile_elems[0]) {  // same tile size: one array serves both kernels
-        t->d_tiles[1] = t->d_tiles[0];
-        continue;
-      }
       tiles.resize(size_t(n_tiles));
       int p = 0;
       for (int64_t tile = 0; tile < n_tiles; tile++) {
-        const int64_t t0 = tile * tile_elems[w];
+        const int64_t t0 = tile * t->tile_elems;
         while (p < n_tensors && t->offsets[p + 1] <= t0) p++;
         TileRec& r = tiles[size_t(tile)];
         r.first = p;
-        r.full = (p < n_tensors && t->offsets[p + 1] - t0 >= tile_elems[w]) ? 1 : 0;
+        r.full = (p < n_tensors && t->offsets[p + 1] - t0 >= t->tile_elems) ? 1 : 0;
         r.delta = p < n_tensors ? t0 - t->offsets[p] : 0;
       }
-      if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_tiles[w]), tiles.size() * sizeof(TileRec))) != hipSuccess) break;
-      if ((e = hipMemcpy(t->d_tiles[w], tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
+      if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_tiles), tiles.size() * sizeof(TileRec))) != hipSuccess) break;
+      if ((e = hipMemcpy(t->d_tiles, tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
     }
-    if (e != hipSuccess) break;
     if (n_tensors > kSmallMax) {
       t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
       for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
@@ -425,20 +423,20 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   hipStream_t s = static_cast<hipStream_t>(stream);
   int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
-  const int n_tiles = table->n_tiles[0];
+  const int n_tiles = table->n_tiles;
   const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax) {
     SmallMeta meta;
-    fill_small(table, tensor_ptrs, mode, kGatherTileElems, &meta);
-    return int(launch_gather<SmallMeta>(tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
-                                        zero_pad ? 1 : 0, grid, s));
+    fill_small(table, tensor_ptrs, mode, &meta);
+    return int(launch_gather<SmallMeta>(table->block, tensor_dtype, flat_dtype, scale, meta, flat, table->padded,
+                                        n_tiles, k, zero_pad ? 1 : 0, grid, s));
   }
   std::lock_guard<std::mutex> lock(table->mu);
   LargeMeta meta;
   int slot = -1;
-  rc = stage_large(table, tensor_ptrs, mode, 0, &meta, &slot, s);
+  rc = stage_large(table, tensor_ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
-  e = launch_gather<LargeMeta>(tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
+  e = launch_gather<LargeMeta>(table->block, tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
                                zero_pad ? 1 : 0, grid, s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
@@ -459,19 +457,20 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   const void* const* ptrs = const_cast<const void* const*>(tensor_ptrs);
   int rc = check_dyn(table, ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
-  const int n_tiles = table->n_tiles[1];
+  const int n_tiles = table->n_tiles;
   const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax) {
     SmallMeta meta;
-    fill_small(table, ptrs, mode, kScatterTileElems, &meta);
-    return int(launch_scatter<SmallMeta>(flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s));
+    fill_small(table, ptrs, mode, &meta);
+    return int(launch_scatter<SmallMeta>(table->block, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,
+                                         grid, s));
   }
   std::lock_guard<std::mutex> lock(table->mu);
   LargeMeta meta;
   int slot = -1;
-  rc = stage_large(table, ptrs, mode, 1, &meta, &slot, s);
+  rc = stage_large(table, ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
-  e = launch_scatter<LargeMeta>(flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s);
+  e = launch_scatter<LargeMeta>(table->block, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }

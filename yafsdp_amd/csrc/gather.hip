@@ -5,32 +5,40 @@
 namespace yafsdp {
 namespace {
 
-template <class META, class S, class D, int SCALE>
+template <class META, class S, class D, int SCALE, int BLOCK>
 hipError_t go(const META& meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero, int grid,
               hipStream_t stream) {
-  gather_in_kernel<META, S, D, SCALE, kTableBlock, kGatherUnroll, kTableNtLoad, kTableNtStore>
-      <<<dim3(grid), dim3(kTableBlock), 0, stream>>>(meta, flat, padded, n_tiles, k, pad_zero);
+  gather_in_kernel<META, S, D, SCALE, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>
+      <<<dim3(grid), dim3(BLOCK), 0, stream>>>(meta, flat, padded, n_tiles, k, pad_zero);
   return hipGetLastError();
 }
 
-template <class META, class S, class D>
-hipError_t by_scale(int scale, const META& meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero,
+template <class META, class S, class D, int SCALE>
+hipError_t by_block(int block, const META& meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero,
                     int grid, hipStream_t stream) {
+  if (block == kTableBlockSmall) return go<META, S, D, SCALE, kTableBlockSmall>(meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+  if (block == kTableBlockLarge) return go<META, S, D, SCALE, kTableBlockLarge>(meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+  return hipErrorInvalidValue;
+}
+
+template <class META, class S, class D>
+hipError_t by_scale(int block, int scale, const META& meta, void* flat, int64_t padded, int n_tiles, float k,
+                    int pad_zero, int grid, hipStream_t stream) {
   switch (scale) {
-    case SCALE_NONE: return go<META, S, D, SCALE_NONE>(meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
-    case SCALE_MUL: return go<META, S, D, SCALE_MUL>(meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
-    case SCALE_DIV: return go<META, S, D, SCALE_DIV>(meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case SCALE_NONE: return by_block<META, S, D, SCALE_NONE>(block, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case SCALE_MUL: return by_block<META, S, D, SCALE_MUL>(block, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case SCALE_DIV: return by_block<META, S, D, SCALE_DIV>(block, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
   }
   return hipErrorInvalidValue;
 }
 
 template <class META, class S>
-hipError_t by_flat(int flat_dt, int scale, const META& meta, void* flat, int64_t padded, int n_tiles, float k,
-                   int pad_zero, int grid, hipStream_t stream) {
+hipError_t by_flat(int block, int flat_dt, int scale, const META& meta, void* flat, int64_t padded, int n_tiles,
+                   float k, int pad_zero, int grid, hipStream_t stream) {
   switch (flat_dt) {
-    case DT_F32: return by_scale<META, S, F32>(scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
-    case DT_BF16: return by_scale<META, S, BF16>(scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
-    case DT_F16: return by_scale<META, S, F16>(scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case DT_F32: return by_scale<META, S, F32>(block, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case DT_BF16: return by_scale<META, S, BF16>(block, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case DT_F16: return by_scale<META, S, F16>(block, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -38,19 +46,19 @@ hipError_t by_flat(int flat_dt, int scale, const META& meta, void* flat, int64_t
 }  // namespace
 
 template <class META>
-hipError_t launch_gather(int tensor_dt, int flat_dt, int scale, const META& meta, void* flat, int64_t padded,
-                         int n_tiles, float k, int pad_zero, int grid, hipStream_t stream) {
+hipError_t launch_gather(int block, int tensor_dt, int flat_dt, int scale, const META& meta, void* flat,
+                         int64_t padded, int n_tiles, float k, int pad_zero, int grid, hipStream_t stream) {
   switch (tensor_dt) {
-    case DT_F32: return by_flat<META, F32>(flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
-    case DT_BF16: return by_flat<META, BF16>(flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
-    case DT_F16: return by_flat<META, F16>(flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case DT_F32: return by_flat<META, F32>(block, flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case DT_BF16: return by_flat<META, BF16>(block, flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
+    case DT_F16: return by_flat<META, F16>(block, flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, grid, stream);
   }
   return hipErrorInvalidValue;
 }
 
-template hipError_t launch_gather<SmallMeta>(int, int, int, const SmallMeta&, void*, int64_t, int, float, int, int,
-                                             hipStream_t);
-template hipError_t launch_gather<LargeMeta>(int, int, int, const LargeMeta&, void*, int64_t, int, float, int, int,
-                                             hipStream_t);
+template hipError_t launch_gather<SmallMeta>(int, int, int, int, const SmallMeta&, void*, int64_t, int, float, int,
+                                             int, hipStream_t);
+template hipError_t launch_gather<LargeMeta>(int, int, int, int, const LargeMeta&, void*, int64_t, int, float, int,
+                                             int, hipStream_t);
 
 }  // namespace yafsdp

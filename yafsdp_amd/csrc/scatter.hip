@@ -5,20 +5,28 @@
 namespace yafsdp {
 namespace {
 
-template <class META, class S, class D>
+template <class META, class S, class D, int BLOCK>
 hipError_t go(const META& meta, const void* flat, int64_t total, int n_tiles, int grid, hipStream_t stream) {
-  scatter_out_kernel<META, S, D, kTableBlock, kScatterUnroll, kTableNtLoad, kTableNtStore>
-      <<<dim3(grid), dim3(kTableBlock), 0, stream>>>(meta, flat, total, n_tiles);
+  scatter_out_kernel<META, S, D, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>
+      <<<dim3(grid), dim3(BLOCK), 0, stream>>>(meta, flat, total, n_tiles);
   return hipGetLastError();
 }
 
+template <class META, class S, class D>
+hipError_t by_block(int block, const META& meta, const void* flat, int64_t total, int n_tiles, int grid,
+                    hipStream_t stream) {
+  if (block == kTableBlockSmall) return go<META, S, D, kTableBlockSmall>(meta, flat, total, n_tiles, grid, stream);
+  if (block == kTableBlockLarge) return go<META, S, D, kTableBlockLarge>(meta, flat, total, n_tiles, grid, stream);
+  return hipErrorInvalidValue;
+}
+
 template <class META, class S>
-hipError_t by_tensor(int tensor_dt, const META& meta, const void* flat, int64_t total, int n_tiles, int grid,
-                     hipStream_t stream) {
+hipError_t by_tensor(int block, int tensor_dt, const META& meta, const void* flat, int64_t total, int n_tiles,
+                     int grid, hipStream_t stream) {
   switch (tensor_dt) {
-    case DT_F32: return go<META, S, F32>(meta, flat, total, n_tiles, grid, stream);
-    case DT_BF16: return go<META, S, BF16>(meta, flat, total, n_tiles, grid, stream);
-    case DT_F16: return go<META, S, F16>(meta, flat, total, n_tiles, grid, stream);
+    case DT_F32: return by_block<META, S, F32>(block, meta, flat, total, n_tiles, grid, stream);
+    case DT_BF16: return by_block<META, S, BF16>(block, meta, flat, total, n_tiles, grid, stream);
+    case DT_F16: return by_block<META, S, F16>(block, meta, flat, total, n_tiles, grid, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -26,17 +34,19 @@ hipError_t by_tensor(int tensor_dt, const META& meta, const void* flat, int64_t 
 }  // namespace
 
 template <class META>
-hipError_t launch_scatter(int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total, int n_tiles,
-                          int grid, hipStream_t stream) {
+hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total,
+                          int n_tiles, int grid, hipStream_t stream) {
   switch (flat_dt) {
-    case DT_F32: return by_tensor<META, F32>(tensor_dt, meta, flat, total, n_tiles, grid, stream);
-    case DT_BF16: return by_tensor<META, BF16>(tensor_dt, meta, flat, total, n_tiles, grid, stream);
-    case DT_F16: return by_tensor<META, F16>(tensor_dt, meta, flat, total, n_tiles, grid, stream);
+    case DT_F32: return by_tensor<META, F32>(block, tensor_dt, meta, flat, total, n_tiles, grid, stream);
+    case DT_BF16: return by_tensor<META, BF16>(block, tensor_dt, meta, flat, total, n_tiles, grid, stream);
+    case DT_F16: return by_tensor<META, F16>(block, tensor_dt, meta, flat, total, n_tiles, grid, stream);
   }
   return hipErrorInvalidValue;
 }
 
-template hipError_t launch_scatter<SmallMeta>(int, int, const SmallMeta&, const void*, int64_t, int, int, hipStream_t);
-template hipError_t launch_scatter<LargeMeta>(int, int, const LargeMeta&, const void*, int64_t, int, int, hipStream_t);
+template hipError_t launch_scatter<SmallMeta>(int, int, int, const SmallMeta&, const void*, int64_t, int, int,
+                                              hipStream_t);
+template hipError_t launch_scatter<LargeMeta>(int, int, int, const LargeMeta&, const void*, int64_t, int, int,
+                                              hipStream_t);
 
 }  // namespace yafsdp

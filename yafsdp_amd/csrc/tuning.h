@@ -11,17 +11,22 @@ constexpr bool kFlatNtStore = true;
 // gather-in / scatter-out: a tile is block * unroll * 8 elements.  Measured with
 // non-zero data and the four kernels of a step running back to back: tiles of
 // 1-2 K elements (2-4 KiB of bf16) in workgroups of one or two waves are the
-// fastest for both kernels (one wave x 2 units ahead by about 1 %); larger
-// workgroups lose 3-10 %.  (All-zero buffers
-// run up to 10 % faster than any other content on this memory system and must
-// not be used for tuning.)
-constexpr int kTableBlock = 64;
-constexpr int kGatherUnroll = 2;
-constexpr int kScatterUnroll = 2;
+// fastest for both kernels; larger workgroups lose 3-10 %.  Between the two,
+// one wave per workgroup wins by 0.4 % on a 218 M-element buffer and two waves
+// win by 2.8 % on an 856 M-element buffer (half as many workgroups to
+// dispatch), so the tile size is chosen per table from its padded size.
+// (All-zero buffers run up to 10 % faster than any other content on this memory
+// system and must not be used for tuning.)
+constexpr int kTableBlockSmall = 64;
+constexpr int kTableBlockLarge = 128;
+constexpr int kTableLargeThresholdLog2 = 28;  // padded size above 2^28 elements: the larger workgroup
+constexpr int kTableUnroll = 2;
 constexpr bool kTableNtLoad = true;
 constexpr bool kTableNtStore = true;
-constexpr long long kGatherTileElems = (long long)kTableBlock * kGatherUnroll * 8;
-constexpr long long kScatterTileElems = (long long)kTableBlock * kScatterUnroll * 8;
+inline int table_block_for(long long padded_elems, int threshold_log2) {
+  return padded_elems > (1LL << threshold_log2) ? kTableBlockLarge : kTableBlockSmall;
+}
+inline long long table_tile_elems(int block) { return (long long)block * kTableUnroll * 8; }
 // default grid cap in workgroups per compute unit.  Measured: one workgroup per
 // tile (no cap reached) beats a persistent grid-stride grid by 5-10 % on every
 // kernel of the path, so the cap is far above any tile count of interest.
