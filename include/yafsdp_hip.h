@@ -28,6 +28,7 @@
 #ifndef YAFSDP_HIP_H_
 #define YAFSDP_HIP_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -135,6 +136,58 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
  * 16-byte aligned; pad lanes are never read. */
 int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
                        const uint8_t* mode, int tensor_dtype, void* stream);
+
+/* ---- optimizer-side passes over the flat shard buffers ------------------------
+ * The reference runs the optimizer and gradient clipping as torch foreach ops
+ * over the per-parameter fragments of the flat shard (dispatch table of its
+ * tensor subclass, ya_fsdp/_tensor.py:122-316).  The fragments of one group are
+ * consecutive ranges of one flat buffer, so each op is one pass over that
+ * buffer here.  Every pointer below is device memory, 16-byte aligned. */
+
+/* dst[0:n] = cast(value).  `_foreach_zero_` of optimizer.zero_grad(set_to_none=False)
+ * (ya_fsdp/_tensor.py:243-245; the legacy wrapper allows no other form,
+ * ya_fsdp/ya_fsdp.py:591-601) and the zero-initialised grad shard
+ * (ya_fsdp/_param_group.py:276). */
+int yafsdp_flat_fill(void* dst, int dtype, int64_t n, double value, void* stream);
+
+/* Bytes of device workspace yafsdp_flat_sumsq needs (a constant). */
+size_t yafsdp_sumsq_workspace_bytes(void);
+
+/* *sumsq = (accumulate ? *sumsq : 0) + sum_i float(src[i])^2, in binary64.
+ * The squared 2-norm behind `_foreach_norm(grads, 2)` (ya_fsdp/_tensor.py:220-242)
+ * and the legacy clip_grad_norm_ (ya_fsdp/ya_fsdp.py:545-556), whose per-buffer
+ * norms are squared and summed again.  The reference adds in binary32 in an
+ * order its backend chooses; this sum is exact to binary64 rounding and its
+ * order depends only on n, so it is reproducible.  `workspace` is scratch for
+ * the duration of the call on `stream`. */
+int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/* norm_and_coef[0] = float(sqrt(*sumsq)); norm_and_coef[1] = min(max_norm /
+ * (norm + 1e-6), 1.0), binary32 like the reference's tensors
+ * (ya_fsdp/ya_fsdp.py:557-559; torch.nn.utils.clip_grads_with_norm_). */
+int yafsdp_clip_coef(const double* sumsq, double max_norm, float* norm_and_coef, void* stream);
+
+/* buf[i] = round(float(buf[i]) * *coef), the coefficient read on the device
+ * (`grad.mul_(total_norm_coef)`, ya_fsdp/ya_fsdp.py:560-561; `_foreach_mul_.Tensor`,
+ * ya_fsdp/_tensor.py:256-262).  Returns without touching memory when *coef == 1. */
+int yafsdp_flat_scale(void* buf, int dtype, int64_t n, const float* coef, void* stream);
+
+/* One Adam / AdamW step on a flat binary32 shard (param, grad, exp_avg,
+ * exp_avg_sq of n elements), in the operation order of torch.optim.Adam(W)
+ * (`_fused_adam_` / `_fused_adamw_` and the foreach lerp / addcmul / addcdiv
+ * ops the reference forwards to the local tensors, ya_fsdp/_tensor.py:269-312),
+ * fused with the copy-in cast of the next iteration
+ * (`all_gather_input.copy_(shard)`, ya_fsdp/_collectives.py:53-54): when `out16` is
+ * not NULL it receives the updated parameters rounded to `out16_dtype` (bf16 or
+ * f16).  `step` is the 1-based step count.  `grad_scale` (device, may be NULL)
+ * multiplies the gradient first, as a preceding `grad.mul_(coef)` would, without
+ * writing it back.  flags: YAFSDP_ADAM_DECOUPLED_DECAY = AdamW, otherwise the
+ * L2 form of Adam; YAFSDP_ADAM_ZERO_GRAD also zero-fills `grad`. */
+enum { YAFSDP_ADAM_DECOUPLED_DECAY = 1, YAFSDP_ADAM_ZERO_GRAD = 2 };
+int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_sq, void* out16, int out16_dtype,
+                      int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,
+                      int64_t step, const float* grad_scale, int flags, void* stream);
 
 /* Launch-shape knobs (process-wide, for measurement): */
 typedef enum yafsdp_option {

@@ -164,3 +164,87 @@ void ref_scatter_out(int n_tensors, void* const* tensors, const int64_t* offsets
     else for (int64_t i = 0; i < n; i++) store_f(tensors[p], tdt, i, load_f(flat, fdt, o + i));
   }
 }
+
+/* ---- optimizer-side passes over the flat shard --------------------------------
+ * The reference forwards torch.optim's foreach / fused Adam ops to the local
+ * fragments of the flat shard (ya_fsdp/_tensor.py:269-312).  Per element, with
+ * every intermediate tensor rounded to binary32, torch.optim.Adam(W) computes
+ * (torch/optim/adam.py, `_single_tensor_adam`, the non-capturable branch):
+ *
+ *   grad = grad.add(param, alpha=wd)               Adam (L2 form) only
+ *   param.mul_(1 - lr*wd)                          AdamW only
+ *   exp_avg.lerp_(grad, 1 - beta1)
+ *   exp_avg_sq.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
+ *   denom = (exp_avg_sq.sqrt() / sqrt(1 - beta2^t)).add_(eps)
+ *   param.addcdiv_(exp_avg, denom, value=-(lr / (1 - beta1^t)))
+ *
+ * torch's CPU kernels evaluate `add(alpha)`, `lerp_` and `addcmul_` with one
+ * fused multiply-add each: fma(param, wd, grad); fma(w, grad - exp_avg, exp_avg)
+ * for |w| < 0.5 and fma(w - 1, grad - exp_avg, grad) otherwise; fma((1-beta2)*grad,
+ * grad, exp_avg_sq).  `addcdiv_` is not fused: param + (value*exp_avg)/denom.
+ * (Established by comparing each torch op with both candidates on a million
+ * random elements; tests/test_optim_oracle.py repeats the comparison.)  Square
+ * root and division are correctly rounded here; torch's CPU sqrt is off by one
+ * ulp for about 0.6 % of inputs, so whole steps agree with torch to 1 ulp, not
+ * bit for bit. */
+#include <math.h>
+
+void ref_adamw_step(float* p, float* g, float* m, float* v, void* out16, int out_dt, int64_t n,
+                    double lr, double beta1, double beta2, double eps, double wd, int64_t step,
+                    int decoupled, int has_scale, float grad_scale, int zero_grad) {
+  const float decay = (float)(1.0 - lr * wd);
+  const float l2 = (float)wd;
+  const float w = (float)(1.0 - beta1);
+  const float w_m1 = w - 1.0f;
+  const float b2 = (float)beta2;
+  const float a = (float)(1.0 - beta2);
+  const double bc1 = 1.0 - pow(beta1, (double)step);
+  const double bc2 = 1.0 - pow(beta2, (double)step);
+  const float bc2_sqrt = (float)pow(bc2, 0.5);
+  const float epsf = (float)eps;
+  const float neg_step = (float)(-(lr / bc1));
+  for (int64_t i = 0; i < n; i++) {
+    float gi = g[i], pi = p[i], mi = m[i], vi = v[i];
+    if (has_scale) gi = gi * grad_scale;
+    if (wd != 0.0) {
+      if (decoupled) pi = pi * decay;
+      else gi = fmaf(pi, l2, gi);
+    }
+    const float d = gi - mi;
+    mi = (fabsf(w) < 0.5f) ? fmaf(w, d, mi) : fmaf(w_m1, d, gi);
+    vi = vi * b2;
+    vi = fmaf(a * gi, gi, vi);
+    const float den = sqrtf(vi) / bc2_sqrt + epsf;
+    pi = pi + (neg_step * mi) / den;
+    p[i] = pi;
+    m[i] = mi;
+    v[i] = vi;
+    if (out16) store_f(out16, out_dt, i, pi);
+    if (zero_grad) g[i] = 0.0f;
+  }
+}
+
+/* sum of squares in binary64, added in index order */
+double ref_sumsq(const void* src, int dt, int64_t n) {
+  double acc = 0.0;
+  for (int64_t i = 0; i < n; i++) {
+    const double x = (double)load_f(src, dt, i);
+    acc += x * x;
+  }
+  return acc;
+}
+
+/* out[0] = float(sqrt(sumsq)); out[1] = min(max_norm / (out[0] + 1e-6), 1)
+ * (ya_fsdp/ya_fsdp.py:557-559), NaN kept */
+void ref_clip_coef(double sumsq, double max_norm, float* out) {
+  const float norm = (float)sqrt(sumsq);
+  float c = (float)max_norm / (norm + 1e-6f);
+  if (c > 1.0f) c = 1.0f;
+  out[0] = norm;
+  out[1] = c;
+}
+
+/* buf[i] = round(float(buf[i]) * coef)   (grad.mul_(coef), ya_fsdp/ya_fsdp.py:560-561) */
+void ref_flat_scale(void* buf, int dt, int64_t n, float coef) {
+  for (int64_t i = 0; i < n; i++) store_f(buf, dt, i, load_f(buf, dt, i) * coef);
+}

@@ -19,7 +19,7 @@ def build(force: bool = True) -> str:
         return OUT
     cmd = [
         "gcc", "-O2", "-std=c11", "-fPIC", "-shared", "-ffp-contract=off",
-        "-fno-fast-math", "-Wall", "-Wextra", "-o", OUT, SRC,
+        "-fno-fast-math", "-Wall", "-Wextra", "-o", OUT, SRC, "-lm",
     ]
     subprocess.run(cmd, check=True)
     return OUT

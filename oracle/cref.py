@@ -41,6 +41,15 @@ def lib() -> ctypes.CDLL:
         L.ref_gather_in.argtypes = [i32, vp, vp, vp, i32, vp, i32, i64, dbl, i32]
         L.ref_scatter_out.restype = None
         L.ref_scatter_out.argtypes = [i32, vp, vp, i32, vp, i32]
+        L.ref_adamw_step.restype = None
+        L.ref_adamw_step.argtypes = [vp, vp, vp, vp, vp, i32, i64, dbl, dbl, dbl, dbl, dbl, i64, i32, i32,
+                                     ctypes.c_float, i32]
+        L.ref_sumsq.restype = dbl
+        L.ref_sumsq.argtypes = [vp, i32, i64]
+        L.ref_clip_coef.restype = None
+        L.ref_clip_coef.argtypes = [dbl, dbl, vp]
+        L.ref_flat_scale.restype = None
+        L.ref_flat_scale.argtypes = [vp, i32, i64, ctypes.c_float]
         _lib = L
     return _lib
 
@@ -95,3 +104,35 @@ def scatter_out(tensors, offsets, flat: torch.Tensor) -> None:
     offs = np.asarray(offsets, dtype=np.int64)
     tdt = DT[tensors[0].dtype] if tensors else DT[flat.dtype]
     lib().ref_scatter_out(len(tensors), ptrs.ctypes.data, offs.ctypes.data, tdt, flat.data_ptr(), DT[flat.dtype])
+
+
+def adamw_step(p, g, m, v, out16, *, lr, beta1, beta2, eps, weight_decay, step, decoupled=True, grad_scale=None,
+               zero_grad=False) -> None:
+    """One Adam(W) step in place on binary32 CPU tensors; `out16` (bf16/f16 or None) receives round16(p)."""
+    for t in (p, g, m, v):
+        _check(t)
+        assert t.dtype == torch.float32 and t.numel() == p.numel()
+    if out16 is not None:
+        _check(out16)
+    lib().ref_adamw_step(
+        p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), None if out16 is None else out16.data_ptr(),
+        0 if out16 is None else DT[out16.dtype], p.numel(), float(lr), float(beta1), float(beta2), float(eps),
+        float(weight_decay), int(step), int(decoupled), int(grad_scale is not None),
+        0.0 if grad_scale is None else float(grad_scale), int(zero_grad),
+    )
+
+
+def sumsq(src: torch.Tensor) -> float:
+    _check(src)
+    return float(lib().ref_sumsq(src.data_ptr(), DT[src.dtype], src.numel()))
+
+
+def clip_coef(sumsq_value: float, max_norm: float) -> tuple[float, float]:
+    out = np.zeros(2, dtype=np.float32)
+    lib().ref_clip_coef(float(sumsq_value), float(max_norm), out.ctypes.data)
+    return float(out[0]), float(out[1])
+
+
+def flat_scale(buf: torch.Tensor, coef: float) -> None:
+    _check(buf)
+    lib().ref_flat_scale(buf.data_ptr(), DT[buf.dtype], buf.numel(), float(np.float32(coef)))

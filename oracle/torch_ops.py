@@ -148,3 +148,57 @@ def reduce_scatter_local(
     else:
         raise ValueError(mode)
     return output_tensor
+
+
+# ---------------------------------------------------------------------------
+# optimizer-side passes over the flat shard (the reference forwards these torch
+# ops to the local fragments, ya_fsdp/_tensor.py:212-312)
+# ---------------------------------------------------------------------------
+def clip_grad_norm_(grads: Sequence[torch.Tensor], max_norm: float) -> torch.Tensor:
+    """Legacy ``YaFSDP.clip_grad_norm_`` (ya_fsdp/ya_fsdp.py:543-562) on one rank,
+    norm_type 2: per-buffer norms in binary32, norm of the stack, squared, (the
+    all-reduce over ranks is the identity here), root, coefficient, in-place
+    scale.  Returns the total norm."""
+    grad_norm = torch.linalg.vector_norm(
+        torch.stack([torch.linalg.vector_norm(g.detach(), 2.0, dtype=torch.float32) for g in grads]),
+        2.0,
+        dtype=torch.float32,
+    )
+    total_norm = grad_norm**2.0
+    total_norm = total_norm ** (1 / 2.0)
+    total_norm_coef = max_norm / (total_norm + 1e-6)
+    total_norm_coef = torch.clamp(total_norm_coef, max=1.0)
+    for g in grads:
+        g.mul_(total_norm_coef)
+    return total_norm
+
+
+def adam_step_torch_ops(
+    param: torch.Tensor,
+    grad: torch.Tensor,
+    exp_avg: torch.Tensor,
+    exp_avg_sq: torch.Tensor,
+    *,
+    lr: float,
+    beta1: float,
+    beta2: float,
+    eps: float,
+    weight_decay: float,
+    step: int,
+    decoupled: bool = True,
+) -> None:
+    """The tensor ops of one torch.optim.Adam(W) step (torch/optim/adam.py,
+    ``_single_tensor_adam``, non-capturable branch), in place."""
+    if weight_decay != 0:
+        if decoupled:
+            param.mul_(1 - lr * weight_decay)
+        else:
+            grad = grad.add(param, alpha=weight_decay)
+    exp_avg.lerp_(grad, 1 - beta1)
+    exp_avg_sq.mul_(beta2).addcmul_(grad, grad, value=1 - beta2)
+    bias_correction1 = 1 - beta1**step
+    bias_correction2 = 1 - beta2**step
+    step_size = lr / bias_correction1
+    bias_correction2_sqrt = bias_correction2**0.5
+    denom = (exp_avg_sq.sqrt() / bias_correction2_sqrt).add_(eps)
+    param.addcdiv_(exp_avg, denom, value=-step_size)

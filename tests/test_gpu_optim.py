@@ -1,0 +1,216 @@
+"""GPU parity of the optimizer-side passes over a flat shard, through the C
+ABI, against the C oracle: bit for bit for fill, scale, clip coefficient and
+the fused Adam(W) step; to binary64 rounding for the sum of squares (its
+order of additions is the kernel's own; the oracle adds in index order)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cref
+
+from helpers import DTYPES, assert_bits_equal, mixed_values
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def nat():
+    from yafsdp_amd import _native
+
+    return _native
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+SIZES = [0, 1, 3, 4, 7, 8, 1023, 2048, 2049, 100_003, (1 << 20) + 5]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("value", [0.0, 1.5, -0.0, 3.0e-41, float("inf"), 0.1])
+def test_flat_fill(nat, dtype, value):
+    for n in SIZES:
+        _say("fill", dtype, value, n)
+        buf = torch.full((n + 16,), 7.0, dtype=dtype, device=DEV)
+        nat.flat_fill(buf[8 : 8 + n], value)
+        want = torch.full((n + 16,), 7.0, dtype=dtype)
+        want[8 : 8 + n] = torch.tensor(value, dtype=torch.float32).to(dtype)
+        assert_bits_equal(buf, want, f"fill n={n}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_flat_sumsq(nat, dtype):
+    g = torch.Generator().manual_seed(201)
+    ws = nat.sumsq_workspace(torch.device(DEV))
+    out = torch.full((2,), 5.0, dtype=torch.float64, device=DEV)
+    for n in SIZES + [(1 << 23) + 11]:
+        _say("sumsq", dtype, n)
+        x = (torch.randn(n, generator=g) * 3e-2).to(dtype)
+        want = cref.sumsq(x)
+        pad = torch.zeros(n + 8, dtype=dtype, device=DEV)  # 16-byte aligned view at any n
+        pad[:n] = x.to(DEV)
+        nat.flat_sumsq(pad[:n], out, ws, accumulate=False)
+        got = out.cpu()
+        assert got[1].item() == 5.0
+        assert abs(got[0].item() - want) <= 1e-12 * want, (n, got[0].item(), want)
+        nat.flat_sumsq(pad[:n], out, ws, accumulate=True)
+        assert abs(out[0].item() - 2 * want) <= 1e-12 * 2 * want
+        # reproducible: same bits on a second run
+        nat.flat_sumsq(pad[:n], out, ws, accumulate=False)
+        assert out[0].item() == got[0].item()
+    # exactness where binary32 accumulation would fail: 2^24 ones plus one tiny term
+    ones = torch.ones((1 << 24) + 4, dtype=torch.float32, device=DEV)
+    ones[-1] = 2.0**-10
+    nat.flat_sumsq(ones, out, ws)
+    assert out[0].item() == float((1 << 24) + 3) + 2.0**-20
+
+
+def test_sumsq_special_values(nat):
+    ws = nat.sumsq_workspace(torch.device(DEV))
+    out = torch.zeros(1, dtype=torch.float64, device=DEV)
+    x = torch.zeros(1000, device=DEV)
+    x[77] = float("inf")
+    nat.flat_sumsq(x, out, ws)
+    assert math.isinf(out.item())
+    x[78] = float("nan")
+    nat.flat_sumsq(x, out, ws)
+    assert math.isnan(out.item())
+    big = torch.full((1000,), 3.0e38, device=DEV)  # squares overflow binary32, not binary64
+    nat.flat_sumsq(big, out, ws)
+    assert abs(out.item() - cref.sumsq(big.cpu())) <= 1e-12 * out.item()
+
+
+@pytest.mark.parametrize("max_norm", [0.5, 1.0, 1e6])
+def test_clip_coef_and_scale(nat, max_norm):
+    g = torch.Generator().manual_seed(202)
+    ws = nat.sumsq_workspace(torch.device(DEV))
+    sumsq = torch.zeros(1, dtype=torch.float64, device=DEV)
+    nc = torch.zeros(2, dtype=torch.float32, device=DEV)
+    bufs = [(torch.randn(n, generator=g) * std).to(dt)
+            for n, std, dt in ((300_001, 1e-2, torch.float32), (5000, 1e-1, torch.bfloat16), (777, 1e-1, torch.float16))]
+    for b in bufs:  # zeros, a subnormal, values that round to ties after scaling
+        b[:6] = torch.tensor([0.0, -0.0, 1e-40, -1e-40, 1.0, -3.0]).to(b.dtype)
+    dbufs = []
+    for i, b in enumerate(bufs):
+        d = torch.zeros(b.numel() + 8, dtype=b.dtype, device=DEV)[: b.numel()]
+        d.copy_(b)
+        dbufs.append(d)
+        nat.flat_sumsq(d, sumsq, ws, accumulate=i > 0)
+    nat.clip_coef(sumsq, max_norm, nc)
+    norm, coef = cref.clip_coef(sumsq.item(), max_norm)
+    assert nc[0].item() == norm and nc[1].item() == coef, (nc.tolist(), norm, coef)
+    total = sum(cref.sumsq(b) for b in bufs)
+    assert abs(sumsq.item() - total) <= 1e-12 * total
+    for d, b in zip(dbufs, bufs):
+        want = b.clone()
+        cref.flat_scale(want, coef)
+        nat.flat_scale(d, nc[1:2])
+        assert_bits_equal(d, want, f"scale {b.dtype} max_norm={max_norm}")
+    if max_norm == 1e6:
+        assert coef == 1.0
+
+
+def test_clip_coef_nan_and_zero(nat):
+    nc = torch.zeros(2, dtype=torch.float32, device=DEV)
+    nat.clip_coef(torch.tensor([float("nan")], dtype=torch.float64, device=DEV), 1.0, nc)
+    assert torch.isnan(nc).all()
+    nat.clip_coef(torch.zeros(1, dtype=torch.float64, device=DEV), 1.0, nc)
+    assert nc.tolist() == [0.0, 1.0]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_scale_by_one_touches_nothing(nat, dtype):
+    g = torch.Generator().manual_seed(203)
+    x = mixed_values(g, 10_000, dtype)
+    d = x.to(DEV)
+    nat.flat_scale(d, torch.ones(1, device=DEV))
+    assert_bits_equal(d, x, "coef 1")
+    torch.testing.assert_close(d.view(torch.int16 if dtype != torch.float32 else torch.int32).cpu(),
+                               x.view(torch.int16 if dtype != torch.float32 else torch.int32))  # NaN payloads too
+
+
+ADAM_CASES = [
+    # decoupled, beta1, weight_decay, step, out16 dtype, grad_scale, zero_grad
+    (True, 0.9, 0.1, 1, torch.bfloat16, None, False),
+    (True, 0.9, 0.1, 7, torch.bfloat16, 0.37, True),
+    (True, 0.9, 0.0, 1000, torch.float16, None, False),
+    (True, 0.3, 0.01, 3, None, None, True),
+    (False, 0.9, 0.1, 2, torch.bfloat16, None, False),
+    (False, 0.4, 0.0, 5, None, 2.5, False),
+]
+
+
+@pytest.mark.parametrize("case", ADAM_CASES)
+def test_adamw_step(nat, case):
+    decoupled, beta1, wd, step, out_dt, gscale, zero_grad = case
+    g = torch.Generator().manual_seed(204 + step)
+    hp = dict(lr=3e-4, beta1=beta1, beta2=0.95, eps=1e-8, weight_decay=wd)
+    for n in SIZES:
+        _say("adamw", case, n)
+        p = mixed_values(g, n, torch.float32, 0.02)
+        grad = mixed_values(g, n, torch.float32, 1e-3).flip(0)
+        m = mixed_values(g, n, torch.float32, 1e-3).roll(n // 3 if n else 0)
+        v = mixed_values(g, n, torch.float32, 1e-3).abs().roll(n // 2 if n else 0) ** 2
+        dev = [torch.zeros(n + 8, device=DEV)[:n].copy_(t) for t in (p, grad, m, v)]
+        out = None if out_dt is None else torch.full((n + 8,), 9.0, dtype=out_dt, device=DEV)
+        gs = None if gscale is None else torch.tensor([gscale], device=DEV)
+        nat.adamw_step(dev[0], dev[1], dev[2], dev[3], None if out is None else out[:n], step=step,
+                       decoupled=decoupled, grad_scale=gs, zero_grad=zero_grad, **hp)
+        want_out = None if out_dt is None else torch.full((n + 8,), 9.0, dtype=out_dt)
+        cref.adamw_step(p, grad, m, v, None if want_out is None else want_out[:n], step=step, decoupled=decoupled,
+                        grad_scale=gscale, zero_grad=zero_grad, **hp)
+        for name, a, b in zip(("param", "grad", "exp_avg", "exp_avg_sq"), dev, (p, grad, m, v)):
+            assert_bits_equal(a, b, f"adamw {name} n={n}")
+        if out is not None:
+            assert_bits_equal(out, want_out, f"adamw out16 n={n}")
+
+
+def test_adamw_many_steps_track_torch_optim(nat):
+    """Ten steps of the fused kernel next to torch.optim.AdamW on the CPU: the
+    moments agree bit for bit, the parameters to the accuracy of torch's own
+    CPU square root (not correctly rounded), i.e. a few ulps of the update."""
+    n = 200_000
+    gen = torch.Generator().manual_seed(205)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    param = torch.nn.Parameter(p0.clone())
+    opt = torch.optim.AdamW([param], lr=1e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    dp, dm, dv = p0.to(DEV), torch.zeros(n, device=DEV), torch.zeros(n, device=DEV)
+    out16 = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    for step in range(1, 11):
+        grad = torch.randn(n, generator=gen) * 1e-3
+        param.grad = grad.clone()
+        opt.step()
+        nat.adamw_step(dp, grad.to(DEV), dm, dv, out16, lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1,
+                       step=step)
+    st = opt.state[param]
+    assert_bits_equal(dm, st["exp_avg"], "exp_avg after 10 steps")
+    assert_bits_equal(dv, st["exp_avg_sq"], "exp_avg_sq after 10 steps")
+    want = param.detach()
+    scale = torch.maximum(want.abs(), torch.full_like(want, 1e-3)).double()
+    err = (dp.cpu().double() - want.double()).abs()
+    assert bool((err <= 10 * 2.0**-22 * scale).all()), float((err / scale).max())
+    assert (dp.cpu().view(torch.int32) != want.view(torch.int32)).float().mean().item() < 0.25
+    assert_bits_equal(out16, dp.bfloat16(), "16-bit copy")
+
+
+def test_optim_errors_are_loud(nat):
+    a = torch.zeros(64, device=DEV)
+    with pytest.raises(RuntimeError):
+        nat.flat_fill(torch.zeros(8))
+    with pytest.raises(RuntimeError, match="aligned"):
+        nat.flat_fill(a[1:9])
+    with pytest.raises(TypeError):
+        nat.adamw_step(a, a.clone(), a.clone(), a.clone().half(), None, lr=1e-3, beta1=0.9, beta2=0.9, eps=1e-8,
+                       weight_decay=0.0, step=1)
+    with pytest.raises(RuntimeError):
+        nat.adamw_step(a, a.clone(), a.clone(), a.clone(), None, lr=1e-3, beta1=0.9, beta2=0.9, eps=1e-8,
+                       weight_decay=0.0, step=0)
+    out = torch.zeros(1, dtype=torch.float64, device=DEV)
+    with pytest.raises(RuntimeError):
+        nat.flat_sumsq(a, out, torch.zeros(16, dtype=torch.uint8, device=DEV))
+    assert nat.lib.yafsdp_flat_fill(a.data_ptr(), 7, 4, 0.0, None) == -2

@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libyafsdp_hip.so")
-SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip"]
+SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip"]
 HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "launch.h", "tuning.h"]
 ARCH = "gfx950"
 

@@ -40,6 +40,12 @@ EXPORTED_SYMBOLS = (
     "yafsdp_table_info",
     "yafsdp_gather_in",
     "yafsdp_scatter_out",
+    "yafsdp_flat_fill",
+    "yafsdp_sumsq_workspace_bytes",
+    "yafsdp_flat_sumsq",
+    "yafsdp_clip_coef",
+    "yafsdp_flat_scale",
+    "yafsdp_adamw_step",
     "yafsdp_set_option",
     "yafsdp_get_option",
 )
@@ -77,6 +83,18 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_gather_in.argtypes = [vp, vp, vp, i32, vp, i32, dbl, i32, vp]
     lib.yafsdp_scatter_out.restype = i32
     lib.yafsdp_scatter_out.argtypes = [vp, vp, i32, vp, vp, i32, vp]
+    lib.yafsdp_flat_fill.restype = i32
+    lib.yafsdp_flat_fill.argtypes = [vp, i32, i64, dbl, vp]
+    lib.yafsdp_sumsq_workspace_bytes.restype = ctypes.c_size_t
+    lib.yafsdp_sumsq_workspace_bytes.argtypes = []
+    lib.yafsdp_flat_sumsq.restype = i32
+    lib.yafsdp_flat_sumsq.argtypes = [vp, i32, i64, vp, i32, vp, ctypes.c_size_t, vp]
+    lib.yafsdp_clip_coef.restype = i32
+    lib.yafsdp_clip_coef.argtypes = [vp, dbl, vp, vp]
+    lib.yafsdp_flat_scale.restype = i32
+    lib.yafsdp_flat_scale.argtypes = [vp, i32, i64, vp, vp]
+    lib.yafsdp_adamw_step.restype = i32
+    lib.yafsdp_adamw_step.argtypes = [vp, vp, vp, vp, vp, i32, i64, dbl, dbl, dbl, dbl, dbl, i64, vp, i32, vp]
     lib.yafsdp_set_option.restype = i32
     lib.yafsdp_set_option.argtypes = [i32, i32]
     lib.yafsdp_get_option.restype = i32
@@ -322,6 +340,104 @@ class TensorTable:
                 ),
                 "yafsdp_scatter_out",
             )
+
+
+# ---- optimizer-side passes over a flat shard ---------------------------------
+ADAM_DECOUPLED_DECAY, ADAM_ZERO_GRAD = 1, 2
+
+
+def flat_fill(dst: torch.Tensor, value: float = 0.0) -> None:
+    """``dst.fill_(value)`` (``zero_()`` by default) on a flat buffer."""
+    _flat_arg(dst, "dst")
+    _check(lib.yafsdp_flat_fill(dst.data_ptr(), _dt(dst), dst.numel(), float(value), _stream(dst)), "yafsdp_flat_fill")
+
+
+def sumsq_workspace(device: torch.device) -> torch.Tensor:
+    """Scratch buffer that ``flat_sumsq`` needs; reusable across calls on one stream."""
+    return torch.empty(lib.yafsdp_sumsq_workspace_bytes(), dtype=torch.uint8, device=device)
+
+
+def flat_sumsq(src: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, accumulate: bool = False) -> None:
+    """``out[0] (+)= sum(float(src)**2)`` in binary64; ``out`` is a float64 device tensor."""
+    _flat_arg(src, "src"), _flat_arg(out, "out"), _flat_arg(workspace, "workspace")
+    if out.dtype != torch.float64 or out.numel() < 1:
+        raise TypeError("out must be a float64 tensor with at least one element")
+    if out.device != src.device or workspace.device != src.device:
+        raise RuntimeError("src, out and workspace must live on one device")
+    _check(
+        lib.yafsdp_flat_sumsq(
+            src.data_ptr(), _dt(src), src.numel(), out.data_ptr(), int(accumulate), workspace.data_ptr(),
+            workspace.numel() * workspace.element_size(), _stream(src),
+        ),
+        "yafsdp_flat_sumsq",
+    )
+
+
+def clip_coef(sumsq: torch.Tensor, max_norm: float, norm_and_coef: torch.Tensor) -> None:
+    """``norm_and_coef[0] = sqrt(sumsq[0])``, ``norm_and_coef[1] = min(max_norm / (norm + 1e-6), 1)`` (float32)."""
+    _flat_arg(sumsq, "sumsq"), _flat_arg(norm_and_coef, "norm_and_coef")
+    if sumsq.dtype != torch.float64 or norm_and_coef.dtype != torch.float32 or norm_and_coef.numel() < 2:
+        raise TypeError("sumsq must be float64 and norm_and_coef float32 with two elements")
+    _check(
+        lib.yafsdp_clip_coef(sumsq.data_ptr(), float(max_norm), norm_and_coef.data_ptr(), _stream(sumsq)),
+        "yafsdp_clip_coef",
+    )
+
+
+def flat_scale(buf: torch.Tensor, coef: torch.Tensor) -> None:
+    """``buf.mul_(coef)`` with a one-element float32 device tensor; a coefficient of exactly 1 costs no traffic."""
+    _flat_arg(buf, "buf"), _flat_arg(coef, "coef")
+    if coef.dtype != torch.float32 or coef.numel() != 1 or coef.device != buf.device:
+        raise TypeError("coef must be a one-element float32 tensor on the buffer's device")
+    _check(lib.yafsdp_flat_scale(buf.data_ptr(), _dt(buf), buf.numel(), coef.data_ptr(), _stream(buf)), "yafsdp_flat_scale")
+
+
+def adamw_step(
+    param: torch.Tensor,
+    grad: torch.Tensor,
+    exp_avg: torch.Tensor,
+    exp_avg_sq: torch.Tensor,
+    out16: torch.Tensor | None,
+    *,
+    lr: float,
+    beta1: float,
+    beta2: float,
+    eps: float,
+    weight_decay: float,
+    step: int,
+    decoupled: bool = True,
+    grad_scale: torch.Tensor | None = None,
+    zero_grad: bool = False,
+) -> None:
+    """One Adam(W) step on a flat float32 shard, fused with the 16-bit copy-in of the next iteration."""
+    n = param.numel()
+    for name, t in (("param", param), ("grad", grad), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+        _flat_arg(t, name)
+        if t.dtype != torch.float32:
+            raise TypeError(f"{name} must be float32, got {t.dtype}")
+        if t.numel() != n or t.device != param.device:
+            raise ValueError(f"{name}: expected {n} elements on {param.device}")
+    out_ptr, out_dt = None, 0
+    if out16 is not None:
+        _flat_arg(out16, "out16")
+        if out16.dtype not in (torch.bfloat16, torch.float16) or out16.numel() != n or out16.device != param.device:
+            raise TypeError("out16 must be a bfloat16 / float16 tensor of the shard's size on its device")
+        out_ptr, out_dt = out16.data_ptr(), _dt(out16)
+    gs_ptr = None
+    if grad_scale is not None:
+        _flat_arg(grad_scale, "grad_scale")
+        if grad_scale.dtype != torch.float32 or grad_scale.numel() != 1 or grad_scale.device != param.device:
+            raise TypeError("grad_scale must be a one-element float32 tensor on the shard's device")
+        gs_ptr = grad_scale.data_ptr()
+    flags = (ADAM_DECOUPLED_DECAY if decoupled else 0) | (ADAM_ZERO_GRAD if zero_grad else 0)
+    _check(
+        lib.yafsdp_adamw_step(
+            param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), out_ptr, out_dt, n,
+            float(lr), float(beta1), float(beta2), float(eps), float(weight_decay), int(step), gs_ptr, flags,
+            _stream(param),
+        ),
+        "yafsdp_adamw_step",
+    )
 
 
 def set_option(option: int, value: int) -> None:

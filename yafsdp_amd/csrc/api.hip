@@ -245,6 +245,113 @@ int yafsdp_get_option(int option, int* value) {
   return YAFSDP_ERR_INVALID_ARGUMENT;
 }
 
+namespace {
+// grid of an optimizer-side pass over `units` 16-byte (fill) or quad units
+int opt_grid(int64_t units, int block, int unroll, int* device_out) {
+  const int64_t tile = int64_t(block) * unroll;
+  const int64_t n_tiles = (units + tile - 1) / tile;
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess) device = 0;
+  if (device_out) *device_out = device;
+  return grid_for(n_tiles, g_flat_blocks_per_cu.load(std::memory_order_relaxed), device);
+}
+
+uint32_t fill_pattern(int dtype, double value) {
+  const float f = static_cast<float>(value);
+  uint32_t bits;
+  std::memcpy(&bits, &f, 4);
+  if (dtype == DT_F32) return bits;
+  uint16_t h;
+  if (dtype == DT_BF16) {
+    if (std::isnan(f)) h = 0x7FC0;
+    else h = uint16_t((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16);  // round to nearest even
+  } else {
+    const _Float16 x = static_cast<_Float16>(f);
+    std::memcpy(&h, &x, 2);
+  }
+  return uint32_t(h) | (uint32_t(h) << 16);
+}
+}  // namespace
+
+int yafsdp_flat_fill(void* dst, int dtype, int64_t n, double value, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && dst == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;
+  if (!aligned_to(dst, 16)) return YAFSDP_ERR_MISALIGNED;
+  const int grid = opt_grid(n / (16 / item_size(dtype)), kOptBlock, kFillUnroll, nullptr);
+  return int(launch_fill(dtype, dst, n, fill_pattern(dtype, value), grid, static_cast<hipStream_t>(stream)));
+}
+
+size_t yafsdp_sumsq_workspace_bytes(void) { return size_t(kSumsqMaxPartials) * sizeof(double); }
+
+int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || sumsq == nullptr || workspace == nullptr || (n > 0 && src == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (workspace_bytes < yafsdp_sumsq_workspace_bytes()) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(src, 16) || !aligned_to(sumsq, 8) || !aligned_to(workspace, 8)) return YAFSDP_ERR_MISALIGNED;
+  int grid = opt_grid(n >> 2, kOptBlock, kSumsqUnroll, nullptr);
+  if (grid > kSumsqMaxPartials) grid = kSumsqMaxPartials;
+  return int(launch_sumsq(dtype, src, n, static_cast<double*>(workspace), grid, sumsq, accumulate ? 1 : 0,
+                          static_cast<hipStream_t>(stream)));
+}
+
+int yafsdp_clip_coef(const double* sumsq, double max_norm, float* norm_and_coef, void* stream) {
+  if (sumsq == nullptr || norm_and_coef == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(sumsq, 8) || !aligned_to(norm_and_coef, 4)) return YAFSDP_ERR_MISALIGNED;
+  return int(launch_clip_coef(sumsq, static_cast<float>(max_norm), norm_and_coef, static_cast<hipStream_t>(stream)));
+}
+
+int yafsdp_flat_scale(void* buf, int dtype, int64_t n, const float* coef, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || coef == nullptr || (n > 0 && buf == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;
+  if (!aligned_to(buf, 16) || !aligned_to(coef, 4)) return YAFSDP_ERR_MISALIGNED;
+  const int grid = opt_grid(n >> 2, kOptBlock, kScaleUnroll, nullptr);
+  return int(launch_scale(dtype, buf, n, coef, grid, static_cast<hipStream_t>(stream)));
+}
+
+int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_sq, void* out16, int out16_dtype,
+                      int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,
+                      int64_t step, const float* grad_scale, int flags, void* stream) {
+  if (n < 0 || step < 1) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (out16 != nullptr && out16_dtype != DT_BF16 && out16_dtype != DT_F16) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n == 0) return YAFSDP_OK;
+  if (param == nullptr || grad == nullptr || exp_avg == nullptr || exp_avg_sq == nullptr)
+    return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(param, 16) || !aligned_to(grad, 16) || !aligned_to(exp_avg, 16) || !aligned_to(exp_avg_sq, 16) ||
+      (out16 != nullptr && !aligned_to(out16, 8)) || (grad_scale != nullptr && !aligned_to(grad_scale, 4)))
+    return YAFSDP_ERR_MISALIGNED;
+  // scalars exactly as torch.optim computes them: Python floats (binary64),
+  // rounded to binary32 where they enter a tensor op
+  AdamScalars s;
+  std::memset(&s, 0, sizeof(s));
+  s.flags = 0;
+  if (weight_decay != 0.0) {
+    if (flags & YAFSDP_ADAM_DECOUPLED_DECAY) {
+      s.flags |= ADAM_DECOUPLED;
+      s.decay = static_cast<float>(1.0 - lr * weight_decay);
+    } else {
+      s.flags |= ADAM_L2;
+      s.l2 = static_cast<float>(weight_decay);
+    }
+  }
+  s.w = static_cast<float>(1.0 - beta1);
+  s.w_m1 = s.w - 1.0f;
+  if (std::fabs(s.w) < 0.5f) s.flags |= ADAM_W_SMALL;
+  s.beta2 = static_cast<float>(beta2);
+  s.one_m_beta2 = static_cast<float>(1.0 - beta2);
+  const double bc1 = 1.0 - std::pow(beta1, double(step));
+  const double bc2 = 1.0 - std::pow(beta2, double(step));
+  s.bc2_sqrt = static_cast<float>(std::pow(bc2, 0.5));
+  s.eps = static_cast<float>(eps);
+  s.neg_step = static_cast<float>(-(lr / bc1));
+  if (flags & YAFSDP_ADAM_ZERO_GRAD) s.flags |= ADAM_ZERO_GRAD;
+  const int grid = opt_grid(n >> 2, kAdamBlock, kAdamUnroll, nullptr);
+  return int(launch_adamw(out16_dtype, param, grad, exp_avg, exp_avg_sq, out16, n, s, grad_scale, grid,
+                          static_cast<hipStream_t>(stream)));
+}
+
 int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, void* stream) {
   if (!valid_dtype(dst_dtype) || !valid_dtype(src_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && (dst == nullptr || src == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;

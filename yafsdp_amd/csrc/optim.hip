@@ -1,0 +1,85 @@
+// Instantiations and dtype dispatch of the optimizer-side kernels.
+#include "launch.h"
+#include "optim_kernels.cuh"
+#include "tuning.h"
+
+namespace yafsdp {
+
+hipError_t launch_fill(int dt, void* dst, int64_t n, uint32_t pattern, int grid, hipStream_t stream) {
+  switch (dt) {
+    case DT_F32:
+      fill_kernel<F32, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, pattern);
+      break;
+    case DT_BF16:
+      fill_kernel<BF16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, pattern);
+      break;
+    case DT_F16:
+      fill_kernel<F16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, pattern);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_scale(int dt, void* buf, int64_t n, const float* coef, int grid, hipStream_t stream) {
+  switch (dt) {
+    case DT_F32:
+      scale_kernel<F32, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
+          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, coef);
+      break;
+    case DT_BF16:
+      scale_kernel<BF16, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
+          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, coef);
+      break;
+    case DT_F16:
+      scale_kernel<F16, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
+          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, coef);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_sumsq(int dt, const void* src, int64_t n, double* partials, int grid, double* out, int accumulate,
+                        hipStream_t stream) {
+  switch (dt) {
+    case DT_F32:
+      sumsq_kernel<F32, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, partials);
+      break;
+    case DT_BF16:
+      sumsq_kernel<BF16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, partials);
+      break;
+    case DT_F16:
+      sumsq_kernel<F16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, partials);
+      break;
+    default: return hipErrorInvalidValue;
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  sumsq_final_kernel<kOptBlock><<<dim3(1), dim3(kOptBlock), 0, stream>>>(partials, grid, out, accumulate);
+  return hipGetLastError();
+}
+
+hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and_coef, hipStream_t stream) {
+  clip_coef_kernel<<<dim3(1), dim3(64), 0, stream>>>(sumsq, max_norm, norm_and_coef);
+  return hipGetLastError();
+}
+
+hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n,
+                        const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream) {
+  if (out16 == nullptr) {
+    adamw_kernel<F32, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
+        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, nullptr, n, s, grad_scale);
+  } else if (out_dt == DT_BF16) {
+    adamw_kernel<BF16, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
+        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, s, grad_scale);
+  } else if (out_dt == DT_F16) {
+    adamw_kernel<F16, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
+        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, s, grad_scale);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace yafsdp

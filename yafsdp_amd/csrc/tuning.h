@@ -27,6 +27,32 @@ inline int table_block_for(long long padded_elems, int threshold_log2) {
   return padded_elems > (1LL << threshold_log2) ? kTableBlockLarge : kTableBlockSmall;
 }
 inline long long table_tile_elems(int block) { return (long long)block * kTableUnroll * 8; }
+// optimizer-side passes: a tile is block * unroll quads (4 elements each)
+#ifndef YAFSDP_FILL_U
+#define YAFSDP_FILL_U 4
+#endif
+#ifndef YAFSDP_SCALE_U
+#define YAFSDP_SCALE_U 2
+#endif
+#ifndef YAFSDP_SUMSQ_U
+#define YAFSDP_SUMSQ_U 4
+#endif
+#ifndef YAFSDP_ADAM_U
+#define YAFSDP_ADAM_U 2
+#endif
+#ifndef YAFSDP_ADAM_BLOCK
+#define YAFSDP_ADAM_BLOCK 256
+#endif
+constexpr int kOptBlock = 256;
+constexpr int kFillUnroll = YAFSDP_FILL_U;    // 16-byte stores per lane per tile
+constexpr int kScaleUnroll = YAFSDP_SCALE_U;
+constexpr int kSumsqUnroll = YAFSDP_SUMSQ_U;
+constexpr int kAdamBlock = YAFSDP_ADAM_BLOCK;
+constexpr int kAdamUnroll = YAFSDP_ADAM_U;
+constexpr bool kOptNtLoad = true;
+constexpr bool kOptNtStore = true;
+// workgroups (= partial sums) of the sum-of-squares pass; the workspace holds one double each
+constexpr int kSumsqMaxPartials = 16384;
 // default grid cap in workgroups per compute unit.  Measured: one workgroup per
 // tile (no cap reached) beats a persistent grid-stride grid by 5-10 % on every
 // kernel of the path, so the cap is far above any tile count of interest.
