@@ -142,7 +142,8 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
  * over the per-parameter fragments of the flat shard (dispatch table of its
  * tensor subclass, ya_fsdp/_tensor.py:122-316).  The fragments of one group are
  * consecutive ranges of one flat buffer, so each op is one pass over that
- * buffer here.  Every pointer below is device memory, 16-byte aligned. */
+ * buffer here.  Every pointer below is device memory; ranges may start at any
+ * element-aligned address (16-byte aligned starts skip the peeled head). */
 
 /* dst[0:n] = cast(value).  `_foreach_zero_` of optimizer.zero_grad(set_to_none=False)
  * (ya_fsdp/_tensor.py:243-245; the legacy wrapper allows no other form,
@@ -183,7 +184,10 @@ int yafsdp_flat_scale(void* buf, int dtype, int64_t n, const float* coef, void* 
  * f16).  `step` is the 1-based step count.  `grad_scale` (device, may be NULL)
  * multiplies the gradient first, as a preceding `grad.mul_(coef)` would, without
  * writing it back.  flags: YAFSDP_ADAM_DECOUPLED_DECAY = AdamW, otherwise the
- * L2 form of Adam; YAFSDP_ADAM_ZERO_GRAD also zero-fills `grad`. */
+ * L2 form of Adam; YAFSDP_ADAM_ZERO_GRAD also zero-fills `grad`.  The four
+ * binary32 arrays must share one address residue modulo 16 bytes and `out16`
+ * half of it modulo 8 (true for one fragment range of identically laid out
+ * shards). */
 enum { YAFSDP_ADAM_DECOUPLED_DECAY = 1, YAFSDP_ADAM_ZERO_GRAD = 2 };
 int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_sq, void* out16, int out16_dtype,
                       int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,

@@ -34,12 +34,13 @@ SIZES = [0, 1, 3, 4, 7, 8, 1023, 2048, 2049, 100_003, (1 << 20) + 5]
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("value", [0.0, 1.5, -0.0, 3.0e-41, float("inf"), 0.1])
 def test_flat_fill(nat, dtype, value):
-    for n in SIZES:
-        _say("fill", dtype, value, n)
-        buf = torch.full((n + 16,), 7.0, dtype=dtype, device=DEV)
-        nat.flat_fill(buf[8 : 8 + n], value)
-        want = torch.full((n + 16,), 7.0, dtype=dtype)
-        want[8 : 8 + n] = torch.tensor(value, dtype=torch.float32).to(dtype)
+    for k, n in enumerate(SIZES):
+        o = 8 + k % 8  # every start residue modulo 16 bytes
+        _say("fill", dtype, value, n, o)
+        buf = torch.full((n + 24,), 7.0, dtype=dtype, device=DEV)
+        nat.flat_fill(buf[o : o + n], value)
+        want = torch.full((n + 24,), 7.0, dtype=dtype)
+        want[o : o + n] = torch.tensor(value, dtype=torch.float32).to(dtype)
         assert_bits_equal(buf, want, f"fill n={n}")
 
 
@@ -48,20 +49,22 @@ def test_flat_sumsq(nat, dtype):
     g = torch.Generator().manual_seed(201)
     ws = nat.sumsq_workspace(torch.device(DEV))
     out = torch.full((2,), 5.0, dtype=torch.float64, device=DEV)
-    for n in SIZES + [(1 << 23) + 11]:
-        _say("sumsq", dtype, n)
+    for k, n in enumerate(SIZES + [(1 << 23) + 11]):
+        o = k % 8
+        _say("sumsq", dtype, n, o)
         x = (torch.randn(n, generator=g) * 3e-2).to(dtype)
         want = cref.sumsq(x)
-        pad = torch.zeros(n + 8, dtype=dtype, device=DEV)  # 16-byte aligned view at any n
-        pad[:n] = x.to(DEV)
-        nat.flat_sumsq(pad[:n], out, ws, accumulate=False)
+        pad = torch.full((n + 16,), 100.0, dtype=dtype, device=DEV)
+        pad = pad[o : o + n]
+        pad.copy_(x)
+        nat.flat_sumsq(pad, out, ws, accumulate=False)
         got = out.cpu()
         assert got[1].item() == 5.0
         assert abs(got[0].item() - want) <= 1e-12 * want, (n, got[0].item(), want)
-        nat.flat_sumsq(pad[:n], out, ws, accumulate=True)
+        nat.flat_sumsq(pad, out, ws, accumulate=True)
         assert abs(out[0].item() - 2 * want) <= 1e-12 * 2 * want
         # reproducible: same bits on a second run
-        nat.flat_sumsq(pad[:n], out, ws, accumulate=False)
+        nat.flat_sumsq(pad, out, ws, accumulate=False)
         assert out[0].item() == got[0].item()
     # exactness where binary32 accumulation would fail: 2^24 ones plus one tiny term
     ones = torch.ones((1 << 24) + 4, dtype=torch.float32, device=DEV)
@@ -97,7 +100,7 @@ def test_clip_coef_and_scale(nat, max_norm):
         b[:6] = torch.tensor([0.0, -0.0, 1e-40, -1e-40, 1.0, -3.0]).to(b.dtype)
     dbufs = []
     for i, b in enumerate(bufs):
-        d = torch.zeros(b.numel() + 8, dtype=b.dtype, device=DEV)[: b.numel()]
+        d = torch.zeros(b.numel() + 8, dtype=b.dtype, device=DEV)[i + 1 : i + 1 + b.numel()]  # unaligned starts
         d.copy_(b)
         dbufs.append(d)
         nat.flat_sumsq(d, sumsq, ws, accumulate=i > 0)
@@ -150,22 +153,26 @@ def test_adamw_step(nat, case):
     decoupled, beta1, wd, step, out_dt, gscale, zero_grad = case
     g = torch.Generator().manual_seed(204 + step)
     hp = dict(lr=3e-4, beta1=beta1, beta2=0.95, eps=1e-8, weight_decay=wd)
-    for n in SIZES:
-        _say("adamw", case, n)
+    for k, n in enumerate(SIZES):
+        o = k % 4  # fragment ranges start at any element of the shard
+        _say("adamw", case, n, o)
         p = mixed_values(g, n, torch.float32, 0.02)
         grad = mixed_values(g, n, torch.float32, 1e-3).flip(0)
         m = mixed_values(g, n, torch.float32, 1e-3).roll(n // 3 if n else 0)
         v = mixed_values(g, n, torch.float32, 1e-3).abs().roll(n // 2 if n else 0) ** 2
-        dev = [torch.zeros(n + 8, device=DEV)[:n].copy_(t) for t in (p, grad, m, v)]
+        full = [torch.full((n + 8,), 5.0, device=DEV) for _ in range(4)]
+        dev = [f[o : o + n].copy_(t) for f, t in zip(full, (p, grad, m, v))]
         out = None if out_dt is None else torch.full((n + 8,), 9.0, dtype=out_dt, device=DEV)
         gs = None if gscale is None else torch.tensor([gscale], device=DEV)
-        nat.adamw_step(dev[0], dev[1], dev[2], dev[3], None if out is None else out[:n], step=step,
+        nat.adamw_step(dev[0], dev[1], dev[2], dev[3], None if out is None else out[o : o + n], step=step,
                        decoupled=decoupled, grad_scale=gs, zero_grad=zero_grad, **hp)
         want_out = None if out_dt is None else torch.full((n + 8,), 9.0, dtype=out_dt)
-        cref.adamw_step(p, grad, m, v, None if want_out is None else want_out[:n], step=step, decoupled=decoupled,
-                        grad_scale=gscale, zero_grad=zero_grad, **hp)
-        for name, a, b in zip(("param", "grad", "exp_avg", "exp_avg_sq"), dev, (p, grad, m, v)):
-            assert_bits_equal(a, b, f"adamw {name} n={n}")
+        cref.adamw_step(p, grad, m, v, None if want_out is None else want_out[o : o + n], step=step,
+                        decoupled=decoupled, grad_scale=gscale, zero_grad=zero_grad, **hp)
+        for name, f, b in zip(("param", "grad", "exp_avg", "exp_avg_sq"), full, (p, grad, m, v)):
+            want_full = torch.full((n + 8,), 5.0)
+            want_full[o : o + n] = b
+            assert_bits_equal(f, want_full, f"adamw {name} n={n}")
         if out is not None:
             assert_bits_equal(out, want_out, f"adamw out16 n={n}")
 
@@ -202,8 +209,9 @@ def test_optim_errors_are_loud(nat):
     a = torch.zeros(64, device=DEV)
     with pytest.raises(RuntimeError):
         nat.flat_fill(torch.zeros(8))
-    with pytest.raises(RuntimeError, match="aligned"):
-        nat.flat_fill(a[1:9])
+    with pytest.raises(RuntimeError, match="aligned"):  # arrays of one call must share their residue mod 16 bytes
+        nat.adamw_step(a[1:9], a.clone()[:8], a.clone()[:8], a.clone()[:8], None, lr=1e-3, beta1=0.9, beta2=0.9,
+                       eps=1e-8, weight_decay=0.0, step=1)
     with pytest.raises(TypeError):
         nat.adamw_step(a, a.clone(), a.clone(), a.clone().half(), None, lr=1e-3, beta1=0.9, beta2=0.9, eps=1e-8,
                        weight_decay=0.0, step=1)

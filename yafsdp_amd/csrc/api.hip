@@ -256,6 +256,12 @@ int opt_grid(int64_t units, int block, int unroll, int* device_out) {
   return grid_for(n_tiles, g_flat_blocks_per_cu.load(std::memory_order_relaxed), device);
 }
 
+// leading elements up to the next 16-byte boundary (at most n)
+int head_elems(const void* p, int elem_size, int64_t n) {
+  int64_t head = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / elem_size;
+  return int(head > n ? n : head);
+}
+
 uint32_t fill_pattern(int dtype, double value) {
   const float f = static_cast<float>(value);
   uint32_t bits;
@@ -277,9 +283,10 @@ int yafsdp_flat_fill(void* dst, int dtype, int64_t n, double value, void* stream
   if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && dst == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (n == 0) return YAFSDP_OK;
-  if (!aligned_to(dst, 16)) return YAFSDP_ERR_MISALIGNED;
-  const int grid = opt_grid(n / (16 / item_size(dtype)), kOptBlock, kFillUnroll, nullptr);
-  return int(launch_fill(dtype, dst, n, fill_pattern(dtype, value), grid, static_cast<hipStream_t>(stream)));
+  if (!aligned_to(dst, item_size(dtype))) return YAFSDP_ERR_MISALIGNED;
+  const int head = head_elems(dst, item_size(dtype), n);
+  const int grid = opt_grid((n - head) / (16 / item_size(dtype)), kOptBlock, kFillUnroll, nullptr);
+  return int(launch_fill(dtype, dst, n, head, fill_pattern(dtype, value), grid, static_cast<hipStream_t>(stream)));
 }
 
 size_t yafsdp_sumsq_workspace_bytes(void) { return size_t(kSumsqMaxPartials) * sizeof(double); }
@@ -289,10 +296,12 @@ int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int 
   if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || sumsq == nullptr || workspace == nullptr || (n > 0 && src == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (workspace_bytes < yafsdp_sumsq_workspace_bytes()) return YAFSDP_ERR_INVALID_ARGUMENT;
-  if (!aligned_to(src, 16) || !aligned_to(sumsq, 8) || !aligned_to(workspace, 8)) return YAFSDP_ERR_MISALIGNED;
-  int grid = opt_grid(n >> 2, kOptBlock, kSumsqUnroll, nullptr);
+  if (!aligned_to(src, item_size(dtype)) || !aligned_to(sumsq, 8) || !aligned_to(workspace, 8))
+    return YAFSDP_ERR_MISALIGNED;
+  const int head = head_elems(src, item_size(dtype), n);
+  int grid = opt_grid((n - head) >> 2, kOptBlock, kSumsqUnroll, nullptr);
   if (grid > kSumsqMaxPartials) grid = kSumsqMaxPartials;
-  return int(launch_sumsq(dtype, src, n, static_cast<double*>(workspace), grid, sumsq, accumulate ? 1 : 0,
+  return int(launch_sumsq(dtype, src, n, head, static_cast<double*>(workspace), grid, sumsq, accumulate ? 1 : 0,
                           static_cast<hipStream_t>(stream)));
 }
 
@@ -306,9 +315,10 @@ int yafsdp_flat_scale(void* buf, int dtype, int64_t n, const float* coef, void* 
   if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || coef == nullptr || (n > 0 && buf == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (n == 0) return YAFSDP_OK;
-  if (!aligned_to(buf, 16) || !aligned_to(coef, 4)) return YAFSDP_ERR_MISALIGNED;
-  const int grid = opt_grid(n >> 2, kOptBlock, kScaleUnroll, nullptr);
-  return int(launch_scale(dtype, buf, n, coef, grid, static_cast<hipStream_t>(stream)));
+  if (!aligned_to(buf, item_size(dtype)) || !aligned_to(coef, 4)) return YAFSDP_ERR_MISALIGNED;
+  const int head = head_elems(buf, item_size(dtype), n);
+  const int grid = opt_grid((n - head) >> 2, kOptBlock, kScaleUnroll, nullptr);
+  return int(launch_scale(dtype, buf, n, head, coef, grid, static_cast<hipStream_t>(stream)));
 }
 
 int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_sq, void* out16, int out16_dtype,
@@ -319,9 +329,16 @@ int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_
   if (n == 0) return YAFSDP_OK;
   if (param == nullptr || grad == nullptr || exp_avg == nullptr || exp_avg_sq == nullptr)
     return YAFSDP_ERR_INVALID_ARGUMENT;
-  if (!aligned_to(param, 16) || !aligned_to(grad, 16) || !aligned_to(exp_avg, 16) || !aligned_to(exp_avg_sq, 16) ||
-      (out16 != nullptr && !aligned_to(out16, 8)) || (grad_scale != nullptr && !aligned_to(grad_scale, 4)))
+  // the four binary32 arrays must share one residue modulo 16 bytes (fragments at
+  // one offset of identically laid out shards do), and out16 the matching one
+  // modulo 8, so that peeling `head` elements aligns all of them at once
+  const uintptr_t res = reinterpret_cast<uintptr_t>(param) & 15;
+  if ((res & 3) != 0 || (reinterpret_cast<uintptr_t>(grad) & 15) != res ||
+      (reinterpret_cast<uintptr_t>(exp_avg) & 15) != res || (reinterpret_cast<uintptr_t>(exp_avg_sq) & 15) != res ||
+      (out16 != nullptr && (reinterpret_cast<uintptr_t>(out16) & 7) != (res >> 1)) ||
+      (grad_scale != nullptr && !aligned_to(grad_scale, 4)))
     return YAFSDP_ERR_MISALIGNED;
+  const int head = head_elems(param, 4, n);
   // scalars exactly as torch.optim computes them: Python floats (binary64),
   // rounded to binary32 where they enter a tensor op
   AdamScalars s;
@@ -347,8 +364,8 @@ int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_
   s.eps = static_cast<float>(eps);
   s.neg_step = static_cast<float>(-(lr / bc1));
   if (flags & YAFSDP_ADAM_ZERO_GRAD) s.flags |= ADAM_ZERO_GRAD;
-  const int grid = opt_grid(n >> 2, kAdamBlock, kAdamUnroll, nullptr);
-  return int(launch_adamw(out16_dtype, param, grad, exp_avg, exp_avg_sq, out16, n, s, grad_scale, grid,
+  const int grid = opt_grid((n - head) >> 2, kAdamBlock, kAdamUnroll, nullptr);
+  return int(launch_adamw(out16_dtype, param, grad, exp_avg, exp_avg_sq, out16, n, head, s, grad_scale, grid,
                           static_cast<hipStream_t>(stream)));
 }
 

@@ -21,7 +21,7 @@ template <class META>
 hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total,
                           int n_tiles, int grid, hipStream_t stream);
 
-// optimizer-side passes (optim.hip); ranges are 16-byte aligned
+// optimizer-side passes (optim.hip); `head` leading elements bring the range to a 16-byte boundary
 // scalars of one Adam step, binary32 as they enter the tensor ops (see adamw_kernel)
 struct AdamScalars {
   float decay;     // 1 - lr*wd (AdamW), unused otherwise
@@ -36,13 +36,13 @@ struct AdamScalars {
   int flags;       // bit 0: decoupled decay, bit 1: L2 decay, bit 2: w < 0.5, bit 3: zero the gradient
 };
 enum : int { ADAM_DECOUPLED = 1, ADAM_L2 = 2, ADAM_W_SMALL = 4, ADAM_ZERO_GRAD = 8 };
-hipError_t launch_fill(int dt, void* dst, int64_t n, uint32_t pattern, int grid, hipStream_t stream);
-hipError_t launch_scale(int dt, void* buf, int64_t n, const float* coef, int grid, hipStream_t stream);
+hipError_t launch_fill(int dt, void* dst, int64_t n, int head, uint32_t pattern, int grid, hipStream_t stream);
+hipError_t launch_scale(int dt, void* buf, int64_t n, int head, const float* coef, int grid, hipStream_t stream);
 // `partials` holds `grid` doubles; out[0] (+)= their sum
-hipError_t launch_sumsq(int dt, const void* src, int64_t n, double* partials, int grid, double* out, int accumulate,
-                        hipStream_t stream);
+hipError_t launch_sumsq(int dt, const void* src, int64_t n, int head, double* partials, int grid, double* out,
+                        int accumulate, hipStream_t stream);
 hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and_coef, hipStream_t stream);
-hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n,
+hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n, int head,
                         const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream);
 
 }  // namespace yafsdp

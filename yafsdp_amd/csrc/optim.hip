@@ -5,52 +5,53 @@
 
 namespace yafsdp {
 
-hipError_t launch_fill(int dt, void* dst, int64_t n, uint32_t pattern, int grid, hipStream_t stream) {
+hipError_t launch_fill(int dt, void* dst, int64_t n, int head, uint32_t pattern, int grid, hipStream_t stream) {
   switch (dt) {
     case DT_F32:
-      fill_kernel<F32, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, pattern);
+      fill_kernel<F32, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, head, pattern);
       break;
     case DT_BF16:
-      fill_kernel<BF16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, pattern);
+      fill_kernel<BF16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, head, pattern);
       break;
     case DT_F16:
-      fill_kernel<F16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, pattern);
+      fill_kernel<F16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, head, pattern);
       break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }
 
-hipError_t launch_scale(int dt, void* buf, int64_t n, const float* coef, int grid, hipStream_t stream) {
+hipError_t launch_scale(int dt, void* buf, int64_t n, int head, const float* coef, int grid, hipStream_t stream) {
   switch (dt) {
     case DT_F32:
       scale_kernel<F32, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
-          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, coef);
+          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, head, coef);
       break;
     case DT_BF16:
       scale_kernel<BF16, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
-          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, coef);
+          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, head, coef);
       break;
     case DT_F16:
       scale_kernel<F16, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
-          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, coef);
+          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, head, coef);
       break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }
 
-hipError_t launch_sumsq(int dt, const void* src, int64_t n, double* partials, int grid, double* out, int accumulate,
+hipError_t launch_sumsq(int dt, const void* src, int64_t n, int head, double* partials, int grid, double* out,
+                        int accumulate,
                         hipStream_t stream) {
   switch (dt) {
     case DT_F32:
-      sumsq_kernel<F32, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, partials);
+      sumsq_kernel<F32, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, head, partials);
       break;
     case DT_BF16:
-      sumsq_kernel<BF16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, partials);
+      sumsq_kernel<BF16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, head, partials);
       break;
     case DT_F16:
-      sumsq_kernel<F16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, partials);
+      sumsq_kernel<F16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, head, partials);
       break;
     default: return hipErrorInvalidValue;
   }
@@ -65,17 +66,17 @@ hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and
   return hipGetLastError();
 }
 
-hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n,
+hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n, int head,
                         const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream) {
   if (out16 == nullptr) {
     adamw_kernel<F32, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
-        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, nullptr, n, s, grad_scale);
+        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, nullptr, n, head, s, grad_scale);
   } else if (out_dt == DT_BF16) {
     adamw_kernel<BF16, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
-        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, s, grad_scale);
+        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, head, s, grad_scale);
   } else if (out_dt == DT_F16) {
     adamw_kernel<F16, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
-        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, s, grad_scale);
+        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, head, s, grad_scale);
   } else {
     return hipErrorInvalidValue;
   }

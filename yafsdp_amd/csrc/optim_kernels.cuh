@@ -3,7 +3,8 @@
 // coefficient (gradient clipping) and the fused AdamW step that also emits the
 // 16-bit all-gather input of the next iteration.
 //
-// All four are single passes over contiguous, 16-byte aligned ranges.  A lane
+// All four are single passes over contiguous ranges (up to 3 or 7 leading
+// elements are peeled to reach a 16-byte boundary).  A lane
 // owns quads (4 consecutive elements); quad j of lane t inside a tile of
 // BLOCK*U quads is t + j*BLOCK, so every wave64 access is one contiguous span
 // (1 KiB of fp32, 512 B of a 2-byte dtype).  All loads of a lane are issued
@@ -16,11 +17,21 @@ namespace yafsdp {
 
 // ------------------------------------------------------------------- fill ----
 // dst[i] = pattern for i in [0, n); `pattern` holds the element replicated to 32
-// bits.  dst is 16-byte aligned.
+// bits.  `head` leading elements bring dst to a 16-byte boundary; workgroup 0
+// writes them and the tail one by one.
+template <class D>
+__device__ __forceinline__ void fill_scalar(void* dst, int64_t i, uint32_t pattern) {
+  if constexpr (D::kSize == 4) reinterpret_cast<uint32_t*>(dst)[i] = pattern;
+  else reinterpret_cast<uint16_t*>(dst)[i] = uint16_t(pattern & 0xFFFFu);
+}
+
 template <class D, int BLOCK, int U, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
-fill_kernel(void* dst, int64_t n, uint32_t pattern) {
+fill_kernel(void* dst0, int64_t n0, int head, uint32_t pattern) {
   constexpr int kPer = 16 / D::kSize;  // elements per 16-byte store
+  if (blockIdx.x == 0 && int(threadIdx.x) < head) fill_scalar<D>(dst0, threadIdx.x, pattern);
+  void* dst = reinterpret_cast<char*>(dst0) + int64_t(head) * D::kSize;
+  const int64_t n = n0 - head;
   const int64_t n_vec = n / kPer;
   constexpr int64_t kTile = int64_t(BLOCK) * U;
   const int64_t n_tiles = (n_vec + kTile - 1) / kTile;
@@ -40,10 +51,7 @@ fill_kernel(void* dst, int64_t n, uint32_t pattern) {
   }
   if (blockIdx.x == 0) {
     const int64_t i = n_vec * kPer + threadIdx.x;
-    if (i < n) {
-      if constexpr (D::kSize == 4) reinterpret_cast<uint32_t*>(dst)[i] = pattern;
-      else reinterpret_cast<uint16_t*>(dst)[i] = uint16_t(pattern & 0xFFFFu);
-    }
+    if (i < n) fill_scalar<D>(dst, i, pattern);
   }
 }
 
@@ -52,11 +60,17 @@ fill_kernel(void* dst, int64_t n, uint32_t pattern) {
 // touched when the coefficient is exactly 1 (x * 1 == x for every x).
 template <class D, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
-scale_kernel(void* buf, int64_t n, const float* coef) {
+scale_kernel(void* buf0, int64_t n0, int head, const float* coef) {
   typedef typename D::storage d_t;
   const float c = *reinterpret_cast<const __attribute__((address_space(4))) float*>(
       reinterpret_cast<uintptr_t>(coef));
   if (c == 1.0f) return;
+  if (blockIdx.x == 0 && int(threadIdx.x) < head) {
+    d_t* p = reinterpret_cast<d_t*>(buf0);
+    p[threadIdx.x] = from_f32<D>(opaque(__fmul_rn(opaque(to_f32<D>(p[threadIdx.x])), c)));
+  }
+  void* buf = reinterpret_cast<char*>(buf0) + int64_t(head) * D::kSize;
+  const int64_t n = n0 - head;
   const int64_t n_quads = n >> 2;
   constexpr int64_t kTile = int64_t(BLOCK) * U;
   const int64_t n_tiles = (n_quads + kTile - 1) / kTile;
@@ -118,9 +132,11 @@ __device__ __forceinline__ double block_sum(double v, double* lds) {
 
 template <class S, int BLOCK, int U, bool NTL>
 __global__ void __launch_bounds__(BLOCK)
-sumsq_kernel(const void* src, int64_t n, double* partials) {
+sumsq_kernel(const void* src0, int64_t n0, int head, double* partials) {
   typedef typename S::storage s_t;
   __shared__ double lds[BLOCK / 64];
+  const void* src = reinterpret_cast<const char*>(src0) + int64_t(head) * S::kSize;
+  const int64_t n = n0 - head;
   const int64_t n_quads = n >> 2;
   constexpr int64_t kTile = int64_t(BLOCK) * U;
   const int64_t n_tiles = (n_quads + kTile - 1) / kTile;
@@ -155,6 +171,10 @@ sumsq_kernel(const void* src, int64_t n, double* partials) {
     if (i < n) {
       const double x = double(to_f32<S>(reinterpret_cast<const s_t*>(src)[i]));
       acc[0] = __fma_rn(x, x, acc[0]);
+    }
+    if (int(threadIdx.x) < head) {
+      const double x = double(to_f32<S>(reinterpret_cast<const s_t*>(src0)[threadIdx.x]));
+      acc[1] = __fma_rn(x, x, acc[1]);
     }
   }
   const double t = block_sum<BLOCK>((acc[0] + acc[1]) + (acc[2] + acc[3]), lds);
@@ -214,13 +234,20 @@ __device__ __forceinline__ void adam_elem(float& p, float g, float& m, float& v,
 // O is the 16-bit output dtype, or F32 for "no 16-bit output".
 template <class O, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
-adamw_kernel(float* p, float* g, float* m, float* v, void* out16, int64_t n, AdamScalars s, const float* grad_scale) {
+adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0, int head, AdamScalars s,
+             const float* grad_scale) {
+  static_assert(BLOCK >= 128, "workgroup 0 peels the tail with wave 0 and the head with wave 1");
   constexpr bool kOut = !same_t<O, F32>::value;
   const bool scaled = grad_scale != nullptr;
   float gs = 1.0f;
   if (scaled)
     gs = *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(grad_scale));
   const bool zero_grad = (s.flags & ADAM_ZERO_GRAD) != 0;
+  // `head` leading elements bring the four binary32 arrays (which share one
+  // residue modulo 16 bytes) to a 16-byte boundary
+  float *p = p0 + head, *g = g0 + head, *m = m0 + head, *v = v0 + head;
+  void* out16 = kOut ? reinterpret_cast<char*>(out0) + int64_t(head) * O::kSize : nullptr;
+  const int64_t n = n0 - head;
   const int64_t n_quads = n >> 2;
   constexpr int64_t kTile = int64_t(BLOCK) * U;
   const int64_t n_tiles = (n_quads + kTile - 1) / kTile;
@@ -279,7 +306,9 @@ adamw_kernel(float* p, float* g, float* m, float* v, void* out16, int64_t n, Ada
     }
   }
   if (blockIdx.x == 0) {
-    const int64_t i = (n_quads << 2) + threadIdx.x;
+    int64_t i = (n_quads << 2) + threadIdx.x;
+    if (int(threadIdx.x) >= 64 && int(threadIdx.x) - 64 < head) i = int64_t(threadIdx.x) - 64 - head;  // head
+    else if (int(threadIdx.x) >= 64) i = n;
     if (i < n) {
       float fp = p[i], fm = m[i], fv = v[i];
       adam_elem(fp, g[i], fm, fv, s, scaled, gs);
