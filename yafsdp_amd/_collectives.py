@@ -75,6 +75,16 @@ def all_gather(
     if yccl_handle is not None:
         raise NotImplementedError("YCCL handles are not part of this build")
     with torch.cuda.stream(all_gather_stream):
+        if (
+            (version := param_group._copy_in_shard_version) is not None
+            and all_gather_dtype in param_group._all_gather_input_set_dtypes
+            and padded_sharded_param_data._version != version
+        ):
+            # a fused optimizer step wrote the all-gather input, and a torch op has
+            # changed the master shard since (load_state_dict, another optimizer):
+            # the 16-bit copy is stale, cast again
+            param_group._all_gather_input_set_dtypes.discard(all_gather_dtype)
+        param_group._copy_in_shard_version = None
         if all_gather_dtype not in param_group._all_gather_input_set_dtypes:
             for fsdp_param in fsdp_params:
                 fsdp_param.set_all_gather_input()

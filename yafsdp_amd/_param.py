@@ -5,6 +5,7 @@ what the buffer path touches: no DTensor wrapping, no module attribute swaps).
 
 from __future__ import annotations
 
+import weakref
 from dataclasses import dataclass, field
 
 import torch
@@ -84,6 +85,7 @@ class YaFSDPParam:
         self.sharded_numel = sharded_param_data.numel()
         self._sharded_param_data = sharded_param_data
         self.sharded_param = nn.Parameter(sharded_param_data, requires_grad=self.requires_grad)
+        self.sharded_param._yafsdp_param = weakref.ref(self)  # lets flat-shard optimizers find the owner
         self.sharded_param_grad = sharded_param_grad if self.requires_grad else None
         del self.param, self.param_data  # the group's flat shard now owns the values
         self._setattr_on_modules(self.sharded_param)
@@ -144,6 +146,7 @@ class YaFSDPParam:
                 )
             _native.flat_copy(self._sharded_param_data, new_param.detach().contiguous().view(-1))
         self.sharded_param = nn.Parameter(self._sharded_param_data, requires_grad=self.sharded_param.requires_grad)
+        self.sharded_param._yafsdp_param = weakref.ref(self)
         self._setattr_on_modules(self.sharded_param)
 
     @property

@@ -28,6 +28,8 @@ What differs
 
 from __future__ import annotations
 
+import weakref
+
 import contextlib
 import logging
 from enum import Enum, auto
@@ -177,7 +179,13 @@ class YaFSDPParamGroup:
                     shard_numels=sn,
                 )  # :379-406
                 pos += n
+        for index, fsdp_param in enumerate(self.fsdp_params):
+            fsdp_param._param_group_ref = weakref.ref(self)
+            fsdp_param._index_in_group = index
         self._table: _native.TensorTable | None = None
+        # version of the master shard at which a fused optimizer step last wrote the
+        # all-gather input (None: never); see all_gather
+        self._copy_in_shard_version: int | None = None
 
     # ------------------------------------------------------------ initialisation --
     def _init_mp_dtypes(self) -> None:

@@ -1,0 +1,377 @@
+"""Optimizer-side passes over the flat shards of ``fully_shard`` modules.
+
+The reference runs gradient clipping and the optimizer as torch foreach ops
+over the per-parameter fragments of each group's flat shard (the dispatch table
+of its tensor subclass, ya_fsdp/_tensor.py:212-312; the legacy wrapper's
+``clip_grad_norm_`` and ``zero_grad``, ya_fsdp/ya_fsdp.py:543-562, 591-601).
+The fragments of one group are consecutive ranges of one buffer, so here each
+of these is ONE kernel launch per group over the flat shard:
+
+=============================================  ==============================
+reference                                      here
+=============================================  ==============================
+``optimizer.zero_grad(set_to_none=False)``     ``zero_grad`` -> ``flat_fill``
+``clip_grad_norm_`` (norms, coefficient,        ``clip_grad_norm_`` ->
+``grad.mul_``)                                  ``flat_sumsq`` + ``clip_coef``
+                                                + ``flat_scale``
+``torch.optim.AdamW.step`` + next iteration's   ``FlatAdamW.step`` ->
+copy-in cast (ya_fsdp/_collectives.py:53-54)    ``adamw_step``
+=============================================  ==============================
+
+There is no torch fallback: parameters must be float32 CUDA tensors.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Iterable, Sequence
+
+import torch
+import torch.nn as nn
+
+from . import _native
+from ._param import YaFSDPParam
+from ._param_group import YaFSDPParamGroup
+from ._state import _get_module_fsdp_state
+
+__all__ = ["FlatAdamW", "clip_grad_norm_", "grad_clip_coef", "zero_grad", "fsdp_param_groups"]
+
+
+def fsdp_param_groups(modules: nn.Module | Iterable[nn.Module]) -> list[YaFSDPParamGroup]:
+    """The parameter groups of every ``fully_shard`` module under ``modules``, in module order."""
+    roots = [modules] if isinstance(modules, nn.Module) else list(modules)
+    groups: list[YaFSDPParamGroup] = []
+    seen: set[int] = set()
+    for root in roots:
+        for module in root.modules():
+            state = _get_module_fsdp_state(module)
+            group = state._fsdp_param_group if state is not None else None
+            if group is not None and id(group) not in seen:
+                seen.add(id(group))
+                groups.append(group)
+    return groups
+
+
+def _owner(param: torch.Tensor) -> YaFSDPParam | None:
+    ref = getattr(param, "_yafsdp_param", None)
+    return ref() if ref is not None else None
+
+
+def _merge(ranges: list[tuple[int, int]]) -> list[tuple[int, int]]:
+    """Sorted half-open ranges with the adjacent ones joined."""
+    out: list[tuple[int, int]] = []
+    for lo, hi in sorted(r for r in ranges if r[1] > r[0]):
+        if out and out[-1][1] == lo:
+            out[-1] = (out[-1][0], hi)
+        else:
+            out.append((lo, hi))
+    return out
+
+
+def _fragment_offsets(group: YaFSDPParamGroup) -> list[int]:
+    offsets = [0]
+    for n in group._sharded_param_numels[None]:
+        offsets.append(offsets[-1] + n)
+    return offsets
+
+
+def _grad_ranges(group: YaFSDPParamGroup, indices: Sequence[int] | None = None) -> list[tuple[int, int]]:
+    """Ranges of the group's flat gradient shard that hold a gradient: the
+    fragments of the parameters whose ``.grad`` is set.  A gradient tensor that
+    is not the group's own view (assigned by the user) is copied into it first.
+    When every fragment has one, the range extends over the pad lanes (zeros)."""
+    grad_shard = group._padded_sharded_param_grad[None]
+    if grad_shard is None:
+        return []
+    offsets = _fragment_offsets(group)
+    ranges = []
+    complete = indices is None or len(indices) == len(group.fsdp_params)
+    for i in range(len(group.fsdp_params)) if indices is None else indices:
+        fsdp_param = group.fsdp_params[i]
+        grad = fsdp_param.sharded_param.grad if fsdp_param.requires_grad else None
+        if grad is None:
+            if offsets[i + 1] > offsets[i]:
+                complete = False
+            continue
+        view = fsdp_param.sharded_param_grad
+        if grad.numel() and grad.data_ptr() != view.data_ptr():
+            _native.flat_copy(view, grad.detach().reshape(-1))
+            fsdp_param.sharded_param.grad = view
+        ranges.append((offsets[i], offsets[i + 1]))
+    merged = _merge(ranges)
+    if complete and merged == [(0, offsets[-1])]:
+        return [(0, grad_shard.numel())]
+    return merged
+
+
+class _ClipState:
+    """Per-device scratch of the norm computation."""
+
+    _by_device: dict[torch.device, "_ClipState"] = {}
+
+    def __init__(self, device: torch.device):
+        self.workspace = _native.sumsq_workspace(device)
+        self.sumsq = torch.zeros(1, dtype=torch.float64, device=device)
+
+    @classmethod
+    def get(cls, device: torch.device) -> "_ClipState":
+        state = cls._by_device.get(device)
+        if state is None:
+            state = cls._by_device[device] = _ClipState(device)
+        return state
+
+
+def grad_clip_coef(
+    modules: nn.Module | Iterable[nn.Module], max_norm: float, norm_type: float = 2.0
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``(total_norm, clip_coef)`` as float32 device scalars, without touching
+    the gradients: ``clip_coef = min(max_norm / (total_norm + 1e-6), 1)``
+    (ya_fsdp/ya_fsdp.py:557-559).  Pass ``clip_coef`` to ``FlatAdamW.step`` to
+    fuse the scaling into the optimizer pass.  No host synchronisation."""
+    if norm_type not in (2, 2.0):
+        raise NotImplementedError("only the 2-norm is implemented (ya_fsdp/ya_fsdp.py:544)")
+    groups = [g for g in fsdp_param_groups(modules) if g._padded_sharded_param_grad[None] is not None]
+    if not groups:
+        raise ValueError("no fully_shard parameter group with gradients under the given modules")
+    device = groups[0].device
+    scratch = _ClipState.get(device)
+    first = True
+    for group in groups:
+        grad_shard = group._padded_sharded_param_grad[None]
+        for lo, hi in _grad_ranges(group):
+            _native.flat_sumsq(grad_shard[lo:hi], scratch.sumsq, scratch.workspace, accumulate=not first)
+            first = False
+    if first:
+        _native.flat_fill(scratch.sumsq.view(torch.float32), 0.0)
+    norm_and_coef = torch.empty(2, dtype=torch.float32, device=device)
+    _native.clip_coef(scratch.sumsq, max_norm, norm_and_coef)
+    return norm_and_coef[0], norm_and_coef[1]
+
+
+def clip_grad_norm_(
+    modules: nn.Module | Iterable[nn.Module], max_norm: float, norm_type: float = 2.0
+) -> torch.Tensor:
+    """Legacy ``YaFSDP.clip_grad_norm_`` (ya_fsdp/ya_fsdp.py:543-562) over the flat
+    gradient shards of every group under ``modules``; returns the total norm.
+    One read pass per group for the norm; the scaling pass costs no memory
+    traffic when nothing is clipped (coefficient exactly 1)."""
+    total_norm, coef = grad_clip_coef(modules, max_norm, norm_type)
+    coef = coef.view(1)
+    for group in fsdp_param_groups(modules):
+        grad_shard = group._padded_sharded_param_grad[None]
+        if grad_shard is None:
+            continue
+        for lo, hi in _grad_ranges(group):
+            _native.flat_scale(grad_shard[lo:hi], coef)
+    return total_norm
+
+
+def zero_grad(modules: nn.Module | Iterable[nn.Module]) -> None:
+    """``zero_grad(set_to_none=False)``: one fill per group over its flat gradient shard."""
+    for group in fsdp_param_groups(modules):
+        grad_shard = group._padded_sharded_param_grad[None]
+        if grad_shard is not None:
+            _native.flat_fill(grad_shard, 0.0)
+
+
+class _Unit:
+    """The parameters of one optimizer param group that live in one flat shard
+    (an fsdp parameter group), or one plain tensor outside any group."""
+
+    def __init__(self, group: YaFSDPParamGroup | None, params: list[torch.Tensor], indices: list[int]):
+        self.group = group
+        self.params = params
+        self.indices = indices  # position of each parameter in group.fsdp_params
+        if group is not None:
+            shard = group._padded_sharded_param_data[None]
+            if shard.dtype != torch.float32:
+                raise TypeError(f"FlatAdamW needs float32 master shards, got {shard.dtype} in {group}")
+            self.numel = shard.numel()
+            self.device = shard.device
+        else:
+            (p,) = params
+            if p.dtype != torch.float32 or p.device.type != "cuda" or not p.is_contiguous():
+                raise TypeError("FlatAdamW handles contiguous float32 CUDA parameters only")
+            self.numel = p.numel()
+            self.device = p.device
+        self.exp_avg = torch.zeros(self.numel, dtype=torch.float32, device=self.device)
+        self.exp_avg_sq = torch.zeros(self.numel, dtype=torch.float32, device=self.device)
+        self.steps = [0] * len(params)
+
+    def fragment(self, k: int) -> tuple[int, int]:
+        if self.group is None:
+            return 0, self.numel
+        offsets = _fragment_offsets(self.group)
+        i = self.indices[k]
+        return offsets[i], offsets[i + 1]
+
+
+class FlatAdamW(torch.optim.Optimizer):
+    """``torch.optim.AdamW`` (or ``Adam`` with ``decoupled_weight_decay=False``)
+    for ``fully_shard`` modules: one fused launch per parameter group over its
+    flat float32 shard (parameters, gradients and both moments are flat buffers
+    of the shard's size), which also writes the 16-bit all-gather input of the
+    next iteration, so that the copy-in cast of the next forward
+    (ya_fsdp/_collectives.py:47-55) is already done.
+
+    ``params`` is what ``torch.optim.AdamW`` takes (``model.parameters()`` after
+    ``fully_shard``, or param-group dicts).  ``state[p]`` holds ``exp_avg`` /
+    ``exp_avg_sq`` as views of the flat moment buffers, so ``state_dict()`` has
+    the layout of torch's.  Operation order and rounding: see
+    ``yafsdp_adamw_step`` in ``include/yafsdp_hip.h``."""
+
+    def __init__(
+        self,
+        params: Iterable[torch.Tensor] | Iterable[dict[str, Any]],
+        lr: float = 1e-3,
+        betas: tuple[float, float] = (0.9, 0.999),
+        eps: float = 1e-8,
+        weight_decay: float = 1e-2,
+        *,
+        decoupled_weight_decay: bool = True,
+        fuse_copy_in: bool = True,
+    ):
+        if not 0.0 <= float(lr):
+            raise ValueError(f"Invalid learning rate: {lr}")
+        if not 0.0 <= eps:
+            raise ValueError(f"Invalid epsilon value: {eps}")
+        if not 0.0 <= betas[0] < 1.0 or not 0.0 <= betas[1] < 1.0:
+            raise ValueError(f"Invalid beta parameters: {betas}")
+        if not 0.0 <= weight_decay:
+            raise ValueError(f"Invalid weight_decay value: {weight_decay}")
+        defaults = dict(lr=lr, betas=betas, eps=eps, weight_decay=weight_decay,
+                        decoupled_weight_decay=decoupled_weight_decay)
+        super().__init__(params, defaults)
+        self.fuse_copy_in = fuse_copy_in
+        self._units: dict[int, list[_Unit]] = {}
+
+    # ------------------------------------------------------------------ planning --
+    def _units_of(self, pg_index: int, pg: dict[str, Any]) -> list[_Unit]:
+        key = pg_index
+        units = self._units.get(key)
+        if units is not None and sum(len(u.params) for u in units) == len(pg["params"]):
+            return units
+        by_group: dict[int, tuple[YaFSDPParamGroup, list[torch.Tensor], list[int]]] = {}
+        units = []
+        for p in pg["params"]:
+            owner = _owner(p)
+            group = owner._param_group_ref() if owner is not None else None
+            if group is None:
+                units.append(_Unit(None, [p], [0]))
+                continue
+            entry = by_group.setdefault(id(group), (group, [], []))
+            entry[1].append(p)
+            entry[2].append(owner._index_in_group)
+        for group, ps, idx in by_group.values():
+            order = sorted(range(len(ps)), key=lambda k: idx[k])
+            units.append(_Unit(group, [ps[k] for k in order], [idx[k] for k in order]))
+        for unit in units:
+            for k, p in enumerate(unit.params):
+                lo, hi = unit.fragment(k)
+                st = self.state[p]
+                st["step"] = torch.tensor(0.0)
+                st["exp_avg"] = unit.exp_avg[lo:hi].view(p.shape)
+                st["exp_avg_sq"] = unit.exp_avg_sq[lo:hi].view(p.shape)
+        self._units[key] = units
+        return units
+
+    # ---------------------------------------------------------------------- step --
+    @torch.no_grad()
+    def step(self, closure=None, *, grad_scale: torch.Tensor | None = None, zero_grad: bool = False):
+        """One optimizer step.  ``grad_scale`` (one-element float32 device tensor,
+        e.g. the coefficient from ``grad_clip_coef``) multiplies every gradient
+        first, as a preceding ``grad.mul_`` would, without writing it back;
+        ``zero_grad=True`` zero-fills the gradients in the same pass."""
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        if grad_scale is not None:
+            grad_scale = grad_scale.view(1)
+        for pg_index, pg in enumerate(self.param_groups):
+            beta1, beta2 = pg["betas"]
+            hyper = dict(lr=float(pg["lr"]), beta1=beta1, beta2=beta2, eps=pg["eps"],
+                         weight_decay=pg["weight_decay"], decoupled=pg["decoupled_weight_decay"])
+            for unit in self._units_of(pg_index, pg):
+                self._step_unit(unit, hyper, grad_scale, zero_grad)
+        return loss
+
+    def _step_unit(self, unit: _Unit, hyper: dict[str, Any], grad_scale, zero_grad: bool) -> None:
+        group = unit.group
+        if group is None:
+            (p,) = unit.params
+            if p.grad is None:
+                return
+            unit.steps[0] += 1
+            grad = p.grad
+            if grad.dtype != torch.float32 or not grad.is_contiguous():
+                raise TypeError("FlatAdamW needs contiguous float32 gradients")
+            _native.adamw_step(p.view(-1), grad.view(-1), unit.exp_avg, unit.exp_avg_sq, None,
+                               step=unit.steps[0], grad_scale=grad_scale, zero_grad=zero_grad, **hyper)
+            return
+        shard = group._padded_sharded_param_data[None]
+        grad_shard = group._padded_sharded_param_grad[None]
+        if grad_shard is None:
+            return
+        # launches: maximal runs of fragments that have a gradient and share a step count
+        ranges = _grad_ranges(group, unit.indices)
+        whole = ranges == [(0, shard.numel())]
+        with_grad = [k for k, p in enumerate(unit.params) if p.grad is not None]
+        if not with_grad:
+            return
+        for k in with_grad:
+            unit.steps[k] += 1
+        uniform = len({unit.steps[k] for k in with_grad}) == 1
+        # the fused copy-in needs the whole shard rewritten in this pass; otherwise the
+        # next forward casts the shard itself, as it does in the reference
+        out16 = None
+        if (self.fuse_copy_in and whole and uniform and len(unit.indices) == len(group.fsdp_params)
+                and group.param_dtype is not None and hasattr(group, "_all_gather_input")):
+            out16 = group._all_gather_input[None]
+        if whole and uniform:
+            runs = [(0, shard.numel(), unit.steps[with_grad[0]])]
+        else:
+            runs = []
+            for k in with_grad:
+                lo, hi = unit.fragment(k)
+                if hi > lo:
+                    if runs and runs[-1][1] == lo and runs[-1][2] == unit.steps[k]:
+                        runs[-1] = (runs[-1][0], hi, unit.steps[k])
+                    else:
+                        runs.append((lo, hi, unit.steps[k]))
+        for lo, hi, step in runs:
+            _native.adamw_step(
+                shard[lo:hi], grad_shard[lo:hi], unit.exp_avg[lo:hi], unit.exp_avg_sq[lo:hi],
+                None if out16 is None else out16[lo:hi], step=step, grad_scale=grad_scale, zero_grad=zero_grad,
+                **hyper,
+            )
+        if out16 is not None:
+            # the next unshard finds its all-gather input ready (ya_fsdp/_collectives.py:47-55)
+            for fsdp_param in group.fsdp_params:
+                fsdp_param.set_all_gather_input()
+            group._all_gather_input_set_dtypes.add(None)
+            group._copy_in_shard_version = shard._version
+
+    # --------------------------------------------------------------- state dicts --
+    def state_dict(self) -> dict[str, Any]:
+        for units in self._units.values():
+            for unit in units:
+                for k, p in enumerate(unit.params):
+                    self.state[p]["step"] = torch.tensor(float(unit.steps[k]))
+        return super().state_dict()
+
+    def load_state_dict(self, state_dict: dict[str, Any]) -> None:
+        super().load_state_dict(state_dict)
+        self._units.clear()
+        loaded = {p: dict(st) for p, st in self.state.items()}
+        for pg_index, pg in enumerate(self.param_groups):
+            for unit in self._units_of(pg_index, pg):  # re-creates zeroed flat moments and their views
+                for k, p in enumerate(unit.params):
+                    st = loaded.get(p)
+                    if not st:
+                        continue
+                    unit.steps[k] = int(float(st.get("step", 0)))
+                    for name in ("exp_avg", "exp_avg_sq"):
+                        if name in st and st[name].numel():
+                            _native.flat_copy(self.state[p][name].view(-1),
+                                              st[name].to(p.device, torch.float32).contiguous().view(-1))
+                    self.state[p]["step"] = torch.tensor(float(unit.steps[k]))
