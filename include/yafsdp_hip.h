@@ -160,9 +160,22 @@ size_t yafsdp_sumsq_workspace_bytes(void);
  * norms are squared and summed again.  The reference adds in binary32 in an
  * order its backend chooses; this sum is exact to binary64 rounding and its
  * order depends only on n, so it is reproducible.  `workspace` is scratch for
- * the duration of the call on `stream`. */
+ * the duration of the call on `stream` (calls sharing one workspace must not
+ * overlap).  Two launches: per-workgroup partial sums, then their sum. */
 int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* workspace,
                       size_t workspace_bytes, void* stream);
+
+/* The same split in two for several buffers (the groups of a model): each call
+ * of yafsdp_sumsq_partials writes at most `capacity` per-workgroup sums of
+ * squares of one buffer to `partials` and reports how many (*n_written, at most
+ * yafsdp_sumsq_workspace_bytes() / 8 per call); the caller lays the calls out
+ * one after the other in one array, and yafsdp_clip_coef_from_partials adds
+ * the whole array in a fixed order and derives the norm and the coefficient
+ * (and stores the sum to *sumsq if not NULL): one launch per buffer plus one. */
+int yafsdp_sumsq_partials(const void* src, int dtype, int64_t n, double* partials, int64_t capacity,
+                          int64_t* n_written, void* stream);
+int yafsdp_clip_coef_from_partials(const double* partials, int64_t n_partials, double max_norm, double* sumsq,
+                                   float* norm_and_coef, void* stream);
 
 /* norm_and_coef[0] = float(sqrt(*sumsq)); norm_and_coef[1] = min(max_norm /
  * (norm + 1e-6), 1.0), binary32 like the reference's tensors

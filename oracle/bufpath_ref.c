@@ -224,14 +224,21 @@ void ref_adamw_step(float* p, float* g, float* m, float* v, void* out16, int out
   }
 }
 
-/* sum of squares in binary64, added in index order */
+/* sum of squares in binary64 (each square is exact there), added in index order
+ * with Neumaier's compensation, so the result is the exact sum rounded to
+ * binary64 to within an ulp or two whatever the length */
 double ref_sumsq(const void* src, int dt, int64_t n) {
-  double acc = 0.0;
+  double sum = 0.0, comp = 0.0;
   for (int64_t i = 0; i < n; i++) {
     const double x = (double)load_f(src, dt, i);
-    acc += x * x;
+    const double y = x * x;
+    const double t = sum + y;
+    if (fabs(sum) >= fabs(y)) comp += (sum - t) + y;
+    else comp += (y - t) + sum;
+    sum = t;
   }
-  return acc;
+  if (!isfinite(sum)) return sum; /* overflow or NaN input: the compensation term is meaningless */
+  return sum + comp;
 }
 
 /* out[0] = float(sqrt(sumsq)); out[1] = min(max_norm / (out[0] + 1e-6), 1)

@@ -118,6 +118,37 @@ def test_clip_coef_and_scale(nat, max_norm):
         assert coef == 1.0
 
 
+def test_sumsq_partials_of_several_buffers(nat):
+    """One launch per buffer appends partial sums; one finishing launch adds them all and derives the
+    coefficient.  A small capacity makes the workgroups stride over several tiles each."""
+    g = torch.Generator().manual_seed(206)
+    bufs = [(torch.randn(n, generator=g) * std).to(dt)
+            for n, std, dt in ((2_000_003, 1e-2, torch.float32), (0, 1.0, torch.float32), (70_001, 1e-1, torch.bfloat16),
+                               (5, 1.0, torch.float16), (4_100_000, 1e-3, torch.float32))]
+    total = sum(cref.sumsq(b) for b in bufs)
+    nc = torch.zeros(2, dtype=torch.float32, device=DEV)
+    sumsq = torch.zeros(1, dtype=torch.float64, device=DEV)
+    for capacity_limit in (None, 7):
+        partials = torch.full((len(bufs) * nat.SUMSQ_MAX_PARTIALS,), float("nan"), dtype=torch.float64, device=DEV)
+        count = 0
+        for k, b in enumerate(bufs):
+            d = torch.zeros(b.numel() + 8, dtype=b.dtype, device=DEV)[k : k + b.numel()]
+            d.copy_(b)
+            if capacity_limit is None:
+                count = nat.sumsq_partials(d, partials, count)
+            else:
+                count = nat.sumsq_partials(d, partials[: count + capacity_limit], count)
+                assert count <= (k + 1) * capacity_limit
+        nat.clip_coef_from_partials(partials, count, 0.25, nc, sumsq)
+        assert abs(sumsq.item() - total) <= 1e-12 * total
+        norm, coef = cref.clip_coef(sumsq.item(), 0.25)
+        assert nc.tolist() == [norm, coef]
+    nat.clip_coef_from_partials(partials, 0, 0.25, nc, sumsq)  # nothing to add: zero norm, nothing clipped
+    assert sumsq.item() == 0.0 and nc.tolist() == [0.0, 1.0]
+    with pytest.raises(ValueError):
+        nat.sumsq_partials(torch.zeros(8, device=DEV), partials[:3], 3)
+
+
 def test_clip_coef_nan_and_zero(nat):
     nc = torch.zeros(2, dtype=torch.float32, device=DEV)
     nat.clip_coef(torch.tensor([float("nan")], dtype=torch.float64, device=DEV), 1.0, nc)

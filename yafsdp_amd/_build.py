@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libyafsdp_hip.so")
 SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip"]
-HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "launch.h", "tuning.h"]
+HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "optim_kernels.cuh", "launch.h", "tuning.h"]
 ARCH = "gfx950"
 
 # -ffp-contract=off: every multiply and add of the path rounds on its own, as

@@ -43,6 +43,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_flat_fill",
     "yafsdp_sumsq_workspace_bytes",
     "yafsdp_flat_sumsq",
+    "yafsdp_sumsq_partials",
+    "yafsdp_clip_coef_from_partials",
     "yafsdp_clip_coef",
     "yafsdp_flat_scale",
     "yafsdp_adamw_step",
@@ -89,6 +91,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_sumsq_workspace_bytes.argtypes = []
     lib.yafsdp_flat_sumsq.restype = i32
     lib.yafsdp_flat_sumsq.argtypes = [vp, i32, i64, vp, i32, vp, ctypes.c_size_t, vp]
+    lib.yafsdp_sumsq_partials.restype = i32
+    lib.yafsdp_sumsq_partials.argtypes = [vp, i32, i64, vp, i64, ctypes.POINTER(i64), vp]
+    lib.yafsdp_clip_coef_from_partials.restype = i32
+    lib.yafsdp_clip_coef_from_partials.argtypes = [vp, i64, dbl, vp, vp, vp]
     lib.yafsdp_clip_coef.restype = i32
     lib.yafsdp_clip_coef.argtypes = [vp, dbl, vp, vp]
     lib.yafsdp_flat_scale.restype = i32
@@ -353,7 +359,7 @@ def flat_fill(dst: torch.Tensor, value: float = 0.0) -> None:
 
 
 def sumsq_workspace(device: torch.device) -> torch.Tensor:
-    """Scratch buffer that ``flat_sumsq`` needs; reusable across calls on one stream."""
+    """Scratch buffer that ``flat_sumsq`` needs; reusable across calls that do not overlap."""
     return torch.empty(lib.yafsdp_sumsq_workspace_bytes(), dtype=torch.uint8, device=device)
 
 
@@ -370,6 +376,46 @@ def flat_sumsq(src: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, ac
             workspace.numel() * workspace.element_size(), _stream(src),
         ),
         "yafsdp_flat_sumsq",
+    )
+
+
+SUMSQ_MAX_PARTIALS = lib.yafsdp_sumsq_workspace_bytes() // 8
+
+
+def sumsq_partials(src: torch.Tensor, partials: torch.Tensor, offset: int) -> int:
+    """Per-workgroup sums of squares of ``src`` into ``partials[offset:]`` (float64); returns the new offset."""
+    _flat_arg(src, "src"), _flat_arg(partials, "partials")
+    if partials.dtype != torch.float64 or partials.device != src.device:
+        raise TypeError("partials must be a float64 tensor on the source's device")
+    capacity = partials.numel() - offset
+    if capacity < 1:
+        raise ValueError("partials is full")
+    written = ctypes.c_int64()
+    _check(
+        lib.yafsdp_sumsq_partials(
+            src.data_ptr(), _dt(src), src.numel(), partials.data_ptr() + 8 * offset, capacity, ctypes.byref(written),
+            _stream(src),
+        ),
+        "yafsdp_sumsq_partials",
+    )
+    return offset + written.value
+
+
+def clip_coef_from_partials(
+    partials: torch.Tensor, count: int, max_norm: float, norm_and_coef: torch.Tensor, sumsq: torch.Tensor | None = None
+) -> None:
+    """Adds ``partials[:count]`` and writes ``{norm, clip coefficient}`` (float32), optionally the sum (float64)."""
+    _flat_arg(partials, "partials"), _flat_arg(norm_and_coef, "norm_and_coef")
+    if partials.dtype != torch.float64 or norm_and_coef.dtype != torch.float32 or norm_and_coef.numel() < 2:
+        raise TypeError("partials must be float64 and norm_and_coef float32 with two elements")
+    if not 0 <= count <= partials.numel():
+        raise ValueError("count out of range")
+    _check(
+        lib.yafsdp_clip_coef_from_partials(
+            partials.data_ptr(), count, float(max_norm), None if sumsq is None else sumsq.data_ptr(),
+            norm_and_coef.data_ptr(), _stream(partials),
+        ),
+        "yafsdp_clip_coef_from_partials",
     )
 
 

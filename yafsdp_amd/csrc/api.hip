@@ -285,24 +285,47 @@ int yafsdp_flat_fill(void* dst, int dtype, int64_t n, double value, void* stream
   if (n == 0) return YAFSDP_OK;
   if (!aligned_to(dst, item_size(dtype))) return YAFSDP_ERR_MISALIGNED;
   const int head = head_elems(dst, item_size(dtype), n);
-  const int grid = opt_grid((n - head) / (16 / item_size(dtype)), kOptBlock, kFillUnroll, nullptr);
+  const int grid = opt_grid((n - head) / (16 / item_size(dtype)), kFillBlock, kFillUnroll, nullptr);
   return int(launch_fill(dtype, dst, n, head, fill_pattern(dtype, value), grid, static_cast<hipStream_t>(stream)));
 }
 
 size_t yafsdp_sumsq_workspace_bytes(void) { return size_t(kSumsqMaxPartials) * sizeof(double); }
 
+int yafsdp_sumsq_partials(const void* src, int dtype, int64_t n, double* partials, int64_t capacity,
+                          int64_t* n_written, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || partials == nullptr || n_written == nullptr || capacity < 1 || (n > 0 && src == nullptr))
+    return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(src, item_size(dtype)) || !aligned_to(partials, 8)) return YAFSDP_ERR_MISALIGNED;
+  const int head = head_elems(src, item_size(dtype), n);
+  int64_t grid = opt_grid((n - head) >> 2, kSumsqBlock, kSumsqUnroll, nullptr);
+  if (grid > kSumsqMaxPartials) grid = kSumsqMaxPartials;
+  if (grid > capacity) grid = capacity;  // fewer workgroups, each striding over more tiles
+  *n_written = grid;
+  return int(launch_sumsq_partials(dtype, src, n, head, partials, int(grid), static_cast<hipStream_t>(stream)));
+}
+
 int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* workspace,
                       size_t workspace_bytes, void* stream) {
-  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
-  if (n < 0 || sumsq == nullptr || workspace == nullptr || (n > 0 && src == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (sumsq == nullptr || workspace == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (workspace_bytes < yafsdp_sumsq_workspace_bytes()) return YAFSDP_ERR_INVALID_ARGUMENT;
-  if (!aligned_to(src, item_size(dtype)) || !aligned_to(sumsq, 8) || !aligned_to(workspace, 8))
+  if (!aligned_to(sumsq, 8)) return YAFSDP_ERR_MISALIGNED;
+  int64_t count = 0;
+  const int rc = yafsdp_sumsq_partials(src, dtype, n, static_cast<double*>(workspace), kSumsqMaxPartials, &count,
+                                       stream);
+  if (rc != YAFSDP_OK) return rc;
+  return int(launch_sumsq_finish(static_cast<double*>(workspace), count, sumsq, accumulate ? 1 : 0, 0.0f, nullptr,
+                                 static_cast<hipStream_t>(stream)));
+}
+
+int yafsdp_clip_coef_from_partials(const double* partials, int64_t n_partials, double max_norm, double* sumsq,
+                                   float* norm_and_coef, void* stream) {
+  if (n_partials < 0 || norm_and_coef == nullptr || (n_partials > 0 && partials == nullptr))
+    return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(partials, 8) || !aligned_to(norm_and_coef, 4) || (sumsq != nullptr && !aligned_to(sumsq, 8)))
     return YAFSDP_ERR_MISALIGNED;
-  const int head = head_elems(src, item_size(dtype), n);
-  int grid = opt_grid((n - head) >> 2, kOptBlock, kSumsqUnroll, nullptr);
-  if (grid > kSumsqMaxPartials) grid = kSumsqMaxPartials;
-  return int(launch_sumsq(dtype, src, n, head, static_cast<double*>(workspace), grid, sumsq, accumulate ? 1 : 0,
-                          static_cast<hipStream_t>(stream)));
+  return int(launch_sumsq_finish(partials, n_partials, sumsq, 0, static_cast<float>(max_norm), norm_and_coef,
+                                 static_cast<hipStream_t>(stream)));
 }
 
 int yafsdp_clip_coef(const double* sumsq, double max_norm, float* norm_and_coef, void* stream) {
@@ -317,7 +340,7 @@ int yafsdp_flat_scale(void* buf, int dtype, int64_t n, const float* coef, void* 
   if (n == 0) return YAFSDP_OK;
   if (!aligned_to(buf, item_size(dtype)) || !aligned_to(coef, 4)) return YAFSDP_ERR_MISALIGNED;
   const int head = head_elems(buf, item_size(dtype), n);
-  const int grid = opt_grid((n - head) >> 2, kOptBlock, kScaleUnroll, nullptr);
+  const int grid = opt_grid((n - head) >> 2, kScaleBlock, kScaleUnroll, nullptr);
   return int(launch_scale(dtype, buf, n, head, coef, grid, static_cast<hipStream_t>(stream)));
 }
 

@@ -38,9 +38,12 @@ struct AdamScalars {
 enum : int { ADAM_DECOUPLED = 1, ADAM_L2 = 2, ADAM_W_SMALL = 4, ADAM_ZERO_GRAD = 8 };
 hipError_t launch_fill(int dt, void* dst, int64_t n, int head, uint32_t pattern, int grid, hipStream_t stream);
 hipError_t launch_scale(int dt, void* buf, int64_t n, int head, const float* coef, int grid, hipStream_t stream);
-// `partials` holds `grid` doubles; out[0] (+)= their sum
-hipError_t launch_sumsq(int dt, const void* src, int64_t n, int head, double* partials, int grid, double* out,
-                        int accumulate, hipStream_t stream);
+// partials[0:grid] = per-workgroup sums of squares
+hipError_t launch_sumsq_partials(int dt, const void* src, int64_t n, int head, double* partials, int grid,
+                                 hipStream_t stream);
+// sumsq[0] (+)= sum(partials[0:count]) (if given); norm_and_coef = {norm, clip coefficient} (if given)
+hipError_t launch_sumsq_finish(const double* partials, int64_t count, double* sumsq, int accumulate, float max_norm,
+                               float* norm_and_coef, hipStream_t stream);
 hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and_coef, hipStream_t stream);
 hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n, int head,
                         const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream);

@@ -8,13 +8,13 @@ namespace yafsdp {
 hipError_t launch_fill(int dt, void* dst, int64_t n, int head, uint32_t pattern, int grid, hipStream_t stream) {
   switch (dt) {
     case DT_F32:
-      fill_kernel<F32, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, head, pattern);
+      fill_kernel<F32, kFillBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kFillBlock), 0, stream>>>(dst, n, head, pattern);
       break;
     case DT_BF16:
-      fill_kernel<BF16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, head, pattern);
+      fill_kernel<BF16, kFillBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kFillBlock), 0, stream>>>(dst, n, head, pattern);
       break;
     case DT_F16:
-      fill_kernel<F16, kOptBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(dst, n, head, pattern);
+      fill_kernel<F16, kFillBlock, kFillUnroll, kOptNtStore><<<dim3(grid), dim3(kFillBlock), 0, stream>>>(dst, n, head, pattern);
       break;
     default: return hipErrorInvalidValue;
   }
@@ -24,40 +24,43 @@ hipError_t launch_fill(int dt, void* dst, int64_t n, int head, uint32_t pattern,
 hipError_t launch_scale(int dt, void* buf, int64_t n, int head, const float* coef, int grid, hipStream_t stream) {
   switch (dt) {
     case DT_F32:
-      scale_kernel<F32, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
-          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, head, coef);
+      scale_kernel<F32, kScaleBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
+          <<<dim3(grid), dim3(kScaleBlock), 0, stream>>>(buf, n, head, coef);
       break;
     case DT_BF16:
-      scale_kernel<BF16, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
-          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, head, coef);
+      scale_kernel<BF16, kScaleBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
+          <<<dim3(grid), dim3(kScaleBlock), 0, stream>>>(buf, n, head, coef);
       break;
     case DT_F16:
-      scale_kernel<F16, kOptBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
-          <<<dim3(grid), dim3(kOptBlock), 0, stream>>>(buf, n, head, coef);
+      scale_kernel<F16, kScaleBlock, kScaleUnroll, kOptNtLoad, kOptNtStore>
+          <<<dim3(grid), dim3(kScaleBlock), 0, stream>>>(buf, n, head, coef);
       break;
     default: return hipErrorInvalidValue;
   }
   return hipGetLastError();
 }
 
-hipError_t launch_sumsq(int dt, const void* src, int64_t n, int head, double* partials, int grid, double* out,
-                        int accumulate,
-                        hipStream_t stream) {
+hipError_t launch_sumsq_partials(int dt, const void* src, int64_t n, int head, double* partials, int grid,
+                                 hipStream_t stream) {
   switch (dt) {
     case DT_F32:
-      sumsq_kernel<F32, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, head, partials);
+      sumsq_kernel<F32, kSumsqBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kSumsqBlock), 0, stream>>>(src, n, head, partials);
       break;
     case DT_BF16:
-      sumsq_kernel<BF16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, head, partials);
+      sumsq_kernel<BF16, kSumsqBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kSumsqBlock), 0, stream>>>(src, n, head, partials);
       break;
     case DT_F16:
-      sumsq_kernel<F16, kOptBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kOptBlock), 0, stream>>>(src, n, head, partials);
+      sumsq_kernel<F16, kSumsqBlock, kSumsqUnroll, kOptNtLoad><<<dim3(grid), dim3(kSumsqBlock), 0, stream>>>(src, n, head, partials);
       break;
     default: return hipErrorInvalidValue;
   }
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return e;
-  sumsq_final_kernel<kOptBlock><<<dim3(1), dim3(kOptBlock), 0, stream>>>(partials, grid, out, accumulate);
+  return hipGetLastError();
+}
+
+hipError_t launch_sumsq_finish(const double* partials, int64_t count, double* sumsq, int accumulate, float max_norm,
+                               float* norm_and_coef, hipStream_t stream) {
+  sumsq_finish_kernel<1024><<<dim3(1), dim3(1024), 0, stream>>>(partials, count, sumsq, accumulate, max_norm,
+                                                              norm_and_coef);
   return hipGetLastError();
 }
 

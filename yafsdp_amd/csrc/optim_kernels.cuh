@@ -114,7 +114,9 @@ scale_kernel(void* buf0, int64_t n0, int head, const float* coef) {
 // partials[blockIdx.x] = sum over this workgroup's tiles of x^2, accumulated in
 // binary64 (the square of a binary32 number is exact there).  The order of the
 // additions depends only on (n, gridDim, BLOCK, U): results are reproducible
-// from run to run.
+// from run to run.  (Folding the final sum into this kernel with a last-
+// workgroup ticket was measured: the agent-scope release/acquire that it needs
+// per workgroup makes the pass ten times slower.)
 template <int BLOCK>
 __device__ __forceinline__ double block_sum(double v, double* lds) {
 #pragma unroll
@@ -181,15 +183,35 @@ sumsq_kernel(const void* src0, int64_t n0, int head, double* partials) {
   if (threadIdx.x == 0) partials[blockIdx.x] = t;
 }
 
-// out[0] = (accumulate ? out[0] : 0) + sum(partials[0..count)), one workgroup
+// One workgroup adds `count` partial sums in a fixed order:
+//   sumsq[0] = (accumulate ? sumsq[0] : 0) + sum          (when sumsq is given)
+//   norm_and_coef = {float(sqrt(total)), min(max_norm / (norm + 1e-6), 1)}   (when given; NaN kept, as
+//   torch.clamp(max=1.0) keeps it)
 template <int BLOCK>
 __global__ void __launch_bounds__(BLOCK)
-sumsq_final_kernel(const double* partials, int count, double* out, int accumulate) {
+sumsq_finish_kernel(const double* partials, int64_t count, double* sumsq, int accumulate, float max_norm,
+                    float* norm_and_coef) {
   __shared__ double lds[BLOCK / 64];
-  double acc = 0.0;
-  for (int i = threadIdx.x; i < count; i += BLOCK) acc += partials[i];
-  const double t = block_sum<BLOCK>(acc, lds);
-  if (threadIdx.x == 0) out[0] = accumulate ? out[0] + t : t;
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  int64_t i = threadIdx.x;
+  for (; i + 3 * BLOCK < count; i += 4 * BLOCK) {  // four independent loads in flight per lane
+    const double a = partials[i], b = partials[i + BLOCK], c = partials[i + 2 * BLOCK], d = partials[i + 3 * BLOCK];
+    acc[0] += a; acc[1] += b; acc[2] += c; acc[3] += d;
+  }
+  for (; i < count; i += BLOCK) acc[0] += partials[i];
+  double total = block_sum<BLOCK>((acc[0] + acc[1]) + (acc[2] + acc[3]), lds);
+  if (threadIdx.x != 0) return;
+  if (sumsq != nullptr) {
+    if (accumulate) total += sumsq[0];
+    sumsq[0] = total;
+  }
+  if (norm_and_coef != nullptr) {
+    const float norm = float(__builtin_sqrt(total));
+    float c = __fdiv_rn(max_norm, __fadd_rn(norm, 1e-6f));
+    if (c > 1.0f) c = 1.0f;
+    norm_and_coef[0] = norm;
+    norm_and_coef[1] = c;
+  }
 }
 
 // norm_and_coef[0] = sqrt(sumsq) as binary32; norm_and_coef[1] = min(max_norm /
@@ -236,7 +258,7 @@ template <class O, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
 adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0, int head, AdamScalars s,
              const float* grad_scale) {
-  static_assert(BLOCK >= 128, "workgroup 0 peels the tail with wave 0 and the head with wave 1");
+  static_assert(BLOCK >= 8, "workgroup 0 peels the tail with lanes 0-3 and the head with lanes 4-7");
   constexpr bool kOut = !same_t<O, F32>::value;
   const bool scaled = grad_scale != nullptr;
   float gs = 1.0f;
@@ -306,9 +328,10 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
     }
   }
   if (blockIdx.x == 0) {
-    int64_t i = (n_quads << 2) + threadIdx.x;
-    if (int(threadIdx.x) >= 64 && int(threadIdx.x) - 64 < head) i = int64_t(threadIdx.x) - 64 - head;  // head
-    else if (int(threadIdx.x) >= 64) i = n;
+    // lanes 0-3: tail elements; lanes 4-7: head elements (negative indices from the aligned base)
+    int64_t i = n;
+    if (threadIdx.x < 4) i = (n_quads << 2) + threadIdx.x;
+    else if (int(threadIdx.x) - 4 < head) i = int64_t(threadIdx.x) - 4 - head;
     if (i < n) {
       float fp = p[i], fm = m[i], fv = v[i];
       adam_elem(fp, g[i], fm, fv, s, scaled, gs);

@@ -28,24 +28,35 @@ inline int table_block_for(long long padded_elems, int threshold_log2) {
 }
 inline long long table_tile_elems(int block) { return (long long)block * kTableUnroll * 8; }
 // optimizer-side passes: a tile is block * unroll quads (4 elements each)
+#ifndef YAFSDP_FILL_BLOCK
+#define YAFSDP_FILL_BLOCK 256
+#endif
 #ifndef YAFSDP_FILL_U
-#define YAFSDP_FILL_U 4
+#define YAFSDP_FILL_U 1
+#endif
+#ifndef YAFSDP_SCALE_BLOCK
+#define YAFSDP_SCALE_BLOCK 256
 #endif
 #ifndef YAFSDP_SCALE_U
 #define YAFSDP_SCALE_U 2
 #endif
+#ifndef YAFSDP_SUMSQ_BLOCK
+#define YAFSDP_SUMSQ_BLOCK 512
+#endif
 #ifndef YAFSDP_SUMSQ_U
 #define YAFSDP_SUMSQ_U 4
+#endif
+#ifndef YAFSDP_ADAM_BLOCK
+#define YAFSDP_ADAM_BLOCK 128
 #endif
 #ifndef YAFSDP_ADAM_U
 #define YAFSDP_ADAM_U 2
 #endif
-#ifndef YAFSDP_ADAM_BLOCK
-#define YAFSDP_ADAM_BLOCK 256
-#endif
-constexpr int kOptBlock = 256;
+constexpr int kFillBlock = YAFSDP_FILL_BLOCK;
 constexpr int kFillUnroll = YAFSDP_FILL_U;    // 16-byte stores per lane per tile
+constexpr int kScaleBlock = YAFSDP_SCALE_BLOCK;
 constexpr int kScaleUnroll = YAFSDP_SCALE_U;
+constexpr int kSumsqBlock = YAFSDP_SUMSQ_BLOCK;
 constexpr int kSumsqUnroll = YAFSDP_SUMSQ_U;
 constexpr int kAdamBlock = YAFSDP_ADAM_BLOCK;
 constexpr int kAdamUnroll = YAFSDP_ADAM_U;

@@ -104,13 +104,14 @@ def _grad_ranges(group: YaFSDPParamGroup, indices: Sequence[int] | None = None) 
 
 
 class _ClipState:
-    """Per-device scratch of the norm computation."""
+    """Per-device scratch of the norm computation: room for the partial sums of
+    many buffers (grown on demand)."""
 
     _by_device: dict[torch.device, "_ClipState"] = {}
 
     def __init__(self, device: torch.device):
-        self.workspace = _native.sumsq_workspace(device)
-        self.sumsq = torch.zeros(1, dtype=torch.float64, device=device)
+        self.device = device
+        self.partials = torch.empty(16 * _native.SUMSQ_MAX_PARTIALS, dtype=torch.float64, device=device)
 
     @classmethod
     def get(cls, device: torch.device) -> "_ClipState":
@@ -119,6 +120,12 @@ class _ClipState:
             state = cls._by_device[device] = _ClipState(device)
         return state
 
+    def reserve(self, n_buffers: int) -> torch.Tensor:
+        need = n_buffers * _native.SUMSQ_MAX_PARTIALS
+        if self.partials.numel() < need:
+            self.partials = torch.empty(need, dtype=torch.float64, device=self.device)
+        return self.partials
+
 
 def grad_clip_coef(
     modules: nn.Module | Iterable[nn.Module], max_norm: float, norm_type: float = 2.0
@@ -126,24 +133,22 @@ def grad_clip_coef(
     """``(total_norm, clip_coef)`` as float32 device scalars, without touching
     the gradients: ``clip_coef = min(max_norm / (total_norm + 1e-6), 1)``
     (ya_fsdp/ya_fsdp.py:557-559).  Pass ``clip_coef`` to ``FlatAdamW.step`` to
-    fuse the scaling into the optimizer pass.  No host synchronisation."""
+    fuse the scaling into the optimizer pass.  One launch per gradient range
+    plus one; no host synchronisation.  Calls on one device share a scratch
+    buffer and must be ordered on one stream."""
     if norm_type not in (2, 2.0):
         raise NotImplementedError("only the 2-norm is implemented (ya_fsdp/ya_fsdp.py:544)")
     groups = [g for g in fsdp_param_groups(modules) if g._padded_sharded_param_grad[None] is not None]
     if not groups:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
     device = groups[0].device
-    scratch = _ClipState.get(device)
-    first = True
-    for group in groups:
-        grad_shard = group._padded_sharded_param_grad[None]
-        for lo, hi in _grad_ranges(group):
-            _native.flat_sumsq(grad_shard[lo:hi], scratch.sumsq, scratch.workspace, accumulate=not first)
-            first = False
-    if first:
-        _native.flat_fill(scratch.sumsq.view(torch.float32), 0.0)
+    work = [(g._padded_sharded_param_grad[None], lo, hi) for g in groups for lo, hi in _grad_ranges(g)]
+    partials = _ClipState.get(device).reserve(max(len(work), 1))
+    count = 0
+    for grad_shard, lo, hi in work:
+        count = _native.sumsq_partials(grad_shard[lo:hi], partials, count)
     norm_and_coef = torch.empty(2, dtype=torch.float32, device=device)
-    _native.clip_coef(scratch.sumsq, max_norm, norm_and_coef)
+    _native.clip_coef_from_partials(partials, count, max_norm, norm_and_coef)
     return norm_and_coef[0], norm_and_coef[1]
 
 
