@@ -69,21 +69,28 @@ hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and
   return hipGetLastError();
 }
 
+namespace {
+template <class O, bool ZERO_GRAD>
+hipError_t adamw_go(float* p, float* g, float* m, float* v, void* out16, int64_t n, int head, const AdamScalars& s,
+                    const float* grad_scale, int grid, hipStream_t stream) {
+  adamw_kernel<O, ZERO_GRAD, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
+      <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, head, s, grad_scale);
+  return hipGetLastError();
+}
+template <class O>
+hipError_t adamw_by_zero(float* p, float* g, float* m, float* v, void* out16, int64_t n, int head,
+                         const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream) {
+  if (s.flags & ADAM_ZERO_GRAD) return adamw_go<O, true>(p, g, m, v, out16, n, head, s, grad_scale, grid, stream);
+  return adamw_go<O, false>(p, g, m, v, out16, n, head, s, grad_scale, grid, stream);
+}
+}  // namespace
+
 hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n, int head,
                         const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream) {
-  if (out16 == nullptr) {
-    adamw_kernel<F32, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
-        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, nullptr, n, head, s, grad_scale);
-  } else if (out_dt == DT_BF16) {
-    adamw_kernel<BF16, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
-        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, head, s, grad_scale);
-  } else if (out_dt == DT_F16) {
-    adamw_kernel<F16, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>
-        <<<dim3(grid), dim3(kAdamBlock), 0, stream>>>(p, g, m, v, out16, n, head, s, grad_scale);
-  } else {
-    return hipErrorInvalidValue;
-  }
-  return hipGetLastError();
+  if (out16 == nullptr) return adamw_by_zero<F32>(p, g, m, v, nullptr, n, head, s, grad_scale, grid, stream);
+  if (out_dt == DT_BF16) return adamw_by_zero<BF16>(p, g, m, v, out16, n, head, s, grad_scale, grid, stream);
+  if (out_dt == DT_F16) return adamw_by_zero<F16>(p, g, m, v, out16, n, head, s, grad_scale, grid, stream);
+  return hipErrorInvalidValue;
 }
 
 }  // namespace yafsdp

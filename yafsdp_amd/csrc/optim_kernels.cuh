@@ -253,8 +253,8 @@ __device__ __forceinline__ void adam_elem(float& p, float g, float& m, float& v,
   p = __fadd_rn(p, __fdiv_rn(__fmul_rn(s.neg_step, m), den));
 }
 
-// O is the 16-bit output dtype, or F32 for "no 16-bit output".
-template <class O, int BLOCK, int U, bool NTL, bool NTS>
+// O is the 16-bit output dtype, or F32 for "no 16-bit output"; ZERO_GRAD also zero-fills the gradient.
+template <class O, bool ZERO_GRAD, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
 adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0, int head, AdamScalars s,
              const float* grad_scale) {
@@ -264,7 +264,6 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
   float gs = 1.0f;
   if (scaled)
     gs = *reinterpret_cast<const __attribute__((address_space(4))) float*>(reinterpret_cast<uintptr_t>(grad_scale));
-  const bool zero_grad = (s.flags & ADAM_ZERO_GRAD) != 0;
   // `head` leading elements bring the four binary32 arrays (which share one
   // residue modulo 16 bytes) to a 16-byte boundary
   float *p = p0 + head, *g = g0 + head, *m = m0 + head, *v = v0 + head;
@@ -299,7 +298,7 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
         store_quad<F32, NTS>(m + e, pack_quad<F32>(fm));
         store_quad<F32, NTS>(v + e, pack_quad<F32>(fv));
         if constexpr (kOut) store_quad<O, NTS>(reinterpret_cast<char*>(out16) + e * O::kSize, pack_quad<O>(fp));
-        if (zero_grad) {
+        if constexpr (ZERO_GRAD) {
           Quad<F32> z;
           z.v = u32x4{0u, 0u, 0u, 0u};
           store_quad<F32, NTS>(g + e, z);
@@ -319,7 +318,7 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
         store_quad<F32, NTS>(m + e, pack_quad<F32>(fm));
         store_quad<F32, NTS>(v + e, pack_quad<F32>(fv));
         if constexpr (kOut) store_quad<O, NTS>(reinterpret_cast<char*>(out16) + e * O::kSize, pack_quad<O>(fp));
-        if (zero_grad) {
+        if constexpr (ZERO_GRAD) {
           Quad<F32> z;
           z.v = u32x4{0u, 0u, 0u, 0u};
           store_quad<F32, NTS>(g + e, z);
@@ -339,7 +338,7 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
       m[i] = fm;
       v[i] = fv;
       if constexpr (kOut) reinterpret_cast<typename O::storage*>(out16)[i] = from_f32<O>(fp);
-      if (zero_grad) g[i] = 0.0f;
+      if constexpr (ZERO_GRAD) g[i] = 0.0f;
     }
   }
 }
