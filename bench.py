@@ -64,6 +64,16 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def _event_pair():
+    """Two timing events whose HIP handles exist (torch creates them on the first record)."""
+    import torch
+
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    b.record()
+    return a, b
+
+
 def numel_of(shape):
     n = 1
     for d in shape:
@@ -345,16 +355,14 @@ def run_optim(args) -> int:
         step()
     torch.cuda.synchronize()
     sampled = [k for k in range(args.steps) if k % 4 == 0]
-    ev = {k: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for k in sampled}
+    ev = {k: _event_pair() for k in sampled}
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
         ops[0][1]()
         if k in ev:
-            ev[k][0].record()
-            ops[1][1]()
-            ev[k][1].record()
-        else:
-            ops[1][1]()
+            _native.time_next_launch(*ev[k])  # events attached to the AdamW dispatch itself
+        ops[1][1]()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
@@ -368,15 +376,19 @@ def run_optim(args) -> int:
     for name, fn, nbytes in ops + extra:
         times = []
         for _ in range(20):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a, b = _event_pair()
             for n2, f, _ in ops + extra:  # evict: the other ops stream the other buffers through the caches
                 if n2 != name:
                     f()
             refresh_grad()
-            a.record()
-            fn()
-            b.record()
-            b.synchronize()
+            if name == "grad_sumsq":  # two launches: bracket the pair with recorded events
+                a.record()
+                fn()
+                b.record()
+            else:
+                _native.time_next_launch(a, b)
+                fn()
+            torch.cuda.synchronize()
             times.append(a.elapsed_time(b) * 1e3)
         med = statistics.median(times)
         kernels[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
@@ -577,21 +589,18 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     dom_index = 2  # reduce copy-in: most bytes, fused arithmetic
-    # the dominant kernel is bracketed by events on every 4th step of the timed region (an event record costs
-    # about a microsecond of stream time, so not every launch carries a pair)
+    # on every 4th step of the timed region the dominant kernel's dispatch carries a pair of HIP events (attached to
+    # the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
     sampled = [k for k in range(args.steps) if k % 4 == 0]
-    ev = {k: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for k in sampled}
+    ev = {k: _event_pair() for k in sampled}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
         ops[0][1]()
         ops[1][1]()
         if k in ev:
-            ev[k][0].record()
-            ops[2][1]()
-            ev[k][1].record()
-        else:
-            ops[2][1]()
+            _native.time_next_launch(*ev[k])
+        ops[2][1]()
         ops[3][1]()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
@@ -602,29 +611,27 @@ def main() -> int:
     dom_bytes = ops[dom_index][2]
     achieved = dom_bytes / dom_avg_us / 1e3
 
-    # ---- per-kernel table (outside the timed region): each op on its own between events
+    # ---- per-kernel table (outside the timed region): each op's dispatch timed on its own
     kernels = {}
     for name, fn, nbytes in ops:
         times = []
         for _ in range(20):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a, b = _event_pair()
             step_others = [f for n2, f, _ in ops if n2 != name]
             for f in step_others:  # evict: the other ops stream 1-2 GB through the caches
                 f()
-            a.record()
+            _native.time_next_launch(a, b)
             fn()
-            b.record()
-            b.synchronize()
+            torch.cuda.synchronize()
             times.append(a.elapsed_time(b) * 1e3)
         med = statistics.median(times)
         warm = []  # same op back to back: whatever fits stays in the 256 MB memory-side cache
         for _ in range(20):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a, b = _event_pair()
             fn()
-            a.record()
+            _native.time_next_launch(a, b)
             fn()
-            b.record()
-            b.synchronize()
+            torch.cuda.synchronize()
             warm.append(a.elapsed_time(b) * 1e3)
         kernels[name] = {
             "bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),

@@ -206,6 +206,15 @@ int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_
                       int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,
                       int64_t step, const float* grad_scale, int flags, void* stream);
 
+/* Measurement hook: arms a pair of HIP events (hipEvent_t, created with timing
+ * enabled) for the calling thread.  The next kernel this thread launches
+ * through the library is dispatched with the pair attached to that dispatch
+ * (hipExtLaunchKernel), so hipEventElapsedTime(start, stop) is the kernel's own
+ * duration without the launch gap an event record around the call would add.
+ * The pair is consumed by that one launch (the first one, for entry points that
+ * launch several kernels); NULL, NULL disarms. */
+int yafsdp_time_next_launch(void* start_event, void* stop_event);
+
 /* Launch-shape knobs (process-wide, for measurement): */
 typedef enum yafsdp_option {
   YAFSDP_OPT_FLAT_BLOCKS_PER_CU = 0,  /* workgroups per compute unit of the flat kernels' grid */

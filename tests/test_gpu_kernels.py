@@ -262,3 +262,35 @@ def test_errors_are_loud(nat):
         table.gather_in([a[:8], a[8:]], buf[1:17])
     assert "invalid argument" in nat.error_string(-1)
     assert nat.lib.yafsdp_flat_copy(a.data_ptr(), 7, a.data_ptr(), 0, 4, None) == -2
+
+
+def test_time_next_launch_brackets_exactly_one_dispatch(nat):
+    """Events armed with time_next_launch ride on the next dispatch only: the measured time is that kernel's
+    own duration (shorter than a record / launch / record bracket) and results are unchanged."""
+    n = 1 << 26
+    src = torch.randn(n, device=DEV)
+    dst = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(3):
+        nat.flat_copy(dst, src)
+    nat.time_next_launch(a, b)
+    nat.flat_copy(dst, src)
+    small = torch.empty(8, dtype=torch.bfloat16, device=DEV)
+    nat.flat_copy(small, src[:8])  # not timed: the pair was consumed
+    torch.cuda.synchronize()
+    attached = a.elapsed_time(b) * 1e3
+    c, d = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c.record()
+    nat.flat_copy(dst, src)
+    d.record()
+    torch.cuda.synchronize()
+    bracket = c.elapsed_time(d) * 1e3
+    _say("attached", attached, "bracket", bracket)
+    assert 20.0 < attached < 500.0  # 403 MB: about 65 us at 6 TB/s
+    assert attached <= bracket + 2.0
+    assert_bits_equal(dst, src.bfloat16(), "timed launch result")
+    nat.time_next_launch(a, b)
+    nat.time_next_launch(None, None)  # disarm
+    nat.flat_copy(dst, src)
+    torch.cuda.synchronize()
+    assert abs(a.elapsed_time(b) * 1e3 - attached) < 1e-6  # untouched by the disarmed launch

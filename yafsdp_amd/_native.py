@@ -48,6 +48,7 @@ EXPORTED_SYMBOLS = (
     "yafsdp_clip_coef",
     "yafsdp_flat_scale",
     "yafsdp_adamw_step",
+    "yafsdp_time_next_launch",
     "yafsdp_set_option",
     "yafsdp_get_option",
 )
@@ -101,6 +102,8 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_flat_scale.argtypes = [vp, i32, i64, vp, vp]
     lib.yafsdp_adamw_step.restype = i32
     lib.yafsdp_adamw_step.argtypes = [vp, vp, vp, vp, vp, i32, i64, dbl, dbl, dbl, dbl, dbl, i64, vp, i32, vp]
+    lib.yafsdp_time_next_launch.restype = i32
+    lib.yafsdp_time_next_launch.argtypes = [vp, vp]
     lib.yafsdp_set_option.restype = i32
     lib.yafsdp_set_option.argtypes = [i32, i32]
     lib.yafsdp_get_option.restype = i32
@@ -484,6 +487,19 @@ def adamw_step(
         ),
         "yafsdp_adamw_step",
     )
+
+
+def time_next_launch(start: torch.cuda.Event | None, stop: torch.cuda.Event | None) -> None:
+    """Measurement hook: the next kernel launched through the library from this thread carries ``start`` /
+    ``stop`` on its own dispatch (kernel begin and end, no launch gap); ``start.elapsed_time(stop)`` after a
+    synchronisation is the kernel's duration.  Both events need ``enable_timing=True``."""
+    if start is None or stop is None:
+        _check(lib.yafsdp_time_next_launch(None, None), "yafsdp_time_next_launch")
+        return
+    for ev in (start, stop):
+        if not ev.cuda_event:  # torch creates the HIP event lazily, on its first record
+            ev.record()
+    _check(lib.yafsdp_time_next_launch(start.cuda_event, stop.cuda_event), "yafsdp_time_next_launch")
 
 
 def set_option(option: int, value: int) -> None:

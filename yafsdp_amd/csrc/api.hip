@@ -14,6 +14,8 @@
 
 using namespace yafsdp;
 
+thread_local yafsdp::TimedLaunch yafsdp::tl_timed_launch;
+
 namespace {
 
 std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
@@ -219,6 +221,13 @@ const char* yafsdp_error_string(int code) {
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
   return "yafsdp: unknown error code";
+}
+
+int yafsdp_time_next_launch(void* start_event, void* stop_event) {
+  if ((start_event == nullptr) != (stop_event == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  tl_timed_launch.start = static_cast<hipEvent_t>(start_event);
+  tl_timed_launch.stop = static_cast<hipEvent_t>(stop_event);
+  return YAFSDP_OK;
 }
 
 int yafsdp_set_option(int option, int value) {

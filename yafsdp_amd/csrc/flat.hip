@@ -7,9 +7,8 @@ namespace {
 
 template <class S, class D, int SCALE, bool ACC>
 hipError_t go(void* dst, const void* src, int64_t n, int head, float k, int grid, hipStream_t stream) {
-  flat_kernel<S, D, SCALE, ACC, kFlatBlock, kFlatUnroll, kFlatNtLoad, kFlatNtStore>
-      <<<dim3(grid), dim3(kFlatBlock), 0, stream>>>(dst, src, n, head, k);
-  return hipGetLastError();
+  return launch_kernel(flat_kernel<S, D, SCALE, ACC, kFlatBlock, kFlatUnroll, kFlatNtLoad, kFlatNtStore>, grid,
+                       kFlatBlock, stream, dst, src, n, head, k);
 }
 
 template <class S, class D>

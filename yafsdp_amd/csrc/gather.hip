@@ -8,9 +8,8 @@ namespace {
 template <class META, class S, class D, int SCALE, int BLOCK>
 hipError_t go(const META& meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero, int grid,
               hipStream_t stream) {
-  gather_in_kernel<META, S, D, SCALE, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>
-      <<<dim3(grid), dim3(BLOCK), 0, stream>>>(meta, flat, padded, n_tiles, k, pad_zero);
-  return hipGetLastError();
+  return launch_kernel(gather_in_kernel<META, S, D, SCALE, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>, grid,
+                       BLOCK, stream, meta, flat, padded, n_tiles, k, pad_zero);
 }
 
 template <class META, class S, class D, int SCALE>

@@ -2,11 +2,34 @@
 // units that instantiate the kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "table_kernels.cuh"
 
 namespace yafsdp {
+
+// Measurement hook: when a start/stop event pair has been armed on this thread
+// (yafsdp_time_next_launch), the next kernel launched through the library is
+// dispatched with the events attached to that dispatch, so that they carry the
+// kernel's own begin and end timestamps (no launch gap in between).
+struct TimedLaunch {
+  hipEvent_t start = nullptr, stop = nullptr;
+};
+extern thread_local TimedLaunch tl_timed_launch;
+
+template <class... Params, class... Args>
+inline hipError_t launch_kernel(void (*kernel)(Params...), int grid, int block, hipStream_t stream, Args... args) {
+  TimedLaunch& t = tl_timed_launch;
+  if (t.start != nullptr) {
+    const hipEvent_t a = t.start, b = t.stop;
+    t.start = t.stop = nullptr;
+    hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, a, b, 0, static_cast<Params>(args)...);
+  } else {
+    kernel<<<dim3(grid), dim3(block), 0, stream>>>(static_cast<Params>(args)...);
+  }
+  return hipGetLastError();
+}
 
 // dst[i] = post_elem(src[i], dst[i]); scale is SCALE_NONE / SCALE_MUL / SCALE_DIV
 hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,

@@ -7,9 +7,8 @@ namespace {
 
 template <class META, class S, class D, int BLOCK>
 hipError_t go(const META& meta, const void* flat, int64_t total, int n_tiles, int grid, hipStream_t stream) {
-  scatter_out_kernel<META, S, D, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>
-      <<<dim3(grid), dim3(BLOCK), 0, stream>>>(meta, flat, total, n_tiles);
-  return hipGetLastError();
+  return launch_kernel(scatter_out_kernel<META, S, D, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>, grid, BLOCK,
+                       stream, meta, flat, total, n_tiles);
 }
 
 template <class META, class S, class D>
