@@ -202,3 +202,55 @@ def adam_step_torch_ops(
     bias_correction2_sqrt = bias_correction2**0.5
     denom = (exp_avg_sq.sqrt() / bias_correction2_sqrt).add_(eps)
     param.addcdiv_(exp_avg, denom, value=-step_size)
+
+
+# ---------------------------------------------------------------------------
+# legacy ``YaFSDP`` class (ya_fsdp/ya_fsdp.py, ya_fsdp/meta_param.py): the same
+# flat-buffer ops under other names
+# ---------------------------------------------------------------------------
+def legacy_flatten_and_shard(params: Sequence[torch.Tensor], world_size: int, rank: int, yccl_padding: bool):
+    """ya_fsdp/ya_fsdp.py:836-866: pad the total to a multiple of the world size (and the chunk to 8 elements
+    with YCCL padding), concatenate the parameters and zeros, keep this rank's chunk.  Returns
+    ``(padded_numel, shard)``."""
+    total = sum(p.numel() for p in params)
+    padded = total
+    if padded % world_size != 0:
+        padded += world_size - padded % world_size
+    if yccl_padding:
+        chunk = padded // world_size
+        if chunk % 8 != 0:
+            chunk += 8 - chunk % 8
+            padded = chunk * world_size
+    flat = torch.cat([p.reshape(-1) for p in params] + [torch.zeros(padded - total, dtype=params[0].dtype)])
+    shard_size = padded // world_size
+    return padded, flat.narrow(0, shard_size * rank, shard_size).clone()
+
+
+def legacy_bit16_copy(bit16: torch.Tensor, master: torch.Tensor) -> None:
+    """ya_fsdp/ya_fsdp.py:519-520: ``_main_parameter_bit16.data.copy_(_main_parameter)``."""
+    bit16.copy_(master)
+
+
+def legacy_grad_buffer_upcast(fp32_buffer: torch.Tensor, grad_buffer: torch.Tensor) -> None:
+    """ya_fsdp/ya_fsdp.py:945-954: ``reusable_fp32_grad_buffer.get().copy_(grad_reusable_buffer.get())``."""
+    fp32_buffer.copy_(grad_buffer)
+
+
+def legacy_accumulate_shard(fp32_grad_shard: torch.Tensor, target: torch.Tensor) -> None:
+    """ya_fsdp/ya_fsdp.py:991-992: ``self.fp32_grad_shard.add_(target_tensor)``."""
+    fp32_grad_shard.add_(target)
+
+
+def legacy_final_divide(grad: torch.Tensor, world_size: int, accumulation_steps: int) -> None:
+    """ya_fsdp/ya_fsdp.py:499-501: ``grad.data.div_(world_size * gradient_accumulation_steps)``."""
+    grad.div_(world_size * accumulation_steps)
+
+
+def legacy_narrow_backward(grad_buffer: torch.Tensor, offset: int, grad_output: torch.Tensor, accumulate: bool) -> None:
+    """ya_fsdp/meta_param.py:16-27: the per-parameter gradient lands in its range of the flat gradient buffer,
+    ``copy_`` on the first micro-batch and ``add_`` afterwards."""
+    view = grad_buffer.narrow(0, offset, grad_output.numel())
+    if not accumulate:
+        view.copy_(grad_output.reshape(-1))
+    else:
+        view.add_(grad_output.reshape(-1))

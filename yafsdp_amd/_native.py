@@ -358,7 +358,8 @@ ADAM_DECOUPLED_DECAY, ADAM_ZERO_GRAD = 1, 2
 def flat_fill(dst: torch.Tensor, value: float = 0.0) -> None:
     """``dst.fill_(value)`` (``zero_()`` by default) on a flat buffer."""
     _flat_arg(dst, "dst")
-    _check(lib.yafsdp_flat_fill(dst.data_ptr(), _dt(dst), dst.numel(), float(value), _stream(dst)), "yafsdp_flat_fill")
+    with torch.cuda.device(dst.device):
+        _check(lib.yafsdp_flat_fill(dst.data_ptr(), _dt(dst), dst.numel(), float(value), _stream(dst)), "yafsdp_flat_fill")
 
 
 def sumsq_workspace(device: torch.device) -> torch.Tensor:
@@ -373,13 +374,14 @@ def flat_sumsq(src: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, ac
         raise TypeError("out must be a float64 tensor with at least one element")
     if out.device != src.device or workspace.device != src.device:
         raise RuntimeError("src, out and workspace must live on one device")
-    _check(
-        lib.yafsdp_flat_sumsq(
-            src.data_ptr(), _dt(src), src.numel(), out.data_ptr(), int(accumulate), workspace.data_ptr(),
-            workspace.numel() * workspace.element_size(), _stream(src),
-        ),
-        "yafsdp_flat_sumsq",
-    )
+    with torch.cuda.device(src.device):
+        _check(
+            lib.yafsdp_flat_sumsq(
+                src.data_ptr(), _dt(src), src.numel(), out.data_ptr(), int(accumulate), workspace.data_ptr(),
+                workspace.numel() * workspace.element_size(), _stream(src),
+            ),
+            "yafsdp_flat_sumsq",
+        )
 
 
 SUMSQ_MAX_PARTIALS = lib.yafsdp_sumsq_workspace_bytes() // 8
@@ -394,13 +396,14 @@ def sumsq_partials(src: torch.Tensor, partials: torch.Tensor, offset: int) -> in
     if capacity < 1:
         raise ValueError("partials is full")
     written = ctypes.c_int64()
-    _check(
-        lib.yafsdp_sumsq_partials(
-            src.data_ptr(), _dt(src), src.numel(), partials.data_ptr() + 8 * offset, capacity, ctypes.byref(written),
-            _stream(src),
-        ),
-        "yafsdp_sumsq_partials",
-    )
+    with torch.cuda.device(src.device):
+        _check(
+            lib.yafsdp_sumsq_partials(
+                src.data_ptr(), _dt(src), src.numel(), partials.data_ptr() + 8 * offset, capacity, ctypes.byref(written),
+                _stream(src),
+            ),
+            "yafsdp_sumsq_partials",
+        )
     return offset + written.value
 
 
@@ -413,13 +416,14 @@ def clip_coef_from_partials(
         raise TypeError("partials must be float64 and norm_and_coef float32 with two elements")
     if not 0 <= count <= partials.numel():
         raise ValueError("count out of range")
-    _check(
-        lib.yafsdp_clip_coef_from_partials(
-            partials.data_ptr(), count, float(max_norm), None if sumsq is None else sumsq.data_ptr(),
-            norm_and_coef.data_ptr(), _stream(partials),
-        ),
-        "yafsdp_clip_coef_from_partials",
-    )
+    with torch.cuda.device(partials.device):
+        _check(
+            lib.yafsdp_clip_coef_from_partials(
+                partials.data_ptr(), count, float(max_norm), None if sumsq is None else sumsq.data_ptr(),
+                norm_and_coef.data_ptr(), _stream(partials),
+            ),
+            "yafsdp_clip_coef_from_partials",
+        )
 
 
 def clip_coef(sumsq: torch.Tensor, max_norm: float, norm_and_coef: torch.Tensor) -> None:
@@ -427,10 +431,11 @@ def clip_coef(sumsq: torch.Tensor, max_norm: float, norm_and_coef: torch.Tensor)
     _flat_arg(sumsq, "sumsq"), _flat_arg(norm_and_coef, "norm_and_coef")
     if sumsq.dtype != torch.float64 or norm_and_coef.dtype != torch.float32 or norm_and_coef.numel() < 2:
         raise TypeError("sumsq must be float64 and norm_and_coef float32 with two elements")
-    _check(
-        lib.yafsdp_clip_coef(sumsq.data_ptr(), float(max_norm), norm_and_coef.data_ptr(), _stream(sumsq)),
-        "yafsdp_clip_coef",
-    )
+    with torch.cuda.device(sumsq.device):
+        _check(
+            lib.yafsdp_clip_coef(sumsq.data_ptr(), float(max_norm), norm_and_coef.data_ptr(), _stream(sumsq)),
+            "yafsdp_clip_coef",
+        )
 
 
 def flat_scale(buf: torch.Tensor, coef: torch.Tensor) -> None:
@@ -438,7 +443,8 @@ def flat_scale(buf: torch.Tensor, coef: torch.Tensor) -> None:
     _flat_arg(buf, "buf"), _flat_arg(coef, "coef")
     if coef.dtype != torch.float32 or coef.numel() != 1 or coef.device != buf.device:
         raise TypeError("coef must be a one-element float32 tensor on the buffer's device")
-    _check(lib.yafsdp_flat_scale(buf.data_ptr(), _dt(buf), buf.numel(), coef.data_ptr(), _stream(buf)), "yafsdp_flat_scale")
+    with torch.cuda.device(buf.device):
+        _check(lib.yafsdp_flat_scale(buf.data_ptr(), _dt(buf), buf.numel(), coef.data_ptr(), _stream(buf)), "yafsdp_flat_scale")
 
 
 def adamw_step(
@@ -479,14 +485,15 @@ def adamw_step(
             raise TypeError("grad_scale must be a one-element float32 tensor on the shard's device")
         gs_ptr = grad_scale.data_ptr()
     flags = (ADAM_DECOUPLED_DECAY if decoupled else 0) | (ADAM_ZERO_GRAD if zero_grad else 0)
-    _check(
-        lib.yafsdp_adamw_step(
-            param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), out_ptr, out_dt, n,
-            float(lr), float(beta1), float(beta2), float(eps), float(weight_decay), int(step), gs_ptr, flags,
-            _stream(param),
-        ),
-        "yafsdp_adamw_step",
-    )
+    with torch.cuda.device(param.device):
+        _check(
+            lib.yafsdp_adamw_step(
+                param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), out_ptr, out_dt, n,
+                float(lr), float(beta1), float(beta2), float(eps), float(weight_decay), int(step), gs_ptr, flags,
+                _stream(param),
+            ),
+            "yafsdp_adamw_step",
+        )
 
 
 def time_next_launch(start: torch.cuda.Event | None, stop: torch.cuda.Event | None) -> None:
