@@ -1,0 +1,90 @@
+"""Sharded <-> full parameters on one GPU: the logical ranks' flat shards are
+reassembled into full parameters by the copy-out kernel, and full parameters
+are loaded back fragment by fragment; both directions are byte identities."""
+
+import copy
+
+import pytest
+import torch
+
+from helpers import assert_bits_equal
+from test_gpu_fully_shard import DEV, MP, _make
+
+pytestmark = pytest.mark.gpu
+
+
+def _rank_groups(model0, w, alignment=8):
+    from yafsdp_amd import fully_shard
+
+    blocks = []
+    for r in range(w):
+        blk = copy.deepcopy(model0.blocks[0])
+        fully_shard(blk, mesh=(w, r), mp_policy=MP, shard_alignment=alignment)
+        blocks.append(blk)
+    return blocks, [b._get_fsdp_state()._fsdp_param_group for b in blocks]
+
+
+@pytest.mark.parametrize("w,alignment", [(1, 8), (3, 8), (5, 1)])
+def test_full_tensors_round_trip(w, alignment):
+    from yafsdp_amd.checkpoint import full_tensors, group_meta_info, load_full_tensors, sharded_state_dict
+
+    model0 = _make(21)
+    want = {n: p.detach().clone() for n, p in model0.blocks[0].named_parameters()}
+    blocks, groups = _rank_groups(model0, w, alignment)
+    full = full_tensors(groups)
+    assert set(full) == set(want)
+    for k in want:
+        assert_bits_equal(full[k], want[k], f"full tensor {k}")
+    # chunks of the ranks' sharded state dicts tile each flattened parameter
+    for k in want:
+        pieces = []
+        for g in groups:
+            local, meta = sharded_state_dict(g)[k]
+            assert local.numel() == meta.sizes[0] and meta.size == (want[k].numel(),)
+            if meta.sizes[0]:
+                assert_bits_equal(local, want[k].view(-1)[meta.offsets[0] : meta.offsets[0] + meta.sizes[0]], k)
+                pieces.append(local)
+        assert_bits_equal(torch.cat(pieces), want[k].view(-1), f"chunks of {k}")
+    info = group_meta_info(groups[w - 1])
+    assert info["numels"] == [p.numel() for p in want.values()] and info["fqns"] == list(want)
+    assert info["shard_boundaries"][1] == info["padded_numel"]
+    # load new values into every rank and read them back
+    gen = torch.Generator(device=DEV).manual_seed(22)
+    new = {k: torch.randn(v.shape, device=DEV, generator=gen) for k, v in want.items()}
+    load_full_tensors(groups, new)
+    out = {k: torch.empty_like(v) for k, v in new.items()}
+    again = full_tensors(groups, out=out)
+    for k in new:
+        assert again[k] is out[k]
+        assert_bits_equal(again[k], new[k], f"reloaded {k}")
+    # pad lanes of the last rank's shard stay zero
+    lay = groups[0].layout
+    pad = lay.pad_numel(w - 1)
+    if pad:
+        assert float(groups[w - 1]._padded_sharded_param_data[None][-pad:].abs().max()) == 0.0
+
+
+def test_load_casts_to_the_master_dtype_and_resets_the_copy_in_flag():
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.checkpoint import fsdp_groups_of, load_full_tensors
+
+    model = _make(23)
+    for b in model.blocks:
+        fully_shard(b, mp_policy=MP)
+    fully_shard(model.norm, mp_policy=MP)
+    fully_shard(model, mp_policy=MP)
+    x = torch.randn(4, 128, device=DEV)
+    model(x)
+    groups = fsdp_groups_of(model)
+    g = groups[0]
+    for m in (model.blocks[2], model.norm):
+        m.reshard()
+    full16 = {p._param_fqn: torch.randn(p._orig_size, device=DEV).bfloat16() for p in g.fsdp_params}
+    load_full_tensors(g, full16)
+    for p in g.fsdp_params:
+        assert_bits_equal(p._sharded_param_data, full16[p._param_fqn].float().view(-1), p._param_fqn)
+    model(x)  # the forward casts the new masters into the all-gather input
+    torch.cuda.synchronize()
+    assert_bits_equal(g._all_gather_input[None], g._padded_sharded_param_data[None].bfloat16(), "copy-in after load")
+    with pytest.raises(KeyError):
+        load_full_tensors(g, {})

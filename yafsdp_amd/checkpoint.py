@@ -1,0 +1,153 @@
+"""Sharded checkpoint format of the ragged shards, and conversion to and from
+full parameters on one GPU.
+
+In the reference a sharded parameter is saved as ONE chunk of the parameter
+flattened to 1-D: ``offsets = (global_offset,)`` (or ``(numel,)`` when the rank
+holds nothing of it), ``sizes = (local_numel,)``, full ``size = (numel,)``
+(``__create_write_items__`` / ``__create_chunk_list__``,
+ya_fsdp/_tensor.py:365-423), and ``full_tensor()`` is an all-gather of the
+local tensors into ``full.split(shard_numels)`` (ya_fsdp/_tensor.py:345-363).
+The legacy wrapper stores names, element counts and shapes per module next to
+its flat shards (``_meta_info``, ya_fsdp/ya_fsdp.py:236-245).
+
+Here the same metadata comes from the closed-form layout, and the byte
+movement runs on the buffer kernels: the ranks' flat shards are copied into a
+flat buffer (``flat_copy``) and split into the full parameters by the copy-out
+kernel (``scatter_out``); loading copies each rank's fragment out of the full
+parameter (``flat_copy``).  One GPU: the "ranks" are the logical ranks of a
+layout, e.g. modules wrapped with ``mesh=(W, r)``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Iterable, Mapping, Sequence
+
+import torch
+import torch.nn as nn
+
+from . import _native
+from ._layout import RaggedShard
+from ._param_group import YaFSDPParamGroup
+
+__all__ = ["ChunkMeta", "chunk_meta", "sharded_state_dict", "group_meta_info", "full_tensors", "load_full_tensors"]
+
+
+@dataclass(frozen=True)
+class ChunkMeta:
+    """What the reference writes for one sharded parameter on one rank."""
+
+    fqn: str
+    offsets: tuple[int, ...]  # position of the chunk in the flattened parameter
+    sizes: tuple[int, ...]  # its length
+    size: tuple[int, ...]  # the flattened parameter's size
+    shape: tuple[int, ...]  # the parameter's original shape
+
+
+def chunk_meta(fqn: str, placement: RaggedShard, shape: Sequence[int]) -> ChunkMeta:
+    """ya_fsdp/_tensor.py:365-392 for a 1-D shard mesh: an empty fragment is
+    placed at ``offset == numel`` (its ``global_offset`` already is,
+    ya_fsdp/_param_group.py:365-377)."""
+    numel = 1
+    for d in shape:
+        numel *= int(d)
+    if placement.local_numel == 0:
+        offsets = (numel,)
+    else:
+        offsets = (placement.global_offset,)
+    return ChunkMeta(fqn, offsets, (placement.local_numel,), (numel,), tuple(int(d) for d in shape))
+
+
+def sharded_state_dict(group: YaFSDPParamGroup) -> dict[str, tuple[torch.Tensor, ChunkMeta]]:
+    """``{fqn: (local 1-D tensor, chunk)}`` of one parameter group on this rank;
+    the tensors are views of the flat master shard (no copy)."""
+    out = {}
+    for fsdp_param in group.fsdp_params:
+        meta = chunk_meta(fsdp_param._param_fqn, fsdp_param.placement, fsdp_param._orig_size)
+        out[fsdp_param._param_fqn] = (fsdp_param._sharded_param_data, meta)
+    return out
+
+
+def group_meta_info(group: YaFSDPParamGroup) -> dict[str, list]:
+    """The per-module record the legacy wrapper keeps in its state dict
+    (ya_fsdp/ya_fsdp.py:236-245), for one group."""
+    return {
+        "shard_boundaries": list(group.layout.rank_range(group.mesh_info.shard_mesh_rank)),
+        "padded_numel": group.layout.padded_unsharded_numel,
+        "fqns": [p._param_fqn for p in group.fsdp_params],
+        "numels": [p._orig_size.numel() for p in group.fsdp_params],
+        "orig_shapes": [tuple(p._orig_size) for p in group.fsdp_params],
+    }
+
+
+def _check_ranks(groups: Sequence[YaFSDPParamGroup]) -> None:
+    w = groups[0].layout.world_size
+    if len(groups) != w:
+        raise ValueError(f"need the groups of all {w} ranks, got {len(groups)}")
+    for r, g in enumerate(groups):
+        if g.layout != groups[0].layout or g.mesh_info.shard_mesh_rank != r:
+            raise ValueError("groups must be the same parameter group on ranks 0..W-1, in rank order")
+
+
+def full_tensors(
+    rank_groups: Sequence[YaFSDPParamGroup], out: Mapping[str, torch.Tensor] | None = None
+) -> dict[str, torch.Tensor]:
+    """``full_tensor()`` of every parameter of a group (ya_fsdp/_tensor.py:345-363)
+    from the flat master shards of all its ranks: W ``flat_copy`` launches into a
+    flat buffer, one ``scatter_out`` launch into the full parameters.  ``out``
+    may provide destination tensors (master dtype, contiguous) by fqn."""
+    _check_ranks(rank_groups)
+    g0 = rank_groups[0]
+    lay = g0.layout
+    s = lay.padded_sharded_numel
+    dtype, device = g0.orig_dtype, g0.device
+    flat = torch.empty(lay.padded_unsharded_numel, dtype=dtype, device=device)
+    for r, g in enumerate(rank_groups):
+        _native.flat_copy(flat[r * s : (r + 1) * s], g._padded_sharded_param_data[None])
+    result, dsts = {}, []
+    for fsdp_param in g0.fsdp_params:
+        fqn = fsdp_param._param_fqn
+        t = out[fqn] if out is not None and fqn in out else torch.empty(fsdp_param._orig_size, dtype=dtype, device=device)
+        if t.dtype != dtype or tuple(t.shape) != tuple(fsdp_param._orig_size) or not t.is_contiguous():
+            raise ValueError(f"{fqn}: destination must be a contiguous {dtype} tensor of shape {tuple(fsdp_param._orig_size)}")
+        result[fqn] = t
+        dsts.append(t.view(-1))
+    table = _native.TensorTable([d.numel() for d in dsts], lay.padded_unsharded_numel, device)
+    try:
+        table.scatter_out(flat, dsts)
+    finally:
+        table.close()
+    return result
+
+
+def load_full_tensors(groups: YaFSDPParamGroup | Iterable[YaFSDPParamGroup], full: Mapping[str, torch.Tensor]) -> None:
+    """The reverse: each given group (one rank of it, or several) takes its
+    fragment ``full[fqn].view(-1)[offset : offset + size]`` of every parameter
+    (the chunk of ``chunk_meta``), cast to the master dtype.  Runs on the
+    current stream; the next unshard casts the new masters (the group's
+    once-per-iteration copy-in flag is cleared)."""
+    if isinstance(groups, YaFSDPParamGroup):
+        groups = [groups]
+    for group in groups:
+        for fsdp_param in group.fsdp_params:
+            fqn = fsdp_param._param_fqn
+            if fqn not in full:
+                raise KeyError(f"{fqn} is missing from the full state dict")
+            src = full[fqn]
+            if src.numel() != fsdp_param._orig_size.numel():
+                raise ValueError(f"{fqn}: expected {fsdp_param._orig_size.numel()} elements, got {src.numel()}")
+            n = fsdp_param.placement.local_numel
+            if n == 0:
+                continue
+            go = fsdp_param.placement.global_offset
+            src = src.detach().to(group.device).contiguous().view(-1)
+            _native.flat_copy(fsdp_param._sharded_param_data, src[go : go + n])
+        group._all_gather_input_set_dtypes.clear()
+        group._copy_in_shard_version = None
+
+
+def fsdp_groups_of(module: nn.Module) -> list[YaFSDPParamGroup]:
+    """Parameter groups of every ``fully_shard`` module under ``module``."""
+    from .optim import fsdp_param_groups
+
+    return fsdp_param_groups(module)
