@@ -516,12 +516,15 @@ def main() -> int:
     d_shard = shard0.to(dev)
     d_chunk = d_rs[r * s : (r + 1) * s]
     table = _native.TensorTable(numels, t_pad, dev)
+    # the copy-out destinations persist across steps: their side of the table is bound once.  Gradients are fresh
+    # allocations of autograd in a training step, so the reduce copy-in passes its pointers on every call.
+    out_binding = table.bind(d_outs)
 
     def op_copy_in():
         _native.flat_copy(d_ag_in, d_master)
 
     def op_copy_out():
-        table.scatter_out(d_gathered, d_outs)
+        out_binding.scatter_out(d_gathered)
 
     def op_reduce_copy_in():
         table.gather_in(d_grads, d_rs, None, pre, True)
@@ -696,6 +699,7 @@ def main() -> int:
         "kernels": kernels,
     }
     print(json.dumps(out), flush=True)
+    out_binding.close()
     table.close()
     return 0
 

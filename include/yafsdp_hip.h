@@ -137,6 +137,25 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
 int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
                        const uint8_t* mode, int tensor_dtype, void* stream);
 
+/* The tensor side of a table fixed for many calls.  The reference's unsharded
+ * parameters and gradient accumulators are views of pre-allocated buffers that
+ * live as long as the group (ya_fsdp/_param_group.py:409-457), and consumers of
+ * the materialising copy-out keep their tensors as well: for such tensor sets
+ * the pointers, modes and dtype are validated (and, for tables with more than
+ * 16 tensors, copied to device memory) once, here; the bound calls then pass
+ * only the flat buffer.  No per-call host work beyond the launch and no
+ * per-call staging copy, so bound calls can be captured into a HIP graph
+ * whatever the table size.  The tensors must stay allocated, and the table
+ * alive, while the binding is used.  Semantics are those of yafsdp_gather_in /
+ * yafsdp_scatter_out. */
+typedef struct yafsdp_binding yafsdp_binding;
+int yafsdp_binding_create(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
+                          int tensor_dtype, yafsdp_binding** out);
+int yafsdp_binding_destroy(yafsdp_binding* binding);
+int yafsdp_gather_in_bound(yafsdp_binding* binding, void* flat, int flat_dtype, double pre_factor, int zero_pad,
+                           void* stream);
+int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat_dtype, void* stream);
+
 /* ---- optimizer-side passes over the flat shard buffers ------------------------
  * The reference runs the optimizer and gradient clipping as torch foreach ops
  * over the per-parameter fragments of the flat shard (dispatch table of its

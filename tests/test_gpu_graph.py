@@ -70,3 +70,52 @@ def test_captured_step_replays_match_eager():
         assert_bits_equal(rs, e_rs.cpu(), f"replay {it}: reduce copy-in")
         assert_bits_equal(shard_graph, shard_eager.cpu(), f"replay {it}: post-reduce")
     table.close()
+
+
+def test_bound_large_table_replays_match_eager():
+    """With a binding, a table of more than 16 tensors (metadata in device memory) needs no per-call staging
+    copy, so its launches can be captured too."""
+    import numpy as np
+
+    from yafsdp_amd import _native
+
+    rng = np.random.default_rng(5)
+    numels = (np.floor(np.exp2(rng.uniform(0, 15, size=120))).astype(np.int64) | 1).tolist()
+    t = sum(numels)
+    t_pad = t + 37
+    g = torch.Generator(device=DEV).manual_seed(78)
+    grads = [(torch.randn(n, device=DEV, generator=g) * 1e-3).bfloat16() for n in numels]
+    gathered = (torch.randn(t_pad, device=DEV, generator=g) * 0.02).bfloat16()
+    outs = [torch.zeros(n, dtype=torch.bfloat16, device=DEV) for n in numels]
+    rs = torch.zeros(t_pad, dtype=torch.float32, device=DEV)
+    table = _native.TensorTable(numels, t_pad, DEV)
+    gb, sb = table.bind(grads), table.bind(outs)
+
+    def step():
+        sb.scatter_out(gathered)
+        gb.gather_in(rs, 8.0, True)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for it in range(3):
+        gathered.mul_(1.0 + 0.25 * it)
+        for gr in grads:
+            gr.mul_(0.5)
+        e_outs = [torch.zeros_like(o) for o in outs]
+        e_rs = torch.zeros_like(rs)
+        table.scatter_out(gathered, e_outs)
+        table.gather_in(grads, e_rs, None, 8.0, True)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(outs, e_outs):
+            assert_bits_equal(a, b.cpu(), f"replay {it}: copy-out")
+        assert_bits_equal(rs, e_rs.cpu(), f"replay {it}: reduce copy-in")
+    gb.close(), sb.close(), table.close()

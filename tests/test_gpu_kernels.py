@@ -244,6 +244,48 @@ def test_scatter_out(nat, table_workgroup, case, flat_dt, out_dt):
     table.close()
 
 
+@pytest.mark.parametrize("case", [TABLE_CASES[1], TABLE_CASES[4], TABLE_CASES[5]])
+def test_bound_calls_match_per_call_pointers(nat, table_workgroup, case):
+    """A binding fixes pointers, modes and dtype once; bound launches give the same bits as per-call ones,
+    call after call, for tables that travel in the kernel arguments and for staged ones."""
+    p, max_log2, with_empty, pad = case
+    rng = np.random.default_rng(p * 77 + pad)
+    g = torch.Generator().manual_seed(140 + p)
+    numels = _random_numels(rng, p, max_log2, with_empty)
+    t = sum(numels)
+    t_pad = t + pad
+    modes = rng.integers(0, 3, size=p).tolist()
+    grads = [mixed_values(g, n, torch.bfloat16, 1e-3).to(DEV) for n in numels]
+    old = mixed_values(g, t_pad, torch.float32, 1e-3)
+    table = nat.TensorTable(numels, t_pad, torch.device(DEV))
+    want = old.to(DEV)
+    table.gather_in(grads, want, modes, 3.0, True)
+    binding = table.bind(grads, modes)
+    for _ in range(2):
+        got = old.to(DEV)
+        binding.gather_in(got, 3.0, True)
+        assert_bits_equal(got, want, "bound gather_in")
+    # the tensors' contents may change between calls, their addresses may not
+    for x in grads:
+        x.mul_(2)
+    table.gather_in(grads, want := old.to(DEV), modes, None, True)
+    binding.gather_in(got := old.to(DEV), None, True)
+    assert_bits_equal(got, want, "bound gather_in after the tensors changed")
+    # scatter
+    flat = mixed_values(g, t_pad, torch.bfloat16).to(DEV)
+    smodes = [int(m > 0) for m in modes]
+    outs_a = [torch.full((n,), 3.0, dtype=torch.float32, device=DEV) for n in numels]
+    outs_b = [torch.full((n,), 3.0, dtype=torch.float32, device=DEV) for n in numels]
+    table.scatter_out(flat, outs_a, smodes)
+    sb = table.bind(outs_b, smodes)
+    sb.scatter_out(flat)
+    for i, (a, b) in enumerate(zip(outs_a, outs_b)):
+        assert_bits_equal(b, a, f"bound scatter_out tensor {i}")
+    with pytest.raises(ValueError):
+        table.bind(grads[:-1])
+    sb.close(), binding.close(), table.close()
+
+
 def test_errors_are_loud(nat):
     a = torch.zeros(16, dtype=torch.float32, device=DEV)
     with pytest.raises(RuntimeError):

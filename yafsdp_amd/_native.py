@@ -40,6 +40,10 @@ EXPORTED_SYMBOLS = (
     "yafsdp_table_info",
     "yafsdp_gather_in",
     "yafsdp_scatter_out",
+    "yafsdp_binding_create",
+    "yafsdp_binding_destroy",
+    "yafsdp_gather_in_bound",
+    "yafsdp_scatter_out_bound",
     "yafsdp_flat_fill",
     "yafsdp_sumsq_workspace_bytes",
     "yafsdp_flat_sumsq",
@@ -86,6 +90,14 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_gather_in.argtypes = [vp, vp, vp, i32, vp, i32, dbl, i32, vp]
     lib.yafsdp_scatter_out.restype = i32
     lib.yafsdp_scatter_out.argtypes = [vp, vp, i32, vp, vp, i32, vp]
+    lib.yafsdp_binding_create.restype = i32
+    lib.yafsdp_binding_create.argtypes = [vp, vp, vp, i32, ctypes.POINTER(vp)]
+    lib.yafsdp_binding_destroy.restype = i32
+    lib.yafsdp_binding_destroy.argtypes = [vp]
+    lib.yafsdp_gather_in_bound.restype = i32
+    lib.yafsdp_gather_in_bound.argtypes = [vp, vp, i32, dbl, i32, vp]
+    lib.yafsdp_scatter_out_bound.restype = i32
+    lib.yafsdp_scatter_out_bound.argtypes = [vp, vp, i32, vp]
     lib.yafsdp_flat_fill.restype = i32
     lib.yafsdp_flat_fill.argtypes = [vp, i32, i64, dbl, vp]
     lib.yafsdp_sumsq_workspace_bytes.restype = ctypes.c_size_t
@@ -250,6 +262,10 @@ class TensorTable:
         if h:
             lib.yafsdp_table_destroy(h)
 
+    def bind(self, tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None = None) -> "TensorBinding":
+        """Fix the tensor side for many calls (see ``TensorBinding``)."""
+        return TensorBinding(self, tensors, modes)
+
     def __del__(self) -> None:
         try:
             self.close()
@@ -348,6 +364,65 @@ class TensorTable:
                     _stream(flat),
                 ),
                 "yafsdp_scatter_out",
+            )
+
+
+class TensorBinding:
+    """The tensor side of a ``TensorTable`` fixed for many calls (tensors that
+    persist across steps: copy-out destinations, gradient accumulators).
+    Pointers, modes and dtype are checked and staged once; ``gather_in`` /
+    ``scatter_out`` then cost one launch and no per-tensor host work, and can be
+    captured into a HIP graph whatever the table size.  Holds references to the
+    tensors and the table."""
+
+    def __init__(self, table: "TensorTable", tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None = None):
+        self.table = table
+        self.tensors = list(tensors)
+        handle = ctypes.c_void_p()
+        with table._lock, torch.cuda.device(table.device):
+            tdt = table._fill(self.tensors, modes, "tensors")
+            self._all_skipped = tdt < 0
+            _check(
+                lib.yafsdp_binding_create(
+                    table._handle, table._ptrs.ctypes.data, table._modes.ctypes.data, max(tdt, 0), ctypes.byref(handle)
+                ),
+                "yafsdp_binding_create",
+            )
+        self._handle = handle
+
+    def close(self) -> None:
+        h, self._handle = getattr(self, "_handle", None), None
+        if h:
+            lib.yafsdp_binding_destroy(h)
+
+    def __del__(self) -> None:
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def gather_in(self, flat: torch.Tensor, pre_factor: float | None = None, zero_pad: bool = True) -> None:
+        _flat_arg(flat, "flat")
+        if flat.numel() < self.table.padded_numel:
+            raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.table.padded_numel}")
+        with torch.cuda.device(self.table.device):
+            _check(
+                lib.yafsdp_gather_in_bound(
+                    self._handle, flat.data_ptr(), _dt(flat), _factor(pre_factor), int(bool(zero_pad)), _stream(flat)
+                ),
+                "yafsdp_gather_in_bound",
+            )
+
+    def scatter_out(self, flat: torch.Tensor) -> None:
+        _flat_arg(flat, "flat")
+        if flat.numel() < self.table.total_numel:
+            raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.table.total_numel}")
+        if self._all_skipped:
+            return
+        with torch.cuda.device(self.table.device):
+            _check(
+                lib.yafsdp_scatter_out_bound(self._handle, flat.data_ptr(), _dt(flat), _stream(flat)),
+                "yafsdp_scatter_out_bound",
             )
 
 

@@ -123,6 +123,16 @@ struct yafsdp_table {
   std::mutex mu;
 };
 
+// The tensor side of a table fixed for many calls: validated once, and for
+// tables with more than kSmallMax tensors staged to device memory once.
+struct yafsdp_binding {
+  yafsdp_table* table = nullptr;
+  int tensor_dtype = 0;
+  SmallMeta small;             // tables with at most kSmallMax tensors
+  char* d_arrays = nullptr;    // others: pointers (8 bytes each) then modes (4 bytes each)
+  LargeMeta large;
+};
+
 namespace {
 
 void table_free(yafsdp_table* t) {
@@ -221,6 +231,98 @@ const char* yafsdp_error_string(int code) {
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
   return "yafsdp: unknown error code";
+}
+
+int yafsdp_binding_create(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
+                          int tensor_dtype, yafsdp_binding** out) {
+  if (out == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  *out = nullptr;
+  if (table == nullptr || (table->n_tensors > 0 && tensor_ptrs == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!valid_dtype(tensor_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
+  const int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
+  if (rc != YAFSDP_OK) return rc;
+  yafsdp_binding* b = new (std::nothrow) yafsdp_binding();
+  if (b == nullptr) return YAFSDP_ERR_OUT_OF_MEMORY;
+  b->table = table;
+  b->tensor_dtype = tensor_dtype;
+  const int n = table->n_tensors;
+  if (n <= kSmallMax) {
+    fill_small(table, tensor_ptrs, mode, &b->small);
+  } else {
+    const size_t bytes = size_t(n) * (sizeof(void*) + sizeof(uint32_t));
+    std::vector<char> host(bytes);
+    std::memcpy(host.data(), tensor_ptrs, size_t(n) * sizeof(void*));
+    uint32_t* hm = reinterpret_cast<uint32_t*>(host.data() + size_t(n) * sizeof(void*));
+    for (int p = 0; p < n; p++) hm[p] = mode ? mode[p] : uint32_t(MODE_COPY);
+    if ((e = hipMalloc(reinterpret_cast<void**>(&b->d_arrays), bytes)) != hipSuccess ||
+        (e = hipMemcpy(b->d_arrays, host.data(), bytes, hipMemcpyHostToDevice)) != hipSuccess) {
+      if (b->d_arrays) (void)hipFree(b->d_arrays);
+      delete b;
+      return int(e);
+    }
+    b->large.offsets = table->d_offsets;
+    b->large.tiles = table->d_tiles;
+    b->large.ptrs = reinterpret_cast<const void* const*>(b->d_arrays);
+    b->large.modes_ = reinterpret_cast<const uint32_t*>(b->d_arrays + size_t(n) * sizeof(void*));
+    b->large.n_tensors = n;
+  }
+  *out = b;
+  return YAFSDP_OK;
+}
+
+int yafsdp_binding_destroy(yafsdp_binding* binding) {
+  if (binding == nullptr) return YAFSDP_OK;
+  if (binding->d_arrays) (void)hipFree(binding->d_arrays);
+  delete binding;
+  return YAFSDP_OK;
+}
+
+int yafsdp_gather_in_bound(yafsdp_binding* binding, void* flat, int flat_dtype, double pre_factor, int zero_pad,
+                           void* stream) {
+  if (binding == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  const yafsdp_table* table = binding->table;
+  if (!valid_dtype(flat_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (table->padded == 0) return YAFSDP_OK;
+  if (flat == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(flat, 16)) return YAFSDP_ERR_MISALIGNED;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
+  int scale;
+  float k;
+  scale_plan(pre_factor, &scale, &k);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  if (table->n_tensors <= kSmallMax)
+    return int(launch_gather<SmallMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->small, flat,
+                                        table->padded, table->n_tiles, k, zero_pad ? 1 : 0, grid, s));
+  return int(launch_gather<LargeMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->large, flat,
+                                      table->padded, table->n_tiles, k, zero_pad ? 1 : 0, grid, s));
+}
+
+int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat_dtype, void* stream) {
+  if (binding == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  const yafsdp_table* table = binding->table;
+  if (!valid_dtype(flat_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (table->total == 0) return YAFSDP_OK;
+  if (flat == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(flat, 16)) return YAFSDP_ERR_MISALIGNED;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  if (table->n_tensors <= kSmallMax)
+    return int(launch_scatter<SmallMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->small, flat,
+                                         table->total, table->n_tiles, grid, s));
+  return int(launch_scatter<LargeMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->large, flat,
+                                       table->total, table->n_tiles, grid, s));
 }
 
 int yafsdp_time_next_launch(void* start_event, void* stop_event) {
