@@ -57,7 +57,9 @@ def _ragged_stress_shapes(seed=1005, p=2000):
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
 # (factors 1.99988 and 0.99986): (213037.875 * 1.99988 + 426022.75 * 0.99986) KiB.
 # Summary and commands: profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_461_600}
+# "llama3-8b-layer-w8-optim": adamw_kernel, (213045.6 * 1.99946 + 372753.5 * 0.99996) KiB, scaled by the plain
+# fp32 copy of the same run; profiles/bench_llama3-8b-layer-w8-optim_hbm_traffic.md.
+MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_461_600, "llama3-8b-layer-w8-optim": 817_885_000}
 
 
 def log(*a):
@@ -436,8 +438,8 @@ def run_optim(args) -> int:
                           "fused grad scale and bf16 all-gather input"},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "parity": parity,
         "roofline": {"bound": "hbm", "kernel": "adamw_kernel (fused AdamW step)", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                     "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2),
                      "launches_timed": len(dom_us)},
         "cpu_baseline": cpu_baseline, "kernels": kernels,
     }
