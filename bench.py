@@ -425,6 +425,36 @@ def run_optim(args) -> int:
         }
         log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads ({len(times)} passes)")
 
+    torch_gpu = None
+    if not args.no_torch_gpu:
+        # what the reference runs on this hardware: torch's clipping, fused AdamW and the copy-in cast on the GPU
+        gparam = torch.nn.Parameter(master.to(dev))
+        gopt = torch.optim.AdamW([gparam], lr=hp["lr"], betas=(hp["beta1"], hp["beta2"]), eps=hp["eps"],
+                                 weight_decay=hp["weight_decay"], fused=True)
+        g_ag_in = torch.zeros(s, dtype=torch.bfloat16, device=dev)
+        gparam.grad = d_g_keep.clone()
+
+        def gpu_torch_step():
+            torch.nn.utils.clip_grad_norm_([gparam], max_norm, foreach=True)
+            gopt.step()
+            torch_ops.copy_in(g_ag_in, gparam.detach())
+
+        for _ in range(3):
+            gpu_torch_step()
+        torch.cuda.synchronize()
+        reps = 20
+        c0 = time.perf_counter()
+        for _ in range(reps):
+            gpu_torch_step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - c0) / reps
+        torch_gpu = {
+            "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
+            "sample": f"{reps} passes of torch.nn.utils.clip_grad_norm_ + torch.optim.AdamW(fused=True).step + copy-in "
+                      f"cast on device tensors with torch {torch.__version__}, rated with the fused pass's bytes",
+        }
+        log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
+
     out = {
         "metric": "HBM GB/s + % of peak for the optimizer-side flat-shard passes (grad norm + fused AdamW/copy-in), "
                   "Llama-3-8B layer @W=8" if base == "llama3-8b-layer-w8" else
@@ -441,7 +471,7 @@ def run_optim(args) -> int:
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2),
                      "launches_timed": len(dom_us)},
-        "cpu_baseline": cpu_baseline, "kernels": kernels,
+        "cpu_baseline": cpu_baseline, "torch_gpu_baseline": torch_gpu, "kernels": kernels,
     }
     print(json.dumps(out), flush=True)
     return 0
@@ -457,6 +487,8 @@ def main() -> int:
                                                  "llama3-70b-layer-w64-optim"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
+    ap.add_argument("--no-torch-gpu", action="store_true",
+                    help="skip the leg that times the reference's torch ops on the GPU (outside the timed region)")
     ap.add_argument("--sweep-grid-cap", action="store_true",
                     help="llama3-8b-full-w8 only: repeat the overlap measurement with the copy kernels' grids capped "
                          "at 16/8/4/2/1 workgroups per compute unit")
@@ -669,6 +701,42 @@ def main() -> int:
         }
         log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads ({reps} passes)")
 
+    # ---- the same torch-op sequence on the GPU (torch's own ROCm kernels): what the reference runs on this
+    # hardware today.  Outside the timed region; reported next to the CPU baseline, not a target.
+    torch_gpu = None
+    if cpu_state is not None and not args.no_torch_gpu:
+        from oracle import torch_ops  # noqa: F811
+
+        g_rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=dev)
+        g_state = {
+            "ag_in": torch.zeros(s, dtype=torch.bfloat16, device=dev),
+            "outs": [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels],
+            "rs": g_rs, "rs_views": list(g_rs[:t].split(numels)), "shard": shard0.to(dev),
+        }
+
+        def gpu_torch_step(st):
+            torch_ops.copy_in(st["ag_in"], d_master)
+            torch_ops.copy_out_materialize(d_gathered, numels, st["outs"])
+            torch_ops.reduce_copy_in(st["rs_views"], d_grads, False)
+            torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
+
+        for _ in range(3):
+            gpu_torch_step(g_state)
+        torch.cuda.synchronize()
+        reps = 20
+        c0 = time.perf_counter()
+        for _ in range(reps):
+            gpu_torch_step(g_state)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - c0) / reps
+        torch_gpu = {
+            "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
+            "sample": f"{reps} passes of the reference's torch ops (copy_, split + copy_, _foreach_copy_, div_, add_) on "
+                      f"device tensors with torch {torch.__version__}, same inputs, rated with the same algorithmic bytes",
+        }
+        log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
+        del g_state, g_rs
+
     out = {
         "metric": "HBM GB/s + % of peak for copy-in/out+grad-reduce, Llama-3-8B layer @W=8",
         "value": round(value, 1),
@@ -698,6 +766,7 @@ def main() -> int:
             "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2), "launches_timed": len(dom_us),
         },
         "cpu_baseline": cpu_baseline,
+        "torch_gpu_baseline": torch_gpu,
         "kernels": kernels,
     }
     print(json.dumps(out), flush=True)

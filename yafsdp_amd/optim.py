@@ -330,7 +330,7 @@ class FlatAdamW(torch.optim.Optimizer):
         # next forward casts the shard itself, as it does in the reference
         out16 = None
         if (self.fuse_copy_in and whole and uniform and len(unit.indices) == len(group.fsdp_params)
-                and group.param_dtype is not None and hasattr(group, "_all_gather_input")):
+                and group.param_dtype is not None and hasattr(group, "_all_gather_input") and group.is_sharded):
             out16 = group._all_gather_input[None]
         if whole and uniform:
             runs = [(0, shard.numel(), unit.steps[with_grad[0]])]
