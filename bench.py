@@ -42,16 +42,17 @@ WORKLOADS = {
 }
 
 
-def _ragged_stress_shapes(seed=1005, p=2000):
-    """2,000 tensors with odd element counts, log-uniform in [1, 2^22]; the 70 % drawn as fp32 masters with bf16
-    compute form the group measured here (a group has one master dtype)."""
+def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
+    """2,000 tensors with odd element counts, log-uniform in [1, 2^22], 70 % drawn as fp32 masters with bf16
+    compute and 30 % as bf16 masters with fp32 reduce; a group has one master dtype, so the two classes are two
+    groups (two workloads here)."""
     import torch
 
     g = torch.Generator().manual_seed(seed)
     u = torch.rand(p, generator=g, dtype=torch.float64) * 22 * 0.6931471805599453
     numels = (torch.exp(u).floor().to(torch.int64) | 1).tolist()
     is_fp32_master = (torch.rand(p, generator=g) < 0.7).tolist()
-    return [(n,) for n, f in zip(numels, is_fp32_master) if f]
+    return [(n,) for n, f in zip(numels, is_fp32_master) if f == fp32_masters]
 
 # HBM bytes per launch of the dominant kernel (gather_in_kernel), from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
@@ -483,7 +484,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="llama3-8b-layer-w8",
-                    choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256", "llama3-8b-layer-w8-optim",
+                    choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256", "ragged-stress-w256-bf16-masters",
+                                                 "llama3-8b-layer-w8-optim",
                                                  "llama3-70b-layer-w64-optim"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
@@ -516,10 +518,18 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    # master / compute / reduce dtypes of the group: fp32 masters with bf16 compute and reduce, except the stress
+    # test's second group (bf16 masters: no copy-in cast, fp32 reduce buffer, bf16 gradient shard)
+    master_dt, rs_dt = torch.float32, torch.bfloat16
     if args.workload == "ragged-stress-w256":
         shapes, w, r, align, seed = _ragged_stress_shapes(), 256, 1, 512, 1005
+    elif args.workload == "ragged-stress-w256-bf16-masters":
+        shapes, w, r, align, seed = _ragged_stress_shapes(fp32_masters=False), 256, 1, 512, 1005
+        master_dt, rs_dt = torch.bfloat16, torch.float32
     else:
         shapes, w, r, align, seed = WORKLOADS[args.workload]
+    msz, rsz = master_dt.itemsize, rs_dt.itemsize
+    has_copy_in = master_dt != torch.bfloat16
     numels = [numel_of(s) for s in shapes]
     lay = make_layout(numels, w, align)
     t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
@@ -529,7 +539,7 @@ def main() -> int:
     # ---- synthetic inputs, generated on the CPU so that the oracle sees the same bits
     g = torch.Generator().manual_seed(seed)
     t0 = time.perf_counter()
-    master = torch.randn(s, generator=g) * 0.02  # fp32 master shard
+    master = (torch.randn(s, generator=g) * 0.02).to(master_dt)  # master shard
     gathered = torch.empty(t_pad, dtype=torch.bfloat16)
     grads = []
     pos = 0
@@ -538,7 +548,7 @@ def main() -> int:
         grads.append((torch.randn(n, generator=g) * 1e-3).bfloat16())
         pos += n
     gathered[t:] = 0
-    shard0 = torch.randn(s, generator=g) * 1e-4  # existing fp32 gradient shard
+    shard0 = (torch.randn(s, generator=g) * 1e-4).to(master_dt)  # existing gradient shard (master dtype)
     log(f"inputs generated in {time.perf_counter() - t0:.1f}s")
 
     d_master = master.to(dev)
@@ -546,7 +556,7 @@ def main() -> int:
     d_grads = [x.to(dev) for x in grads]
     d_ag_in = torch.zeros(s, dtype=torch.bfloat16, device=dev)
     d_outs = [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels]
-    d_rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=dev)
+    d_rs = torch.zeros(t_pad, dtype=rs_dt, device=dev)
     d_shard = shard0.to(dev)
     d_chunk = d_rs[r * s : (r + 1) * s]
     table = _native.TensorTable(numels, t_pad, dev)
@@ -567,11 +577,13 @@ def main() -> int:
         _native.post_reduce(d_shard, d_chunk, None, True)
 
     ops = [
-        ("copy_in", op_copy_in, s * (4 + 2)),
+        ("copy_in", op_copy_in, s * (msz + 2)),
         ("copy_out", op_copy_out, 2 * t * 2),
-        ("reduce_copy_in", op_reduce_copy_in, t * (2 + 2) + (t_pad - t) * 2),
-        ("post_reduce", op_post_reduce, s * (2 + 4 + 4)),
+        ("reduce_copy_in", op_reduce_copy_in, t * (2 + rsz) + (t_pad - t) * rsz),
+        ("post_reduce", op_post_reduce, s * (rsz + 2 * msz)),
     ]
+    if not has_copy_in:  # the all-gather input aliases the master shard (ya_fsdp/_param_group.py:502-505)
+        ops = ops[1:]
     bytes_per_step = sum(b for _, _, b in ops)
 
     def step():
@@ -585,12 +597,13 @@ def main() -> int:
         from oracle import torch_ops
 
         def cpu_step(st):
-            torch_ops.copy_in(st["ag_in"], master)
+            if has_copy_in:
+                torch_ops.copy_in(st["ag_in"], master)
             torch_ops.copy_out_materialize(gathered, numels, st["outs"])
             torch_ops.reduce_copy_in(st["rs_views"], grads, False)
             torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
 
-        rs_cpu = torch.zeros(t_pad, dtype=torch.bfloat16)
+        rs_cpu = torch.zeros(t_pad, dtype=rs_dt)
         cpu_state = {
             "ag_in": torch.zeros(s, dtype=torch.bfloat16),
             "outs": [torch.empty(n, dtype=torch.bfloat16) for n in numels],
@@ -606,7 +619,7 @@ def main() -> int:
             iv = torch.int32 if a.dtype == torch.float32 else torch.int16
             return torch.equal(a.cpu().view(iv), b.view(iv))
 
-        ok = same(d_ag_in, cpu_state["ag_in"]) and same(d_rs, cpu_state["rs"]) and same(d_shard, cpu_state["shard"])
+        ok = same(d_ag_in, cpu_state["ag_in"]) and same(d_rs, cpu_state["rs"]) and same(d_shard, cpu_state["shard"])  # noqa: E501 (d_ag_in stays zero on both sides without a copy-in)
         ok = ok and all(same(a, b) for a, b in zip(d_outs, cpu_state["outs"]))
         parity = "bit-exact" if ok else "MISMATCH"
         log("parity vs oracle:", parity)
@@ -625,20 +638,19 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    dom_index = 2  # reduce copy-in: most bytes, fused arithmetic
+    dom_index = [n for n, _, _ in ops].index("reduce_copy_in")  # most bytes, fused arithmetic
     # on every 4th step of the timed region the dominant kernel's dispatch carries a pair of HIP events (attached to
     # the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
     sampled = [k for k in range(args.steps) if k % 4 == 0]
     ev = {k: _event_pair() for k in sampled}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    fns = [fn for _, fn, _ in ops]
     for k in range(args.steps):
-        ops[0][1]()
-        ops[1][1]()
-        if k in ev:
-            _native.time_next_launch(*ev[k])
-        ops[2][1]()
-        ops[3][1]()
+        for i, fn in enumerate(fns):
+            if i == dom_index and k in ev:
+                _native.time_next_launch(*ev[k])
+            fn()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
@@ -707,7 +719,7 @@ def main() -> int:
     if cpu_state is not None and not args.no_torch_gpu:
         from oracle import torch_ops  # noqa: F811
 
-        g_rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=dev)
+        g_rs = torch.zeros(t_pad, dtype=rs_dt, device=dev)
         g_state = {
             "ag_in": torch.zeros(s, dtype=torch.bfloat16, device=dev),
             "outs": [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels],
@@ -715,7 +727,8 @@ def main() -> int:
         }
 
         def gpu_torch_step(st):
-            torch_ops.copy_in(st["ag_in"], d_master)
+            if has_copy_in:
+                torch_ops.copy_in(st["ag_in"], d_master)
             torch_ops.copy_out_materialize(d_gathered, numels, st["outs"])
             torch_ops.reduce_copy_in(st["rs_views"], d_grads, False)
             torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
@@ -754,8 +767,10 @@ def main() -> int:
             "workload": args.workload, "params": len(numels), "total_numel": t, "padded_numel": t_pad,
             "shard_numel": s, "logical_world_size": w, "rank": r, "shard_alignment": align,
             "predivide": pre, "bytes_per_step": bytes_per_step,
-            "ops": "copy-in fp32->bf16 [S]; copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
-                   "post-reduce bf16 chunk += fp32 shard [S]",
+            "master_dtype": str(master_dt).replace("torch.", ""), "reduce_dtype": str(rs_dt).replace("torch.", ""),
+            "ops": ("copy-in master->bf16 [S]; " if has_copy_in else "") +
+                   "copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
+                   "post-reduce chunk += gradient shard (master dtype) [S]",
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "parity": parity,
