@@ -217,3 +217,49 @@ def test_logical_world_size_gives_each_rank_its_ragged_shard():
         assert [p.numel() for p in sharded] == lay.sharded_numels(r)
         pieces.append(torch.cat([p.detach() for p in sharded]))
     assert torch.equal(torch.cat(pieces), full)  # the ranks' fragments tile the flat parameter space
+
+
+def test_list_of_modules_forms_one_group():
+    """``fully_shard([a, b])``: one parameter group gathered before the first of the modules runs and released
+    after the last (ya_fsdp/_state.py:575-613); training matches wrapping the same modules one by one."""
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.fully_shard import YaFSDPModule
+    from yafsdp_amd.optim import fsdp_param_groups
+
+    model0 = _make(31)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(40 + s)) for s in range(3)]
+
+    def train(grouped: bool):
+        model = copy.deepcopy(model0)
+        if grouped:
+            out = fully_shard([model.blocks[0], model.blocks[1], model.blocks[0].up], mp_policy=MP)  # nested one dropped
+            assert isinstance(out, list) and isinstance(model.blocks[0], YaFSDPModule) and isinstance(model.blocks[1], YaFSDPModule)
+            assert not isinstance(model.blocks[0].up, YaFSDPModule)
+        else:
+            fully_shard(model.blocks[0], mp_policy=MP)
+            fully_shard(model.blocks[1], mp_policy=MP)
+        fully_shard(model.blocks[2], mp_policy=MP)
+        fully_shard(model.norm, mp_policy=MP)
+        fully_shard(model, mp_policy=MP)
+        groups = fsdp_param_groups(model)
+        assert len(groups) == (3 if grouped else 4)
+        if grouped:
+            assert len(groups[0].fsdp_params) == 6 and groups[0].modules == (model.blocks[0], model.blocks[1])
+        opt = torch.optim.SGD(model.parameters(), lr=0.05)
+        for x in xs:
+            model(x).float().pow(2).mean().backward()
+            if grouped:
+                assert groups[0].is_sharded and not model._get_fsdp_state()._modules_to_run_forward
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+        torch.cuda.synchronize()
+        return _gather_full(model)
+
+    a, b = train(True), train(False)
+    assert set(a) == set(b)
+    for k in a:
+        assert torch.equal(a[k].view(torch.int32), b[k].view(torch.int32)), k
+    with pytest.raises(RuntimeError, match="single root"):
+        m = _make(32)
+        fully_shard([m.blocks[0], m.blocks[1]], mp_policy=MP)
+        m.blocks[0](xs[0])

@@ -52,22 +52,50 @@ class YaFSDPState(_State):
         self._states_to_forward_prefetch: list[YaFSDPState] = []
         self._states_to_backward_prefetch: list[YaFSDPState] = []
         self._auto_reshard_after_forward: bool | None = True
+        self._modules_to_run_forward: set[nn.Module] = set()
 
     def init(self, modules: tuple, device: torch.device, mp_policy: MixedPrecisionPolicy,
              auto_reshard_after_forward: bool) -> None:
-        """ya_fsdp/_state.py:72-101 for a single module per call."""
-        if len(modules) != 1:
-            raise NotImplementedError("fully_shard over a list of modules is not part of this build")
+        """ya_fsdp/_state.py:72-101."""
         for module in modules:
             _insert_module_state(module, self)
         self._modules = modules
         self._device = device
         self._mp_policy = mp_policy
         self._auto_reshard_after_forward = auto_reshard_after_forward
-        self._pre_forward_hook_handle = modules[0].register_forward_pre_hook(
-            self._pre_forward, prepend=True, with_kwargs=True
-        )
-        self._post_forward_hook_handle = modules[0].register_forward_hook(self._post_forward, prepend=False)
+        if len(modules) == 1:
+            self._pre_forward_hook_handle = modules[0].register_forward_pre_hook(
+                self._pre_forward, prepend=True, with_kwargs=True
+            )
+            self._post_forward_hook_handle = modules[0].register_forward_hook(self._post_forward, prepend=False)
+        else:
+            self._pre_forward_hook_handle = self._post_forward_hook_handle = self._register_group_forward_hooks()
+
+    def _register_group_forward_hooks(self) -> list:
+        """Several modules, one group (ya_fsdp/_state.py:575-613): the pre-forward
+        logic runs before whichever module runs first in an iteration, the
+        post-forward logic after the last of them has run."""
+        pending = self._modules_to_run_forward
+        members = set(self._modules)
+
+        def pre_hook(module: nn.Module, args: tuple, kwargs: dict):
+            if pending:
+                return None
+            pending.update(members)  # first of the group to run
+            return self._pre_forward(module, args, kwargs)
+
+        def post_hook_for(member: nn.Module):
+            def post_hook(module: nn.Module, input: Any, output: Any):
+                pending.discard(member)
+                if pending:
+                    return None
+                return self._post_forward(module, input, output)
+
+            return post_hook
+
+        handles = [m.register_forward_pre_hook(pre_hook, prepend=True, with_kwargs=True) for m in self._modules]
+        handles += [m.register_forward_hook(post_hook_for(m), prepend=False, always_call=True) for m in self._modules]
+        return handles
 
     # ---------------------------------------------------------------- lazy init --
     def _root_pre_forward(self, module: nn.Module, args: tuple, kwargs: dict) -> tuple[tuple, dict]:
@@ -95,6 +123,8 @@ class YaFSDPState(_State):
         if self._is_root is not None:
             return
         self._is_root = True
+        if len(self._modules) > 1:
+            raise RuntimeError(f"YaFSDP requires a single root module but got {self._modules}")  # ya_fsdp/_state.py:143-146
         root_module = self._modules[0]
         visited_states: set[YaFSDPState] = set()
         for module_name, module in root_module.named_modules():
@@ -304,6 +334,13 @@ class YaFSDPState(_State):
             self._state_ctx.post_backward_final_callback_queued = False
 
     def _finalize_backward(self) -> None:
+        if self._modules_to_run_forward:  # ya_fsdp/_state.py:534-546
+            logger.warning(
+                "%d of the %d modules passed to fully_shard did not run forward before backward; pass only modules "
+                "that run forward together. Modules that did not run forward: %s",
+                len(self._modules_to_run_forward), len(self._modules), list(self._modules_to_run_forward),
+            )
+            self._modules_to_run_forward.clear()  # the next forward starts afresh
         if self._fsdp_param_group:
             self._fsdp_param_group.finalize_backward()
 

@@ -23,7 +23,7 @@ cls_to_fsdp_cls: dict[type, type] = {}
 
 
 def fully_shard(
-    module: nn.Module,
+    module: "nn.Module | list[nn.Module]",
     *,
     mesh: Any = None,
     reshard_after_forward: bool | None = True,
@@ -31,39 +31,65 @@ def fully_shard(
     ignored_params: set[nn.Parameter] | None = None,
     shard_alignment: int = 8,
     device: torch.device | str | None = None,
-) -> "YaFSDPModule":
-    """ya_fsdp/fully_shard.py:67-129."""
+) -> "YaFSDPModule | list[YaFSDPModule]":
+    """ya_fsdp/fully_shard.py:67-129.  A list of modules forms ONE parameter group
+    whose parameters are gathered before the first of them runs forward and
+    released after the last one has (ya_fsdp/_state.py:575-613)."""
     if isinstance(module, (nn.ModuleList, nn.ModuleDict)):
         raise ValueError(f"fully_shard does not support containers that do not implement forward: {module}")
-    if not isinstance(module, nn.Module):
-        raise NotImplementedError("fully_shard over a list of modules is not part of this build")
-    if _get_module_fsdp_state(module) is not None:
-        raise AssertionError(f"fully_shard has already been applied to {type(module).__name__}")
+    arg_module = module
+    if isinstance(module, nn.Module):
+        modules = (module,)
+    else:
+        modules = tuple(_get_root_modules(list(module)))
+        if not modules or not all(isinstance(m, nn.Module) for m in modules):
+            raise ValueError("fully_shard expects a module or a non-empty list of modules")
+    for m in modules:
+        if _get_module_fsdp_state(m) is not None:
+            raise AssertionError(f"fully_shard has already been applied to {type(m).__name__}")
     mesh_info = mesh_info_from(mesh)
     device = torch.device(device if device is not None else f"cuda:{torch.cuda.current_device()}")
     auto_reshard_after_forward = reshard_after_forward is not None
-    modules = (module,)
     state = YaFSDPState()
     state.init(modules, device, mp_policy, auto_reshard_after_forward)
     managed_modules = _get_managed_modules(modules, _get_module_fsdp_state, ignored_params)
     params, buffers = _get_managed_states(managed_modules, ignored_params)
     _move_states_to_device(params, buffers, device)
     if params:
-        names = _param_names(module, params)
+        names = _param_names(modules, params)
         group = YaFSDPParamGroup(params, mesh_info, device, mp_policy, shard_alignment, names=names, modules=modules)
         group.reshard_after_forward = True if reshard_after_forward is None else bool(reshard_after_forward)
         state._fsdp_param_group = group
-    cls = module.__class__
-    new_cls = cls_to_fsdp_cls.get(cls)
-    if not new_cls:
-        new_cls = type(f"YaFSDP{cls.__name__}", (YaFSDPModule, cls), {"__deepcopy__": _unimplemented_deepcopy})
-        cls_to_fsdp_cls[cls] = new_cls
-    module.__class__ = new_cls
-    return module  # type: ignore[return-value]
+    for m in modules:
+        cls = m.__class__
+        new_cls = cls_to_fsdp_cls.get(cls)
+        if not new_cls:
+            new_cls = type(f"YaFSDP{cls.__name__}", (YaFSDPModule, cls), {"__deepcopy__": _unimplemented_deepcopy})
+            cls_to_fsdp_cls[cls] = new_cls
+        m.__class__ = new_cls
+    return arg_module  # type: ignore[return-value]
 
 
-def _param_names(module: nn.Module, params: list) -> list[str]:
-    by_id = {id(p): n for n, p in module.named_parameters(remove_duplicate=False)}
+def _get_root_modules(modules: list) -> list:
+    """The modules of the list that are not inside another module of the list
+    (ya_fsdp/fully_shard.py:99-101), in list order."""
+    roots = []
+    for candidate in modules:
+        inside = any(
+            other is not candidate and any(sub is candidate for sub in other.modules())
+            for other in modules
+        )
+        if not inside and not any(r is candidate for r in roots):
+            roots.append(candidate)
+    return roots
+
+
+def _param_names(modules: tuple, params: list) -> list[str]:
+    by_id: dict[int, str] = {}
+    for k, module in enumerate(modules):
+        prefix = "" if len(modules) == 1 else f"{k}."
+        for n, p in module.named_parameters(remove_duplicate=False):
+            by_id.setdefault(id(p), prefix + n)
     return [by_id.get(id(p), f"param{i}") for i, p in enumerate(params)]
 
 
