@@ -109,8 +109,12 @@ struct yafsdp_table {
   int64_t* d_offsets = nullptr;
   int block = kTableBlockSmall;  // workgroup size of the table kernels, chosen from the padded size
   int64_t tile_elems = 0;        // block * kTableUnroll * 8
-  int32_t n_tiles = 0;
+  int32_t n_tiles = 0;           // gather-in: tiles of the flat buffer
   TileRec* d_tiles = nullptr;    // only for tables with more than kSmallMax tensors
+  // scatter-out: tile slots per tensor (ceil(numel / tile) + 1 for a non-empty tensor)
+  std::vector<int64_t> slot_start;  // host, n_tensors + 1
+  int32_t n_slots = 0;
+  TileRec* d_slots = nullptr;    // only for tables with more than kSmallMax tensors
   // staging ring for the per-call pointer/mode arrays of tables with more than
   // kSmallMax tensors: pinned host slot -> device slot, one event per slot
   static constexpr int kRing = 4;
@@ -139,6 +143,7 @@ void table_free(yafsdp_table* t) {
   if (t == nullptr) return;
   if (t->d_offsets) (void)hipFree(t->d_offsets);
   if (t->d_tiles) (void)hipFree(t->d_tiles);
+  if (t->d_slots) (void)hipFree(t->d_slots);
   for (int i = 0; i < yafsdp_table::kRing; i++) {
     if (t->ev[i]) (void)hipEventDestroy(t->ev[i]);
     if (t->h_stage[i]) (void)hipHostFree(t->h_stage[i]);
@@ -172,6 +177,7 @@ void fill_small(const yafsdp_table* t, const void* const* ptrs, const uint8_t* m
     const int64_t o = t->offsets[i <= n ? i : n];
     m->off[i] = o;
     m->tile_start[i] = i <= n ? int32_t((o + tile_elems - 1) / tile_elems) : INT32_MAX;
+    m->slot_start[i] = i <= n ? int32_t(t->slot_start[i]) : INT32_MAX;
   }
   for (int p = 0; p < n; p++) {
     m->ptr[p] = ptrs[p];
@@ -199,6 +205,7 @@ int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, L
   if (e != hipSuccess) return int(e);
   m->offsets = t->d_offsets;
   m->tiles = t->d_tiles;
+  m->slots = t->d_slots;
   m->ptrs = reinterpret_cast<const void* const*>(t->d_stage[s]);
   m->modes_ = reinterpret_cast<const uint32_t*>(t->d_stage[s] + size_t(n) * sizeof(void*));
   m->n_tensors = n;
@@ -266,6 +273,7 @@ int yafsdp_binding_create(yafsdp_table* table, const void* const* tensor_ptrs, c
     }
     b->large.offsets = table->d_offsets;
     b->large.tiles = table->d_tiles;
+    b->large.slots = table->d_slots;
     b->large.ptrs = reinterpret_cast<const void* const*>(b->d_arrays);
     b->large.modes_ = reinterpret_cast<const uint32_t*>(b->d_arrays + size_t(n) * sizeof(void*));
     b->large.n_tensors = n;
@@ -317,12 +325,12 @@ int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat
   if (e != hipSuccess) return int(e);
   if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table->n_slots, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax)
     return int(launch_scatter<SmallMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->small, flat,
-                                         table->total, table->n_tiles, grid, s));
+                                         table->total, table->n_slots, grid, s));
   return int(launch_scatter<LargeMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->large, flat,
-                                       table->total, table->n_tiles, grid, s));
+                                       table->total, table->n_slots, grid, s));
 }
 
 int yafsdp_time_next_launch(void* start_event, void* stop_event) {
@@ -625,6 +633,27 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
       if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_tiles), tiles.size() * sizeof(TileRec))) != hipSuccess) break;
       if ((e = hipMemcpy(t->d_tiles, tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
     }
+    // scatter-out tile slots
+    t->slot_start.assign(size_t(n_tensors) + 1, 0);
+    for (int p = 0; p < n_tensors; p++) {
+      const int64_t n = t->offsets[p + 1] - t->offsets[p];
+      t->slot_start[p + 1] = t->slot_start[p] + (n > 0 ? (n + t->tile_elems - 1) / t->tile_elems + 1 : 0);
+    }
+    if (t->slot_start[n_tensors] > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    t->n_slots = int32_t(t->slot_start[n_tensors]);
+    if (n_tensors > kSmallMax && t->n_slots > 0) {
+      tiles.resize(size_t(t->n_slots));
+      for (int p = 0; p < n_tensors; p++) {
+        for (int64_t k = t->slot_start[p]; k < t->slot_start[p + 1]; k++) {
+          TileRec& r = tiles[size_t(k)];
+          r.first = p;
+          r.full = 0;
+          r.delta = k - t->slot_start[p];
+        }
+      }
+      if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_slots), tiles.size() * sizeof(TileRec))) != hipSuccess) break;
+      if ((e = hipMemcpy(t->d_slots, tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
+    }
     if (n_tensors > kSmallMax) {
       t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
       for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
@@ -715,7 +744,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   const void* const* ptrs = const_cast<const void* const*>(tensor_ptrs);
   int rc = check_dyn(table, ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
-  const int n_tiles = table->n_tiles;
+  const int n_tiles = table->n_slots;
   const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax) {
     SmallMeta meta;

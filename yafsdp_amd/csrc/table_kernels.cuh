@@ -15,6 +15,16 @@
 // each segment peels up to 7 elements on either end so that its unit loop is
 // again aligned on the flat side.
 //
+// Scatter-out tiles the DESTINATION instead: tile j of tensor p covers the
+// elements of p between two consecutive multiples of the tile size counted from
+// the 128-byte line that holds the tensor's first element, so no two workgroups
+// ever write the same cache line and every 16-byte store is aligned; the flat
+// side is then read at whatever alignment results (unaligned loads are nearly
+// free, unaligned stores and shared lines are not).  Every non-empty tensor owns
+// ceil(numel / tile) + 1 tile slots, whatever its address (the last slot is
+// empty when the tensor starts on a line boundary), so the slot table does not
+// depend on the per-call pointers.
+//
 // Metadata reaches a workgroup through scalar loads only (one tile is one
 // wave-uniform lookup), by one of two routes:
 //  * SmallMeta (up to kSmallMax tensors, e.g. one decoder layer): tensor
@@ -47,14 +57,30 @@ struct TileLookup {
   int64_t delta;
 };
 
+struct ScatterLookup {
+  int tensor;   // n_tensors or more: nothing to do
+  int index;    // tile slot inside the tensor
+};
+
 #define YAFSDP_CONST_AS __attribute__((address_space(4)))
 
 struct SmallMeta {
   const void* ptr[kSmallMax];
   int64_t off[kSmallMax + 1];         // prefix offsets; entries past n_tensors repeat the total
   int32_t tile_start[kSmallMax + 1];  // ceil(off[i] / tile elements); INT32_MAX past n_tensors
+  int32_t slot_start[kSmallMax + 1];  // scatter-out: first tile slot of tensor i; INT32_MAX past n_tensors
   uint32_t modes;                     // 2 bits per tensor
   int32_t n_tensors;
+
+  __device__ __forceinline__ ScatterLookup lookup_scatter(int tile) const {
+    int p = 0;
+#pragma unroll
+    for (int i = 1; i <= kSmallMax; i++) p += (slot_start[i] <= tile) ? 1 : 0;
+    ScatterLookup r;
+    r.tensor = p;
+    r.index = tile - slot_start[p < kSmallMax ? p : kSmallMax - 1];
+    return r;
+  }
 
   __device__ __forceinline__ TileLookup lookup(int tile, int64_t t0, int64_t tile_elems) const {
     int p = 0;
@@ -75,7 +101,8 @@ struct SmallMeta {
 
 struct LargeMeta {
   const int64_t* offsets;    // n_tensors + 1 prefix offsets (elements)
-  const TileRec* tiles;      // n_tiles records
+  const TileRec* tiles;      // n_tiles records (gather-in: tiles of the flat buffer)
+  const TileRec* slots;      // scatter-out tile slots: first = tensor, delta = slot index inside it
   const void* const* ptrs;   // n_tensors device pointers (per call)
   const uint32_t* modes_;    // n_tensors modes (per call)
   int32_t n_tensors;
@@ -87,6 +114,14 @@ struct LargeMeta {
     r.first = t[tile].first;
     r.full = t[tile].full != 0;
     r.delta = t[tile].delta;
+    return r;
+  }
+  __device__ __forceinline__ ScatterLookup lookup_scatter(int tile) const {
+    typedef const TileRec YAFSDP_CONST_AS* cptr;
+    const cptr t = (cptr)(uintptr_t)slots;
+    ScatterLookup r;
+    r.tensor = t[tile].first;
+    r.index = int(t[tile].delta);
     return r;
   }
   __device__ __forceinline__ const void* tensor(int p) const {
@@ -264,13 +299,11 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
 }
 
 // ---------------------------------------------------------------- scatter-out --
-// One full tile of the flat buffer (src, 16-byte aligned) into a tensor (dst, at
-// whatever element-aligned address the ragged offset gives).  Measured on a
-// 1427-tensor table with odd offsets: these unaligned stores cost 13 % against
-// the aligned case (reads at the same offsets cost 1 %); shifting the tile so
-// that stores are aligned and loads are not gains only 2 %, because what hurts
-// is the cache line shared by two tiles at every tile boundary, not the access
-// width - so the plain form is kept.
+// One full tile: dst (tensor side) starts on a 128-byte line, src (flat side)
+// sits at whatever element-aligned address results.  (Tiling the flat side
+// instead and storing at odd tensor offsets measured 13 % slower on a
+// 1427-tensor table: two workgroups then share the cache line at every tile
+// boundary.  Loads at odd offsets cost about 1 %.)
 template <class S, class D, int BLOCK, int U, bool NTL, bool NTS>
 __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
   if constexpr (wide_pair<S, D>::value) {
@@ -292,10 +325,12 @@ __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
     store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE_NONE, false>(s[j], unused, 0.f));
 }
 
+// n elements (fewer than a tile): up to 7 leading elements bring dst to a
+// 16-byte boundary, then whole units, then the tail.
 template <class S, class D, int BLOCK, bool NTL, bool NTS>
-__device__ __forceinline__ void scatter_segment(char* dst, const char* src, int64_t n, int64_t flat_index) {
+__device__ __forceinline__ void scatter_segment(char* dst, const char* src, int64_t n) {
   const int tid = threadIdx.x;
-  int64_t head = (8 - (flat_index & 7)) & 7;
+  int64_t head = ((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / D::kSize;
   if (head > n) head = n;
   const int64_t units = (n - head) >> 3;
   const int64_t body_end = head + (units << 3);
@@ -312,39 +347,33 @@ __device__ __forceinline__ void scatter_segment(char* dst, const char* src, int6
   }
 }
 
-// S: flat buffer dtype, D: tensor dtype.  Tensors with mode 0 are not written.
+// S: flat buffer dtype, D: tensor dtype.  Tensors with mode 0 are not written;
+// pad lanes of the flat buffer are never read.  n_tiles counts tile slots.
 template <class META, class S, class D, int BLOCK, int U, bool NTL, bool NTS>
 __global__ void __launch_bounds__(BLOCK)
 scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
+  constexpr int64_t kLineElems = 128 / D::kSize;
   const char* fbase = reinterpret_cast<const char*>(flat);
+  (void)total;
   for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-    const int64_t t0 = int64_t(tile) * kTile;
-    if (t0 >= total) break;  // pad lanes are never read
-    const int64_t t1 = (t0 + kTile < total) ? t0 + kTile : total;
-    const TileLookup rec = meta.lookup(tile, t0, kTile);
-    int p = rec.first;
+    const ScatterLookup rec = meta.lookup_scatter(tile);
+    const int p = rec.tensor;
     if (p >= meta.n_tensors) continue;
-    if (rec.full) {
-      if (meta.mode(p) != MODE_SKIP) {
-        char* dst = reinterpret_cast<char*>(const_cast<void*>(meta.tensor(p))) + rec.delta * D::kSize;
-        scatter_full_tile<S, D, BLOCK, U, NTL, NTS>(dst, fbase + t0 * S::kSize);
-      }
-      continue;
-    }
-    int64_t pos = t0;
-    while (pos < t1 && p < meta.n_tensors) {
-      const int64_t o1 = meta.offset(p + 1);
-      if (o1 <= pos) { ++p; continue; }
-      const int64_t o0 = meta.offset(p);
-      const int64_t e = o1 < t1 ? o1 : t1;
-      if (meta.mode(p) != MODE_SKIP) {
-        char* dst = reinterpret_cast<char*>(const_cast<void*>(meta.tensor(p))) + (pos - o0) * D::kSize;
-        scatter_segment<S, D, BLOCK, NTL, NTS>(dst, fbase + pos * S::kSize, e - pos, pos);
-      }
-      pos = e;
-      if (e == o1) ++p;
-    }
+    if (meta.mode(p) == MODE_SKIP) continue;
+    const int64_t o0 = meta.offset(p);
+    const int64_t n = meta.offset(p + 1) - o0;
+    char* tbase = reinterpret_cast<char*>(const_cast<void*>(meta.tensor(p)));
+    // elements between the start of the tensor's first cache line and the tensor
+    const int64_t lead = int64_t((reinterpret_cast<uintptr_t>(tbase) / D::kSize) & uintptr_t(kLineElems - 1));
+    const int64_t start = int64_t(rec.index) * kTile - lead;
+    const int64_t lo = start > 0 ? start : 0;
+    const int64_t hi = start + kTile < n ? start + kTile : n;
+    if (lo >= hi) continue;
+    char* dst = tbase + lo * D::kSize;
+    const char* src = fbase + (o0 + lo) * S::kSize;
+    if (hi - lo == kTile) scatter_full_tile<S, D, BLOCK, U, NTL, NTS>(dst, src);
+    else scatter_segment<S, D, BLOCK, NTL, NTS>(dst, src, hi - lo);
   }
 }
 
