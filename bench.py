@@ -478,6 +478,158 @@ def run_optim(args) -> int:
     return 0
 
 
+def run_exchange(args) -> int:
+    """The two exchange points of the path as one-GPU kernels over W local buffers: the copy-in cast written to
+    this rank's slot of W gathered buffers (direct all-gather, sender side) and the reduce over this rank's chunk
+    of W reduce buffers fused with post-divide and accumulation (direct reduce-scatter, receiver side)."""
+    import torch
+
+    from oracle import torch_ops
+    from yafsdp_amd import _native
+    from yafsdp_amd._layout import make_layout
+
+    base = args.workload[: -len("-exchange")]
+    shapes, w, r, align, seed = WORKLOADS[base]
+    if w > 16:
+        log(f"bench.py: the fan kernels take at most 16 buffers; {base} has W={w}")
+        return 2
+    lay = make_layout([numel_of(s) for s in shapes], w, align)
+    s = lay.padded_sharded_numel
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    log(f"workload {args.workload}: shard S={s}, W={w} buffers on one GPU")
+    g = torch.Generator().manual_seed(seed + 200)
+    master = torch.randn(s, generator=g) * 0.02
+    chunks = [(torch.randn(s, generator=g) * 1e-3).bfloat16() for _ in range(w)]
+    shard0 = torch.randn(s, generator=g) * 1e-4
+    d_master = master.to(dev)
+    d_slots = [torch.zeros(s, dtype=torch.bfloat16, device=dev) for _ in range(w)]
+    d_chunks = [c.to(dev) for c in chunks]
+    d_shard = shard0.to(dev)
+    post = float(w)
+
+    def op_fanout():
+        _native.flat_copy_fanout(d_slots, d_master)
+
+    def op_fanin():
+        _native.post_reduce_fanin(d_shard, d_chunks, post, True)
+
+    ops = [("copy_in_fanout", op_fanout, s * (4 + 2 * w)), ("reduce_fanin", op_fanin, s * (2 * w + 4 + 4))]
+    bytes_per_step = sum(b for _, _, b in ops)
+
+    parity = "skipped"
+    if not args.no_parity:
+        op_fanout()
+        op_fanin()
+        torch.cuda.synchronize()
+        want_slot = torch.zeros(s, dtype=torch.bfloat16)
+        torch_ops.copy_in_fanout([want_slot], master)
+        want_shard = shard0.clone()
+        torch_ops.reduce_scatter_fanin(want_shard, chunks, post, True)
+        ok = all(torch.equal(x.cpu().view(torch.int16), want_slot.view(torch.int16)) for x in d_slots)
+        ok = ok and torch.equal(d_shard.cpu().view(torch.int32), want_shard.view(torch.int32))
+        parity = "bit-exact" if ok else "MISMATCH"
+        log("parity vs oracle:", parity)
+        if not ok:
+            log("bench.py: GPU results differ from the oracle; refusing to report a throughput.")
+            return 4
+
+    for _ in range(args.warmup):
+        for _, fn, _ in ops:
+            fn()
+    torch.cuda.synchronize()
+    sampled = [k for k in range(args.steps) if k % 4 == 0]
+    ev = {k: _event_pair() for k in sampled}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        op_fanout()
+        if k in ev:
+            _native.time_next_launch(*ev[k])
+        op_fanin()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = bytes_per_step * args.steps / elapsed / 1e9
+    dom_us = [a.elapsed_time(b) * 1e3 for a, b in ev.values()]
+    dom_avg_us = sum(dom_us) / len(dom_us)
+    dom_bytes = ops[1][2]
+    achieved = dom_bytes / dom_avg_us / 1e3
+
+    kernels = {}
+    for name, fn, nbytes in ops:
+        times = []
+        for _ in range(20):
+            a, b = _event_pair()
+            for n2, f, _ in ops:
+                if n2 != name:
+                    f()
+            _native.time_next_launch(a, b)
+            fn()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b) * 1e3)
+        med = statistics.median(times)
+        kernels[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
+                         "GBps": round(nbytes / med / 1e3, 1), "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+        log(f"  {name:15s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s "
+            f"({100 * nbytes / med / 1e3 / HBM_PEAK_GBS:.1f}% of peak)")
+
+    def torch_step(slots, shard, cks, src):
+        torch_ops.copy_in_fanout(slots, src)
+        torch_ops.reduce_scatter_fanin(shard, cks, post, True)
+
+    cpu_baseline = None
+    if args.cpu_seconds > 0:
+        c_slots = [torch.zeros(s, dtype=torch.bfloat16) for _ in range(w)]
+        c_shard = shard0.clone()
+        times, spent = [], 0.0
+        while spent < args.cpu_seconds and len(times) < 500:
+            c0 = time.perf_counter()
+            torch_step(c_slots, c_shard, chunks, master)
+            dt = time.perf_counter() - c0
+            times.append(dt)
+            spent += dt
+        med = statistics.median(times)
+        cpu_baseline = {"value": round(bytes_per_step / med / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
+                        "kind": "port",
+                        "sample": f"{len(times)} passes of the same two steps with torch ops on CPU tensors (W copy_ calls; "
+                                  f"fp32 sum of W chunks, cast, div_, add_), median, {spent:.1f}s total"}
+        log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads ({len(times)} passes)")
+    torch_gpu = None
+    if not args.no_torch_gpu:
+        g_slots = [torch.zeros(s, dtype=torch.bfloat16, device=dev) for _ in range(w)]
+        g_shard = shard0.to(dev)
+        for _ in range(3):
+            torch_step(g_slots, g_shard, d_chunks, d_master)
+        torch.cuda.synchronize()
+        reps = 20
+        c0 = time.perf_counter()
+        for _ in range(reps):
+            torch_step(g_slots, g_shard, d_chunks, d_master)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - c0) / reps
+        torch_gpu = {"value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
+                     "sample": f"{reps} passes of the same torch ops on device tensors with torch {torch.__version__}, "
+                               f"rated with the fused passes' bytes"}
+        log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
+
+    out = {
+        "metric": "HBM GB/s + % of peak for the exchange-point kernels (copy-in fan-out, reduce fan-in) over W local buffers",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "shard_numel": s, "buffers": w, "rank": r, "bytes_per_step": bytes_per_step,
+                   "ops": "fp32 master shard [S] -> bf16 into W buffers; W bf16 chunks [S] summed in fp32, /W, += fp32 shard"},
+        "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "parity": parity,
+        "roofline": {"bound": "hbm", "kernel": "fanin_kernel (reduce fan-in)", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2), "launches_timed": len(dom_us)},
+        "cpu_baseline": cpu_baseline, "torch_gpu_baseline": torch_gpu, "kernels": kernels,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -486,7 +638,7 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3-8b-layer-w8",
                     choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256", "ragged-stress-w256-bf16-masters",
                                                  "llama3-8b-layer-w8-optim",
-                                                 "llama3-70b-layer-w64-optim"])
+                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
     ap.add_argument("--no-torch-gpu", action="store_true",
@@ -513,6 +665,8 @@ def main() -> int:
         return run_full_model(args)
     if args.workload.endswith("-optim"):
         return run_optim(args)
+    if args.workload.endswith("-exchange"):
+        return run_exchange(args)
     from yafsdp_amd import _native
     from yafsdp_amd._layout import make_layout
 

@@ -137,6 +137,30 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
 int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
                        const uint8_t* mode, int tensor_dtype, void* stream);
 
+/* ---- the two exchange points, over several buffers ------------------------------
+ * One GPU: all buffers are local.  With peer-mapped pointers the same two calls
+ * are the direct (non-ring) forms of the all-gather and the reduce-scatter; no
+ * inter-GPU code is part of this library.  All buffers 16-byte aligned; at most
+ * 16 destinations / sources. */
+
+/* dst_k[0:n] = cast(src[0:n]) for every k < n_dst: the copy-in cast
+ * (ya_fsdp/_collectives.py:53-54) written straight to this rank's slot of several
+ * gathered buffers, i.e. the cast plus the placement that
+ * all_gather_into_tensor performs (:60-65), reading the master shard once. */
+int yafsdp_flat_copy_fanout(void* const* dsts, int n_dst, int dst_dtype, const void* src, int src_dtype, int64_t n,
+                            void* stream);
+
+/* The reduce-scatter result and what follows it, from the ranks' reduce buffers:
+ *   sum   = chunk_0 + chunk_1 + ... in binary32, in index order (the binary32
+ *           accumulation the reference asks of its collective with
+ *           bit32_acc_for_bit16_reduce_scatter, ya_fsdp/_collectives.py:157-161)
+ *   out   = round(sum) to the chunk dtype        (the collective's output tensor)
+ *   out   = _div_if_needed(out, post_factor)     (:165)
+ *   shard = out or shard + out                   (:185 / :189)
+ * chunk_k is this rank's chunk of rank k's reduce buffer. */
+int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* chunks, int n_src, int chunk_dtype,
+                             int64_t n, double post_factor, int accumulate, void* stream);
+
 /* The tensor side of a table fixed for many calls.  The reference's unsharded
  * parameters and gradient accumulators are views of pre-allocated buffers that
  * live as long as the group (ya_fsdp/_param_group.py:409-457), and consumers of

@@ -254,3 +254,35 @@ def legacy_narrow_backward(grad_buffer: torch.Tensor, offset: int, grad_output: 
         view.copy_(grad_output.reshape(-1))
     else:
         view.add_(grad_output.reshape(-1))
+
+
+# ---------------------------------------------------------------------------
+# the two exchange points over several buffers (one GPU: all local)
+# ---------------------------------------------------------------------------
+def copy_in_fanout(dsts: Sequence[torch.Tensor], padded_sharded_param_data: torch.Tensor) -> None:
+    """The copy-in cast (ya_fsdp/_collectives.py:53-54) landing in this rank's slot of
+    several gathered buffers, which is where ``all_gather_into_tensor`` puts it
+    (:60-65)."""
+    for d in dsts:
+        d.copy_(padded_sharded_param_data)
+
+
+def reduce_scatter_fanin(
+    padded_sharded_param_grad: torch.Tensor,
+    chunks: Sequence[torch.Tensor],
+    postdivide_factor: float | None,
+    accumulate: bool,
+) -> None:
+    """A reduce-scatter over the ranks' chunks with binary32 accumulation in rank
+    order (``acc_type=torch.float32``, ya_fsdp/_collectives.py:157-161) whose output
+    has the reduce dtype, then the post-divide (:165) and ``copy_`` / ``add_``
+    into the gradient shard (:185 / :189)."""
+    acc = chunks[0].to(torch.float32).clone()
+    for c in chunks[1:]:
+        acc.add_(c.to(torch.float32))
+    output_tensor = acc.to(chunks[0].dtype)
+    div_if_needed(output_tensor, postdivide_factor)
+    if accumulate:
+        padded_sharded_param_grad.add_(output_tensor)
+    else:
+        padded_sharded_param_grad.copy_(output_tensor)

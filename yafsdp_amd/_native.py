@@ -40,6 +40,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_table_info",
     "yafsdp_gather_in",
     "yafsdp_scatter_out",
+    "yafsdp_flat_copy_fanout",
+    "yafsdp_post_reduce_fanin",
     "yafsdp_binding_create",
     "yafsdp_binding_destroy",
     "yafsdp_gather_in_bound",
@@ -90,6 +92,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_gather_in.argtypes = [vp, vp, vp, i32, vp, i32, dbl, i32, vp]
     lib.yafsdp_scatter_out.restype = i32
     lib.yafsdp_scatter_out.argtypes = [vp, vp, i32, vp, vp, i32, vp]
+    lib.yafsdp_flat_copy_fanout.restype = i32
+    lib.yafsdp_flat_copy_fanout.argtypes = [vp, i32, i32, vp, i32, i64, vp]
+    lib.yafsdp_post_reduce_fanin.restype = i32
+    lib.yafsdp_post_reduce_fanin.argtypes = [vp, i32, vp, i32, i32, i64, dbl, i32, vp]
     lib.yafsdp_binding_create.restype = i32
     lib.yafsdp_binding_create.argtypes = [vp, vp, vp, i32, ctypes.POINTER(vp)]
     lib.yafsdp_binding_destroy.restype = i32
@@ -365,6 +371,46 @@ class TensorTable:
                 ),
                 "yafsdp_scatter_out",
             )
+
+
+def flat_copy_fanout(dsts: Sequence[torch.Tensor], src: torch.Tensor) -> None:
+    """``d.copy_(src)`` for every ``d`` in ``dsts`` in one pass over ``src`` (at most 16 destinations)."""
+    _flat_arg(src, "src")
+    if not dsts:
+        raise ValueError("at least one destination")
+    for d in dsts:
+        _flat_arg(d, "dst")
+        if d.numel() != src.numel() or d.dtype != dsts[0].dtype or d.device != src.device:
+            raise ValueError("destinations must match the source's size and device and share a dtype")
+    ptrs = (ctypes.c_void_p * len(dsts))(*[d.data_ptr() for d in dsts])
+    with torch.cuda.device(src.device):
+        _check(
+            lib.yafsdp_flat_copy_fanout(ptrs, len(dsts), _dt(dsts[0]), src.data_ptr(), _dt(src), src.numel(), _stream(src)),
+            "yafsdp_flat_copy_fanout",
+        )
+
+
+def post_reduce_fanin(
+    shard: torch.Tensor, chunks: Sequence[torch.Tensor], post_factor: float | None, accumulate: bool
+) -> None:
+    """``shard (+)= div(round(sum of chunks in float32))``: the reduce-scatter of the ranks' chunks, the
+    post-divide and the accumulation into the gradient shard in one pass (at most 16 chunks)."""
+    _flat_arg(shard, "shard")
+    if not chunks:
+        raise ValueError("at least one chunk")
+    for c in chunks:
+        _flat_arg(c, "chunk")
+        if c.numel() != shard.numel() or c.dtype != chunks[0].dtype or c.device != shard.device:
+            raise ValueError("chunks must match the shard's size and device and share a dtype")
+    ptrs = (ctypes.c_void_p * len(chunks))(*[c.data_ptr() for c in chunks])
+    with torch.cuda.device(shard.device):
+        _check(
+            lib.yafsdp_post_reduce_fanin(
+                shard.data_ptr(), _dt(shard), ptrs, len(chunks), _dt(chunks[0]), shard.numel(), _factor(post_factor),
+                int(bool(accumulate)), _stream(shard),
+            ),
+            "yafsdp_post_reduce_fanin",
+        )
 
 
 class TensorBinding:

@@ -398,6 +398,48 @@ uint32_t fill_pattern(int dtype, double value) {
 }
 }  // namespace
 
+int yafsdp_flat_copy_fanout(void* const* dsts, int n_dst, int dst_dtype, const void* src, int src_dtype, int64_t n,
+                            void* stream) {
+  if (!valid_dtype(dst_dtype) || !valid_dtype(src_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || n_dst < 1 || n_dst > kFanMax || dsts == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;
+  if (src == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(src, 16)) return YAFSDP_ERR_MISALIGNED;
+  FanPtrs ptrs;
+  std::memset(&ptrs, 0, sizeof(ptrs));
+  ptrs.n = n_dst;
+  for (int k = 0; k < n_dst; k++) {
+    if (dsts[k] == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+    if (!aligned_to(dsts[k], 16)) return YAFSDP_ERR_MISALIGNED;
+    ptrs.p[k] = dsts[k];
+  }
+  const int grid = opt_grid(n >> 3, kFanBlock, kFanOutUnroll, nullptr);
+  return int(launch_fanout(src_dtype, dst_dtype, ptrs, src, n, grid, static_cast<hipStream_t>(stream)));
+}
+
+int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* chunks, int n_src, int chunk_dtype,
+                             int64_t n, double post_factor, int accumulate, void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || n_src < 1 || n_src > kFanMax || chunks == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;
+  if (shard == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (!aligned_to(shard, 16)) return YAFSDP_ERR_MISALIGNED;
+  FanPtrs ptrs;
+  std::memset(&ptrs, 0, sizeof(ptrs));
+  ptrs.n = n_src;
+  for (int k = 0; k < n_src; k++) {
+    if (chunks[k] == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+    if (!aligned_to(chunks[k], 16)) return YAFSDP_ERR_MISALIGNED;
+    ptrs.p[k] = const_cast<void*>(chunks[k]);
+  }
+  int scale;
+  float k;
+  scale_plan(post_factor, &scale, &k);
+  const int grid = opt_grid(n >> 2, kFanBlock, kFanInUnroll, nullptr);
+  return int(launch_fanin(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, ptrs, n, k, grid,
+                          static_cast<hipStream_t>(stream)));
+}
+
 int yafsdp_flat_fill(void* dst, int dtype, int64_t n, double value, void* stream) {
   if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && dst == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;

@@ -44,6 +44,17 @@ template <class META>
 hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total,
                           int n_tiles, int grid, hipStream_t stream);
 
+// fan-out / fan-in over several buffers (fan.hip); all buffers 16-byte aligned
+constexpr int kFanMax = 16;
+struct FanPtrs {
+  void* p[kFanMax];
+  int n;
+};
+hipError_t launch_fanout(int src_dt, int dst_dt, const FanPtrs& dsts, const void* src, int64_t n, int grid,
+                         hipStream_t stream);
+hipError_t launch_fanin(int chunk_dt, int shard_dt, int scale, bool acc, void* shard, const FanPtrs& chunks, int64_t n,
+                        float k, int grid, hipStream_t stream);
+
 // optimizer-side passes (optim.hip); `head` leading elements bring the range to a 16-byte boundary
 // scalars of one Adam step, binary32 as they enter the tensor ops (see adamw_kernel)
 struct AdamScalars {

@@ -62,6 +62,23 @@ constexpr int kAdamBlock = YAFSDP_ADAM_BLOCK;
 constexpr int kAdamUnroll = YAFSDP_ADAM_U;
 constexpr bool kOptNtLoad = true;
 constexpr bool kOptNtStore = true;
+// fan-out / fan-in: a tile is block * unroll quads
+#ifndef YAFSDP_FAN_BLOCK
+#define YAFSDP_FAN_BLOCK 64
+#endif
+#ifndef YAFSDP_FANOUT_U
+#define YAFSDP_FANOUT_U 1
+#endif
+#ifndef YAFSDP_FANIN_U
+#define YAFSDP_FANIN_U 1
+#endif
+#ifndef YAFSDP_FAN_NTS
+#define YAFSDP_FAN_NTS true
+#endif
+constexpr bool kFanNtStore = YAFSDP_FAN_NTS;
+constexpr int kFanBlock = YAFSDP_FAN_BLOCK;
+constexpr int kFanOutUnroll = YAFSDP_FANOUT_U;
+constexpr int kFanInUnroll = YAFSDP_FANIN_U;
 // workgroups (= partial sums) of the sum-of-squares pass; the workspace holds one double each
 constexpr int kSumsqMaxPartials = 16384;
 // default grid cap in workgroups per compute unit.  Measured: one workgroup per
