@@ -4,8 +4,14 @@
 namespace yafsdp {
 // flat kernels: workgroup size, units (8 elements) per lane per tile,
 // non-temporal loads / stores
-constexpr int kFlatBlock = 256;
-constexpr int kFlatUnroll = 2;
+#ifndef YAFSDP_FLAT_BLOCK
+#define YAFSDP_FLAT_BLOCK 256
+#endif
+#ifndef YAFSDP_FLAT_U
+#define YAFSDP_FLAT_U 2
+#endif
+constexpr int kFlatBlock = YAFSDP_FLAT_BLOCK;
+constexpr int kFlatUnroll = YAFSDP_FLAT_U;
 constexpr bool kFlatNtLoad = true;
 constexpr bool kFlatNtStore = true;
 // gather-in / scatter-out: a tile is block * unroll * 8 elements.  Measured with
