@@ -9,8 +9,10 @@ fallback.
 =====================================================  =========================
 reference op                                           here
 =====================================================  =========================
-``all_gather_input.copy_(shard)`` (:53-54)             ``flat_copy``
-``all_gather_output.copy_(all_gather_input)`` (:56-58)  ``flat_copy``
+``all_gather_input.copy_(shard)`` (:53-54)             ``flat_copy_fanout`` (cast
+``all_gather_output.copy_(all_gather_input)`` (:56-58)  and placement in one pass
+                                                        over the shard), or
+                                                        ``flat_copy`` each
 ``_div_if_needed(rs_input, pre)`` (:139)               fused into the reduce
                                                         copy-in launch, or
                                                         ``flat_div``
@@ -85,22 +87,27 @@ def all_gather(
             # the 16-bit copy is stale, cast again
             param_group._all_gather_input_set_dtypes.discard(all_gather_dtype)
         param_group._copy_in_shard_version = None
+        world_size = all_gather_group.size()
+        shard_numel = all_gather_input.numel()
+        rank = all_gather_group.rank()
+        slot = all_gather_output if world_size == 1 else all_gather_output[rank * shard_numel : (rank + 1) * shard_numel]
+        placed = False
         if all_gather_dtype not in param_group._all_gather_input_set_dtypes:
             for fsdp_param in fsdp_params:
                 fsdp_param.set_all_gather_input()
             if all_gather_dtype is None and param_dtype is not None:
-                # copy-in: cast the master shard (:53-54); the version counter of
-                # the destination is untouched because no autograd op is involved
-                _native.flat_copy(all_gather_input, padded_sharded_param_data)
+                # copy-in: cast the master shard (:53-54) and, in the same pass over it, place the result where
+                # the all-gather would (:56-58, :60-65); the version counter of the destination is untouched
+                # because no autograd op is involved
+                if all(t.data_ptr() % 16 == 0 for t in (slot, all_gather_input, padded_sharded_param_data)):
+                    _native.flat_copy_fanout([all_gather_input, slot], padded_sharded_param_data)
+                    placed = True
+                else:
+                    _native.flat_copy(all_gather_input, padded_sharded_param_data)
             param_group._all_gather_input_set_dtypes.add(all_gather_dtype)
-        world_size = all_gather_group.size()
-        if world_size == 1:
-            _native.flat_copy(all_gather_output, all_gather_input)  # :56-58
-        else:
-            # this rank's share of all_gather_into_tensor (:60-65)
-            shard_numel = all_gather_input.numel()
-            rank = all_gather_group.rank()
-            _native.flat_copy(all_gather_output[rank * shard_numel : (rank + 1) * shard_numel], all_gather_input)
+        if not placed:
+            # size-1 group (:56-58), or this rank's share of all_gather_into_tensor (:60-65)
+            _native.flat_copy(slot, all_gather_input)
         all_gather_work = None
         all_gather_event = all_gather_stream.record_event()
     return AllGatherResult(all_gather_event, all_gather_work)
