@@ -123,6 +123,8 @@ def test_sharded_llama_trains_like_the_unsharded_model():
         opt.zero_grad(set_to_none=True)
         losses.append(loss.item())
 
+    print("loss first/last:", losses[0], losses[-1], "reference:", ref_losses[0], ref_losses[-1],
+          "max relative gap:", max(abs(a - b) / max(abs(b), 1.0) for a, b in zip(losses, ref_losses)), flush=True)
     assert all(math.isfinite(x) for x in losses)
     assert losses[0] > 5.0 and losses[-1] < 0.5 * losses[0], (losses[0], losses[-1])
     assert abs(losses[0] - ref_losses[0]) < 1e-2
