@@ -641,6 +641,8 @@ def main() -> int:
                                                  "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the leg that replays the step from a HIP graph (outside the timed region)")
     ap.add_argument("--no-torch-gpu", action="store_true",
                     help="skip the leg that times the reference's torch ops on the GPU (outside the timed region)")
     ap.add_argument("--sweep-grid-cap", action="store_true",
@@ -814,6 +816,41 @@ def main() -> int:
     dom_bytes = ops[dom_index][2]
     achieved = dom_bytes / dom_avg_us / 1e3
 
+    # ---- the same step captured into a HIP graph and replayed (outside the timed region): both sides of the table
+    # are bound, so the captured launches carry no per-call host work and no staging copy
+    graph_replay = None
+    if not args.no_graph:
+        grad_binding = table.bind(d_grads)
+
+        def bound_step():
+            if has_copy_in:
+                _native.flat_copy(d_ag_in, d_master)
+            out_binding.scatter_out(d_gathered)
+            grad_binding.gather_in(d_rs, pre, True)
+            _native.post_reduce(d_shard, d_chunk, None, True)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            bound_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            bound_step()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        g0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        g_dt = (time.perf_counter() - g0) / args.steps
+        graph_replay = {"ms_per_step": round(g_dt * 1e3, 4), "value": round(bytes_per_step / g_dt / 1e9, 1), "unit": "GB/s"}
+        log(f"HIP graph replay of the step: {graph_replay['ms_per_step']} ms, {graph_replay['value']} GB/s")
+        del graph
+        grad_binding.close()
+
     # ---- per-kernel table (outside the timed region): each op's dispatch timed on its own
     kernels = {}
     for name, fn, nbytes in ops:
@@ -936,6 +973,7 @@ def main() -> int:
         },
         "cpu_baseline": cpu_baseline,
         "torch_gpu_baseline": torch_gpu,
+        "graph_replay": graph_replay,
         "kernels": kernels,
     }
     print(json.dumps(out), flush=True)
