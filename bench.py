@@ -820,36 +820,40 @@ def main() -> int:
     # are bound, so the captured launches carry no per-call host work and no staging copy
     graph_replay = None
     if not args.no_graph:
-        grad_binding = table.bind(d_grads)
+        try:
+            grad_binding = table.bind(d_grads)
 
-        def bound_step():
-            if has_copy_in:
-                _native.flat_copy(d_ag_in, d_master)
-            out_binding.scatter_out(d_gathered)
-            grad_binding.gather_in(d_rs, pre, True)
-            _native.post_reduce(d_shard, d_chunk, None, True)
+            def bound_step():
+                if has_copy_in:
+                    _native.flat_copy(d_ag_in, d_master)
+                out_binding.scatter_out(d_gathered)
+                grad_binding.gather_in(d_rs, pre, True)
+                _native.post_reduce(d_shard, d_chunk, None, True)
 
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            bound_step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            bound_step()
-        for _ in range(3):
-            graph.replay()
-        torch.cuda.synchronize()
-        g0 = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
-        torch.cuda.synchronize()
-        g_dt = (time.perf_counter() - g0) / args.steps
-        graph_replay = {"ms_per_step": round(g_dt * 1e3, 4), "value": round(bytes_per_step / g_dt / 1e9, 1), "unit": "GB/s"}
-        log(f"HIP graph replay of the step: {graph_replay['ms_per_step']} ms, {graph_replay['value']} GB/s")
-        del graph
-        grad_binding.close()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                bound_step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                bound_step()
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+            g0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            g_dt = (time.perf_counter() - g0) / args.steps
+            graph_replay = {"ms_per_step": round(g_dt * 1e3, 4), "value": round(bytes_per_step / g_dt / 1e9, 1), "unit": "GB/s"}
+            log(f"HIP graph replay of the step: {graph_replay['ms_per_step']} ms, {graph_replay['value']} GB/s")
+            del graph
+            grad_binding.close()
+        except Exception as exc:  # an optional leg must not cost the measurement above
+            log(f"HIP graph leg skipped: {type(exc).__name__}: {exc}")
+            graph_replay = None
 
     # ---- per-kernel table (outside the timed region): each op's dispatch timed on its own
     kernels = {}
@@ -908,38 +912,42 @@ def main() -> int:
     # hardware today.  Outside the timed region; reported next to the CPU baseline, not a target.
     torch_gpu = None
     if cpu_state is not None and not args.no_torch_gpu:
-        from oracle import torch_ops  # noqa: F811
+        try:
+            from oracle import torch_ops  # noqa: F811
 
-        g_rs = torch.zeros(t_pad, dtype=rs_dt, device=dev)
-        g_state = {
-            "ag_in": torch.zeros(s, dtype=torch.bfloat16, device=dev),
-            "outs": [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels],
-            "rs": g_rs, "rs_views": list(g_rs[:t].split(numels)), "shard": shard0.to(dev),
-        }
+            g_rs = torch.zeros(t_pad, dtype=rs_dt, device=dev)
+            g_state = {
+                "ag_in": torch.zeros(s, dtype=torch.bfloat16, device=dev),
+                "outs": [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels],
+                "rs": g_rs, "rs_views": list(g_rs[:t].split(numels)), "shard": shard0.to(dev),
+            }
 
-        def gpu_torch_step(st):
-            if has_copy_in:
-                torch_ops.copy_in(st["ag_in"], d_master)
-            torch_ops.copy_out_materialize(d_gathered, numels, st["outs"])
-            torch_ops.reduce_copy_in(st["rs_views"], d_grads, False)
-            torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
+            def gpu_torch_step(st):
+                if has_copy_in:
+                    torch_ops.copy_in(st["ag_in"], d_master)
+                torch_ops.copy_out_materialize(d_gathered, numels, st["outs"])
+                torch_ops.reduce_copy_in(st["rs_views"], d_grads, False)
+                torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
 
-        for _ in range(3):
-            gpu_torch_step(g_state)
-        torch.cuda.synchronize()
-        reps = 20
-        c0 = time.perf_counter()
-        for _ in range(reps):
-            gpu_torch_step(g_state)
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - c0) / reps
-        torch_gpu = {
-            "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
-            "sample": f"{reps} passes of the reference's torch ops (copy_, split + copy_, _foreach_copy_, div_, add_) on "
-                      f"device tensors with torch {torch.__version__}, same inputs, rated with the same algorithmic bytes",
-        }
-        log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
-        del g_state, g_rs
+            for _ in range(3):
+                gpu_torch_step(g_state)
+            torch.cuda.synchronize()
+            reps = 20
+            c0 = time.perf_counter()
+            for _ in range(reps):
+                gpu_torch_step(g_state)
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - c0) / reps
+            torch_gpu = {
+                "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
+                "sample": f"{reps} passes of the reference's torch ops (copy_, split + copy_, _foreach_copy_, div_, add_) on "
+                          f"device tensors with torch {torch.__version__}, same inputs, rated with the same algorithmic bytes",
+            }
+            log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
+            del g_state, g_rs
+        except Exception as exc:  # an optional leg must not cost the measurement above
+            log(f"torch-on-GPU leg skipped: {type(exc).__name__}: {exc}")
+            torch_gpu = None
 
     out = {
         "metric": "HBM GB/s + % of peak for copy-in/out+grad-reduce, Llama-3-8B layer @W=8",
