@@ -1,0 +1,46 @@
+"""Host-side helpers that need no GPU."""
+
+import torch.nn as nn
+
+
+def test_merge_joins_adjacent_ranges_only():
+    from yafsdp_amd.optim import _merge
+
+    assert _merge([]) == []
+    assert _merge([(5, 9), (0, 5), (9, 9), (12, 20)]) == [(0, 9), (12, 20)]
+    assert _merge([(3, 3)]) == []
+    assert _merge([(0, 4), (6, 8), (4, 6)]) == [(0, 8)]
+
+
+def test_root_modules_of_a_list():
+    from yafsdp_amd.fully_shard import _get_root_modules
+
+    a = nn.Sequential(nn.Linear(2, 2), nn.Linear(2, 2))
+    b = nn.Linear(2, 2)
+    assert _get_root_modules([a, b]) == [a, b]
+    assert _get_root_modules([a[0], a, b, a[1]]) == [a, b]  # members of `a` are dropped
+    assert _get_root_modules([b, b]) == [b]
+
+
+def test_param_names_of_a_module_list():
+    from yafsdp_amd.fully_shard import _param_names
+
+    a, b = nn.Linear(2, 2), nn.Linear(2, 2, bias=False)
+    assert _param_names((a,), list(a.parameters())) == ["weight", "bias"]
+    assert _param_names((a, b), [b.weight, a.bias]) == ["1.weight", "0.bias"]
+
+
+def test_flat_adamw_rejects_bad_hyperparameters():
+    import pytest
+    import torch
+
+    from yafsdp_amd.optim import FlatAdamW
+
+    p = [nn.Parameter(torch.zeros(4))]
+    for kw in (dict(lr=-1.0), dict(eps=-1e-8), dict(betas=(1.0, 0.9)), dict(weight_decay=-0.1)):
+        with pytest.raises(ValueError):
+            FlatAdamW(p, **kw)
+    opt = FlatAdamW(p, lr=1e-3)  # construction needs no GPU; stepping a CPU parameter does
+    p[0].grad = torch.zeros(4)
+    with pytest.raises(TypeError):
+        opt.step()
