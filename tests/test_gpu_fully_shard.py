@@ -50,9 +50,9 @@ def _wrap(model, **kw):
     return fully_shard(model, **kw)  # the root holds no parameters of its own: siblings only
 
 
-def _reference_steps(model0, xs, lr, accumulate_pairs=False):
-    """fp32 masters; bf16 compute copies; bf16 gradients (summed in bf16 over the micro-batches of a step, as
-    the reduce buffer does) upcast into fp32; SGD on the masters."""
+def _reference_steps(model0, xs, lr, accumulate_pairs=False, reduce_fp32=False):
+    """fp32 masters; bf16 compute copies; bf16 gradients (summed over the micro-batches of a step in the dtype of
+    the reduce buffer: bf16, or fp32 with ``reduce_dtype=torch.float32``) upcast into fp32; SGD on the masters."""
     ref = copy.deepcopy(model0)
     masters = [p for p in ref.parameters()]
     opt = torch.optim.SGD(masters, lr=lr)
@@ -63,7 +63,7 @@ def _reference_steps(model0, xs, lr, accumulate_pairs=False):
             lowp = copy.deepcopy(ref).to(torch.bfloat16)
             y = lowp(x.to(torch.bfloat16))
             y.float().pow(2).mean().backward()
-            grads = [p.grad for p in lowp.parameters()]
+            grads = [p.grad.float() if reduce_fp32 else p.grad for p in lowp.parameters()]
             if acc is None:
                 acc = [g.clone() for g in grads]          # view.copy_(grad)
             else:
@@ -137,6 +137,33 @@ def test_gradient_accumulation_without_sync():
     torch.cuda.synchronize()
     got, want = _gather_full(model), dict(ref.named_parameters())
     assert set(got) == set(want)
+    for k in want:
+        assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
+
+
+def test_fp32_reduce_buffer_with_accumulation():
+    """param_dtype=bf16, reduce_dtype=fp32: gradients are upcast on their way into the reduce buffer and the
+    micro-batches of a step add up in fp32 there."""
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.float32, cast_forward_inputs=True)
+    model0 = _make(6)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(70 + s)) for s in range(4)]
+    ref = _reference_steps(model0, xs, lr=0.02, accumulate_pairs=True, reduce_fp32=True)
+    model = _wrap(copy.deepcopy(model0), mp_policy=mp)
+    opt = torch.optim.SGD(model.parameters(), lr=0.02)
+    model._get_fsdp_state()._lazy_init(allow_no_grad_reduce=True)
+    for i in range(0, 4, 2):
+        model.set_requires_gradient_sync(False)
+        model.set_is_last_backward(False)
+        model(xs[i]).float().pow(2).mean().backward()
+        model.set_requires_gradient_sync(True)
+        model.set_is_last_backward(True)
+        model(xs[i + 1]).float().pow(2).mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    group = model.blocks[0]._get_fsdp_state()._fsdp_param_group
+    assert group.reduce_scatter_dtype == torch.float32 and group.all_gather_dtype == torch.bfloat16
+    got, want = _gather_full(model), dict(ref.named_parameters())
     for k in want:
         assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
 
