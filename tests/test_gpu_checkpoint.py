@@ -88,3 +88,41 @@ def test_load_casts_to_the_master_dtype_and_resets_the_copy_in_flag():
     assert_bits_equal(g._all_gather_input[None], g._padded_sharded_param_data[None].bfloat16(), "copy-in after load")
     with pytest.raises(KeyError):
         load_full_tensors(g, {})
+
+
+def test_full_state_dict_round_trip_through_the_unwrapped_model():
+    """Train a wrapped model, save a plain state dict, load it into (a) the unwrapped torch model and (b) a
+    freshly wrapped one: all three give the same outputs / masters."""
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.checkpoint import full_state_dict, load_full_state_dict
+
+    def wrap(m):
+        for b in m.blocks:
+            fully_shard(b, mp_policy=MP)
+        fully_shard(m.norm, mp_policy=MP)
+        return fully_shard(m, mp_policy=MP)
+
+    model0 = _make(24)
+    model = wrap(copy.deepcopy(model0))
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    x = torch.randn(8, 128, device=DEV)
+    for _ in range(2):
+        model(x).float().pow(2).mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    sd = full_state_dict(model)
+    plain = copy.deepcopy(model0)
+    plain.load_state_dict(sd)  # names and shapes are those of the unwrapped model
+    for k, v in plain.state_dict().items():
+        assert_bits_equal(v, sd[k], k)
+    fresh = wrap(copy.deepcopy(model0))
+    load_full_state_dict(fresh, sd)
+    y1, y2 = model(x), fresh(x)
+    assert_bits_equal(y2, y1.detach(), "outputs after reload")
+    for m in (fresh.blocks[2], fresh.norm):
+        m.reshard()  # a forward without a backward leaves the last users of the buffers unsharded
+    with pytest.raises(KeyError):
+        load_full_state_dict(fresh, {})
+    fresh.blocks[1].unshard()
+    with pytest.raises(RuntimeError, match="sharded state"):
+        full_state_dict(fresh)

@@ -101,6 +101,7 @@ class YaFSDPParam:
     ) -> None:
         unsharded_tensor = all_gather_output.view(self._orig_size)  # zero-copy copy-out
         self.unsharded_param = nn.Parameter(unsharded_tensor, requires_grad=self.requires_grad)
+        self.unsharded_param._yafsdp_param = weakref.ref(self)
         if self.requires_grad:
             assert reduce_scatter_input is not None
             self._unsharded_accumulated_grad = reduce_scatter_input.view(self._orig_size)

@@ -30,7 +30,8 @@ from . import _native
 from ._layout import RaggedShard
 from ._param_group import YaFSDPParamGroup
 
-__all__ = ["ChunkMeta", "chunk_meta", "sharded_state_dict", "group_meta_info", "full_tensors", "load_full_tensors"]
+__all__ = ["ChunkMeta", "chunk_meta", "sharded_state_dict", "group_meta_info", "full_tensors", "load_full_tensors",
+           "full_state_dict", "load_full_state_dict"]
 
 
 @dataclass(frozen=True)
@@ -151,3 +152,68 @@ def fsdp_groups_of(module: nn.Module) -> list[YaFSDPParamGroup]:
     from .optim import fsdp_param_groups
 
     return fsdp_param_groups(module)
+
+
+def _owners_by_name(module: nn.Module) -> dict[str, object]:
+    """``{root-relative parameter name: owning YaFSDPParam or the plain parameter}`` of a module whose
+    ``fully_shard`` groups are all in the sharded state."""
+    out = {}
+    for name, p in module.named_parameters(remove_duplicate=False):
+        ref = getattr(p, "_yafsdp_param", None)
+        owner = ref() if ref is not None else None
+        if owner is not None and owner.sharded_param is not p:
+            raise RuntimeError(f"{name} is not in the sharded state; call reshard() on its module first")
+        out[name] = owner if owner is not None else p
+    return out
+
+
+def full_state_dict(module: nn.Module) -> dict[str, torch.Tensor]:
+    """Parameters in their original shapes and master dtype (copies) plus buffers, for a module whose
+    groups all have world size 1 (one GPU holds every parameter whole): the ordinary ``state_dict`` of the
+    unwrapped model.  Larger logical world sizes go through ``full_tensors`` with the groups of all ranks."""
+    out: dict[str, torch.Tensor] = {}
+    for name, owner in _owners_by_name(module).items():
+        if isinstance(owner, torch.Tensor):
+            out[name] = owner.detach().clone()
+            continue
+        if owner.mesh_info.shard_mesh_size != 1:
+            raise ValueError(f"{name} is sharded over {owner.mesh_info.shard_mesh_size} logical ranks; use full_tensors")
+        out[name] = owner._sharded_param_data.detach().view(owner._orig_size).clone()
+    for name, b in module.named_buffers():
+        out[name] = b.detach().clone()
+    return out
+
+
+def load_full_state_dict(module: nn.Module, state_dict: Mapping[str, torch.Tensor], strict: bool = True) -> None:
+    """Loads full parameters (any logical world size: each rank keeps its fragment) and buffers by name."""
+    owners = _owners_by_name(module)
+    missing = [k for k in owners if k not in state_dict]
+    if strict and missing:
+        raise KeyError(f"missing keys: {missing}")
+    touched = set()
+    for name, owner in owners.items():
+        if name not in state_dict:
+            continue
+        src = state_dict[name]
+        if isinstance(owner, torch.Tensor):
+            with torch.no_grad():
+                owner.copy_(src)
+            continue
+        if src.numel() != owner._orig_size.numel():
+            raise ValueError(f"{name}: expected {owner._orig_size.numel()} elements, got {src.numel()}")
+        n, go = owner.placement.local_numel, owner.placement.global_offset
+        if n:
+            flat = src.detach().to(owner.device).contiguous().view(-1)
+            _native.flat_copy(owner._sharded_param_data, flat[go : go + n])
+        group = owner._param_group_ref()
+        if group is not None and id(group) not in touched:
+            touched.add(id(group))
+            group._all_gather_input_set_dtypes.clear()
+            group._copy_in_shard_version = None
+    buffers = dict(module.named_buffers())
+    for name, b in buffers.items():
+        if name in state_dict:
+            with torch.no_grad():
+                b.copy_(state_dict[name])
+        elif strict:
+            raise KeyError(f"missing buffer: {name}")
