@@ -630,6 +630,73 @@ def run_exchange(args) -> int:
     return 0
 
 
+def run_ceilings(args) -> int:
+    """What this chip's HBM gives streaming kernels of the library at the size of the headline buffer (one bf16
+    layer buffer, 436 MB): read-only (sum of squares), write-only (fill), 1:1 copy (same-dtype flat copy), and
+    torch's device-to-device copy_ for comparison.  Random data (all-zero buffers run faster on this memory)."""
+    import torch
+
+    from yafsdp_amd import _native
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    n = 218_112_000
+    g = torch.Generator(device=dev).manual_seed(7)
+    a = (torch.randn(n // 2, device=dev, generator=g) * 0.02).bfloat16().repeat(2)
+    b = torch.empty_like(a)
+    big = (torch.randn(n // 2, device=dev, generator=g)).bfloat16().repeat(2)  # evictor: another 436 MB
+    big2 = torch.empty_like(big)
+    out = torch.zeros(1, dtype=torch.float64, device=dev)
+    partials = torch.empty(_native.SUMSQ_MAX_PARTIALS, dtype=torch.float64, device=dev)
+    cases = [
+        ("read_only_sumsq_bf16", lambda: _native.sumsq_partials(a, partials, 0), n * 2),
+        ("write_only_fill_bf16", lambda: _native.flat_fill(b, 1.5), n * 2),
+        ("copy_bf16_to_bf16", lambda: _native.flat_copy(b, a), n * 4),
+        ("copy_f32_to_f32", lambda: _native.flat_copy(b.view(torch.float32), a.view(torch.float32)), n * 4),
+    ]
+    kernels = {}
+    for name, fn, nbytes in cases:
+        times = []
+        for _ in range(max(args.steps, 20)):
+            _native.flat_copy(big2, big)  # evict
+            x, y = _event_pair()
+            _native.time_next_launch(x, y)
+            fn()
+            torch.cuda.synchronize()
+            times.append(x.elapsed_time(y) * 1e3)
+        med = statistics.median(times)
+        kernels[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
+                         "GBps": round(nbytes / med / 1e3, 1), "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+        log(f"  {name:24s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s "
+            f"({100 * nbytes / med / 1e3 / HBM_PEAK_GBS:.1f}% of peak)")
+    times = []
+    for _ in range(20):  # torch's own device-to-device copy (a runtime blit kernel), bracketed by events
+        _native.flat_copy(big2, big)
+        x, y = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        x.record()
+        b.copy_(a)
+        y.record()
+        torch.cuda.synchronize()
+        times.append(x.elapsed_time(y) * 1e3)
+    med = statistics.median(times)
+    kernels["torch_copy_bf16"] = {"bytes": n * 4, "us_median": round(med, 2), "us_min": round(min(times), 2),
+                                  "GBps": round(n * 4 / med / 1e3, 1), "frac_of_peak": round(n * 4 / med / 1e3 / HBM_PEAK_GBS, 4)}
+    log(f"  {'torch_copy_bf16':24s} {n * 4 / 1e6:8.1f} MB  median {med:7.1f} us  {n * 4 / med / 1e3:7.1f} GB/s")
+    best = kernels["copy_bf16_to_bf16"]
+    out_line = {
+        "metric": "HBM GB/s of plain streaming kernels (read-only, write-only, 1:1 copy) at the headline buffer size",
+        "value": best["GBps"], "unit": "GB/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": 0,
+        "ms_per_step": round(best["us_median"] / 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "elements": n},
+        "roofline": {"bound": "hbm", "kernel": "flat_kernel (bf16 -> bf16 copy)", "achieved": best["GBps"],
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac_of_peak"], "traffic": None},
+        "cpu_baseline": None, "kernels": kernels,
+    }
+    print(json.dumps(out_line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -638,7 +705,7 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3-8b-layer-w8",
                     choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256", "ragged-stress-w256-bf16-masters",
                                                  "llama3-8b-layer-w8-optim",
-                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange"])
+                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange", "hbm-ceilings"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
     ap.add_argument("--no-graph", action="store_true",
@@ -669,6 +736,8 @@ def main() -> int:
         return run_optim(args)
     if args.workload.endswith("-exchange"):
         return run_exchange(args)
+    if args.workload == "hbm-ceilings":
+        return run_ceilings(args)
     from yafsdp_amd import _native
     from yafsdp_amd._layout import make_layout
 
