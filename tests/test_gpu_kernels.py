@@ -336,3 +336,32 @@ def test_time_next_launch_brackets_exactly_one_dispatch(nat):
     nat.flat_copy(dst, src)
     torch.cuda.synchronize()
     assert abs(a.elapsed_time(b) * 1e3 - attached) < 1e-6  # untouched by the disarmed launch
+
+
+def test_table_with_the_maximum_number_of_tensors(nat):
+    """65,534 tensors of 0-5 elements (the reference allows fewer than 65,535 parameters per group,
+    ya_fsdp/_param_group.py:284-287): almost every tile crosses many tensor boundaries."""
+    p = 65_534
+    rng = np.random.default_rng(9)
+    numels = rng.integers(0, 6, size=p).tolist()
+    t = sum(numels)
+    t_pad = t + 11
+    g = torch.Generator().manual_seed(150)
+    src = mixed_values(g, t, torch.bfloat16, 1e-3)
+    grads = list(src.split(numels))
+    old = mixed_values(g, t_pad, torch.float32, 1e-3)
+    want = old.clone()
+    torch_ops.reduce_copy_in(list(want[:t].split(numels)), grads, False)
+    want[t:] = 0
+    torch_ops.div_if_needed(want, 8.0)
+    dsrc = src.to(DEV)
+    dgrads = list(dsrc.split(numels))
+    table = nat.TensorTable(numels, t_pad, torch.device(DEV))
+    got = old.to(DEV)
+    table.gather_in(dgrads, got, None, 8.0, True)
+    assert_bits_equal(got, want, "gather_in, 65,534 tensors")
+    flat = mixed_values(g, t_pad, torch.float32).to(DEV)
+    out = torch.zeros(t, dtype=torch.bfloat16, device=DEV)
+    table.scatter_out(flat, list(out.split(numels)))
+    assert_bits_equal(out, flat[:t].cpu().bfloat16(), "scatter_out, 65,534 tensors")
+    table.close()
