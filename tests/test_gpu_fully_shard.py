@@ -290,3 +290,28 @@ def test_list_of_modules_forms_one_group():
         m = _make(32)
         fully_shard([m.blocks[0], m.blocks[1]], mp_policy=MP)
         m.blocks[0](xs[0])
+
+
+def test_state_dict_sees_sharded_parameters_even_when_unsharded():
+    """ya_fsdp/_param_group.py:886-909: state_dict() / load_state_dict() first put the sharded parameters back."""
+    model = _wrap(_make(41), mp_policy=MP)
+    x = torch.randn(4, 128, device=DEV)
+    model(x)  # forward only: the last users of the data buffers stay unsharded
+    blk = model.blocks[2]
+    assert blk.up.weight.dtype == torch.bfloat16 and blk.up.weight.dim() == 2
+    sd = model.state_dict()
+    assert all(v.dtype == torch.float32 and v.dim() == 1 for v in sd.values())
+    assert blk.up.weight.dtype == torch.float32  # swapped back by the hook
+    new = {k: torch.full_like(v, 0.25) for k, v in sd.items()}
+    # the hook swaps the registered parameters only; the buffers are handed back by reshard(), as after any
+    # forward without backward
+    for m in (model.blocks[2], model.norm):
+        m.reshard()
+    model(x)
+    assert blk.up.weight.dtype == torch.bfloat16
+    model.load_state_dict(new)  # pre-hook: the load goes into the sharded masters
+    assert blk.up.weight.dtype == torch.float32
+    for m in (model.blocks[2], model.norm):
+        m.reshard()
+    group = blk._get_fsdp_state()._fsdp_param_group
+    assert float(group._padded_sharded_param_data[None][: group.layout.total_numel].min()) == 0.25

@@ -183,6 +183,7 @@ class YaFSDPParamGroup:
             fsdp_param._param_group_ref = weakref.ref(self)
             fsdp_param._index_in_group = index
         self._table: _native.TensorTable | None = None
+        self._state_dict_hook_handles: list = []
         # version of the master shard at which a fused optimizer step last wrote the
         # all-gather input (None: never); see all_gather
         self._copy_in_shard_version: int | None = None
@@ -248,6 +249,7 @@ class YaFSDPParamGroup:
             raise RuntimeError(
                 "the data buffer of this group is not allocated: call init_shared_state(groups, device) first"
             )
+        self._register_state_dict_hooks()  # :492
         self._init_unsharded_params()
         shard = self._padded_sharded_param_data[None]
         sharded_numels = self._sharded_param_numels[None]
@@ -524,6 +526,22 @@ class YaFSDPParamGroup:
         storage.  Runs on the current stream; call after ``wait_for_unshard``."""
         assert self._table is not None, "lazy_init() first"
         self._table.scatter_out(self._all_gather_output[None], [o.view(-1) if o is not None else None for o in outs])
+
+    def _register_state_dict_hooks(self) -> None:
+        """ya_fsdp/_param_group.py:886-909: ``state_dict()`` and ``load_state_dict()`` of a
+        module that owns parameters of this group first put the sharded
+        parameters back in place, so both see the fp32 shards whatever state the
+        last forward left the group in."""
+        if self._state_dict_hook_handles:
+            return  # already registered
+        modules_with_params = {p._module_info.module for p in self.fsdp_params if p._module_info is not None}
+
+        def to_sharded_hook(*args: Any, **kwargs: Any) -> None:
+            self._to_sharded()
+
+        for module in modules_with_params:
+            self._state_dict_hook_handles.append(module.register_state_dict_pre_hook(to_sharded_hook))
+            self._state_dict_hook_handles.append(module._register_load_state_dict_pre_hook(to_sharded_hook))
 
     # ------------------------------------------------------------------ utilities --
     def _to_sharded(self) -> None:
