@@ -84,6 +84,30 @@ def numel_of(shape):
     return n
 
 
+def _cu_masked_streams(torch, dev, k: int):
+    """Two streams of the HIP runtime this process already uses: one limited to compute units [0, k), one to
+    [k, 256)."""
+    import ctypes
+
+    if not 0 < k < 256:
+        raise SystemExit("--copy-cus must lie in 1..255")
+    path = next(line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line)
+    hip = ctypes.CDLL(path)
+    hip.hipExtStreamCreateWithCUMask.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_uint32,
+                                                 ctypes.POINTER(ctypes.c_uint32)]
+    out = []
+    for bits in (range(k), range(k, 256)):
+        words = [0] * 8
+        for b in bits:
+            words[b // 32] |= 1 << (b % 32)
+        handle = ctypes.c_void_p()
+        rc = hip.hipExtStreamCreateWithCUMask(ctypes.byref(handle), 8, (ctypes.c_uint32 * 8)(*words))
+        if rc != 0:
+            raise RuntimeError(f"hipExtStreamCreateWithCUMask failed with {rc}")
+        out.append(torch.cuda.ExternalStream(handle.value, device=dev))
+    return out
+
+
 def run_full_model(args) -> int:
     """Full Llama-3-8B per-rank pass at logical W=8 on one GPU: embedding, 32 decoder layers, lm_head and
     the final norm as 35 parameter groups.  Forward: copy-in + copy-out of group i+1 run on a side stream while a
@@ -138,6 +162,11 @@ def run_full_model(args) -> int:
     c = torch.empty(4096, 4096, dtype=torch.bfloat16, device=dev)
     side = torch.cuda.Stream(device=dev)  # default priority
     main = torch.cuda.current_stream(dev)
+    if args.copy_cus:
+        # partition the compute units instead: the copies' stream may use the K lowest-numbered ones, the
+        # GEMMs' stream the others (the HIP runtime's per-stream CU mask; both at default priority)
+        side, main = _cu_masked_streams(torch, dev, args.copy_cus)
+        torch.cuda.set_stream(main)
 
     def unshard(i):  # copy-in + copy-out of group i (current stream)
         g = groups[i]
@@ -248,7 +277,8 @@ def run_full_model(args) -> int:
         "ms_per_step": round(t_both, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "llama3-8b-full-w8", "groups": n, "logical_world_size": w, "rank": r,
-                   "gemm": "bf16 4096x4096x4096, 1 per group forward, 2 per group backward"},
+                   "gemm": "bf16 4096x4096x4096, 1 per group forward, 2 per group backward",
+                   "copy_stream_compute_units": args.copy_cus or 256},
         "ms_copies_alone": round(t_copy, 4), "ms_gemms_alone": round(t_gemm, 4), "ms_overlapped": round(t_both, 4),
         "hidden_fraction": round(hidden, 4), "grid_cap_sweep": sweep, "grid_cap_used": best, "copy_GBps_alone": round(bytes_step / t_copy / 1e6, 1),
         "copy_GBps_overlapped_lower_bound": round(bytes_step / t_both / 1e6, 1), "bytes_per_step": bytes_step,
@@ -715,6 +745,9 @@ def main() -> int:
     ap.add_argument("--sweep-grid-cap", action="store_true",
                     help="llama3-8b-full-w8 only: repeat the overlap measurement with the copy kernels' grids capped "
                          "at 16/8/4/2/1 workgroups per compute unit")
+    ap.add_argument("--copy-cus", type=int, default=0, metavar="K",
+                    help="llama3-8b-full-w8 only: run the copies on a stream limited to K of the 256 compute units "
+                         "and the GEMMs on a stream limited to the others")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
