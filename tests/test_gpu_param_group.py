@@ -163,6 +163,23 @@ def test_backward_reduce_copy_then_accumulate(shapes, w, r, align, force_sum):
         assert group.grad_buffer_ctx.owner is None and group._training_state.name == "IDLE"
 
 
+def test_bit32_acc_flag_leaves_the_one_contribution_result_unchanged():
+    """ya_fsdp/_collectives.py:152-162: the flag only selects the accumulator of the collective; with this rank's
+    chunk as the only contribution the result is the chunk, as without the flag."""
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=torch.bfloat16,
+                              bit32_acc_for_bit16_reduce_scatter=True)
+    w, r, align = 4, 2, 8
+    group, cpu_params = _make_group(ODD_SHAPES, w, r, align, mp)
+    ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    ref.unshard()
+    _run_backward(group, ref, _grads(ODD_SHAPES, torch.bfloat16, 77))
+    ref.reduce(None, float(w), "copy")
+    group.finalize_backward()
+    torch.cuda.synchronize()
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
+
+
 def test_gradient_accumulation_without_sync_uses_add():
     shapes, w, r, align = ODD_SHAPES, 4, 1, 8
     group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)

@@ -44,3 +44,12 @@ def test_flat_adamw_rejects_bad_hyperparameters():
     p[0].grad = torch.zeros(4)
     with pytest.raises(TypeError):
         opt.step()
+
+
+def test_sizes_to_slices_docstring_example():
+    """The one worked example the reference holds for this path (ya_fsdp/_collectives.py:79-90)."""
+    from yafsdp_amd._collectives import sizes_to_slices
+
+    assert sizes_to_slices([20, 20, 30]) == [slice(0, 20, None), slice(20, 40, None), slice(40, 70, None)]
+    assert sizes_to_slices([]) == []
+    assert sizes_to_slices([0, 3, 0]) == [slice(0, 0), slice(0, 3), slice(3, 3)]

@@ -33,6 +33,8 @@ by the custom factor) applied as a post-divide in the same launch.
 
 from __future__ import annotations
 
+import itertools
+
 from typing import TYPE_CHECKING, Any, NamedTuple, Optional, Sequence
 
 import torch
@@ -113,6 +115,16 @@ def all_gather(
     return AllGatherResult(all_gather_event, all_gather_work)
 
 
+def sizes_to_slices(sizes: list[int]) -> list[slice]:
+    """ya_fsdp/_collectives.py:79-90: consecutive slices of the given lengths.
+
+    >>> sizes_to_slices([20, 20, 30])
+    [slice(0, 20, None), slice(20, 40, None), slice(40, 70, None)]
+    """
+    ends = list(itertools.accumulate(sizes))
+    return [slice(end - size, end) for size, end in zip(sizes, ends)]
+
+
 def foreach_reduce_copy_in(
     param_group: "YaFSDPParamGroup",
     table: "_native.TensorTable",
@@ -159,10 +171,10 @@ def reduce_scatter(
     """
     if yccl_handle is not None:
         raise NotImplementedError("YCCL handles are not part of this build")
-    if bit32_acc_for_bit16_reduce_scatter:
-        # the reference passes acc_type= to dist.reduce_scatter_tensor (:157-161),
-        # which only exists in a patched torch; there is no collective here
-        raise NotImplementedError("bit32_acc_for_bit16_reduce_scatter needs an inter-GPU reduce-scatter")
+    # bit32_acc_for_bit16_reduce_scatter only reaches the collective (acc_type=, :157-161) and is unused for a
+    # group of size 1 (:140-150).  Here this rank's chunk is the only contribution to its reduce-scatter output,
+    # and a binary32 sum of one 16-bit value rounds back to that value, so the flag changes nothing; the sum over
+    # several contributions in binary32 is ``post_reduce_fanin``.
     reduce_scatter_stream.wait_stream(torch.cuda.current_stream(padded_sharded_param_grad.device))
     with torch.cuda.stream(reduce_scatter_stream):
         world_size, rank = reduce_scatter_group.size(), reduce_scatter_group.rank()
