@@ -288,6 +288,197 @@ def run_full_model(args) -> int:
     return 0
 
 
+def run_trainer(args) -> int:
+    """Whole training iterations on one GPU at world size 1: Llama-3-8B decoder layers (real shapes, random init)
+    wrapped one by one with ``fully_shard`` (fp32 masters, bf16 compute), forward + backward + gradient norm +
+    AdamW.  Three loops over the same model and inputs:
+
+    * ``fully_shard`` + ``FlatAdamW`` (buffer kernels; the optimizer pass also writes the next copy-in);
+    * ``fully_shard`` + ``torch.optim.AdamW(fused=True)`` on the sharded parameters;
+    * no wrapper: the same mixed precision written by hand with torch ops (``_foreach_copy_`` of the fp32 masters
+      into a bf16 copy of the model, gradients copied back into fp32, fused torch AdamW).
+
+    The compute floor (bf16 forward + backward only, no masters, no optimizer) is reported beside them."""
+    import copy
+
+    import torch
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    from yafsdp_amd import MixedPrecisionPolicy, fully_shard
+    from yafsdp_amd.optim import FlatAdamW, clip_grad_norm_, grad_clip_coef
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    dim, ffn, heads, kv_heads, layers, seq = 4096, 14336, 32, 8, args.layers, args.seq_len
+    hd = dim // heads
+
+    class RMSNorm(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.weight = nn.Parameter(torch.ones(dim))
+
+        def forward(self, x):
+            return F.rms_norm(x, (dim,), self.weight, 1e-5)
+
+    class Layer(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q = nn.Linear(dim, dim, bias=False)
+            self.k = nn.Linear(dim, kv_heads * hd, bias=False)
+            self.v = nn.Linear(dim, kv_heads * hd, bias=False)
+            self.o = nn.Linear(dim, dim, bias=False)
+            self.gate = nn.Linear(dim, ffn, bias=False)
+            self.up = nn.Linear(dim, ffn, bias=False)
+            self.down = nn.Linear(ffn, dim, bias=False)
+            self.n1, self.n2 = RMSNorm(), RMSNorm()
+
+        def forward(self, x):
+            b, s_, _ = x.shape
+            h = self.n1(x)
+            q = self.q(h).view(b, s_, heads, hd).transpose(1, 2)
+            k = self.k(h).view(b, s_, kv_heads, hd).transpose(1, 2)
+            v = self.v(h).view(b, s_, kv_heads, hd).transpose(1, 2)
+            a = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+            x = x + self.o(a.transpose(1, 2).reshape(b, s_, dim))
+            h = self.n2(x)
+            return x + self.down(F.silu(self.gate(h)) * self.up(h))
+
+    class Stack(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = nn.ModuleList([Layer() for _ in range(layers)])
+
+        def forward(self, x):
+            for layer in self.layers:
+                x = layer(x)
+            return x
+
+    torch.manual_seed(1006)
+    with torch.device(dev):
+        model0 = Stack()
+    for p in model0.parameters():
+        if p.dim() > 1:
+            nn.init.normal_(p, std=0.02)
+    n_params = sum(p.numel() for p in model0.parameters())
+    x = torch.randn(1, seq, dim, device=dev, dtype=torch.bfloat16)
+    log(f"{layers} layers, {n_params / 1e6:.0f} M parameters, {seq} tokens per iteration")
+    hyper = dict(lr=1e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+
+    def loss_of(y):
+        return y.float().pow(2).mean()
+
+    spread = {}
+
+    def timed(step, reps, warm, name):
+        """Median over the iterations (events at the iteration boundaries, no host synchronisation between
+        them); the mean over the same iterations, host clock, is kept beside it."""
+        import gc
+
+        for _ in range(warm):
+            step()
+        gc.collect()
+        torch.cuda.synchronize()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(reps + 1)]
+        t0 = time.perf_counter()
+        marks[0].record()
+        for i in range(reps):
+            step()
+            marks[i + 1].record()
+        torch.cuda.synchronize()
+        mean = (time.perf_counter() - t0) / reps * 1e3
+        per = [marks[i].elapsed_time(marks[i + 1]) for i in range(reps)]
+        spread[name] = {"mean": round(mean, 3), "min": round(min(per), 3), "max": round(max(per), 3)}
+        return statistics.median(per)
+
+    reps, warm = max(3, args.steps // 5), max(2, args.warmup // 5)
+    results = {}
+
+    # ---- compute floor: bf16 forward + backward only
+    lowp = copy.deepcopy(model0).to(torch.bfloat16)
+
+    def floor_step():
+        loss_of(lowp(x)).backward()
+        for p in lowp.parameters():
+            p.grad = None
+
+    results["compute_only_bf16"] = timed(floor_step, reps, warm, "compute_only_bf16")
+
+    # ---- hand-written mixed precision with torch ops
+    masters = [p.detach().clone().requires_grad_(True) for p in model0.parameters()]
+    lowp_params = list(lowp.parameters())
+    for m in masters:
+        m.grad = torch.zeros_like(m)
+    opt_t = torch.optim.AdamW(masters, fused=True, **hyper)
+
+    def torch_step():
+        with torch.no_grad():
+            torch._foreach_copy_(lowp_params, masters)          # the cast the copy-in does
+        loss_of(lowp(x)).backward()
+        with torch.no_grad():
+            torch._foreach_copy_([m.grad for m in masters], [p.grad for p in lowp_params])  # bf16 -> fp32 gradients
+        for p in lowp_params:
+            p.grad = None
+        torch.nn.utils.clip_grad_norm_(masters, 1.0, foreach=True)
+        opt_t.step()
+
+    results["torch_ops_by_hand"] = timed(torch_step, reps, warm, "torch_ops_by_hand")
+    del masters, opt_t, lowp, lowp_params
+    torch.cuda.empty_cache()
+
+    # ---- fully_shard, two optimizers
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16)
+
+    def wrapped():
+        m = copy.deepcopy(model0)
+        for layer in m.layers:
+            fully_shard(layer, mp_policy=mp)
+        return fully_shard(m, mp_policy=mp)
+
+    for name in ("fully_shard_torch_adamw", "fully_shard_flat_adamw"):
+        model = wrapped()
+        params = list(model.parameters())
+        flat = name == "fully_shard_flat_adamw"
+        if flat:
+            opt = FlatAdamW(params, **hyper)
+        else:
+            opt = torch.optim.AdamW(params, fused=True, **hyper)
+
+        def fs_step():
+            loss_of(model(x)).backward()
+            if flat:
+                _, coef = grad_clip_coef(model, 1.0)   # the norm only; the optimizer pass applies the coefficient
+                opt.step(grad_scale=coef)
+            else:
+                clip_grad_norm_(model, 1.0)
+                opt.step()
+            # gradients stay allocated (the flat gradient shard); the next backward accumulates into them
+            # unless they are cleared, as with torch.optim
+            opt.zero_grad(set_to_none=True)
+
+        results[name] = timed(fs_step, reps, warm, name)
+        del model, params, opt
+        torch.cuda.empty_cache()
+
+    for k_, v_ in results.items():
+        log(f"  {k_:28s} {v_:8.3f} ms / iteration (median; {spread[k_]})  ({seq / v_ * 1e3:9.0f} tokens/s)")
+    best = results["fully_shard_flat_adamw"]
+    out = {
+        "metric": f"training iteration at world size 1: {layers} Llama-3-8B decoder layers through fully_shard + flat AdamW",
+        "value": round(seq / best * 1e3, 1), "unit": "tokens/s", "n_gpus": 1, "steps": reps, "warmup": warm,
+        "ms_per_step": round(best, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "fully-shard-trainer-w1", "layers": layers, "parameters": n_params, "tokens_per_step": seq,
+                   "master_dtype": "float32", "optimizer": "AdamW + gradient clipping"},
+        "ms_per_iteration": {k_: round(v_, 4) for k_, v_ in results.items()},
+        "ms_per_iteration_mean_min_max": spread,
+        "overhead_over_compute_ms": {k_: round(v_ - results["compute_only_bf16"], 4) for k_, v_ in results.items()
+                                     if k_ != "compute_only_bf16"},
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def run_optim(args) -> int:
     """Optimizer-side passes over one rank's flat shard of the layer (what follows the backward pass of a step):
     squared gradient norm, clip coefficient, and the fused AdamW step that scales the gradient by the coefficient
@@ -735,7 +926,8 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3-8b-layer-w8",
                     choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256", "ragged-stress-w256-bf16-masters",
                                                  "llama3-8b-layer-w8-optim",
-                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange", "hbm-ceilings"])
+                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange", "hbm-ceilings",
+                                                 "fully-shard-trainer-w1"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
     ap.add_argument("--no-graph", action="store_true",
@@ -748,6 +940,8 @@ def main() -> int:
     ap.add_argument("--copy-cus", type=int, default=0, metavar="K",
                     help="llama3-8b-full-w8 only: run the copies on a stream limited to K of the 256 compute units "
                          "and the GEMMs on a stream limited to the others")
+    ap.add_argument("--layers", type=int, default=4, help="fully-shard-trainer-w1 only: decoder layers")
+    ap.add_argument("--seq-len", type=int, default=4096, help="fully-shard-trainer-w1 only: tokens per iteration")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
@@ -771,6 +965,8 @@ def main() -> int:
         return run_exchange(args)
     if args.workload == "hbm-ceilings":
         return run_ceilings(args)
+    if args.workload == "fully-shard-trainer-w1":
+        return run_trainer(args)
     from yafsdp_amd import _native
     from yafsdp_amd._layout import make_layout
 
