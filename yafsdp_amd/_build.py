@@ -62,5 +62,34 @@ def build(force: bool = True, jobs: int = 6) -> str:
     return OUT
 
 
+TENSORLIST_SRC = os.path.join(CSRC, "tensorlist.cpp")
+TENSORLIST_OUT = os.path.join(HERE, "_tensorlist.so")
+
+
+def build_tensorlist(force: bool = True) -> str:
+    """Compile the host-side tensor-list helper of the Python binding (plain C++ against the installed torch's
+    headers; no device code)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    if not force and os.path.exists(TENSORLIST_OUT) and os.path.getmtime(TENSORLIST_OUT) >= os.path.getmtime(TENSORLIST_SRC):
+        return TENSORLIST_OUT
+    lib_dir = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [
+        os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wno-unused-function",
+        TENSORLIST_SRC, "-o", TENSORLIST_OUT,
+        f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-DTORCH_API_INCLUDE_EXTENSION_H",
+        *[f"-I{p}" for p in cpp_extension.include_paths()], f"-I{sysconfig.get_paths()['include']}",
+        f"-L{lib_dir}", "-ltorch", "-ltorch_cpu", "-lc10", "-ltorch_python", f"-Wl,-rpath,{lib_dir}",
+    ]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"compiling tensorlist.cpp failed:\n{r.stderr[-4000:]}")
+    return TENSORLIST_OUT
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_tensorlist())

@@ -138,12 +138,10 @@ def foreach_reduce_copy_in(
     with the pre-divide of ya_fsdp/_collectives.py:139 and the zero-fill of the
     pad lanes fused in.  Runs on the current (compute) stream, like the
     reference's foreach calls."""
-    prepared = []
-    for g in grads:
-        if g is not None and not g.is_contiguous():
-            g = g.contiguous()  # the reference's foreach ops accept strided gradients
-        prepared.append(g)
-    table.gather_in(prepared, reduce_scatter_input, modes, predivide_factor, zero_pad=True)
+    if not _native.all_contiguous(grads):
+        # the reference's foreach ops accept strided gradients
+        grads = [g if g is None or g.is_contiguous() else g.contiguous() for g in grads]
+    table.gather_in(grads, reduce_scatter_input, modes, predivide_factor, zero_pad=True)
 
 
 def reduce_scatter(

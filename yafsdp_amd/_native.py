@@ -22,6 +22,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # YAFSDP_HIP_LIBRARY points at a library built elsewhere (same C ABI); default: the in-tree build
 LIB_PATH = os.environ.get("YAFSDP_HIP_LIBRARY") or os.path.join(_HERE, "libyafsdp_hip.so")
 
+# optional host-side helper (csrc/tensorlist.cpp): validates a tensor list and writes its pointer array in one
+# C++ pass; without it the same checks run in Python.  It launches nothing and touches no tensor data.
+try:
+    from . import _tensorlist
+except ImportError:  # not built: the Python checks below do the same work, slower for large tables
+    _tensorlist = None
+
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MODE_SKIP, MODE_COPY, MODE_ADD = 0, 1, 2
 OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU, OPT_TABLE_LARGE_LOG2 = 0, 1, 2
@@ -237,6 +244,13 @@ def post_reduce_fragments(
 
 
 # --------------------------------------------------------------- table ops --
+def all_contiguous(tensors: Sequence[torch.Tensor | None]) -> bool:
+    """True if every tensor of the list (``None`` entries aside) is contiguous."""
+    if _tensorlist is not None and isinstance(tensors, (list, tuple)):
+        return _tensorlist.all_contiguous(tensors)
+    return all(t is None or t.is_contiguous() for t in tensors)
+
+
 class TensorTable:
     """Device-resident metadata of one flat buffer (tensor boundaries and the
     tile -> tensor map).  Static for the life of a parameter group; the tensor
@@ -259,6 +273,7 @@ class TensorTable:
         self._handle = handle
         # per-call pointer / mode arrays; the lock keeps "fill, then launch" atomic when the table is used from
         # two host threads (the main thread and the autograd engine thread)
+        self._numels_arr = np.ascontiguousarray(self.numels, dtype=np.int64)
         self._ptrs = np.zeros(max(1, len(self.numels)), dtype=np.uint64)
         self._modes = np.zeros(max(1, len(self.numels)), dtype=np.uint8)
         self._lock = threading.Lock()
@@ -290,6 +305,14 @@ class TensorTable:
             raise ValueError(f"{what}: expected {n} modes, got {len(modes)}")
         if n == 0:
             return -1
+        if _tensorlist is not None:
+            code = _tensorlist.fill(
+                tensors, modes, self._numels_arr.ctypes.data, self._ptrs.ctypes.data, self._modes.ctypes.data,
+                self.device.type == "cuda", self.device.index if self.device.index is not None else -1,
+            )
+            if code != _tensorlist.REJECTED:
+                return code
+            # not accepted as it stands: the checks below find out why and raise
         if modes is None:
             live = [t for t in tensors if t is not None]
             if len(live) == n:
