@@ -315,3 +315,34 @@ def test_state_dict_sees_sharded_parameters_even_when_unsharded():
         m.reshard()
     group = blk._get_fsdp_state()._fsdp_param_group
     assert float(group._padded_sharded_param_data[None][: group.layout.total_numel].min()) == 0.25
+
+
+def test_custom_gradient_buffer_assignment():
+    """ya_fsdp/_state.py:127-136, 617-660: a group -> buffer-context index map replaces the round-robin
+    assignment of the gradient buffers (accepted together with allow_no_grad_reduce, as in the reference)."""
+    model0 = _make(8)
+    xs = [torch.randn(16, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(90 + s)) for s in range(3)]
+    ref = _reference_steps(model0, xs, lr=0.05)
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    groups = [m._get_fsdp_state()._fsdp_param_group for m in (*model.blocks, model.norm)]
+    model._get_fsdp_state()._lazy_init(
+        allow_no_grad_reduce=True,
+        param_group_to_grad_buffer_ctx_idx={groups[0]: 0, groups[1]: 1, groups[2]: 0, groups[3]: 1},
+    )
+    assert groups[0].grad_buffer_ctx is groups[2].grad_buffer_ctx
+    assert groups[1].grad_buffer_ctx is groups[3].grad_buffer_ctx
+    assert groups[0].grad_buffer_ctx is not groups[1].grad_buffer_ctx
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    for x in xs:
+        model(x).float().pow(2).mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    got, want = _gather_full(model), dict(ref.named_parameters())
+    for k in want:
+        assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
+    # without allow_no_grad_reduce the default is one shared buffer and a map is refused (:659-660)
+    other = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    g2 = [m._get_fsdp_state()._fsdp_param_group for m in (*other.blocks, other.norm)]
+    with pytest.raises(AssertionError):
+        other._get_fsdp_state()._lazy_init(param_group_to_grad_buffer_ctx_idx={g: 0 for g in g2})

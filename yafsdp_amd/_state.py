@@ -116,10 +116,19 @@ class YaFSDPState(_State):
             args, kwargs = args_tuple[0], kwargs_tuple[0]
         return args, kwargs
 
-    def _lazy_init(self, allow_no_grad_reduce: bool = False) -> None:
+    def _lazy_init(
+        self,
+        allow_no_grad_reduce: bool = False,
+        param_group_to_data_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
+        param_group_to_grad_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
+    ) -> None:
         """ya_fsdp/_state.py:127-175.  ``allow_no_grad_reduce`` gives every group
         its own gradient buffer, which gradient accumulation without
-        synchronisation needs (the unreduced gradients live in that buffer)."""
+        synchronisation needs (the unreduced gradients live in that buffer).
+        The two maps replace the round-robin buffer assignment: group -> index
+        (in module order) of the group whose buffer context it uses; as in the
+        reference (:645-660) a map is only accepted where the default would give
+        every group its own buffer."""
         if self._is_root is not None:
             return
         self._is_root = True
@@ -141,13 +150,19 @@ class YaFSDPState(_State):
                 self._state_ctx.all_states.append(state)
             visited_states.add(state)
         self._init_fqns()
-        self._init_shared_state(allow_no_grad_reduce)
+        self._init_shared_state(allow_no_grad_reduce, param_group_to_data_buffer_ctx_idx,
+                                param_group_to_grad_buffer_ctx_idx)
         self.validate_shared_state()
         for state in self._state_ctx.all_states:
             if state._fsdp_param_group:
                 state._fsdp_param_group.lazy_init()
 
-    def _init_shared_state(self, allow_no_grad_reduce: bool = False) -> None:
+    def _init_shared_state(
+        self,
+        allow_no_grad_reduce: bool = False,
+        param_group_to_data_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
+        param_group_to_grad_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
+    ) -> None:
         """ya_fsdp/_state.py:177-288 and :617-678: one communication context;
         two data buffers handed out round-robin in module order and one gradient
         buffer, each as large as the largest group that uses it; the last group on
@@ -163,14 +178,24 @@ class YaFSDPState(_State):
             return
         no_reshard_after_forward = all(not g.reshard_after_forward for g in param_groups)
 
-        def assign(groups, attr, count, size_of):
+        def assign(groups, attr, count, size_of, ctx_idx=None):
             if not groups:
                 return []
-            n = len(groups) if count is None else min(count, len(groups))
-            ctxs = [getattr(groups[i], attr) for i in range(n)]
-            users = [[] for _ in range(n)]
-            for i, g in enumerate(groups):
-                users[i % n].append(g)
+            if ctx_idx is not None:
+                assert count is None  # ya_fsdp/_state.py:659-660
+                ctxs, users = [], []
+                for g in groups:  # buffer contexts in order of first use (:661-669)
+                    ctx = getattr(groups[ctx_idx[g]], attr)
+                    if not any(ctx is c for c in ctxs):
+                        ctxs.append(ctx)
+                        users.append([])
+                    users[next(i for i, c in enumerate(ctxs) if c is ctx)].append(g)
+            else:
+                n = len(groups) if count is None else min(count, len(groups))
+                ctxs = [getattr(groups[i], attr) for i in range(n)]
+                users = [[] for _ in range(n)]
+                for i, g in enumerate(groups):
+                    users[i % n].append(g)
             for ctx, gs in zip(ctxs, users):
                 ctx.lazy_init({None: max(size_of(g) for g in gs)}, self._device)
                 for g in gs:
@@ -178,14 +203,15 @@ class YaFSDPState(_State):
             return users
 
         data_users = assign(param_groups, "data_buffer_ctx", None if no_reshard_after_forward else 2,
-                            lambda g: g.data_buffer_bytes())
+                            lambda g: g.data_buffer_bytes(), param_group_to_data_buffer_ctx_idx)
         for state_groups in data_users:
             last = state_groups[-1]
             owner_state = next(s for s in self._state_ctx.all_states if s._fsdp_param_group is last)
             if owner_state._auto_reshard_after_forward:
                 last.reshard_after_forward = False  # ya_fsdp/_state.py:256-260
         assign([g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx",
-               None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes())
+               None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes(),
+               param_group_to_grad_buffer_ctx_idx)
 
     def validate_shared_state(self) -> None:
         """ya_fsdp/_state.py:290-414: enough buffers for overlap; at most one
