@@ -126,3 +126,55 @@ def test_full_state_dict_round_trip_through_the_unwrapped_model():
     fresh.blocks[1].unshard()
     with pytest.raises(RuntimeError, match="sharded state"):
         full_state_dict(fresh)
+
+
+def test_torch_distributed_checkpoint_round_trip(tmp_path):
+    """A trained wrapped model saved with torch.distributed.checkpoint through RaggedShardTensor handles
+    (views of the flat master shards) and loaded into a freshly wrapped model and into plain flattened tensors."""
+    import torch.distributed.checkpoint as dcp
+
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.checkpoint import checkpointable_state_dict, fsdp_groups_of
+
+    def wrap(m):
+        for b in m.blocks:
+            fully_shard(b, mp_policy=MP)
+        fully_shard(m.norm, mp_policy=MP)
+        return fully_shard(m, mp_policy=MP)
+
+    def handles(m):
+        out = {}
+        for g in fsdp_groups_of(m):
+            out.update(checkpointable_state_dict(g))
+        return out
+
+    model0 = _make(31)
+    model = wrap(copy.deepcopy(model0))
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    x = torch.randn(8, 128, device=DEV)
+    for _ in range(2):
+        model(x).float().pow(2).mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    sd = handles(model)
+    assert set(sd) == {n for n, _ in model0.named_parameters()}
+    assert all(tuple(h.size()) == (p.numel(),) for h, p in ((sd[n], p) for n, p in model0.named_parameters()))
+    with pytest.raises(NotImplementedError, match="checkpoint handle"):
+        sd["norm.weight"] + 1
+    dcp.save(sd, checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    # (a) plain flattened tensors
+    flat = {n: torch.full((p.numel(),), float("nan"), device=DEV) for n, p in model0.named_parameters()}
+    dcp.load(flat, checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    for n, h in sd.items():
+        assert_bits_equal(flat[n], h.local_tensor, n)
+    # (b) a freshly wrapped model: the load writes its flat master shards
+    fresh = wrap(copy.deepcopy(model0))
+    fresh(x)  # lazy init (then hand the buffers back, as after any forward without backward)
+    for m in (fresh.blocks[2], fresh.norm):
+        m.reshard()
+    dcp.load(handles(fresh), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    for g in fsdp_groups_of(fresh):
+        g._all_gather_input_set_dtypes.clear()
+    for ga, gb in zip(fsdp_groups_of(model), fsdp_groups_of(fresh)):
+        assert_bits_equal(gb._padded_sharded_param_data[None], ga._padded_sharded_param_data[None], "masters")
+    assert_bits_equal(fresh(x), model(x).detach(), "outputs after reload")

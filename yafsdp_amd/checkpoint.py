@@ -15,7 +15,9 @@ movement runs on the buffer kernels: the ranks' flat shards are copied into a
 flat buffer (``flat_copy``) and split into the full parameters by the copy-out
 kernel (``scatter_out``); loading copies each rank's fragment out of the full
 parameter (``flat_copy``).  One GPU: the "ranks" are the logical ranks of a
-layout, e.g. modules wrapped with ``mesh=(W, r)``.
+layout, e.g. modules wrapped with ``mesh=(W, r)``.  ``RaggedShardTensor`` hands the
+same chunks to ``torch.distributed.checkpoint`` (the hooks of
+ya_fsdp/_tensor.py:365-432).
 """
 
 from __future__ import annotations
@@ -31,7 +33,7 @@ from ._layout import RaggedShard
 from ._param_group import YaFSDPParamGroup
 
 __all__ = ["ChunkMeta", "chunk_meta", "sharded_state_dict", "group_meta_info", "full_tensors", "load_full_tensors",
-           "full_state_dict", "load_full_state_dict"]
+           "full_state_dict", "load_full_state_dict", "RaggedShardTensor", "checkpointable_state_dict"]
 
 
 @dataclass(frozen=True)
@@ -67,6 +69,88 @@ def sharded_state_dict(group: YaFSDPParamGroup) -> dict[str, tuple[torch.Tensor,
         meta = chunk_meta(fsdp_param._param_fqn, fsdp_param.placement, fsdp_param._orig_size)
         out[fsdp_param._param_fqn] = (fsdp_param._sharded_param_data, meta)
     return out
+
+
+class RaggedShardTensor(torch.Tensor):
+    """Checkpoint handle of one parameter on one rank: stands for the parameter
+    flattened to ``(numel,)`` (that is its ``size()``; it has no storage of its
+    own) and holds the rank's local 1-D fragment, with the three hooks that
+    ``torch.distributed.checkpoint`` looks for on a state-dict value
+    (``__create_write_items__``, ``__create_chunk_list__``, ``__get_tensor_shard__``)
+    and the chunk the reference declares (ya_fsdp/_tensor.py:365-432): this
+    rank contributes ``[offset, offset + local_numel)`` of the flattened
+    parameter, or an empty chunk at ``offset == numel``.  The local fragment
+    aliases the tensor given (normally a view of the flat master shard), so
+    saving reads the masters and loading writes them; after a load, clear the
+    group's copy-in flags (``load_full_tensors`` shows how) so that the next
+    unshard casts the new values.  No tensor op runs on the handle itself."""
+
+    __slots__ = ["_local_tensor", "_chunk"]
+
+    @staticmethod
+    def __new__(cls, local: torch.Tensor, meta: ChunkMeta) -> "RaggedShardTensor":
+        if local.dim() != 1 or local.numel() != meta.sizes[0]:
+            raise ValueError(f"{meta.fqn}: local tensor {tuple(local.shape)} does not match the chunk size {meta.sizes}")
+        r = torch.Tensor._make_wrapper_subclass(
+            cls, torch.Size(meta.size), dtype=local.dtype, device=local.device, layout=local.layout, requires_grad=False
+        )
+        r._local_tensor = local.detach()
+        r._chunk = meta
+        return r
+
+    @classmethod
+    def wrap(cls, local: torch.Tensor, meta: ChunkMeta) -> "RaggedShardTensor":
+        return cls(local, meta)
+
+    @classmethod
+    def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+        raise NotImplementedError(f"{func}: a RaggedShardTensor is a checkpoint handle; operate on .local_tensor")
+
+    def __repr__(self) -> str:  # type: ignore[override]
+        return f"RaggedShardTensor({self._chunk}, local_tensor={self._local_tensor!r})"
+
+    @property
+    def chunk(self) -> ChunkMeta:
+        return self._chunk
+
+    @property
+    def local_tensor(self) -> torch.Tensor:
+        return self._local_tensor
+
+    def _local(self) -> torch.Tensor:
+        return self._local_tensor
+
+    def __create_write_items__(self, fqn: str, object):  # noqa: A002  (the protocol's argument name)
+        from torch.distributed.checkpoint.metadata import ChunkStorageMetadata, MetadataIndex, TensorProperties
+        from torch.distributed.checkpoint.planner import TensorWriteData, WriteItem, WriteItemType
+
+        offsets, sizes = torch.Size(self._chunk.offsets), torch.Size(self._chunk.sizes)
+        return [
+            WriteItem(
+                index=MetadataIndex(fqn, offsets),
+                type=WriteItemType.SHARD,
+                tensor_data=TensorWriteData(
+                    chunk=ChunkStorageMetadata(offsets=offsets, sizes=sizes),
+                    properties=TensorProperties.create_from_tensor(self._local()),
+                    size=torch.Size(self._chunk.size),
+                ),
+            )
+        ]
+
+    def __create_chunk_list__(self):
+        from torch.distributed.checkpoint.metadata import ChunkStorageMetadata
+
+        return [ChunkStorageMetadata(offsets=torch.Size(self._chunk.offsets), sizes=torch.Size(self._chunk.sizes))]
+
+    def __get_tensor_shard__(self, index) -> torch.Tensor:
+        return self._local()
+
+
+def checkpointable_state_dict(group: YaFSDPParamGroup) -> dict[str, RaggedShardTensor]:
+    """``{fqn: RaggedShardTensor}`` of one parameter group on this rank, for
+    ``torch.distributed.checkpoint.save`` / ``load`` (views of the flat master
+    shard: no copy)."""
+    return {fqn: RaggedShardTensor.wrap(local, meta) for fqn, (local, meta) in sharded_state_dict(group).items()}
 
 
 def group_meta_info(group: YaFSDPParamGroup) -> dict[str, list]:
