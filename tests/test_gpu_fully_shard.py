@@ -346,3 +346,100 @@ def test_custom_gradient_buffer_assignment():
     g2 = [m._get_fsdp_state()._fsdp_param_group for m in (*other.blocks, other.norm)]
     with pytest.raises(AssertionError):
         other._get_fsdp_state()._lazy_init(param_group_to_grad_buffer_ctx_idx={g: 0 for g in g2})
+
+
+def _train(model, xs, lr, after_step=None):
+    opt = torch.optim.SGD(model.parameters(), lr=lr)
+    for x in xs:
+        model(x).float().pow(2).mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+        if after_step is not None:
+            after_step()
+    torch.cuda.synchronize()
+    return _gather_full(model)
+
+
+def _assert_same_masters(got, want):
+    assert set(got) == set(want)
+    for k in want:
+        assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
+
+
+def test_setters_that_must_not_change_the_numbers():
+    """ya_fsdp/fully_shard.py:138-239: keeping parameters unsharded after backward, forcing SUM (at world size 1
+    no division either way, ya_fsdp/_collectives.py:221-267), a post-optimizer event for the all-gather stream to
+    wait on, and explicit prefetch orders leave the training bit-identical."""
+    model0 = _make(51)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(60 + s)) for s in range(3)]
+    want = dict(_reference_steps(model0, xs, lr=0.05).named_parameters())
+
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    for m in (*model.blocks, model.norm):
+        m.set_force_sum_reduction_for_comms(True)
+    _assert_same_masters(_train(model, xs, 0.05), want)
+
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+
+    def mark():  # what a trainer does after optimizer.step(): the next all-gather waits for it
+        model.set_post_optim_event(torch.cuda.current_stream().record_event())
+
+    _assert_same_masters(_train(model, xs, 0.05, after_step=mark), want)
+
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    blocks = list(model.blocks)
+    blocks[0].set_modules_to_forward_prefetch([blocks[1]])
+    blocks[1].set_modules_to_forward_prefetch([blocks[2]])
+    blocks[2].set_modules_to_backward_prefetch([blocks[1]])
+    blocks[1].set_modules_to_backward_prefetch([blocks[0]])
+    _assert_same_masters(_train(model, xs, 0.05), want)
+
+
+
+def test_parameters_kept_unsharded_between_micro_batches():
+    """set_reshard_after_backward(False) for all but the last micro-batch of a step (every group on a data buffer
+    of its own: reshard_after_forward=False): the second micro-batch finds the parameters gathered and skips the
+    all-gather; the numbers equal those of the default schedule."""
+    model0 = _make(53)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(85 + s)) for s in range(4)]
+
+    def run(keep: bool):
+        model = _wrap(copy.deepcopy(model0), mp_policy=MP, reshard_after_forward=False)
+        opt = torch.optim.SGD(model.parameters(), lr=0.05)
+        groups = [m._get_fsdp_state()._fsdp_param_group for m in (*model.blocks, model.norm)]
+        for i in range(0, 4, 2):
+            if keep:
+                model.set_reshard_after_backward(False)
+            model(xs[i]).float().pow(2).mean().backward()
+            if keep:
+                assert all(g.is_unsharded for g in groups)
+                model.set_reshard_after_backward(True)
+            model(xs[i + 1]).float().pow(2).mean().backward()
+            assert all(g.is_sharded for g in groups)
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+        torch.cuda.synchronize()
+        return _gather_full(model)
+
+    _assert_same_masters(run(True), run(False))
+
+
+def test_custom_gradient_divide_factor():
+    """set_gradient_divide_factor(4) at world size 1 copies the reduce buffer divided by 4 into the gradient shard
+    (ya_fsdp/_collectives.py:140-148): with bf16 gradients the division by a power of two is exact, so the run
+    equals plain training with a quarter of the learning rate... of the gradients that reach the masters."""
+    model0 = _make(52)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(80 + s)) for s in range(2)]
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    for m in (*model.blocks, model.norm):
+        m.set_gradient_divide_factor(4.0)
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    plain = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    opt_plain = torch.optim.SGD(plain.parameters(), lr=0.05)
+    for x in xs[:1]:  # one step from identical masters: the gradients differ by exactly the factor
+        model(x).float().pow(2).mean().backward()
+        plain(x).float().pow(2).mean().backward()
+        for p, q in zip(model.parameters(), plain.parameters()):
+            assert torch.equal(p.grad * 4.0, q.grad)
+        opt.step(); opt_plain.step()
+    torch.cuda.synchronize()
