@@ -10,6 +10,7 @@ exactly where the reference's torch ops would have been
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import os
 import threading
@@ -163,8 +164,23 @@ def _flat_arg(t: torch.Tensor, what: str) -> torch.Tensor:
     return t
 
 
+_raw_current_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_NO_SWITCH = contextlib.nullcontext()
+
+
 def _stream(t: torch.Tensor) -> int:
+    """``hipStream_t`` of torch's current stream on the tensor's device."""
+    if _raw_current_stream is not None:  # the handle itself, without building a Stream object (2 us less per call)
+        index = t.device.index
+        return _raw_current_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _on(device: torch.device):
+    """Context that makes ``device`` current for a library call; free when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _factor(f: float | None) -> float:
@@ -177,7 +193,7 @@ def flat_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
     _flat_arg(dst, "dst"), _flat_arg(src, "src")
     if dst.numel() != src.numel():
         raise ValueError(f"numel mismatch: {dst.numel()} vs {src.numel()}")
-    with torch.cuda.device(dst.device):
+    with _on(dst.device):
         _check(
             lib.yafsdp_flat_copy(dst.data_ptr(), _dt(dst), src.data_ptr(), _dt(src), dst.numel(), _stream(dst)),
             "yafsdp_flat_copy",
@@ -187,7 +203,7 @@ def flat_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
 def flat_div(buf: torch.Tensor, factor: float | None) -> None:
     """``_div_if_needed(buf, factor)``."""
     _flat_arg(buf, "buf")
-    with torch.cuda.device(buf.device):
+    with _on(buf.device):
         _check(
             lib.yafsdp_flat_div(buf.data_ptr(), _dt(buf), buf.numel(), _factor(factor), _stream(buf)),
             "yafsdp_flat_div",
@@ -199,7 +215,7 @@ def flat_div_copy(dst: torch.Tensor, src: torch.Tensor, divisor: float) -> None:
     _flat_arg(dst, "dst"), _flat_arg(src, "src")
     if dst.numel() != src.numel():
         raise ValueError(f"numel mismatch: {dst.numel()} vs {src.numel()}")
-    with torch.cuda.device(dst.device):
+    with _on(dst.device):
         _check(
             lib.yafsdp_flat_div_copy(
                 dst.data_ptr(), _dt(dst), src.data_ptr(), _dt(src), dst.numel(), float(divisor), _stream(dst)
@@ -212,7 +228,7 @@ def post_reduce(shard: torch.Tensor, chunk: torch.Tensor, post_factor: float | N
     _flat_arg(shard, "shard"), _flat_arg(chunk, "chunk")
     if shard.numel() != chunk.numel():
         raise ValueError(f"numel mismatch: {shard.numel()} vs {chunk.numel()}")
-    with torch.cuda.device(shard.device):
+    with _on(shard.device):
         _check(
             lib.yafsdp_post_reduce(
                 shard.data_ptr(), _dt(shard), chunk.data_ptr(), _dt(chunk), shard.numel(),
@@ -233,7 +249,7 @@ def post_reduce_fragments(
         raise ValueError("frag_numels and frag_modes differ in length")
     if int(numels.sum()) > min(shard.numel(), chunk.numel()):
         raise ValueError("fragments exceed the shard")
-    with torch.cuda.device(shard.device):
+    with _on(shard.device):
         _check(
             lib.yafsdp_post_reduce_fragments(
                 shard.data_ptr(), _dt(shard), chunk.data_ptr(), _dt(chunk), int(numels.size),
@@ -265,7 +281,7 @@ class TensorTable:
             raise RuntimeError(f"TensorTable needs a GPU device, got {device}")
         arr = np.ascontiguousarray(self.numels, dtype=np.int64)
         handle = ctypes.c_void_p()
-        with torch.cuda.device(self.device):
+        with _on(self.device):
             _check(
                 lib.yafsdp_table_create(len(self.numels), arr.ctypes.data, self.padded_numel, ctypes.byref(handle)),
                 "yafsdp_table_create",
@@ -364,7 +380,7 @@ class TensorTable:
         _flat_arg(flat, "flat")
         if flat.numel() < self.padded_numel:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.padded_numel}")
-        with self._lock, torch.cuda.device(self.device):
+        with self._lock, _on(self.device):
             tdt = self._fill(tensors, modes, "tensors")
             if tdt < 0:
                 tdt = _dt(flat)
@@ -383,7 +399,7 @@ class TensorTable:
         _flat_arg(flat, "flat")
         if flat.numel() < self.total_numel:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.total_numel}")
-        with self._lock, torch.cuda.device(self.device):
+        with self._lock, _on(self.device):
             tdt = self._fill(tensors, modes, "tensors")
             if tdt < 0:
                 return
@@ -406,7 +422,7 @@ def flat_copy_fanout(dsts: Sequence[torch.Tensor], src: torch.Tensor) -> None:
         if d.numel() != src.numel() or d.dtype != dsts[0].dtype or d.device != src.device:
             raise ValueError("destinations must match the source's size and device and share a dtype")
     ptrs = (ctypes.c_void_p * len(dsts))(*[d.data_ptr() for d in dsts])
-    with torch.cuda.device(src.device):
+    with _on(src.device):
         _check(
             lib.yafsdp_flat_copy_fanout(ptrs, len(dsts), _dt(dsts[0]), src.data_ptr(), _dt(src), src.numel(), _stream(src)),
             "yafsdp_flat_copy_fanout",
@@ -426,7 +442,7 @@ def post_reduce_fanin(
         if c.numel() != shard.numel() or c.dtype != chunks[0].dtype or c.device != shard.device:
             raise ValueError("chunks must match the shard's size and device and share a dtype")
     ptrs = (ctypes.c_void_p * len(chunks))(*[c.data_ptr() for c in chunks])
-    with torch.cuda.device(shard.device):
+    with _on(shard.device):
         _check(
             lib.yafsdp_post_reduce_fanin(
                 shard.data_ptr(), _dt(shard), ptrs, len(chunks), _dt(chunks[0]), shard.numel(), _factor(post_factor),
@@ -448,7 +464,7 @@ class TensorBinding:
         self.table = table
         self.tensors = list(tensors)
         handle = ctypes.c_void_p()
-        with table._lock, torch.cuda.device(table.device):
+        with table._lock, _on(table.device):
             tdt = table._fill(self.tensors, modes, "tensors")
             self._all_skipped = tdt < 0
             _check(
@@ -474,7 +490,7 @@ class TensorBinding:
         _flat_arg(flat, "flat")
         if flat.numel() < self.table.padded_numel:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.table.padded_numel}")
-        with torch.cuda.device(self.table.device):
+        with _on(self.table.device):
             _check(
                 lib.yafsdp_gather_in_bound(
                     self._handle, flat.data_ptr(), _dt(flat), _factor(pre_factor), int(bool(zero_pad)), _stream(flat)
@@ -488,7 +504,7 @@ class TensorBinding:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.table.total_numel}")
         if self._all_skipped:
             return
-        with torch.cuda.device(self.table.device):
+        with _on(self.table.device):
             _check(
                 lib.yafsdp_scatter_out_bound(self._handle, flat.data_ptr(), _dt(flat), _stream(flat)),
                 "yafsdp_scatter_out_bound",
@@ -502,7 +518,7 @@ ADAM_DECOUPLED_DECAY, ADAM_ZERO_GRAD = 1, 2
 def flat_fill(dst: torch.Tensor, value: float = 0.0) -> None:
     """``dst.fill_(value)`` (``zero_()`` by default) on a flat buffer."""
     _flat_arg(dst, "dst")
-    with torch.cuda.device(dst.device):
+    with _on(dst.device):
         _check(lib.yafsdp_flat_fill(dst.data_ptr(), _dt(dst), dst.numel(), float(value), _stream(dst)), "yafsdp_flat_fill")
 
 
@@ -518,7 +534,7 @@ def flat_sumsq(src: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, ac
         raise TypeError("out must be a float64 tensor with at least one element")
     if out.device != src.device or workspace.device != src.device:
         raise RuntimeError("src, out and workspace must live on one device")
-    with torch.cuda.device(src.device):
+    with _on(src.device):
         _check(
             lib.yafsdp_flat_sumsq(
                 src.data_ptr(), _dt(src), src.numel(), out.data_ptr(), int(accumulate), workspace.data_ptr(),
@@ -540,7 +556,7 @@ def sumsq_partials(src: torch.Tensor, partials: torch.Tensor, offset: int) -> in
     if capacity < 1:
         raise ValueError("partials is full")
     written = ctypes.c_int64()
-    with torch.cuda.device(src.device):
+    with _on(src.device):
         _check(
             lib.yafsdp_sumsq_partials(
                 src.data_ptr(), _dt(src), src.numel(), partials.data_ptr() + 8 * offset, capacity, ctypes.byref(written),
@@ -560,7 +576,7 @@ def clip_coef_from_partials(
         raise TypeError("partials must be float64 and norm_and_coef float32 with two elements")
     if not 0 <= count <= partials.numel():
         raise ValueError("count out of range")
-    with torch.cuda.device(partials.device):
+    with _on(partials.device):
         _check(
             lib.yafsdp_clip_coef_from_partials(
                 partials.data_ptr(), count, float(max_norm), None if sumsq is None else sumsq.data_ptr(),
@@ -575,7 +591,7 @@ def clip_coef(sumsq: torch.Tensor, max_norm: float, norm_and_coef: torch.Tensor)
     _flat_arg(sumsq, "sumsq"), _flat_arg(norm_and_coef, "norm_and_coef")
     if sumsq.dtype != torch.float64 or norm_and_coef.dtype != torch.float32 or norm_and_coef.numel() < 2:
         raise TypeError("sumsq must be float64 and norm_and_coef float32 with two elements")
-    with torch.cuda.device(sumsq.device):
+    with _on(sumsq.device):
         _check(
             lib.yafsdp_clip_coef(sumsq.data_ptr(), float(max_norm), norm_and_coef.data_ptr(), _stream(sumsq)),
             "yafsdp_clip_coef",
@@ -587,7 +603,7 @@ def flat_scale(buf: torch.Tensor, coef: torch.Tensor) -> None:
     _flat_arg(buf, "buf"), _flat_arg(coef, "coef")
     if coef.dtype != torch.float32 or coef.numel() != 1 or coef.device != buf.device:
         raise TypeError("coef must be a one-element float32 tensor on the buffer's device")
-    with torch.cuda.device(buf.device):
+    with _on(buf.device):
         _check(lib.yafsdp_flat_scale(buf.data_ptr(), _dt(buf), buf.numel(), coef.data_ptr(), _stream(buf)), "yafsdp_flat_scale")
 
 
@@ -629,7 +645,7 @@ def adamw_step(
             raise TypeError("grad_scale must be a one-element float32 tensor on the shard's device")
         gs_ptr = grad_scale.data_ptr()
     flags = (ADAM_DECOUPLED_DECAY if decoupled else 0) | (ADAM_ZERO_GRAD if zero_grad else 0)
-    with torch.cuda.device(param.device):
+    with _on(param.device):
         _check(
             lib.yafsdp_adamw_step(
                 param.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), out_ptr, out_dt, n,
