@@ -63,14 +63,15 @@ def _reference_steps(model0, xs, lr, accumulate_pairs=False, reduce_fp32=False):
             lowp = copy.deepcopy(ref).to(torch.bfloat16)
             y = lowp(x.to(torch.bfloat16))
             y.float().pow(2).mean().backward()
-            grads = [p.grad.float() if reduce_fp32 else p.grad for p in lowp.parameters()]
+            grads = [None if p.grad is None else (p.grad.float() if reduce_fp32 else p.grad) for p in lowp.parameters()]
             if acc is None:
-                acc = [g.clone() for g in grads]          # view.copy_(grad)
+                acc = [None if g is None else g.clone() for g in grads]   # view.copy_(grad)
             else:
                 for a, g in zip(acc, grads):
-                    a.add_(g)                             # view.add_(grad): bf16 result
+                    if g is not None:
+                        a.add_(g)                         # view.add_(grad): bf16 result
         for m, a in zip(masters, acc):
-            m.grad = a.float()                            # shard.copy_(chunk): exact upcast
+            m.grad = None if a is None else a.float()     # shard.copy_(chunk): exact upcast
         opt.step()
         opt.zero_grad(set_to_none=True)
     return ref
@@ -443,3 +444,74 @@ def test_custom_gradient_divide_factor():
             assert torch.equal(p.grad * 4.0, q.grad)
         opt.step(); opt_plain.step()
     torch.cuda.synchronize()
+
+
+def test_frozen_and_tied_parameters():
+    """A frozen parameter takes part in the all-gather but not in the reduce (ya_fsdp/_param_group.py:669-708,
+    ya_fsdp/_collectives.py:166-170); a parameter registered on two modules is managed once and set on both
+    (ya_fsdp/_init.py:150-189, ya_fsdp/_param.py:226-236)."""
+    model0 = _make(61)
+    model0.blocks[0].up.bias.requires_grad_(False)
+    model0.blocks[1].down.weight.requires_grad_(False)
+    model0.blocks[2].up.weight = model0.blocks[1].up.weight            # tied across two wrapped modules' parent
+    model0.blocks[2].up.bias = model0.blocks[1].up.bias
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(95 + s)) for s in range(3)]
+    want = dict(_reference_steps(model0, xs, lr=0.05).named_parameters())
+
+    from yafsdp_amd import fully_shard
+
+    model = copy.deepcopy(model0)
+    assert model.blocks[2].up.weight is model.blocks[1].up.weight
+    fully_shard(model.blocks[0], mp_policy=MP)
+    fully_shard([model.blocks[1], model.blocks[2]], mp_policy=MP)       # the tie lives inside one group
+    fully_shard(model.norm, mp_policy=MP)
+    fully_shard(model, mp_policy=MP)
+    params = list(model.parameters())
+    assert len(params) == len(list(model0.parameters()))               # the tied pair counts once
+    assert model.blocks[2].up.weight is model.blocks[1].up.weight
+    frozen = [p for p in params if not p.requires_grad]
+    assert len(frozen) == 2
+    opt = torch.optim.SGD([p for p in params if p.requires_grad], lr=0.05)
+    for x in xs:
+        model(x).float().pow(2).mean().backward()
+        assert all(p.grad is None for p in frozen)
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    got = dict(model.named_parameters())  # world size 1: every sharded parameter is the whole flattened master
+    assert set(got) == set(want)
+    for k, v in want.items():
+        assert torch.equal(got[k].detach().view(v.shape).view(torch.int32), v.detach().view(torch.int32)), k
+
+
+def test_ignored_parameters_stay_plain():
+    """ignored_params (ya_fsdp/fully_shard.py:72, ya_fsdp/_init.py:123-189) are neither sharded nor cast: they
+    keep their shape, dtype and ordinary autograd gradients."""
+    from yafsdp_amd import fully_shard
+
+    class Gained(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.Linear(128, 128)
+            self.gain = nn.Parameter(torch.full((128,), 1.5))
+
+        def forward(self, x):
+            return self.lin(x) * self.gain.to(x.dtype)  # the module itself deals with the fp32 parameter
+
+    torch.manual_seed(62)
+    model = nn.Sequential(Gained(), Gained()).to(DEV)
+    ignored = {model[0].gain, model[1].gain}
+    for m in model:
+        fully_shard(m, mp_policy=MP, ignored_params=ignored)
+    fully_shard(model, mp_policy=MP)
+    for m in model:
+        group = m._get_fsdp_state()._fsdp_param_group
+        assert len(group.fsdp_params) == 2  # weight and bias of the linear layer only
+        assert m.gain.shape == (128,) and m.gain.dtype == torch.float32 and isinstance(m.gain, nn.Parameter)
+    x = torch.randn(4, 128, device=DEV)
+    model(x).float().pow(2).mean().backward()
+    torch.cuda.synchronize()
+    for m in model:
+        assert m.gain.grad is not None and m.gain.grad.shape == (128,) and m.gain.grad.dtype == torch.float32
+        assert m.gain.dim() == 1 and m.gain.numel() == 128
+    assert all(p.grad is not None for p in model.parameters())
