@@ -63,7 +63,9 @@ const char* yafsdp_error_string(int code);
  *           all_gather_output.copy_(all_gather_input) (:56-58); the size-1-group
  *           reduce-scatter output_tensor.copy_(rs_input) (:140-150); and
  *           padded_sharded_param_grad.copy_(output_tensor) (:185).
- * Same dtype: a byte copy.  dst and src must not partially overlap. */
+ * Same dtype: a byte copy.  dst == src with equal element sizes is in place;
+ * any other overlap of the two byte ranges is refused (this holds for every
+ * flat entry point below). */
 int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, void* stream);
 
 /* buf[i] = round(buf[i] / factor) in place, only if factor > 1.

@@ -48,6 +48,21 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_set_option(2, 28) == 0
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
+    # operands that overlap without being the same buffer are refused (addresses are never dereferenced here)
+    assert L.yafsdp_flat_copy(0x10000, 1, 0x10008, 1, 64, None) == -1          # shifted by 4 elements
+    assert L.yafsdp_flat_copy(0x10000, 1, 0x10000, 0, 64, None) == -1          # same base, 2-byte over 4-byte elements
+    assert L.yafsdp_post_reduce(0x10000, 0, 0x100f0, 1, 64, 0.0, 1, None) == -1  # chunk inside the shard
+    assert L.yafsdp_flat_copy(0x10000, 1, 0x10000, 1, 64, None) == 0           # self-copy: nothing to do
+    # element counts that cannot be a real buffer are refused at table creation
+    import ctypes
+
+    import numpy as np
+
+    handle = ctypes.c_void_p()
+    huge = np.array([1 << 61, 1 << 61], dtype=np.int64)
+    assert L.yafsdp_table_create(2, huge.ctypes.data, 1 << 62, ctypes.byref(handle)) == -1
+    neg = np.array([4, -1], dtype=np.int64)
+    assert L.yafsdp_table_create(2, neg.ctypes.data, 8, ctypes.byref(handle)) == -1
 
 
 def test_no_product_module_imports_the_oracle():

@@ -85,6 +85,14 @@ int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const vo
                 hipStream_t stream) {
   if (n == 0) return YAFSDP_OK;
   if (!aligned_to(dst, item_size(dst_dt)) || !aligned_to(src, item_size(src_dt))) return YAFSDP_ERR_MISALIGNED;
+  {
+    // in place (same address, same element size) is fine: every element is read before it is written by the
+    // same lane; any other overlap of the two byte ranges has no defined result (torch's copy_ refuses it too)
+    const uintptr_t d0 = reinterpret_cast<uintptr_t>(dst), s0 = reinterpret_cast<uintptr_t>(src);
+    const uintptr_t d1 = d0 + uintptr_t(n) * item_size(dst_dt), s1 = s0 + uintptr_t(n) * item_size(src_dt);
+    const bool in_place = d0 == s0 && item_size(dst_dt) == item_size(src_dt);
+    if (!in_place && d0 < s1 && s0 < d1) return YAFSDP_ERR_INVALID_ARGUMENT;
+  }
   int64_t head = ((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / item_size(dst_dt);
   if (head > n) head = n;
   const int64_t units = (n - head) >> 3;
@@ -261,7 +269,13 @@ int yafsdp_binding_create(yafsdp_table* table, const void* const* tensor_ptrs, c
     fill_small(table, tensor_ptrs, mode, &b->small);
   } else {
     const size_t bytes = size_t(n) * (sizeof(void*) + sizeof(uint32_t));
-    std::vector<char> host(bytes);
+    std::vector<char> host;
+    try {
+      host.resize(bytes);
+    } catch (const std::bad_alloc&) {
+      delete b;
+      return YAFSDP_ERR_OUT_OF_MEMORY;
+    }
     std::memcpy(host.data(), tensor_ptrs, size_t(n) * sizeof(void*));
     uint32_t* hm = reinterpret_cast<uint32_t*>(host.data() + size_t(n) * sizeof(void*));
     for (int p = 0; p < n; p++) hm[p] = mode ? mode[p] : uint32_t(MODE_COPY);
@@ -641,17 +655,18 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
   int rc = YAFSDP_OK;
   hipError_t e = hipSuccess;
   std::vector<TileRec> tiles;
+  try {
   do {
     t->n_tensors = n_tensors;
     t->offsets.assign(size_t(n_tensors) + 1, 0);
     for (int p = 0; p < n_tensors; p++) {
-      if (numels[p] < 0) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+      if (numels[p] < 0 || numels[p] > (int64_t(1) << 60) - t->offsets[p]) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
       t->offsets[p + 1] = t->offsets[p] + numels[p];
     }
     if (rc != YAFSDP_OK) break;
     t->total = t->offsets[n_tensors];
     t->padded = padded_numel;
-    if (padded_numel < t->total) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    if (padded_numel < t->total || padded_numel > (int64_t(1) << 60)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->block = table_block_for(padded_numel, g_table_large_log2.load(std::memory_order_relaxed));
     t->tile_elems = table_tile_elems(t->block);
     const int64_t n_tiles = (padded_numel + t->tile_elems - 1) / t->tile_elems;
@@ -705,6 +720,9 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
       }
     }
   } while (false);
+  } catch (const std::bad_alloc&) {  // host-side vectors: no exception may cross the C ABI
+    rc = YAFSDP_ERR_OUT_OF_MEMORY;
+  }
   if (rc == YAFSDP_OK && e != hipSuccess) rc = int(e);
   if (rc != YAFSDP_OK) {
     table_free(t);
