@@ -1154,18 +1154,21 @@ def main() -> int:
             graph_replay = None
 
     # ---- per-kernel table (outside the timed region): each op's dispatch timed on its own
-    kernels = {}
-    for name, fn, nbytes in ops:
+    def time_alone(fn, others, reps=20):
         times = []
-        for _ in range(20):
+        for _ in range(reps):
             a, b = _event_pair()
-            step_others = [f for n2, f, _ in ops if n2 != name]
-            for f in step_others:  # evict: the other ops stream 1-2 GB through the caches
+            for f in others:  # evict: the other ops stream 1-2 GB through the caches
                 f()
             _native.time_next_launch(a, b)
             fn()
             torch.cuda.synchronize()
             times.append(a.elapsed_time(b) * 1e3)
+        return times
+
+    kernels = {}
+    for name, fn, nbytes in ops:
+        times = time_alone(fn, [f for n2, f, _ in ops if n2 != name])
         med = statistics.median(times)
         warm = []  # same op back to back: whatever fits stays in the 256 MB memory-side cache
         for _ in range(20):
@@ -1182,6 +1185,36 @@ def main() -> int:
         }
         log(f"  {name:15s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s "
             f"({100 * nbytes / med / 1e3 / HBM_PEAK_GBS:.1f}% of peak)")
+
+    # ---- the other forms of the same kernels (ya_fsdp/_param_group.py:701-708, ya_fsdp/_collectives.py:56-58, 139,
+    # 185): gradient accumulation into the reduce buffer, the first reduce of an iteration (copy instead of add),
+    # the all-gather of a size-1 group, and the pre-divide as a pass of its own
+    variants = {}
+    try:
+        d_shard_b = torch.empty_like(d_shard)
+        d_gathered_b = torch.empty_like(d_gathered)
+        d_rs_b = torch.zeros_like(d_rs)
+        add_modes = [_native.MODE_ADD] * len(numels)
+        variant_ops = [
+            ("reduce_copy_in_accumulate", lambda: table.gather_in(d_grads, d_rs_b, add_modes, None, True),
+             t * (2 + 2 * rsz) + (t_pad - t) * rsz),
+            ("post_reduce_copy", lambda: _native.post_reduce(d_shard_b, d_chunk, None, False), s * (rsz + msz)),
+            ("all_gather_size1_copy", lambda: _native.flat_copy(d_gathered_b, d_gathered), 2 * t_pad * 2),
+            ("divide_in_place", lambda: _native.flat_div(d_rs_b, 2.0), 2 * t_pad * rsz),
+        ]
+        evict = [f for _, f, _ in ops]
+        for name, fn, nbytes in variant_ops:
+            fn()
+            times = time_alone(fn, evict[:2], reps=10)
+            med = statistics.median(times)
+            variants[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
+                              "GBps": round(nbytes / med / 1e3, 1),
+                              "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+            log(f"  {name:26s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s")
+        del d_shard_b, d_gathered_b, d_rs_b
+    except Exception as exc:  # an optional leg must not cost the measurement above
+        log(f"variant table skipped: {type(exc).__name__}: {exc}")
+        variants = None
 
     # ---- CPU baseline: the oracle (reference torch-op sequence) on the host cores
     cpu_baseline = None
@@ -1281,6 +1314,7 @@ def main() -> int:
         "torch_gpu_baseline": torch_gpu,
         "graph_replay": graph_replay,
         "kernels": kernels,
+        "kernel_variants": variants,
     }
     print(json.dumps(out), flush=True)
     out_binding.close()
