@@ -60,7 +60,10 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 # Summary and commands: profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.  None = not measured.
 # "llama3-8b-layer-w8-optim": adamw_kernel, (213045.6 * 1.99946 + 372753.5 * 0.99996) KiB, scaled by the plain
 # fp32 copy of the same run; profiles/bench_llama3-8b-layer-w8-optim_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_461_600, "llama3-8b-layer-w8-optim": 817_885_000}
+# "ragged-stress-w256": gather_in_kernel<LargeMeta>, (379903.9 * 1.99992 + 710944.2 * 0.99984) KiB;
+# profiles/bench_ragged-stress-w256_hbm_traffic.md.
+MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_461_600, "llama3-8b-layer-w8-optim": 817_885_000,
+                          "ragged-stress-w256": 1_505_902_865}
 
 
 def log(*a):

@@ -27,8 +27,14 @@ constexpr int kTableBlockSmall = 64;
 constexpr int kTableBlockLarge = 128;
 constexpr int kTableLargeThresholdLog2 = 28;  // padded size above 2^28 elements: the larger workgroup
 constexpr int kTableUnroll = 2;
-constexpr bool kTableNtLoad = true;
-constexpr bool kTableNtStore = true;
+#ifndef YAFSDP_TABLE_NTL
+#define YAFSDP_TABLE_NTL true
+#endif
+#ifndef YAFSDP_TABLE_NTS
+#define YAFSDP_TABLE_NTS true
+#endif
+constexpr bool kTableNtLoad = YAFSDP_TABLE_NTL;
+constexpr bool kTableNtStore = YAFSDP_TABLE_NTS;
 inline int table_block_for(long long padded_elems, int threshold_log2) {
   return padded_elems > (1LL << threshold_log2) ? kTableBlockLarge : kTableBlockSmall;
 }
