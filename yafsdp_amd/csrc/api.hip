@@ -81,6 +81,12 @@ int grid_for(int64_t n_tiles, int blocks_per_cu, int device) {
   return g < 1 ? 1 : int(g);
 }
 
+// workgroups a table kernel needs for n tiles (see kTableXcd)
+int64_t table_blocks(int64_t n_tiles) {
+  constexpr int64_t win = kTableXcd > 0 ? int64_t(kTableXcd) * kTableXcdRun : 1;
+  return (n_tiles + win - 1) / win * win;
+}
+
 int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, float k,
                 hipStream_t stream) {
   if (n == 0) return YAFSDP_OK;
@@ -319,7 +325,7 @@ int yafsdp_gather_in_bound(yafsdp_binding* binding, void* flat, int flat_dtype, 
   float k;
   scale_plan(pre_factor, &scale, &k);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table_blocks(table->n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax)
     return int(launch_gather<SmallMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->small, flat,
                                         table->padded, table->n_tiles, k, zero_pad ? 1 : 0, grid, s));
@@ -339,7 +345,7 @@ int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat
   if (e != hipSuccess) return int(e);
   if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int grid = grid_for(table->n_slots, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table_blocks(table->n_slots), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax)
     return int(launch_scatter<SmallMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->small, flat,
                                          table->total, table->n_slots, grid, s));
@@ -670,7 +676,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     t->block = table_block_for(padded_numel, g_table_large_log2.load(std::memory_order_relaxed));
     t->tile_elems = table_tile_elems(t->block);
     const int64_t n_tiles = (padded_numel + t->tile_elems - 1) / t->tile_elems;
-    if (n_tiles > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    if (n_tiles > int64_t(INT32_MAX) - 4096) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->n_tiles = int32_t(n_tiles);
     if ((e = hipGetDevice(&t->device)) != hipSuccess) break;
     if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_offsets), t->offsets.size() * sizeof(int64_t))) != hipSuccess) break;
@@ -696,7 +702,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
       const int64_t n = t->offsets[p + 1] - t->offsets[p];
       t->slot_start[p + 1] = t->slot_start[p] + (n > 0 ? (n + t->tile_elems - 1) / t->tile_elems + 1 : 0);
     }
-    if (t->slot_start[n_tensors] > int64_t(INT32_MAX)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
+    if (t->slot_start[n_tensors] > int64_t(INT32_MAX) - 4096) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->n_slots = int32_t(t->slot_start[n_tensors]);
     if (n_tensors > kSmallMax && t->n_slots > 0) {
       tiles.resize(size_t(t->n_slots));
@@ -771,7 +777,7 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
   const int n_tiles = table->n_tiles;
-  const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table_blocks(n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax) {
     SmallMeta meta;
     fill_small(table, tensor_ptrs, mode, &meta);
@@ -805,7 +811,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   int rc = check_dyn(table, ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
   const int n_tiles = table->n_slots;
-  const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table_blocks(n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax) {
     SmallMeta meta;
     fill_small(table, ptrs, mode, &meta);

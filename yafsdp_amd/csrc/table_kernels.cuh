@@ -39,6 +39,7 @@
 //    All of it is read through the constant address space, i.e. as scalar loads.
 #pragma once
 #include "flat_kernels.cuh"
+#include "tuning.h"
 
 namespace yafsdp {
 
@@ -252,6 +253,15 @@ __device__ __forceinline__ void gather_segment(char* dst, const char* src, int64
   }
 }
 
+// Tile handled by workgroup b: b itself, or the XCD-aware permutation inside windows of kWin tiles.
+template <int kX, int kWin>
+__device__ __forceinline__ int tile_of_block(int b) {
+  if constexpr (kX == 1) return b;
+  constexpr int kRun = kWin / kX;
+  const int w = b / kWin, r = b % kWin;
+  return w * kWin + (r % kX) * kRun + r / kX;
+}
+
 // S: tensor dtype, D: flat buffer dtype.  pad_zero != 0 writes zeros to
 // [total, padded); otherwise pad lanes only see the divide (as in the
 // reference, whose pad content is whatever the buffer held).
@@ -260,7 +270,12 @@ __global__ void __launch_bounds__(BLOCK)
 gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   char* fbase = reinterpret_cast<char*>(flat);
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+  constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
+  constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
+  const int n_blocks = (n_tiles + kWin - 1) / kWin * kWin;
+  for (int b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+    const int tile = tile_of_block<kX, kWin>(b);
+    if (tile >= n_tiles) continue;
     const int64_t t0 = int64_t(tile) * kTile;
     const int64_t t1 = (t0 + kTile < padded) ? t0 + kTile : padded;
     const TileLookup rec = meta.lookup(tile, t0, kTile);
@@ -356,7 +371,12 @@ scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
   constexpr int64_t kLineElems = 128 / D::kSize;
   const char* fbase = reinterpret_cast<const char*>(flat);
   (void)total;
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+  constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
+  constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
+  const int n_blocks = (n_tiles + kWin - 1) / kWin * kWin;
+  for (int b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+    const int tile = tile_of_block<kX, kWin>(b);
+    if (tile >= n_tiles) continue;
     const ScatterLookup rec = meta.lookup_scatter(tile);
     const int p = rec.tensor;
     if (p >= meta.n_tensors) continue;

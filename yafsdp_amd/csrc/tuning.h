@@ -33,6 +33,17 @@ constexpr int kTableUnroll = 2;
 #ifndef YAFSDP_TABLE_NTS
 #define YAFSDP_TABLE_NTS true
 #endif
+// 0: workgroup b handles tile b.  X > 0: workgroups are assumed to be dealt round-robin to X XCDs, and within every
+// window of X * R tiles each XCD takes a run of R neighbouring tiles (tile = window + (b % X) * R + (b / X) % R), so
+// that neighbouring tiles, which share a cache line on the side with odd offsets, meet in one L2.
+#ifndef YAFSDP_TABLE_XCD
+#define YAFSDP_TABLE_XCD 0
+#endif
+#ifndef YAFSDP_TABLE_XCD_RUN
+#define YAFSDP_TABLE_XCD_RUN 8
+#endif
+constexpr int kTableXcd = YAFSDP_TABLE_XCD;
+constexpr int kTableXcdRun = YAFSDP_TABLE_XCD_RUN;
 constexpr bool kTableNtLoad = YAFSDP_TABLE_NTL;
 constexpr bool kTableNtStore = YAFSDP_TABLE_NTS;
 inline int table_block_for(long long padded_elems, int threshold_log2) {
