@@ -515,3 +515,25 @@ def test_ignored_parameters_stay_plain():
         assert m.gain.grad is not None and m.gain.grad.shape == (128,) and m.gain.grad.dtype == torch.float32
         assert m.gain.dim() == 1 and m.gain.numel() == 128
     assert all(p.grad is not None for p in model.parameters())
+
+
+def test_profiler_ranges_appear_only_while_a_profiler_runs():
+    """The reference's record_function ranges (ya_fsdp/_param_group.py:563, 669, 710, 740) are opened while a torch
+    profiler is running, and skipped otherwise."""
+    from torch.profiler import ProfilerActivity, profile
+
+    from yafsdp_amd._common import _NO_RANGE, profiler_range
+
+    assert profiler_range("x") is _NO_RANGE
+    model = _wrap(_make(71), mp_policy=MP)
+    x = torch.randn(4, 128, device=DEV)
+    model(x).float().sum().backward()
+    with profile(activities=[ProfilerActivity.CPU]) as prof:
+        assert profiler_range("x") is not _NO_RANGE
+        model(x).float().sum().backward()
+        torch.cuda.synchronize()
+    names = {e.name for e in prof.events()}
+    for want in ("YaFSDP::all_gather", "YaFSDP::pre_forward", "YaFSDP::post_forward", "YaFSDP::pre_backward",
+                 "YaFSDP::post_backward_reduce"):
+        assert any(n.startswith(want) for n in names), (want, sorted(n for n in names if "FSDP" in n))
+    assert profiler_range("x") is _NO_RANGE

@@ -8,6 +8,7 @@ pair with the two methods of ``ProcessGroup`` the buffer path calls.
 
 from __future__ import annotations
 
+import contextlib
 from dataclasses import dataclass
 from enum import Enum, auto
 
@@ -67,3 +68,15 @@ class ShardedState(Enum):
 def is_bw() -> bool:
     """ya_fsdp/_common.py:73-74."""
     return torch._C._current_graph_task_id() != -1
+
+
+_NO_RANGE = contextlib.nullcontext()
+
+
+def profiler_range(name: str):
+    """``torch.profiler.record_function(name)`` while a torch profiler (or an NVTX / ITT emitter) is running, a
+    shared no-op context otherwise: the ranges the reference opens around every hook cost about 7 us each on the
+    host when nobody records them."""
+    if torch.autograd.profiler._is_profiler_enabled:
+        return torch.profiler.record_function(name)
+    return _NO_RANGE

@@ -36,7 +36,6 @@ from enum import Enum, auto
 from typing import Any, Generator, Sequence
 
 import torch
-from torch.profiler import record_function
 
 from . import _native
 from ._api import MixedPrecisionPolicy
@@ -50,7 +49,7 @@ from ._collectives import (
     foreach_reduce_copy_in,
     reduce_scatter,
 )
-from ._common import FSDPMeshInfo, ShardedState, TrainingState, is_bw
+from ._common import FSDPMeshInfo, ShardedState, TrainingState, is_bw, profiler_range
 from ._layout import ShardLayout, make_layout
 from ._param import ParamModuleInfo, YaFSDPParam
 
@@ -290,7 +289,7 @@ class YaFSDPParamGroup:
         if not self.unshard_in_backward and self._training_state == TrainingState.PRE_BACKWARD:
             return
         logger.debug("%s", self._with_fqn(f"YaFSDP::{self._training_state.name.lower()}_unshard"))
-        with record_function(self._with_fqn("YaFSDP::all_gather")):
+        with profiler_range(self._with_fqn("YaFSDP::all_gather")):
             all_gather_stream = self.comm_ctx.get_all_gather_stream(async_op, self._training_state)
             data_buffer_ctx = self.data_buffer_ctx
             if (owner := data_buffer_ctx.owner) is not None and owner is not self:
@@ -338,7 +337,7 @@ class YaFSDPParamGroup:
         unshards; with the hook arguments it also registers the post-backward
         hook on the inputs and returns ``(args, kwargs)``."""
         kwargs = {} if kwargs is None else kwargs
-        with record_function(self._with_fqn("YaFSDP::pre_forward")):
+        with profiler_range(self._with_fqn("YaFSDP::pre_forward")):
             self._training_state = TrainingState.FORWARD
             self.unshard(self.unshard_async_op)
             self.wait_for_unshard()
@@ -348,7 +347,7 @@ class YaFSDPParamGroup:
 
     def post_forward(self, module: Any = None, input: Any = None, output: Any = None) -> Any:
         """ya_fsdp/_param_group.py:628-635."""
-        with record_function(self._with_fqn("YaFSDP::post_forward")):
+        with profiler_range(self._with_fqn("YaFSDP::post_forward")):
             if not is_bw():
                 self.reshard()
                 self._record_post_forward()
@@ -384,7 +383,7 @@ class YaFSDPParamGroup:
         """ya_fsdp/_param_group.py:644-653."""
         if self._training_state == TrainingState.PRE_BACKWARD:
             return
-        with record_function(self._with_fqn("YaFSDP::pre_backward")):
+        with profiler_range(self._with_fqn("YaFSDP::pre_backward")):
             self._training_state = TrainingState.PRE_BACKWARD
             self.unshard(self.unshard_async_op)
             self.wait_for_unshard()
@@ -403,7 +402,7 @@ class YaFSDPParamGroup:
                 grad_buffer_ctx.release_event = None
             grad_buffer_ctx.owner = self
         predivide_fused = False
-        with record_function(self._with_fqn("FSDP::post_backward_accumulate")):
+        with profiler_range(self._with_fqn("FSDP::post_backward_accumulate")):
             grads: list[torch.Tensor | None] = []
             modes: list[int] = []
             for fsdp_param in self.fsdp_params:
@@ -431,7 +430,7 @@ class YaFSDPParamGroup:
                     predivide_fused = True
                 foreach_reduce_copy_in(self, self._table, self._reduce_scatter_input[None], grads, modes, pre)
         fsdp_params_with_grad_per_dtype: dict[torch.dtype | None, list[YaFSDPParam]] = {}
-        with record_function(self._with_fqn("YaFSDP::post_backward_reshard")):
+        with profiler_range(self._with_fqn("YaFSDP::post_backward_reshard")):
             if not self.reduce_grads:
                 if self.reshard_after_backward:
                     self.reshard()
@@ -451,7 +450,7 @@ class YaFSDPParamGroup:
                 grad_buffer_ctx.owner = None
             return
         assert grad_buffer_ctx is not None
-        with record_function(self._with_fqn("YaFSDP::post_backward_reduce")):
+        with profiler_range(self._with_fqn("YaFSDP::post_backward_reduce")):
             for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
                 self._post_reduce_event = reduce_scatter(
                     fsdp_params,
@@ -513,7 +512,7 @@ class YaFSDPParamGroup:
             training_state = TrainingState.FORWARD
         else:
             raise ValueError(f"Unknown pass type: {pass_type}")
-        with record_function(f"YaFSDP::{pass_type}_prefetch for {target._module_fqn}"), target.use_training_state(
+        with profiler_range(f"YaFSDP::{pass_type}_prefetch for {target._module_fqn}"), target.use_training_state(
             training_state
         ):
             target.unshard(target.unshard_async_op)

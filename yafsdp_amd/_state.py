@@ -17,7 +17,7 @@ from torch.distributed.utils import _apply_to_tensors, _to_kwargs
 from torch.utils._pytree import tree_flatten
 
 from ._api import MixedPrecisionPolicy
-from ._common import TrainingState
+from ._common import TrainingState, profiler_range
 from ._param_group import YaFSDPCommContext, YaFSDPParamGroup
 
 logger = logging.getLogger("yafsdp_amd")
@@ -104,14 +104,14 @@ class YaFSDPState(_State):
         if self._state_ctx.iter_forward_root is not None:
             return args, kwargs
         self._state_ctx.iter_forward_root = self
-        with torch.profiler.record_function("YaFSDP::root_pre_forward"):
+        with profiler_range("YaFSDP::root_pre_forward"):
             if (event := self._state_ctx.post_optim_event) is not None:
                 self._comm_ctx.all_gather_stream.wait_event(event)
                 self._state_ctx.post_optim_event = None
             else:
                 # wait for the optimizer step before the implicitly prefetched unshards
                 self._comm_ctx.all_gather_stream.wait_stream(torch.cuda.current_stream(self._device))
-            with torch.profiler.record_function("YaFSDP::inputs_to_device"):
+            with profiler_range("YaFSDP::inputs_to_device"):
                 args_tuple, kwargs_tuple = _to_kwargs(args, kwargs, self._device, False)
             args, kwargs = args_tuple[0], kwargs_tuple[0]
         return args, kwargs
@@ -305,7 +305,7 @@ class YaFSDPState(_State):
         self._training_state = TrainingState.FORWARD
         args, kwargs = self._root_pre_forward(module, args, kwargs)
         if self._mp_policy.cast_forward_inputs and self._mp_policy.param_dtype:
-            with torch.profiler.record_function("YaFSDP::cast_forward_inputs"):
+            with profiler_range("YaFSDP::cast_forward_inputs"):
                 cast_fn = functools.partial(_cast_fp_tensor, self._mp_policy.param_dtype)
                 args, kwargs = _apply_to_tensors(cast_fn, args), _apply_to_tensors(cast_fn, kwargs)
         if self._fsdp_param_group:
@@ -326,7 +326,7 @@ class YaFSDPState(_State):
         if self._state_ctx.iter_forward_root is self:
             self._state_ctx.iter_forward_root = None
         if self._mp_policy.output_dtype is not None:
-            with torch.profiler.record_function("YaFSDP::cast_forward_outputs"):
+            with profiler_range("YaFSDP::cast_forward_outputs"):
                 output = _apply_to_tensors(functools.partial(_cast_fp_tensor, self._mp_policy.output_dtype), output)
         return output
 
@@ -344,7 +344,7 @@ class YaFSDPState(_State):
 
     def _root_post_backward_final_callback(self) -> None:
         """ya_fsdp/_state.py:501-532."""
-        with torch.profiler.record_function("YaFSDP::root_post_backward_callback"):
+        with profiler_range("YaFSDP::root_post_backward_callback"):
             for state in self._state_ctx.all_states:
                 group = state._fsdp_param_group
                 if group and group._training_state != TrainingState.POST_BACKWARD:
