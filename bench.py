@@ -296,7 +296,8 @@ def run_trainer(args) -> int:
     wrapped one by one with ``fully_shard`` (fp32 masters, bf16 compute), forward + backward + gradient norm +
     AdamW.  Three loops over the same model and inputs:
 
-    * ``fully_shard`` + ``FlatAdamW`` (buffer kernels; the optimizer pass also writes the next copy-in);
+    * ``fully_shard`` + ``FlatAdamW`` (buffer kernels; the post-reduce leaves the gradient norm, the optimizer pass
+      applies the clip coefficient and writes the next copy-in);
     * ``fully_shard`` + ``torch.optim.AdamW(fused=True)`` on the sharded parameters;
     * no wrapper: the same mixed precision written by hand with torch ops (``_foreach_copy_`` of the fp32 masters
       into a bf16 copy of the model, gradients copied back into fp32, fused torch AdamW).
@@ -309,7 +310,7 @@ def run_trainer(args) -> int:
     import torch.nn.functional as F
 
     from yafsdp_amd import MixedPrecisionPolicy, fully_shard
-    from yafsdp_amd.optim import FlatAdamW, clip_grad_norm_, grad_clip_coef
+    from yafsdp_amd.optim import FlatAdamW, clip_grad_norm_, enable_fused_grad_norm, grad_clip_coef
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -444,6 +445,7 @@ def run_trainer(args) -> int:
         flat = name == "fully_shard_flat_adamw"
         if flat:
             opt = FlatAdamW(params, **hyper)
+            enable_fused_grad_norm(model)  # the post-reduce also leaves the squared norm of each gradient shard
         else:
             opt = torch.optim.AdamW(params, fused=True, **hyper)
 
@@ -537,6 +539,20 @@ def run_optim(args) -> int:
         _native.flat_scale(d_g_keep, d_half)
 
     d_half = torch.full((1,), 0.5, device=dev)
+    # the post-reduce that precedes these passes in a step, without and with the fused sum of squares (which makes
+    # grad_sumsq's read pass unnecessary)
+    d_chunk = (torch.randn(s, generator=g) * 1e-3).bfloat16().to(dev)
+    d_pr = torch.zeros(s, device=dev)
+    d_pr_partials = torch.empty(_native.post_reduce_sumsq_count(s), dtype=torch.float64, device=dev)
+
+    def op_post_reduce():
+        _native.post_reduce(d_pr, d_chunk, None, True)
+
+    def op_post_reduce_sumsq():
+        count = _native.post_reduce_sumsq(d_pr, d_chunk, None, True, d_pr_partials)
+        _native.clip_coef_from_partials(d_pr_partials, count, max_norm, d_nc2)
+
+    d_nc2 = torch.zeros(2, dtype=torch.float32, device=dev)
     # the timed step leaves the gradient in place (a training step rewrites it in its backward pass); the
     # variant that zero-fills it is timed on its own below, with the gradient restored before each launch
     ops = [
@@ -544,7 +560,8 @@ def run_optim(args) -> int:
         ("adamw_step", op_adamw, s * (16 + 12 + 2)),
     ]
     extra = [("adamw_step_zero_grad", op_adamw_zero, s * (16 + 12 + 2 + 4)), ("zero_fill", op_fill, s * 4),
-             ("grad_scale", op_scale, s * 8)]
+             ("grad_scale", op_scale, s * 8), ("post_reduce", op_post_reduce, s * 10),
+             ("post_reduce_with_norm", op_post_reduce_sumsq, s * 10)]
     bytes_per_step = sum(b for _, _, b in ops)
 
     parity = "skipped"
@@ -608,7 +625,7 @@ def run_optim(args) -> int:
                 if n2 != name:
                     f()
             refresh_grad()
-            if name == "grad_sumsq":  # two launches: bracket the pair with recorded events
+            if name in ("grad_sumsq", "post_reduce_with_norm"):  # two launches: bracket the pair with recorded events
                 a.record()
                 fn()
                 b.record()
@@ -697,6 +714,10 @@ def run_optim(args) -> int:
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload), "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2),
                      "launches_timed": len(dom_us)},
         "cpu_baseline": cpu_baseline, "torch_gpu_baseline": torch_gpu, "kernels": kernels,
+        "fused_norm": {
+            "post_reduce_then_grad_sumsq_us": round(kernels["post_reduce"]["us_median"] + kernels["grad_sumsq"]["us_median"], 2),
+            "post_reduce_with_norm_us": kernels["post_reduce_with_norm"]["us_median"],
+        },
     }
     print(json.dumps(out), flush=True)
     return 0

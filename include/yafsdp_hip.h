@@ -91,6 +91,21 @@ int yafsdp_flat_div_copy(void* dst, int dst_dtype, const void* src, int src_dtyp
 int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
                        double post_factor, int accumulate, void* stream);
 
+/* yafsdp_post_reduce that also returns the sum of squares of the shard it
+ * writes, as per-workgroup partial sums in binary64 (squares of binary32
+ * numbers are exact there): the gradient norm of clip_grad_norm_
+ * (ya_fsdp/_tensor.py:220-242, ya_fsdp/ya_fsdp.py:543-562) then needs no
+ * pass of its own over the gradient shard.  partials[0 : *n_written] are
+ * written (`capacity` doubles available; at least
+ * yafsdp_post_reduce_sumsq_count(n) are needed); hand them to
+ * yafsdp_clip_coef_from_partials, alone or next to the partial sums of other
+ * shards.  The values squared are the stored ones (after rounding to the
+ * shard's dtype).  shard and chunk must not overlap. */
+int64_t yafsdp_post_reduce_sumsq_count(int64_t n);
+int yafsdp_post_reduce_sumsq(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
+                             double post_factor, int accumulate, double* partials, int64_t capacity,
+                             int64_t* n_written, void* stream);
+
 /* Same as yafsdp_post_reduce but per ragged fragment: fragment f covers
  * elements [sum(numels[:f]), sum(numels[:f+1])) of both shard and chunk and is
  * copied (YAFSDP_MODE_COPY), accumulated (YAFSDP_MODE_ADD) or left untouched
@@ -221,6 +236,15 @@ int yafsdp_sumsq_partials(const void* src, int dtype, int64_t n, double* partial
                           int64_t* n_written, void* stream);
 int yafsdp_clip_coef_from_partials(const double* partials, int64_t n_partials, double max_norm, double* sumsq,
                                    float* norm_and_coef, void* stream);
+
+/* First stage for long arrays of partial sums (many shards, or shards of
+ * hundreds of millions of elements through yafsdp_post_reduce_sumsq):
+ * out[b] = sum(partials[4096 b : 4096 (b + 1)]), b < ceil(n_partials / 4096),
+ * one workgroup each, in a fixed order; *n_written receives that count
+ * (`capacity` doubles available in `out`).  yafsdp_clip_coef_from_partials adds
+ * with a single workgroup, which is the faster way below about 16 K sums. */
+int yafsdp_sumsq_reduce_partials(const double* partials, int64_t n_partials, double* out, int64_t capacity,
+                                 int64_t* n_written, void* stream);
 
 /* norm_and_coef[0] = float(sqrt(*sumsq)); norm_and_coef[1] = min(max_norm /
  * (norm + 1e-6), 1.0), binary32 like the reference's tensors

@@ -50,9 +50,11 @@ def randn(gen: torch.Generator, n, std: float, dtype: torch.dtype) -> torch.Tens
     return (torch.randn(n, generator=gen, dtype=torch.float32) * std).to(dtype)
 
 
-def mixed_values(gen: torch.Generator, n: int, dtype: torch.dtype, std: float = 0.02) -> torch.Tensor:
-    """Seeded normal data with the special patterns spliced in at the front."""
+def mixed_values(gen: torch.Generator, n: int, dtype: torch.dtype, std: float = 0.02, specials: bool = True) -> torch.Tensor:
+    """Seeded normal data with the special patterns spliced in at the front (``specials=False``: plain finite data)."""
     x = torch.randn(n, generator=gen, dtype=torch.float32) * std
+    if not specials:
+        return x.to(dtype)
     sp = special_values_f32()
     k = min(n, sp.numel())
     x[:k] = sp[:k]

@@ -255,3 +255,117 @@ def test_plain_parameters_and_errors():
         clip_grad_norm_(nn.Linear(2, 2).to(DEV), 1.0)
     with pytest.raises(NotImplementedError):
         clip_grad_norm_(_wrap(_make(14), mp_policy=MP), 1.0, norm_type=1.0)
+
+
+def test_fused_grad_norm_matches_the_read_pass():
+    """enable_fused_grad_norm: the post-reduce leaves the squared norm of every gradient shard; grad_clip_coef adds
+    those sums up and reads a shard again only when they no longer describe its gradients."""
+    from yafsdp_amd import _native
+    from yafsdp_amd.optim import (disable_fused_grad_norm, enable_fused_grad_norm, fsdp_param_groups,
+                                  grad_clip_coef, zero_grad)
+
+    model = _wrap(_make(41), mp_policy=MP)
+    x = torch.randn(8, 128, device=DEV)
+    model(x).float().pow(2).mean().backward()  # lazy init
+    zero_grad(model)
+    model.zero_grad(set_to_none=True)
+    enable_fused_grad_norm(model)
+    groups = fsdp_param_groups(model)
+    calls = {"read": 0}
+    real = _native.sumsq_partials
+
+    def counting(*a, **k):
+        calls["read"] += 1
+        return real(*a, **k)
+
+    _native.sumsq_partials = counting
+    try:
+        model(x).float().pow(2).mean().backward()
+        assert all(g._grad_sumsq_token is not None for g in groups)
+        norm_fused, coef_fused = grad_clip_coef(model, 1e-3)
+        assert calls["read"] == 0                      # every sum came from the post-reduce
+        disable_fused_grad_norm(model)
+        norm_read, coef_read = grad_clip_coef(model, 1e-3)
+        assert calls["read"] == len(groups)
+        assert torch.allclose(norm_fused, norm_read, rtol=2e-7, atol=0) and float(norm_read) > 0
+        assert torch.allclose(coef_fused, coef_read, rtol=2e-7, atol=0)
+        # a torch op on one gradient: that group, and only that group, is read again
+        enable_fused_grad_norm(model)
+        model.zero_grad(set_to_none=True)
+        model(x).float().pow(2).mean().backward()
+        calls["read"] = 0
+        next(iter(model.blocks[1].parameters())).grad.mul_(3.0)
+        norm_a, _ = grad_clip_coef(model, 1e-3)
+        assert calls["read"] == 1
+        disable_fused_grad_norm(model)
+        norm_b, _ = grad_clip_coef(model, 1e-3)
+        assert torch.allclose(norm_a, norm_b, rtol=2e-7, atol=0) and float(norm_b) > float(norm_read)
+        # gradient accumulation: the second reduce adds into the shard and its sums describe the total
+        enable_fused_grad_norm(model)
+        model(x).float().pow(2).mean().backward()
+        calls["read"] = 0
+        norm_c, _ = grad_clip_coef(model, 1e-3)
+        assert calls["read"] == 0
+        disable_fused_grad_norm(model)
+        norm_d, _ = grad_clip_coef(model, 1e-3)
+        assert torch.allclose(norm_c, norm_d, rtol=2e-7, atol=0)
+        # set_to_none: no gradients, nothing to add up from stale sums
+        enable_fused_grad_norm(model)
+        model.zero_grad(set_to_none=True)
+        model(x).float().pow(2).mean().backward()
+        model.blocks[0].zero_grad(set_to_none=True)
+        calls["read"] = 0
+        norm_e, _ = grad_clip_coef(model, 1e-3)
+        disable_fused_grad_norm(model)
+        norm_f, _ = grad_clip_coef(model, 1e-3)
+        assert torch.allclose(norm_e, norm_f, rtol=2e-7, atol=0) and float(norm_f) < float(norm_read)
+    finally:
+        _native.sumsq_partials = real
+        disable_fused_grad_norm(model)
+
+
+def test_training_with_fused_grad_norm_equals_training_without():
+    from yafsdp_amd.optim import FlatAdamW, enable_fused_grad_norm, grad_clip_coef
+
+    model0 = _make(42)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(300 + s)) for s in range(4)]
+
+    def run(fused: bool):
+        model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+        opt = FlatAdamW(model.parameters(), lr=1e-2, weight_decay=0.1)
+        norms = []
+        for i, x in enumerate(xs):
+            model(x).float().pow(2).mean().backward()
+            if fused and i == 0:
+                enable_fused_grad_norm(model)  # after the first backward: the groups exist and hold gradients
+            norm, coef = grad_clip_coef(model, 0.05)
+            norms.append(float(norm))
+            opt.step(grad_scale=coef)
+            opt.zero_grad(set_to_none=True)
+        torch.cuda.synchronize()
+        return norms, [p.detach().clone() for p in model.parameters()]
+
+    n1, p1 = run(True)
+    n0, p0 = run(False)
+    assert n1 == pytest.approx(n0, rel=3e-7)
+    for a, b in zip(p1, p0):
+        assert torch.allclose(a, b, rtol=0, atol=2e-7)
+
+
+def test_fused_grad_norm_falls_back_when_the_reduce_writes_the_shard_directly():
+    """Without mixed precision a size-1 group reduces straight into the gradient shard
+    (ya_fsdp/_collectives.py:112-125): no post-reduce runs, so the norm is read from the shards as before."""
+    from yafsdp_amd.optim import disable_fused_grad_norm, enable_fused_grad_norm, fsdp_param_groups, grad_clip_coef
+
+    model = _wrap(_make(43))
+    x = torch.randn(8, 128, device=DEV)
+    model(x).pow(2).mean().backward()
+    enable_fused_grad_norm(model)
+    model.zero_grad(set_to_none=True)
+    model(x).pow(2).mean().backward()
+    assert all(g._grad_sumsq_token is None for g in fsdp_param_groups(model))
+    norm_a, _ = grad_clip_coef(model, 1.0)
+    disable_fused_grad_norm(model)
+    norm_b, _ = grad_clip_coef(model, 1.0)
+    want = torch.sqrt(sum(p.grad.double().pow(2).sum() for p in model.parameters())).float()
+    assert torch.allclose(norm_a, norm_b, rtol=2e-7, atol=0) and torch.allclose(norm_b, want, rtol=1e-6, atol=0)

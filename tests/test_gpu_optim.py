@@ -253,3 +253,94 @@ def test_optim_errors_are_loud(nat):
     with pytest.raises(RuntimeError):
         nat.flat_sumsq(a, out, torch.zeros(16, dtype=torch.uint8, device=DEV))
     assert nat.lib.yafsdp_flat_fill(a.data_ptr(), 7, 4, 0.0, None) == -2
+
+
+@pytest.mark.parametrize("shard_dt", DTYPES)
+@pytest.mark.parametrize("chunk_dt", DTYPES)
+@pytest.mark.parametrize("post", [None, 8.0, 3.0])
+@pytest.mark.parametrize("acc", [False, True])
+def test_post_reduce_sumsq(nat, shard_dt, chunk_dt, post, acc):
+    """The post-reduce that also returns the squared norm of the shard it writes: the shard bit for bit as
+    post_reduce gives it (and as the reference's div_ + copy_/add_ do), the partial sums adding up to the sum of
+    squares of that shard to binary64 rounding, and the clip coefficient equal to the separate norm pass's."""
+    from oracle import torch_ops
+
+    g = torch.Generator().manual_seed(301)
+    ws = nat.sumsq_workspace(torch.device(DEV))
+    for k, n in enumerate([1, 5, 8, 1023, 4096, 4097, 100_003, (1 << 21) + 13]):
+        o = k % 8  # every start residue of the shard modulo 16 bytes
+        _say("post_reduce_sumsq", shard_dt, chunk_dt, post, acc, n, o)
+        chunk = mixed_values(g, n, chunk_dt, 1e-3, specials=False)
+        shard0 = mixed_values(g, n, shard_dt, 1e-4, specials=False).flip(0).contiguous()
+        want = shard0.clone()
+        torch_ops.reduce_scatter_local(want, chunk.clone(), 1, 0, None, post, "add" if acc else "copy")
+        buf = torch.full((n + 24,), 9.0, dtype=shard_dt, device=DEV)
+        got = buf[o : o + n]
+        got.copy_(shard0)
+        count_max = nat.post_reduce_sumsq_count(n)
+        partials = torch.full((count_max + 3,), -1.0, dtype=torch.float64, device=DEV)
+        end = nat.post_reduce_sumsq(got, chunk.to(DEV), post, acc, partials, 1)
+        assert 1 < end <= 1 + count_max
+        assert_bits_equal(got, want, f"shard n={n}")
+        guard = torch.cat([buf[:o], buf[o + n :]]).float()  # lanes around the shard stay untouched
+        assert float(guard.min()) == 9.0 and float(guard.max()) == 9.0
+        assert float(partials[0]) == -1.0 and float(partials[end:].max()) == -1.0
+        total = float(partials[1:end].sum())
+        ref = cref.sumsq(want)
+        assert math.isclose(total, ref, rel_tol=1e-12, abs_tol=1e-300), (total, ref)
+        # same norm and coefficient as the separate pass over the result
+        a = torch.empty(2, dtype=torch.float32, device=DEV)
+        b = torch.empty(2, dtype=torch.float32, device=DEV)
+        nat.clip_coef_from_partials(partials[1:end], end - 1, 1e-3, a)
+        sep = torch.zeros(1, dtype=torch.float64, device=DEV)
+        nat.flat_sumsq(got, sep, ws, accumulate=False)
+        nat.clip_coef(sep, 1e-3, b)
+        av, bv = a.cpu(), b.cpu()
+        assert torch.allclose(av, bv, rtol=2e-7, atol=0.0), (av, bv)
+
+
+def test_post_reduce_sumsq_special_values_and_errors(nat):
+    # a NaN or an infinity in the result makes the norm non-finite, as torch's norm would
+    chunk = torch.tensor([1.0, float("inf"), 2.0, 3.0, 0.5, 0.25, 7.0, 8.0, 9.0], device=DEV).bfloat16()
+    shard = torch.zeros(9, device=DEV)
+    partials = torch.zeros(4, dtype=torch.float64, device=DEV)
+    end = nat.post_reduce_sumsq(shard, chunk, None, False, partials)
+    assert end == 1 and math.isinf(float(partials[0]))
+    assert torch.equal(shard.cpu(), chunk.float().cpu())
+    chunk[1] = float("nan")
+    nat.post_reduce_sumsq(shard, chunk, None, True, partials)
+    assert math.isnan(float(partials[0]))
+    # empty shard: nothing written, nothing launched
+    assert nat.post_reduce_sumsq(shard[:0], chunk[:0], None, False, partials, 2) == 2
+    big = torch.zeros(1 << 16, device=DEV)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        nat.post_reduce_sumsq(big, big.bfloat16(), None, False, partials[:1])  # needs 16 partial sums
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        nat.post_reduce_sumsq(big[:64], big[32:96], None, False, partials)      # overlapping operands
+    with pytest.raises(TypeError):
+        nat.post_reduce_sumsq(shard, chunk, None, False, partials.float())
+    assert nat.post_reduce_sumsq_count(0) == 0 and nat.post_reduce_sumsq_count(1) == 1
+    assert nat.post_reduce_sumsq_count(1 << 16) == 16
+
+
+def test_sumsq_reduce_partials(nat):
+    """The many-workgroup first stage for long arrays of partial sums: each output is the sum of 4096 consecutive
+    inputs, and norm / coefficient through the two stages equal those of the single-workgroup finish."""
+    g = torch.Generator().manual_seed(401)
+    for n in [1, 4095, 4096, 4097, 250_001]:
+        x = torch.rand(n, generator=g, dtype=torch.float64) * 1e-3
+        d = x.to(DEV)
+        out = torch.full(((n + 4095) // 4096 + 2,), -1.0, dtype=torch.float64, device=DEV)
+        count = nat.sumsq_reduce_partials(d, n, out)
+        assert count == (n + 4095) // 4096 and float(out[count:].max()) == -1.0
+        want = torch.stack([c.sum() for c in x.split(4096)])
+        assert torch.allclose(out[:count].cpu(), want, rtol=1e-13, atol=0)
+        a = torch.empty(2, dtype=torch.float32, device=DEV)
+        b = torch.empty(2, dtype=torch.float32, device=DEV)
+        nat.clip_coef_from_partials(out, count, 0.01, a)
+        nat.clip_coef_from_partials(d, n, 0.01, b)
+        assert torch.allclose(a, b, rtol=2e-7, atol=0), (a, b)
+        assert math.isclose(float(a[0]), math.sqrt(float(x.sum())), rel_tol=1e-6)
+    with pytest.raises(RuntimeError, match="invalid argument"):
+        nat.sumsq_reduce_partials(torch.zeros(10000, dtype=torch.float64, device=DEV), 10000,
+                                  torch.zeros(2, dtype=torch.float64, device=DEV))

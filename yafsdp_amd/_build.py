@@ -13,8 +13,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libyafsdp_hip.so")
-SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip", "fan.hip"]
-HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "optim_kernels.cuh", "fan_kernels.cuh", "launch.h", "tuning.h"]
+SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip", "fan.hip", "postsumsq.hip"]
+HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "optim_kernels.cuh", "fan_kernels.cuh",
+           "post_sumsq_kernels.cuh", "launch.h", "tuning.h"]
 ARCH = "gfx950"
 
 # -ffp-contract=off: every multiply and add of the path rounds on its own, as
@@ -45,7 +46,7 @@ def _compile(src: str, obj: str) -> None:
         print(err)
 
 
-def build(force: bool = True, jobs: int = 6) -> str:
+def build(force: bool = True, jobs: int = 7) -> str:
     """Compile every translation unit and link the shared library."""
     srcs = [os.path.join(CSRC, s) for s in SOURCES + HEADERS] + [os.path.join(HERE, "..", "include", "yafsdp_hip.h")]
     if not force and os.path.exists(OUT) and all(os.path.getmtime(OUT) >= os.path.getmtime(s) for s in srcs):

@@ -223,9 +223,15 @@ def reduce_scatter(
             output_tensor = chunk
         # post-divide (:165) fused with the copy / accumulate into the gradient shard (:166-214)
         post = postdivide_factor if collective_divide is None else collective_divide
+        group_ref = getattr(fsdp_params[0], "_param_group_ref", None) if fsdp_params else None
+        param_group = group_ref() if group_ref is not None else None
+        # every parameter of the group gets a gradient in this pass: the whole shard is meaningful afterwards
+        whole = len(fsdp_params_with_grad) == len(fsdp_params)
+        if param_group is not None:
+            param_group._grad_sumsq_token = None
         if world_size > 1 and reduce_in_sharded:
             # the collective would have written straight into the shard (:124-125)
-            _native.post_reduce(padded_sharded_param_grad, chunk, post, False)
+            _post_reduce(param_group, whole, padded_sharded_param_grad, chunk, post, False)
         elif world_size == 1 and reduce_in_sharded:
             _div_if_needed(padded_sharded_param_grad, post)
         else:
@@ -233,9 +239,9 @@ def reduce_scatter(
             without_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is None]
             with_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is not None]
             if len(without_sharded_grad) == len(fsdp_params_which_require_grad):
-                _native.post_reduce(padded_sharded_param_grad, output_tensor, post, False)  # :185
+                _post_reduce(param_group, whole, padded_sharded_param_grad, output_tensor, post, False)  # :185
             elif len(with_sharded_grad) == len(fsdp_params_which_require_grad):
-                _native.post_reduce(padded_sharded_param_grad, output_tensor, post, True)  # :189
+                _post_reduce(param_group, whole, padded_sharded_param_grad, output_tensor, post, True)  # :189
             else:
                 with_ids = {id(p) for p in with_sharded_grad}
                 without_ids = {id(p) for p in without_sharded_grad}
@@ -249,6 +255,22 @@ def reduce_scatter(
         for fsdp_param in fsdp_params_with_grad:
             fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad  # :216-217
         return post_reduce_event
+
+
+def _post_reduce(
+    param_group: "YaFSDPParamGroup | None", whole: bool, shard: torch.Tensor, chunk: torch.Tensor,
+    post: float | None, accumulate: bool,
+) -> None:
+    """``post_reduce``; for a group with a slot for partial sums of squares
+    (``optim.enable_fused_grad_norm``) and a pass that gives every parameter
+    its gradient, the variant that also leaves the squared norm of the shard."""
+    slot = param_group._grad_sumsq_slot if param_group is not None else None
+    if slot is None or not whole:
+        _native.post_reduce(shard, chunk, post, accumulate)
+        return
+    lo, hi = slot
+    _native.post_reduce_sumsq(shard, chunk, post, accumulate, param_group._grad_sumsq_partials[:hi], lo)
+    param_group._grad_sumsq_token = shard._version
 
 
 def _get_gradient_divide_factors(

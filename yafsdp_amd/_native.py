@@ -42,6 +42,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_flat_div",
     "yafsdp_flat_div_copy",
     "yafsdp_post_reduce",
+    "yafsdp_post_reduce_sumsq_count",
+    "yafsdp_post_reduce_sumsq",
     "yafsdp_post_reduce_fragments",
     "yafsdp_table_create",
     "yafsdp_table_destroy",
@@ -58,6 +60,7 @@ EXPORTED_SYMBOLS = (
     "yafsdp_sumsq_workspace_bytes",
     "yafsdp_flat_sumsq",
     "yafsdp_sumsq_partials",
+    "yafsdp_sumsq_reduce_partials",
     "yafsdp_clip_coef_from_partials",
     "yafsdp_clip_coef",
     "yafsdp_flat_scale",
@@ -88,6 +91,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_flat_div_copy.argtypes = [vp, i32, vp, i32, i64, dbl, vp]
     lib.yafsdp_post_reduce.restype = i32
     lib.yafsdp_post_reduce.argtypes = [vp, i32, vp, i32, i64, dbl, i32, vp]
+    lib.yafsdp_post_reduce_sumsq_count.restype = i64
+    lib.yafsdp_post_reduce_sumsq_count.argtypes = [i64]
+    lib.yafsdp_post_reduce_sumsq.restype = i32
+    lib.yafsdp_post_reduce_sumsq.argtypes = [vp, i32, vp, i32, i64, dbl, i32, vp, i64, ctypes.POINTER(i64), vp]
     lib.yafsdp_post_reduce_fragments.restype = i32
     lib.yafsdp_post_reduce_fragments.argtypes = [vp, i32, vp, i32, i32, vp, vp, dbl, vp]
     lib.yafsdp_table_create.restype = i32
@@ -120,6 +127,8 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_flat_sumsq.argtypes = [vp, i32, i64, vp, i32, vp, ctypes.c_size_t, vp]
     lib.yafsdp_sumsq_partials.restype = i32
     lib.yafsdp_sumsq_partials.argtypes = [vp, i32, i64, vp, i64, ctypes.POINTER(i64), vp]
+    lib.yafsdp_sumsq_reduce_partials.restype = i32
+    lib.yafsdp_sumsq_reduce_partials.argtypes = [vp, i64, vp, i64, ctypes.POINTER(i64), vp]
     lib.yafsdp_clip_coef_from_partials.restype = i32
     lib.yafsdp_clip_coef_from_partials.argtypes = [vp, i64, dbl, vp, vp, vp]
     lib.yafsdp_clip_coef.restype = i32
@@ -236,6 +245,36 @@ def post_reduce(shard: torch.Tensor, chunk: torch.Tensor, post_factor: float | N
             ),
             "yafsdp_post_reduce",
         )
+
+
+def post_reduce_sumsq_count(numel: int) -> int:
+    """Partial sums ``post_reduce_sumsq`` writes at most for a shard of ``numel`` elements."""
+    return int(lib.yafsdp_post_reduce_sumsq_count(int(numel)))
+
+
+def post_reduce_sumsq(
+    shard: torch.Tensor, chunk: torch.Tensor, post_factor: float | None, accumulate: bool, partials: torch.Tensor,
+    offset: int = 0,
+) -> int:
+    """``post_reduce`` that also writes the per-workgroup sums of squares of the resulting shard into
+    ``partials[offset:]`` (float64); returns the new offset."""
+    _flat_arg(shard, "shard"), _flat_arg(chunk, "chunk"), _flat_arg(partials, "partials")
+    if shard.numel() != chunk.numel():
+        raise ValueError(f"numel mismatch: {shard.numel()} vs {chunk.numel()}")
+    if partials.dtype != torch.float64 or partials.device != shard.device:
+        raise TypeError("partials must be a float64 tensor on the shard's device")
+    capacity = partials.numel() - offset
+    written = ctypes.c_int64()
+    with _on(shard.device):
+        _check(
+            lib.yafsdp_post_reduce_sumsq(
+                shard.data_ptr(), _dt(shard), chunk.data_ptr(), _dt(chunk), shard.numel(), _factor(post_factor),
+                int(bool(accumulate)), partials.data_ptr() + 8 * offset, max(capacity, 0), ctypes.byref(written),
+                _stream(shard),
+            ),
+            "yafsdp_post_reduce_sumsq",
+        )
+    return offset + written.value
 
 
 def post_reduce_fragments(
@@ -565,6 +604,25 @@ def sumsq_partials(src: torch.Tensor, partials: torch.Tensor, offset: int) -> in
             "yafsdp_sumsq_partials",
         )
     return offset + written.value
+
+
+def sumsq_reduce_partials(partials: torch.Tensor, count: int, out: torch.Tensor) -> int:
+    """``out[b] = sum(partials[4096 b : 4096 (b + 1)])`` over the first ``count`` partial sums; returns how many
+    sums ``out`` now holds."""
+    _flat_arg(partials, "partials"), _flat_arg(out, "out")
+    if partials.dtype != torch.float64 or out.dtype != torch.float64:
+        raise TypeError("partial sums are float64")
+    if count > partials.numel():
+        raise ValueError("count exceeds the partials buffer")
+    written = ctypes.c_int64()
+    with _on(partials.device):
+        _check(
+            lib.yafsdp_sumsq_reduce_partials(
+                partials.data_ptr(), int(count), out.data_ptr(), out.numel(), ctypes.byref(written), _stream(partials)
+            ),
+            "yafsdp_sumsq_reduce_partials",
+        )
+    return written.value
 
 
 def clip_coef_from_partials(

@@ -186,6 +186,11 @@ class YaFSDPParamGroup:
         # version of the master shard at which a fused optimizer step last wrote the
         # all-gather input (None: never); see all_gather
         self._copy_in_shard_version: int | None = None
+        # gradient norm fused into the post-reduce (optim.enable_fused_grad_norm): float64 buffer of partial sums,
+        # this group's slice of it, and the version of the gradient shard those sums describe
+        self._grad_sumsq_partials: torch.Tensor | None = None
+        self._grad_sumsq_slot: tuple[int, int] | None = None
+        self._grad_sumsq_token: int | None = None
 
     # ------------------------------------------------------------ initialisation --
     def _init_mp_dtypes(self) -> None:

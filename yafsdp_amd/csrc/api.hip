@@ -509,6 +509,21 @@ int yafsdp_clip_coef_from_partials(const double* partials, int64_t n_partials, d
                                  static_cast<hipStream_t>(stream)));
 }
 
+int yafsdp_sumsq_reduce_partials(const double* partials, int64_t n_partials, double* out, int64_t capacity,
+                                 int64_t* n_written, void* stream) {
+  if (n_partials < 0 || n_written == nullptr || (n_partials > 0 && (partials == nullptr || out == nullptr)))
+    return YAFSDP_ERR_INVALID_ARGUMENT;
+  *n_written = 0;
+  if (n_partials == 0) return YAFSDP_OK;
+  if (!aligned_to(partials, 8) || !aligned_to(out, 8)) return YAFSDP_ERR_MISALIGNED;
+  const int64_t grid = (n_partials + 4095) / 4096;
+  if (grid > capacity || grid > int64_t(INT32_MAX)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  const hipError_t e = launch_sumsq_reduce(partials, n_partials, out, int(grid), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return int(e);
+  *n_written = grid;
+  return YAFSDP_OK;
+}
+
 int yafsdp_clip_coef(const double* sumsq, double max_norm, float* norm_and_coef, void* stream) {
   if (sumsq == nullptr || norm_and_coef == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (!aligned_to(sumsq, 8) || !aligned_to(norm_and_coef, 4)) return YAFSDP_ERR_MISALIGNED;
@@ -616,6 +631,44 @@ int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chun
   }
   return flat_launch(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, chunk, n, k,
                      static_cast<hipStream_t>(stream));
+}
+
+int64_t yafsdp_post_reduce_sumsq_count(int64_t n) {
+  if (n <= 0) return 0;
+  const int64_t tile = int64_t(kFlatBlock) * kFlatUnroll;
+  const int64_t n_tiles = ((n >> 3) + tile - 1) / tile;  // the peeled head can only lower the unit count
+  return n_tiles < 1 ? 1 : n_tiles;
+}
+
+int yafsdp_post_reduce_sumsq(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
+                             double post_factor, int accumulate, double* partials, int64_t capacity,
+                             int64_t* n_written, void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || n_written == nullptr || (n > 0 && (shard == nullptr || chunk == nullptr || partials == nullptr)))
+    return YAFSDP_ERR_INVALID_ARGUMENT;
+  *n_written = 0;
+  if (n == 0) return YAFSDP_OK;
+  if (!aligned_to(shard, item_size(shard_dtype)) || !aligned_to(chunk, item_size(chunk_dtype)) ||
+      !aligned_to(partials, 8))
+    return YAFSDP_ERR_MISALIGNED;
+  {
+    const uintptr_t d0 = reinterpret_cast<uintptr_t>(shard), s0 = reinterpret_cast<uintptr_t>(chunk);
+    const uintptr_t d1 = d0 + uintptr_t(n) * item_size(shard_dtype), s1 = s0 + uintptr_t(n) * item_size(chunk_dtype);
+    if (d0 < s1 && s0 < d1) return YAFSDP_ERR_INVALID_ARGUMENT;
+  }
+  const int head = head_elems(shard, item_size(shard_dtype), n);
+  const int64_t tile = int64_t(kFlatBlock) * kFlatUnroll;
+  int64_t n_tiles = (((n - head) >> 3) + tile - 1) / tile;
+  if (n_tiles < 1) n_tiles = 1;  // workgroup 0 handles head and tail
+  if (n_tiles > capacity || n_tiles > int64_t(INT32_MAX)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  scale_plan(post_factor, &scale, &k);
+  const hipError_t e = launch_post_reduce_sumsq(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, chunk, n, head,
+                                                k, partials, int(n_tiles), static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return int(e);
+  *n_written = n_tiles;
+  return YAFSDP_OK;
 }
 
 int yafsdp_post_reduce_fragments(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int n_fragments,

@@ -303,4 +303,22 @@ __device__ __forceinline__ float post_elem(float s, float d_old, float k) {
   return y;  // caller rounds to D on store
 }
 
+// Sum of one binary64 value per lane over a workgroup of BLOCK lanes, in a fixed
+// order (wave shuffles, then the waves' sums through `lds[BLOCK / 64]`).  Valid
+// in thread 0.
+template <int BLOCK>
+__device__ __forceinline__ double block_sum(double v, double* lds) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  double t = 0.0;
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int w = 0; w < BLOCK / 64; w++) t += lds[w];
+  }
+  return t;
+}
+
 }  // namespace yafsdp

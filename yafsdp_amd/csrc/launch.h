@@ -34,6 +34,10 @@ inline hipError_t launch_kernel(void (*kernel)(Params...), int grid, int block, 
 // dst[i] = post_elem(src[i], dst[i]); scale is SCALE_NONE / SCALE_MUL / SCALE_DIV
 hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,
                        float k, int grid, hipStream_t stream);
+// the same pass, also writing partials[0:grid] = per-workgroup sums of squares of the stored values (postsumsq.hip);
+// grid must equal the number of tiles
+hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n,
+                                    int head, float k, double* partials, int grid, hipStream_t stream);
 
 // META is SmallMeta or LargeMeta (explicitly instantiated in gather.hip / scatter.hip);
 // `block` is the workgroup size the table was built for (kTableBlockSmall or kTableBlockLarge)
@@ -78,6 +82,8 @@ hipError_t launch_sumsq_partials(int dt, const void* src, int64_t n, int head, d
 // sumsq[0] (+)= sum(partials[0:count]) (if given); norm_and_coef = {norm, clip coefficient} (if given)
 hipError_t launch_sumsq_finish(const double* partials, int64_t count, double* sumsq, int accumulate, float max_norm,
                                float* norm_and_coef, hipStream_t stream);
+// out[b] = sum(in[b * 4096 : (b + 1) * 4096]) for b < grid = ceil(count / 4096)
+hipError_t launch_sumsq_reduce(const double* in, int64_t count, double* out, int grid, hipStream_t stream);
 hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and_coef, hipStream_t stream);
 hipError_t launch_adamw(int out_dt, float* p, float* g, float* m, float* v, void* out16, int64_t n, int head,
                         const AdamScalars& s, const float* grad_scale, int grid, hipStream_t stream);

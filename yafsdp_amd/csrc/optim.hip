@@ -57,6 +57,10 @@ hipError_t launch_sumsq_finish(const double* partials, int64_t count, double* su
                        norm_and_coef);
 }
 
+hipError_t launch_sumsq_reduce(const double* in, int64_t count, double* out, int grid, hipStream_t stream) {
+  return launch_kernel(sumsq_reduce_kernel<1024>, grid, 1024, stream, in, count, out);
+}
+
 hipError_t launch_clip_coef(const double* sumsq, float max_norm, float* norm_and_coef, hipStream_t stream) {
   return launch_kernel(clip_coef_kernel, 1, 64, stream, sumsq, max_norm, norm_and_coef);
 }

@@ -117,21 +117,6 @@ scale_kernel(void* buf0, int64_t n0, int head, const float* coef) {
 // from run to run.  (Folding the final sum into this kernel with a last-
 // workgroup ticket was measured: the agent-scope release/acquire that it needs
 // per workgroup makes the pass ten times slower.)
-template <int BLOCK>
-__device__ __forceinline__ double block_sum(double v, double* lds) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  if (lane == 0) lds[wave] = v;
-  __syncthreads();
-  double t = 0.0;
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int w = 0; w < BLOCK / 64; w++) t += lds[w];
-  }
-  return t;  // valid in thread 0
-}
-
 template <class S, int BLOCK, int U, bool NTL>
 __global__ void __launch_bounds__(BLOCK)
 sumsq_kernel(const void* src0, int64_t n0, int head, double* partials) {
@@ -181,6 +166,27 @@ sumsq_kernel(const void* src0, int64_t n0, int head, double* partials) {
   }
   const double t = block_sum<BLOCK>((acc[0] + acc[1]) + (acc[2] + acc[3]), lds);
   if (threadIdx.x == 0) partials[blockIdx.x] = t;
+}
+
+// First stage for long arrays of partial sums: workgroup b adds in[b * kChunk : (b + 1) * kChunk] (bounded by count)
+// in a fixed order and writes out[b].
+constexpr int kSumsqReduceChunk = 4096;
+template <int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+sumsq_reduce_kernel(const double* in, int64_t count, double* out) {
+  __shared__ double lds[BLOCK / 64];
+  const int64_t base = int64_t(blockIdx.x) * kSumsqReduceChunk;
+  double acc[kSumsqReduceChunk / BLOCK];
+#pragma unroll
+  for (int j = 0; j < kSumsqReduceChunk / BLOCK; j++) {
+    const int64_t i = base + threadIdx.x + int64_t(j) * BLOCK;
+    acc[j] = i < count ? in[i] : 0.0;
+  }
+  double v = acc[0];
+#pragma unroll
+  for (int j = 1; j < kSumsqReduceChunk / BLOCK; j++) v += acc[j];
+  const double t = block_sum<BLOCK>(v, lds);
+  if (threadIdx.x == 0) out[blockIdx.x] = t;
 }
 
 // One workgroup adds `count` partial sums in a fixed order:

@@ -33,7 +33,8 @@ from ._param import YaFSDPParam
 from ._param_group import YaFSDPParamGroup
 from ._state import _get_module_fsdp_state
 
-__all__ = ["FlatAdamW", "clip_grad_norm_", "grad_clip_coef", "zero_grad", "fsdp_param_groups"]
+__all__ = ["FlatAdamW", "clip_grad_norm_", "grad_clip_coef", "zero_grad", "fsdp_param_groups",
+           "enable_fused_grad_norm", "disable_fused_grad_norm"]
 
 
 def fsdp_param_groups(modules: nn.Module | Iterable[nn.Module]) -> list[YaFSDPParamGroup]:
@@ -127,6 +128,54 @@ class _ClipState:
         return self.partials
 
 
+def enable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
+    """From now on the post-reduce of every ``fully_shard`` group under
+    ``modules`` also leaves the partial sums of squares of the gradient shard it
+    writes (``yafsdp_post_reduce_sumsq``), and ``grad_clip_coef`` /
+    ``clip_grad_norm_`` over the same ``modules`` add those up instead of
+    reading the shards again: 4 bytes per element less per step.  A group
+    falls back to the read pass whenever its sums do not describe its current
+    gradients: a parameter without a gradient, a torch op on a gradient since
+    the reduce (seen through the shard's version counter), or one of this
+    module's own passes that rewrites gradients (scaling, zero-fill).  Kernels
+    launched on the gradient shard through ``_native`` directly are not seen."""
+    groups = [g for g in fsdp_param_groups(modules) if g._padded_sharded_param_grad[None] is not None]
+    if not groups:
+        raise ValueError("no fully_shard parameter group with gradients under the given modules")
+    device = groups[0].device
+    slots, total = [], 0
+    for g in groups:
+        n = _native.post_reduce_sumsq_count(g._padded_sharded_param_grad[None].numel())
+        slots.append((total, total + n))
+        total += n
+    partials = torch.zeros(total, dtype=torch.float64, device=device)
+    for g, slot in zip(groups, slots):
+        g._grad_sumsq_partials, g._grad_sumsq_slot, g._grad_sumsq_token = partials, slot, None
+
+
+def disable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
+    for g in fsdp_param_groups(modules):
+        g._grad_sumsq_partials, g._grad_sumsq_slot, g._grad_sumsq_token = None, None, None
+
+
+def _invalidate_grad_sumsq(groups: Iterable[YaFSDPParamGroup]) -> None:
+    for g in groups:
+        g._grad_sumsq_token = None
+
+
+def _fused_partials(groups: Sequence[YaFSDPParamGroup]) -> torch.Tensor | None:
+    """The shared buffer of partial sums if exactly these groups fill it, slot after slot."""
+    partials = groups[0]._grad_sumsq_partials
+    if partials is None:
+        return None
+    end = 0
+    for g in groups:
+        if g._grad_sumsq_partials is not partials or g._grad_sumsq_slot is None or g._grad_sumsq_slot[0] != end:
+            return None
+        end = g._grad_sumsq_slot[1]
+    return partials if end == partials.numel() else None
+
+
 def grad_clip_coef(
     modules: nn.Module | Iterable[nn.Module], max_norm: float, norm_type: float = 2.0
 ) -> tuple[torch.Tensor, torch.Tensor]:
@@ -142,12 +191,34 @@ def grad_clip_coef(
     if not groups:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
     device = groups[0].device
+    norm_and_coef = torch.empty(2, dtype=torch.float32, device=device)
+    fused = _fused_partials(groups)
+    if fused is not None:
+        # sums left by the post-reduce where they still describe the gradients; a read pass into the group's own
+        # slot (zeroed first: it may write fewer sums than the slot holds) where they do not
+        for g in groups:
+            grad_shard = g._padded_sharded_param_grad[None]
+            ranges = _grad_ranges(g)
+            if ranges == [(0, grad_shard.numel())] and g._grad_sumsq_token == grad_shard._version:
+                continue
+            lo, hi = g._grad_sumsq_slot
+            fused[lo:hi].zero_()
+            pos = lo
+            for a, b in ranges:
+                pos = _native.sumsq_partials(grad_shard[a:b], fused[:hi], pos)
+            g._grad_sumsq_token = None
+        if fused.numel() > 4 * _native.SUMSQ_MAX_PARTIALS:  # long array: many workgroups first, then one
+            scratch = _ClipState.get(device).reserve(1 + fused.numel() // (4096 * _native.SUMSQ_MAX_PARTIALS))
+            count = _native.sumsq_reduce_partials(fused, fused.numel(), scratch)
+            _native.clip_coef_from_partials(scratch, count, max_norm, norm_and_coef)
+        else:
+            _native.clip_coef_from_partials(fused, fused.numel(), max_norm, norm_and_coef)
+        return norm_and_coef[0], norm_and_coef[1]
     work = [(g._padded_sharded_param_grad[None], lo, hi) for g in groups for lo, hi in _grad_ranges(g)]
     partials = _ClipState.get(device).reserve(max(len(work), 1))
     count = 0
     for grad_shard, lo, hi in work:
         count = _native.sumsq_partials(grad_shard[lo:hi], partials, count)
-    norm_and_coef = torch.empty(2, dtype=torch.float32, device=device)
     _native.clip_coef_from_partials(partials, count, max_norm, norm_and_coef)
     return norm_and_coef[0], norm_and_coef[1]
 
@@ -165,6 +236,7 @@ def clip_grad_norm_(
         grad_shard = group._padded_sharded_param_grad[None]
         if grad_shard is None:
             continue
+        group._grad_sumsq_token = None  # the gradients are rewritten
         for lo, hi in _grad_ranges(group):
             _native.flat_scale(grad_shard[lo:hi], coef)
     return total_norm
@@ -175,6 +247,7 @@ def zero_grad(modules: nn.Module | Iterable[nn.Module]) -> None:
     for group in fsdp_param_groups(modules):
         grad_shard = group._padded_sharded_param_grad[None]
         if grad_shard is not None:
+            group._grad_sumsq_token = None
             _native.flat_fill(grad_shard, 0.0)
 
 
@@ -343,6 +416,8 @@ class FlatAdamW(torch.optim.Optimizer):
                         runs[-1] = (runs[-1][0], hi, unit.steps[k])
                     else:
                         runs.append((lo, hi, unit.steps[k]))
+        if zero_grad:
+            group._grad_sumsq_token = None  # the gradients are rewritten
         for lo, hi, step in runs:
             _native.adamw_step(
                 shard[lo:hi], grad_shard[lo:hi], unit.exp_avg[lo:hi], unit.exp_avg_sq[lo:hi],
