@@ -122,6 +122,38 @@ int main(void) {
   HIP(hipMemcpy(h_shard, d_shard, (size_t)s * 4, hipMemcpyDeviceToHost));
   if (!same("post_reduce bf16 /3 += f32", h_shard, h_shard_want, (size_t)s * 4)) return 1;
 
+  /* ---- the same post-reduce through the entry point that also leaves the squared norm of the shard */
+  {
+    float* d_shard2;
+    double* d_part;
+    const int64_t cap = yafsdp_post_reduce_sumsq_count(s);
+    int64_t n_part = 0;
+    HIP(hipMalloc((void**)&d_shard2, (size_t)s * 4));
+    HIP(hipMalloc((void**)&d_part, (size_t)cap * 8));
+    for (int64_t i = 0; i < s; i++) h_shard[i] = h_shard_want[i];  /* start from the first result: accumulate again */
+    float* h_twice = malloc((size_t)s * 4);
+    memcpy(h_twice, h_shard_want, (size_t)s * 4);
+    ref_post_reduce(h_twice, YAFSDP_F32, h_grads[0], YAFSDP_BF16, s, 3.0, 1);
+    HIP(hipMemcpy(d_shard2, h_shard, (size_t)s * 4, hipMemcpyHostToDevice));
+    YA(yafsdp_post_reduce_sumsq(d_shard2, YAFSDP_F32, d_grads[0], YAFSDP_BF16, s, 3.0, 1, d_part, cap, &n_part, stream));
+    HIP(hipStreamSynchronize(stream));
+    HIP(hipMemcpy(h_shard, d_shard2, (size_t)s * 4, hipMemcpyDeviceToHost));
+    if (!same("post_reduce_sumsq shard", h_shard, h_twice, (size_t)s * 4)) return 1;
+    double* h_part = malloc((size_t)cap * 8);
+    HIP(hipMemcpy(h_part, d_part, (size_t)n_part * 8, hipMemcpyDeviceToHost));
+    double got = 0.0;
+    for (int64_t i = 0; i < n_part; i++) got += h_part[i];
+    const double want = ref_sumsq(h_twice, YAFSDP_F32, s);
+    if (n_part < 1 || n_part > cap || fabs(got - want) > 1e-12 * want) {
+      printf("MISMATCH post_reduce_sumsq: %lld sums, %.17g vs %.17g\n", (long long)n_part, got, want);
+      return 1;
+    }
+    printf("ok post_reduce_sumsq %.17g in %lld partial sums\n", got, (long long)n_part);
+    free(h_twice); free(h_part);
+    HIP(hipFree(d_shard2)); HIP(hipFree(d_part));
+    memcpy(h_shard, h_shard_want, (size_t)s * 4);
+  }
+
   /* ---- gradient norm, clip coefficient, fused AdamW with bf16 copy-in */
   double want_sumsq = ref_sumsq(h_shard_want, YAFSDP_F32, s);
   float want_nc[2];
