@@ -5,6 +5,8 @@ compared element for element with the oracle.  Config 3 (Llama-3-70B layer,
 W=64; 856 M elements) is checked through size-independent properties at full
 size (round trips, linearity of the divide, pad zero-fill, checksums) and
 against the oracle on the last rank's shard, which holds the pad lanes.
+Config 4 (the full 8B model) adds the embedding / head group (525 M elements,
+one tensor) and the final-norm group (4096 elements) to config 2's layers.
 Inputs are generated on the GPU from a fixed seed and copied to the host for
 the oracle, so both sides see the same bits.
 """
@@ -231,4 +233,68 @@ def test_config5_ragged_stress_w256(nat, which):
             want = torch.zeros(s, dtype=ag_dt)
             torch_ops.copy_in(want, master.cpu())
             assert_bits_equal(ag_in, want, f"copy-in rank {r}")
+    table.close()
+
+
+def test_config4_full_8b_groups_besides_the_decoder_layers(nat):
+    """Config 4 (the full Llama-3-8B at W=8) adds three groups to the 32 decoder layers of config 2: the token
+    embedding and the output head (one [128256, 4096] tensor each: T = 525,336,576, S = 65,667,072) and the final
+    norm ([4096]: S = 512).  The large group is checked through size-independent properties at full size and against
+    the oracle on one rank's shard, the small one element for element on every rank."""
+    print("config 4: embedding / head group", flush=True)
+    numels = [128256 * 4096]
+    w, r = 8, 5
+    lay = make_layout(numels, w, 512)
+    t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+    assert (t, t_pad, s) == (525_336_576, 525_336_576, 65_667_072)
+    gen = torch.Generator(device=DEV).manual_seed(1004)
+    gathered = _randn_dev(t_pad, 0.02, torch.bfloat16, gen)
+    table = nat.TensorTable(numels, t_pad, DEV)
+    out = torch.full((t,), 3.0, dtype=torch.bfloat16, device=DEV)
+    table.scatter_out(gathered, [out])
+    assert torch.equal(out.view(torch.int16), gathered.view(torch.int16))              # copy-out: byte identity
+    fused = torch.full((t_pad,), 5.0, dtype=torch.bfloat16, device=DEV)
+    table.gather_in([out], fused, None, 8.0, True)                                    # reduce copy-in with /8
+    assert torch.equal(fused.view(torch.int16), (gathered.float() / 8.0).bfloat16().view(torch.int16))
+    del out
+    chunk = fused[r * s : (r + 1) * s]
+    shard = _randn_dev(s, 1e-4, torch.float32, gen)
+    shard_cpu, chunk_cpu = shard.cpu(), chunk.cpu()
+    nat.post_reduce(shard, chunk, None, True)
+    shard_cpu.add_(chunk_cpu)  # ya_fsdp/_collectives.py:189
+    assert_bits_equal(shard, shard_cpu, "post-reduce")
+    master = _randn_dev(s, 0.02, torch.float32, gen)
+    ag_in = torch.zeros(s, dtype=torch.bfloat16, device=DEV)
+    nat.flat_copy(ag_in, master)
+    want = torch.zeros(s, dtype=torch.bfloat16)
+    torch_ops.copy_in(want, master.cpu())
+    assert_bits_equal(ag_in, want, "copy-in")
+    table.close()
+    del gathered, fused, shard, master
+
+    print("config 4: final norm group", flush=True)
+    numels = [4096]
+    lay = make_layout(numels, w, 512)
+    t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+    assert (t, t_pad, s) == (4096, 4096, 512)
+    g = torch.Generator().manual_seed(1004)
+    gathered = (torch.randn(t_pad, generator=g) * 0.02).bfloat16()
+    grad = (torch.randn(t, generator=g) * 1e-3).bfloat16()
+    table = nat.TensorTable(numels, t_pad, DEV)
+    out = torch.empty(t, dtype=torch.bfloat16, device=DEV)
+    table.scatter_out(gathered.to(DEV), [out])
+    assert_bits_equal(out, gathered[:t], "copy-out")
+    rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=DEV)
+    table.gather_in([grad.to(DEV)], rs, None, 8.0, True)
+    rs_cpu = torch.zeros(t_pad, dtype=torch.bfloat16)
+    torch_ops.reduce_copy_in([rs_cpu[:t]], [grad], False)
+    torch_ops.div_if_needed(rs_cpu, 8.0)
+    assert_bits_equal(rs, rs_cpu, "reduce copy-in")
+    for rank in range(w):
+        shard0 = torch.randn(s, generator=g) * 1e-4
+        shard = shard0.to(DEV)
+        nat.post_reduce(shard, rs[rank * s : (rank + 1) * s], None, True)
+        want = shard0.clone()
+        torch_ops.reduce_scatter_local(want, rs_cpu.clone(), w, rank, None, None, "add")
+        assert_bits_equal(shard, want, f"post-reduce rank {rank}")
     table.close()
