@@ -42,6 +42,9 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_flat_copy(None, 0, None, 0, 0, None) == 0
     assert L.yafsdp_flat_div(None, 0, 0, 8.0, None) == 0
     assert L.yafsdp_post_reduce(None, 0, None, 5, 0, 0.0, 0, None) == -2
+    # empty ranges are fine whatever their pointers (torch hands out null for empty tensors)
+    assert L.yafsdp_post_reduce(None, 1, None, 0, 0, 8.0, 1, None) == 0
+    assert L.yafsdp_flat_div_copy(None, 1, None, 0, 0, 3.0, None) == 0
     assert L.yafsdp_set_option(99, 1) == -1
     assert L.yafsdp_set_option(0, 0) == -1
     assert L.yafsdp_set_option(2, 63) == -1

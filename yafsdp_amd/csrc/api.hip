@@ -609,6 +609,7 @@ int yafsdp_flat_div_copy(void* dst, int dst_dtype, const void* src, int src_dtyp
                          void* stream) {
   if (!valid_dtype(dst_dtype) || !valid_dtype(src_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && (dst == nullptr || src == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;  // empty ranges may come with null or equal pointers
   if (dst == src && dst_dtype != src_dtype) return YAFSDP_ERR_INVALID_ARGUMENT;
   int scale;
   float k;
@@ -620,6 +621,7 @@ int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chun
                        int accumulate, void* stream) {
   if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && (shard == nullptr || chunk == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;  // empty ranges may come with null or equal pointers
   int scale;
   float k;
   scale_plan(post_factor, &scale, &k);
