@@ -125,3 +125,94 @@ def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bou
         assert_bits_equal(bufs[i], ref, f"tensor {i} with its guard lanes")
         pos += n
     table.close()
+
+
+# ------------------------------------------------------------ optimizer side --
+@settings(max_examples=80, **COMMON)
+@given(n=st.integers(1, 40_000), off=st.integers(0, 3), decoupled=st.booleans(),
+       beta1=st.sampled_from([0.9, 0.5, 0.3, 0.0]), beta2=st.sampled_from([0.95, 0.999, 0.5]),
+       wd=st.sampled_from([0.0, 0.1, 1e-2]), lr=st.sampled_from([3e-4, 1e-2, 0.0]), step=st.integers(1, 2000),
+       out_dt=st.sampled_from([None, torch.bfloat16, torch.float16]), gscale=st.sampled_from([None, 0.5, 0.19153, 1.0]),
+       zero_grad=st.booleans(), seed=st.integers(0, 2**20))
+def test_adamw_any_shape(nat, n, off, decoupled, beta1, beta2, wd, lr, step, out_dt, gscale, zero_grad, seed):
+    from oracle import cref
+
+    print("adamw", n, off, decoupled, beta1, beta2, wd, lr, step, out_dt, gscale, zero_grad, seed, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    hp = dict(lr=lr, beta1=beta1, beta2=beta2, eps=1e-8, weight_decay=wd)
+    p = mixed_values(g, n, torch.float32, 0.02)
+    grad = mixed_values(g, n, torch.float32, 1e-3).flip(0).contiguous()
+    m = mixed_values(g, n, torch.float32, 1e-3, specials=False)
+    v = mixed_values(g, n, torch.float32, 1e-3, specials=False) ** 2
+    full = [torch.full((n + 8,), 5.0, device=DEV) for _ in range(4)]
+    dev = [f[off : off + n].copy_(t) for f, t in zip(full, (p, grad, m, v))]
+    out = None if out_dt is None else torch.full((n + 8,), 9.0, dtype=out_dt, device=DEV)
+    gs = None if gscale is None else torch.tensor([gscale], device=DEV)
+    nat.adamw_step(dev[0], dev[1], dev[2], dev[3], None if out is None else out[off : off + n], step=step,
+                   decoupled=decoupled, grad_scale=gs, zero_grad=zero_grad, **hp)
+    want_out = None if out_dt is None else torch.full((n + 8,), 9.0, dtype=out_dt)
+    cref.adamw_step(p, grad, m, v, None if want_out is None else want_out[off : off + n], step=step,
+                    decoupled=decoupled, grad_scale=gscale, zero_grad=zero_grad, **hp)
+    for name, f, b in zip(("param", "grad", "exp_avg", "exp_avg_sq"), full, (p, grad, m, v)):
+        want_full = torch.full((n + 8,), 5.0)
+        want_full[off : off + n] = b
+        assert_bits_equal(f, want_full, name)
+    if out is not None:
+        assert_bits_equal(out, want_out, "out16")
+
+
+@settings(max_examples=60, **COMMON)
+@given(dt=st.sampled_from(DTYPES), n=st.integers(0, 300_000), off=st.integers(0, 8),
+       coef=st.sampled_from([1.0, 0.5, 0.19153, 3.0]), seed=st.integers(0, 2**20))
+def test_sumsq_fill_scale_any_shape(nat, dt, n, off, coef, seed):
+    import math
+
+    from oracle import cref
+
+    print("sumsq/scale/fill", dt, n, off, coef, seed, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    x = mixed_values(g, n, dt, 3e-2, specials=False)
+    buf, d = _view_at(x, off, fill=7.0)
+    ws = nat.sumsq_workspace(DEV)
+    out = torch.zeros(1, dtype=torch.float64, device=DEV)
+    nat.flat_sumsq(d, out, ws, accumulate=False)
+    want = cref.sumsq(x)
+    assert math.isclose(float(out), want, rel_tol=1e-12, abs_tol=1e-300), (float(out), want)
+    nat.flat_scale(d, torch.tensor([coef], device=DEV))
+    ref = x.clone()
+    cref.flat_scale(ref, coef)
+    assert_bits_equal(d, ref, "scale")
+    nat.flat_fill(d, -0.25)
+    assert int((d.float() != -0.25).sum()) == 0
+    guard = torch.cat([buf[:off], buf[off + n :]]).float()
+    assert float(guard.min()) == 7.0 and float(guard.max()) == 7.0
+
+
+@settings(max_examples=60, **COMMON)
+@given(src_dt=st.sampled_from(DTYPES), dst_dt=st.sampled_from(DTYPES), n=st.integers(0, 60_000),
+       k=st.integers(1, 16), seed=st.integers(0, 2**20))
+def test_fanout_any_shape(nat, src_dt, dst_dt, n, k, seed):
+    print("fanout", src_dt, dst_dt, n, k, seed, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    src = mixed_values(g, n, src_dt)
+    want = torch.empty(n, dtype=dst_dt)
+    torch_ops.copy_in(want, src)
+    dsts = [torch.full((n,), 3.0, dtype=dst_dt, device=DEV) for _ in range(k)]
+    nat.flat_copy_fanout(dsts, src.to(DEV))
+    for i, d in enumerate(dsts):
+        assert_bits_equal(d, want, f"destination {i}")
+
+
+@settings(max_examples=60, **COMMON)
+@given(chunk_dt=st.sampled_from(DTYPES), shard_dt=st.sampled_from(DTYPES), n=st.integers(0, 60_000),
+       k=st.integers(1, 16), post=st.sampled_from(FACTORS), acc=st.booleans(), seed=st.integers(0, 2**20))
+def test_fanin_any_shape(nat, chunk_dt, shard_dt, n, k, post, acc, seed):
+    print("fanin", chunk_dt, shard_dt, n, k, post, acc, seed, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    chunks = [mixed_values(g, n, chunk_dt, 1e-3).roll(i) for i in range(k)]
+    shard0 = mixed_values(g, n, shard_dt, 1e-4).flip(0).contiguous()
+    want = shard0.clone()
+    torch_ops.reduce_scatter_fanin(want, [c.clone() for c in chunks], post, acc)
+    got = shard0.to(DEV)
+    nat.post_reduce_fanin(got, [c.to(DEV) for c in chunks], post, acc)
+    assert_bits_equal(got, want, "shard")
