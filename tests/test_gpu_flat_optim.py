@@ -3,7 +3,6 @@ AdamW step, gradient clipping and zero_grad run as one launch per parameter
 group and match the C oracle bit for bit on the same gradients."""
 
 import copy
-import math
 
 import pytest
 import torch
