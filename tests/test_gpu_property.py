@@ -216,3 +216,68 @@ def test_fanin_any_shape(nat, chunk_dt, shard_dt, n, k, post, acc, seed):
     got = shard0.to(DEV)
     nat.post_reduce_fanin(got, [c.to(DEV) for c in chunks], post, acc)
     assert_bits_equal(got, want, "shard")
+
+
+# ------------------------------------------------------------- group level --
+shape_st = st.one_of(st.tuples(st.integers(1, 300)), st.tuples(st.integers(1, 40), st.integers(1, 40)),
+                     st.tuples(st.integers(1, 6), st.integers(1, 9), st.integers(1, 9)))
+
+
+@settings(max_examples=40, **COMMON)
+@given(shapes=st.lists(shape_st, min_size=1, max_size=6), w=st.integers(1, 6), r_frac=st.floats(0, 0.999),
+       align=st.sampled_from([1, 2, 8, 16]), policy=st.sampled_from(["bf16", "bf16-fp32reduce", "fp16"]),
+       iterations=st.integers(1, 3), seed=st.integers(0, 2**20))
+def test_param_group_any_layout(shapes, w, r_frac, align, policy, iterations, seed):
+    """A parameter group with drawn shapes, world size, rank, alignment and precision policy through
+    unshard -> backward -> reduce for a few iterations (some parameters without a gradient in some of them),
+    against the reference's op sequence on CPU tensors."""
+    from test_gpu_param_group import CpuGroup, _make_group, _run_backward
+
+    from yafsdp_amd import MixedPrecisionPolicy
+
+    r = int(r_frac * w)
+    print("param group", shapes, w, r, align, policy, iterations, seed, flush=True)
+    low = torch.float16 if policy == "fp16" else torch.bfloat16
+    mp = MixedPrecisionPolicy(param_dtype=low, reduce_dtype=torch.float32 if policy == "bf16-fp32reduce" else None)
+    if policy == "fp16":  # ya_fsdp/_collectives.py:252-262
+        pre = 1
+        while w % pre == 0 and w / pre > pre:
+            pre *= 2
+        pre, post = float(pre), float(w / pre)
+    else:                 # AVG inside the collective: this rank's share is its chunk divided by W
+        pre, post = None, (float(w) if w > 1 else None)
+    group, cpu_params = _make_group(shapes, w, r, align, mp, seed=seed % 1000)
+    ref = CpuGroup(cpu_params, w, r, align, mp)
+    rng = np.random.default_rng(seed)
+    owns = [False] * len(shapes)  # parameters whose sharded gradient exists already
+    for it in range(iterations):
+        group.pre_forward(); group.post_forward(); group.pre_backward()
+        got_views = [fp.unsharded_param for fp in group.fsdp_params]
+        for v, w_ in zip(got_views, ref.unshard(first_of_iteration=True)):
+            assert_bits_equal(v.detach(), w_, "unsharded parameter")
+        g = torch.Generator().manual_seed(seed + it)
+        grads = [(torch.randn(s, generator=g) * 1e-3).to(low) for s in shapes]
+        present = rng.random(len(shapes)) < 0.8
+        if not present.any():
+            present[int(rng.integers(0, len(shapes)))] = True
+        grads = [x if p else None for x, p in zip(grads, present)]
+        _run_backward(group, ref, grads)
+        with_grad = [i for i, x in enumerate(grads) if x is not None]
+        if all(not owns[i] for i in with_grad) and len(with_grad) == len(shapes):
+            ref.reduce(pre, post, "copy")
+        elif all(owns[i] for i in with_grad) and len(with_grad) == len(shapes):
+            ref.reduce(pre, post, "add")
+        else:
+            ref.reduce(pre, post, "mixed", [None if x is None else owns[i] for i, x in enumerate(grads)])
+        for i in with_grad:
+            owns[i] = True
+        group.finalize_backward()
+        torch.cuda.synchronize()
+        got, want = group._padded_sharded_param_grad[None], ref.grad_shard
+        # fragments of parameters that never had a gradient hold unspecified values in the reference; compare the
+        # fragments that are defined
+        pos = 0
+        for i, n in enumerate(ref.lay.sharded_numels(r)):
+            if owns[i]:
+                assert_bits_equal(got[pos : pos + n], want[pos : pos + n], f"gradient fragment {i}, iteration {it}")
+            pos += n
