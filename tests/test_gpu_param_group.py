@@ -197,7 +197,13 @@ def test_gradient_accumulation_without_sync_uses_add():
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
 
 
-def test_mixed_params_with_and_without_sharded_grad():
+def test_mixed_params_with_and_without_sharded_grad(monkeypatch):
+    from yafsdp_amd import _native
+
+    def per_run_launches(*a, **k):  # the group-level path is one launch over a fragment table
+        raise AssertionError("post_reduce_fragments (one launch per run of fragments) must not be used here")
+
+    monkeypatch.setattr(_native, "post_reduce_fragments", per_run_launches)
     shapes, w, r, align = ODD_SHAPES, 2, 0, 8
     group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
     ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
@@ -217,6 +223,7 @@ def test_mixed_params_with_and_without_sharded_grad():
     group.finalize_backward()
     torch.cuda.synchronize()
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
+    assert group._fragment_table is not None and group._fragment_table.numels == ref.lay.sharded_numels(r)
 
 
 def test_fp16_reduce_uses_pre_and_post_divide():

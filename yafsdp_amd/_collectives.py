@@ -20,7 +20,8 @@ reference op                                           here
                                                         ``flat_div_copy``
 ``_div_if_needed(output, post)`` + ``copy_``/``add_``   ``post_reduce``
 (:165, :185, :189)
-``_foreach_copy_`` + ``_foreach_add_`` (:191-214)       ``post_reduce_fragments``
+``_foreach_copy_`` + ``_foreach_add_`` (:191-214)       ``gather_in`` over the
+                                                        chunk's fragments
 =====================================================  =========================
 
 One GPU: ``all_gather_group.size()`` may exceed 1 (logical world size).  The
@@ -250,7 +251,19 @@ def reduce_scatter(
                     for p in fsdp_params
                 ]
                 numels = [p.sharded_numel for p in fsdp_params]
-                _native.post_reduce_fragments(padded_sharded_param_grad, output_tensor, numels, modes, post)  # :191-214
+                if param_group is None:
+                    _native.post_reduce_fragments(padded_sharded_param_grad, output_tensor, numels, modes, post)
+                else:
+                    # :165 in place on the chunk, as the reference does it, then :191-214 as ONE launch whatever the
+                    # pattern of modes: the chunk's fragments are the "tensors" of a table over the gradient shard
+                    _div_if_needed(output_tensor, post)
+                    table = param_group._fragment_table
+                    if table is None:
+                        table = param_group._fragment_table = _native.TensorTable(
+                            numels, padded_sharded_param_grad.numel(), padded_sharded_param_grad.device
+                        )
+                    fragments = list(output_tensor[: sum(numels)].split(numels))
+                    table.gather_in(fragments, padded_sharded_param_grad, modes, None, zero_pad=False)
         post_reduce_event = reduce_scatter_stream.record_event()
         for fsdp_param in fsdp_params_with_grad:
             fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad  # :216-217

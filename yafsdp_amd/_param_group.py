@@ -182,6 +182,7 @@ class YaFSDPParamGroup:
             fsdp_param._param_group_ref = weakref.ref(self)
             fsdp_param._index_in_group = index
         self._table: _native.TensorTable | None = None
+        self._fragment_table: _native.TensorTable | None = None  # this rank's fragments of the gradient shard
         self._state_dict_hook_handles: list = []
         # version of the master shard at which a fused optimizer step last wrote the
         # all-gather input (None: never); see all_gather
