@@ -537,3 +537,26 @@ def test_profiler_ranges_appear_only_while_a_profiler_runs():
                  "YaFSDP::post_backward_reduce"):
         assert any(n.startswith(want) for n in names), (want, sorted(n for n in names if "FSDP" in n))
     assert profiler_range("x") is _NO_RANGE
+
+
+def test_activation_checkpointing_recomputes_through_the_hooks():
+    """Blocks run under torch.utils.checkpoint (non-reentrant): their forward is recomputed during backward, so the
+    forward hooks fire again while the group is in its backward states (ya_fsdp/_state.py:301-345,
+    ya_fsdp/_param_group.py:550-560).  The masters must come out as without checkpointing."""
+    from torch.utils.checkpoint import checkpoint
+
+    class CkptNet(Net):
+        def forward(self, x):
+            for b in self.blocks:
+                x = checkpoint(b, x, use_reentrant=False)
+            return self.norm(x)
+
+    torch.manual_seed(81)
+    plain0 = Net().to(DEV)
+    ckpt0 = CkptNet().to(DEV)
+    ckpt0.load_state_dict(plain0.state_dict())
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(120 + s),
+                      requires_grad=True) for s in range(3)]
+    want = _train(_wrap(plain0, mp_policy=MP), xs, 0.05)
+    got = _train(_wrap(ckpt0, mp_policy=MP), xs, 0.05)
+    _assert_same_masters(got, want)
