@@ -119,3 +119,54 @@ def test_bound_large_table_replays_match_eager():
             assert_bits_equal(a, b.cpu(), f"replay {it}: copy-out")
         assert_bits_equal(rs, e_rs.cpu(), f"replay {it}: reduce copy-in")
     gb.close(), sb.close(), table.close()
+
+
+def test_captured_optimizer_side_replays_match_eager():
+    """Post-reduce with the fused squared norm, the two-stage sum of its partial sums, the clip coefficient and the
+    fused AdamW pass captured into one HIP graph (kernel launches only) and replayed with new gradients each time."""
+    from yafsdp_amd import _native
+
+    n = 300_000
+    g = torch.Generator(device=DEV).manual_seed(78)
+
+    def rnd(std, dt=torch.float32):
+        return (torch.randn(n, device=DEV, generator=g) * std).to(dt)
+
+    chunk = rnd(1e-3, torch.bfloat16)
+    state0 = [rnd(0.02), rnd(1e-4), rnd(1e-3), rnd(1e-3) ** 2]           # param, grad shard, exp_avg, exp_avg_sq
+    hp = dict(lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=3)
+
+    def make():
+        return dict(
+            st=[x.clone() for x in state0], out16=torch.zeros(n, dtype=torch.bfloat16, device=DEV),
+            partials=torch.zeros(_native.post_reduce_sumsq_count(n), dtype=torch.float64, device=DEV),
+            stage=torch.zeros(8, dtype=torch.float64, device=DEV), nc=torch.zeros(2, device=DEV),
+        )
+
+    def step(b):
+        p, grad, m, v = b["st"]
+        count = _native.post_reduce_sumsq(grad, chunk, 8.0, True, b["partials"])
+        count = _native.sumsq_reduce_partials(b["partials"], count, b["stage"])
+        _native.clip_coef_from_partials(b["stage"], count, 1e-3, b["nc"])
+        _native.adamw_step(p, grad, m, v, b["out16"], grad_scale=b["nc"][1:2], zero_grad=False, **hp)
+
+    eager, captured = make(), make()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(make())  # warm up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(captured)
+    for it in range(4):
+        chunk.mul_(0.5 + 0.25 * it)   # new gradients in place, eager work between the replays
+        step(eager)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("param", "grad", "exp_avg", "exp_avg_sq"), captured["st"], eager["st"]):
+            assert_bits_equal(a, b, f"{name}, replay {it}")
+        assert_bits_equal(captured["out16"], eager["out16"], f"out16, replay {it}")
+        assert torch.equal(captured["nc"], eager["nc"]), it
+    del graph
