@@ -969,6 +969,9 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
+    ap.add_argument("--table-large-log2", type=int, default=None, metavar="N",
+                    help="tables with more than 2^N padded elements run two waves per workgroup instead of one "
+                         "(the library's launch-shape option; default: the library's own threshold)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -996,6 +999,8 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.table_large_log2 is not None:
+        _native.set_option(_native.OPT_TABLE_LARGE_LOG2, args.table_large_log2)
     # master / compute / reduce dtypes of the group: fp32 masters with bf16 compute and reduce, except the stress
     # test's second group (bf16 masters: no copy-in cast, fp32 reduce buffer, bf16 gradient shard)
     master_dt, rs_dt = torch.float32, torch.bfloat16

@@ -288,8 +288,12 @@ int yafsdp_time_next_launch(void* start_event, void* stop_event);
 typedef enum yafsdp_option {
   YAFSDP_OPT_FLAT_BLOCKS_PER_CU = 0,  /* workgroups per compute unit of the flat kernels' grid */
   YAFSDP_OPT_TABLE_BLOCKS_PER_CU = 1, /* same for gather-in / scatter-out */
-  YAFSDP_OPT_TABLE_LARGE_LOG2 = 2     /* 0..62: tables created from now on whose padded size exceeds
+  YAFSDP_OPT_TABLE_LARGE_LOG2 = 2,    /* 0..62: tables created from now on whose padded size exceeds
                                          2^value elements run two waves per workgroup instead of one */
+  YAFSDP_OPT_SCATTER_TILE = 3         /* tile of yafsdp_scatter_out for tables created from now on: 0 = from the
+                                         layout (short 512-element tiles when every tensor starts on a 128-byte
+                                         line of the flat buffer, the gather-in tile otherwise), 1 = always
+                                         short, 2 = never short */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);

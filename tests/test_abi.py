@@ -49,6 +49,8 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_set_option(0, 0) == -1
     assert L.yafsdp_set_option(2, 63) == -1
     assert L.yafsdp_set_option(2, 28) == 0
+    assert L.yafsdp_set_option(3, 3) == -1
+    assert L.yafsdp_set_option(3, 0) == 0
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
     # operands that overlap without being the same buffer are refused (addresses are never dereferenced here)
@@ -72,7 +74,7 @@ def test_no_product_module_imports_the_oracle():
     pkg = os.path.join(ROOT, "yafsdp_amd")
     for dirpath, _, files in os.walk(pkg):
         for f in files:
-            if f.endswith((".py", ".hip", ".cuh", ".h")):
+            if f.endswith((".py", ".hip", ".hip.h", ".h")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
                 assert "libbufpath_ref" not in src, f

@@ -135,13 +135,16 @@ def _random_numels(rng: np.random.Generator, p: int, max_log2: float, with_empty
     return n.tolist()
 
 
-@pytest.fixture(params=["one_wave", "two_waves"])
+@pytest.fixture(params=["one_wave", "two_waves", "short_scatter_tiles"])
 def table_workgroup(request, nat):
-    """Run a table test at both workgroup sizes the library picks between by table size."""
+    """Run a table test at both workgroup sizes the library picks between by table size, and with the short
+    scatter-out tile it picks for tables whose tensors all start on a cache line."""
     default = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
-    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default if request.param == "one_wave" else 0)
+    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0 if request.param == "two_waves" else default)
+    nat.set_option(nat.OPT_SCATTER_TILE, 1 if request.param == "short_scatter_tiles" else 2)
     yield request.param
     nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default)
+    nat.set_option(nat.OPT_SCATTER_TILE, 0)
 
 
 TABLE_CASES = [

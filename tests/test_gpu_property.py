@@ -94,9 +94,9 @@ def test_gather_in_any_table(nat, numels, pad, grad_dt, rs_dt, pre, two_waves, z
 
 @settings(max_examples=80, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), flat_dt=st.sampled_from(DTYPES), out_dt=st.sampled_from(DTYPES),
-       two_waves=st.booleans(), bound=st.booleans(), seed=st.integers(0, 2**20))
-def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bound, seed):
-    print("scatter_out", numels, pad, flat_dt, out_dt, two_waves, bound, seed, flush=True)
+       two_waves=st.booleans(), bound=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2))
+def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bound, seed, tile_mode):
+    print("scatter_out", numels, pad, flat_dt, out_dt, two_waves, bound, seed, tile_mode, flush=True)
     rng = np.random.default_rng(seed)
     g = torch.Generator().manual_seed(seed)
     p, t = len(numels), sum(numels)
@@ -106,10 +106,12 @@ def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bou
     bufs, views = zip(*[_view_at(torch.full((n,), 3.0, dtype=out_dt), o) for n, o in zip(numels, offs)])
     default = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
     nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0 if two_waves else default)
+    nat.set_option(nat.OPT_SCATTER_TILE, tile_mode)  # 0 from the layout, 1 short tiles, 2 the gather-in tile
     try:
         table = nat.TensorTable(numels, t + pad, DEV)
     finally:
         nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default)
+        nat.set_option(nat.OPT_SCATTER_TILE, 0)
     d_flat = flat.to(DEV)
     if bound:
         binding = table.bind(list(views), modes)

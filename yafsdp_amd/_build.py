@@ -14,8 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libyafsdp_hip.so")
 SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip", "fan.hip", "postsumsq.hip"]
-HEADERS = ["elem.cuh", "flat_kernels.cuh", "table_kernels.cuh", "optim_kernels.cuh", "fan_kernels.cuh",
-           "post_sumsq_kernels.cuh", "launch.h", "tuning.h"]
+HEADERS = ["elem.hip.h", "flat_kernels.hip.h", "table_kernels.hip.h", "optim_kernels.hip.h", "fan_kernels.hip.h",
+           "post_sumsq_kernels.hip.h", "launch.h", "tuning.h"]
 ARCH = "gfx950"
 
 # -ffp-contract=off: every multiply and add of the path rounds on its own, as

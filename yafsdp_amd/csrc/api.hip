@@ -21,6 +21,7 @@ namespace {
 std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
 std::atomic<int> g_table_blocks_per_cu{kTableBlocksPerCu};
 std::atomic<int> g_table_large_log2{kTableLargeThresholdLog2};
+std::atomic<int> g_scatter_tile_mode{0};
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
@@ -122,7 +123,9 @@ struct yafsdp_table {
   std::vector<int64_t> offsets;  // host copy, n_tensors + 1
   int64_t* d_offsets = nullptr;
   int block = kTableBlockSmall;  // workgroup size of the table kernels, chosen from the padded size
-  int64_t tile_elems = 0;        // block * kTableUnroll * 8
+  int64_t tile_elems = 0;        // gather-in tile: block * kGatherUnroll * 8 elements of the flat buffer
+  int scatter_shape = 0;         // scatter-out: workgroup size * 16 + units per lane (see scatter_shape_for)
+  int64_t slot_elems = 0;        // scatter-out tile (elements of one tensor)
   int32_t n_tiles = 0;           // gather-in: tiles of the flat buffer
   TileRec* d_tiles = nullptr;    // only for tables with more than kSmallMax tensors
   // scatter-out: tile slots per tensor (ceil(numel / tile) + 1 for a non-empty tensor)
@@ -347,9 +350,9 @@ int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int grid = grid_for(table_blocks(table->n_slots), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallMax)
-    return int(launch_scatter<SmallMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->small, flat,
+    return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->small, flat,
                                          table->total, table->n_slots, grid, s));
-  return int(launch_scatter<LargeMeta>(table->block, flat_dtype, binding->tensor_dtype, binding->large, flat,
+  return int(launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->large, flat,
                                        table->total, table->n_slots, grid, s));
 }
 
@@ -366,6 +369,11 @@ int yafsdp_set_option(int option, int value) {
     g_table_large_log2.store(value);
     return YAFSDP_OK;
   }
+  if (option == YAFSDP_OPT_SCATTER_TILE) {
+    if (value < 0 || value > 2) return YAFSDP_ERR_INVALID_ARGUMENT;
+    g_scatter_tile_mode.store(value);
+    return YAFSDP_OK;
+  }
   if (value < 1 || value > 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
   switch (option) {
     case YAFSDP_OPT_FLAT_BLOCKS_PER_CU: g_flat_blocks_per_cu.store(value); return YAFSDP_OK;
@@ -380,6 +388,7 @@ int yafsdp_get_option(int option, int* value) {
     case YAFSDP_OPT_FLAT_BLOCKS_PER_CU: *value = g_flat_blocks_per_cu.load(); return YAFSDP_OK;
     case YAFSDP_OPT_TABLE_BLOCKS_PER_CU: *value = g_table_blocks_per_cu.load(); return YAFSDP_OK;
     case YAFSDP_OPT_TABLE_LARGE_LOG2: *value = g_table_large_log2.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_SCATTER_TILE: *value = g_scatter_tile_mode.load(); return YAFSDP_OK;
   }
   return YAFSDP_ERR_INVALID_ARGUMENT;
 }
@@ -637,7 +646,7 @@ int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chun
 
 int64_t yafsdp_post_reduce_sumsq_count(int64_t n) {
   if (n <= 0) return 0;
-  const int64_t tile = int64_t(kFlatBlock) * kFlatUnroll;
+  const int64_t tile = int64_t(kPostSumsqBlock) * kPostSumsqUnroll;
   const int64_t n_tiles = ((n >> 3) + tile - 1) / tile;  // the peeled head can only lower the unit count
   return n_tiles < 1 ? 1 : n_tiles;
 }
@@ -659,7 +668,7 @@ int yafsdp_post_reduce_sumsq(void* shard, int shard_dtype, const void* chunk, in
     if (d0 < s1 && s0 < d1) return YAFSDP_ERR_INVALID_ARGUMENT;
   }
   const int head = head_elems(shard, item_size(shard_dtype), n);
-  const int64_t tile = int64_t(kFlatBlock) * kFlatUnroll;
+  const int64_t tile = int64_t(kPostSumsqBlock) * kPostSumsqUnroll;
   int64_t n_tiles = (((n - head) >> 3) + tile - 1) / tile;
   if (n_tiles < 1) n_tiles = 1;  // workgroup 0 handles head and tail
   if (n_tiles > capacity || n_tiles > int64_t(INT32_MAX)) return YAFSDP_ERR_INVALID_ARGUMENT;
@@ -729,7 +738,16 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     t->padded = padded_numel;
     if (padded_numel < t->total || padded_numel > (int64_t(1) << 60)) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->block = table_block_for(padded_numel, g_table_large_log2.load(std::memory_order_relaxed));
-    t->tile_elems = table_tile_elems(t->block);
+    t->tile_elems = gather_tile_elems(t->block);
+    {
+      bool line_aligned = true;  // every non-empty tensor starts on a multiple of 64 elements (128 bytes of a 2-byte dtype)
+      for (int p = 0; p < n_tensors; p++)
+        if (numels[p] > 0 && (t->offsets[p] & 63) != 0) line_aligned = false;
+      const ScatterShape sh = scatter_shape_for(padded_numel, line_aligned, g_table_large_log2.load(std::memory_order_relaxed),
+                                                g_scatter_tile_mode.load(std::memory_order_relaxed));
+      t->scatter_shape = sh.block * 16 + sh.unroll;
+      t->slot_elems = scatter_tile_elems(sh);
+    }
     const int64_t n_tiles = (padded_numel + t->tile_elems - 1) / t->tile_elems;
     if (n_tiles > int64_t(INT32_MAX) - 4096) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->n_tiles = int32_t(n_tiles);
@@ -755,7 +773,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     t->slot_start.assign(size_t(n_tensors) + 1, 0);
     for (int p = 0; p < n_tensors; p++) {
       const int64_t n = t->offsets[p + 1] - t->offsets[p];
-      t->slot_start[p + 1] = t->slot_start[p] + (n > 0 ? (n + t->tile_elems - 1) / t->tile_elems + 1 : 0);
+      t->slot_start[p + 1] = t->slot_start[p] + (n > 0 ? (n + t->slot_elems - 1) / t->slot_elems + 1 : 0);
     }
     if (t->slot_start[n_tensors] > int64_t(INT32_MAX) - 4096) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->n_slots = int32_t(t->slot_start[n_tensors]);
@@ -870,7 +888,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   if (table->n_tensors <= kSmallMax) {
     SmallMeta meta;
     fill_small(table, ptrs, mode, &meta);
-    return int(launch_scatter<SmallMeta>(table->block, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,
+    return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,
                                          grid, s));
   }
   std::lock_guard<std::mutex> lock(table->mu);
@@ -878,7 +896,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   int slot = -1;
   rc = stage_large(table, ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
-  e = launch_scatter<LargeMeta>(table->block, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s);
+  e = launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }

@@ -91,6 +91,49 @@ __device__ __forceinline__ void store_unit(void* p, const Unit<T>& u) {
   }
 }
 
+// ---- stores of one tile with a cache policy --------------------------------------
+// ST_PLAIN and ST_NT are ordinary global stores (non-temporal for ST_NT: the line
+// is kept in the L2 with streaming priority and written back when it is evicted
+// or when the kernel ends).  ST_WT writes through: buffer stores carrying sc0 sc1
+// hand every line to the memory side at once, in the order the tile loop produces
+// them, so the L2 does not fill up with dirty lines whose write-back the kernel's
+// end (and the loads of the kernel after it) would have to wait for.  Measured on
+// the 27 M-element shard kernels of a Llama-3-8B layer: bf16 -> fp32 copy 29.3 ->
+// 24.3 us, accumulate 43.3 -> 40.0 us, fp32 -> bf16 cast 26.5 -> 25.1 us; on
+// 400 MB tables the two policies are level.
+// Buffer stores address `base + byte offset` with a wave-uniform base (the tile's
+// first byte; readfirstlane is free when the compiler already knows that) and a
+// per-lane 32-bit offset; stores beyond `bytes` would be dropped by the hardware.
+enum : int { ST_PLAIN = 0, ST_NT = 1, ST_WT = 2 };
+
+template <class T, int POLICY>
+struct TileStore {
+  char* base;
+  __amdgpu_buffer_rsrc_t rsrc;
+  static constexpr int kAux = 1 | 16;  // sc0 | sc1
+
+  __device__ __forceinline__ TileStore(char* tile_base, int bytes) : base(tile_base) {
+    if constexpr (POLICY == ST_WT) {
+      const uint64_t a = reinterpret_cast<uint64_t>(tile_base);
+      const uint32_t lo = __builtin_amdgcn_readfirstlane(uint32_t(a));
+      const uint32_t hi = __builtin_amdgcn_readfirstlane(uint32_t(a >> 32));
+      rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>((uint64_t(hi) << 32) | lo), 0, bytes, 0x00020000);
+    }
+  }
+  // 16 bytes (4 fp32 or 8 two-byte elements) at byte offset `off`, 16-byte aligned
+  __device__ __forceinline__ void vec(int off, u32x4 v) const {
+    if constexpr (POLICY == ST_WT) __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, off, 0, kAux);
+    else if constexpr (POLICY == ST_NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(base + off));
+    else *reinterpret_cast<u32x4*>(base + off) = v;
+  }
+  // 8 bytes (4 two-byte elements) at byte offset `off`, 8-byte aligned
+  __device__ __forceinline__ void half(int off, u32x2 v) const {
+    if constexpr (POLICY == ST_WT) __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, off, 0, kAux);
+    else if constexpr (POLICY == ST_NT) __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(base + off));
+    else *reinterpret_cast<u32x2*>(base + off) = v;
+  }
+};
+
 // ---- scalar conversions -------------------------------------------------------
 __device__ __forceinline__ float bits_to_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t f32_to_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
@@ -232,6 +275,19 @@ __device__ __forceinline__ Quad<T> pack_quad(const float (&f)[4]) {
     }
   }
   return u;
+}
+
+// one unit / one quad of a tile through its TileStore (byte offset inside the tile)
+template <class T, int POLICY>
+__device__ __forceinline__ void store_unit_at(const TileStore<T, POLICY>& ts, int off, const Unit<T>& u) {
+#pragma unroll
+  for (int i = 0; i < T::kVecs; i++) ts.vec(off + 16 * i, u.v[i]);
+}
+
+template <class T, int POLICY>
+__device__ __forceinline__ void store_quad_at(const TileStore<T, POLICY>& ts, int off, const Quad<T>& u) {
+  if constexpr (T::kSize == 4) ts.vec(off, u.v);
+  else ts.half(off, u.v);
 }
 
 // a pair of dtypes takes the quad arrangement when either side is fp32

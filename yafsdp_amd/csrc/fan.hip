@@ -1,5 +1,5 @@
 // Instantiations and dtype dispatch of the fan-out / fan-in kernels.
-#include "fan_kernels.cuh"
+#include "fan_kernels.hip.h"
 #include "launch.h"
 #include "tuning.h"
 

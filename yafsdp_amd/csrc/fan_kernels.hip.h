@@ -9,7 +9,7 @@
 // BLOCK*U quads is t + j*BLOCK, so every wave64 access is one contiguous span.
 // All buffers are 16-byte aligned.
 #pragma once
-#include "flat_kernels.cuh"
+#include "flat_kernels.hip.h"
 #include "launch.h"
 
 namespace yafsdp {

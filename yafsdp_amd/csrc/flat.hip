@@ -7,7 +7,7 @@ namespace {
 
 template <class S, class D, int SCALE, bool ACC>
 hipError_t go(void* dst, const void* src, int64_t n, int head, float k, int grid, hipStream_t stream) {
-  return launch_kernel(flat_kernel<S, D, SCALE, ACC, kFlatBlock, kFlatUnroll, kFlatNtLoad, kFlatNtStore>, grid,
+  return launch_kernel(flat_kernel<S, D, SCALE, ACC, kFlatBlock, kFlatUnroll, kFlatNtLoad, kFlatStorePolicy>, grid,
                        kFlatBlock, stream, dst, src, n, head, k);
 }
 

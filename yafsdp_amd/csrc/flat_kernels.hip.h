@@ -7,14 +7,14 @@
 // elements), one workgroup per tile (grid-stride if the grid is capped).
 //  * pairs of 2-byte dtypes: lane l touches units l, l+BLOCK, ...: every wave64
 //    access is one contiguous 1 KiB span;
-//  * pairs with an fp32 side: quad arrangement (see elem.cuh): every wave64
+//  * pairs with an fp32 side: quad arrangement (see elem.hip.h): every wave64
 //    access is a contiguous 1 KiB (fp32) or 512 B (2-byte) span.
 // All loads of a lane are issued before its first store.  The destination is
 // 16-byte aligned for the tile loop (the host peels up to 7 leading elements,
 // handled by workgroup 0 together with the tail); the source may sit at any
 // element-aligned address.
 #pragma once
-#include "elem.cuh"
+#include "elem.hip.h"
 
 namespace yafsdp {
 
@@ -60,9 +60,10 @@ __device__ __forceinline__ Quad<D> flat_quad(const Quad<S>& s, const Quad<D>& d_
   }
 }
 
-// One full tile (BLOCK*U units) at dst/src; dst 16-byte aligned.
-template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
+// One full tile (BLOCK*U units) at dst/src; dst 16-byte aligned.  STP: store policy (ST_PLAIN / ST_NT / ST_WT).
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float k) {
+  const TileStore<D, STP> out(dst, BLOCK * U * 8 * D::kSize);
   if constexpr (wide_pair<S, D>::value) {
     Quad<S> s[2 * U];
     Quad<D> d[2 * U];
@@ -74,7 +75,7 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
     }
 #pragma unroll
     for (int q = 0; q < 2 * U; q++)
-      store_quad<D, NTS>(dst + quad_elem<BLOCK, U>(q) * D::kSize, flat_quad<S, D, SCALE, ACC>(s[q], d[q], k));
+      store_quad_at<D, STP>(out, quad_elem<BLOCK, U>(q) * D::kSize, flat_quad<S, D, SCALE, ACC>(s[q], d[q], k));
   } else {
     Unit<S> s[U];
     Unit<D> d[U];
@@ -86,13 +87,13 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
     }
 #pragma unroll
     for (int j = 0; j < U; j++)
-      store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
+      store_unit_at<D, STP>(out, unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s[j], d[j], k));
   }
 }
 
 // dst[i] = op(src[i], dst[i]) for i in [0, n).  `head` leading elements bring
 // dst to a 16-byte boundary.  dst == src is allowed (in-place divide).
-template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
   const int tid = threadIdx.x;
@@ -110,14 +111,14 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
   const int64_t n_tiles = (n_units + kTile - 1) / kTile;
   for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     if (tile * kTile + kTile <= n_units) {
-      flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, NTS>(dbase + tile * kTile * (8 * D::kSize),
+      flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dbase + tile * kTile * (8 * D::kSize),
                                                            sbase + tile * kTile * (8 * S::kSize), k);
     } else {  // last, partial tile
       for (int64_t u = tile * kTile + tid; u < n_units; u += BLOCK) {
         Unit<S> s = load_unit<S, NTL>(sbase + u * (8 * S::kSize));
         Unit<D> d;
         if constexpr (ACC) d = load_unit<D, NTL>(dbase + u * (8 * D::kSize));
-        store_unit<D, NTS>(dbase + u * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s, d, k));
+        store_unit<D, STP == ST_NT>(dbase + u * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s, d, k));
       }
     }
   }

@@ -8,7 +8,7 @@ namespace {
 template <class META, class S, class D, int SCALE, int BLOCK>
 hipError_t go(const META& meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero, int grid,
               hipStream_t stream) {
-  return launch_kernel(gather_in_kernel<META, S, D, SCALE, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>, grid,
+  return launch_kernel(gather_in_kernel<META, S, D, SCALE, BLOCK, kGatherUnroll, kTableNtLoad, kGatherStorePolicy>, grid,
                        BLOCK, stream, meta, flat, padded, n_tiles, k, pad_zero);
 }
 

@@ -5,7 +5,7 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
-#include "table_kernels.cuh"
+#include "table_kernels.hip.h"
 
 namespace yafsdp {
 
@@ -40,7 +40,8 @@ hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc,
                                     int head, float k, double* partials, int grid, hipStream_t stream);
 
 // META is SmallMeta or LargeMeta (explicitly instantiated in gather.hip / scatter.hip);
-// `block` is the workgroup size the table was built for (kTableBlockSmall or kTableBlockLarge)
+// `block` is the workgroup size the table was built for (kTableBlockSmall or kTableBlockLarge); for launch_scatter
+// it is the table's scatter shape packed as workgroup size * 16 + units per lane
 template <class META>
 hipError_t launch_gather(int block, int tensor_dt, int flat_dt, int scale, const META& meta, void* flat,
                          int64_t padded, int n_tiles, float k, int pad_zero, int grid, hipStream_t stream);

@@ -1,6 +1,6 @@
 // Instantiations and dtype dispatch of the optimizer-side kernels.
 #include "launch.h"
-#include "optim_kernels.cuh"
+#include "optim_kernels.hip.h"
 #include "tuning.h"
 
 namespace yafsdp {

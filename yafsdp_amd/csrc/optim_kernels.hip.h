@@ -10,7 +10,7 @@
 // (1 KiB of fp32, 512 B of a 2-byte dtype).  All loads of a lane are issued
 // before its first store.
 #pragma once
-#include "elem.cuh"
+#include "elem.hip.h"
 #include "launch.h"
 
 namespace yafsdp {

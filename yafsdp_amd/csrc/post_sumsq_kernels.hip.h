@@ -9,7 +9,7 @@
 // partials[blockIdx.x].  One workgroup per tile, so the number of partial sums
 // and the order of all additions depend only on (n, head).
 #pragma once
-#include "flat_kernels.cuh"
+#include "flat_kernels.hip.h"
 
 namespace yafsdp {
 
@@ -49,10 +49,11 @@ __device__ __forceinline__ double post_scalar_sumsq(void* dst, const void* src, 
   return double(stored) * double(stored);
 }
 
-template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float k, double* partials) {
   __shared__ double lds[BLOCK / 64];
+  constexpr bool NTS = (STP == ST_NT);  // the partial last tile keeps ordinary global stores
   const int tid = threadIdx.x;
   const int64_t n_units = (n - head) >> 3;
   const int64_t body_end = head + (n_units << 3);
@@ -71,6 +72,7 @@ post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float 
     char* dt = dbase + tile * kTile * (8 * D::kSize);
     const char* st = sbase + tile * kTile * (8 * S::kSize);
     if (tile * kTile + kTile <= n_units) {
+      const TileStore<D, STP> out(dt, BLOCK * U * 8 * D::kSize);
       if constexpr (wide_pair<S, D>::value) {
         Quad<S> s[2 * U];
         Quad<D> d[2 * U];
@@ -83,7 +85,7 @@ post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float 
 #pragma unroll
         for (int q = 0; q < 2 * U; q++) {
           const Quad<D> r = flat_quad<S, D, SCALE, ACC>(s[q], d[q], k);
-          store_quad<D, NTS>(dt + quad_elem<BLOCK, U>(q) * D::kSize, r);
+          store_quad_at<D, STP>(out, quad_elem<BLOCK, U>(q) * D::kSize, r);
           if (q & 1) acc1 = quad_sumsq<D>(r, acc1);
           else acc0 = quad_sumsq<D>(r, acc0);
         }
@@ -99,7 +101,7 @@ post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float 
 #pragma unroll
         for (int j = 0; j < U; j++) {
           const Unit<D> r = flat_unit<S, D, SCALE, ACC>(s[j], d[j], k);
-          store_unit<D, NTS>(dt + unit_index<BLOCK, U>(j) * (8 * D::kSize), r);
+          store_unit_at<D, STP>(out, unit_index<BLOCK, U>(j) * (8 * D::kSize), r);
           if (j & 1) acc1 = unit_sumsq<D>(r, acc1);
           else acc0 = unit_sumsq<D>(r, acc0);
         }

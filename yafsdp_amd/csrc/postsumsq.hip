@@ -1,7 +1,7 @@
 // Instantiations and dtype dispatch of the post-reduce kernel that also returns
 // the sum of squares of the gradient shard it writes.
 #include "launch.h"
-#include "post_sumsq_kernels.cuh"
+#include "post_sumsq_kernels.hip.h"
 #include "tuning.h"
 
 namespace yafsdp {
@@ -10,8 +10,8 @@ namespace {
 template <class S, class D, int SCALE, bool ACC>
 hipError_t go(void* dst, const void* src, int64_t n, int head, float k, double* partials, int grid,
               hipStream_t stream) {
-  return launch_kernel(post_reduce_sumsq_kernel<S, D, SCALE, ACC, kFlatBlock, kFlatUnroll, kFlatNtLoad, kFlatNtStore>,
-                       grid, kFlatBlock, stream, dst, src, n, head, k, partials);
+  return launch_kernel(post_reduce_sumsq_kernel<S, D, SCALE, ACC, kPostSumsqBlock, kPostSumsqUnroll, kFlatNtLoad, kFlatStorePolicy>,
+                       grid, kPostSumsqBlock, stream, dst, src, n, head, k, partials);
 }
 
 template <class S, class D>

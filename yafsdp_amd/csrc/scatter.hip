@@ -5,17 +5,23 @@
 namespace yafsdp {
 namespace {
 
-template <class META, class S, class D, int BLOCK>
+template <class META, class S, class D, int BLOCK, int U>
 hipError_t go(const META& meta, const void* flat, int64_t total, int n_tiles, int grid, hipStream_t stream) {
-  return launch_kernel(scatter_out_kernel<META, S, D, BLOCK, kTableUnroll, kTableNtLoad, kTableNtStore>, grid, BLOCK,
+  return launch_kernel(scatter_out_kernel<META, S, D, BLOCK, U, kTableNtLoad, kScatterStorePolicy>, grid, BLOCK,
                        stream, meta, flat, total, n_tiles);
 }
 
+// `block` packs the shape the table was built for: workgroup size * 16 + units per lane
 template <class META, class S, class D>
 hipError_t by_block(int block, const META& meta, const void* flat, int64_t total, int n_tiles, int grid,
                     hipStream_t stream) {
-  if (block == kTableBlockSmall) return go<META, S, D, kTableBlockSmall>(meta, flat, total, n_tiles, grid, stream);
-  if (block == kTableBlockLarge) return go<META, S, D, kTableBlockLarge>(meta, flat, total, n_tiles, grid, stream);
+  const int wg = block >> 4, unroll = block & 15;
+  if (wg == kTableBlockSmall && unroll == kScatterShortUnroll)
+    return go<META, S, D, kTableBlockSmall, kScatterShortUnroll>(meta, flat, total, n_tiles, grid, stream);
+  if (wg == kTableBlockSmall && unroll == kGatherUnroll)
+    return go<META, S, D, kTableBlockSmall, kGatherUnroll>(meta, flat, total, n_tiles, grid, stream);
+  if (wg == kTableBlockLarge && unroll == kGatherUnroll)
+    return go<META, S, D, kTableBlockLarge, kGatherUnroll>(meta, flat, total, n_tiles, grid, stream);
   return hipErrorInvalidValue;
 }
 

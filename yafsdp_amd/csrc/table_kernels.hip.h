@@ -38,7 +38,7 @@
 //    afresh) is refreshed by the host on the same stream before the launch.
 //    All of it is read through the constant address space, i.e. as scalar loads.
 #pragma once
-#include "flat_kernels.cuh"
+#include "flat_kernels.hip.h"
 #include "tuning.h"
 
 namespace yafsdp {
@@ -192,10 +192,11 @@ __device__ __forceinline__ Quad<D> gather_quad(const Quad<S>& s, const Quad<D>& 
   }
 }
 
-template <class S, class D, int SCALE, int MODE, int BLOCK, int U, bool NTL, bool NTS>
+template <class S, class D, int SCALE, int MODE, int BLOCK, int U, bool NTL, int STP>
 __device__ __forceinline__ void gather_full_tile(char* dst, const char* src, float k) {
   constexpr bool kReadSrc = (MODE == MODE_COPY || MODE == MODE_ADD);
   constexpr bool kReadDst = (MODE == MODE_ADD || MODE == MODE_SKIP);
+  const TileStore<D, STP> out(dst, BLOCK * U * 8 * D::kSize);
   if constexpr (wide_pair<S, D>::value) {
     Quad<S> s[2 * U];
     Quad<D> d[2 * U];
@@ -209,7 +210,7 @@ __device__ __forceinline__ void gather_full_tile(char* dst, const char* src, flo
     }
 #pragma unroll
     for (int q = 0; q < 2 * U; q++)
-      store_quad<D, NTS>(dst + quad_elem<BLOCK, U>(q) * D::kSize, gather_quad<S, D, SCALE, MODE>(s[q], d[q], k));
+      store_quad_at<D, STP>(out, quad_elem<BLOCK, U>(q) * D::kSize, gather_quad<S, D, SCALE, MODE>(s[q], d[q], k));
     return;
   }
   Unit<S> s[U];
@@ -224,7 +225,7 @@ __device__ __forceinline__ void gather_full_tile(char* dst, const char* src, flo
   }
 #pragma unroll
   for (int j = 0; j < U; j++)
-    store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), gather_unit<S, D, SCALE, MODE>(s[j], d[j], k));
+    store_unit_at<D, STP>(out, unit_index<BLOCK, U>(j) * (8 * D::kSize), gather_unit<S, D, SCALE, MODE>(s[j], d[j], k));
 }
 
 // n elements; dst points at flat element `flat_index`, src at the matching
@@ -265,10 +266,11 @@ __device__ __forceinline__ int tile_of_block(int b) {
 // S: tensor dtype, D: flat buffer dtype.  pad_zero != 0 writes zeros to
 // [total, padded); otherwise pad lanes only see the divide (as in the
 // reference, whose pad content is whatever the buffer held).
-template <class META, class S, class D, int SCALE, int BLOCK, int U, bool NTL, bool NTS>
+template <class META, class S, class D, int SCALE, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
+  constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   char* fbase = reinterpret_cast<char*>(flat);
   constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
   constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
@@ -284,9 +286,9 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
       const int mode = meta.mode(p);
       const char* src = reinterpret_cast<const char*>(meta.tensor(p)) + rec.delta * S::kSize;
       char* dst = fbase + t0 * D::kSize;
-      if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, NTS>(dst, src, k);
-      else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, NTS>(dst, src, k);
-      else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, NTS>(dst, src, k);
+      if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, STP>(dst, src, k);
+      else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, STP>(dst, src, k);
+      else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, STP>(dst, src, k);
       continue;
     }
     int64_t pos = t0;
@@ -319,8 +321,9 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
 // instead and storing at odd tensor offsets measured 13 % slower on a
 // 1427-tensor table: two workgroups then share the cache line at every tile
 // boundary.  Loads at odd offsets cost about 1 %.)
-template <class S, class D, int BLOCK, int U, bool NTL, bool NTS>
+template <class S, class D, int BLOCK, int U, bool NTL, int STP>
 __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
+  const TileStore<D, STP> out(dst, BLOCK * U * 8 * D::kSize);
   if constexpr (wide_pair<S, D>::value) {
     Quad<S> s[2 * U];
     Quad<D> unused_q;
@@ -328,7 +331,7 @@ __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
     for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(src + quad_elem<BLOCK, U>(q) * S::kSize);
 #pragma unroll
     for (int q = 0; q < 2 * U; q++)
-      store_quad<D, NTS>(dst + quad_elem<BLOCK, U>(q) * D::kSize, flat_quad<S, D, SCALE_NONE, false>(s[q], unused_q, 0.f));
+      store_quad_at<D, STP>(out, quad_elem<BLOCK, U>(q) * D::kSize, flat_quad<S, D, SCALE_NONE, false>(s[q], unused_q, 0.f));
     return;
   }
   Unit<S> s[U];
@@ -337,7 +340,7 @@ __device__ __forceinline__ void scatter_full_tile(char* dst, const char* src) {
   for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(src + unit_index<BLOCK, U>(j) * (8 * S::kSize));
 #pragma unroll
   for (int j = 0; j < U; j++)
-    store_unit<D, NTS>(dst + unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE_NONE, false>(s[j], unused, 0.f));
+    store_unit_at<D, STP>(out, unit_index<BLOCK, U>(j) * (8 * D::kSize), flat_unit<S, D, SCALE_NONE, false>(s[j], unused, 0.f));
 }
 
 // n elements (fewer than a tile): up to 7 leading elements bring dst to a
@@ -364,10 +367,11 @@ __device__ __forceinline__ void scatter_segment(char* dst, const char* src, int6
 
 // S: flat buffer dtype, D: tensor dtype.  Tensors with mode 0 are not written;
 // pad lanes of the flat buffer are never read.  n_tiles counts tile slots.
-template <class META, class S, class D, int BLOCK, int U, bool NTL, bool NTS>
+template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
+  constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   constexpr int64_t kLineElems = 128 / D::kSize;
   const char* fbase = reinterpret_cast<const char*>(flat);
   (void)total;
@@ -392,7 +396,7 @@ scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
     if (lo >= hi) continue;
     char* dst = tbase + lo * D::kSize;
     const char* src = fbase + (o0 + lo) * S::kSize;
-    if (hi - lo == kTile) scatter_full_tile<S, D, BLOCK, U, NTL, NTS>(dst, src);
+    if (hi - lo == kTile) scatter_full_tile<S, D, BLOCK, U, NTL, STP>(dst, src);
     else scatter_segment<S, D, BLOCK, NTL, NTS>(dst, src, hi - lo);
   }
 }

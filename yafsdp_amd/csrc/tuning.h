@@ -8,12 +8,26 @@ namespace yafsdp {
 #define YAFSDP_FLAT_BLOCK 256
 #endif
 #ifndef YAFSDP_FLAT_U
-#define YAFSDP_FLAT_U 2
+#define YAFSDP_FLAT_U 1
+#endif
+// store policy of whole tiles: 0 ordinary, 1 non-temporal, 2 write-through (see TileStore)
+#ifndef YAFSDP_FLAT_STP
+#define YAFSDP_FLAT_STP 2
+#endif
+#ifndef YAFSDP_TABLE_STP
+#define YAFSDP_TABLE_STP 1
 #endif
 constexpr int kFlatBlock = YAFSDP_FLAT_BLOCK;
 constexpr int kFlatUnroll = YAFSDP_FLAT_U;
-constexpr bool kFlatNtLoad = true;
-constexpr bool kFlatNtStore = true;
+// the post-reduce that also sums squares keeps tiles of 4096 elements: one partial sum per tile is part of its
+// interface (yafsdp_post_reduce_sumsq_count), and the order of the additions must not move with the flat tuning
+constexpr int kPostSumsqBlock = 256;
+constexpr int kPostSumsqUnroll = 2;
+#ifndef YAFSDP_FLAT_NTL
+#define YAFSDP_FLAT_NTL true
+#endif
+constexpr bool kFlatNtLoad = YAFSDP_FLAT_NTL;
+constexpr int kFlatStorePolicy = YAFSDP_FLAT_STP;
 // gather-in / scatter-out: a tile is block * unroll * 8 elements.  Measured with
 // non-zero data and the four kernels of a step running back to back: tiles of
 // 1-2 K elements (2-4 KiB of bf16) in workgroups of one or two waves are the
@@ -26,12 +40,21 @@ constexpr bool kFlatNtStore = true;
 constexpr int kTableBlockSmall = 64;
 constexpr int kTableBlockLarge = 128;
 constexpr int kTableLargeThresholdLog2 = 28;  // padded size above 2^28 elements: the larger workgroup
-constexpr int kTableUnroll = 2;
+#ifndef YAFSDP_TABLE_U
+#define YAFSDP_TABLE_U 2
+#endif
+#ifndef YAFSDP_GATHER_U
+#define YAFSDP_GATHER_U YAFSDP_TABLE_U
+#endif
+constexpr int kGatherUnroll = YAFSDP_GATHER_U;    // units per lane of a gather-in tile (tiles of the flat buffer)
+// scatter-out picks its tile per table (scatter_shape_for): one wave with ONE unit per lane (512-element tiles)
+// when every tensor starts on a 128-byte line of the flat buffer, as the tensors of a transformer layer do
+// (8B layer: 137.5 -> 133 us, 70B layer: 534 -> 517 us against two units per lane), and the gather-in shape
+// otherwise (on a 1427-tensor table at odd offsets the short tiles lose 9 %: every tile then reads one more
+// cache line than it writes, and shorter tiles make that line a larger share).
+constexpr int kScatterShortUnroll = 1;
 #ifndef YAFSDP_TABLE_NTL
 #define YAFSDP_TABLE_NTL true
-#endif
-#ifndef YAFSDP_TABLE_NTS
-#define YAFSDP_TABLE_NTS true
 #endif
 // 0: workgroup b handles tile b.  X > 0: workgroups are assumed to be dealt round-robin to X XCDs, and within every
 // window of X * R tiles each XCD takes a run of R neighbouring tiles (tile = window + (b % X) * R + (b / X) % R), so
@@ -45,11 +68,25 @@ constexpr int kTableUnroll = 2;
 constexpr int kTableXcd = YAFSDP_TABLE_XCD;
 constexpr int kTableXcdRun = YAFSDP_TABLE_XCD_RUN;
 constexpr bool kTableNtLoad = YAFSDP_TABLE_NTL;
-constexpr bool kTableNtStore = YAFSDP_TABLE_NTS;
+#ifndef YAFSDP_GATHER_STP
+#define YAFSDP_GATHER_STP YAFSDP_TABLE_STP
+#endif
+#ifndef YAFSDP_SCATTER_STP
+#define YAFSDP_SCATTER_STP YAFSDP_TABLE_STP
+#endif
+constexpr int kGatherStorePolicy = YAFSDP_GATHER_STP;
+constexpr int kScatterStorePolicy = YAFSDP_SCATTER_STP;
 inline int table_block_for(long long padded_elems, int threshold_log2) {
   return padded_elems > (1LL << threshold_log2) ? kTableBlockLarge : kTableBlockSmall;
 }
-inline long long table_tile_elems(int block) { return (long long)block * kTableUnroll * 8; }
+inline long long gather_tile_elems(int block) { return (long long)block * kGatherUnroll * 8; }
+struct ScatterShape { int block, unroll; };
+// mode: 0 from the layout, 1 always the short tile, 2 never
+inline ScatterShape scatter_shape_for(long long padded_elems, bool line_aligned, int threshold_log2, int mode) {
+  if (mode == 1 || (mode == 0 && line_aligned)) return ScatterShape{kTableBlockSmall, kScatterShortUnroll};
+  return ScatterShape{table_block_for(padded_elems, threshold_log2), kGatherUnroll};
+}
+inline long long scatter_tile_elems(ScatterShape s) { return (long long)s.block * s.unroll * 8; }
 // optimizer-side passes: a tile is block * unroll quads (4 elements each)
 #ifndef YAFSDP_FILL_BLOCK
 #define YAFSDP_FILL_BLOCK 256
