@@ -43,7 +43,8 @@ typedef enum yafsdp_status {
   YAFSDP_ERR_UNSUPPORTED_DTYPE = -2,
   YAFSDP_ERR_MISALIGNED = -3,
   YAFSDP_ERR_WRONG_DEVICE = -4,
-  YAFSDP_ERR_OUT_OF_MEMORY = -5
+  YAFSDP_ERR_OUT_OF_MEMORY = -5,
+  YAFSDP_ERR_TOO_LARGE = -6
 } yafsdp_status;
 
 /* per-tensor mode of yafsdp_gather_in / yafsdp_scatter_out / fragments */
@@ -224,6 +225,18 @@ size_t yafsdp_sumsq_workspace_bytes(void);
  * overlap).  Two launches: per-workgroup partial sums, then their sum. */
 int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* workspace,
                       size_t workspace_bytes, void* stream);
+
+/* yafsdp_flat_sumsq for callers that cannot allocate and have no workspace to hand over (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * kernels, same order of additions and so the same bits as yafsdp_flat_sumsq; the per-workgroup partial sums go to a
+ * fixed 128 KiB array in the library's own device image (one copy per GPU, held until the process ends) instead of
+ * a workspace argument.  The call allocates and frees nothing.  n is limited to
+ * yafsdp_flat_sumsq_static_max_numel() = 2^31 elements; more returns YAFSDP_ERR_TOO_LARGE.  The first call on a
+ * device looks the array's address up; a call with n == 0 does only that (make one before capturing a graph).
+ * All calls on one GPU share the array: calls that overlap in time (different streams, or threads) race on it, and
+ * the caller has to order them.  Nothing in it needs clearing between calls. */
+int64_t yafsdp_flat_sumsq_static_max_numel(void);
+int yafsdp_flat_sumsq_static(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* stream);
 
 /* The same split in two for several buffers (the groups of a model): each call
  * of yafsdp_sumsq_partials writes at most `capacity` per-workgroup sums of

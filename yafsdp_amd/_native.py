@@ -59,6 +59,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_flat_fill",
     "yafsdp_sumsq_workspace_bytes",
     "yafsdp_flat_sumsq",
+    "yafsdp_flat_sumsq_static_max_numel",
+    "yafsdp_flat_sumsq_static",
     "yafsdp_sumsq_partials",
     "yafsdp_sumsq_reduce_partials",
     "yafsdp_clip_coef_from_partials",
@@ -125,6 +127,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_sumsq_workspace_bytes.argtypes = []
     lib.yafsdp_flat_sumsq.restype = i32
     lib.yafsdp_flat_sumsq.argtypes = [vp, i32, i64, vp, i32, vp, ctypes.c_size_t, vp]
+    lib.yafsdp_flat_sumsq_static_max_numel.restype = i64
+    lib.yafsdp_flat_sumsq_static_max_numel.argtypes = []
+    lib.yafsdp_flat_sumsq_static.restype = i32
+    lib.yafsdp_flat_sumsq_static.argtypes = [vp, i32, i64, vp, i32, vp]
     lib.yafsdp_sumsq_partials.restype = i32
     lib.yafsdp_sumsq_partials.argtypes = [vp, i32, i64, vp, i64, ctypes.POINTER(i64), vp]
     lib.yafsdp_sumsq_reduce_partials.restype = i32
@@ -580,6 +586,21 @@ def flat_sumsq(src: torch.Tensor, out: torch.Tensor, workspace: torch.Tensor, ac
                 workspace.numel() * workspace.element_size(), _stream(src),
             ),
             "yafsdp_flat_sumsq",
+        )
+
+
+def flat_sumsq_static(src: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """``flat_sumsq`` without a workspace and without any allocation: the partial sums live in a fixed array inside
+    the library (one per GPU), so calls on one GPU must not overlap in time."""
+    _flat_arg(src, "src"), _flat_arg(out, "out")
+    if out.dtype != torch.float64 or out.numel() < 1:
+        raise TypeError("out must be a float64 tensor with at least one element")
+    if out.device != src.device:
+        raise RuntimeError("src and out must live on one device")
+    with _on(src.device):
+        _check(
+            lib.yafsdp_flat_sumsq_static(src.data_ptr(), _dt(src), src.numel(), out.data_ptr(), int(accumulate), _stream(src)),
+            "yafsdp_flat_sumsq_static",
         )
 
 

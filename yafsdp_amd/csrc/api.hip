@@ -16,6 +16,11 @@ using namespace yafsdp;
 
 thread_local yafsdp::TimedLaunch yafsdp::tl_timed_launch;
 
+// Scratch of yafsdp_flat_sumsq_static: the per-workgroup partial sums that yafsdp_flat_sumsq keeps in the caller's
+// workspace.  One copy per GPU the library runs on (128 KiB each), held until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; device memory is reached through the per-device pointer below.
+static __device__ __align__(256) double g_sumsq_static_scratch[yafsdp::kSumsqMaxPartials];
+
 namespace {
 
 std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
@@ -25,6 +30,27 @@ std::atomic<int> g_scatter_tile_mode{0};
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cu_count[kMaxDevices];
+// device address of g_sumsq_static_scratch on each device (every GPU holds its own copy at its own address)
+std::atomic<double*> g_sumsq_static_ptr[kMaxDevices];
+
+// Address of the static scratch on the current device, looked up once per device.
+int sumsq_static_scratch(double** out) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  if (device < 0 || device >= kMaxDevices) return YAFSDP_ERR_WRONG_DEVICE;
+  double* p = g_sumsq_static_ptr[device].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(g_sumsq_static_scratch));
+    if (e != hipSuccess) return int(e);
+    if (sym == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+    p = static_cast<double*>(sym);
+    g_sumsq_static_ptr[device].store(p, std::memory_order_release);  // the same value from whichever thread wins
+  }
+  *out = p;
+  return YAFSDP_OK;
+}
 
 int cu_count(int device) {
   if (device < 0 || device >= kMaxDevices) return 256;
@@ -251,6 +277,8 @@ const char* yafsdp_error_string(int code) {
     case YAFSDP_ERR_MISALIGNED: return "yafsdp: pointer not aligned (element size; 16 bytes for flat table buffers)";
     case YAFSDP_ERR_WRONG_DEVICE: return "yafsdp: table belongs to another device than the current one";
     case YAFSDP_ERR_OUT_OF_MEMORY: return "yafsdp: host allocation failed";
+    case YAFSDP_ERR_TOO_LARGE:
+      return "yafsdp: more elements than the entry point's fixed scratch is specified for (yafsdp_flat_sumsq_static: 2^31)";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -505,6 +533,25 @@ int yafsdp_flat_sumsq(const void* src, int dtype, int64_t n, double* sumsq, int 
                                        stream);
   if (rc != YAFSDP_OK) return rc;
   return int(launch_sumsq_finish(static_cast<double*>(workspace), count, sumsq, accumulate ? 1 : 0, 0.0f, nullptr,
+                                 static_cast<hipStream_t>(stream)));
+}
+
+int64_t yafsdp_flat_sumsq_static_max_numel(void) { return int64_t(1) << 31; }
+
+int yafsdp_flat_sumsq_static(const void* src, int dtype, int64_t n, double* sumsq, int accumulate, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && (src == nullptr || sumsq == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n > yafsdp_flat_sumsq_static_max_numel()) return YAFSDP_ERR_TOO_LARGE;
+  if (n > 0 && (!aligned_to(src, item_size(dtype)) || !aligned_to(sumsq, 8))) return YAFSDP_ERR_MISALIGNED;
+  double* scratch = nullptr;
+  const int rc0 = sumsq_static_scratch(&scratch);  // set-up on the first call on this device
+  if (rc0 != YAFSDP_OK) return rc0;
+  if (n == 0) return YAFSDP_OK;  // a call that only performs the set-up
+  // every partial sum the finishing launch reads is written by the launch before it: nothing has to start at zero
+  int64_t count = 0;
+  const int rc = yafsdp_sumsq_partials(src, dtype, n, scratch, kSumsqMaxPartials, &count, stream);
+  if (rc != YAFSDP_OK) return rc;
+  return int(launch_sumsq_finish(scratch, count, sumsq, accumulate ? 1 : 0, 0.0f, nullptr,
                                  static_cast<hipStream_t>(stream)));
 }
 
