@@ -101,7 +101,11 @@ int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chun
  * yafsdp_post_reduce_sumsq_count(n) are needed); hand them to
  * yafsdp_clip_coef_from_partials, alone or next to the partial sums of other
  * shards.  The values squared are the stored ones (after rounding to the
- * shard's dtype).  shard and chunk must not overlap. */
+ * shard's dtype).  shard and chunk must not overlap.  For a shard that does
+ * not start on a 16-byte boundary *n_written can be one less than
+ * yafsdp_post_reduce_sumsq_count(n); entries of a larger slot beyond
+ * *n_written are not touched, so a caller that adds up the whole slot zeroes
+ * them first. */
 int64_t yafsdp_post_reduce_sumsq_count(int64_t n);
 int yafsdp_post_reduce_sumsq(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
                              double post_factor, int accumulate, double* partials, int64_t capacity,

@@ -6,6 +6,7 @@ import copy
 
 import pytest
 import torch
+import torch.nn as nn
 
 from helpers import assert_bits_equal
 from test_gpu_fully_shard import DEV, MP, _make
@@ -126,6 +127,33 @@ def test_full_state_dict_round_trip_through_the_unwrapped_model():
     fresh.blocks[1].unshard()
     with pytest.raises(RuntimeError, match="sharded state"):
         full_state_dict(fresh)
+
+
+def test_full_state_dict_leaves_non_persistent_buffers_out():
+    """Buffers registered with persistent=False (rotary tables and the like) are not part of module.state_dict();
+    the full state dict follows it, so an ordinary state dict loads with strict=True."""
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.checkpoint import full_state_dict, load_full_state_dict
+
+    class WithBuffers(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = nn.Linear(64, 64)
+            self.register_buffer("scale", torch.full((64,), 2.0))
+            self.register_buffer("inv_freq", torch.arange(64.0), persistent=False)
+
+        def forward(self, x):
+            return self.lin(x) * self.scale + self.inv_freq
+
+    torch.manual_seed(31)
+    plain = WithBuffers().to(DEV)
+    model = fully_shard(copy.deepcopy(plain), mp_policy=MP)
+    sd = full_state_dict(model)
+    assert sorted(sd) == sorted(plain.state_dict()) and "inv_freq" not in sd
+    fresh = fully_shard(WithBuffers().to(DEV), mp_policy=MP)
+    load_full_state_dict(fresh, plain.state_dict(), strict=True)
+    x = torch.randn(4, 64, device=DEV)
+    assert_bits_equal(fresh(x), model(x).detach(), "outputs after loading an ordinary state dict")
 
 
 def test_torch_distributed_checkpoint_round_trip(tmp_path):

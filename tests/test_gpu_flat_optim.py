@@ -368,3 +368,76 @@ def test_fused_grad_norm_falls_back_when_the_reduce_writes_the_shard_directly():
     norm_b, _ = grad_clip_coef(model, 1.0)
     want = torch.sqrt(sum(p.grad.double().pow(2).sum() for p in model.parameters())).float()
     assert torch.allclose(norm_a, norm_b, rtol=2e-7, atol=0) and torch.allclose(norm_b, want, rtol=1e-6, atol=0)
+
+
+def test_fused_grad_norm_small_group_with_a_frozen_parameter_in_the_middle():
+    """A group of three 512-element parameters whose middle one is frozen: its gradient shard has two disjoint
+    ranges, more than the one tile its post-reduce covers.  The read pass must find room for both."""
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.optim import disable_fused_grad_norm, enable_fused_grad_norm, fsdp_param_groups, grad_clip_coef
+
+    class Tiny3(nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(5)
+            self.a = nn.Parameter(torch.randn(512, generator=g))
+            self.b = nn.Parameter(torch.randn(512, generator=g), requires_grad=False)
+            self.c = nn.Parameter(torch.randn(512, generator=g))
+
+        def forward(self, x):
+            return (x * self.a + self.b) * self.c
+
+    model = fully_shard(Tiny3().to(DEV), mp_policy=MP)
+    x = torch.randn(4, 512, device=DEV)
+    model(x).float().pow(2).mean().backward()
+    (group,) = fsdp_param_groups(model)
+    assert group._padded_sharded_param_grad[None].numel() <= 4096
+    enable_fused_grad_norm(model)
+    try:
+        assert group._grad_sumsq_slot[1] - group._grad_sumsq_slot[0] >= 2
+        model.zero_grad(set_to_none=True)
+        model(x).float().pow(2).mean().backward()
+        norm_fused, coef_fused = grad_clip_coef(model, 1e-3)   # two ranges: read pass into the group's slot
+        norm_again, _ = grad_clip_coef(model, 1e-3)            # and again over the same slot
+    finally:
+        disable_fused_grad_norm(model)
+    norm_read, coef_read = grad_clip_coef(model, 1e-3)
+    want = torch.sqrt(sum(p.grad.double().pow(2).sum() for p in model.parameters() if p.grad is not None)).float()
+    assert float(norm_read) > 0 and torch.allclose(norm_read, want, rtol=1e-6, atol=0)
+    assert torch.equal(norm_fused, norm_read) and torch.equal(norm_again, norm_read) and torch.equal(coef_fused, coef_read)
+
+
+def test_fused_grad_norm_slot_is_clean_after_a_read_pass_left_more_sums():
+    """Three trainable 512-element parameters: an iteration whose middle gradient is dropped goes through the read
+    pass and leaves two sums in the group's slot; the next iteration's post-reduce writes one.  The second sum must
+    not be counted again."""
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.optim import disable_fused_grad_norm, enable_fused_grad_norm, grad_clip_coef
+
+    class Tiny3(nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(6)
+            self.a = nn.Parameter(torch.randn(512, generator=g))
+            self.b = nn.Parameter(torch.randn(512, generator=g))
+            self.c = nn.Parameter(torch.randn(512, generator=g))
+
+        def forward(self, x):
+            return (x * self.a + self.b) * self.c
+
+    model = fully_shard(Tiny3().to(DEV), mp_policy=MP)
+    x = torch.randn(4, 512, device=DEV)
+    model(x).float().pow(2).mean().backward()
+    enable_fused_grad_norm(model)
+    try:
+        model.zero_grad(set_to_none=True)
+        model(x).float().pow(2).mean().backward()
+        model.b.grad = None                       # two ranges: read pass, two sums in the slot
+        grad_clip_coef(model, 1e-3)
+        model.zero_grad(set_to_none=True)
+        model(x).float().pow(2).mean().backward()  # all three gradients: the post-reduce's own single sum
+        norm_fused, _ = grad_clip_coef(model, 1e-3)
+    finally:
+        disable_fused_grad_norm(model)
+    norm_read, _ = grad_clip_coef(model, 1e-3)
+    assert float(norm_read) > 0 and torch.equal(norm_fused, norm_read)

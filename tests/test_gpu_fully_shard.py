@@ -560,3 +560,47 @@ def test_activation_checkpointing_recomputes_through_the_hooks():
     want = _train(_wrap(plain0, mp_policy=MP), xs, 0.05)
     got = _train(_wrap(ckpt0, mp_policy=MP), xs, 0.05)
     _assert_same_masters(got, want)
+
+
+def test_device_without_an_index_means_the_current_gpu():
+    """fully_shard(device="cuda") and YaFSDPParamGroup / TensorTable with torch.device("cuda") resolve to the current
+    GPU (tensors always report an indexed device)."""
+    from yafsdp_amd import _native, fully_shard
+
+    model = _make(3)
+    x = torch.randn(4, 128, device=DEV)
+    want = copy.deepcopy(model).to(torch.bfloat16)(x.to(torch.bfloat16))
+    for b in model.blocks:
+        fully_shard(b, mp_policy=MP, device="cuda")
+    fully_shard(model.norm, mp_policy=MP, device=torch.device("cuda"))
+    fully_shard(model, mp_policy=MP, device="cuda")
+    got = model(x)
+    assert torch.equal(got, want)
+    got.float().pow(2).mean().backward()
+    table = _native.TensorTable([8, 24], 32, torch.device("cuda"))
+    flat = torch.zeros(32, dtype=torch.bfloat16, device=DEV)
+    table.gather_in([torch.ones(8, dtype=torch.bfloat16, device=DEV), torch.ones(24, dtype=torch.bfloat16, device=DEV)],
+                    flat, None, None, True)
+    assert float(flat.float().sum()) == 32.0
+    table.close()
+
+
+def test_meta_device_model_is_materialised_empty_and_trains_after_initialisation():
+    """Deferred initialisation as in ya_fsdp/_init.py:205-211: parameters on the meta device become uninitialised
+    device tensors; the caller initialises the sharded parameters afterwards."""
+    from yafsdp_amd import fully_shard
+
+    ref = _make(9)
+    with torch.device("meta"):
+        model = Net()
+    for b in model.blocks:
+        fully_shard(b, mp_policy=MP, device=DEV)
+    fully_shard(model.norm, mp_policy=MP, device=DEV)
+    fully_shard(model, mp_policy=MP, device=DEV)
+    assert all(p.device == DEV for p in model.parameters())
+    with torch.no_grad():
+        for p, q in zip(model.parameters(), ref.parameters()):
+            p.copy_(q.reshape(p.shape))
+    x = torch.randn(4, 128, device=DEV)
+    want = copy.deepcopy(ref).to(torch.bfloat16)(x.to(torch.bfloat16))
+    assert torch.equal(model(x), want)

@@ -282,7 +282,9 @@ def _post_reduce(
         _native.post_reduce(shard, chunk, post, accumulate)
         return
     lo, hi = slot
-    _native.post_reduce_sumsq(shard, chunk, post, accumulate, param_group._grad_sumsq_partials[:hi], lo)
+    end = _native.post_reduce_sumsq(shard, chunk, post, accumulate, param_group._grad_sumsq_partials[:hi], lo)
+    if end < hi:  # the slot is added up as a whole: entries a read pass may have left beyond these sums go
+        param_group._grad_sumsq_partials[end:hi].zero_()
     param_group._grad_sumsq_token = shard._version
 
 

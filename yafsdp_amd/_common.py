@@ -65,6 +65,16 @@ class ShardedState(Enum):
     UNSHARDED = auto()
 
 
+def resolve_device(device: "torch.device | str | int | None") -> torch.device:
+    """A device with an explicit index: ``"cuda"`` means the current GPU, as the reference's device handle
+    resolves it (ya_fsdp/fully_shard.py:110-113 through ``_get_device_from_mesh``).  Tensors always report an
+    indexed device, so comparisons against ``cuda`` without an index would never match."""
+    device = torch.device(f"cuda:{torch.cuda.current_device()}" if device is None else device)
+    if device.type == "cuda" and device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    return device
+
+
 def is_bw() -> bool:
     """ya_fsdp/_common.py:73-74."""
     return torch._C._current_graph_task_id() != -1

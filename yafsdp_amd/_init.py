@@ -111,8 +111,12 @@ def _move_states_to_device(params, buffers, device: torch.device) -> None:
         if tensor.device == device:
             continue
         if tensor.is_meta:
-            raise RuntimeError(
-                "FSDP parameters should be materialized from meta device before training: call "
-                "module.to_empty(device) and initialise the values first"
-            )
-        tensor.data = tensor.to(device)
+            # deferred initialisation (:205-211): an uninitialised tensor of the same shape takes the meta tensor's
+            # place; the caller fills the sharded parameters in afterwards
+            with torch.no_grad():  # avoid autograd increasing C++ refcount by 1
+                empty = torch.empty_like(tensor, device=device)
+                if isinstance(tensor, nn.Parameter):
+                    empty = nn.Parameter(empty, requires_grad=tensor.requires_grad)
+            torch.utils.swap_tensors(tensor, empty)
+        else:
+            tensor.data = tensor.to(device)

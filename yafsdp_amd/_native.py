@@ -324,6 +324,8 @@ class TensorTable:
         self.device = torch.device(device)
         if self.device.type != "cuda":
             raise RuntimeError(f"TensorTable needs a GPU device, got {device}")
+        if self.device.index is None:  # "cuda" means the current GPU; tensors always report an indexed device
+            self.device = torch.device("cuda", torch.cuda.current_device())
         arr = np.ascontiguousarray(self.numels, dtype=np.int64)
         handle = ctypes.c_void_p()
         with _on(self.device):

@@ -49,7 +49,7 @@ from ._collectives import (
     foreach_reduce_copy_in,
     reduce_scatter,
 )
-from ._common import FSDPMeshInfo, ShardedState, TrainingState, is_bw, profiler_range
+from ._common import FSDPMeshInfo, ShardedState, TrainingState, is_bw, profiler_range, resolve_device
 from ._layout import ShardLayout, make_layout
 from ._param import ParamModuleInfo, YaFSDPParam
 
@@ -115,6 +115,7 @@ class YaFSDPParamGroup:
         device = torch.device(device)
         if device.type != "cuda":
             raise RuntimeError(f"the buffer path runs on the GPU only, got device {device}")
+        device = resolve_device(device)
         if mp_policy.all_gather_dtype_to_param_cls:
             raise NotImplementedError("per-class all-gather dtypes (tensor-subclass extensions) are not part of this build")
         names = list(names) if names is not None else [f"param{i}" for i in range(len(params))]
@@ -246,6 +247,19 @@ class YaFSDPParamGroup:
         for fsdp_param, v, g in zip(self.fsdp_params, ag_views, rs_views):
             fsdp_param.init_unsharded_param(v, g)
 
+    def _validate_no_meta_params(self) -> None:
+        """ya_fsdp/_param_group.py:939-951."""
+        param_names_on_meta = [
+            fsdp_param._param_fqn for fsdp_param in self.fsdp_params if fsdp_param.sharded_param.device.type == "meta"
+        ]
+        if param_names_on_meta:
+            raise RuntimeError(
+                "FSDP parameters should be materialized from meta device before training, "
+                f"but the following were still on meta device: {param_names_on_meta}\n"
+                "For example, call module.to_empty(device) to materialize to device and "
+                "call module.reset_parameters() on each module to initialize values."
+            )
+
     def lazy_init(self) -> None:
         """ya_fsdp/_param_group.py:487-547 (idempotent)."""
         if not hasattr(self.comm_ctx, "all_gather_stream"):
@@ -254,6 +268,7 @@ class YaFSDPParamGroup:
             raise RuntimeError(
                 "the data buffer of this group is not allocated: call init_shared_state(groups, device) first"
             )
+        self._validate_no_meta_params()  # :491
         self._register_state_dict_hooks()  # :492
         self._init_unsharded_params()
         shard = self._padded_sharded_param_data[None]

@@ -263,8 +263,18 @@ def full_state_dict(module: nn.Module) -> dict[str, torch.Tensor]:
         if owner.mesh_info.shard_mesh_size != 1:
             raise ValueError(f"{name} is sharded over {owner.mesh_info.shard_mesh_size} logical ranks; use full_tensors")
         out[name] = owner._sharded_param_data.detach().view(owner._orig_size).clone()
-    for name, b in module.named_buffers():
+    for name, b in _persistent_buffers(module).items():
         out[name] = b.detach().clone()
+    return out
+
+
+def _persistent_buffers(module: nn.Module) -> dict[str, torch.Tensor]:
+    """The buffers ``module.state_dict()`` holds: ``persistent=False`` ones (rotary tables and the like) are left out."""
+    out = {}
+    for prefix, sub in module.named_modules():
+        for name, b in sub.named_buffers(recurse=False):
+            if name not in sub._non_persistent_buffers_set:
+                out[f"{prefix}.{name}" if prefix else name] = b
     return out
 
 
@@ -294,7 +304,7 @@ def load_full_state_dict(module: nn.Module, state_dict: Mapping[str, torch.Tenso
             touched.add(id(group))
             group._all_gather_input_set_dtypes.clear()
             group._copy_in_shard_version = None
-    buffers = dict(module.named_buffers())
+    buffers = _persistent_buffers(module)
     for name, b in buffers.items():
         if name in state_dict:
             with torch.no_grad():

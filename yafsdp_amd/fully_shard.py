@@ -13,6 +13,7 @@ import torch
 import torch.nn as nn
 
 from ._api import MixedPrecisionPolicy
+from ._common import resolve_device
 from ._init import _get_managed_modules, _get_managed_states, _move_states_to_device, mesh_info_from
 from ._param_group import YaFSDPParamGroup
 from ._state import YaFSDPState, _get_module_fsdp_state
@@ -48,7 +49,7 @@ def fully_shard(
         if _get_module_fsdp_state(m) is not None:
             raise AssertionError(f"fully_shard has already been applied to {type(m).__name__}")
     mesh_info = mesh_info_from(mesh)
-    device = torch.device(device if device is not None else f"cuda:{torch.cuda.current_device()}")
+    device = resolve_device(device)
     auto_reshard_after_forward = reshard_after_forward is not None
     state = YaFSDPState()
     state.init(modules, device, mp_policy, auto_reshard_after_forward)

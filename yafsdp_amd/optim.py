@@ -145,7 +145,9 @@ def enable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
     device = groups[0].device
     slots, total = [], 0
     for g in groups:
-        n = _native.post_reduce_sumsq_count(g._padded_sharded_param_grad[None].numel())
+        # one partial sum per tile of the post-reduce; the read pass that replaces it when the sums are stale writes
+        # at least one per gradient range, and a group has at most as many ranges as parameters
+        n = max(_native.post_reduce_sumsq_count(g._padded_sharded_param_grad[None].numel()), len(g.fsdp_params), 1)
         slots.append((total, total + n))
         total += n
     partials = torch.zeros(total, dtype=torch.float64, device=device)
@@ -204,8 +206,9 @@ def grad_clip_coef(
             lo, hi = g._grad_sumsq_slot
             fused[lo:hi].zero_()
             pos = lo
-            for a, b in ranges:
-                pos = _native.sumsq_partials(grad_shard[a:b], fused[:hi], pos)
+            for k, (a, b) in enumerate(ranges):
+                # leave one entry for each range still to come (the slot holds at least one per parameter)
+                pos = _native.sumsq_partials(grad_shard[a:b], fused[: hi - (len(ranges) - 1 - k)], pos)
             g._grad_sumsq_token = None
         if fused.numel() > 4 * _native.SUMSQ_MAX_PARTIALS:  # long array: many workgroups first, then one
             scratch = _ClipState.get(device).reserve(1 + fused.numel() // (4096 * _native.SUMSQ_MAX_PARTIALS))
