@@ -11,8 +11,9 @@
  *    allocates or frees caller memory; the only library-owned objects are
  *    metadata tables (yafsdp_table_create / yafsdp_table_destroy).
  *  - `stream` is a hipStream_t passed as void* (NULL = the null stream).  All
- *    work is enqueued on it; no entry point synchronises the device, except
- *    yafsdp_table_create / yafsdp_table_destroy (one-time set-up / tear-down).
+ *    work is enqueued on it; no entry point waits for the device, except
+ *    yafsdp_table_create / yafsdp_binding_create (one-time set-up: blocking
+ *    copies) and yafsdp_table_destroy (waits for the table's queued calls).
  *  - dtype arguments take the yafsdp_dtype values.
  *  - Return value: 0 on success, a positive hipError_t value if a HIP call
  *    failed, a negative yafsdp_status otherwise.  yafsdp_error_string() turns
@@ -44,7 +45,8 @@ typedef enum yafsdp_status {
   YAFSDP_ERR_MISALIGNED = -3,
   YAFSDP_ERR_WRONG_DEVICE = -4,
   YAFSDP_ERR_OUT_OF_MEMORY = -5,
-  YAFSDP_ERR_TOO_LARGE = -6
+  YAFSDP_ERR_TOO_LARGE = -6,
+  YAFSDP_ERR_BUSY = -7
 } yafsdp_status;
 
 /* per-tensor mode of yafsdp_gather_in / yafsdp_scatter_out / fragments */
@@ -146,7 +148,14 @@ int yafsdp_table_info(const yafsdp_table* table, int* n_tensors, int64_t* total_
  *   flat = round(flat / pre_factor)               _div_if_needed(rs_input, pre)
  *         (ya_fsdp/_collectives.py:139)
  * zero_pad != 0 writes 0 to the pad lanes [total, padded) (the reference leaves
- * them uninitialised).  `flat` must be 16-byte aligned. */
+ * them uninitialised).  `flat` must be 16-byte aligned.
+ * Tables with more than 16 tensors hand `tensor_ptrs` and `mode` to the kernel
+ * through one of 8 staging slots inside the table (a pinned-host to device
+ * copy on `stream`).  A call whose arrays equal those of an earlier call still
+ * held by a slot reuses that slot's device copy: no copy is enqueued.  The host
+ * never waits: if all 8 slots belong to calls whose kernels have not finished
+ * yet, the call returns YAFSDP_ERR_BUSY and enqueues nothing (the same holds
+ * for yafsdp_scatter_out, which shares the slots). */
 int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode, int tensor_dtype,
                      void* flat, int flat_dtype, double pre_factor, int zero_pad, void* stream);
 

@@ -159,6 +159,9 @@ def error_string(code: int) -> str:
     return lib.yafsdp_error_string(int(code)).decode()
 
 
+ERR_BUSY = -7  # YAFSDP_ERR_BUSY: every staging slot of a table is held by a queued call
+
+
 def _check(code: int, what: str) -> None:
     if code != 0:
         raise RuntimeError(f"{what} failed: {error_string(code)} (code {code})")
@@ -315,7 +318,11 @@ def all_contiguous(tensors: Sequence[torch.Tensor | None]) -> bool:
 class TensorTable:
     """Device-resident metadata of one flat buffer (tensor boundaries and the
     tile -> tensor map).  Static for the life of a parameter group; the tensor
-    pointers are passed with every call."""
+    pointers are passed with every call.  Tables with more than 16 tensors pass
+    them through 8 staging slots; a call with the same tensors as an earlier
+    one reuses its slot.  Only when 8 calls with 8 different tensor sets are
+    still queued does a further call wait (for the current stream) before it
+    stages its own."""
 
     def __init__(self, numels: Sequence[int], padded_numel: int, device: torch.device):
         self.numels = [int(n) for n in numels]
@@ -431,13 +438,13 @@ class TensorTable:
             tdt = self._fill(tensors, modes, "tensors")
             if tdt < 0:
                 tdt = _dt(flat)
-            _check(
-                lib.yafsdp_gather_in(
-                    self._handle, self._ptrs.ctypes.data, self._modes.ctypes.data, tdt, flat.data_ptr(), _dt(flat),
-                    _factor(pre_factor), int(bool(zero_pad)), _stream(flat),
-                ),
-                "yafsdp_gather_in",
-            )
+            args = (self._handle, self._ptrs.ctypes.data, self._modes.ctypes.data, tdt, flat.data_ptr(), _dt(flat),
+                    _factor(pre_factor), int(bool(zero_pad)), _stream(flat))
+            code = lib.yafsdp_gather_in(*args)
+            if code == ERR_BUSY:  # back-pressure: 8 calls with different tensor sets are still queued on this table
+                torch.cuda.current_stream(self.device).synchronize()
+                code = lib.yafsdp_gather_in(*args)
+            _check(code, "yafsdp_gather_in")
 
     def scatter_out(
         self, flat: torch.Tensor, tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None = None
@@ -450,13 +457,13 @@ class TensorTable:
             tdt = self._fill(tensors, modes, "tensors")
             if tdt < 0:
                 return
-            _check(
-                lib.yafsdp_scatter_out(
-                    self._handle, flat.data_ptr(), _dt(flat), self._ptrs.ctypes.data, self._modes.ctypes.data, tdt,
-                    _stream(flat),
-                ),
-                "yafsdp_scatter_out",
-            )
+            args = (self._handle, flat.data_ptr(), _dt(flat), self._ptrs.ctypes.data, self._modes.ctypes.data, tdt,
+                    _stream(flat))
+            code = lib.yafsdp_scatter_out(*args)
+            if code == ERR_BUSY:  # back-pressure, as in gather_in
+                torch.cuda.current_stream(self.device).synchronize()
+                code = lib.yafsdp_scatter_out(*args)
+            _check(code, "yafsdp_scatter_out")
 
 
 def flat_copy_fanout(dsts: Sequence[torch.Tensor], src: torch.Tensor) -> None:

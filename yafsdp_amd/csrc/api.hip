@@ -158,14 +158,19 @@ struct yafsdp_table {
   std::vector<int64_t> slot_start;  // host, n_tensors + 1
   int32_t n_slots = 0;
   TileRec* d_slots = nullptr;    // only for tables with more than kSmallMax tensors
-  // staging ring for the per-call pointer/mode arrays of tables with more than
-  // kSmallMax tensors: pinned host slot -> device slot, one event per slot
-  static constexpr int kRing = 4;
+  // staging slots for the per-call pointer/mode arrays of tables with more than kSmallMax tensors: pinned host
+  // slot -> device slot.  A slot keeps what was staged into it, so a call whose arrays equal a slot's content
+  // (the caching allocator hands autograd the same addresses step after step) reuses the device copy without
+  // copying again.  ev[s] marks the end of the last kernel that reads slot s.
+  static constexpr int kRing = 8;
   size_t stage_bytes = 0;
-  char* h_stage[kRing] = {nullptr, nullptr, nullptr, nullptr};
-  char* d_stage[kRing] = {nullptr, nullptr, nullptr, nullptr};
-  hipEvent_t ev[kRing] = {nullptr, nullptr, nullptr, nullptr};
-  bool ev_pending[kRing] = {false, false, false, false};
+  char* h_stage[kRing] = {};
+  char* d_stage[kRing] = {};
+  hipEvent_t ev[kRing] = {};
+  bool ev_pending[kRing] = {};
+  bool filled[kRing] = {};          // h_stage[s] / d_stage[s] hold a staged set
+  hipStream_t staged_on[kRing] = {};  // stream the copy into d_stage[s] was enqueued on
+  std::vector<char> scratch;        // host: the arrays of the current call in staging format
   int next = 0;
   std::mutex mu;
 };
@@ -228,24 +233,47 @@ void fill_small(const yafsdp_table* t, const void* const* ptrs, const uint8_t* m
   }
 }
 
-// Large tables: stage pointers (8 bytes each) and modes (4 bytes each) through
-// the ring.  Returns 0 or an error code; *slot is the ring slot used.
+// Large tables: pointers (8 bytes each) and modes (4 bytes each) reach the kernel through a staging slot.
+// Returns 0 or an error code; *slot is the slot used.  Never blocks the host: a slot whose last kernel has not
+// finished is not overwritten, and when every slot is in that state the call fails with YAFSDP_ERR_BUSY.
 int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, LargeMeta* m, int* slot,
                 hipStream_t stream) {
   const int n = t->n_tensors;
-  const int s = t->next;
-  t->next = (t->next + 1) % yafsdp_table::kRing;
-  if (t->ev_pending[s]) {
-    hipError_t e = hipEventSynchronize(t->ev[s]);
-    if (e != hipSuccess) return int(e);
-    t->ev_pending[s] = false;
+  char* cur = t->scratch.data();
+  std::memcpy(cur, ptrs, size_t(n) * sizeof(void*));
+  uint32_t* cm = reinterpret_cast<uint32_t*>(cur + size_t(n) * sizeof(void*));
+  for (int p = 0; p < n; p++) cm[p] = mode ? mode[p] : uint32_t(MODE_COPY);
+  const size_t used = size_t(n) * (sizeof(void*) + sizeof(uint32_t));
+  int s = -1;
+  for (int i = 0; i < yafsdp_table::kRing; i++) {
+    if (t->filled[i] && std::memcmp(t->h_stage[i], cur, used) == 0) { s = i; break; }
   }
-  char* h = t->h_stage[s];
-  std::memcpy(h, ptrs, size_t(n) * sizeof(void*));
-  uint32_t* hm = reinterpret_cast<uint32_t*>(h + size_t(n) * sizeof(void*));
-  for (int p = 0; p < n; p++) hm[p] = mode ? mode[p] : uint32_t(MODE_COPY);
-  hipError_t e = hipMemcpyAsync(t->d_stage[s], h, t->stage_bytes, hipMemcpyHostToDevice, stream);
-  if (e != hipSuccess) return int(e);
+  if (s >= 0) {
+    // same arrays as an earlier call: the device copy is reused.  A kernel on another stream than the one the
+    // copy was enqueued on is ordered behind it (on the device; the host does not wait).
+    if (t->ev_pending[s] && t->staged_on[s] != stream) {
+      hipError_t e = hipStreamWaitEvent(stream, t->ev[s], 0);
+      if (e != hipSuccess) return int(e);
+    }
+  } else {
+    for (int k = 0; k < yafsdp_table::kRing && s < 0; k++) {
+      const int i = (t->next + k) % yafsdp_table::kRing;
+      if (t->ev_pending[i]) {
+        const hipError_t q = hipEventQuery(t->ev[i]);
+        if (q == hipErrorNotReady) continue;  // its last kernel (and the copy before it) is still in flight
+        if (q != hipSuccess) return int(q);
+        t->ev_pending[i] = false;
+      }
+      s = i;
+    }
+    if (s < 0) return YAFSDP_ERR_BUSY;
+    t->next = (s + 1) % yafsdp_table::kRing;
+    std::memcpy(t->h_stage[s], cur, used);
+    t->filled[s] = true;
+    t->staged_on[s] = stream;
+    hipError_t e = hipMemcpyAsync(t->d_stage[s], t->h_stage[s], t->stage_bytes, hipMemcpyHostToDevice, stream);
+    if (e != hipSuccess) { t->filled[s] = false; return int(e); }
+  }
   m->offsets = t->d_offsets;
   m->tiles = t->d_tiles;
   m->slots = t->d_slots;
@@ -277,6 +305,9 @@ const char* yafsdp_error_string(int code) {
     case YAFSDP_ERR_MISALIGNED: return "yafsdp: pointer not aligned (element size; 16 bytes for flat table buffers)";
     case YAFSDP_ERR_WRONG_DEVICE: return "yafsdp: table belongs to another device than the current one";
     case YAFSDP_ERR_OUT_OF_MEMORY: return "yafsdp: host allocation failed";
+    case YAFSDP_ERR_BUSY:
+      return "yafsdp: every staging slot of this table is still in use by a queued call (more than 8 different "
+             "tensor sets in flight): synchronise the stream, or bind tensor sets that persist";
     case YAFSDP_ERR_TOO_LARGE:
       return "yafsdp: more elements than the entry point's fixed scratch is specified for (yafsdp_flat_sumsq_static: 2^31)";
     default: break;
@@ -839,6 +870,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     }
     if (n_tensors > kSmallMax) {
       t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
+      t->scratch.assign(t->stage_bytes, 0);
       for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
         if ((e = hipHostMalloc(reinterpret_cast<void**>(&t->h_stage[i]), t->stage_bytes, hipHostMallocDefault)) != hipSuccess) break;
         if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_stage[i]), t->stage_bytes)) != hipSuccess) break;
