@@ -969,6 +969,12 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="default workload only: skip the `configs` block (the other configurations of the path, each "
+                         "with its own oracle check, about a minute in total)")
+    ap.add_argument("--sustained-seconds", type=float, default=1.5,
+                    help="length of the sustained leg: back-to-back steps of the workload for at least this long "
+                         "(0 disables it)")
     ap.add_argument("--table-large-log2", type=int, default=None, metavar="N",
                     help="tables with more than 2^N padded elements run two waves per workgroup instead of one "
                          "(the library's launch-shape option; default: the library's own threshold)")
@@ -994,6 +1000,45 @@ def main() -> int:
         return run_ceilings(args)
     if args.workload == "fully-shard-trainer-w1":
         return run_trainer(args)
+    try:
+        out = run_layer(args, args.workload, args.steps, args.warmup, full=True)
+        if args.workload == "llama3-8b-layer-w8" and not args.no_configs:
+            # the other configurations of the path, each with its own in-run oracle check (outside the headline's
+            # timed region; bounded: fewer steps, no per-kernel tables, no baselines)
+            out["configs"] = {}
+            for wl, steps in (("tiny-layer-w1", 200), ("llama3-70b-layer-w64", 20), ("ragged-stress-w256", 30),
+                              ("ragged-stress-w256-bf16-masters", 30)):
+                t0 = time.perf_counter()
+                out["configs"][wl] = run_layer(args, wl, steps, 5, full=False)
+                log(f"config {wl}: {out['configs'][wl]['value']} GB/s, {time.perf_counter() - t0:.1f}s wall")
+    except ParityError as exc:
+        log(f"bench.py: {exc}; refusing to report a throughput.")
+        return 4
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+class ParityError(RuntimeError):
+    pass
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -> dict:
+    """One parameter group's pass (copy-in, copy-out, reduce copy-in, post-reduce) on synthetic inputs of the named
+    workload: parity against the oracle, `warmup` untimed and `steps` timed passes.  `full` adds the per-kernel
+    tables, the sustained leg, graph replay and the baselines; without it only the timed passes and the parity
+    check run, and a compact record comes back."""
+    import torch
+
     from yafsdp_amd import _native
     from yafsdp_amd._layout import make_layout
 
@@ -1004,20 +1049,20 @@ def main() -> int:
     # master / compute / reduce dtypes of the group: fp32 masters with bf16 compute and reduce, except the stress
     # test's second group (bf16 masters: no copy-in cast, fp32 reduce buffer, bf16 gradient shard)
     master_dt, rs_dt = torch.float32, torch.bfloat16
-    if args.workload == "ragged-stress-w256":
+    if workload == "ragged-stress-w256":
         shapes, w, r, align, seed = _ragged_stress_shapes(), 256, 1, 512, 1005
-    elif args.workload == "ragged-stress-w256-bf16-masters":
+    elif workload == "ragged-stress-w256-bf16-masters":
         shapes, w, r, align, seed = _ragged_stress_shapes(fp32_masters=False), 256, 1, 512, 1005
         master_dt, rs_dt = torch.bfloat16, torch.float32
     else:
-        shapes, w, r, align, seed = WORKLOADS[args.workload]
+        shapes, w, r, align, seed = WORKLOADS[workload]
     msz, rsz = master_dt.itemsize, rs_dt.itemsize
     has_copy_in = master_dt != torch.bfloat16
     numels = [numel_of(s) for s in shapes]
     lay = make_layout(numels, w, align)
     t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
     pre = float(w) if w > 1 else None
-    log(f"workload {args.workload}: P={len(numels)} T={t} T_pad={t_pad} S={s} W={w} rank={r} pre-divide={pre}")
+    log(f"workload {workload}: P={len(numels)} T={t} T_pad={t_pad} S={s} W={w} rank={r} pre-divide={pre}")
 
     # ---- synthetic inputs, generated on the CPU so that the oracle sees the same bits
     g = torch.Generator().manual_seed(seed)
@@ -1107,8 +1152,7 @@ def main() -> int:
         parity = "bit-exact" if ok else "MISMATCH"
         log("parity vs oracle:", parity)
         if not ok:
-            log("bench.py: GPU results differ from the oracle; refusing to report a throughput.")
-            return 4
+            raise ParityError(f"{workload}: GPU results differ from the oracle")
 
     if args.calibrate_copy > 0:
         d_copy = torch.empty(t_pad, dtype=torch.bfloat16, device=dev)
@@ -1118,30 +1162,57 @@ def main() -> int:
         del d_copy
 
     # ---- timed region
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     dom_index = [n for n, _, _ in ops].index("reduce_copy_in")  # most bytes, fused arithmetic
     # on every 4th step of the timed region the dominant kernel's dispatch carries a pair of HIP events (attached to
     # the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
-    sampled = [k for k in range(args.steps) if k % 4 == 0]
+    sampled = [k for k in range(steps) if k % 4 == 0]
     ev = {k: _event_pair() for k in sampled}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     fns = [fn for _, fn, _ in ops]
-    for k in range(args.steps):
+    for k in range(steps):
         for i, fn in enumerate(fns):
             if i == dom_index and k in ev:
                 _native.time_next_launch(*ev[k])
             fn()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    value = bytes_per_step * args.steps / elapsed / 1e9
+    ms_per_step = elapsed * 1e3 / steps
+    value = bytes_per_step * steps / elapsed / 1e9
     dom_us = [a.elapsed_time(b) * 1e3 for a, b in ev.values()]
     dom_avg_us = sum(dom_us) / len(dom_us)
     dom_bytes = ops[dom_index][2]
     achieved = dom_bytes / dom_avg_us / 1e3
+
+    if not full:
+        out_binding.close()
+        table.close()
+        return {
+            "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms_per_step, 4), "steps": steps,
+            "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "parity": parity, "bytes_per_step": bytes_per_step,
+            "params": len(numels), "padded_numel": t_pad, "shard_numel": s, "logical_world_size": w,
+            "dominant_kernel_us": round(dom_avg_us, 2), "dominant_kernel_GBps": round(achieved, 1),
+        }
+
+    # ---- sustained leg: back-to-back steps for at least --sustained-seconds (outside the timed region above; the
+    # same eager calls, long enough for clocks and the memory system to settle)
+    sustained = None
+    if args.sustained_seconds > 0:
+        n_sus = max(steps, int(args.sustained_seconds / (ms_per_step * 1e-3)) + 1)
+        torch.cuda.synchronize()
+        s0 = time.perf_counter()
+        for _ in range(n_sus):
+            for fn in fns:
+                fn()
+        torch.cuda.synchronize()
+        s_dt = time.perf_counter() - s0
+        sustained = {"steps": n_sus, "seconds": round(s_dt, 3), "ms_per_step": round(s_dt * 1e3 / n_sus, 4),
+                     "value": round(bytes_per_step * n_sus / s_dt / 1e9, 1), "unit": "GB/s",
+                     "frac_of_hbm_peak": round(bytes_per_step * n_sus / s_dt / 1e9 / HBM_PEAK_GBS, 4)}
+        log(f"sustained: {n_sus} steps in {s_dt:.2f}s, {sustained['value']} GB/s")
 
     # ---- the same step captured into a HIP graph and replayed (outside the timed region): both sides of the table
     # are bound, so the captured launches carry no per-call host work and no staging copy
@@ -1170,10 +1241,10 @@ def main() -> int:
                 graph.replay()
             torch.cuda.synchronize()
             g0 = time.perf_counter()
-            for _ in range(args.steps):
+            for _ in range(steps):
                 graph.replay()
             torch.cuda.synchronize()
-            g_dt = (time.perf_counter() - g0) / args.steps
+            g_dt = (time.perf_counter() - g0) / steps
             graph_replay = {"ms_per_step": round(g_dt * 1e3, 4), "value": round(bytes_per_step / g_dt / 1e9, 1), "unit": "GB/s"}
             log(f"HIP graph replay of the step: {graph_replay['ms_per_step']} ms, {graph_replay['value']} GB/s")
             del graph
@@ -1250,9 +1321,13 @@ def main() -> int:
     if args.cpu_seconds > 0 and cpu_state is not None:
         from oracle import torch_ops  # noqa: F811
 
+        cores = os.cpu_count() or 1
+        torch.set_num_threads(cores)  # every host core the box shows
+        for _ in range(3):            # warm-up passes (page faults, thread pool start-up), not timed
+            cpu_step(cpu_state)
         reps, spent = 0, 0.0
         times = []
-        while spent < args.cpu_seconds and reps < 2000:
+        while (spent < args.cpu_seconds or reps < 10) and reps < 2000:
             c0 = time.perf_counter()
             cpu_step(cpu_state)
             dt = time.perf_counter() - c0
@@ -1261,10 +1336,10 @@ def main() -> int:
             reps += 1
         med = statistics.median(times)
         cpu_baseline = {
-            "value": round(bytes_per_step / med / 1e9, 2), "unit": "GB/s", "cores": torch.get_num_threads(),
-            "kind": "port",
-            "sample": f"{reps} full passes of the same workload ({args.workload}) with the reference's torch ops "
-                      f"on CPU tensors, median of {reps}, {spent:.1f}s total",
+            "value": round(bytes_per_step / med / 1e9, 2), "unit": "GB/s", "cores": cores,
+            "kind": "port", "cpu_model": cpu_model(), "torch_threads": torch.get_num_threads(),
+            "sample": f"{reps} full passes of the same workload ({workload}) with the reference's torch ops "
+                      f"on CPU tensors after 3 warm-up passes, median of {reps}, {spent:.1f}s total",
         }
         log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads ({reps} passes)")
 
@@ -1314,8 +1389,8 @@ def main() -> int:
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -1323,7 +1398,7 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": args.workload, "params": len(numels), "total_numel": t, "padded_numel": t_pad,
+            "workload": workload, "params": len(numels), "total_numel": t, "padded_numel": t_pad,
             "shard_numel": s, "logical_world_size": w, "rank": r, "shard_alignment": align,
             "predivide": pre, "bytes_per_step": bytes_per_step,
             "master_dtype": str(master_dt).replace("torch.", ""), "reduce_dtype": str(rs_dt).replace("torch.", ""),
@@ -1336,19 +1411,20 @@ def main() -> int:
         "roofline": {
             "bound": "hbm", "kernel": "gather_in_kernel (reduce copy-in)", "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
             "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2), "launches_timed": len(dom_us),
         },
         "cpu_baseline": cpu_baseline,
         "torch_gpu_baseline": torch_gpu,
         "graph_replay": graph_replay,
+        "sustained": sustained,
+        "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
         "kernels": kernels,
         "kernel_variants": variants,
     }
-    print(json.dumps(out), flush=True)
     out_binding.close()
     table.close()
-    return 0
+    return out
 
 
 if __name__ == "__main__":

@@ -3,8 +3,9 @@
 Config 2 (Llama-3-8B layer, W=8) and config 5 (2000 ragged tensors, W=256) are
 compared element for element with the oracle.  Config 3 (Llama-3-70B layer,
 W=64; 856 M elements) is checked through size-independent properties at full
-size (round trips, linearity of the divide, pad zero-fill, checksums) and
-against the oracle on the last rank's shard, which holds the pad lanes.
+size (round trips, linearity of the divide, pad zero-fill, checksums), against
+the oracle element for element on the fused reduce copy-in with its divide by
+64, and against the oracle on the last rank's shard, which holds the pad lanes.
 Config 4 (the full 8B model) adds the embedding / head group (525 M elements,
 one tensor) and the final-norm group (4096 elements) to config 2's layers.
 Inputs are generated on the GPU from a fixed seed and copied to the host for
@@ -130,6 +131,16 @@ def test_config3_llama70b_layer_w64_properties(nat):
     table.gather_in(outs, fused, None, 64.0, True)
     nat.flat_div(back, 64.0)
     assert torch.equal(fused.view(torch.int16), back.view(torch.int16))
+    # (d') the fused copy + divide by 64 against the reference's ops at full size, element for element:
+    # _foreach_copy_ into the views of the reduce buffer (ya_fsdp/_param_group.py:693-700), then div_ of the padded
+    # buffer (ya_fsdp/_collectives.py:139) on an 856 M-element bf16 buffer on the host
+    outs_cpu = [o.cpu() for o in outs]
+    rs_cpu = torch.zeros(t_pad, dtype=torch.bfloat16)
+    torch_ops.reduce_copy_in(list(rs_cpu[:t].split(numels)), outs_cpu, False)
+    torch_ops.div_if_needed(rs_cpu, 64.0)
+    fused_cpu = fused.cpu()
+    assert torch.equal(fused_cpu.view(torch.int16), rs_cpu.view(torch.int16)), "fused reduce copy-in /64 vs the oracle"
+    del outs_cpu, rs_cpu, fused_cpu
     # (e) accumulate twice == exact doubling (x + x is exact in bf16 unless it overflows)
     acc = torch.zeros(t_pad, dtype=torch.bfloat16, device=DEV)
     table.gather_in(outs, acc, None, None, True)
