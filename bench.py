@@ -111,12 +111,84 @@ def _cu_masked_streams(torch, dev, k: int):
     return out
 
 
+def analyze_overlap_trace(path: str) -> int:
+    """Reads the kernel trace (CSV) that ``rocprofv3 --kernel-trace --output-format csv`` wrote for
+    ``--workload llama3-8b-full-w8 --steps 10 --no-parity`` and prints, per GEMM stand-in: the register, LDS and
+    workgroup columns of the GEMM kernel, kernel durations alone and inside the overlapped pass, and for how long
+    GEMMs, copy kernels and both at once were running during that pass."""
+    import csv
+
+    def kind(name):
+        if name.startswith("Cijk"):
+            return "gemm"
+        for key, k in (("scatter_out_kernel", "copy_out"), ("gather_in_kernel", "reduce_copy_in"),
+                       ("flat_kernel<yafsdp::F32", "copy_in"), ("flat_kernel<yafsdp::BF16", "post_reduce")):
+            if key in name:
+                return k
+        return None
+
+    rows = [r for r in csv.DictReader(open(path)) if kind(r["Kernel_Name"])]
+    ev = sorted((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), kind(r["Kernel_Name"]), int(r["Grid_Size_X"]), r)
+                for r in rows)
+    gem = [e for e in ev if e[2] == "gemm"]
+    if len(gem) != 3 * 945:
+        log(f"expected 2835 GEMM launches (3 stand-ins x 3 phases - alone, overlapped, overlapped with the other "
+            f"stream plan - x 3 passes x 105), found {len(gem)}: take the trace with --steps 10 --no-parity")
+
+    def union(iv):
+        iv = sorted(iv)
+        out, (cs, ce) = [], iv[0]
+        for a_, b_ in iv[1:]:
+            if a_ <= ce:
+                ce = max(ce, b_)
+            else:
+                out.append((cs, ce))
+                cs, ce = a_, b_
+        out.append((cs, ce))
+        return out
+
+    per = len(gem) // 3  # GEMM launches per stand-in: passes alone, overlapped, overlapped with the other plan
+    passes = per // 105
+    for shape in range(3):
+        g = gem[shape * per : (shape + 1) * per]
+        alone, both = g[2 * 105 : 3 * 105], g[(passes // 3 + 2) * 105 : (passes // 3 + 3) * 105]
+        r0 = g[0][4]
+        print(f"GEMM stand-in {shape}: {r0['Kernel_Name'][:60]}... workgroup {r0['Workgroup_Size_X']}, grid "
+              f"{int(r0['Grid_Size_X']) // int(r0['Workgroup_Size_X'])} workgroups, VGPR {r0['VGPR_Count']}, accum VGPR "
+              f"{r0['Accum_VGPR_Count']}, SGPR {r0['SGPR_Count']}, LDS {r0['LDS_Block_Size']} B, scratch {r0['Scratch_Size']}")
+        t0, t1 = both[0][0], both[-1][1]
+        cop = [e for e in ev if e[2] != "gemm" and e[1] > t0 and e[0] < t1]
+        ug = union([(e[0], e[1]) for e in both])
+        uc = union([(max(e[0], t0), min(e[1], t1)) for e in cop])
+        i = j = ov = 0
+        while i < len(ug) and j < len(uc):
+            a_, b_ = max(ug[i][0], uc[j][0]), min(ug[i][1], uc[j][1])
+            if a_ < b_:
+                ov += b_ - a_
+            if ug[i][1] < uc[j][1]:
+                i += 1
+            else:
+                j += 1
+        tot = lambda u: sum(b_ - a_ for a_, b_ in u)  # noqa: E731
+        avg = lambda xs: sum(xs) / max(len(xs), 1) / 1e3  # noqa: E731
+        print(f"  overlapped pass: {(t1 - t0) / 1e6:.2f} ms from first to last GEMM; GEMM kernels running {tot(ug) / 1e6:.2f} ms, "
+              f"copy kernels running {tot(uc) / 1e6:.2f} ms, both at once {ov / 1e6:.2f} ms")
+        print(f"  GEMM kernel: {avg([e[1] - e[0] for e in alone]):.1f} us alone, {avg([e[1] - e[0] for e in both]):.1f} us in the overlapped pass")
+        for k in ("copy_in", "copy_out", "reduce_copy_in", "post_reduce"):
+            d1 = [e[1] - e[0] for e in cop if e[2] == k and e[3] > 1_000_000]
+            print(f"  {k:15s} (decoder layers) {avg(d1):7.1f} us per launch in the overlapped pass")
+    return 0
+
+
 def run_full_model(args) -> int:
     """Full Llama-3-8B per-rank pass at logical W=8 on one GPU: embedding, 32 decoder layers, lm_head and
     the final norm as 35 parameter groups.  Forward: copy-in + copy-out of group i+1 run on a side stream while a
-    bf16 [4096x4096]x[4096x4096] GEMM stands in for the compute of group i.  Backward (reverse order): two GEMMs
-    per group, then reduce copy-in on the compute stream and post-reduce on the side stream.  Reports the overlap
-    efficiency and per-kernel GB/s (un-overlapped)."""
+    bf16 GEMM stands in for the compute of group i.  Backward (reverse order): two GEMMs per group, then reduce
+    copy-in on the compute stream and post-reduce on the side stream, all groups sharing one reduce buffer per
+    shape.  One overlapped pass is checked against the oracle (embedding, a decoder layer, the final norm: all-gather
+    input, copy-out tensors, gradient shard; every group has gradients of its own, so a pass that let two groups
+    meet in the shared reduce buffer would show).  Reports the overlap efficiency for three GEMM stand-ins (the
+    4096^3 square and the two MLP GEMMs of a Llama-3-8B layer at 4096 tokens) and per-kernel GB/s (un-overlapped)."""
     import torch
 
     from yafsdp_amd import _native
@@ -137,7 +209,8 @@ def run_full_model(args) -> int:
             out[i : i + m] = (torch.randn(m, device=dev, generator=gen) * std).to(dtype)
         return out
 
-    # per-shape shared resources (synthetic gathered buffers, gradients, output tensors and tables)
+    # per-shape shared resources (the 2 shared data buffers, the shared gradient buffer, output tensors, tables);
+    # master shard, gradient shard and gradients are each group's own
     shape_res = {}
     groups = []
     for name, shapes in zip(names, group_shapes):
@@ -147,22 +220,18 @@ def run_full_model(args) -> int:
         if key not in shape_res:
             t_pad = lay.padded_unsharded_numel
             shape_res[key] = {
-                "lay": lay, "table": _native.TensorTable(numels, t_pad, dev),
-                "gathered": [randn(t_pad, 0.02, torch.bfloat16) for _ in range(2)],  # the 2 shared data buffers
+                "lay": lay, "table": _native.TensorTable(numels, t_pad, dev), "numels": numels,
+                "gathered": [randn(t_pad, 0.02, torch.bfloat16) for _ in range(2)],
                 "outs": [[torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels] for _ in range(2)],
-                "grads": [randn(n, 1e-3, torch.bfloat16) for n in numels],
-                "rs": torch.zeros(t_pad, dtype=torch.bfloat16, device=dev),  # the shared gradient buffer
+                "rs": torch.zeros(t_pad, dtype=torch.bfloat16, device=dev),
             }
         s_ = lay.padded_sharded_numel
         groups.append({
             "name": name, "res": shape_res[key], "lay": lay,
             "master": randn(s_, 0.02, torch.float32), "ag_in": torch.zeros(s_, dtype=torch.bfloat16, device=dev),
-            "shard": randn(s_, 1e-4, torch.float32),
+            "shard": randn(s_, 1e-4, torch.float32), "grads": [randn(n, 1e-3, torch.bfloat16) for n in numels],
         })
     log(f"{len(groups)} groups, {torch.cuda.memory_allocated() / 1e9:.1f} GB allocated")
-    a = randn(4096 * 4096, 0.02, torch.bfloat16).view(4096, 4096)
-    b = randn(4096 * 4096, 0.02, torch.bfloat16).view(4096, 4096)
-    c = torch.empty(4096, 4096, dtype=torch.bfloat16, device=dev)
     side = torch.cuda.Stream(device=dev)  # default priority
     main = torch.cuda.current_stream(dev)
     if args.copy_cus:
@@ -170,6 +239,16 @@ def run_full_model(args) -> int:
         # GEMMs' stream the others (the HIP runtime's per-stream CU mask; both at default priority)
         side, main = _cu_masked_streams(torch, dev, args.copy_cus)
         torch.cuda.set_stream(main)
+
+    gemm_state = {}
+
+    def set_gemm(m, k, n_):
+        gemm_state["a"] = randn(m * k, 0.02, torch.bfloat16).view(m, k)
+        gemm_state["b"] = randn(k * n_, 0.02, torch.bfloat16).view(k, n_)
+        gemm_state["c"] = torch.empty(m, n_, dtype=torch.bfloat16, device=dev)
+
+    def gemm():
+        torch.matmul(gemm_state["a"], gemm_state["b"], out=gemm_state["c"])
 
     def unshard(i):  # copy-in + copy-out of group i (current stream)
         g = groups[i]
@@ -179,7 +258,7 @@ def run_full_model(args) -> int:
 
     def reduce_in(i):
         g = groups[i]
-        g["res"]["table"].gather_in(g["res"]["grads"], g["res"]["rs"], None, float(w), True)
+        g["res"]["table"].gather_in(g["grads"], g["res"]["rs"], None, float(w), True)
 
     def post(i):
         g = groups[i]
@@ -188,7 +267,7 @@ def run_full_model(args) -> int:
 
     n = len(groups)
 
-    def step(copies=True, gemms=True):
+    def step(copies=True, gemms=True, gather_on_side=False):
         # forward
         ready = [None] * n
         if copies:
@@ -203,52 +282,144 @@ def run_full_model(args) -> int:
             if copies:
                 main.wait_event(ready[i])
             if gemms:
-                torch.matmul(a, b, out=c)
+                gemm()
         # backward, reverse order
-        freed = None
+        freed = {}
         for i in reversed(range(n)):
             if gemms:
-                torch.matmul(a, b, out=c)
-                torch.matmul(a, b, out=c)
-            if copies:
-                if freed is not None:
-                    main.wait_event(freed)        # the single gradient buffer is released by the previous post-reduce
+                gemm()
+                gemm()
+            if copies and not gather_on_side:
+                key = id(groups[i]["res"])
+                if key in freed:
+                    main.wait_event(freed[key])   # a shared gradient buffer is released by the post-reduce before
                 reduce_in(i)                      # compute stream, like the reference's foreach calls
                 done = main.record_event()
                 with torch.cuda.stream(side):     # reduce-scatter stream: waits for the compute stream
                     side.wait_event(done)
                     post(i)
-                    freed = side.record_event()
+                    freed[key] = side.record_event()
+            elif copies:
+                # not the reference's plan: the reduce copy-in leaves the compute stream as well (the side stream
+                # waits for the gradients, then runs both kernels; its own order keeps the shared buffer safe)
+                done = main.record_event()
+                with torch.cuda.stream(side):
+                    side.wait_event(done)
+                    reduce_in(i)
+                    post(i)
 
-    def timed(copies, gemms, reps):
+    def timed(copies, gemms, reps, gather_on_side=False):
         for _ in range(2):
-            step(copies, gemms)
+            step(copies, gemms, gather_on_side)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(reps):
-            step(copies, gemms)
+            step(copies, gemms, gather_on_side)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / reps * 1e3
 
+    def timed_loop(fn, reps):
+        """ms per pass of fn(i) over all groups, back to back on the current stream."""
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            for i in range(n):
+                fn(i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    # ---- parity of one overlapped pass against the oracle (three groups; both streams busy)
+    parity = "skipped"
+    set_gemm(4096, 4096, 4096)
+    if not args.no_parity:
+        from oracle import torch_ops
+
+        checked = [0, 17, n - 1]  # embedding, a decoder layer in the middle, the final norm
+        before = {i: groups[i]["shard"].cpu() for i in checked}
+        step(True, True)
+        torch.cuda.synchronize()
+
+        def same(a, b):
+            iv = torch.int32 if a.dtype == torch.float32 else torch.int16
+            return torch.equal(a.cpu().view(iv), b.view(iv))
+
+        ok = True
+        for i in checked:
+            g, res, lay = groups[i], groups[i]["res"], groups[i]["lay"]
+            numels = res["numels"]
+            t_, tp, s_ = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+            ag = torch.zeros(s_, dtype=torch.bfloat16)
+            torch_ops.copy_in(ag, g["master"].cpu())
+            outs = [torch.empty(m, dtype=torch.bfloat16) for m in numels]
+            torch_ops.copy_out_materialize(res["gathered"][i % 2].cpu(), numels, outs)
+            rs = torch.zeros(tp, dtype=torch.bfloat16)
+            torch_ops.reduce_copy_in(list(rs[:t_].split(numels)), [x.cpu() for x in g["grads"]], False)
+            shard = before[i].clone()
+            torch_ops.reduce_scatter_local(shard, rs, w, r, float(w), None, "add")
+            good = same(g["ag_in"], ag) and same(g["shard"], shard)
+            # the copy-out tensors of a buffer index are rewritten by every group of that shape and index from the
+            # same source, so their final content is this group's as well
+            good = good and all(same(a_, b_) for a_, b_ in zip(res["outs"][i % 2], outs))
+            log(f"  parity of group {g['name']}: {'bit-exact' if good else 'MISMATCH'}")
+            ok = ok and good
+        parity = "bit-exact" if ok else "MISMATCH"
+        if not ok:
+            log("bench.py: the overlapped pass differs from the oracle; refusing to report a throughput.")
+            return 4
+        del before
+
     reps = max(1, args.steps // 10)
-    t_gemm = timed(False, True, reps)
-    sweep = {}
     caps = (4096, 16, 8, 4, 2, 1) if args.sweep_grid_cap else (4096,)
-    for bpc in caps:  # grid cap of the copy kernels in workgroups per compute unit
-        _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, bpc)
-        _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, bpc)
-        tc = timed(True, False, reps)
-        tb = timed(True, True, reps)
-        sweep[bpc] = {"ms_copies_alone": round(tc, 3), "ms_overlapped": round(tb, 3),
-                      "overlap_efficiency": round(max(tc, t_gemm) / tb, 4)}
-        log(f"  grid cap {bpc:5d} workgroups/CU: copies alone {tc:.3f} ms, overlapped {tb:.3f} ms, "
-            f"efficiency {max(tc, t_gemm) / tb:.3f}")
-    best = min(sweep, key=lambda k: sweep[k]["ms_overlapped"])
-    _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, 4096)
-    _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, 4096)
-    t_copy, t_both = sweep[best]["ms_copies_alone"], sweep[best]["ms_overlapped"]
-    eff = max(t_copy, t_gemm) / t_both
-    hidden = (t_copy + t_gemm - t_both) / min(t_copy, t_gemm)
+    gemm_shapes = [("4096x4096x4096", (4096, 4096, 4096)), ("llama-mlp-up 4096x4096x14336", (4096, 4096, 14336)),
+                   ("llama-mlp-down 4096x14336x4096", (4096, 14336, 4096))]
+    per_gemm = {}
+    t_copy_first = None
+    # the three kinds of copy work on their own: what the forward prefetch has to hide (copy-in + copy-out), what the
+    # reference's plan leaves on the compute stream (reduce copy-in), and what follows it on the side stream
+    t_unshard, t_gather, t_post = timed_loop(unshard, reps), timed_loop(reduce_in, reps), timed_loop(post, reps)
+    log(f"  copies by kind, alone: copy-in + copy-out {t_unshard:.3f} ms, reduce copy-in {t_gather:.3f} ms, "
+        f"post-reduce {t_post:.3f} ms per pass over {n} groups")
+    for gname, (m_, k_, n_) in gemm_shapes:
+        set_gemm(m_, k_, n_)
+        t_gemm = timed(False, True, reps)
+        sweep = {}
+        for bpc in caps:  # grid cap of the copy kernels in workgroups per compute unit
+            _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, bpc)
+            _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, bpc)
+            tc = timed(True, False, reps)
+            tb = timed(True, True, reps)
+            sweep[bpc] = {"ms_copies_alone": round(tc, 3), "ms_overlapped": round(tb, 3),
+                          "overlap_efficiency": round(max(tc, t_gemm) / tb, 4)}
+            log(f"  {gname}: grid cap {bpc:5d} workgroups/CU: copies alone {tc:.3f} ms, gemms alone {t_gemm:.3f} ms, "
+                f"overlapped {tb:.3f} ms, efficiency {max(tc, t_gemm) / tb:.3f}")
+        best = min(sweep, key=lambda k: sweep[k]["ms_overlapped"])
+        _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, 4096)
+        _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, 4096)
+        t_copy, t_both = sweep[best]["ms_copies_alone"], sweep[best]["ms_overlapped"]
+        # what the stream plan allows at best: in the forward pass copy-out of group i+1 hides behind GEMM i (or
+        # the other way round), with the first group's copies exposed; in the backward pass the reduce copy-in is
+        # on the compute stream (ya_fsdp/_param_group.py:669-708), in line with the GEMMs, and only the
+        # post-reduce is on the side stream
+        critical = max(t_gemm / 3.0, t_unshard) + t_unshard / n + t_gemm * 2.0 / 3.0 + t_gather + t_post / n
+        t_alt = timed(True, True, reps, gather_on_side=True)
+        log(f"  {gname}: critical path of the reference's stream plan {critical:.3f} ms; with the reduce copy-in on "
+            f"the side stream as well: overlapped {t_alt:.3f} ms")
+        per_gemm[gname] = {
+            "critical_path_ms": round(critical, 4), "efficiency_vs_critical_path": round(critical / t_both, 4),
+            "ms_overlapped_reduce_copy_in_on_side_stream": round(t_alt, 4),
+            "ms_copies_alone": round(t_copy, 4), "ms_gemms_alone": round(t_gemm, 4), "ms_overlapped": round(t_both, 4),
+            "overlap_efficiency": round(max(t_copy, t_gemm) / t_both, 4),
+            "hidden_fraction": round((t_copy + t_gemm - t_both) / min(t_copy, t_gemm), 4),
+            "gemm_TFLOPs_alone": round(2.0 * m_ * k_ * n_ * 3 * n / t_gemm / 1e9, 1),
+            "grid_cap_sweep": sweep, "grid_cap_used": best,
+        }
+        if t_copy_first is None:
+            t_copy_first = t_copy
+    first = per_gemm[gemm_shapes[0][0]]
+    t_copy, t_gemm, t_both = first["ms_copies_alone"], first["ms_gemms_alone"], first["ms_overlapped"]
+    eff, hidden = first["overlap_efficiency"], first["hidden_fraction"]
     bytes_step = 0
     for g in groups:
         lay = g["lay"]
@@ -278,12 +449,16 @@ def run_full_model(args) -> int:
         "metric": "overlap efficiency of the buffer path against a GEMM stand-in, full Llama-3-8B per-rank pass @W=8",
         "value": round(eff, 4), "unit": "max(copies, gemms) / overlapped", "n_gpus": 1, "steps": reps, "warmup": 2,
         "ms_per_step": round(t_both, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "bf16", "data": "synthetic", "parity": parity,
         "config": {"workload": "llama3-8b-full-w8", "groups": n, "logical_world_size": w, "rank": r,
-                   "gemm": "bf16 4096x4096x4096, 1 per group forward, 2 per group backward",
+                   "gemm": "bf16 4096x4096x4096, 1 per group forward, 2 per group backward (headline value); "
+                           "the two Llama-3-8B MLP GEMMs at 4096 tokens under `gemm_shapes`",
                    "copy_stream_compute_units": args.copy_cus or 256},
         "ms_copies_alone": round(t_copy, 4), "ms_gemms_alone": round(t_gemm, 4), "ms_overlapped": round(t_both, 4),
-        "hidden_fraction": round(hidden, 4), "grid_cap_sweep": sweep, "grid_cap_used": best, "copy_GBps_alone": round(bytes_step / t_copy / 1e6, 1),
+        "hidden_fraction": round(hidden, 4),
+        "ms_copies_by_kind_alone": {"copy_in_and_copy_out": round(t_unshard, 4), "reduce_copy_in": round(t_gather, 4),
+                                    "post_reduce": round(t_post, 4)},
+        "gemm_shapes": per_gemm, "copy_GBps_alone": round(bytes_step / t_copy / 1e6, 1),
         "copy_GBps_overlapped_lower_bound": round(bytes_step / t_both / 1e6, 1), "bytes_per_step": bytes_step,
         "kernels": kernels,
     }
@@ -978,8 +1153,13 @@ def main() -> int:
     ap.add_argument("--table-large-log2", type=int, default=None, metavar="N",
                     help="tables with more than 2^N padded elements run two waves per workgroup instead of one "
                          "(the library's launch-shape option; default: the library's own threshold)")
+    ap.add_argument("--analyze-trace", metavar="CSV", default=None,
+                    help="llama3-8b-full-w8 only: no GPU work; summarise the kernel-trace CSV that rocprofv3 wrote for "
+                         "`--workload llama3-8b-full-w8 --steps 10 --no-parity` (GEMM resource columns, concurrency)")
     args = ap.parse_args()
 
+    if args.analyze_trace:
+        return analyze_overlap_trace(args.analyze_trace)
     if args.gpus != 1:
         log(f"bench.py: this build runs on ONE GPU (the logical world size is a layout parameter); "
             f"--gpus {args.gpus} is not supported.")
