@@ -62,3 +62,11 @@ def mixed_values(gen: torch.Generator, n: int, dtype: torch.dtype, std: float = 
     if n > k + 64:
         x[k : k + 64] = torch.randn(64, generator=gen) * torch.logspace(-45, 38, 64)
     return x.to(dtype)
+
+
+def loc(t: torch.Tensor) -> torch.Tensor:
+    """The local 1-D fragment behind a sharded parameter / gradient (a ``RaggedShardDTensor``); plain tensors as
+    they are.  Detached, so that it can be compared and copied freely."""
+    from yafsdp_amd._tensor import local_tensor
+
+    return local_tensor(t.detach())

@@ -8,7 +8,7 @@ import pytest
 import torch
 import torch.nn as nn
 
-from helpers import assert_bits_equal
+from helpers import assert_bits_equal, loc
 from test_gpu_fully_shard import DEV, MP, _make
 
 pytestmark = pytest.mark.gpu
@@ -129,6 +129,61 @@ def test_full_state_dict_round_trip_through_the_unwrapped_model():
         full_state_dict(fresh)
 
 
+def test_dcp_through_module_state_dict_and_the_sharded_parameter_surface(tmp_path):
+    """model.state_dict() of a fully_shard model holds the sharded parameters themselves: torch.distributed.checkpoint
+    saves and loads them without any helper; p.to_local(), p.placements and p.full_tensor() are the reference's."""
+    import torch.distributed.checkpoint as dcp
+
+    from yafsdp_amd import RaggedShardDTensor, fully_shard
+    from yafsdp_amd.checkpoint import RaggedShardLoadPlanner, fsdp_groups_of
+
+    def wrap(m):
+        for b in m.blocks:
+            fully_shard(b, mp_policy=MP)
+        fully_shard(m.norm, mp_policy=MP)
+        return fully_shard(m, mp_policy=MP)
+
+    model0 = _make(33)
+    model = wrap(copy.deepcopy(model0))
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    x = torch.randn(8, 128, device=DEV)
+    for _ in range(2):
+        model(x).float().pow(2).mean().backward()
+        opt.step()
+        opt.zero_grad(set_to_none=True)
+    for (name, p), (_, p0) in zip(model.named_parameters(), model0.named_parameters()):
+        assert isinstance(p, RaggedShardDTensor) and p.shape == p0.shape
+        (placement,) = p.placements
+        assert (placement.local_numel, placement.global_offset, placement.shard_numels) == (p0.numel(), 0, (p0.numel(),))
+        with pytest.raises(NotImplementedError):
+            p.to_local()  # under autograd, as in the reference (ya_fsdp/_tensor.py:318-321)
+        with torch.no_grad():
+            local = p.to_local()
+        assert local.dim() == 1 and local.numel() == p0.numel()
+        full = p.full_tensor()
+        assert full.shape == p0.shape and full.data_ptr() != local.data_ptr()
+        assert_bits_equal(full.reshape(-1), local, name)
+    sd = model.state_dict()
+    assert all(isinstance(v, RaggedShardDTensor) for k, v in sd.items())
+    dcp.save(sd, checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    fresh = wrap(copy.deepcopy(model0))
+    fresh(x)
+    for m in (fresh.blocks[2], fresh.norm):
+        m.reshard()
+    dcp.load(fresh.state_dict(), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True, planner=RaggedShardLoadPlanner())
+    for g in fsdp_groups_of(fresh):
+        g._all_gather_input_set_dtypes.clear()
+    for ga, gb in zip(fsdp_groups_of(model), fsdp_groups_of(fresh)):
+        assert_bits_equal(gb._padded_sharded_param_data[None], ga._padded_sharded_param_data[None], "masters")
+    assert_bits_equal(fresh(x), model(x).detach(), "outputs after reload")
+    # an ordinary state dict of full tensors loads as well: every rank keeps its fragment
+    for m in (fresh.blocks[2], fresh.norm, model.blocks[2], model.norm):
+        m.reshard()
+    fresh.load_state_dict(model0.state_dict())
+    for g, (_, p0) in zip([fp for gr in fsdp_groups_of(fresh) for fp in gr.fsdp_params], model0.named_parameters()):
+        assert_bits_equal(g._sharded_param_data, p0.detach().reshape(-1), "loaded from full tensors")
+
+
 def test_full_state_dict_leaves_non_persistent_buffers_out():
     """Buffers registered with persistent=False (rotary tables and the like) are not part of module.state_dict();
     the full state dict follows it, so an ordinary state dict loads with strict=True."""
@@ -157,12 +212,13 @@ def test_full_state_dict_leaves_non_persistent_buffers_out():
 
 
 def test_torch_distributed_checkpoint_round_trip(tmp_path):
-    """A trained wrapped model saved with torch.distributed.checkpoint through RaggedShardTensor handles
-    (views of the flat master shards) and loaded into a freshly wrapped model and into plain flattened tensors."""
+    """A trained wrapped model saved with torch.distributed.checkpoint through its own sharded parameters
+    (RaggedShardDTensor: local fragments that are views of the flat master shards, and the checkpoint hooks of
+    ya_fsdp/_tensor.py:365-432) and loaded into a freshly wrapped model and into plain flattened tensors."""
     import torch.distributed.checkpoint as dcp
 
     from yafsdp_amd import fully_shard
-    from yafsdp_amd.checkpoint import checkpointable_state_dict, fsdp_groups_of
+    from yafsdp_amd.checkpoint import RaggedShardLoadPlanner, checkpointable_state_dict, fsdp_groups_of
 
     def wrap(m):
         for b in m.blocks:
@@ -186,21 +242,25 @@ def test_torch_distributed_checkpoint_round_trip(tmp_path):
         opt.zero_grad(set_to_none=True)
     sd = handles(model)
     assert set(sd) == {n for n, _ in model0.named_parameters()}
-    assert all(tuple(h.size()) == (p.numel(),) for h, p in ((sd[n], p) for n, p in model0.named_parameters()))
-    with pytest.raises(NotImplementedError, match="checkpoint handle"):
-        sd["norm.weight"] + 1
+    assert all(h.size() == p.size() and loc(h).numel() == p.numel() for h, p in ((sd[n], p) for n, p in model0.named_parameters()))
+    with pytest.raises(NotImplementedError, match="dispatch"):
+        sd["norm.weight"].sin()
     dcp.save(sd, checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
     # (a) plain flattened tensors
     flat = {n: torch.full((p.numel(),), float("nan"), device=DEV) for n, p in model0.named_parameters()}
     dcp.load(flat, checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
     for n, h in sd.items():
-        assert_bits_equal(flat[n], h.local_tensor, n)
+        assert_bits_equal(flat[n], loc(h), n)
     # (b) a freshly wrapped model: the load writes its flat master shards
     fresh = wrap(copy.deepcopy(model0))
     fresh(x)  # lazy init (then hand the buffers back, as after any forward without backward)
     for m in (fresh.blocks[2], fresh.norm):
         m.reshard()
-    dcp.load(handles(fresh), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    from torch.distributed.checkpoint.api import CheckpointException
+
+    with pytest.raises(CheckpointException, match="Size mismatch"):  # the default planner wants the flattened size
+        dcp.load(handles(fresh), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    dcp.load(handles(fresh), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True, planner=RaggedShardLoadPlanner())
     for g in fsdp_groups_of(fresh):
         g._all_gather_input_set_dtypes.clear()
     for ga, gb in zip(fsdp_groups_of(model), fsdp_groups_of(fresh)):

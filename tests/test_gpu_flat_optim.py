@@ -10,7 +10,7 @@ import torch.nn as nn
 
 from oracle import cref
 
-from helpers import assert_bits_equal
+from helpers import assert_bits_equal, loc
 from test_gpu_fully_shard import DEV, MP, Net, _make, _wrap
 
 pytestmark = pytest.mark.gpu
@@ -71,7 +71,8 @@ def test_flat_adamw_matches_the_oracle_and_prefills_the_all_gather_input():
         assert_bits_equal(unit.exp_avg_sq, mirror.v[i], "exp_avg_sq")
     # state views alias the flat moments
     p0 = groups[0].fsdp_params[0].sharded_param
-    assert opt.state[p0]["exp_avg"].data_ptr() == [u for u in opt._units[0] if u.group is groups[0]][0].exp_avg.data_ptr()
+    assert loc(opt.state[p0]["exp_avg"]).data_ptr() == [u for u in opt._units[0] if u.group is groups[0]][0].exp_avg.data_ptr()
+    assert opt.state[p0]["exp_avg"].shape == p0.shape  # shaped (and wrapped) like the sharded parameter
 
 
 def test_fused_copy_in_changes_nothing_downstream():
@@ -109,9 +110,9 @@ def test_clip_grad_norm_matches_the_oracle_and_torch():
         n_dev, c_dev = grad_clip_coef(model, max_norm)
         assert abs(n_dev.item() - norm) <= 6e-8 * norm and abs(c_dev.item() - coef) <= 1.2e-7 * coef
         # torch's own clipping on copies of the per-parameter gradients
-        tparams = [nn.Parameter(p.detach().clone()) for p in model.parameters()]
+        tparams = [nn.Parameter(loc(p).clone()) for p in model.parameters()]
         for tp, p in zip(tparams, model.parameters()):
-            tp.grad = p.grad.detach().clone()
+            tp.grad = loc(p.grad).clone()
         tnorm = torch.nn.utils.clip_grad_norm_(tparams, max_norm)
         got_norm = clip_grad_norm_(model, max_norm)
         assert abs(got_norm.item() - tnorm.item()) <= 2e-6 * tnorm.item()
@@ -121,7 +122,7 @@ def test_clip_grad_norm_matches_the_oracle_and_torch():
             cref.flat_scale(want, coef_used)
             assert_bits_equal(g._padded_sharded_param_grad[None], want, f"clipped grads max_norm={max_norm}")
         for tp, p in zip(tparams, model.parameters()):
-            torch.testing.assert_close(p.grad, tp.grad, rtol=3e-6, atol=0)
+            torch.testing.assert_close(loc(p.grad), tp.grad, rtol=3e-6, atol=0)
         grads = [g._padded_sharded_param_grad[None].detach().cpu().clone() for g in groups]
         total = sum(cref.sumsq(x) for x in grads)
     assert coef_used == 1.0  # nothing clipped at 1e9: gradients untouched
@@ -227,7 +228,7 @@ def test_zero_grad_and_stale_copy_guard():
     opt.step()
     zero_grad(model)
     for p in model.parameters():
-        assert p.grad is not None and float(p.grad.abs().max()) == 0.0
+        assert p.grad is not None and float(loc(p.grad).abs().max()) == 0.0
     # a torch op changes the masters after the fused step: the next forward must cast again
     g = _groups(model)[0]
     with torch.no_grad():
@@ -342,7 +343,7 @@ def test_training_with_fused_grad_norm_equals_training_without():
             opt.step(grad_scale=coef)
             opt.zero_grad(set_to_none=True)
         torch.cuda.synchronize()
-        return norms, [p.detach().clone() for p in model.parameters()]
+        return norms, [loc(p).clone() for p in model.parameters()]
 
     n1, p1 = run(True)
     n0, p0 = run(False)
@@ -366,7 +367,7 @@ def test_fused_grad_norm_falls_back_when_the_reduce_writes_the_shard_directly():
     norm_a, _ = grad_clip_coef(model, 1.0)
     disable_fused_grad_norm(model)
     norm_b, _ = grad_clip_coef(model, 1.0)
-    want = torch.sqrt(sum(p.grad.double().pow(2).sum() for p in model.parameters())).float()
+    want = torch.sqrt(sum(loc(p.grad).double().pow(2).sum() for p in model.parameters())).float()
     assert torch.allclose(norm_a, norm_b, rtol=2e-7, atol=0) and torch.allclose(norm_b, want, rtol=1e-6, atol=0)
 
 
@@ -402,7 +403,7 @@ def test_fused_grad_norm_small_group_with_a_frozen_parameter_in_the_middle():
     finally:
         disable_fused_grad_norm(model)
     norm_read, coef_read = grad_clip_coef(model, 1e-3)
-    want = torch.sqrt(sum(p.grad.double().pow(2).sum() for p in model.parameters() if p.grad is not None)).float()
+    want = torch.sqrt(sum(loc(p.grad).double().pow(2).sum() for p in model.parameters() if p.grad is not None)).float()
     assert float(norm_read) > 0 and torch.allclose(norm_read, want, rtol=1e-6, atol=0)
     assert torch.equal(norm_fused, norm_read) and torch.equal(norm_again, norm_read) and torch.equal(coef_fused, coef_read)
 

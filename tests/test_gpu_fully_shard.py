@@ -8,7 +8,9 @@ import pytest
 import torch
 import torch.nn as nn
 
+from helpers import loc
 from yafsdp_amd import MixedPrecisionPolicy, make_layout
+from yafsdp_amd._tensor import RaggedShardDTensor
 
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
@@ -97,10 +99,12 @@ def test_training_is_bit_identical_to_manual_mixed_precision():
     xs = [torch.randn(16, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(s)) for s in range(4)]
     ref = _reference_steps(model0, xs, lr=0.05)
     model = _wrap(copy.deepcopy(model0), mp_policy=MP)
-    # the optimizer sees one fp32 1-D shard per original parameter
+    # the optimizer sees one fp32 sharded parameter per original parameter: it stands for the whole parameter (its
+    # shape) and holds this rank's 1-D fragment of the flat master shard
     params = list(model.parameters())
-    assert all(p.dtype == torch.float32 and p.dim() == 1 for p in params)
-    assert sum(p.numel() for p in params) == sum(p.numel() for p in model0.parameters())
+    assert all(isinstance(p, RaggedShardDTensor) and p.dtype == torch.float32 and loc(p).dim() == 1 for p in params)
+    assert [p.shape for p in params] == [p.shape for p in model0.parameters()]
+    assert sum(loc(p).numel() for p in params) == sum(p.numel() for p in model0.parameters())
     opt = torch.optim.SGD(params, lr=0.05)
     for x in xs:
         y = model(x)
@@ -190,7 +194,7 @@ def test_module_api_and_states():
     handle.wait()
     assert blk.up.weight.dtype == torch.bfloat16 and blk.up.weight.shape == (256, 128)
     blk.reshard()
-    assert blk.up.weight.dtype == torch.float32 and blk.up.weight.dim() == 1
+    assert blk.up.weight.dtype == torch.float32 and isinstance(blk.up.weight, RaggedShardDTensor)
     # the last user of each data buffer keeps its parameters unsharded after forward
     model(x)
     groups = [m._get_fsdp_state()._fsdp_param_group for m in [*model.blocks, model.norm]]
@@ -242,8 +246,9 @@ def test_logical_world_size_gives_each_rank_its_ragged_shard():
         blk = copy.deepcopy(model0.blocks[0])
         fully_shard(blk, mesh=(w, r), mp_policy=MP)
         sharded = list(blk.parameters())
-        assert [p.numel() for p in sharded] == lay.sharded_numels(r)
-        pieces.append(torch.cat([p.detach() for p in sharded]))
+        assert [loc(p).numel() for p in sharded] == lay.sharded_numels(r)
+        assert [p.placements[0].global_offset for p in sharded] == lay.global_offsets(r)
+        pieces.append(torch.cat([loc(p) for p in sharded]))
     assert torch.equal(torch.cat(pieces), full)  # the ranks' fragments tile the flat parameter space
 
 
@@ -301,9 +306,9 @@ def test_state_dict_sees_sharded_parameters_even_when_unsharded():
     blk = model.blocks[2]
     assert blk.up.weight.dtype == torch.bfloat16 and blk.up.weight.dim() == 2
     sd = model.state_dict()
-    assert all(v.dtype == torch.float32 and v.dim() == 1 for v in sd.values())
+    assert all(v.dtype == torch.float32 and isinstance(v, RaggedShardDTensor) for v in sd.values())
     assert blk.up.weight.dtype == torch.float32  # swapped back by the hook
-    new = {k: torch.full_like(v, 0.25) for k, v in sd.items()}
+    new = {k: torch.zeros_like(v).fill_(0.25) for k, v in sd.items()}
     # the hook swaps the registered parameters only; the buffers are handed back by reshard(), as after any
     # forward without backward
     for m in (model.blocks[2], model.norm):
@@ -441,7 +446,7 @@ def test_custom_gradient_divide_factor():
         model(x).float().pow(2).mean().backward()
         plain(x).float().pow(2).mean().backward()
         for p, q in zip(model.parameters(), plain.parameters()):
-            assert torch.equal(p.grad * 4.0, q.grad)
+            assert torch.equal(loc(p.grad) * 4.0, loc(q.grad))
         opt.step(); opt_plain.step()
     torch.cuda.synchronize()
 
@@ -481,7 +486,7 @@ def test_frozen_and_tied_parameters():
     got = dict(model.named_parameters())  # world size 1: every sharded parameter is the whole flattened master
     assert set(got) == set(want)
     for k, v in want.items():
-        assert torch.equal(got[k].detach().view(v.shape).view(torch.int32), v.detach().view(torch.int32)), k
+        assert torch.equal(loc(got[k]).view(v.shape).view(torch.int32), v.detach().view(torch.int32)), k
 
 
 def test_ignored_parameters_stay_plain():
@@ -604,3 +609,41 @@ def test_meta_device_model_is_materialised_empty_and_trains_after_initialisation
     x = torch.randn(4, 128, device=DEV)
     want = copy.deepcopy(ref).to(torch.bfloat16)(x.to(torch.bfloat16))
     assert torch.equal(model(x), want)
+
+
+@pytest.mark.parametrize("impl", ["foreach", "fused"])
+def test_torch_adamw_and_clip_grad_norm_on_the_sharded_parameters(impl):
+    """torch's own optimizer (foreach and fused) and torch.nn.utils.clip_grad_norm_ reach the local fragments through
+    the sharded parameters' dispatch list (ya_fsdp/_tensor.py:122-316): the same calls on plain copies of the
+    fragments give the same bits."""
+    model = _wrap(_make(61), mp_policy=MP)
+    xs = [torch.randn(8, 128, device=DEV, generator=torch.Generator(device=DEV).manual_seed(300 + s)) for s in range(3)]
+    model(xs[0]).float().pow(2).mean().backward()  # lazy init
+    model.zero_grad(set_to_none=True)
+    params = list(model.parameters())
+    twins = [nn.Parameter(loc(p).clone()) for p in params]
+    opt = torch.optim.AdamW(params, lr=1e-3, weight_decay=0.1, **{impl: True})
+    topt = torch.optim.AdamW(twins, lr=1e-3, weight_decay=0.1, **{impl: True})
+    for x in xs:
+        (model(x).float().pow(2).mean() * 100.0).backward()
+        for t, p in zip(twins, params):
+            t.grad = loc(p.grad).clone()
+        norm = torch.nn.utils.clip_grad_norm_(params, 0.05, foreach=True)
+        tnorm = torch.nn.utils.clip_grad_norm_(twins, 0.05, foreach=True)
+        assert torch.equal(norm, tnorm) and float(norm) > 0.05
+        opt.step()
+        topt.step()
+        for t, p in zip(twins, params):
+            assert torch.equal(loc(p).view(torch.int32), t.detach().view(torch.int32))
+            assert torch.equal(loc(p.grad).view(torch.int32), t.grad.view(torch.int32))
+        opt.zero_grad(set_to_none=True)
+        topt.zero_grad(set_to_none=True)
+    st = opt.state[params[0]]
+    assert isinstance(st["exp_avg"], RaggedShardDTensor) and st["exp_avg"].shape == params[0].shape
+    # the next forward sees the updated masters (torch's step went through the version counter of the flat shard)
+    y = model(xs[0])
+    twin_model = _make(61)
+    with torch.no_grad():
+        for q, t in zip(twin_model.parameters(), twins):
+            q.copy_(t.view(q.shape))
+    assert torch.equal(y, twin_model.to(torch.bfloat16)(xs[0].to(torch.bfloat16)))

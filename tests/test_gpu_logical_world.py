@@ -19,6 +19,9 @@ import copy
 import pytest
 import torch
 
+from helpers import loc
+from yafsdp_amd import connect_logical_ranks
+
 from yafsdp_amd import _native, fully_shard
 from yafsdp_amd.checkpoint import full_tensors
 
@@ -109,7 +112,7 @@ def test_logical_ranks_train_like_one_unsharded_model(w, alignment):
         model._get_fsdp_state()._lazy_init(allow_no_grad_reduce=True)  # one reduce buffer per group
         model.set_requires_gradient_sync(False)                        # gradients stay unreduced in it
     # every rank's shards together are the model: some parameter is split between ranks
-    sizes = [[p.numel() for p in model.parameters()] for model in ranks]
+    sizes = [[loc(p).numel() for p in model.parameters()] for model in ranks]
     assert any(0 < a < b for a, b in zip(sizes[0], [p.numel() for p in model0.parameters()]))
     for xs in batches:
         _all_gather(ranks)
@@ -127,3 +130,14 @@ def test_logical_ranks_train_like_one_unsharded_model(w, alignment):
     assert set(got) == set(want)
     for k, v in want.items():
         assert torch.equal(got[k].view(torch.int32), v.detach().view(torch.int32)), k
+    # the same through the sharded parameters themselves: once the logical ranks know each other, full_tensor() of
+    # any rank's parameter assembles the whole parameter from all ranks' fragments (ya_fsdp/_tensor.py:341-363)
+    with pytest.raises(RuntimeError, match="connect_logical_ranks"):
+        next(p for p in ranks[0].parameters() if 0 < loc(p).numel() < p.numel()).full_tensor()
+    connect_logical_ranks(ranks)
+    for r in (0, w - 1):
+        for k, p in ranks[r].named_parameters():
+            assert p.placements[0].shard_numels == tuple(loc(q).numel() for q in
+                                                          (dict(m.named_parameters())[k] for m in ranks))
+            full = p.full_tensor()
+            assert full.shape == want[k].shape and torch.equal(full.view(torch.int32), want[k].detach().view(torch.int32)), k

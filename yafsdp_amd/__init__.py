@@ -31,6 +31,8 @@ __all__ = [
     "fully_shard",
     "YaFSDPModule",
     "UnshardHandle",
+    "RaggedShardDTensor",
+    "connect_logical_ranks",
 ]
 
 _LAZY = {
@@ -44,6 +46,8 @@ _LAZY = {
     "fully_shard": "fully_shard",
     "YaFSDPModule": "fully_shard",
     "UnshardHandle": "fully_shard",
+    "RaggedShardDTensor": "_tensor",
+    "connect_logical_ranks": "_tensor",
 }
 
 

@@ -1,6 +1,8 @@
 """Per-parameter bookkeeping of a parameter group: every tensor here is a VIEW
 into one of the group's flat buffers (mirror of ya_fsdp/_param.py, restricted to
-what the buffer path touches: no DTensor wrapping, no module attribute swaps).
+what the buffer path touches).  The sharded parameter and its gradient are
+``RaggedShardDTensor`` wrappers around 1-D views of the flat master / gradient
+shard (ya_fsdp/_param.py:142-151).
 """
 
 from __future__ import annotations
@@ -14,6 +16,7 @@ import torch.nn as nn
 from ._api import MixedPrecisionPolicy
 from ._common import FSDPMeshInfo, ShardedState
 from ._layout import RaggedShard
+from ._tensor import RaggedShardDTensor, RaggedShardSpec, TensorMeta, local_tensor
 
 
 @dataclass
@@ -84,11 +87,35 @@ class YaFSDPParam:
         )
         self.sharded_numel = sharded_param_data.numel()
         self._sharded_param_data = sharded_param_data
-        self.sharded_param = nn.Parameter(sharded_param_data, requires_grad=self.requires_grad)
+        self._sharding_spec = RaggedShardSpec(  # :136-140 with the logical mesh in the DeviceMesh's place
+            self.mesh_info, (self.placement,), TensorMeta(self._orig_size, self.param.stride(), self.param.dtype),
+            weakref.ref(self), "param",
+        )
+        self.sharded_param = nn.Parameter(self.to_sharded_dtensor(sharded_param_data), requires_grad=self.requires_grad)
         self.sharded_param._yafsdp_param = weakref.ref(self)  # lets flat-shard optimizers find the owner
-        self.sharded_param_grad = sharded_param_grad if self.requires_grad else None
+        if self.requires_grad:
+            assert sharded_param_grad is not None
+            self.sharded_param_grad = self.to_sharded_dtensor(sharded_param_grad, "grad")
+        else:
+            self.sharded_param_grad = None
         del self.param, self.param_data  # the group's flat shard now owns the values
         self._setattr_on_modules(self.sharded_param)
+
+    def to_sharded_dtensor(self, tensor: torch.Tensor, kind: str = "param") -> RaggedShardDTensor:
+        """ya_fsdp/_param.py:298-310: wrap a local 1-D fragment of this parameter (same length as the sharded
+        parameter's) with the parameter's sharding spec."""
+        if tensor.shape != self._sharded_param_data.shape:
+            raise AssertionError(f"Expects size {self._sharded_param_data.shape} but got {tensor.shape}")
+        spec = self._sharding_spec
+        if kind != spec.kind or tensor.dtype != spec.tensor_meta.dtype:
+            spec = RaggedShardSpec(spec.mesh, spec.placements,
+                                   TensorMeta(spec.tensor_meta.shape, spec.tensor_meta.stride, tensor.dtype), spec.owner, kind)
+        return RaggedShardDTensor(tensor, spec, requires_grad=False)
+
+    @property
+    def _sharded_local_tensor(self) -> torch.Tensor:
+        """ya_fsdp/_param.py:312-314."""
+        return self.sharded_param._local_tensor
 
     def init_all_gather_input(self, all_gather_input: torch.Tensor) -> None:
         self._all_gather_input = all_gather_input
@@ -138,15 +165,18 @@ class YaFSDPParam:
         if info is None:
             return
         new_param = getattr(info.module, info.param_name)
-        if new_param.data_ptr() != self._sharded_param_data.data_ptr() and self.sharded_numel > 0:
+        new_local = local_tensor(new_param.detach())
+        if new_local.data_ptr() != self._sharded_param_data.data_ptr() and self.sharded_numel > 0:
             from . import _native
 
-            if new_param.device != self._sharded_param_data.device or new_param.numel() != self.sharded_numel:
+            if new_local.device != self._sharded_param_data.device or new_local.numel() != self.sharded_numel:
                 raise NotImplementedError(
                     "moving a sharded module to another device or changing its parameter sizes is not supported"
                 )
-            _native.flat_copy(self._sharded_param_data, new_param.detach().contiguous().view(-1))
-        self.sharded_param = nn.Parameter(self._sharded_param_data, requires_grad=self.sharded_param.requires_grad)
+            _native.flat_copy(self._sharded_param_data, new_local.contiguous().view(-1))
+        self.sharded_param = nn.Parameter(
+            self.to_sharded_dtensor(self._sharded_param_data), requires_grad=self.sharded_param.requires_grad
+        )
         self.sharded_param._yafsdp_param = weakref.ref(self)
         self._setattr_on_modules(self.sharded_param)
 

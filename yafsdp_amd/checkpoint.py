@@ -33,7 +33,8 @@ from ._layout import RaggedShard
 from ._param_group import YaFSDPParamGroup
 
 __all__ = ["ChunkMeta", "chunk_meta", "sharded_state_dict", "group_meta_info", "full_tensors", "load_full_tensors",
-           "full_state_dict", "load_full_state_dict", "RaggedShardTensor", "checkpointable_state_dict"]
+           "full_state_dict", "load_full_state_dict", "RaggedShardTensor", "checkpointable_state_dict",
+           "RaggedShardLoadPlanner"]
 
 
 @dataclass(frozen=True)
@@ -146,11 +147,55 @@ class RaggedShardTensor(torch.Tensor):
         return self._local()
 
 
-def checkpointable_state_dict(group: YaFSDPParamGroup) -> dict[str, RaggedShardTensor]:
-    """``{fqn: RaggedShardTensor}`` of one parameter group on this rank, for
-    ``torch.distributed.checkpoint.save`` / ``load`` (views of the flat master
-    shard: no copy)."""
-    return {fqn: RaggedShardTensor.wrap(local, meta) for fqn, (local, meta) in sharded_state_dict(group).items()}
+def checkpointable_state_dict(group: YaFSDPParamGroup) -> dict[str, torch.Tensor]:
+    """``{fqn: sharded parameter}`` of one parameter group on this rank, for
+    ``torch.distributed.checkpoint.save`` / ``load``: the group's own
+    ``RaggedShardDTensor`` parameters (detached; their local fragments are views
+    of the flat master shard, so nothing is copied), which carry the checkpoint
+    hooks themselves.  ``module.state_dict()`` of a ``fully_shard`` module holds
+    the same tensors under the module's own names."""
+    return {fsdp_param._param_fqn: fsdp_param.sharded_param.detach() for fsdp_param in group.fsdp_params}
+
+
+class _FlattenedView:
+    """What the load planner looks at in place of a sharded parameter: the flattened size the chunk format
+    declares, and the parameter's own chunk list."""
+
+    def __init__(self, tensor: torch.Tensor):
+        self._tensor = tensor
+
+    def size(self) -> torch.Size:
+        return torch.Size((self._tensor.numel(),))
+
+    def __create_chunk_list__(self):
+        return self._tensor.__create_chunk_list__()
+
+
+def _load_planner_base():
+    from torch.distributed.checkpoint.default_planner import DefaultLoadPlanner
+
+    return DefaultLoadPlanner
+
+
+class RaggedShardLoadPlanner(_load_planner_base()):  # type: ignore[misc]
+    """``torch.distributed.checkpoint.load(module.state_dict(), ..., planner=RaggedShardLoadPlanner())``.
+
+    The chunk format of a ragged shard (ya_fsdp/_tensor.py:365-423) declares the parameter FLATTENED:
+    ``size = (numel,)`` with 1-D offsets and lengths, while the sharded parameter itself reports the parameter's
+    original shape.  The default load planner of the installed torch compares the two sizes before it plans
+    anything and refuses; this planner shows it the flattened size for ``RaggedShardDTensor`` values and leaves
+    everything else to the default (saving needs no planner).  Loaded values land in the local fragments, i.e.
+    in the flat master shards."""
+
+    def create_local_plan(self):
+        from ._tensor import RaggedShardDTensor
+
+        real = self.state_dict
+        self.state_dict = {k: _FlattenedView(v) if isinstance(v, RaggedShardDTensor) else v for k, v in real.items()}
+        try:
+            return super().create_local_plan()
+        finally:
+            self.state_dict = real
 
 
 def group_meta_info(group: YaFSDPParamGroup) -> dict[str, list]:

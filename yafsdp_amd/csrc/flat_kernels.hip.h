@@ -15,6 +15,7 @@
 // element-aligned address.
 #pragma once
 #include "elem.hip.h"
+#include "tuning.h"
 
 namespace yafsdp {
 
@@ -96,6 +97,7 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
+  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   const int tid = threadIdx.x;
   const int64_t n_units = (n - head) >> 3;
   const int64_t body_end = head + (n_units << 3);

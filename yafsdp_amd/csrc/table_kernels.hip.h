@@ -269,6 +269,7 @@ __device__ __forceinline__ int tile_of_block(int b) {
 template <class META, class S, class D, int SCALE, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero) {
+  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   char* fbase = reinterpret_cast<char*>(flat);
@@ -370,6 +371,7 @@ __device__ __forceinline__ void scatter_segment(char* dst, const char* src, int6
 template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
+  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   constexpr int64_t kLineElems = 128 / D::kSize;

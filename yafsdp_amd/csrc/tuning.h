@@ -10,6 +10,11 @@ namespace yafsdp {
 #ifndef YAFSDP_FLAT_U
 #define YAFSDP_FLAT_U 1
 #endif
+// issue priority the copy kernels' waves ask for (s_setprio, 0..3; 0 leaves the default)
+#ifndef YAFSDP_WAVE_PRIO
+#define YAFSDP_WAVE_PRIO 0
+#endif
+constexpr int kWavePrio = YAFSDP_WAVE_PRIO;
 // store policy of whole tiles: 0 ordinary, 1 non-temporal, 2 write-through (see TileStore)
 #ifndef YAFSDP_FLAT_STP
 #define YAFSDP_FLAT_STP 2

@@ -31,6 +31,7 @@ import torch.nn as nn
 from . import _native
 from ._param import YaFSDPParam
 from ._param_group import YaFSDPParamGroup
+from ._tensor import local_tensor
 from ._state import _get_module_fsdp_state
 
 __all__ = ["FlatAdamW", "clip_grad_norm_", "grad_clip_coef", "zero_grad", "fsdp_param_groups",
@@ -94,8 +95,9 @@ def _grad_ranges(group: YaFSDPParamGroup, indices: Sequence[int] | None = None) 
                 complete = False
             continue
         view = fsdp_param.sharded_param_grad
-        if grad.numel() and grad.data_ptr() != view.data_ptr():
-            _native.flat_copy(view, grad.detach().reshape(-1))
+        grad_local, view_local = local_tensor(grad.detach()), view._local_tensor
+        if grad_local.numel() and grad_local.data_ptr() != view_local.data_ptr():
+            _native.flat_copy(view_local, grad_local.reshape(-1))
             fsdp_param.sharded_param.grad = view
         ranges.append((offsets[i], offsets[i + 1]))
     merged = _merge(ranges)
@@ -278,6 +280,14 @@ class _Unit:
         self.exp_avg_sq = torch.zeros(self.numel, dtype=torch.float32, device=self.device)
         self.steps = [0] * len(params)
 
+    def state_view(self, k: int, flat: torch.Tensor) -> torch.Tensor:
+        """A range of a flat moment buffer as the optimizer state of parameter k: shaped like the parameter, i.e.
+        wrapped like the sharded parameter itself (what ``torch.zeros_like(p)`` gives torch's own optimizers)."""
+        p = self.params[k]
+        if self.group is None:
+            return flat.view(p.shape)
+        return self.group.fsdp_params[self.indices[k]].to_sharded_dtensor(flat, kind="")
+
     def fragment(self, k: int) -> tuple[int, int]:
         if self.group is None:
             return 0, self.numel
@@ -350,8 +360,8 @@ class FlatAdamW(torch.optim.Optimizer):
                 lo, hi = unit.fragment(k)
                 st = self.state[p]
                 st["step"] = torch.tensor(0.0)
-                st["exp_avg"] = unit.exp_avg[lo:hi].view(p.shape)
-                st["exp_avg_sq"] = unit.exp_avg_sq[lo:hi].view(p.shape)
+                st["exp_avg"] = unit.state_view(k, unit.exp_avg[lo:hi])
+                st["exp_avg_sq"] = unit.state_view(k, unit.exp_avg_sq[lo:hi])
         self._units[key] = units
         return units
 
@@ -454,7 +464,8 @@ class FlatAdamW(torch.optim.Optimizer):
                         continue
                     unit.steps[k] = int(float(st.get("step", 0)))
                     for name in ("exp_avg", "exp_avg_sq"):
-                        if name in st and st[name].numel():
-                            _native.flat_copy(self.state[p][name].view(-1),
-                                              st[name].to(p.device, torch.float32).contiguous().view(-1))
+                        src = local_tensor(st[name]) if name in st else None
+                        if src is not None and src.numel():
+                            _native.flat_copy(local_tensor(self.state[p][name]).view(-1),
+                                              src.to(p.device, torch.float32).contiguous().view(-1))
                     self.state[p]["step"] = torch.tensor(float(unit.steps[k]))
