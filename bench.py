@@ -56,13 +56,13 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 
 # HBM bytes per launch of the dominant kernel (gather_in_kernel), from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
-# (factors 1.99988 and 0.99986): (213037.875 * 1.99988 + 426022.75 * 0.99986) KiB.
+# (factors 1.99990 and 1.00000): (213040.75 * 1.99990 + 426103.375 * 1.00000) KiB.
 # Summary and commands: profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.  None = not measured.
 # "llama3-8b-layer-w8-optim": adamw_kernel, (213045.6 * 1.99946 + 372753.5 * 0.99996) KiB, scaled by the plain
 # fp32 copy of the same run; profiles/bench_llama3-8b-layer-w8-optim_hbm_traffic.md.
 # "ragged-stress-w256": gather_in_kernel<LargeMeta>, (379903.9 * 1.99992 + 710944.2 * 0.99984) KiB;
 # profiles/bench_ragged-stress-w256_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_461_600, "llama3-8b-layer-w8-optim": 817_885_000,
+MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872615800, "llama3-8b-layer-w8-optim": 817_885_000,
                           "ragged-stress-w256": 1_505_902_865}
 
 
@@ -463,6 +463,155 @@ def run_full_model(args) -> int:
         "kernels": kernels,
     }
     print(json.dumps(out), flush=True)
+    return 0
+
+
+def run_timeline(args) -> int:
+    """Where the time of the short kernels goes, and what other stream plans would give (headline workload).
+
+    (1) Per-workgroup timeline of copy-in, post-reduce (copy form) and post-reduce (accumulate) on one rank's shard
+    of the Llama-3-8B layer: every workgroup records the GPU's 100 MHz wall clock at its start and after its last
+    store has been acknowledged; the dispatch itself is timed with HIP events attached to it.  Reported per kernel:
+    dispatch time, time from the first workgroup's start to the last one's end, the rest (before the first wave and
+    after the last), time until the first workgroup completes, workgroup life, the plateau rate (workgroups ending
+    in the middle half of the span) and the time the launch loses against running at that rate from start to end.
+    (2) The step of the headline workload on one stream, with the reference's stream plan (copy-in, copy-out and
+    post-reduce on a side stream, reduce copy-in on the compute stream, ya_fsdp/_collectives.py:46, 110-111,
+    ya_fsdp/_param_group.py:669), and as two independent chains on two streams."""
+    import torch
+
+    from yafsdp_amd import _native
+    from yafsdp_amd._layout import make_layout
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    shapes, w, r, align, seed = WORKLOADS["llama3-8b-layer-w8"]
+    numels = [numel_of(s_) for s_ in shapes]
+    lay = make_layout(numels, w, align)
+    t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
+    gen = torch.Generator(device=dev).manual_seed(seed)
+
+    def randn(n, std, dtype):
+        out = torch.empty(n, dtype=dtype, device=dev)
+        for i in range(0, n, 1 << 26):
+            m = min(1 << 26, n - i)
+            out[i : i + m] = (torch.randn(m, device=dev, generator=gen) * std).to(dtype)
+        return out
+
+    master = randn(s, 0.02, torch.float32)
+    ag_in = torch.zeros(s, dtype=torch.bfloat16, device=dev)
+    gathered = randn(t_pad, 0.02, torch.bfloat16)
+    grads = [randn(n, 1e-3, torch.bfloat16) for n in numels]
+    outs = [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels]
+    rs = torch.zeros(t_pad, dtype=torch.bfloat16, device=dev)
+    shard, shard_b = randn(s, 1e-4, torch.float32), torch.empty(s, dtype=torch.float32, device=dev)
+    chunk = rs[r * s : (r + 1) * s]
+    table = _native.TensorTable(numels, t_pad, dev)
+    out_binding = table.bind(outs)
+
+    def op_copy_in():
+        _native.flat_copy(ag_in, master)
+
+    def op_copy_out():
+        out_binding.scatter_out(gathered)
+
+    def op_reduce_copy_in():
+        table.gather_in(grads, rs, None, float(w), True)
+
+    def op_post_reduce():
+        _native.post_reduce(shard, chunk, None, True)
+
+    op_reduce_copy_in()
+    torch.cuda.synchronize()
+    tile_elems = 256 * 8  # elements per workgroup of the flat kernels (256 lanes x one 8-element unit)
+    timeline = {}
+    for name, fn, bytes_per_elem in (("copy_in", op_copy_in, 6), ("post_reduce_copy", lambda: _native.post_reduce(shard_b, chunk, None, False), 6),
+                                     ("post_reduce", op_post_reduce, 10)):
+        recs = []
+        for _ in range(7):
+            op_copy_out()           # 1.7 GB of other traffic in front, as in a step
+            op_reduce_copy_in()
+            ev = _event_pair()
+            with _native.FlatLaunchTrace(1 << 16, dev) as tr:
+                _native.time_next_launch(*ev)
+                fn()
+            torch.cuda.synchronize()
+            tm = tr.times().double() * 0.01  # microseconds
+            first, last = float(tm[:, 0].min()), float(tm[:, 1].max())
+            span = last - first
+            ends = tm[:, 1] - first
+            life = (tm[:, 1] - tm[:, 0]).sort().values
+            mid = ((ends >= 0.25 * span) & (ends < 0.75 * span)).sum().item()
+            wg_bytes = tile_elems * bytes_per_elem
+            plateau = mid * wg_bytes / (0.5 * span) / 1e3  # GB/s
+            total_bytes = tm.shape[0] * wg_bytes
+            bins = torch.histc(ends.float(), bins=int(span) + 1, min=0.0, max=float(int(span) + 1))
+            recs.append({
+                "dispatch_us": ev[0].elapsed_time(ev[1]) * 1e3, "first_start_to_last_end_us": span,
+                "first_completion_us": float(ends.min()), "last_start_us": float(tm[:, 0].max()) - first,
+                "workgroup_life_us_median": float(life[len(life) // 2]), "workgroup_life_us_p90": float(life[len(life) * 9 // 10]),
+                "plateau_GBps": plateau, "lost_against_plateau_us": span - total_bytes / plateau / 1e3,
+                "GBps_of_workgroups_ending_per_us": [round(float(b) * wg_bytes / 1e3) for b in bins],
+                "workgroups": tm.shape[0],
+            })
+        recs.sort(key=lambda d: d["dispatch_us"])
+        med = recs[len(recs) // 2]
+        med["outside_first_start_to_last_end_us"] = med["dispatch_us"] - med["first_start_to_last_end_us"]
+        med["bytes"] = med["workgroups"] * tile_elems * bytes_per_elem
+        med["GBps_dispatch"] = med["bytes"] / med["dispatch_us"] / 1e3
+        timeline[name] = {k: (round(v, 2) if isinstance(v, float) else v) for k, v in med.items()}
+        log(f"  {name:17s} dispatch {med['dispatch_us']:.2f} us = span {med['first_start_to_last_end_us']:.2f} + "
+            f"{med['outside_first_start_to_last_end_us']:.2f} outside; first completion after {med['first_completion_us']:.2f} us, "
+            f"plateau {med['plateau_GBps']:.0f} GB/s, {med['lost_against_plateau_us']:.2f} us lost against it")
+
+    # ---- stream plans for the whole step
+    main, side = torch.cuda.current_stream(dev), torch.cuda.Stream(device=dev)
+    bytes_per_step = s * 6 + 4 * t + (4 * t + 2 * (t_pad - t)) + s * 10
+
+    def one_stream():
+        op_copy_in(); op_copy_out(); op_reduce_copy_in(); op_post_reduce()
+
+    def reference_plan():
+        with torch.cuda.stream(side):      # all-gather side: copy-in, copy-out
+            op_copy_in(); op_copy_out()
+        op_reduce_copy_in()                # compute stream
+        done = main.record_event()
+        with torch.cuda.stream(side):      # reduce-scatter side: after the compute stream
+            side.wait_event(done)
+            op_post_reduce()
+
+    def two_chains():
+        with torch.cuda.stream(side):
+            op_copy_in(); op_copy_out()
+        op_reduce_copy_in(); op_post_reduce()
+
+    plans = {}
+    for name, fn in (("one_stream", one_stream), ("reference_stream_plan", reference_plan), ("two_chains_two_streams", two_chains)):
+        side.wait_stream(main)
+        for _ in range(args.warmup):
+            fn()
+        main.wait_stream(side)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        main.wait_stream(side)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        plans[name] = {"ms_per_step": round(dt * 1e3, 4), "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s",
+                       "frac_of_hbm_peak": round(bytes_per_step / dt / 1e9 / HBM_PEAK_GBS, 4)}
+        log(f"  {name:24s} {plans[name]['ms_per_step']} ms per step, {plans[name]['value']} GB/s")
+    out = {
+        "metric": "launch timeline of the short flat kernels and stream plans of the step, Llama-3-8B layer @W=8",
+        "value": plans["one_stream"]["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": plans["one_stream"]["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "launch-timeline", "shard_numel": s, "padded_numel": t_pad, "logical_world_size": w},
+        "timeline": timeline, "stream_plans": plans,
+    }
+    print(json.dumps(out), flush=True)
+    out_binding.close()
+    table.close()
     return 0
 
 
@@ -1125,7 +1274,7 @@ def main() -> int:
     ap.add_argument("--workload", default="llama3-8b-layer-w8",
                     choices=sorted(WORKLOADS) + ["llama3-8b-full-w8", "ragged-stress-w256", "ragged-stress-w256-bf16-masters",
                                                  "llama3-8b-layer-w8-optim",
-                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange", "hbm-ceilings",
+                                                 "llama3-70b-layer-w64-optim", "llama3-8b-layer-w8-exchange", "hbm-ceilings", "launch-timeline",
                                                  "fully-shard-trainer-w1"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
@@ -1178,6 +1327,8 @@ def main() -> int:
         return run_exchange(args)
     if args.workload == "hbm-ceilings":
         return run_ceilings(args)
+    if args.workload == "launch-timeline":
+        return run_timeline(args)
     if args.workload == "fully-shard-trainer-w1":
         return run_trainer(args)
     try:

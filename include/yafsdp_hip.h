@@ -310,6 +310,14 @@ int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_
  * launch several kernels); NULL, NULL disarms. */
 int yafsdp_time_next_launch(void* start_event, void* stop_event);
 
+/* Measurement hook: per-workgroup timeline of the next kernel that this thread launches through
+ * yafsdp_flat_copy / yafsdp_flat_div / yafsdp_flat_div_copy / yafsdp_post_reduce.  Workgroup b of that launch
+ * stores the GPU's 100 MHz wall-clock count at its start into trace[2 b] and, once its loads have arrived and its
+ * stores are acknowledged, at its end into trace[2 b + 1] (`trace`: device memory for 2 * capacity 64-bit
+ * counts).  *n_workgroups (host memory, may be NULL) receives the grid size when the launch is made, or minus the
+ * grid size if it exceeded `capacity` (then nothing is traced).  Consumed by one launch; NULL disarms. */
+int yafsdp_trace_next_flat_launch(uint64_t* trace, int64_t capacity, int64_t* n_workgroups);
+
 /* Launch-shape knobs (process-wide, for measurement): */
 typedef enum yafsdp_option {
   YAFSDP_OPT_FLAT_BLOCKS_PER_CU = 0,  /* workgroups per compute unit of the flat kernels' grid */

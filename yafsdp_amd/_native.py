@@ -68,6 +68,7 @@ EXPORTED_SYMBOLS = (
     "yafsdp_flat_scale",
     "yafsdp_adamw_step",
     "yafsdp_time_next_launch",
+    "yafsdp_trace_next_flat_launch",
     "yafsdp_set_option",
     "yafsdp_get_option",
 )
@@ -145,6 +146,8 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_adamw_step.argtypes = [vp, vp, vp, vp, vp, i32, i64, dbl, dbl, dbl, dbl, dbl, i64, vp, i32, vp]
     lib.yafsdp_time_next_launch.restype = i32
     lib.yafsdp_time_next_launch.argtypes = [vp, vp]
+    lib.yafsdp_trace_next_flat_launch.restype = i32
+    lib.yafsdp_trace_next_flat_launch.argtypes = [vp, i64, ctypes.POINTER(i64)]
     lib.yafsdp_set_option.restype = i32
     lib.yafsdp_set_option.argtypes = [i32, i32]
     lib.yafsdp_get_option.restype = i32
@@ -755,6 +758,30 @@ def time_next_launch(start: torch.cuda.Event | None, stop: torch.cuda.Event | No
         if not ev.cuda_event:  # torch creates the HIP event lazily, on its first record
             ev.record()
     _check(lib.yafsdp_time_next_launch(start.cuda_event, stop.cuda_event), "yafsdp_time_next_launch")
+
+
+class FlatLaunchTrace:
+    """Per-workgroup timeline of one flat-kernel launch: ``with FlatLaunchTrace(capacity, device) as tr: <one flat
+    call>``; afterwards (and after a synchronize) ``tr.times()`` is an ``(n_workgroups, 2)`` int64 tensor of start /
+    end counts of the GPU's 100 MHz wall clock."""
+
+    def __init__(self, capacity: int, device: torch.device):
+        self.buf = torch.zeros(2 * capacity, dtype=torch.int64, device=device)
+        self.capacity = int(capacity)
+        self._n = ctypes.c_int64(0)
+
+    def __enter__(self) -> "FlatLaunchTrace":
+        _check(lib.yafsdp_trace_next_flat_launch(self.buf.data_ptr(), self.capacity, ctypes.byref(self._n)),
+               "yafsdp_trace_next_flat_launch")
+        return self
+
+    def __exit__(self, *exc) -> None:
+        lib.yafsdp_trace_next_flat_launch(None, 0, None)
+
+    def times(self) -> torch.Tensor:
+        if self._n.value <= 0:
+            raise RuntimeError(f"no flat launch was traced (grid {-self._n.value} against capacity {self.capacity})")
+        return self.buf[: 2 * self._n.value].view(-1, 2).cpu()
 
 
 def set_option(option: int, value: int) -> None:

@@ -422,6 +422,21 @@ int yafsdp_time_next_launch(void* start_event, void* stop_event) {
   return YAFSDP_OK;
 }
 
+int yafsdp_trace_next_flat_launch(uint64_t* trace, int64_t capacity, int64_t* n_workgroups) {
+  if (trace == nullptr) {  // disarm
+    tl_timed_launch.trace = nullptr;
+    tl_timed_launch.trace_capacity = 0;
+    tl_timed_launch.trace_workgroups = nullptr;
+    return YAFSDP_OK;
+  }
+  if (capacity < 1 || !aligned_to(trace, 8)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  tl_timed_launch.trace = reinterpret_cast<unsigned long long*>(trace);
+  tl_timed_launch.trace_capacity = capacity;
+  tl_timed_launch.trace_workgroups = n_workgroups;
+  if (n_workgroups != nullptr) *n_workgroups = 0;
+  return YAFSDP_OK;
+}
+
 int yafsdp_set_option(int option, int value) {
   if (option == YAFSDP_OPT_TABLE_LARGE_LOG2) {
     if (value < 0 || value > 62) return YAFSDP_ERR_INVALID_ARGUMENT;

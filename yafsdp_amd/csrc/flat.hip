@@ -7,8 +7,22 @@ namespace {
 
 template <class S, class D, int SCALE, bool ACC>
 hipError_t go(void* dst, const void* src, int64_t n, int head, float k, int grid, hipStream_t stream) {
+  // an armed timeline buffer is consumed by this launch if it is large enough for the grid
+  TimedLaunch& t = tl_timed_launch;
+  unsigned long long* trace = nullptr;
+  if (t.trace != nullptr) {
+    if (int64_t(grid) <= t.trace_capacity) {
+      trace = t.trace;
+      if (t.trace_workgroups != nullptr) *t.trace_workgroups = grid;
+    } else if (t.trace_workgroups != nullptr) {
+      *t.trace_workgroups = -int64_t(grid);  // not traced: the buffer is too small for this many workgroups
+    }
+    t.trace = nullptr;
+    t.trace_capacity = 0;
+    t.trace_workgroups = nullptr;
+  }
   return launch_kernel(flat_kernel<S, D, SCALE, ACC, kFlatBlock, kFlatUnroll, kFlatNtLoad, kFlatStorePolicy>, grid,
-                       kFlatBlock, stream, dst, src, n, head, k);
+                       kFlatBlock, stream, dst, src, n, head, k, trace);
 }
 
 template <class S, class D>

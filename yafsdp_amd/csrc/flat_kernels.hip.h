@@ -94,11 +94,16 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
 
 // dst[i] = op(src[i], dst[i]) for i in [0, n).  `head` leading elements bring
 // dst to a 16-byte boundary.  dst == src is allowed (in-place divide).
+// `trace` (normally null) is a measurement hook: workgroup b stores the 100 MHz
+// wall-clock count at its start and, after its stores have been acknowledged,
+// at its end into trace[2 b], trace[2 b + 1].
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
-flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
+flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned long long* trace) {
   if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   const int tid = threadIdx.x;
+  unsigned long long t_start = 0;
+  if (trace != nullptr) t_start = wall_clock64();
   const int64_t n_units = (n - head) >> 3;
   const int64_t body_end = head + (n_units << 3);
   if (blockIdx.x == 0) {
@@ -122,6 +127,13 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k) {
         if constexpr (ACC) d = load_unit<D, NTL>(dbase + u * (8 * D::kSize));
         store_unit<D, STP == ST_NT>(dbase + u * (8 * D::kSize), flat_unit<S, D, SCALE, ACC>(s, d, k));
       }
+    }
+  }
+  if (trace != nullptr) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every load has arrived, every store is acknowledged
+    if (tid == 0) {
+      trace[2 * blockIdx.x] = t_start;
+      trace[2 * blockIdx.x + 1] = wall_clock64();
     }
   }
 }

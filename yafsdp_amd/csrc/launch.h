@@ -15,6 +15,11 @@ namespace yafsdp {
 // kernel's own begin and end timestamps (no launch gap in between).
 struct TimedLaunch {
   hipEvent_t start = nullptr, stop = nullptr;
+  // per-workgroup timeline of the next flat kernel (yafsdp_trace_next_flat_launch): device buffer of 2 * capacity
+  // counts, and where to report the number of workgroups that wrote into it
+  unsigned long long* trace = nullptr;
+  int64_t trace_capacity = 0;
+  int64_t* trace_workgroups = nullptr;
 };
 extern thread_local TimedLaunch tl_timed_launch;
 

@@ -69,7 +69,7 @@ namespace {
 template <class O, bool ZERO_GRAD>
 hipError_t adamw_go(float* p, float* g, float* m, float* v, void* out16, int64_t n, int head, const AdamScalars& s,
                     const float* grad_scale, int grid, hipStream_t stream) {
-  return launch_kernel(adamw_kernel<O, ZERO_GRAD, kAdamBlock, kAdamUnroll, kOptNtLoad, kOptNtStore>, grid, kAdamBlock,
+  return launch_kernel(adamw_kernel<O, ZERO_GRAD, kAdamBlock, kAdamUnroll, kOptNtLoad, kAdamStorePolicy>, grid, kAdamBlock,
                        stream, p, g, m, v, out16, n, head, s, grad_scale);
 }
 template <class O>

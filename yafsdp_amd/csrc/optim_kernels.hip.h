@@ -260,12 +260,13 @@ __device__ __forceinline__ void adam_elem(float& p, float g, float& m, float& v,
 }
 
 // O is the 16-bit output dtype, or F32 for "no 16-bit output"; ZERO_GRAD also zero-fills the gradient.
-template <class O, bool ZERO_GRAD, int BLOCK, int U, bool NTL, bool NTS>
+template <class O, bool ZERO_GRAD, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0, int head, AdamScalars s,
              const float* grad_scale) {
   static_assert(BLOCK >= 8, "workgroup 0 peels the tail with lanes 0-3 and the head with lanes 4-7");
   constexpr bool kOut = !same_t<O, F32>::value;
+  constexpr bool NTS = (STP == ST_NT);  // the partial last tile keeps ordinary global stores
   const bool scaled = grad_scale != nullptr;
   float gs = 1.0f;
   if (scaled)
@@ -290,9 +291,17 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
         qm[j] = load_quad<F32, NTL>(m + e);
         qv[j] = load_quad<F32, NTL>(v + e);
       }
+      // the tile's first byte in every array it writes (wave-uniform), lane offsets inside the tile
+      const int64_t t0 = tile * kTile * 4;
+      constexpr int kTileBytes = int(kTile) * 16;
+      const TileStore<F32, STP> sp(reinterpret_cast<char*>(p + t0), kTileBytes);
+      const TileStore<F32, STP> sm(reinterpret_cast<char*>(m + t0), kTileBytes);
+      const TileStore<F32, STP> sv(reinterpret_cast<char*>(v + t0), kTileBytes);
+      const TileStore<F32, STP> sg(reinterpret_cast<char*>(g + t0), kTileBytes);
+      const TileStore<O, STP> so(reinterpret_cast<char*>(out16) + t0 * O::kSize, int(kTile) * 4 * O::kSize);
 #pragma unroll
       for (int j = 0; j < U; j++) {
-        const int64_t e = (q0 + j * BLOCK) << 2;
+        const int off = (int(threadIdx.x) + j * BLOCK) * 16;  // bytes inside the tile, binary32 arrays
         float fp[4], fg[4], fm[4], fv[4];
         unpack_quad<F32>(qp[j], fp);
         unpack_quad<F32>(qg[j], fg);
@@ -300,14 +309,14 @@ adamw_kernel(float* p0, float* g0, float* m0, float* v0, void* out0, int64_t n0,
         unpack_quad<F32>(qv[j], fv);
 #pragma unroll
         for (int i = 0; i < 4; i++) adam_elem(fp[i], fg[i], fm[i], fv[i], s, scaled, gs);
-        store_quad<F32, NTS>(p + e, pack_quad<F32>(fp));
-        store_quad<F32, NTS>(m + e, pack_quad<F32>(fm));
-        store_quad<F32, NTS>(v + e, pack_quad<F32>(fv));
-        if constexpr (kOut) store_quad<O, NTS>(reinterpret_cast<char*>(out16) + e * O::kSize, pack_quad<O>(fp));
+        store_quad_at<F32, STP>(sp, off, pack_quad<F32>(fp));
+        store_quad_at<F32, STP>(sm, off, pack_quad<F32>(fm));
+        store_quad_at<F32, STP>(sv, off, pack_quad<F32>(fv));
+        if constexpr (kOut) store_quad_at<O, STP>(so, off / 4 * O::kSize, pack_quad<O>(fp));
         if constexpr (ZERO_GRAD) {
           Quad<F32> z;
           z.v = u32x4{0u, 0u, 0u, 0u};
-          store_quad<F32, NTS>(g + e, z);
+          store_quad_at<F32, STP>(sg, off, z);
         }
       }
     } else {

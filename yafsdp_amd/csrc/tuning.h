@@ -127,6 +127,11 @@ constexpr int kAdamBlock = YAFSDP_ADAM_BLOCK;
 constexpr int kAdamUnroll = YAFSDP_ADAM_U;
 constexpr bool kOptNtLoad = true;
 constexpr bool kOptNtStore = true;
+// store policy of the fused Adam(W) pass (see TileStore)
+#ifndef YAFSDP_ADAM_STP
+#define YAFSDP_ADAM_STP 1
+#endif
+constexpr int kAdamStorePolicy = YAFSDP_ADAM_STP;
 // fan-out / fan-in: a tile is block * unroll quads
 #ifndef YAFSDP_FAN_BLOCK
 #define YAFSDP_FAN_BLOCK 64
