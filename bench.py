@@ -1293,6 +1293,9 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
+    ap.add_argument("--no-fused", action="store_true",
+                    help="shard groups of size one: four launches per step as for any other size, instead of the "
+                         "two launches that each do the work of two")
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: skip the `configs` block (the other configurations of the path, each "
                          "with its own oracle check, about a minute in total)")
@@ -1443,7 +1446,27 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     ]
     if not has_copy_in:  # the all-gather input aliases the master shard (ya_fsdp/_param_group.py:502-505)
         ops = ops[1:]
-    bytes_per_step = sum(b for _, _, b in ops)
+    bytes_per_step = sum(b for _, _, b in ops)  # what the reference's four ops move, however many launches do it
+    dominant = "reduce_copy_in"
+    fused = False
+    if w == 1 and has_copy_in and not args.no_fused:
+        # a shard group of size one: copy-in + copy-out as one launch, reduce copy-in + post-reduce as one launch
+        # (nothing happens between the two halves of either pair, ya_fsdp/_collectives.py:140-150).  The library
+        # declines tables it does not serve that way (more than 16 tensors); then the four calls above stay.
+        def op_unshard():
+            if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
+                raise RuntimeError("copy_in_scatter_out declined")
+
+        def op_reduce():
+            if not table.gather_in_post_reduce(d_grads, d_rs, d_shard, True):
+                raise RuntimeError("gather_in_post_reduce declined")
+
+        if len(numels) <= 16:
+            ops = [
+                ("copy_in_and_copy_out", op_unshard, ops[0][2] + ops[1][2]),
+                ("reduce_copy_in_and_post_reduce", op_reduce, ops[2][2] + ops[3][2]),
+            ]
+            dominant, fused = "reduce_copy_in_and_post_reduce", True
 
     def step():
         for _, fn, _ in ops:
@@ -1496,10 +1519,12 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    dom_index = [n for n, _, _ in ops].index("reduce_copy_in")  # most bytes, fused arithmetic
-    # on every 4th step of the timed region the dominant kernel's dispatch carries a pair of HIP events (attached to
-    # the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
-    sampled = [k for k in range(steps) if k % 4 == 0]
+    dom_index = [n for n, _, _ in ops].index(dominant)  # most bytes, fused arithmetic
+    # on every 4th step of the timed region (of a long region: on 16 steps spread evenly; attaching the pair costs
+    # host time that a launch-bound workload would see) the dominant kernel's dispatch carries a pair of HIP events
+    # (attached to the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
+    every = max(4, -(-steps // 16))
+    sampled = [k for k in range(steps) if k % every == 0]
     ev = {k: _event_pair() for k in sampled}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -1526,6 +1551,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "parity": parity, "bytes_per_step": bytes_per_step,
             "params": len(numels), "padded_numel": t_pad, "shard_numel": s, "logical_world_size": w,
             "dominant_kernel_us": round(dom_avg_us, 2), "dominant_kernel_GBps": round(achieved, 1),
+            "launches_per_step": len(ops), "dominant_kernel": dominant,
         }
 
     # ---- sustained leg: back-to-back steps for at least --sustained-seconds (outside the timed region above; the
@@ -1553,6 +1579,10 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             grad_binding = table.bind(d_grads)
 
             def bound_step():
+                if fused:  # the two launches of a size-one group carry their pointers as kernel arguments
+                    for f in fns:
+                        f()
+                    return
                 if has_copy_in:
                     _native.flat_copy(d_ag_in, d_master)
                 out_binding.scatter_out(d_gathered)
@@ -1634,9 +1664,19 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             ("divide_in_place", lambda: _native.flat_div(d_rs_b, 2.0), 2 * t_pad * rsz),
         ]
         evict = [f for _, f, _ in ops]
+        own_evict = {}
+        if has_copy_in and len(numels) <= 16 and not fused:
+            # copy-in and copy-out as ONE launch (two independent jobs in one grid); compare with the sum of the
+            # two rows of the per-kernel table.  Evicted by the two reduce-side ops.
+            def one_launch_unshard():
+                if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
+                    raise RuntimeError("copy_in_scatter_out declined")
+
+            variant_ops.append(("copy_in_and_copy_out_one_launch", one_launch_unshard, s * (msz + 2) + 2 * t * 2))
+            own_evict["copy_in_and_copy_out_one_launch"] = evict[2:]
         for name, fn, nbytes in variant_ops:
             fn()
-            times = time_alone(fn, evict[:2], reps=10)
+            times = time_alone(fn, own_evict.get(name, evict[:2]), reps=10)
             med = statistics.median(times)
             variants[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
                               "GBps": round(nbytes / med / 1e3, 1),

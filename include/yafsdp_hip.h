@@ -46,7 +46,8 @@ typedef enum yafsdp_status {
   YAFSDP_ERR_WRONG_DEVICE = -4,
   YAFSDP_ERR_OUT_OF_MEMORY = -5,
   YAFSDP_ERR_TOO_LARGE = -6,
-  YAFSDP_ERR_BUSY = -7
+  YAFSDP_ERR_BUSY = -7,
+  YAFSDP_ERR_UNSUPPORTED = -8
 } yafsdp_status;
 
 /* per-tensor mode of yafsdp_gather_in / yafsdp_scatter_out / fragments */
@@ -167,6 +168,42 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
  * 16-byte aligned; pad lanes are never read. */
 int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
                        const uint8_t* mode, int tensor_dtype, void* stream);
+
+/* ---- two launches that do the work of two each --------------------------------
+ * For groups whose per-launch cost matters (a small layer takes 4-7 us per
+ * launch whatever it moves).  Both serve tables of at most 16 tensors and
+ * return YAFSDP_ERR_UNSUPPORTED otherwise, without launching anything; the
+ * separate entry points remain the general route. */
+
+/* Copy-in and materialising copy-out as one grid:
+ *   ag_in[0:n] = cast(master[0:n])                       yafsdp_flat_copy
+ *     (all_gather_input.copy_(padded_sharded_param_data), ya_fsdp/_collectives.py:53-54)
+ *   tensor_p   = flat[offset_p : offset_p + numel_p]     yafsdp_scatter_out
+ *     (the split of the gathered buffer, ya_fsdp/_param_group.py:441-457)
+ * The two jobs are independent: `flat` is a gathered buffer that is already
+ * complete (in the reference both sit back to back on the all-gather stream:
+ * the cast of the next group's shard and the views of the group just
+ * gathered).  ag_in and the tensors have the dtype of `flat`; tables with more
+ * than 2^28 padded elements at odd tensor offsets are not served. */
+int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
+                               const uint8_t* mode, void* ag_in, const void* master, int master_dtype, int64_t n,
+                               void* stream);
+
+/* Reduce copy-in and post-reduce of a shard group of size ONE as one pass.
+ * There the rank's chunk of the reduce buffer is the whole buffer and nothing
+ * happens between the two steps (ya_fsdp/_collectives.py:140-150: the
+ * "reduce-scatter" copies the buffer onto itself), so per element
+ *   flat  = COPY: cast(tensor) | ADD: round(flat + tensor) | SKIP: flat
+ *           (ya_fsdp/_param_group.py:693-708; pad lanes: 0 if zero_pad)
+ *   shard = accumulate ? round(shard + flat) : cast(flat)
+ *           (ya_fsdp/_collectives.py:185 / :189)
+ * with the same two roundings and the same contents of `flat` afterwards as
+ * yafsdp_gather_in followed by yafsdp_post_reduce.  No divide factors: at size
+ * one the reference's are absent or 1.  `shard` has the table's padded element
+ * count; `flat` has the tensors' dtype or binary32.  Both 16-byte aligned. */
+int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
+                                 int tensor_dtype, void* flat, int flat_dtype, int zero_pad, void* shard,
+                                 int shard_dtype, int accumulate, void* stream);
 
 /* ---- the two exchange points, over several buffers ------------------------------
  * One GPU: all buffers are local.  With peer-mapped pointers the same two calls

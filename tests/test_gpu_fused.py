@@ -1,0 +1,213 @@
+"""GPU parity of the two launches that do the work of two each, through the C ABI: against the oracle's torch ops
+(the reference's own calls) and against the separate entry points they stand for."""
+
+from __future__ import annotations
+
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import torch_ops
+from tests.helpers import DTYPES, assert_bits_equal, mixed_values
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def nat():
+    from yafsdp_amd import _native
+
+    return _native
+
+
+def _say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _numels(rng, p, max_log2, with_empty):
+    n = np.floor(np.exp2(rng.uniform(0, max_log2, size=p))).astype(np.int64) | 1
+    if with_empty and p > 3:
+        n[rng.integers(0, p, size=max(1, p // 10))] = 0
+    return n.tolist()
+
+
+# (P, max log2 numel, with_empty, pad, line_aligned)
+CASES = [
+    (1, 3, False, 0, False),
+    (3, 4, False, 5, False),
+    (9, 16, True, 17, False),
+    (16, 14, True, 9, False),
+    (9, 17, False, 64, True),
+    (7, 19, False, 513, False),
+]
+
+
+def _case_numels(case, salt):
+    p, max_log2, with_empty, pad, aligned = case
+    rng = np.random.default_rng(p * 1000 + pad + salt)
+    numels = _numels(rng, p, max_log2, with_empty)
+    if aligned:  # every tensor starts on a 128-byte line of a bf16 buffer: the short scatter-out tile
+        numels = [((n + 63) // 64) * 64 for n in numels]
+    return rng, numels
+
+
+# ----------------------------------------------------- copy-in + copy-out --
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("master_dt,param_dt", [(torch.float32, torch.bfloat16), (torch.float32, torch.float16),
+                                                (torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                                (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("shard_n", [0, 1, 77, 4099, 300_001])
+def test_copy_in_scatter_out(nat, case, master_dt, param_dt, shard_n):
+    rng, numels = _case_numels(case, 11)
+    pad = case[3]
+    t = sum(numels)
+    g = torch.Generator().manual_seed(301 + case[0] + shard_n % 7)
+    _say("copy_in_scatter_out", case, master_dt, param_dt, shard_n, "T", t)
+    gathered = mixed_values(g, t + pad, param_dt)
+    master = mixed_values(g, shard_n + 3, master_dt)
+    # oracle: the cast of the master shard and the split of the gathered buffer
+    want_ag = torch.full((shard_n + 5,), 3.0, dtype=param_dt)
+    torch_ops.copy_in(want_ag[1 : 1 + shard_n], master[3:])
+    want = [torch.full((n + 2,), 3.0, dtype=param_dt) for n in numels]
+    torch_ops.copy_out_materialize(gathered, numels, [w[1 : 1 + n] for w, n in zip(want, numels)])
+    table = nat.TensorTable(numels, t + pad, torch.device(DEV))
+    got_ag = torch.full((shard_n + 5,), 3.0, dtype=param_dt, device=DEV)
+    got = [torch.full((n + 2,), 3.0, dtype=param_dt, device=DEV) for n in numels]
+    dmaster, dgathered = master.to(DEV), gathered.to(DEV)
+    served = table.copy_in_scatter_out(
+        dgathered, [x[1 : 1 + n] for x, n in zip(got, numels)], got_ag[1 : 1 + shard_n], dmaster[3:]
+    )
+    assert served
+    assert_bits_equal(got_ag, want_ag, "all-gather input (guard lanes included)")
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert_bits_equal(a, b, f"tensor {i}")
+    # the separate entry points give the same bytes
+    two_ag = torch.full((shard_n + 5,), 3.0, dtype=param_dt, device=DEV)
+    two = [torch.full((n + 2,), 3.0, dtype=param_dt, device=DEV) for n in numels]
+    nat.flat_copy(two_ag[1 : 1 + shard_n], dmaster[3:])
+    table.scatter_out(dgathered, [x[1 : 1 + n] for x, n in zip(two, numels)])
+    assert torch.equal(two_ag.view(torch.uint8), got_ag.view(torch.uint8))
+    for a, b in zip(two, got):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    # skip modes leave their tensors alone
+    if len(numels) > 1:
+        modes = rng.integers(0, 2, size=len(numels)).tolist()
+        got2 = [torch.full((n,), 3.0, dtype=param_dt, device=DEV) for n in numels]
+        got_ag.fill_(3.0)
+        assert table.copy_in_scatter_out(dgathered, got2, got_ag[1 : 1 + shard_n], dmaster[3:], modes)
+        assert_bits_equal(got_ag, want_ag, "all-gather input, call with modes")
+        pos = 0
+        for i, n in enumerate(numels):
+            ref = torch.full((n,), 3.0, dtype=param_dt)
+            if modes[i]:
+                ref.copy_(gathered[pos : pos + n])
+            assert_bits_equal(got2[i], ref, f"modes tensor {i}")
+            pos += n
+    table.close()
+
+
+def test_copy_in_scatter_out_declines_what_it_does_not_serve(nat):
+    numels = [7] * 17  # more tensors than fit the kernel arguments
+    table = nat.TensorTable(numels, sum(numels), torch.device(DEV))
+    flat = torch.ones(sum(numels), dtype=torch.bfloat16, device=DEV)
+    outs = [torch.zeros(7, dtype=torch.bfloat16, device=DEV) for _ in numels]
+    ag = torch.zeros(8, dtype=torch.bfloat16, device=DEV)
+    master = torch.ones(8, dtype=torch.float32, device=DEV)
+    assert table.copy_in_scatter_out(flat, outs, ag, master) is False
+    torch.cuda.synchronize()
+    assert float(ag.float().abs().sum()) == 0.0 and all(float(o.float().abs().sum()) == 0.0 for o in outs)
+    table.close()
+    table = nat.TensorTable([8, 8], 16, torch.device(DEV))
+    outs = [torch.zeros(8, dtype=torch.float32, device=DEV) for _ in range(2)]
+    assert table.copy_in_scatter_out(flat[:16], outs, ag, master) is False  # tensors of another dtype than the buffer
+    with pytest.raises(ValueError):
+        table.copy_in_scatter_out(flat[:16], [o.bfloat16() for o in outs], ag[:4], master)
+    with pytest.raises(RuntimeError):  # in-place cast
+        both = torch.zeros(16, dtype=torch.float32, device=DEV)
+        table.copy_in_scatter_out(flat[:16], [o.bfloat16() for o in outs], both.view(torch.bfloat16)[:8], both[:8])
+    table.close()
+
+
+# --------------------------------------------- reduce copy-in + post-reduce --
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("grad_dt,rs_dt,shard_dt", [
+    (torch.bfloat16, torch.bfloat16, torch.float32),
+    (torch.bfloat16, torch.float32, torch.float32),
+    (torch.float32, torch.float32, torch.float32),
+    (torch.float16, torch.float16, torch.float32),
+    (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+    (torch.float16, torch.float32, torch.float16),
+])
+@pytest.mark.parametrize("acc", [False, True])
+@pytest.mark.parametrize("zero_pad", [True, False])
+def test_gather_in_post_reduce(nat, case, grad_dt, rs_dt, shard_dt, acc, zero_pad):
+    rng, numels = _case_numels(case, 12)
+    p, pad = len(numels), case[3]
+    t = sum(numels)
+    t_pad = t + pad
+    g = torch.Generator().manual_seed(311 + p)
+    _say("gather_in_post_reduce", case, grad_dt, rs_dt, shard_dt, acc, zero_pad, "T", t)
+    grads = [mixed_values(g, n, grad_dt, 1e-3) for n in numels]
+    modes = rng.integers(0, 3, size=p).tolist() if p > 1 else [1]
+    old = torch.zeros(t_pad + 8, dtype=rs_dt)
+    old[:t_pad] = mixed_values(g, t_pad, rs_dt, 1e-3).flip(0)
+    old[t_pad:] = 5.0
+    shard0 = mixed_values(g, t_pad, shard_dt, 1e-3, specials=False)
+    # oracle: foreach copy / foreach add into the views of the reduce buffer, pad zeroed, then the shard group of
+    # size one's "reduce-scatter" (the buffer itself) copied or added into the gradient shard
+    want_flat = old.clone()
+    views = list(want_flat[:t].split(numels))
+    cp = [i for i, m in enumerate(modes) if m == 1]
+    ad = [i for i, m in enumerate(modes) if m == 2]
+    torch_ops.reduce_copy_in([views[i] for i in cp], [grads[i] for i in cp], False)
+    torch_ops.reduce_copy_in([views[i] for i in ad], [grads[i] for i in ad], True)
+    if zero_pad:
+        want_flat[t:t_pad].zero_()
+    want_shard = shard0.clone()
+    torch_ops.reduce_scatter_local(want_shard, want_flat[:t_pad].clone(), 1, 0, None, None, "add" if acc else "copy")
+    table = nat.TensorTable(numels, t_pad, torch.device(DEV))
+    got_flat, got_shard = old.to(DEV), shard0.to(DEV)
+    dgrads = [torch.cat([x.new_zeros(i % 5), x]).to(DEV)[i % 5 :] for i, x in enumerate(grads)]
+    assert table.gather_in_post_reduce(dgrads, got_flat, got_shard, acc, modes, zero_pad=zero_pad)
+    assert_bits_equal(got_flat, want_flat, "reduce buffer afterwards (guard lanes included)")
+    assert_bits_equal(got_shard, want_shard, "gradient shard")
+    # the two separate calls give the same bytes
+    two_flat, two_shard = old.to(DEV), shard0.to(DEV)
+    table.gather_in(dgrads, two_flat, modes, None, zero_pad=zero_pad)
+    nat.post_reduce(two_shard, two_flat[:t_pad], None, acc)
+    assert_bits_equal(got_flat, two_flat, "reduce buffer against the two calls")
+    assert_bits_equal(got_shard, two_shard, "gradient shard against the two calls")
+    table.close()
+
+
+def test_gather_in_post_reduce_declines_and_errors(nat):
+    numels = [5] * 17
+    table = nat.TensorTable(numels, 96, torch.device(DEV))
+    grads = [torch.ones(5, dtype=torch.bfloat16, device=DEV) for _ in numels]
+    flat = torch.zeros(96, dtype=torch.bfloat16, device=DEV)
+    shard = torch.zeros(96, dtype=torch.float32, device=DEV)
+    assert table.gather_in_post_reduce(grads, flat, shard, False) is False
+    torch.cuda.synchronize()
+    assert float(shard.abs().sum()) == 0.0
+    table.close()
+    table = nat.TensorTable([40, 40], 96, torch.device(DEV))
+    # float32 gradients into a bf16 reduce buffer: not in the list of the fused launch
+    assert table.gather_in_post_reduce([g.float().repeat(8) for g in grads[:2]], flat, shard, False) is False
+    with pytest.raises(ValueError):
+        table.gather_in_post_reduce([g.repeat(8) for g in grads[:2]], flat, shard[:95], False)
+    with pytest.raises(RuntimeError):  # shard not 16-byte aligned
+        wide = torch.zeros(97, dtype=torch.float32, device=DEV)
+        table.gather_in_post_reduce([g.repeat(8) for g in grads[:2]], flat, wide[1:], False)
+    table.close()
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+def test_gather_in_post_reduce_empty_table(nat, dt):
+    table = nat.TensorTable([], 0, torch.device(DEV))
+    flat = torch.zeros(0, dtype=dt, device=DEV)
+    shard = torch.zeros(0, dtype=torch.float32, device=DEV)
+    assert table.gather_in_post_reduce([], flat, shard, True)
+    table.close()

@@ -197,6 +197,61 @@ def test_gradient_accumulation_without_sync_uses_add():
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
 
 
+def test_size_one_group_reduces_in_one_launch(monkeypatch):
+    """A shard group of size one takes the launch that does reduce copy-in and post-reduce together (no collective
+    and no divide sit between them, ya_fsdp/_collectives.py:140-150); a backward that leaves one parameter
+    without a gradient goes the general way.  Both against the reference's op sequence."""
+    from yafsdp_amd import _native
+
+    calls = {"one": 0, "gather": 0}
+    real_one, real_gather = _native.TensorTable.gather_in_post_reduce, _native.TensorTable.gather_in
+
+    def count_one(self, *a, **k):
+        served = real_one(self, *a, **k)
+        calls["one"] += int(served)
+        return served
+
+    def count_gather(self, *a, **k):
+        calls["gather"] += 1
+        return real_gather(self, *a, **k)
+
+    monkeypatch.setattr(_native.TensorTable, "gather_in_post_reduce", count_one)
+    monkeypatch.setattr(_native.TensorTable, "gather_in", count_gather)
+    shapes, w, r, align = ODD_SHAPES, 1, 0, 8
+    group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
+    ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.bfloat16, 30), reduce=False)   # copy into the buffer, no reduce
+    assert calls == {"one": 0, "gather": 1}
+    group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.bfloat16, 31), reduce=True)    # add + copy into the shard
+    ref.reduce(None, None, "copy")
+    group.finalize_backward()
+    assert calls == {"one": 1, "gather": 1}
+    assert_bits_equal(group._reduce_scatter_input[None], ref.rs, "reduce buffer after the first reduce")
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard after the first reduce")
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    _run_backward(group, ref, _grads(shapes, torch.bfloat16, 32), reduce=True)    # copy + add into the shard
+    ref.reduce(None, None, "add")
+    group.finalize_backward()
+    assert calls == {"one": 2, "gather": 1}
+    assert_bits_equal(group._reduce_scatter_input[None], ref.rs, "reduce buffer after the second reduce")
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard after the second reduce")
+    for fp in group.fsdp_params:
+        assert fp.sharded_param.grad is fp.sharded_param_grad
+    assert group.grad_buffer_ctx.owner is None and group._training_state.name == "IDLE"
+    # one parameter without a gradient: its fragment keeps the old value (:191-214), the general route
+    group.pre_forward(); group.post_forward(); group.pre_backward()
+    grads = _grads(shapes, torch.bfloat16, 33)
+    grads[2] = None
+    _run_backward(group, ref, grads, reduce=True)
+    ref.reduce(None, None, "mixed", [None if g is None else True for g in grads])
+    group.finalize_backward()
+    assert calls == {"one": 2, "gather": 3}  # reduce copy-in, and the fragment-wise accumulation into the shard
+    torch.cuda.synchronize()
+    assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard after the partial backward")
+
+
 def test_mixed_params_with_and_without_sharded_grad(monkeypatch):
     from yafsdp_amd import _native
 

@@ -13,9 +13,9 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libyafsdp_hip.so")
-SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip", "fan.hip", "postsumsq.hip"]
+SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip", "fan.hip", "postsumsq.hip", "fused.hip"]
 HEADERS = ["elem.hip.h", "flat_kernels.hip.h", "table_kernels.hip.h", "optim_kernels.hip.h", "fan_kernels.hip.h",
-           "post_sumsq_kernels.hip.h", "launch.h", "tuning.h"]
+           "post_sumsq_kernels.hip.h", "fused_kernels.hip.h", "launch.h", "tuning.h"]
 ARCH = "gfx950"
 
 # -ffp-contract=off: every multiply and add of the path rounds on its own, as
@@ -46,7 +46,7 @@ def _compile(src: str, obj: str) -> None:
         print(err)
 
 
-def build(force: bool = True, jobs: int = 7) -> str:
+def build(force: bool = True, jobs: int = 8) -> str:
     """Compile every translation unit and link the shared library."""
     srcs = [os.path.join(CSRC, s) for s in SOURCES + HEADERS] + [os.path.join(HERE, "..", "include", "yafsdp_hip.h")]
     if not force and os.path.exists(OUT) and all(os.path.getmtime(OUT) >= os.path.getmtime(s) for s in srcs):

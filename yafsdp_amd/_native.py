@@ -50,6 +50,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_table_info",
     "yafsdp_gather_in",
     "yafsdp_scatter_out",
+    "yafsdp_copy_in_scatter_out",
+    "yafsdp_gather_in_post_reduce",
     "yafsdp_flat_copy_fanout",
     "yafsdp_post_reduce_fanin",
     "yafsdp_binding_create",
@@ -110,6 +112,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_gather_in.argtypes = [vp, vp, vp, i32, vp, i32, dbl, i32, vp]
     lib.yafsdp_scatter_out.restype = i32
     lib.yafsdp_scatter_out.argtypes = [vp, vp, i32, vp, vp, i32, vp]
+    lib.yafsdp_copy_in_scatter_out.restype = i32
+    lib.yafsdp_copy_in_scatter_out.argtypes = [vp, vp, i32, vp, vp, vp, vp, i32, i64, vp]
+    lib.yafsdp_gather_in_post_reduce.restype = i32
+    lib.yafsdp_gather_in_post_reduce.argtypes = [vp, vp, vp, i32, vp, i32, i32, vp, i32, i32, vp]
     lib.yafsdp_flat_copy_fanout.restype = i32
     lib.yafsdp_flat_copy_fanout.argtypes = [vp, i32, i32, vp, i32, i64, vp]
     lib.yafsdp_post_reduce_fanin.restype = i32
@@ -163,6 +169,7 @@ def error_string(code: int) -> str:
 
 
 ERR_BUSY = -7  # YAFSDP_ERR_BUSY: every staging slot of a table is held by a queued call
+ERR_UNSUPPORTED = -8  # YAFSDP_ERR_UNSUPPORTED: a fused entry point does not serve this table / dtype combination
 
 
 def _check(code: int, what: str) -> None:
@@ -448,6 +455,54 @@ class TensorTable:
                 torch.cuda.current_stream(self.device).synchronize()
                 code = lib.yafsdp_gather_in(*args)
             _check(code, "yafsdp_gather_in")
+
+    def copy_in_scatter_out(
+        self, flat: torch.Tensor, tensors: Sequence[torch.Tensor | None], ag_in: torch.Tensor, master: torch.Tensor,
+        modes: Sequence[int] | None = None,
+    ) -> bool:
+        """``flat_copy(ag_in, master)`` and ``scatter_out(flat, tensors)`` as ONE launch (two independent jobs in
+        one grid).  Returns False without launching anything when the library does not serve this table that way
+        (more than 16 tensors); the caller then makes the two calls."""
+        _flat_arg(flat, "flat"), _flat_arg(ag_in, "ag_in"), _flat_arg(master, "master")
+        if flat.numel() < self.total_numel:
+            raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.total_numel}")
+        if ag_in.numel() != master.numel() or ag_in.dtype != flat.dtype:
+            raise ValueError("ag_in must have the master shard's element count and the gathered buffer's dtype")
+        with self._lock, _on(self.device):
+            tdt = self._fill(tensors, modes, "tensors")
+            if tdt >= 0 and tdt != _dt(flat):
+                return False
+            code = lib.yafsdp_copy_in_scatter_out(
+                self._handle, flat.data_ptr(), _dt(flat), self._ptrs.ctypes.data, self._modes.ctypes.data,
+                ag_in.data_ptr(), master.data_ptr(), _dt(master), master.numel(), _stream(flat),
+            )
+        if code == ERR_UNSUPPORTED:
+            return False
+        _check(code, "yafsdp_copy_in_scatter_out")
+        return True
+
+    def gather_in_post_reduce(
+        self, tensors: Sequence[torch.Tensor | None], flat: torch.Tensor, shard: torch.Tensor, accumulate: bool,
+        modes: Sequence[int] | None = None, zero_pad: bool = True,
+    ) -> bool:
+        """Reduce copy-in into ``flat`` and post-reduce of the whole buffer into ``shard`` as ONE launch: what a
+        shard group of size one does between backward and optimizer (no collective in between, no divide).
+        Returns False without launching anything when the library does not serve this table / dtype combination."""
+        _flat_arg(flat, "flat"), _flat_arg(shard, "shard")
+        if flat.numel() < self.padded_numel or shard.numel() != self.padded_numel:
+            raise ValueError(f"flat / shard hold {flat.numel()} / {shard.numel()} elements, table needs {self.padded_numel}")
+        with self._lock, _on(self.device):
+            tdt = self._fill(tensors, modes, "tensors")
+            if tdt < 0:
+                tdt = _dt(flat)
+            code = lib.yafsdp_gather_in_post_reduce(
+                self._handle, self._ptrs.ctypes.data, self._modes.ctypes.data, tdt, flat.data_ptr(), _dt(flat),
+                int(bool(zero_pad)), shard.data_ptr(), _dt(shard), int(bool(accumulate)), _stream(flat),
+            )
+        if code == ERR_UNSUPPORTED:
+            return False
+        _check(code, "yafsdp_gather_in_post_reduce")
+        return True
 
     def scatter_out(
         self, flat: torch.Tensor, tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None = None

@@ -423,6 +423,7 @@ class YaFSDPParamGroup:
                 grad_buffer_ctx.release_event = None
             grad_buffer_ctx.owner = self
         predivide_fused = False
+        reduced_in_one_launch = False
         with profiler_range(self._with_fqn("FSDP::post_backward_accumulate")):
             grads: list[torch.Tensor | None] = []
             modes: list[int] = []
@@ -449,7 +450,9 @@ class YaFSDPParamGroup:
                         self.force_sum_reduction_for_comms,
                     )
                     predivide_fused = True
-                foreach_reduce_copy_in(self, self._table, self._reduce_scatter_input[None], grads, modes, pre)
+                    reduced_in_one_launch = self._reduce_in_one_launch(grads, modes)
+                if not reduced_in_one_launch:
+                    foreach_reduce_copy_in(self, self._table, self._reduce_scatter_input[None], grads, modes, pre)
         fsdp_params_with_grad_per_dtype: dict[torch.dtype | None, list[YaFSDPParam]] = {}
         with profiler_range(self._with_fqn("YaFSDP::post_backward_reshard")):
             if not self.reduce_grads:
@@ -471,6 +474,15 @@ class YaFSDPParamGroup:
                 grad_buffer_ctx.owner = None
             return
         assert grad_buffer_ctx is not None
+        if reduced_in_one_launch:
+            # the gradient shard is already written, on this stream (ya_fsdp/_collectives.py:216-217 for the rest)
+            with profiler_range(self._with_fqn("YaFSDP::post_backward_reduce")):
+                self._post_reduce_event = current_stream.record_event()
+                for fsdp_param in fsdp_params_with_grad_per_dtype[None]:
+                    fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad
+            grad_buffer_ctx.release_event = self._post_reduce_event
+            grad_buffer_ctx.owner = None
+            return
         with profiler_range(self._with_fqn("YaFSDP::post_backward_reduce")):
             for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
                 self._post_reduce_event = reduce_scatter(
@@ -492,6 +504,43 @@ class YaFSDPParamGroup:
                 )
         grad_buffer_ctx.release_event = self._post_reduce_event
         grad_buffer_ctx.owner = None
+
+    def _reduce_in_one_launch(self, grads: "list[torch.Tensor | None]", modes: "list[int]") -> bool:
+        """A shard group of size ONE whose gradients pass through the reduce buffer: the rank's chunk is the whole
+        buffer, the "reduce-scatter" copies it onto itself (ya_fsdp/_collectives.py:140-150) and, without a custom
+        divide factor, nothing is divided, so the reduce copy-in (ya_fsdp/_param_group.py:693-708) and the copy or
+        accumulation into the gradient shard (ya_fsdp/_collectives.py:185 / :189) run as one launch on the current
+        stream, with the same rounding points and the same contents of the reduce buffer afterwards.  Returns
+        False, having launched nothing, for every other case; the caller then takes the general route."""
+        group = self._reduce_scatter_process_group
+        if group.size() != 1 or self.gradient_divide_factor is not None or self._grad_sumsq_slot is not None:
+            return False
+        if list(self._all_gather_dtype_to_fsdp_params) != [None] or self._table is None:
+            return False
+        need = [p for p in self.fsdp_params if p.sharded_param.requires_grad]
+        in_sharded = (
+            (self.reduce_dtype is None and self.param_dtype is None) or self.reduce_dtype == self.orig_dtype
+        ) and all(p.sharded_param.grad is None for p in need)  # ya_fsdp/_collectives.py:112-123
+        if in_sharded:
+            return False
+        with_grad = [p for p in self.fsdp_params if p.unsharded_accumulated_grad is not None]
+        if len(with_grad) != len(need):
+            return False  # some fragments keep their old gradient: ya_fsdp/_collectives.py:191-214
+        n_acc = sum(p.sharded_param.grad is not None for p in with_grad)
+        if n_acc not in (0, len(with_grad)):
+            return False
+        pre, post, _, _ = _get_gradient_divide_factors(
+            group, self.reduce_scatter_dtype, None, self.force_sum_reduction_for_comms
+        )
+        if (pre is not None and pre > 1) or (post is not None and post > 1):
+            return False
+        shard = self._padded_sharded_param_grad[None]
+        if shard is None:
+            return False
+        if not _native.all_contiguous(grads):
+            grads = [g if g is None or g.is_contiguous() else g.contiguous() for g in grads]
+        self._grad_sumsq_token = None
+        return self._table.gather_in_post_reduce(grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes)
 
     def finalize_backward(self) -> None:
         """ya_fsdp/_param_group.py:773-783."""

@@ -97,16 +97,15 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
 // `trace` (normally null) is a measurement hook: workgroup b stores the 100 MHz
 // wall-clock count at its start and, after its stores have been acknowledged,
 // at its end into trace[2 b], trace[2 b + 1].
+// The flat pass as seen by workgroup `block` of `n_blocks` (the whole grid of flat_kernel, or the part of a
+// larger grid that serves this job).
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
-__global__ void __launch_bounds__(BLOCK)
-flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned long long* trace) {
-  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
+__device__ __forceinline__ void flat_body(void* dst, const void* src, int64_t n, int head, float k, int block,
+                                          int n_blocks) {
   const int tid = threadIdx.x;
-  unsigned long long t_start = 0;
-  if (trace != nullptr) t_start = wall_clock64();
   const int64_t n_units = (n - head) >> 3;
   const int64_t body_end = head + (n_units << 3);
-  if (blockIdx.x == 0) {
+  if (block == 0) {
     if (tid < head) flat_scalar<S, D, SCALE, ACC>(dst, src, tid, k);
     const int tail = int(n - body_end);
     const int t = BLOCK - 1 - tid;
@@ -116,7 +115,7 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned l
   const char* sbase = reinterpret_cast<const char*>(src) + int64_t(head) * S::kSize;
   constexpr int64_t kTile = int64_t(BLOCK) * U;
   const int64_t n_tiles = (n_units + kTile - 1) / kTile;
-  for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+  for (int64_t tile = block; tile < n_tiles; tile += n_blocks) {
     if (tile * kTile + kTile <= n_units) {
       flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dbase + tile * kTile * (8 * D::kSize),
                                                            sbase + tile * kTile * (8 * S::kSize), k);
@@ -129,9 +128,18 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned l
       }
     }
   }
+}
+
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
+__global__ void __launch_bounds__(BLOCK)
+flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned long long* trace) {
+  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
+  unsigned long long t_start = 0;
+  if (trace != nullptr) t_start = wall_clock64();
+  flat_body<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dst, src, n, head, k, int(blockIdx.x), int(gridDim.x));
   if (trace != nullptr) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every load has arrived, every store is acknowledged
-    if (tid == 0) {
+    if (threadIdx.x == 0) {
       trace[2 * blockIdx.x] = t_start;
       trace[2 * blockIdx.x + 1] = wall_clock64();
     }

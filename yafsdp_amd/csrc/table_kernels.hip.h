@@ -367,20 +367,18 @@ __device__ __forceinline__ void scatter_segment(char* dst, const char* src, int6
 }
 
 // S: flat buffer dtype, D: tensor dtype.  Tensors with mode 0 are not written;
-// pad lanes of the flat buffer are never read.  n_tiles counts tile slots.
+// pad lanes of the flat buffer are never read.  n_tiles counts tile slots.  `block` of `n_blocks`: the workgroup's
+// place in the grid of scatter_out_kernel, or in the part of a larger grid that serves this job.
 template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
-__global__ void __launch_bounds__(BLOCK)
-scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
-  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
+__device__ __forceinline__ void scatter_body(const META& meta, const void* flat, int n_tiles, int block, int n_blocks) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   constexpr int64_t kLineElems = 128 / D::kSize;
   const char* fbase = reinterpret_cast<const char*>(flat);
-  (void)total;
   constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
   constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
-  const int n_blocks = (n_tiles + kWin - 1) / kWin * kWin;
-  for (int b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+  const int n_rounded = (n_tiles + kWin - 1) / kWin * kWin;
+  for (int b = block; b < n_rounded; b += n_blocks) {
     const int tile = tile_of_block<kX, kWin>(b);
     if (tile >= n_tiles) continue;
     const ScatterLookup rec = meta.lookup_scatter(tile);
@@ -401,6 +399,14 @@ scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
     if (hi - lo == kTile) scatter_full_tile<S, D, BLOCK, U, NTL, STP>(dst, src);
     else scatter_segment<S, D, BLOCK, NTL, NTS>(dst, src, hi - lo);
   }
+}
+
+template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
+__global__ void __launch_bounds__(BLOCK)
+scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
+  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
+  (void)total;
+  scatter_body<META, S, D, BLOCK, U, NTL, STP>(meta, flat, n_tiles, int(blockIdx.x), int(gridDim.x));
 }
 
 }  // namespace yafsdp
