@@ -1294,8 +1294,9 @@ def main() -> int:
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
     ap.add_argument("--no-fused", action="store_true",
-                    help="shard groups of size one: four launches per step as for any other size, instead of the "
-                         "two launches that each do the work of two")
+                    help="four launches per step, one per op of the path.  Default: copy-in and copy-out share one "
+                         "launch where the library serves the table that way (at most 16 tensors), and a shard group "
+                         "of size one also runs reduce copy-in and post-reduce as one launch")
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: skip the `configs` block (the other configurations of the path, each "
                          "with its own oracle check, about a minute in total)")
@@ -1467,6 +1468,15 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                 ("reduce_copy_in_and_post_reduce", op_reduce, ops[2][2] + ops[3][2]),
             ]
             dominant, fused = "reduce_copy_in_and_post_reduce", True
+    elif has_copy_in and not args.no_fused and len(numels) <= 16:
+        # any group size: copy-in and copy-out as one grid (both sit back to back on the all-gather stream in the
+        # reference, ya_fsdp/_collectives.py:46-58 and ya_fsdp/_param_group.py:581-594)
+        def op_unshard_w():
+            if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
+                raise RuntimeError("copy_in_scatter_out declined")
+
+        ops = [("copy_in_and_copy_out", op_unshard_w, ops[0][2] + ops[1][2])] + ops[2:]
+        fused = True
 
     def step():
         for _, fn, _ in ops:
@@ -1523,7 +1533,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     # on every 4th step of the timed region (of a long region: on 16 steps spread evenly; attaching the pair costs
     # host time that a launch-bound workload would see) the dominant kernel's dispatch carries a pair of HIP events
     # (attached to the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
-    every = max(4, -(-steps // 16))
+    every = max(4, -(-steps // (16 if full else 4)))  # the compact records of the other configurations: 4 samples
     sampled = [k for k in range(steps) if k % every == 0]
     ev = {k: _event_pair() for k in sampled}
     torch.cuda.synchronize()
@@ -1628,8 +1638,9 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         return times
 
     kernels = {}
-    for name, fn, nbytes in ops:
-        times = time_alone(fn, [f for n2, f, _ in ops if n2 != name])
+    for i, (name, fn, nbytes) in enumerate(ops):
+        # the rest of the step runs before it, in step order, so the op sees the caches as it does inside a step
+        times = time_alone(fn, [f for _, f, _ in ops[i + 1:] + ops[:i]])
         med = statistics.median(times)
         warm = []  # same op back to back: whatever fits stays in the 256 MB memory-side cache
         for _ in range(20):
@@ -1674,6 +1685,11 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
 
             variant_ops.append(("copy_in_and_copy_out_one_launch", one_launch_unshard, s * (msz + 2) + 2 * t * 2))
             own_evict["copy_in_and_copy_out_one_launch"] = evict[2:]
+        elif fused and w > 1:
+            # the step runs copy-in and copy-out as one launch: here each as a launch of its own
+            variant_ops.append(("copy_in_alone", op_copy_in, s * (msz + 2)))
+            variant_ops.append(("copy_out_alone", op_copy_out, 2 * t * 2))
+            own_evict["copy_in_alone"] = own_evict["copy_out_alone"] = evict[1:]
         for name, fn, nbytes in variant_ops:
             fn()
             times = time_alone(fn, own_evict.get(name, evict[:2]), reps=10)
@@ -1776,11 +1792,15 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             "ops": ("copy-in master->bf16 [S]; " if has_copy_in else "") +
                    "copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
                    "post-reduce chunk += gradient shard (master dtype) [S]",
+            "launches_per_step": [n for n, _, _ in ops],
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "parity": parity,
         "roofline": {
-            "bound": "hbm", "kernel": "gather_in_kernel (reduce copy-in)", "achieved": round(achieved, 1),
+            "bound": "hbm",
+            "kernel": "gather_in_kernel (reduce copy-in)" if dominant == "reduce_copy_in"
+                      else "gather_post_kernel (reduce copy-in + post-reduce of a size-one group)",
+            "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
             "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2), "launches_timed": len(dom_us),

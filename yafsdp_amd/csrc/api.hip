@@ -519,7 +519,7 @@ int yafsdp_flat_copy_fanout(void* const* dsts, int n_dst, int dst_dtype, const v
     if (!aligned_to(dsts[k], 16)) return YAFSDP_ERR_MISALIGNED;
     ptrs.p[k] = dsts[k];
   }
-  const int grid = opt_grid(n >> 3, kFanBlock, kFanOutUnroll, nullptr);
+  const int grid = opt_grid(n >> 3, kFanOutBlock, kFanOutUnroll, nullptr);
   return int(launch_fanout(src_dtype, dst_dtype, ptrs, src, n, grid, static_cast<hipStream_t>(stream)));
 }
 
@@ -541,7 +541,7 @@ int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* ch
   int scale;
   float k;
   scale_plan(post_factor, &scale, &k);
-  const int grid = opt_grid(n >> 2, kFanBlock, kFanInUnroll, nullptr);
+  const int grid = opt_grid(n >> 2, kFanInBlock, kFanInUnroll, nullptr);
   return int(launch_fanin(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, ptrs, n, k, grid,
                           static_cast<hipStream_t>(stream)));
 }

@@ -8,7 +8,7 @@ namespace {
 
 template <class S, class D>
 hipError_t fanout_go(const FanPtrs& dsts, const void* src, int64_t n, int grid, hipStream_t stream) {
-  return launch_kernel(fanout_kernel<S, D, kFanBlock, kFanOutUnroll, kOptNtLoad, kFanNtStore>, grid, kFanBlock, stream,
+  return launch_kernel(fanout_kernel<S, D, kFanOutBlock, kFanOutUnroll, kOptNtLoad, kFanOutStorePolicy>, grid, kFanOutBlock, stream,
                        dsts, src, n);
 }
 
@@ -24,7 +24,7 @@ hipError_t fanout_by_dst(int dst_dt, const FanPtrs& dsts, const void* src, int64
 
 template <class S, class D, int SCALE, bool ACC>
 hipError_t fanin_go(void* shard, const FanPtrs& chunks, int64_t n, float k, int grid, hipStream_t stream) {
-  return launch_kernel(fanin_kernel<S, D, SCALE, ACC, kFanBlock, kFanInUnroll, kOptNtLoad, kOptNtStore>, grid, kFanBlock,
+  return launch_kernel(fanin_kernel<S, D, SCALE, ACC, kFanInBlock, kFanInUnroll, kOptNtLoad, kOptNtStore>, grid, kFanInBlock,
                        stream, shard, chunks, n, k);
 }
 

@@ -19,13 +19,15 @@ namespace yafsdp {
 // followed by the placement the all-gather performs, :60-65).  The kernel is
 // dominated by its stores (n_dst of them per load), so lanes own units (8
 // consecutive elements): every store is a full 16 bytes of a 2-byte dtype.
-template <class S, class D, int BLOCK, int U, bool NTL, bool NTS>
+template <class S, class D, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 fanout_kernel(FanPtrs dsts, const void* src, int64_t n) {
   typedef typename S::storage s_t;
   typedef typename D::storage d_t;
+  constexpr bool NTS = (STP == ST_NT);  // the ragged last tile keeps ordinary global stores
   const int64_t n_units = n >> 3;
   constexpr int64_t kTile = int64_t(BLOCK) * U;
+  constexpr int kTileBytes = int(kTile) * 8 * D::kSize;
   const int64_t n_tiles = (n_units + kTile - 1) / kTile;
   const char* sbase = reinterpret_cast<const char*>(src);
   for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
@@ -39,9 +41,9 @@ fanout_kernel(FanPtrs dsts, const void* src, int64_t n) {
         y[j] = flat_unit<S, D, SCALE_NONE, false>(x, unused, 0.f);
       }
       for (int k = 0; k < dsts.n; k++) {
-        char* d = reinterpret_cast<char*>(dsts.p[k]);
+        const TileStore<D, STP> out(reinterpret_cast<char*>(dsts.p[k]) + tile * kTileBytes, kTileBytes);
 #pragma unroll
-        for (int j = 0; j < U; j++) store_unit<D, NTS>(d + (u0 + j * BLOCK) * (8 * D::kSize), y[j]);
+        for (int j = 0; j < U; j++) store_unit_at<D, STP>(out, (int(threadIdx.x) + j * BLOCK) * (8 * D::kSize), y[j]);
       }
     } else {
       for (int64_t u = u0; u < n_units; u += BLOCK) {

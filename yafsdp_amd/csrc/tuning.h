@@ -132,22 +132,31 @@ constexpr bool kOptNtStore = true;
 #define YAFSDP_ADAM_STP 1
 #endif
 constexpr int kAdamStorePolicy = YAFSDP_ADAM_STP;
-// fan-out / fan-in: a tile is block * unroll quads
-#ifndef YAFSDP_FAN_BLOCK
-#define YAFSDP_FAN_BLOCK 64
+// fan-out: a tile is block * unroll units.  With 8 destinations the kernel is 80 % stores.  Write-through stores
+// (see TileStore) with 256 lanes make the kernel itself 5 % faster (94.9 against 99.3 us on a 27 M-element shard),
+// but the kernel that runs after it pays three times that (the fan-in of the same step: 94 -> 113 us), so the
+// stores stay non-temporal.  One pass over the source for all destinations: two passes of four take 115 us.
+// 256 lanes, two units per lane or a fully unrolled destination loop are level or slower (98 -> 99-108 us).
+#ifndef YAFSDP_FANOUT_BLOCK
+#define YAFSDP_FANOUT_BLOCK 64
 #endif
 #ifndef YAFSDP_FANOUT_U
 #define YAFSDP_FANOUT_U 1
 #endif
+#ifndef YAFSDP_FANOUT_STP
+#define YAFSDP_FANOUT_STP 1
+#endif
+// fan-in: a tile is block * unroll quads
+#ifndef YAFSDP_FANIN_BLOCK
+#define YAFSDP_FANIN_BLOCK 64
+#endif
 #ifndef YAFSDP_FANIN_U
 #define YAFSDP_FANIN_U 1
 #endif
-#ifndef YAFSDP_FAN_NTS
-#define YAFSDP_FAN_NTS true
-#endif
-constexpr bool kFanNtStore = YAFSDP_FAN_NTS;
-constexpr int kFanBlock = YAFSDP_FAN_BLOCK;
+constexpr int kFanOutBlock = YAFSDP_FANOUT_BLOCK;
 constexpr int kFanOutUnroll = YAFSDP_FANOUT_U;
+constexpr int kFanOutStorePolicy = YAFSDP_FANOUT_STP;
+constexpr int kFanInBlock = YAFSDP_FANIN_BLOCK;
 constexpr int kFanInUnroll = YAFSDP_FANIN_U;
 // workgroups (= partial sums) of the sum-of-squares pass; the workspace holds one double each
 constexpr int kSumsqMaxPartials = 16384;
