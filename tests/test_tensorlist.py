@@ -16,9 +16,7 @@ def _table(numels, device="cpu"):
     t = _native.TensorTable.__new__(_native.TensorTable)
     t.numels = list(numels)
     t.device = torch.device(device)
-    t._numels_arr = np.ascontiguousarray(t.numels, dtype=np.int64)
-    t._ptrs = np.zeros(max(1, len(numels)), dtype=np.uint64)
-    t._modes = np.zeros(max(1, len(numels)), dtype=np.uint8)
+    t._init_host_arrays()
     return t
 
 
