@@ -1311,8 +1311,7 @@ def main() -> int:
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
     ap.add_argument("--no-fused", action="store_true",
                     help="four launches per step, one per op of the path.  Default: copy-in and copy-out share one "
-                         "launch where the library serves the table that way (at most 16 tensors), and a shard group "
-                         "of size one also runs reduce copy-in and post-reduce as one launch")
+                         "launch, and a shard group of size one also runs reduce copy-in and post-reduce as one launch")
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: skip the `configs` block (the other configurations of the path, each "
                          "with its own oracle check, about a minute in total)")
@@ -1468,8 +1467,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     fused = False
     if w == 1 and has_copy_in and not args.no_fused:
         # a shard group of size one: copy-in + copy-out as one launch, reduce copy-in + post-reduce as one launch
-        # (nothing happens between the two halves of either pair, ya_fsdp/_collectives.py:140-150).  The library
-        # declines tables it does not serve that way (more than 16 tensors); then the four calls above stay.
+        # (nothing happens between the two halves of either pair, ya_fsdp/_collectives.py:140-150)
         def op_unshard():
             if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
                 raise RuntimeError("copy_in_scatter_out declined")
@@ -1478,13 +1476,12 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             if not table.gather_in_post_reduce(d_grads, d_rs, d_shard, True):
                 raise RuntimeError("gather_in_post_reduce declined")
 
-        if len(numels) <= 16:
-            ops = [
-                ("copy_in_and_copy_out", op_unshard, ops[0][2] + ops[1][2]),
-                ("reduce_copy_in_and_post_reduce", op_reduce, ops[2][2] + ops[3][2]),
-            ]
-            dominant, fused = "reduce_copy_in_and_post_reduce", True
-    elif has_copy_in and not args.no_fused and len(numels) <= 16:
+        ops = [
+            ("copy_in_and_copy_out", op_unshard, ops[0][2] + ops[1][2]),
+            ("reduce_copy_in_and_post_reduce", op_reduce, ops[2][2] + ops[3][2]),
+        ]
+        dominant, fused = "reduce_copy_in_and_post_reduce", True
+    elif has_copy_in and not args.no_fused:
         # any group size: copy-in and copy-out as one grid (both sit back to back on the all-gather stream in the
         # reference, ya_fsdp/_collectives.py:46-58 and ya_fsdp/_param_group.py:581-594)
         def op_unshard_w():
@@ -1605,7 +1602,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             grad_binding = table.bind(d_grads)
 
             def bound_step():
-                if fused:  # the two launches of a size-one group carry their pointers as kernel arguments
+                if fused and len(numels) <= 16:  # small tables carry their pointers as kernel arguments
                     for f in fns:
                         f()
                     return
@@ -1692,7 +1689,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         ]
         evict = [f for _, f, _ in ops]
         own_evict = {}
-        if has_copy_in and len(numels) <= 16 and not fused:
+        if has_copy_in and not fused:
             # copy-in and copy-out as ONE launch (two independent jobs in one grid); compare with the sum of the
             # two rows of the per-kernel table.  Evicted by the two reduce-side ops.
             def one_launch_unshard():

@@ -171,9 +171,9 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
 
 /* ---- two launches that do the work of two each --------------------------------
  * For groups whose per-launch cost matters (a small layer takes 4-7 us per
- * launch whatever it moves).  Both serve tables of at most 16 tensors and
- * return YAFSDP_ERR_UNSUPPORTED otherwise, without launching anything; the
- * separate entry points remain the general route. */
+ * launch whatever it moves) and, for the second, for the bytes it saves.  Tables
+ * of any size are served, with the staging rules of yafsdp_gather_in for tables
+ * of more than 16 tensors (YAFSDP_ERR_BUSY included). */
 
 /* Copy-in and materialising copy-out as one grid:
  *   ag_in[0:n] = cast(master[0:n])                       yafsdp_flat_copy
@@ -183,8 +183,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
  * The two jobs are independent: `flat` is a gathered buffer that is already
  * complete (in the reference both sit back to back on the all-gather stream:
  * the cast of the next group's shard and the views of the group just
- * gathered).  ag_in and the tensors have the dtype of `flat`; tables with more
- * than 2^28 padded elements at odd tensor offsets are not served. */
+ * gathered).  ag_in and the tensors have the dtype of `flat`. */
 int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,
                                const uint8_t* mode, void* ag_in, const void* master, int master_dtype, int64_t n,
                                void* stream);
@@ -200,7 +199,11 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
  * with the same two roundings and the same contents of `flat` afterwards as
  * yafsdp_gather_in followed by yafsdp_post_reduce.  No divide factors: at size
  * one the reference's are absent or 1.  `shard` has the table's padded element
- * count; `flat` has the tensors' dtype or binary32.  Both 16-byte aligned. */
+ * count.  Both buffers 16-byte aligned.  `flat` has the tensors' dtype or
+ * binary32; YAFSDP_ERR_UNSUPPORTED otherwise, with nothing launched (the two
+ * separate entry points serve every combination).  The reduce buffer is not
+ * read back: 12 instead of 14 bytes per element for bf16 gradients, a bf16
+ * buffer and a binary32 shard that accumulates. */
 int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
                                  int tensor_dtype, void* flat, int flat_dtype, int zero_pad, void* shard,
                                  int shard_dtype, int accumulate, void* stream);

@@ -42,6 +42,9 @@ CASES = [
     (16, 14, True, 9, False),
     (9, 17, False, 64, True),
     (7, 19, False, 513, False),
+    (33, 14, True, 9, False),      # more than 16 tensors: records and per-call pointers in device memory
+    (200, 12, True, 4096, False),
+    (40, 12, False, 0, True),
 ]
 
 
@@ -109,26 +112,63 @@ def test_copy_in_scatter_out(nat, case, master_dt, param_dt, shard_n):
     table.close()
 
 
-def test_copy_in_scatter_out_declines_what_it_does_not_serve(nat):
-    numels = [7] * 17  # more tensors than fit the kernel arguments
-    table = nat.TensorTable(numels, sum(numels), torch.device(DEV))
-    flat = torch.ones(sum(numels), dtype=torch.bfloat16, device=DEV)
-    outs = [torch.zeros(7, dtype=torch.bfloat16, device=DEV) for _ in numels]
+def test_copy_in_scatter_out_declines_and_errors(nat):
+    flat = torch.ones(16, dtype=torch.bfloat16, device=DEV)
     ag = torch.zeros(8, dtype=torch.bfloat16, device=DEV)
     master = torch.ones(8, dtype=torch.float32, device=DEV)
-    assert table.copy_in_scatter_out(flat, outs, ag, master) is False
-    torch.cuda.synchronize()
-    assert float(ag.float().abs().sum()) == 0.0 and all(float(o.float().abs().sum()) == 0.0 for o in outs)
-    table.close()
     table = nat.TensorTable([8, 8], 16, torch.device(DEV))
     outs = [torch.zeros(8, dtype=torch.float32, device=DEV) for _ in range(2)]
-    assert table.copy_in_scatter_out(flat[:16], outs, ag, master) is False  # tensors of another dtype than the buffer
+    assert table.copy_in_scatter_out(flat, outs, ag, master) is False  # tensors of another dtype than the buffer
+    torch.cuda.synchronize()
+    assert float(ag.float().abs().sum()) == 0.0 and all(float(o.abs().sum()) == 0.0 for o in outs)
     with pytest.raises(ValueError):
-        table.copy_in_scatter_out(flat[:16], [o.bfloat16() for o in outs], ag[:4], master)
+        table.copy_in_scatter_out(flat, [o.bfloat16() for o in outs], ag[:4], master)
     with pytest.raises(RuntimeError):  # in-place cast
         both = torch.zeros(16, dtype=torch.float32, device=DEV)
-        table.copy_in_scatter_out(flat[:16], [o.bfloat16() for o in outs], both.view(torch.bfloat16)[:8], both[:8])
+        table.copy_in_scatter_out(flat, [o.bfloat16() for o in outs], both.view(torch.bfloat16)[:8], both[:8])
     table.close()
+
+
+@pytest.mark.parametrize("two_waves", [False, True])
+def test_both_launches_at_both_workgroup_sizes(nat, two_waves):
+    """Tables above the size threshold run two waves per workgroup (gather-in side always, scatter-out side unless
+    every tensor starts on a cache line): the shared launches follow the table."""
+    default = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
+    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0 if two_waves else default)
+    try:
+        for p in (5, 40):
+            rng = np.random.default_rng(70 + p)
+            numels = _numels(rng, p, 13, True)
+            t, pad = sum(numels), 24
+            g = torch.Generator().manual_seed(71 + p)
+            gathered = mixed_values(g, t + pad, torch.bfloat16)
+            master = mixed_values(g, 5000, torch.float32)
+            grads = [mixed_values(g, n, torch.bfloat16, 1e-3) for n in numels]
+            old = mixed_values(g, t + pad, torch.bfloat16, 1e-3)
+            shard0 = mixed_values(g, t + pad, torch.float32, 1e-3, specials=False)
+            table = nat.TensorTable(numels, t + pad, torch.device(DEV))
+            got = [torch.full((n,), 3.0, dtype=torch.bfloat16, device=DEV) for n in numels]
+            ag = torch.zeros(5000, dtype=torch.bfloat16, device=DEV)
+            assert table.copy_in_scatter_out(gathered.to(DEV), got, ag, master.to(DEV))
+            want_ag = torch.zeros(5000, dtype=torch.bfloat16)
+            torch_ops.copy_in(want_ag, master)
+            assert_bits_equal(ag, want_ag, "all-gather input")
+            want = [torch.empty(n, dtype=torch.bfloat16) for n in numels]
+            torch_ops.copy_out_materialize(gathered, numels, want)
+            for i, (a, b) in enumerate(zip(got, want)):
+                assert_bits_equal(a, b, f"tensor {i}")
+            want_flat = old.clone()
+            torch_ops.reduce_copy_in(list(want_flat[:t].split(numels)), grads, False)
+            want_flat[t:].zero_()
+            want_shard = shard0.clone()
+            torch_ops.reduce_scatter_local(want_shard, want_flat.clone(), 1, 0, None, None, "add")
+            got_flat, got_shard = old.to(DEV), shard0.to(DEV)
+            assert table.gather_in_post_reduce([x.to(DEV) for x in grads], got_flat, got_shard, True)
+            assert_bits_equal(got_flat, want_flat, "reduce buffer")
+            assert_bits_equal(got_shard, want_shard, "gradient shard")
+            table.close()
+    finally:
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default)
 
 
 # --------------------------------------------- reduce copy-in + post-reduce --
@@ -184,23 +224,44 @@ def test_gather_in_post_reduce(nat, case, grad_dt, rs_dt, shard_dt, acc, zero_pa
 
 
 def test_gather_in_post_reduce_declines_and_errors(nat):
-    numels = [5] * 17
-    table = nat.TensorTable(numels, 96, torch.device(DEV))
-    grads = [torch.ones(5, dtype=torch.bfloat16, device=DEV) for _ in numels]
+    grads = [torch.ones(40, dtype=torch.bfloat16, device=DEV) for _ in range(2)]
     flat = torch.zeros(96, dtype=torch.bfloat16, device=DEV)
     shard = torch.zeros(96, dtype=torch.float32, device=DEV)
-    assert table.gather_in_post_reduce(grads, flat, shard, False) is False
-    torch.cuda.synchronize()
-    assert float(shard.abs().sum()) == 0.0
-    table.close()
     table = nat.TensorTable([40, 40], 96, torch.device(DEV))
     # float32 gradients into a bf16 reduce buffer: not in the list of the fused launch
-    assert table.gather_in_post_reduce([g.float().repeat(8) for g in grads[:2]], flat, shard, False) is False
+    assert table.gather_in_post_reduce([g.float() for g in grads], flat, shard, False) is False
+    torch.cuda.synchronize()
+    assert float(shard.abs().sum()) == 0.0 and float(flat.float().abs().sum()) == 0.0
     with pytest.raises(ValueError):
-        table.gather_in_post_reduce([g.repeat(8) for g in grads[:2]], flat, shard[:95], False)
+        table.gather_in_post_reduce(grads, flat, shard[:95], False)
     with pytest.raises(RuntimeError):  # shard not 16-byte aligned
         wide = torch.zeros(97, dtype=torch.float32, device=DEV)
-        table.gather_in_post_reduce([g.repeat(8) for g in grads[:2]], flat, wide[1:], False)
+        table.gather_in_post_reduce(grads, flat, wide[1:], False)
+    with pytest.raises(RuntimeError):  # shard inside the reduce buffer
+        both = torch.zeros(96, dtype=torch.float32, device=DEV)
+        table.gather_in_post_reduce([g.float() for g in grads], both, both, False)
+    table.close()
+
+
+def test_changing_pointer_sets_on_a_large_table(nat):
+    """A table with more than 16 tensors stages its per-call pointers: unchanged and changed sets alternate, every
+    call against the oracle."""
+    rng = np.random.default_rng(81)
+    numels = _numels(rng, 60, 10, True)
+    t = sum(numels)
+    g = torch.Generator().manual_seed(82)
+    table = nat.TensorTable(numels, t + 16, torch.device(DEV))
+    shard_cpu = torch.zeros(t + 16, dtype=torch.float32)
+    shard = shard_cpu.to(DEV)
+    flat = torch.zeros(t + 16, dtype=torch.bfloat16, device=DEV)
+    flat_cpu = torch.zeros(t + 16, dtype=torch.bfloat16)
+    sets = [[mixed_values(g, n, torch.bfloat16, 1e-3, specials=False) for n in numels] for _ in range(3)]
+    dsets = [[x.to(DEV) for x in s_] for s_ in sets]
+    for k in (0, 0, 1, 0, 2, 2, 1):
+        assert table.gather_in_post_reduce(dsets[k], flat, shard, True)
+        torch_ops.reduce_copy_in(list(flat_cpu[:t].split(numels)), sets[k], False)
+        torch_ops.reduce_scatter_local(shard_cpu, flat_cpu.clone(), 1, 0, None, None, "add")
+        assert_bits_equal(shard, shard_cpu, f"gradient shard after set {k}")
     table.close()
 
 

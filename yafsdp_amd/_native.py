@@ -469,8 +469,8 @@ class TensorTable:
         modes: Sequence[int] | None = None,
     ) -> bool:
         """``flat_copy(ag_in, master)`` and ``scatter_out(flat, tensors)`` as ONE launch (two independent jobs in
-        one grid).  Returns False without launching anything when the library does not serve this table that way
-        (more than 16 tensors); the caller then makes the two calls."""
+        one grid).  Returns False without launching anything when the tensors' dtype differs from the gathered
+        buffer's (``scatter_out`` casts; this launch does not); the caller then makes the two calls."""
         _flat_arg(flat, "flat"), _flat_arg(ag_in, "ag_in"), _flat_arg(master, "master")
         if flat.numel() < self.total_numel:
             raise ValueError(f"flat buffer holds {flat.numel()} elements, table needs {self.total_numel}")
@@ -480,10 +480,12 @@ class TensorTable:
             tdt = self._fill(tensors, modes, "tensors")
             if tdt >= 0 and tdt != _dt(flat):
                 return False
-            code = lib.yafsdp_copy_in_scatter_out(
-                self._handle, flat.data_ptr(), _dt(flat), self._ptrs_addr, self._modes_addr,
-                ag_in.data_ptr(), master.data_ptr(), _dt(master), master.numel(), _stream(flat),
-            )
+            args = (self._handle, flat.data_ptr(), _dt(flat), self._ptrs_addr, self._modes_addr,
+                    ag_in.data_ptr(), master.data_ptr(), _dt(master), master.numel(), _stream(flat))
+            code = lib.yafsdp_copy_in_scatter_out(*args)
+            if code == ERR_BUSY:  # back-pressure, as in gather_in
+                torch.cuda.current_stream(self.device).synchronize()
+                code = lib.yafsdp_copy_in_scatter_out(*args)
         if code == ERR_UNSUPPORTED:
             return False
         _check(code, "yafsdp_copy_in_scatter_out")
@@ -495,7 +497,8 @@ class TensorTable:
     ) -> bool:
         """Reduce copy-in into ``flat`` and post-reduce of the whole buffer into ``shard`` as ONE launch: what a
         shard group of size one does between backward and optimizer (no collective in between, no divide).
-        Returns False without launching anything when the library does not serve this table / dtype combination."""
+        Returns False without launching anything when the library does not serve the dtype combination (a reduce
+        buffer that has neither the gradients' dtype nor float32)."""
         _flat_arg(flat, "flat"), _flat_arg(shard, "shard")
         if flat.numel() < self.padded_numel or shard.numel() != self.padded_numel:
             raise ValueError(f"flat / shard hold {flat.numel()} / {shard.numel()} elements, table needs {self.padded_numel}")
@@ -503,10 +506,12 @@ class TensorTable:
             tdt = self._fill(tensors, modes, "tensors")
             if tdt < 0:
                 tdt = _dt(flat)
-            code = lib.yafsdp_gather_in_post_reduce(
-                self._handle, self._ptrs_addr, self._modes_addr, tdt, flat.data_ptr(), _dt(flat),
-                int(bool(zero_pad)), shard.data_ptr(), _dt(shard), int(bool(accumulate)), _stream(flat),
-            )
+            args = (self._handle, self._ptrs_addr, self._modes_addr, tdt, flat.data_ptr(), _dt(flat),
+                    int(bool(zero_pad)), shard.data_ptr(), _dt(shard), int(bool(accumulate)), _stream(flat))
+            code = lib.yafsdp_gather_in_post_reduce(*args)
+            if code == ERR_BUSY:  # back-pressure, as in gather_in
+                torch.cuda.current_stream(self.device).synchronize()
+                code = lib.yafsdp_gather_in_post_reduce(*args)
         if code == ERR_UNSUPPORTED:
             return False
         _check(code, "yafsdp_gather_in_post_reduce")

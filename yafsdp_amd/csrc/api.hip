@@ -306,8 +306,8 @@ const char* yafsdp_error_string(int code) {
     case YAFSDP_ERR_WRONG_DEVICE: return "yafsdp: table belongs to another device than the current one";
     case YAFSDP_ERR_OUT_OF_MEMORY: return "yafsdp: host allocation failed";
     case YAFSDP_ERR_UNSUPPORTED:
-      return "yafsdp: this fused entry point does not serve the table or dtype combination (more than 16 tensors, or "
-             "dtypes outside its list): use the two separate entry points";
+      return "yafsdp: this fused entry point does not serve the dtype combination (a reduce buffer that has neither "
+             "the gradients' dtype nor binary32): use the two separate entry points";
     case YAFSDP_ERR_BUSY:
       return "yafsdp: every staging slot of this table is still in use by a queued call (more than 8 different "
              "tensor sets in flight): synchronise the stream, or bind tensor sets that persist";
@@ -971,7 +971,6 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   if (table == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (!valid_dtype(flat_dtype) || !valid_dtype(master_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && (ag_in == nullptr || master == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
-  if (table->n_tensors > kSmallMax || (table->scatter_shape >> 4) != kTableBlockSmall) return YAFSDP_ERR_UNSUPPORTED;
   if (table->total > 0 && (flat == nullptr || tensor_ptrs == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (table->total > 0 && !aligned_to(flat, 16)) return YAFSDP_ERR_MISALIGNED;
   if (n > 0 && (!aligned_to(ag_in, item_size(flat_dtype)) || !aligned_to(master, item_size(master_dtype))))
@@ -990,20 +989,35 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
     const int rc = check_dyn(table, ptrs, mode, item_size(flat_dtype));
     if (rc != YAFSDP_OK) return rc;
   }
-  SmallMeta meta;
-  static const void* const kNoPtrs[kSmallMax] = {};
-  fill_small(table, table->total > 0 ? ptrs : kNoPtrs, mode, &meta);
+  const int block = table->scatter_shape >> 4;  // the whole grid has the scatter-out workgroup size
   int64_t head = n > 0 ? ((16 - (reinterpret_cast<uintptr_t>(ag_in) & 15)) & 15) / item_size(flat_dtype) : 0;
   if (head > n) head = n;
-  const int64_t flat_tile = int64_t(kTableBlockSmall) * kFusedFlatUnroll;  // units per workgroup of the flat job
+  const int64_t flat_tile = int64_t(block) * kFusedFlatUnroll;  // units per workgroup of the flat job
   int64_t n_flat_blocks = n > 0 ? (((n - head) >> 3) + flat_tile - 1) / flat_tile : 0;
   if (n > 0 && n_flat_blocks < 1) n_flat_blocks = 1;  // workgroup 0 of the flat job peels head and tail
   const int64_t n_slots = table->total > 0 ? table->n_slots : 0;
   const int64_t grid = n_flat_blocks + table_blocks(n_slots);
   if (grid == 0) return YAFSDP_OK;
   if (grid > int64_t(INT32_MAX) - 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
-  return int(launch_unshard(table->scatter_shape & 15, master_dtype, flat_dtype, meta, flat, int(n_slots), ag_in, master,
-                            n, int(head), int(n_flat_blocks), int(grid), static_cast<hipStream_t>(stream)));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (table->n_tensors <= kSmallMax) {
+    SmallMeta meta;
+    static const void* const kNoPtrs[kSmallMax] = {};
+    fill_small(table, table->total > 0 ? ptrs : kNoPtrs, mode, &meta);
+    return int(launch_unshard<SmallMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots),
+                                         ag_in, master, n, int(head), int(n_flat_blocks), int(grid), s));
+  }
+  if (table->total == 0)  // nothing to split: the cast alone
+    return flat_launch(master_dtype, flat_dtype, SCALE_NONE, false, ag_in, master, n, 1.0f, s);
+  std::lock_guard<std::mutex> lock(table->mu);
+  LargeMeta meta;
+  int slot = -1;
+  const int rc = stage_large(table, ptrs, mode, &meta, &slot, s);
+  if (rc != YAFSDP_OK) return rc;
+  e = launch_unshard<LargeMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots), ag_in, master,
+                                n, int(head), int(n_flat_blocks), int(grid), s);
+  if (e != hipSuccess) return int(e);
+  return finish_large(table, slot, s);
 }
 
 int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
@@ -1012,7 +1026,7 @@ int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_
   if (table == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (!valid_dtype(tensor_dtype) || !valid_dtype(flat_dtype) || !valid_dtype(shard_dtype))
     return YAFSDP_ERR_UNSUPPORTED_DTYPE;
-  if (table->n_tensors > kSmallMax || !fused_reduce_supports(tensor_dtype, flat_dtype)) return YAFSDP_ERR_UNSUPPORTED;
+  if (!fused_reduce_supports(tensor_dtype, flat_dtype)) return YAFSDP_ERR_UNSUPPORTED;
   if (table->padded == 0) return YAFSDP_OK;
   if (flat == nullptr || shard == nullptr || (table->n_tensors > 0 && tensor_ptrs == nullptr))
     return YAFSDP_ERR_INVALID_ARGUMENT;
@@ -1027,14 +1041,26 @@ int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return int(e);
   if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
-  const int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
+  int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
-  SmallMeta meta;
-  fill_small(table, tensor_ptrs, mode, &meta);
+  hipStream_t s = static_cast<hipStream_t>(stream);
   const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  return int(launch_gather_post(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard, table->padded,
-                                table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, grid,
-                                static_cast<hipStream_t>(stream)));
+  if (table->n_tensors <= kSmallMax) {
+    SmallMeta meta;
+    fill_small(table, tensor_ptrs, mode, &meta);
+    return int(launch_gather_post<SmallMeta>(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard,
+                                             table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, grid,
+                                             s));
+  }
+  std::lock_guard<std::mutex> lock(table->mu);
+  LargeMeta meta;
+  int slot = -1;
+  rc = stage_large(table, tensor_ptrs, mode, &meta, &slot, s);
+  if (rc != YAFSDP_OK) return rc;
+  e = launch_gather_post<LargeMeta>(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard,
+                                    table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, grid, s);
+  if (e != hipSuccess) return int(e);
+  return finish_large(table, slot, s);
 }
 
 int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, void* const* tensor_ptrs,

@@ -17,24 +17,25 @@
 //    the reduce buffer written as they would leave it.  No divide: at size one
 //    the reference's factors are absent or 1 (ya_fsdp/_collectives.py:221-267).
 //
-// Both serve tables of at most kSmallMax tensors (metadata in the kernel
-// arguments).  Lanes of gather_post_kernel always take the quad arrangement
-// (elem.hip.h): the gradient shard is binary32 in the usual case.
+// META is SmallMeta (at most kSmallMax tensors: metadata in the kernel arguments)
+// or LargeMeta (records and per-call pointers in device memory), as in the
+// kernels they stand for.  Lanes of gather_post_kernel always take the quad
+// arrangement (elem.hip.h): the gradient shard is binary32 in the usual case.
 #pragma once
 #include "table_kernels.hip.h"
 
 namespace yafsdp {
 
 // M: master dtype, P: dtype of the all-gather input, of the gathered buffer and of the tensors.
-template <class M, class P, int BLOCK, int UF, int US, bool NTL, int STP_FLAT, int STP_SCATTER>
+template <class META, class M, class P, int BLOCK, int UF, int US, bool NTL, int STP_FLAT, int STP_SCATTER>
 __global__ void __launch_bounds__(BLOCK)
-unshard_kernel(SmallMeta meta, const void* gathered, int n_slots, void* ag_in, const void* master, int64_t n, int head,
+unshard_kernel(META meta, const void* gathered, int n_slots, void* ag_in, const void* master, int64_t n, int head,
                int n_flat_blocks) {
   const int b = blockIdx.x;
   if (b < n_flat_blocks) {
     flat_body<M, P, SCALE_NONE, false, BLOCK, UF, NTL, STP_FLAT>(ag_in, master, n, head, 1.0f, b, n_flat_blocks);
   } else {
-    scatter_body<SmallMeta, P, P, BLOCK, US, NTL, STP_SCATTER>(meta, gathered, n_slots, b - n_flat_blocks,
+    scatter_body<META, P, P, BLOCK, US, NTL, STP_SCATTER>(meta, gathered, n_slots, b - n_flat_blocks,
                                                               int(gridDim.x) - n_flat_blocks);
   }
 }
@@ -131,9 +132,9 @@ __device__ __forceinline__ void gather_post_segment(char* flat, const char* src,
 // S: gradient dtype, D: reduce buffer dtype, O: gradient shard dtype.  `shard` has `padded` elements like `flat`.
 // pad_zero != 0 writes zeros to the pad lanes of the reduce buffer (otherwise they stay as they are); in both cases
 // the pad lanes of the shard receive what the separate post-reduce would give them.
-template <class S, class D, class O, int BLOCK, int U, bool NTL>
+template <class META, class S, class D, class O, int BLOCK, int U, bool NTL>
 __global__ void __launch_bounds__(BLOCK)
-gather_post_kernel(SmallMeta meta, void* flat, void* shard, int64_t padded, int n_tiles, int pad_zero, int accumulate) {
+gather_post_kernel(META meta, void* flat, void* shard, int64_t padded, int n_tiles, int pad_zero, int accumulate) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   char* fbase = reinterpret_cast<char*>(flat);
   char* obase = reinterpret_cast<char*>(shard);

@@ -54,16 +54,19 @@ template <class META>
 hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total,
                           int n_tiles, int grid, hipStream_t stream);
 
-// the two fused launches (fused.hip), tables of at most kSmallMax tensors.  launch_unshard: the first
-// n_flat_blocks workgroups of the grid cast master[0:n] into ag_in, the others run the scatter-out tile slots
-// (`scatter_unroll`: units per lane the table's slots were built for; workgroups of kTableBlockSmall lanes).
+// the two fused launches (fused.hip).  launch_unshard: the first n_flat_blocks workgroups of the grid cast
+// master[0:n] into ag_in (tiles of workgroup size * kFusedFlatUnroll units), the others run the scatter-out tile
+// slots; `scatter_shape` is the table's (workgroup size * 16 + units per lane), and the whole grid has its
+// workgroup size.
 constexpr int kFusedFlatUnroll = 2;
-hipError_t launch_unshard(int scatter_unroll, int master_dt, int param_dt, const SmallMeta& meta, const void* gathered,
+template <class META>
+hipError_t launch_unshard(int scatter_shape, int master_dt, int param_dt, const META& meta, const void* gathered,
                           int n_slots, void* ag_in, const void* master, int64_t n, int head, int n_flat_blocks,
                           int grid, hipStream_t stream);
 // reduce copy-in + post-reduce of a size-1 shard group; `block`: the table's gather-in workgroup size
 bool fused_reduce_supports(int tensor_dt, int flat_dt);
-hipError_t launch_gather_post(int block, int tensor_dt, int flat_dt, int shard_dt, const SmallMeta& meta, void* flat,
+template <class META>
+hipError_t launch_gather_post(int block, int tensor_dt, int flat_dt, int shard_dt, const META& meta, void* flat,
                               void* shard, int64_t padded, int n_tiles, int pad_zero, int acc, int grid,
                               hipStream_t stream);
 
