@@ -129,6 +129,88 @@ def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bou
     table.close()
 
 
+@settings(max_examples=80, **COMMON)
+@given(numels=tables, pad=st.integers(0, 700), master_dt=st.sampled_from(DTYPES), param_dt=st.sampled_from(DTYPES),
+       shard_n=st.integers(0, 9000), two_waves=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2))
+def test_copy_in_scatter_out_any_table(nat, numels, pad, master_dt, param_dt, shard_n, two_waves, seed, tile_mode):
+    """Copy-in and copy-out as one launch: both halves with their guard lanes against the oracle."""
+    print("copy_in_scatter_out", numels, pad, master_dt, param_dt, shard_n, two_waves, seed, tile_mode, flush=True)
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    p, t = len(numels), sum(numels)
+    gathered = mixed_values(g, t + pad, param_dt)
+    master = mixed_values(g, shard_n, master_dt)
+    modes = rng.integers(0, 2, size=p).tolist()
+    offs = [int(rng.integers(0, 8)) for _ in numels]
+    bufs, views = zip(*[_view_at(torch.full((n,), 3.0, dtype=param_dt), o) for n, o in zip(numels, offs)])
+    m_buf, m_view = _view_at(master, int(rng.integers(0, 4)))
+    a_off = int(rng.integers(0, 8))
+    a_buf, a_view = _view_at(torch.full((shard_n,), 3.0, dtype=param_dt), a_off)
+    default = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
+    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0 if two_waves else default)
+    nat.set_option(nat.OPT_SCATTER_TILE, tile_mode)
+    try:
+        table = nat.TensorTable(numels, t + pad, DEV)
+    finally:
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default)
+        nat.set_option(nat.OPT_SCATTER_TILE, 0)
+    assert table.copy_in_scatter_out(gathered.to(DEV), list(views), a_view, m_view, modes)
+    want_ag = torch.full((shard_n + a_off + 9,), 3.0, dtype=param_dt)
+    torch_ops.copy_in(want_ag[a_off : a_off + shard_n], master)
+    assert_bits_equal(a_buf, want_ag, "all-gather input with its guard lanes")
+    pos = 0
+    for i, n in enumerate(numels):
+        ref = torch.full((n + offs[i] + 9,), 3.0, dtype=param_dt)
+        if modes[i]:
+            ref[offs[i] : offs[i] + n].copy_(gathered[pos : pos + n])
+        assert_bits_equal(bufs[i], ref, f"tensor {i} with its guard lanes")
+        pos += n
+    table.close()
+
+
+@settings(max_examples=100, **COMMON)
+@given(numels=tables, pad=st.integers(0, 700), grad_dt=st.sampled_from(DTYPES), wide_buffer=st.booleans(),
+       shard_dt=st.sampled_from(DTYPES), acc=st.booleans(), two_waves=st.booleans(), zero_pad=st.booleans(),
+       seed=st.integers(0, 2**20))
+def test_gather_in_post_reduce_any_table(nat, numels, pad, grad_dt, wide_buffer, shard_dt, acc, two_waves, zero_pad, seed):
+    """Reduce copy-in and post-reduce of a size-one group as one launch: the reduce buffer (guard lanes included)
+    and the gradient shard against the reference's op sequence."""
+    rs_dt = torch.float32 if wide_buffer else grad_dt
+    print("gather_in_post_reduce", numels, pad, grad_dt, rs_dt, shard_dt, acc, two_waves, zero_pad, seed, flush=True)
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    p, t = len(numels), sum(numels)
+    t_pad = t + pad
+    grads = [mixed_values(g, n, grad_dt, 1e-3) for n in numels]
+    modes = rng.integers(0, 3, size=p).tolist()
+    old = torch.zeros(t_pad + 8, dtype=rs_dt)
+    old[:t_pad] = mixed_values(g, t_pad, rs_dt, 1e-3).flip(0)
+    old[t_pad:] = 5.0
+    shard0 = mixed_values(g, t_pad, shard_dt, 1e-3, specials=False)
+    want = old.clone()
+    views = list(want[:t].split(numels))
+    cp = [i for i, m in enumerate(modes) if m == 1]
+    ad = [i for i, m in enumerate(modes) if m == 2]
+    torch_ops.reduce_copy_in([views[i] for i in cp], [grads[i] for i in cp], False)
+    torch_ops.reduce_copy_in([views[i] for i in ad], [grads[i] for i in ad], True)
+    if zero_pad:
+        want[t:t_pad] = 0
+    want_shard = shard0.clone()
+    torch_ops.reduce_scatter_local(want_shard, want[:t_pad].clone(), 1, 0, None, None, "add" if acc else "copy")
+    default = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
+    nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0 if two_waves else default)
+    try:
+        table = nat.TensorTable(numels, t_pad, DEV)
+    finally:
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default)
+    got, got_shard = old.to(DEV), shard0.to(DEV)
+    dgrads = [_view_at(x, int(rng.integers(0, 8)))[1] for x in grads]
+    assert table.gather_in_post_reduce(dgrads, got, got_shard, acc, modes, zero_pad=zero_pad)
+    assert_bits_equal(got, want, "reduce buffer")
+    assert_bits_equal(got_shard, want_shard, "gradient shard")
+    table.close()
+
+
 # ------------------------------------------------------------ optimizer side --
 @settings(max_examples=80, **COMMON)
 @given(n=st.integers(1, 40_000), off=st.integers(0, 3), decoupled=st.booleans(),
