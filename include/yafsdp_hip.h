@@ -189,24 +189,29 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
                                void* stream);
 
 /* Reduce copy-in and post-reduce of a shard group of size ONE as one pass.
- * There the rank's chunk of the reduce buffer is the whole buffer and nothing
- * happens between the two steps (ya_fsdp/_collectives.py:140-150: the
- * "reduce-scatter" copies the buffer onto itself), so per element
+ * There the rank's chunk of the reduce buffer is the whole buffer and the
+ * "reduce-scatter" copies the buffer onto itself (ya_fsdp/_collectives.py:
+ * 140-150), so per element
  *   flat  = COPY: cast(tensor) | ADD: round(flat + tensor) | SKIP: flat
  *           (ya_fsdp/_param_group.py:693-708; pad lanes: 0 if zero_pad)
- *   shard = accumulate ? round(shard + flat) : cast(flat)
- *           (ya_fsdp/_collectives.py:185 / :189)
- * with the same two roundings and the same contents of `flat` afterwards as
- * yafsdp_gather_in followed by yafsdp_post_reduce.  No divide factors: at size
- * one the reference's are absent or 1.  `shard` has the table's padded element
- * count.  Both buffers 16-byte aligned.  `flat` has the tensors' dtype or
- * binary32; YAFSDP_ERR_UNSUPPORTED otherwise, with nothing launched (the two
- * separate entry points serve every combination).  The reduce buffer is not
- * read back: 12 instead of 14 bytes per element for bf16 gradients, a bf16
- * buffer and a binary32 shard that accumulates. */
+ *   flat  = round(flat / pre_factor)      if pre_factor > 1        (:139)
+ *   flat  = round(flat / custom_divisor)  if custom_divisor != 0   (:146-148;
+ *           any divisor, as yafsdp_flat_div_copy; excludes the other two)
+ *   chunk = round(flat / post_factor)     if post_factor > 1       (:165)
+ *   shard = accumulate ? round(shard + chunk) : cast(chunk)        (:185 / :189)
+ * with the roundings and the contents of `flat` afterwards (everything up to
+ * the post-divide, which only the shard sees) that yafsdp_gather_in,
+ * yafsdp_flat_div_copy and yafsdp_post_reduce give in a row.  Pass 0 for an
+ * absent factor.  `shard` has the table's padded element count.  Both buffers
+ * 16-byte aligned.  `flat` has the tensors' dtype or binary32;
+ * YAFSDP_ERR_UNSUPPORTED otherwise, with nothing launched (the separate entry
+ * points serve every combination).  The reduce buffer is not read back: 12
+ * instead of 14 bytes per element for bf16 gradients, a bf16 buffer and a
+ * binary32 shard that accumulates. */
 int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
-                                 int tensor_dtype, void* flat, int flat_dtype, int zero_pad, void* shard,
-                                 int shard_dtype, int accumulate, void* stream);
+                                 int tensor_dtype, void* flat, int flat_dtype, double pre_factor, double custom_divisor,
+                                 double post_factor, int zero_pad, void* shard, int shard_dtype, int accumulate,
+                                 void* stream);
 
 /* ---- the two exchange points, over several buffers ------------------------------
  * One GPU: all buffers are local.  With peer-mapped pointers the same two calls

@@ -223,6 +223,62 @@ def test_gather_in_post_reduce(nat, case, grad_dt, rs_dt, shard_dt, acc, zero_pa
     table.close()
 
 
+@pytest.mark.parametrize("case", [CASES[2], CASES[4], CASES[6]])
+@pytest.mark.parametrize("grad_dt,rs_dt,shard_dt", [
+    (torch.bfloat16, torch.bfloat16, torch.float32),
+    (torch.float16, torch.float16, torch.float32),
+    (torch.bfloat16, torch.float32, torch.bfloat16),
+])
+@pytest.mark.parametrize("factors", [
+    # (pre, custom, post)
+    (None, None, 8.0), (None, None, 3.0), (4.0, None, 2.0), (16.0, None, 16.0), (3.0, None, None),
+    (None, 4.0, None), (None, 3.0, None), (None, 0.5, None), (None, -7.0, None), (None, 1.0, None), (1.0, None, 0.5),
+])
+@pytest.mark.parametrize("acc", [False, True])
+def test_gather_in_post_reduce_with_divide_factors(nat, case, grad_dt, rs_dt, shard_dt, factors, acc):
+    """The divides of the reduce step inside the one-pass reduce: the pre-divide and the custom division act on the
+    reduce buffer in place (ya_fsdp/_collectives.py:139, 146-148), the post-divide on what goes on to the shard
+    (:165); each rounds to the buffer's dtype.  Against the op sequence and against the separate entry points."""
+    pre, custom, post = factors
+    rng, numels = _case_numels(case, 13)
+    p, pad = len(numels), case[3]
+    t = sum(numels)
+    t_pad = t + pad
+    g = torch.Generator().manual_seed(331 + p)
+    _say("gather_in_post_reduce factors", case, grad_dt, rs_dt, shard_dt, factors, acc)
+    grads = [mixed_values(g, n, grad_dt, 1e-3) for n in numels]
+    modes = rng.integers(0, 3, size=p).tolist()
+    old = mixed_values(g, t_pad, rs_dt, 1e-3).flip(0).contiguous()
+    shard0 = mixed_values(g, t_pad, shard_dt, 1e-3, specials=False)
+    want_flat = old.clone()
+    views = list(want_flat[:t].split(numels))
+    cp = [i for i, m in enumerate(modes) if m == 1]
+    ad = [i for i, m in enumerate(modes) if m == 2]
+    torch_ops.reduce_copy_in([views[i] for i in cp], [grads[i] for i in cp], False)
+    torch_ops.reduce_copy_in([views[i] for i in ad], [grads[i] for i in ad], True)
+    want_flat[t:].zero_()
+    torch_ops.div_if_needed(want_flat, pre)                      # :139
+    if custom is not None:
+        want_flat.copy_(want_flat / custom)                      # :146-148 (output aliases the input at size one)
+    want_shard = shard0.clone()
+    torch_ops.reduce_scatter_local(want_shard, want_flat.clone(), 1, 0, None, post, "add" if acc else "copy")
+    table = nat.TensorTable(numels, t_pad, torch.device(DEV))
+    dgrads = [x.to(DEV) for x in grads]
+    got_flat, got_shard = old.to(DEV), shard0.to(DEV)
+    assert table.gather_in_post_reduce(dgrads, got_flat, got_shard, acc, modes, pre_factor=pre, post_factor=post,
+                                       custom_divisor=custom)
+    assert_bits_equal(got_flat, want_flat, "reduce buffer (before the post-divide)")
+    assert_bits_equal(got_shard, want_shard, "gradient shard")
+    two_flat, two_shard = old.to(DEV), shard0.to(DEV)
+    table.gather_in(dgrads, two_flat, modes, pre, zero_pad=True)
+    if custom is not None:
+        nat.flat_div_copy(two_flat, two_flat, custom)
+    nat.post_reduce(two_shard, two_flat, post, acc)
+    assert_bits_equal(got_flat, two_flat, "reduce buffer against the separate calls")
+    assert_bits_equal(got_shard, two_shard, "gradient shard against the separate calls")
+    table.close()
+
+
 def test_gather_in_post_reduce_declines_and_errors(nat):
     grads = [torch.ones(40, dtype=torch.bfloat16, device=DEV) for _ in range(2)]
     flat = torch.zeros(96, dtype=torch.bfloat16, device=DEV)
@@ -240,6 +296,10 @@ def test_gather_in_post_reduce_declines_and_errors(nat):
     with pytest.raises(RuntimeError):  # shard inside the reduce buffer
         both = torch.zeros(96, dtype=torch.float32, device=DEV)
         table.gather_in_post_reduce([g.float() for g in grads], both, both, False)
+    with pytest.raises(RuntimeError):  # the custom division excludes the other two factors
+        table.gather_in_post_reduce(grads, flat, shard, False, pre_factor=2.0, custom_divisor=3.0)
+    with pytest.raises(RuntimeError):
+        table.gather_in_post_reduce(grads, flat, shard, False, custom_divisor=float("inf"))
     table.close()
 
 

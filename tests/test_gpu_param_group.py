@@ -252,6 +252,46 @@ def test_size_one_group_reduces_in_one_launch(monkeypatch):
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard after the partial backward")
 
 
+@pytest.mark.parametrize("policy,factor,force_sum,want", [
+    ("bf16", 3.0, False, (None, 3.0, None)),     # custom factor: the out-of-place division (:141-148)
+    ("bf16", 4.0, True, (None, None, 4.0)),      # forced sum reduction: post-divide only
+    ("fp16", 8.0, False, (4.0, None, 2.0)),      # fp16 reduce: pre- and post-divide
+])
+def test_size_one_group_divides_inside_the_one_launch(monkeypatch, policy, factor, force_sum, want):
+    from yafsdp_amd import _native
+
+    seen = []
+    real = _native.TensorTable.gather_in_post_reduce
+
+    def spy(self, *a, **k):
+        served = real(self, *a, **k)
+        seen.append((served, k.get("pre_factor"), k.get("custom_divisor"), k.get("post_factor")))
+        return served
+
+    monkeypatch.setattr(_native.TensorTable, "gather_in_post_reduce", spy)
+    dt = torch.bfloat16 if policy == "bf16" else torch.float16
+    mp = MixedPrecisionPolicy(param_dtype=dt)
+    shapes, w, r, align = ODD_SHAPES, 1, 0, 8
+    group, cpu_params = _make_group(shapes, w, r, align, mp)
+    group.gradient_divide_factor = factor
+    group.force_sum_reduction_for_comms = force_sum
+    ref = CpuGroup(cpu_params, w, r, align, mp)
+    pre, custom, post = want
+    for it in range(2):
+        group.pre_forward(); group.post_forward(); group.pre_backward()
+        _run_backward(group, ref, _grads(shapes, dt, 70 + it))
+        torch_ops.div_if_needed(ref.rs, pre)
+        if custom is not None:
+            ref.rs.copy_(ref.rs / custom)
+        rs_before_post = ref.rs.clone()
+        ref.reduce(None, post, "copy" if it == 0 else "add")
+        group.finalize_backward()
+        torch.cuda.synchronize()
+        assert seen[-1] == (True, pre, custom, post)
+        assert_bits_equal(group._reduce_scatter_input[None], rs_before_post, "reduce buffer")
+        assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, f"grad shard after backward {it}")
+
+
 def test_mixed_params_with_and_without_sharded_grad(monkeypatch):
     from yafsdp_amd import _native
 

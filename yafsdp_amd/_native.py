@@ -115,7 +115,7 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_copy_in_scatter_out.restype = i32
     lib.yafsdp_copy_in_scatter_out.argtypes = [vp, vp, i32, vp, vp, vp, vp, i32, i64, vp]
     lib.yafsdp_gather_in_post_reduce.restype = i32
-    lib.yafsdp_gather_in_post_reduce.argtypes = [vp, vp, vp, i32, vp, i32, i32, vp, i32, i32, vp]
+    lib.yafsdp_gather_in_post_reduce.argtypes = [vp, vp, vp, i32, vp, i32, dbl, dbl, dbl, i32, vp, i32, i32, vp]
     lib.yafsdp_flat_copy_fanout.restype = i32
     lib.yafsdp_flat_copy_fanout.argtypes = [vp, i32, i32, vp, i32, i64, vp]
     lib.yafsdp_post_reduce_fanin.restype = i32
@@ -493,12 +493,15 @@ class TensorTable:
 
     def gather_in_post_reduce(
         self, tensors: Sequence[torch.Tensor | None], flat: torch.Tensor, shard: torch.Tensor, accumulate: bool,
-        modes: Sequence[int] | None = None, zero_pad: bool = True,
+        modes: Sequence[int] | None = None, zero_pad: bool = True, pre_factor: float | None = None,
+        post_factor: float | None = None, custom_divisor: float | None = None,
     ) -> bool:
         """Reduce copy-in into ``flat`` and post-reduce of the whole buffer into ``shard`` as ONE launch: what a
-        shard group of size one does between backward and optimizer (no collective in between, no divide).
-        Returns False without launching anything when the library does not serve the dtype combination (a reduce
-        buffer that has neither the gradients' dtype nor float32)."""
+        shard group of size one does between backward and optimizer (no collective in between).  ``pre_factor`` and
+        ``post_factor`` follow ``_div_if_needed`` (applied if > 1); ``custom_divisor`` is the division by a custom
+        gradient divide factor of such a group (any value; excludes the other two).  Returns False without launching
+        anything when the library does not serve the dtype combination (a reduce buffer that has neither the
+        gradients' dtype nor float32)."""
         _flat_arg(flat, "flat"), _flat_arg(shard, "shard")
         if flat.numel() < self.padded_numel or shard.numel() != self.padded_numel:
             raise ValueError(f"flat / shard hold {flat.numel()} / {shard.numel()} elements, table needs {self.padded_numel}")
@@ -507,6 +510,7 @@ class TensorTable:
             if tdt < 0:
                 tdt = _dt(flat)
             args = (self._handle, self._ptrs_addr, self._modes_addr, tdt, flat.data_ptr(), _dt(flat),
+                    _factor(pre_factor), _factor(custom_divisor), _factor(post_factor),
                     int(bool(zero_pad)), shard.data_ptr(), _dt(shard), int(bool(accumulate)), _stream(flat))
             code = lib.yafsdp_gather_in_post_reduce(*args)
             if code == ERR_BUSY:  # back-pressure, as in gather_in

@@ -507,13 +507,13 @@ class YaFSDPParamGroup:
 
     def _reduce_in_one_launch(self, grads: "list[torch.Tensor | None]", modes: "list[int]") -> bool:
         """A shard group of size ONE whose gradients pass through the reduce buffer: the rank's chunk is the whole
-        buffer, the "reduce-scatter" copies it onto itself (ya_fsdp/_collectives.py:140-150) and, without a custom
-        divide factor, nothing is divided, so the reduce copy-in (ya_fsdp/_param_group.py:693-708) and the copy or
-        accumulation into the gradient shard (ya_fsdp/_collectives.py:185 / :189) run as one launch on the current
-        stream, with the same rounding points and the same contents of the reduce buffer afterwards.  Returns
-        False, having launched nothing, for every other case; the caller then takes the general route."""
+        buffer and the "reduce-scatter" copies it onto itself (ya_fsdp/_collectives.py:140-150), so the reduce
+        copy-in (ya_fsdp/_param_group.py:693-708), the divides (:139, :146-148, :165) and the copy or accumulation
+        into the gradient shard (:185 / :189) run as one launch on the current stream, with the same rounding points
+        and the same contents of the reduce buffer afterwards.  Returns False, having launched nothing, for every
+        other case; the caller then takes the general route."""
         group = self._reduce_scatter_process_group
-        if group.size() != 1 or self.gradient_divide_factor is not None or self._grad_sumsq_slot is not None:
+        if group.size() != 1 or self._grad_sumsq_slot is not None:
             return False
         if list(self._all_gather_dtype_to_fsdp_params) != [None] or self._table is None:
             return False
@@ -530,9 +530,14 @@ class YaFSDPParamGroup:
         if n_acc not in (0, len(with_grad)):
             return False
         pre, post, _, _ = _get_gradient_divide_factors(
-            group, self.reduce_scatter_dtype, None, self.force_sum_reduction_for_comms
+            group, self.reduce_scatter_dtype, self.gradient_divide_factor, self.force_sum_reduction_for_comms
         )
-        if (pre is not None and pre > 1) or (post is not None and post > 1):
+        custom = (
+            self.gradient_divide_factor
+            if self.gradient_divide_factor is not None and pre is None and post is None
+            else None
+        )  # ya_fsdp/_collectives.py:141-145
+        if custom is not None and (custom == 0 or custom != custom or abs(custom) == float("inf")):
             return False
         shard = self._padded_sharded_param_grad[None]
         if shard is None:
@@ -540,7 +545,10 @@ class YaFSDPParamGroup:
         if not _native.all_contiguous(grads):
             grads = [g if g is None or g.is_contiguous() else g.contiguous() for g in grads]
         self._grad_sumsq_token = None
-        return self._table.gather_in_post_reduce(grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes)
+        return self._table.gather_in_post_reduce(
+            grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes,
+            pre_factor=pre, post_factor=post, custom_divisor=custom,
+        )
 
     def finalize_backward(self) -> None:
         """ya_fsdp/_param_group.py:773-783."""

@@ -1021,12 +1021,22 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
 }
 
 int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_ptrs, const uint8_t* mode,
-                                 int tensor_dtype, void* flat, int flat_dtype, int zero_pad, void* shard,
-                                 int shard_dtype, int accumulate, void* stream) {
+                                 int tensor_dtype, void* flat, int flat_dtype, double pre_factor, double custom_divisor,
+                                 double post_factor, int zero_pad, void* shard, int shard_dtype, int accumulate,
+                                 void* stream) {
   if (table == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (!valid_dtype(tensor_dtype) || !valid_dtype(flat_dtype) || !valid_dtype(shard_dtype))
     return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (!fused_reduce_supports(tensor_dtype, flat_dtype)) return YAFSDP_ERR_UNSUPPORTED;
+  ReduceDivides dv = {SCALE_NONE, SCALE_NONE, 1.0f, 1.0f};
+  if (custom_divisor != 0.0) {
+    // the reference takes this branch only when neither of the other two factors exists (:141-145)
+    if (pre_factor != 0.0 || post_factor != 0.0) return YAFSDP_ERR_INVALID_ARGUMENT;
+    if (!scale_plan_any(custom_divisor, &dv.a_mode, &dv.a_k)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  } else {
+    scale_plan(pre_factor, &dv.a_mode, &dv.a_k);
+    scale_plan(post_factor, &dv.b_mode, &dv.b_k);
+  }
   if (table->padded == 0) return YAFSDP_OK;
   if (flat == nullptr || shard == nullptr || (table->n_tensors > 0 && tensor_ptrs == nullptr))
     return YAFSDP_ERR_INVALID_ARGUMENT;
@@ -1049,8 +1059,8 @@ int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_
     SmallMeta meta;
     fill_small(table, tensor_ptrs, mode, &meta);
     return int(launch_gather_post<SmallMeta>(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard,
-                                             table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, grid,
-                                             s));
+                                             table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, dv,
+                                             grid, s));
   }
   std::lock_guard<std::mutex> lock(table->mu);
   LargeMeta meta;
@@ -1058,7 +1068,7 @@ int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_
   rc = stage_large(table, tensor_ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
   e = launch_gather_post<LargeMeta>(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard,
-                                    table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, grid, s);
+                                    table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, dv, grid, s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }

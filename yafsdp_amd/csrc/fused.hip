@@ -40,35 +40,43 @@ hipError_t unshard_by_param(int p_dt, int shape, const META& meta, const void* g
 }
 
 // ---- reduce copy-in + post-reduce -------------------------------------------------------------------------------
+template <class META, class S, class D, class O, bool DIV>
+hipError_t gp_launch(int block, const META& meta, void* flat, void* shard, int64_t padded, int n_tiles, int pad_zero,
+                     int acc, const ReduceDivides& dv, int grid, hipStream_t stream) {
+  if (block == kTableBlockSmall)
+    return launch_kernel(gather_post_kernel<META, S, D, O, DIV, kTableBlockSmall, kGatherUnroll, kTableNtLoad>, grid,
+                         kTableBlockSmall, stream, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv);
+  if (block == kTableBlockLarge)
+    return launch_kernel(gather_post_kernel<META, S, D, O, DIV, kTableBlockLarge, kGatherUnroll, kTableNtLoad>, grid,
+                         kTableBlockLarge, stream, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv);
+  return hipErrorInvalidValue;
+}
+
 template <class META, class S, class D, class O>
 hipError_t gp_go(int block, const META& meta, void* flat, void* shard, int64_t padded, int n_tiles, int pad_zero,
-                 int acc, int grid, hipStream_t stream) {
-  if (block == kTableBlockSmall)
-    return launch_kernel(gather_post_kernel<META, S, D, O, kTableBlockSmall, kGatherUnroll, kTableNtLoad>, grid,
-                         kTableBlockSmall, stream, meta, flat, shard, padded, n_tiles, pad_zero, acc);
-  if (block == kTableBlockLarge)
-    return launch_kernel(gather_post_kernel<META, S, D, O, kTableBlockLarge, kGatherUnroll, kTableNtLoad>, grid,
-                         kTableBlockLarge, stream, meta, flat, shard, padded, n_tiles, pad_zero, acc);
-  return hipErrorInvalidValue;
+                 int acc, const ReduceDivides& dv, int grid, hipStream_t stream) {
+  if (dv.a_mode == SCALE_NONE && dv.b_mode == SCALE_NONE)
+    return gp_launch<META, S, D, O, false>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
+  return gp_launch<META, S, D, O, true>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
 }
 
 template <class META, class S, class D>
 hipError_t gp_by_shard(int o_dt, int block, const META& meta, void* flat, void* shard, int64_t padded, int n_tiles,
-                       int pad_zero, int acc, int grid, hipStream_t stream) {
+                       int pad_zero, int acc, const ReduceDivides& dv, int grid, hipStream_t stream) {
   switch (o_dt) {
-    case DT_F32: return gp_go<META, S, D, F32>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
-    case DT_BF16: return gp_go<META, S, D, BF16>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
-    case DT_F16: return gp_go<META, S, D, F16>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
+    case DT_F32: return gp_go<META, S, D, F32>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
+    case DT_BF16: return gp_go<META, S, D, BF16>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
+    case DT_F16: return gp_go<META, S, D, F16>(block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
   }
   return hipErrorInvalidValue;
 }
 
 template <class META, class S>
 hipError_t gp_by_flat(int d_dt, int o_dt, int block, const META& meta, void* flat, void* shard, int64_t padded,
-                      int n_tiles, int pad_zero, int acc, int grid, hipStream_t stream) {
+                      int n_tiles, int pad_zero, int acc, const ReduceDivides& dv, int grid, hipStream_t stream) {
   // the reduce buffer has the gradients' dtype or binary32 (reduce_dtype=float32)
-  if (d_dt == S::kId) return gp_by_shard<META, S, S>(o_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
-  if (d_dt == DT_F32) return gp_by_shard<META, S, F32>(o_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
+  if (d_dt == S::kId) return gp_by_shard<META, S, S>(o_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
+  if (d_dt == DT_F32) return gp_by_shard<META, S, F32>(o_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
   return hipErrorInvalidValue;
 }
 
@@ -90,12 +98,12 @@ hipError_t launch_unshard(int scatter_shape, int master_dt, int param_dt, const 
 
 template <class META>
 hipError_t launch_gather_post(int block, int tensor_dt, int flat_dt, int shard_dt, const META& meta, void* flat,
-                              void* shard, int64_t padded, int n_tiles, int pad_zero, int acc, int grid,
-                              hipStream_t stream) {
+                              void* shard, int64_t padded, int n_tiles, int pad_zero, int acc, const ReduceDivides& dv,
+                              int grid, hipStream_t stream) {
   switch (tensor_dt) {
-    case DT_F32: return gp_by_flat<META, F32>(flat_dt, shard_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
-    case DT_BF16: return gp_by_flat<META, BF16>(flat_dt, shard_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
-    case DT_F16: return gp_by_flat<META, F16>(flat_dt, shard_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, grid, stream);
+    case DT_F32: return gp_by_flat<META, F32>(flat_dt, shard_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
+    case DT_BF16: return gp_by_flat<META, BF16>(flat_dt, shard_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
+    case DT_F16: return gp_by_flat<META, F16>(flat_dt, shard_dt, block, meta, flat, shard, padded, n_tiles, pad_zero, acc, dv, grid, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -105,8 +113,8 @@ template hipError_t launch_unshard<SmallMeta>(int, int, int, const SmallMeta&, c
 template hipError_t launch_unshard<LargeMeta>(int, int, int, const LargeMeta&, const void*, int, void*, const void*,
                                               int64_t, int, int, int, hipStream_t);
 template hipError_t launch_gather_post<SmallMeta>(int, int, int, int, const SmallMeta&, void*, void*, int64_t, int, int,
-                                                  int, int, hipStream_t);
+                                                  int, const ReduceDivides&, int, hipStream_t);
 template hipError_t launch_gather_post<LargeMeta>(int, int, int, int, const LargeMeta&, void*, void*, int64_t, int, int,
-                                                  int, int, hipStream_t);
+                                                  int, const ReduceDivides&, int, hipStream_t);
 
 }  // namespace yafsdp

@@ -13,15 +13,18 @@
 //    (ya_fsdp/_collectives.py:140-150), so every element can go
 //        gradient -> (copy | add) into the reduce buffer, rounded to its dtype
 //                 -> copy | accumulate into the gradient shard, rounded to its dtype
-//    in one go, with the same two rounding points as the separate kernels and
-//    the reduce buffer written as they would leave it.  No divide: at size one
-//    the reference's factors are absent or 1 (ya_fsdp/_collectives.py:221-267).
+//    in one go, with the same rounding points as the separate kernels and the
+//    reduce buffer written as they would leave it.  The divides of the reduce
+//    step (absent at size one unless the caller asks for them,
+//    ya_fsdp/_collectives.py:221-267) are applied at run time, each with its
+//    own rounding.
 //
 // META is SmallMeta (at most kSmallMax tensors: metadata in the kernel arguments)
 // or LargeMeta (records and per-call pointers in device memory), as in the
 // kernels they stand for.  Lanes of gather_post_kernel always take the quad
 // arrangement (elem.hip.h): the gradient shard is binary32 in the usual case.
 #pragma once
+#include "launch.h"
 #include "table_kernels.hip.h"
 
 namespace yafsdp {
@@ -40,17 +43,35 @@ unshard_kernel(META meta, const void* gathered, int n_slots, void* ag_in, const 
   }
 }
 
-// One element of the fused reduce path.  MODE: how the gradient enters the reduce buffer.
-template <class S, class D, class O, int MODE>
-__device__ __forceinline__ void gather_post_elem(float s, float d_old, float o_old, bool acc, float& d_new, float& o_new) {
-  const float y = gather_elem<S, D, SCALE_NONE, MODE>(s, d_old, 1.0f);
-  d_new = round_to<D>(y);                     // what the reduce buffer holds afterwards
-  o_new = acc ? __fadd_rn(o_old, d_new) : d_new;  // caller rounds to O on store
+template <class D>
+__device__ __forceinline__ float divide_stage(float y, int mode, float k) {
+  if (mode == SCALE_MUL) return round_to<D>(apply_scale<SCALE_MUL>(y, k));
+  if (mode == SCALE_DIV) return round_to<D>(apply_scale<SCALE_DIV>(y, k));
+  return y;
 }
 
-template <class S, class D, class O, int MODE>
+// One element of the fused reduce path.  MODE: how the gradient enters the reduce buffer.
+// DIV: whether any divide is applied (the kernel without them is a separate instantiation: the division's code
+// doubles the register count, which the common case should not pay for).
+template <class S, class D, int MODE, bool DIV>
+__device__ __forceinline__ void gather_post_elem(float s, float d_old, float o_old, bool acc, const ReduceDivides& dv,
+                                                 float& d_new, float& o_new) {
+  float y;
+  if constexpr (MODE == MODE_ZERO) y = 0.f;
+  else y = round_to<D>(gather_elem<S, D, SCALE_NONE, MODE>(s, d_old, 1.0f));
+  float c;
+  if constexpr (DIV) {
+    d_new = divide_stage<D>(y, dv.a_mode, dv.a_k);  // what the reduce buffer holds afterwards
+    c = divide_stage<D>(d_new, dv.b_mode, dv.b_k);  // what the "reduce-scatter" hands on
+  } else {
+    d_new = c = y;
+  }
+  o_new = acc ? __fadd_rn(o_old, c) : c;  // caller rounds to O on store
+}
+
+template <class S, class D, class O, int MODE, bool DIV>
 __device__ __forceinline__ void gather_post_scalar(char* flat, const char* src, char* shard, int64_t i, bool acc,
-                                                   bool write_flat) {
+                                                   const ReduceDivides& dv) {
   typedef typename S::storage s_t;
   typedef typename D::storage d_t;
   typedef typename O::storage o_t;
@@ -61,24 +82,21 @@ __device__ __forceinline__ void gather_post_scalar(char* flat, const char* src, 
   if constexpr (MODE == MODE_ADD || MODE == MODE_SKIP) d_old = to_f32<D>(*d);
   if (acc) o_old = to_f32<O>(*o);
   float d_new, o_new;
-  if constexpr (MODE == MODE_ZERO) {
-    d_new = 0.f;
-    o_new = acc ? __fadd_rn(o_old, 0.f) : 0.f;
-  } else {
-    gather_post_elem<S, D, O, MODE>(s, d_old, o_old, acc, d_new, o_new);
-  }
-  if constexpr (MODE == MODE_COPY && same_t<S, D>::value) *d = reinterpret_cast<const s_t*>(src)[i];
-  else if (write_flat) *d = from_f32<D>(d_new);
+  gather_post_elem<S, D, MODE, DIV>(s, d_old, o_old, acc, dv, d_new, o_new);
+  const bool divided = DIV && dv.a_mode != SCALE_NONE;
+  if (MODE == MODE_COPY && same_t<S, D>::value && !divided) *d = reinterpret_cast<const s_t*>(src)[i];
+  else if (MODE != MODE_SKIP || divided) *d = from_f32<D>(d_new);
   *o = from_f32<O>(o_new);
 }
 
 // One full tile (BLOCK*U units) inside one tensor; flat and shard 16-byte aligned at the tile, src at any
 // element-aligned address.
-template <class S, class D, class O, int MODE, int BLOCK, int U, bool NTL>
-__device__ __forceinline__ void gather_post_full_tile(char* flat, const char* src, char* shard, bool acc) {
+template <class S, class D, class O, int MODE, bool DIV, int BLOCK, int U, bool NTL>
+__device__ __forceinline__ void gather_post_full_tile(char* flat, const char* src, char* shard, bool acc,
+                                                      const ReduceDivides& dv) {
   constexpr bool kReadSrc = (MODE == MODE_COPY || MODE == MODE_ADD);
   constexpr bool kReadFlat = (MODE == MODE_ADD || MODE == MODE_SKIP);
-  constexpr bool kWriteFlat = (MODE != MODE_SKIP);
+  const bool divided = DIV && dv.a_mode != SCALE_NONE;
   Quad<S> s[2 * U];
   Quad<D> d[2 * U];
   Quad<O> o[2 * U];
@@ -101,21 +119,16 @@ __device__ __forceinline__ void gather_post_full_tile(char* flat, const char* sr
     if constexpr (kReadFlat) unpack_quad<D>(d[q], fd);
     if (acc) unpack_quad<O>(o[q], fo);
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-      if constexpr (MODE == MODE_ZERO) {
-        nd[e] = 0.f;
-        no[e] = acc ? __fadd_rn(fo[e], 0.f) : 0.f;
-      } else {
-        gather_post_elem<S, D, O, MODE>(fs[e], fd[e], fo[e], acc, nd[e], no[e]);
-      }
-    }
-    if constexpr (MODE == MODE_COPY && same_t<S, D>::value) {
-      // same dtype: the reduce buffer receives the gradient's bytes (NaN payloads included), as the copy kernel does
+    for (int e = 0; e < 4; e++) gather_post_elem<S, D, MODE, DIV>(fs[e], fd[e], fo[e], acc, dv, nd[e], no[e]);
+    char* f = flat + quad_elem<BLOCK, U>(q) * D::kSize;
+    if (MODE == MODE_COPY && same_t<S, D>::value && !divided) {
+      // same dtype, nothing divided: the reduce buffer receives the gradient's bytes (NaN payloads included), as
+      // the copy kernel does
       Quad<D> raw;
-      raw.v = s[q].v;
-      store_quad<D, true>(flat + quad_elem<BLOCK, U>(q) * D::kSize, raw);
-    } else if constexpr (kWriteFlat) {
-      store_quad<D, true>(flat + quad_elem<BLOCK, U>(q) * D::kSize, pack_quad<D>(nd));
+      if constexpr (same_t<S, D>::value) raw.v = s[q].v;
+      store_quad<D, true>(f, raw);
+    } else if (MODE != MODE_SKIP || divided) {
+      store_quad<D, true>(f, pack_quad<D>(nd));
     }
     store_quad<O, true>(shard + quad_elem<BLOCK, U>(q) * O::kSize, pack_quad<O>(no));
   }
@@ -123,18 +136,19 @@ __device__ __forceinline__ void gather_post_full_tile(char* flat, const char* sr
 
 // n elements of one segment (part of a tile that crosses a tensor boundary or the end of the buffer), one element
 // per lane and step: such tiles are rare (at most one per tensor boundary).
-template <class S, class D, class O, int MODE, int BLOCK>
+template <class S, class D, class O, int MODE, bool DIV, int BLOCK>
 __device__ __forceinline__ void gather_post_segment(char* flat, const char* src, char* shard, int64_t n, bool acc,
-                                                    bool write_flat) {
-  for (int64_t i = threadIdx.x; i < n; i += BLOCK) gather_post_scalar<S, D, O, MODE>(flat, src, shard, i, acc, write_flat);
+                                                    const ReduceDivides& dv) {
+  for (int64_t i = threadIdx.x; i < n; i += BLOCK) gather_post_scalar<S, D, O, MODE, DIV>(flat, src, shard, i, acc, dv);
 }
 
 // S: gradient dtype, D: reduce buffer dtype, O: gradient shard dtype.  `shard` has `padded` elements like `flat`.
-// pad_zero != 0 writes zeros to the pad lanes of the reduce buffer (otherwise they stay as they are); in both cases
-// the pad lanes of the shard receive what the separate post-reduce would give them.
-template <class META, class S, class D, class O, int BLOCK, int U, bool NTL>
+// pad_zero != 0 writes zeros (divided like everything else) to the pad lanes of the reduce buffer, otherwise they
+// only see the divide; in both cases the pad lanes of the shard receive what the separate post-reduce would give them.
+template <class META, class S, class D, class O, bool DIV, int BLOCK, int U, bool NTL>
 __global__ void __launch_bounds__(BLOCK)
-gather_post_kernel(META meta, void* flat, void* shard, int64_t padded, int n_tiles, int pad_zero, int accumulate) {
+gather_post_kernel(META meta, void* flat, void* shard, int64_t padded, int n_tiles, int pad_zero, int accumulate,
+                   ReduceDivides dv) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   char* fbase = reinterpret_cast<char*>(flat);
   char* obase = reinterpret_cast<char*>(shard);
@@ -149,9 +163,9 @@ gather_post_kernel(META meta, void* flat, void* shard, int64_t padded, int n_til
       const char* src = reinterpret_cast<const char*>(meta.tensor(p)) + rec.delta * S::kSize;
       char* f = fbase + t0 * D::kSize;
       char* o = obase + t0 * O::kSize;
-      if (mode == MODE_COPY) gather_post_full_tile<S, D, O, MODE_COPY, BLOCK, U, NTL>(f, src, o, acc);
-      else if (mode == MODE_ADD) gather_post_full_tile<S, D, O, MODE_ADD, BLOCK, U, NTL>(f, src, o, acc);
-      else gather_post_full_tile<S, D, O, MODE_SKIP, BLOCK, U, NTL>(f, src, o, acc);
+      if (mode == MODE_COPY) gather_post_full_tile<S, D, O, MODE_COPY, DIV, BLOCK, U, NTL>(f, src, o, acc, dv);
+      else if (mode == MODE_ADD) gather_post_full_tile<S, D, O, MODE_ADD, DIV, BLOCK, U, NTL>(f, src, o, acc, dv);
+      else gather_post_full_tile<S, D, O, MODE_SKIP, DIV, BLOCK, U, NTL>(f, src, o, acc, dv);
       continue;
     }
     int64_t pos = t0;
@@ -159,8 +173,8 @@ gather_post_kernel(META meta, void* flat, void* shard, int64_t padded, int n_til
       char* f = fbase + pos * D::kSize;
       char* o = obase + pos * O::kSize;
       if (p >= meta.n_tensors) {  // pad lanes
-        if (pad_zero) gather_post_segment<S, D, O, MODE_ZERO, BLOCK>(f, nullptr, o, t1 - pos, acc, true);
-        else gather_post_segment<S, D, O, MODE_SKIP, BLOCK>(f, nullptr, o, t1 - pos, acc, false);
+        if (pad_zero) gather_post_segment<S, D, O, MODE_ZERO, DIV, BLOCK>(f, nullptr, o, t1 - pos, acc, dv);
+        else gather_post_segment<S, D, O, MODE_SKIP, DIV, BLOCK>(f, nullptr, o, t1 - pos, acc, dv);
         break;
       }
       const int64_t o1 = meta.offset(p + 1);
@@ -169,9 +183,9 @@ gather_post_kernel(META meta, void* flat, void* shard, int64_t padded, int n_til
       const int64_t e = o1 < t1 ? o1 : t1;
       const int mode = meta.mode(p);
       const char* src = reinterpret_cast<const char*>(meta.tensor(p)) + (pos - o0) * S::kSize;
-      if (mode == MODE_COPY) gather_post_segment<S, D, O, MODE_COPY, BLOCK>(f, src, o, e - pos, acc, true);
-      else if (mode == MODE_ADD) gather_post_segment<S, D, O, MODE_ADD, BLOCK>(f, src, o, e - pos, acc, true);
-      else gather_post_segment<S, D, O, MODE_SKIP, BLOCK>(f, src, o, e - pos, acc, false);
+      if (mode == MODE_COPY) gather_post_segment<S, D, O, MODE_COPY, DIV, BLOCK>(f, src, o, e - pos, acc, dv);
+      else if (mode == MODE_ADD) gather_post_segment<S, D, O, MODE_ADD, DIV, BLOCK>(f, src, o, e - pos, acc, dv);
+      else gather_post_segment<S, D, O, MODE_SKIP, DIV, BLOCK>(f, src, o, e - pos, acc, dv);
       pos = e;
       if (e == o1) ++p;
     }

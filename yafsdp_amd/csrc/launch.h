@@ -64,11 +64,20 @@ hipError_t launch_unshard(int scatter_shape, int master_dt, int param_dt, const 
                           int n_slots, void* ag_in, const void* master, int64_t n, int head, int n_flat_blocks,
                           int grid, hipStream_t stream);
 // reduce copy-in + post-reduce of a size-1 shard group; `block`: the table's gather-in workgroup size
+// The divides of the reduce step, applied by that kernel at run time (wave-uniform branches; a shard group of size
+// one has none unless the caller set a custom factor or reduces in fp16 with one):
+//   a: on the whole reduce buffer, in place (the pre-divide, ya_fsdp/_collectives.py:139, or the custom division
+//      of :146-148), rounded to the buffer's dtype; the buffer keeps this value
+//   b: the post-divide (:165), rounded to the buffer's dtype; only the gradient shard sees it
+struct ReduceDivides {
+  int a_mode, b_mode;  // SCALE_NONE / SCALE_MUL (k = exact reciprocal) / SCALE_DIV (k = factor)
+  float a_k, b_k;
+};
 bool fused_reduce_supports(int tensor_dt, int flat_dt);
 template <class META>
 hipError_t launch_gather_post(int block, int tensor_dt, int flat_dt, int shard_dt, const META& meta, void* flat,
-                              void* shard, int64_t padded, int n_tiles, int pad_zero, int acc, int grid,
-                              hipStream_t stream);
+                              void* shard, int64_t padded, int n_tiles, int pad_zero, int acc, const ReduceDivides& dv,
+                              int grid, hipStream_t stream);
 
 // fan-out / fan-in over several buffers (fan.hip); all buffers 16-byte aligned
 constexpr int kFanMax = 16;
