@@ -3,6 +3,8 @@ examples on every run).  Shapes, dtypes, alignments, factors and per-tensor mode
 reaches combinations the parametrised tests do not enumerate.  Each example is small; every one names itself
 on stdout before it touches the GPU."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -16,7 +18,10 @@ from helpers import DTYPES, assert_bits_equal, mixed_values
 pytestmark = pytest.mark.gpu
 DEV = torch.device("cuda:0")
 FACTORS = [None, 1.0, 2.0, 3.0, 8.0, 0.5, 1000.0, 64.0]
-COMMON = dict(deadline=None, derandomize=True, suppress_health_check=list(HealthCheck), print_blob=False)
+# YAFSDP_PROPERTY_SCALE=k draws k times as many examples, and fresh ones on every run (a longer search by hand; the
+# default is the fixed set)
+SCALE = max(1, int(os.environ.get("YAFSDP_PROPERTY_SCALE", "1")))
+COMMON = dict(deadline=None, derandomize=SCALE == 1, suppress_health_check=list(HealthCheck), print_blob=SCALE > 1)
 
 
 @pytest.fixture(scope="module")
@@ -34,7 +39,7 @@ def _view_at(x: torch.Tensor, offset: int, fill: float = 3.0) -> tuple[torch.Ten
     return buf, view
 
 
-@settings(max_examples=120, **COMMON)
+@settings(max_examples=120 * SCALE, **COMMON)
 @given(src_dt=st.sampled_from(DTYPES), dst_dt=st.sampled_from(DTYPES), n=st.integers(0, 70_000),
        s_off=st.integers(0, 8), d_off=st.integers(0, 8), factor=st.sampled_from(FACTORS), acc=st.booleans(),
        seed=st.integers(0, 2**20))
@@ -56,7 +61,7 @@ def test_post_reduce_any_shape(nat, src_dt, dst_dt, n, s_off, d_off, factor, acc
 tables = st.lists(st.one_of(st.just(0), st.integers(1, 40), st.integers(1, 6000)), min_size=1, max_size=40)
 
 
-@settings(max_examples=80, **COMMON)
+@settings(max_examples=80 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), grad_dt=st.sampled_from(DTYPES), rs_dt=st.sampled_from(DTYPES),
        pre=st.sampled_from(FACTORS), two_waves=st.booleans(), zero_pad=st.booleans(), seed=st.integers(0, 2**20))
 def test_gather_in_any_table(nat, numels, pad, grad_dt, rs_dt, pre, two_waves, zero_pad, seed):
@@ -92,7 +97,7 @@ def test_gather_in_any_table(nat, numels, pad, grad_dt, rs_dt, pre, two_waves, z
     table.close()
 
 
-@settings(max_examples=80, **COMMON)
+@settings(max_examples=80 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), flat_dt=st.sampled_from(DTYPES), out_dt=st.sampled_from(DTYPES),
        two_waves=st.booleans(), bound=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2))
 def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bound, seed, tile_mode):
@@ -129,7 +134,7 @@ def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bou
     table.close()
 
 
-@settings(max_examples=80, **COMMON)
+@settings(max_examples=80 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), master_dt=st.sampled_from(DTYPES), param_dt=st.sampled_from(DTYPES),
        shard_n=st.integers(0, 9000), two_waves=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2))
 def test_copy_in_scatter_out_any_table(nat, numels, pad, master_dt, param_dt, shard_n, two_waves, seed, tile_mode):
@@ -168,7 +173,7 @@ def test_copy_in_scatter_out_any_table(nat, numels, pad, master_dt, param_dt, sh
     table.close()
 
 
-@settings(max_examples=100, **COMMON)
+@settings(max_examples=100 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), grad_dt=st.sampled_from(DTYPES), wide_buffer=st.booleans(),
        shard_dt=st.sampled_from(DTYPES), acc=st.booleans(), two_waves=st.booleans(), zero_pad=st.booleans(),
        seed=st.integers(0, 2**20))
@@ -212,7 +217,7 @@ def test_gather_in_post_reduce_any_table(nat, numels, pad, grad_dt, wide_buffer,
 
 
 # ------------------------------------------------------------ optimizer side --
-@settings(max_examples=80, **COMMON)
+@settings(max_examples=80 * SCALE, **COMMON)
 @given(n=st.integers(1, 40_000), off=st.integers(0, 3), decoupled=st.booleans(),
        beta1=st.sampled_from([0.9, 0.5, 0.3, 0.0]), beta2=st.sampled_from([0.95, 0.999, 0.5]),
        wd=st.sampled_from([0.0, 0.1, 1e-2]), lr=st.sampled_from([3e-4, 1e-2, 0.0]), step=st.integers(1, 2000),
@@ -245,7 +250,7 @@ def test_adamw_any_shape(nat, n, off, decoupled, beta1, beta2, wd, lr, step, out
         assert_bits_equal(out, want_out, "out16")
 
 
-@settings(max_examples=60, **COMMON)
+@settings(max_examples=60 * SCALE, **COMMON)
 @given(dt=st.sampled_from(DTYPES), n=st.integers(0, 300_000), off=st.integers(0, 8),
        coef=st.sampled_from([1.0, 0.5, 0.19153, 3.0]), seed=st.integers(0, 2**20))
 def test_sumsq_fill_scale_any_shape(nat, dt, n, off, coef, seed):
@@ -272,7 +277,7 @@ def test_sumsq_fill_scale_any_shape(nat, dt, n, off, coef, seed):
     assert float(guard.min()) == 7.0 and float(guard.max()) == 7.0
 
 
-@settings(max_examples=60, **COMMON)
+@settings(max_examples=60 * SCALE, **COMMON)
 @given(src_dt=st.sampled_from(DTYPES), dst_dt=st.sampled_from(DTYPES), n=st.integers(0, 60_000),
        k=st.integers(1, 16), seed=st.integers(0, 2**20))
 def test_fanout_any_shape(nat, src_dt, dst_dt, n, k, seed):
@@ -287,7 +292,7 @@ def test_fanout_any_shape(nat, src_dt, dst_dt, n, k, seed):
         assert_bits_equal(d, want, f"destination {i}")
 
 
-@settings(max_examples=60, **COMMON)
+@settings(max_examples=60 * SCALE, **COMMON)
 @given(chunk_dt=st.sampled_from(DTYPES), shard_dt=st.sampled_from(DTYPES), n=st.integers(0, 60_000),
        k=st.integers(1, 16), post=st.sampled_from(FACTORS), acc=st.booleans(), seed=st.integers(0, 2**20))
 def test_fanin_any_shape(nat, chunk_dt, shard_dt, n, k, post, acc, seed):
@@ -307,7 +312,7 @@ shape_st = st.one_of(st.tuples(st.integers(1, 300)), st.tuples(st.integers(1, 40
                      st.tuples(st.integers(1, 6), st.integers(1, 9), st.integers(1, 9)))
 
 
-@settings(max_examples=40, **COMMON)
+@settings(max_examples=40 * SCALE, **COMMON)
 @given(shapes=st.lists(shape_st, min_size=1, max_size=6), w=st.integers(1, 6), r_frac=st.floats(0, 0.999),
        align=st.sampled_from([1, 2, 8, 16]), policy=st.sampled_from(["bf16", "bf16-fp32reduce", "fp16"]),
        iterations=st.integers(1, 3), seed=st.integers(0, 2**20))
