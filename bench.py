@@ -62,8 +62,15 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 # fp32 copy of the same run; profiles/bench_llama3-8b-layer-w8-optim_hbm_traffic.md.
 # "ragged-stress-w256": gather_in_kernel<LargeMeta>, (379903.9 * 1.99992 + 710944.2 * 0.99984) KiB;
 # profiles/bench_ragged-stress-w256_hbm_traffic.md.
+# "llama3-70b-layer-w64": gather_in_kernel<SmallMeta,...,128,2>, (835642.75 * 1.99997 + 1671299.6 * 1.00000) KiB;
+# "ragged-stress-w256-bf16-masters": gather_in_kernel<LargeMeta,BF16,F32>, (178792.9 * 1.99987 + 633008.8) KiB (the
+# reads are 13 % above the algorithmic 323.8 MB: 573 bf16 sources at odd offsets, 2 KB per tile);
+# "tiny-layer-w1": gather_post_kernel, (9309.25 * 1.99322 + 18534.0) KiB, below the algorithmic bytes of the two
+# kernels it replaces because the reduce buffer is not read back;
+# all three in profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.
 MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872615800, "llama3-8b-layer-w8-optim": 817_885_000,
-                          "ragged-stress-w256": 1_505_902_865}
+                          "ragged-stress-w256": 1_505_902_865, "llama3-70b-layer-w64": 3_422_785_664,
+                          "ragged-stress-w256-bf16-masters": 1_014_344_628, "tiny-layer-w1": 37_979_573}
 
 
 def log(*a):
