@@ -107,6 +107,65 @@ int main(void) {
     if (!same(what, h_out[p], h_out_want[p], (size_t)numels[p] * 2)) return 1;
   }
 
+  /* ---- copy-in + copy-out as ONE launch: fp32 master shard -> bf16 all-gather input, next to the split of a bf16
+   * gathered buffer into bf16 tensors */
+  {
+    const int64_t ns = 123457;
+    float* h_master = malloc((size_t)ns * 4);
+    uint16_t *h_ag = malloc((size_t)ns * 2), *h_ag_want = malloc((size_t)ns * 2);
+    uint16_t* h_gathered = malloc((size_t)padded * 2);
+    for (int64_t i = 0; i < ns; i++) h_master[i] = next_float(2e-2f);
+    for (int64_t i = 0; i < padded; i++) h_gathered[i] = to_bf16(next_float(2e-2f));
+    ref_flat_copy(h_ag_want, YAFSDP_BF16, h_master, YAFSDP_F32, ns);
+    ref_scatter_out(P, (void* const*)h_out_want, offsets, YAFSDP_BF16, h_gathered, YAFSDP_BF16);
+    float* d_master;
+    void *d_ag, *d_gathered;
+    HIP(hipMalloc((void**)&d_master, (size_t)ns * 4));
+    HIP(hipMalloc(&d_ag, (size_t)ns * 2));
+    HIP(hipMalloc(&d_gathered, (size_t)padded * 2));
+    HIP(hipMemcpy(d_master, h_master, (size_t)ns * 4, hipMemcpyHostToDevice));
+    HIP(hipMemcpy(d_gathered, h_gathered, (size_t)padded * 2, hipMemcpyHostToDevice));
+    YA(yafsdp_copy_in_scatter_out(table, d_gathered, YAFSDP_BF16, d_out, NULL, d_ag, d_master, YAFSDP_F32, ns, stream));
+    HIP(hipStreamSynchronize(stream));
+    HIP(hipMemcpy(h_ag, d_ag, (size_t)ns * 2, hipMemcpyDeviceToHost));
+    if (!same("copy_in_scatter_out: all-gather input", h_ag, h_ag_want, (size_t)ns * 2)) return 1;
+    for (int p = 0; p < P; p++) {
+      HIP(hipMemcpy(h_out[p], d_out[p], (size_t)numels[p] * 2, hipMemcpyDeviceToHost));
+      char what[64];
+      snprintf(what, sizeof what, "copy_in_scatter_out: tensor %d", p);
+      if (!same(what, h_out[p], h_out_want[p], (size_t)numels[p] * 2)) return 1;
+    }
+    free(h_master); free(h_ag); free(h_ag_want); free(h_gathered);
+    HIP(hipFree(d_master)); HIP(hipFree(d_ag)); HIP(hipFree(d_gathered));
+  }
+
+  /* ---- reduce copy-in + post-reduce of a shard group of size one as ONE launch: bf16 gradients -> fp32 reduce
+   * buffer (copy / add / absent), /4 before and /3 after the "reduce-scatter", accumulated into a bf16 shard */
+  {
+    float *h_rs = malloc((size_t)padded * 4), *h_rs_want = malloc((size_t)padded * 4);
+    uint16_t *h_gs = malloc((size_t)padded * 2), *h_gs_want = malloc((size_t)padded * 2);
+    for (int64_t i = 0; i < padded; i++) { h_rs[i] = next_float(1e-3f); h_gs[i] = to_bf16(next_float(1e-3f)); }
+    memcpy(h_rs_want, h_rs, (size_t)padded * 4);
+    memcpy(h_gs_want, h_gs, (size_t)padded * 2);
+    ref_gather_in(P, (const void* const*)h_grads, offsets, modes, YAFSDP_BF16, h_rs_want, YAFSDP_F32, padded, 4.0, 1);
+    ref_post_reduce(h_gs_want, YAFSDP_BF16, h_rs_want, YAFSDP_F32, padded, 3.0, 1);
+    float* d_rs;
+    void* d_gs;
+    HIP(hipMalloc((void**)&d_rs, (size_t)padded * 4));
+    HIP(hipMalloc(&d_gs, (size_t)padded * 2));
+    HIP(hipMemcpy(d_rs, h_rs, (size_t)padded * 4, hipMemcpyHostToDevice));
+    HIP(hipMemcpy(d_gs, h_gs, (size_t)padded * 2, hipMemcpyHostToDevice));
+    YA(yafsdp_gather_in_post_reduce(table, (const void* const*)d_grads, modes, YAFSDP_BF16, d_rs, YAFSDP_F32, 4.0, 0.0,
+                                    3.0, 1, d_gs, YAFSDP_BF16, 1, stream));
+    HIP(hipStreamSynchronize(stream));
+    HIP(hipMemcpy(h_rs, d_rs, (size_t)padded * 4, hipMemcpyDeviceToHost));
+    HIP(hipMemcpy(h_gs, d_gs, (size_t)padded * 2, hipMemcpyDeviceToHost));
+    if (!same("gather_in_post_reduce: reduce buffer", h_rs, h_rs_want, (size_t)padded * 4)) return 1;
+    if (!same("gather_in_post_reduce: gradient shard", h_gs, h_gs_want, (size_t)padded * 2)) return 1;
+    free(h_rs); free(h_rs_want); free(h_gs); free(h_gs_want);
+    HIP(hipFree(d_rs)); HIP(hipFree(d_gs));
+  }
+
   /* ---- post-reduce: bf16 chunk /3 accumulated into an fp32 shard */
   const int64_t s = 500009;
   float* h_shard = malloc((size_t)s * 4);
