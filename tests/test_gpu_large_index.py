@@ -66,3 +66,39 @@ def test_table_with_offsets_beyond_int32(nat, pattern):
     assert torch.equal(outs[0].view(torch.int16), flat[:n0].view(torch.int16))
     assert torch.equal(outs[1].view(torch.int16), flat[n0:N].view(torch.int16))
     table.close()
+
+
+def test_shared_launches_beyond_int32(nat, pattern):
+    """The two launches that do the work of two each on the same table: copy-in + copy-out as one grid, and the
+    one-pass reduce of a size-one group (with a /4 before and a /2 after the reduce buffer, both exact here)."""
+    n0 = (1 << 31) + 5
+    numels = [n0, N - n0]
+    padded = N + 27
+    print("shared launches, offsets", [0, n0], flush=True)
+    table = nat.TensorTable(numels, padded, DEV)
+    # copy-in + copy-out
+    gathered = torch.empty(padded, dtype=torch.bfloat16, device=DEV)
+    gathered[:N].copy_(pattern)
+    gathered[N:].fill_(7.0)
+    master = pattern[: 1 << 22].float() * 3.0
+    ag = torch.zeros(1 << 22, dtype=torch.bfloat16, device=DEV)
+    outs = [torch.empty(n, dtype=torch.bfloat16, device=DEV) for n in numels]
+    assert table.copy_in_scatter_out(gathered, outs, ag, master)
+    assert torch.equal(ag.view(torch.int16), master.to(torch.bfloat16).view(torch.int16))
+    assert torch.equal(outs[0].view(torch.int16), pattern[:n0].view(torch.int16))
+    assert torch.equal(outs[1].view(torch.int16), pattern[n0:].view(torch.int16))
+    del gathered, outs, ag, master
+    # one-pass reduce: flat = pattern / 4 (pad zero), shard = 1.0 + flat / 2 in binary32 (all exact)
+    flat = torch.full((padded,), 3.0, dtype=torch.bfloat16, device=DEV)
+    shard = torch.ones(padded, dtype=torch.float32, device=DEV)
+    assert table.gather_in_post_reduce([pattern[:n0], pattern[n0:]], flat, shard, True, pre_factor=4.0, post_factor=2.0)
+    for lo, hi in ((0, 1 << 20), (n0 - (1 << 20), N)):
+        want = (pattern[lo:hi].float() / 4.0).to(torch.bfloat16)
+        assert torch.equal(flat[lo:hi].view(torch.int16), want.view(torch.int16)), (lo, hi)
+        assert torch.equal(shard[lo:hi], 1.0 + want.float() / 2.0), (lo, hi)
+    assert flat[:N].float().abs().sum(dtype=torch.float64).item() * 4.0 == pattern.float().abs().sum(dtype=torch.float64).item()
+    assert float(flat[N:].float().abs().max()) == 0.0 and float((shard[N:] - 1.0).abs().max()) == 0.0
+    # the whole shard through an exact checksum: sum(shard - 1) * 8 == sum(pattern) (every term a small power of two)
+    got = (shard[:N] - 1.0).sum(dtype=torch.float64).item() * 8.0
+    assert got == pattern.float().sum(dtype=torch.float64).item(), got
+    table.close()
