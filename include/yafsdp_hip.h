@@ -72,6 +72,21 @@ const char* yafsdp_error_string(int code);
  * flat entry point below). */
 int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, void* stream);
 
+/* dst[0:n_bytes] = src[0:n_bytes]: `Tensor.copy_` between contiguous ranges of
+ * one element type that the arithmetic of this path never touches (1-byte
+ * types: float8, int8, uint8; any other type copies the same way).  The two
+ * ranges may start at any byte address.
+ * Replaces: the per-parameter copy of a tensor-subclass all-gather input into
+ *           its fragment of the flat all-gather input,
+ *           self._all_gather_input.copy_(all_gather_input)
+ *           (ya_fsdp/_param.py:281-291, input from fsdp_pre_all_gather), and the
+ *           size-1-group all-gather all_gather_output.copy_(all_gather_input)
+ *           (ya_fsdp/_collectives.py:56-58) of such an all-gather dtype
+ *           (MixedPrecisionPolicy.all_gather_dtype_to_param_cls,
+ *           ya_fsdp/_api.py:13, ya_fsdp/_param_group.py:194-227).
+ * dst == src is a no-op; any other overlap is refused. */
+int yafsdp_flat_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream);
+
 /* buf[i] = round(buf[i] / factor) in place, only if factor > 1.
  * Replaces: _div_if_needed / tensor.div_ (ya_fsdp/_collectives.py:139, 165,
  * 270-272). */

@@ -24,6 +24,13 @@ def copy_in(all_gather_input: torch.Tensor, padded_sharded_param_data: torch.Ten
     all_gather_input.copy_(padded_sharded_param_data)
 
 
+def extension_copy_in(param_all_gather_input: torch.Tensor, all_gather_input: torch.Tensor) -> None:
+    """The per-parameter copy of a tensor subclass's all-gather input (what its
+    ``fsdp_pre_all_gather`` returned) into the parameter's fragment of the flat
+    all-gather input (ya_fsdp/_param.py:281-291)."""
+    param_all_gather_input.copy_(all_gather_input)
+
+
 def all_gather_single_rank(all_gather_output: torch.Tensor, all_gather_input: torch.Tensor) -> None:
     """The "all-gather" of a size-1 group (ya_fsdp/_collectives.py:56-58)."""
     all_gather_output.copy_(all_gather_input)

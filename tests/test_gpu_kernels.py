@@ -69,6 +69,36 @@ def test_flat_copy_sizes_and_alignments(nat, src_dt, dst_dt):
             assert_bits_equal(got, want, f"flat_copy n={n} offs=({s_off},{d_off})")
 
 
+@pytest.mark.parametrize("dt", [torch.uint8, torch.int8, torch.float8_e4m3fn, torch.float8_e5m2, torch.int32])
+def test_flat_copy_of_opaque_element_types(nat, dt):
+    """Same-dtype copies of element types outside the path's arithmetic (the
+    all-gather dtypes of tensor-subclass parameters) are byte copies at any byte
+    address: every alignment of either side modulo 16 and beyond, sizes around
+    the vector and tile edges, guard bytes on both sides of the destination."""
+    g = torch.Generator().manual_seed(101)
+    size = torch.empty(0, dtype=dt).element_size()
+    sizes = [0, 1, 2, 15, 16, 17, 31, 33, 255, 4095, 4096, 4097, 12_289, 65_536 + 3, 1_048_583]
+    offs = [(0, 0), (1, 0), (0, 1), (1, 1), (3, 2), (2, 3), (15, 16), (16, 15), (7, 9), (13, 5), (32, 17)]
+    if size > 1:
+        sizes, offs = sizes[:10], offs[:6]
+    for n in sizes:
+        for s_off, d_off in offs:
+            _say("flat_copy bytes", dt, n, s_off, d_off)
+            raw = torch.randint(0, 256, ((n + s_off) * size,), generator=g, dtype=torch.uint8)
+            src = raw.view(dt)
+            want = torch.full(((n + d_off + 40) * size,), 0xA5, dtype=torch.uint8).view(dt)
+            torch_ops.extension_copy_in(want[d_off : d_off + n], src[s_off:])
+            got = torch.full(((n + d_off + 40) * size,), 0xA5, dtype=torch.uint8, device=DEV).view(dt)
+            nat.flat_copy(got[d_off : d_off + n], src.to(DEV)[s_off:])
+            assert torch.equal(got.view(torch.uint8).cpu(), want.view(torch.uint8)), (dt, n, s_off, d_off)
+    # a self-copy is a no-op, a partial overlap is refused
+    buf = torch.arange(100, dtype=torch.uint8, device=DEV)
+    nat.flat_copy(buf[1:50], buf[1:50])
+    with pytest.raises(RuntimeError):
+        nat.flat_copy(buf[1:50], buf[4:53])
+    assert torch.equal(buf.cpu(), torch.arange(100, dtype=torch.uint8))
+
+
 def test_flat_copy_same_dtype_is_byte_copy(nat):
     # NaN payloads and every bit pattern pass through a same-dtype copy
     allh = torch.arange(-32768, 32768, dtype=torch.int32).to(torch.int16)

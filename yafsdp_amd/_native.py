@@ -39,6 +39,7 @@ EXPORTED_SYMBOLS = (
     "yafsdp_version",
     "yafsdp_error_string",
     "yafsdp_flat_copy",
+    "yafsdp_flat_copy_bytes",
     "yafsdp_flat_div",
     "yafsdp_flat_div_copy",
     "yafsdp_post_reduce",
@@ -90,6 +91,8 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_error_string.argtypes = [i32]
     lib.yafsdp_flat_copy.restype = i32
     lib.yafsdp_flat_copy.argtypes = [vp, i32, vp, i32, i64, vp]
+    lib.yafsdp_flat_copy_bytes.restype = i32
+    lib.yafsdp_flat_copy_bytes.argtypes = [vp, vp, i64, vp]
     lib.yafsdp_flat_div.restype = i32
     lib.yafsdp_flat_div.argtypes = [vp, i32, i64, dbl, vp]
     lib.yafsdp_flat_div_copy.restype = i32
@@ -217,10 +220,20 @@ def _factor(f: float | None) -> float:
 
 # ------------------------------------------------------------------ flat ops --
 def flat_copy(dst: torch.Tensor, src: torch.Tensor) -> None:
-    """``dst.copy_(src)`` for contiguous tensors of equal numel."""
+    """``dst.copy_(src)`` for contiguous tensors of equal numel.  Two tensors of one dtype outside the arithmetic
+    dtypes of the path (float8, int8, uint8, ...) are copied as bytes."""
     _flat_arg(dst, "dst"), _flat_arg(src, "src")
     if dst.numel() != src.numel():
         raise ValueError(f"numel mismatch: {dst.numel()} vs {src.numel()}")
+    if dst.dtype == src.dtype and dst.dtype not in DTYPE_CODE:
+        if dst.device != src.device:
+            raise RuntimeError(f"dst on {dst.device}, src on {src.device}")
+        with _on(dst.device):
+            _check(
+                lib.yafsdp_flat_copy_bytes(dst.data_ptr(), src.data_ptr(), dst.numel() * dst.element_size(), _stream(dst)),
+                "yafsdp_flat_copy_bytes",
+            )
+        return
     with _on(dst.device):
         _check(
             lib.yafsdp_flat_copy(dst.data_ptr(), _dt(dst), src.data_ptr(), _dt(src), dst.numel(), _stream(dst)),

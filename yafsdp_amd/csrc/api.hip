@@ -700,6 +700,24 @@ int yafsdp_flat_copy(void* dst, int dst_dtype, const void* src, int src_dtype, i
   return flat_launch(src_dtype, dst_dtype, SCALE_NONE, false, dst, src, n, 1.0f, static_cast<hipStream_t>(stream));
 }
 
+int yafsdp_flat_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* stream) {
+  if (n_bytes < 0 || (n_bytes > 0 && (dst == nullptr || src == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n_bytes == 0 || dst == src) return YAFSDP_OK;
+  const uintptr_t d0 = reinterpret_cast<uintptr_t>(dst), s0 = reinterpret_cast<uintptr_t>(src);
+  if (((d0 | s0 | uintptr_t(n_bytes)) & 1) == 0)  // pairs of bytes at even addresses: the tuned 2-byte copy
+    return flat_launch(DT_BF16, DT_BF16, SCALE_NONE, false, dst, src, n_bytes >> 1, 1.0f,
+                       static_cast<hipStream_t>(stream));
+  if (d0 < s0 + uintptr_t(n_bytes) && s0 < d0 + uintptr_t(n_bytes)) return YAFSDP_ERR_INVALID_ARGUMENT;  // overlap
+  int64_t head = int64_t((16 - (d0 & 15)) & 15);
+  if (head > n_bytes) head = n_bytes;
+  const int64_t n_tiles = (((n_bytes - head) >> 4) + kFlatBlock - 1) / kFlatBlock;
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return int(e);
+  const int grid = grid_for(n_tiles, g_flat_blocks_per_cu.load(std::memory_order_relaxed), device);
+  return int(launch_bytes(dst, src, n_bytes, int(head), grid, static_cast<hipStream_t>(stream)));
+}
+
 int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream) {
   if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
   if (n < 0 || (n > 0 && buf == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;

@@ -146,4 +146,47 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned l
   }
 }
 
+// ---- opaque bytes ------------------------------------------------------------
+// dst[0:n] = src[0:n] for byte ranges at ANY byte address: the same-dtype copy of
+// 1-byte element types (fp8, int8, uint8), whose ragged per-parameter fragments
+// start and end at odd addresses.  `head` (0..15) leading bytes bring dst to a
+// 16-byte boundary; the body is 16-byte vectors, one per lane and tile (aligned
+// stores; the loads sit at whatever byte alignment the two addresses leave, which
+// the hardware serves natively like the element-aligned loads of the other
+// kernels); workgroup 0 also copies the head and the up to 15 trailing bytes.
+typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
+
+template <int BLOCK, bool NTL, int STP>
+__global__ void __launch_bounds__(BLOCK)
+bytes_kernel(void* dst, const void* src, int64_t n, int head) {
+  const int tid = threadIdx.x;
+  const int64_t n_vecs = (n - head) >> 4;
+  const int64_t body_end = head + (n_vecs << 4);
+  uint8_t* d8 = reinterpret_cast<uint8_t*>(dst);
+  const uint8_t* s8 = reinterpret_cast<const uint8_t*>(src);
+  if (blockIdx.x == 0) {
+    if (tid < head) d8[tid] = s8[tid];
+    const int tail = int(n - body_end);
+    const int t = BLOCK - 1 - tid;
+    if (t < tail) d8[body_end + t] = s8[body_end + t];
+  }
+  char* dbase = reinterpret_cast<char*>(dst) + head;
+  const char* sbase = reinterpret_cast<const char*>(src) + head;
+  const int64_t n_tiles = (n_vecs + BLOCK - 1) / BLOCK;
+  for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const int64_t v = tile * BLOCK + tid;
+    if (tile * BLOCK + BLOCK <= n_vecs) {
+      const TileStore<BF16, STP> out(dbase + tile * BLOCK * 16, BLOCK * 16);
+      const u32x4_a1* q = reinterpret_cast<const u32x4_a1*>(sbase + v * 16);
+      u32x4 x;
+      if constexpr (NTL) x = __builtin_nontemporal_load(q);
+      else x = *q;
+      out.vec(tid * 16, x);
+    } else if (v < n_vecs) {  // last, partial tile
+      const u32x4 x = *reinterpret_cast<const u32x4_a1*>(sbase + v * 16);
+      *reinterpret_cast<u32x4*>(dbase + v * 16) = x;
+    }
+  }
+}
+
 }  // namespace yafsdp
