@@ -80,16 +80,17 @@ def all_gather(
     if yccl_handle is not None:
         raise NotImplementedError("YCCL handles are not part of this build")
     with torch.cuda.stream(all_gather_stream):
-        if (
-            (version := param_group._copy_in_shard_version) is not None
-            and all_gather_dtype in param_group._all_gather_input_set_dtypes
-            and padded_sharded_param_data._version != version
-        ):
-            # a fused optimizer step wrote the all-gather input, and a torch op has
-            # changed the master shard since (load_state_dict, another optimizer):
-            # the 16-bit copy is stale, cast again
-            param_group._all_gather_input_set_dtypes.discard(all_gather_dtype)
-        param_group._copy_in_shard_version = None
+        if all_gather_dtype is None:
+            if (
+                (version := param_group._copy_in_shard_version) is not None
+                and all_gather_dtype in param_group._all_gather_input_set_dtypes
+                and padded_sharded_param_data._version != version
+            ):
+                # a fused optimizer step wrote the all-gather input, and a torch op has
+                # changed the master shard since (load_state_dict, another optimizer):
+                # the 16-bit copy is stale, cast again
+                param_group._all_gather_input_set_dtypes.discard(all_gather_dtype)
+            param_group._copy_in_shard_version = None
         world_size = all_gather_group.size()
         shard_numel = all_gather_input.numel()
         rank = all_gather_group.rank()
@@ -257,11 +258,7 @@ def reduce_scatter(
                     # :165 in place on the chunk, as the reference does it, then :191-214 as ONE launch whatever the
                     # pattern of modes: the chunk's fragments are the "tensors" of a table over the gradient shard
                     _div_if_needed(output_tensor, post)
-                    table = param_group._fragment_table
-                    if table is None:
-                        table = param_group._fragment_table = _native.TensorTable(
-                            numels, padded_sharded_param_grad.numel(), padded_sharded_param_grad.device
-                        )
+                    table = param_group._fragment_table_for(padded_sharded_param_grad, numels)
                     fragments = list(output_tensor[: sum(numels)].split(numels))
                     table.gather_in(fragments, padded_sharded_param_grad, modes, None, zero_pad=False)
         post_reduce_event = reduce_scatter_stream.record_event()

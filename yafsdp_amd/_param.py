@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import weakref
 from dataclasses import dataclass, field
+from typing import Any
 
 import torch
 import torch.nn as nn
@@ -29,6 +30,24 @@ class ParamModuleInfo:
     param_name: str
     shared_modules: list[nn.Module] = field(default_factory=list)
     shared_param_names: list[str] = field(default_factory=list)
+
+
+@dataclass
+class ExtensionsData:
+    """ya_fsdp/_param.py:35-41: what a tensor subclass's ``fsdp_pre_all_gather`` hands to its
+    ``fsdp_post_all_gather``."""
+
+    all_gather_metadata: Any | None = None
+
+    def clear(self) -> None:
+        self.all_gather_metadata = None
+
+
+def _inner_tensor_names(t: torch.Tensor) -> "list[str] | None":
+    """Attribute names of the inner tensors of a wrapper tensor subclass; None for a plain tensor."""
+    if type(t) in (torch.Tensor, nn.Parameter) or not hasattr(t, "__tensor_flatten__"):
+        return None
+    return list(t.__tensor_flatten__()[0])
 
 
 class YaFSDPParam:
@@ -86,12 +105,33 @@ class YaFSDPParam:
             local_numel=sharded_param_data.numel(), global_offset=global_offset, shard_numels=shard_numels
         )
         self.sharded_numel = sharded_param_data.numel()
-        self._sharded_param_data = sharded_param_data
+        self._sharded_param_data = sharded_param_data  # the plain fragment of the flat master shard
+        # What the sharded parameter wraps (ya_fsdp/_param.py:145-152): for a plain parameter the fragment itself;
+        # for a tensor subclass an instance of that subclass made by its own ``new_zeros``, whose first inner tensor
+        # is then replaced by the fragment, so that the subclass's methods (the all-gather hooks among them) see the
+        # master values of this rank.
+        self._sharded_local: torch.Tensor = sharded_param_data
+        if _inner_tensor_names(self.param_data) is not None:
+            holder = self.param_data.detach().new_zeros(self.sharded_numel)
+            if (holder_names := _inner_tensor_names(holder)) is None:
+                raise AssertionError(
+                    f"{type(self.param_data).__name__}.new_zeros returned a plain tensor: the subclass has to "
+                    "return an instance of itself for the sharded parameter to keep its all-gather hooks"
+                )
+            inner = getattr(holder, holder_names[0])
+            if inner.shape != sharded_param_data.shape or inner.dtype != sharded_param_data.dtype:
+                raise AssertionError(
+                    f"first inner tensor of {type(holder).__name__}.new_zeros({self.sharded_numel}) is "
+                    f"{tuple(inner.shape)} {inner.dtype}, expected {tuple(sharded_param_data.shape)} "
+                    f"{sharded_param_data.dtype}"
+                )
+            setattr(holder, holder_names[0], sharded_param_data)
+            self._sharded_local = holder
         self._sharding_spec = RaggedShardSpec(  # :136-140 with the logical mesh in the DeviceMesh's place
             self.mesh_info, (self.placement,), TensorMeta(self._orig_size, self.param.stride(), self.param.dtype),
             weakref.ref(self), "param",
         )
-        self.sharded_param = nn.Parameter(self.to_sharded_dtensor(sharded_param_data), requires_grad=self.requires_grad)
+        self.sharded_param = nn.Parameter(self.to_sharded_dtensor(self._sharded_local), requires_grad=self.requires_grad)
         self.sharded_param._yafsdp_param = weakref.ref(self)  # lets flat-shard optimizers find the owner
         if self.requires_grad:
             assert sharded_param_grad is not None
@@ -100,6 +140,25 @@ class YaFSDPParam:
             self.sharded_param_grad = None
         del self.param, self.param_data  # the group's flat shard now owns the values
         self._setattr_on_modules(self.sharded_param)
+        self._init_extensions()
+
+    def _init_extensions(self) -> None:
+        """ya_fsdp/_param.py:185-195."""
+        inner_tensor = self._sharded_local_tensor
+        has_fsdp_pre_all_gather = hasattr(inner_tensor, "fsdp_pre_all_gather")
+        has_fsdp_post_all_gather = hasattr(inner_tensor, "fsdp_post_all_gather")
+        if has_fsdp_pre_all_gather != has_fsdp_post_all_gather:
+            raise AssertionError(
+                "Both fsdp_pre_all_gather and fsdp_post_all_gather should be defined "
+                f"if using all-gather extensions: {inner_tensor}"
+            )
+        self._extensions_data = ExtensionsData() if has_fsdp_pre_all_gather else None
+
+    @property
+    def shard_mesh_from_root(self) -> FSDPMeshInfo:
+        """What ``fsdp_pre_all_gather`` receives (ya_fsdp/_param.py:328-337 passes the shard ``DeviceMesh``): the
+        logical shard mesh, i.e. its size and this rank."""
+        return self.mesh_info
 
     def to_sharded_dtensor(self, tensor: torch.Tensor, kind: str = "param") -> RaggedShardDTensor:
         """ya_fsdp/_param.py:298-310: wrap a local 1-D fragment of this parameter (same length as the sharded
@@ -126,7 +185,15 @@ class YaFSDPParam:
     def init_unsharded_param(
         self, all_gather_output: torch.Tensor, reduce_scatter_input: torch.Tensor | None
     ) -> None:
+        """ya_fsdp/_param.py:203-231."""
         unsharded_tensor = all_gather_output.view(self._orig_size)  # zero-copy copy-out
+        if self._extensions_data is not None:
+            # the raw view is what to_unsharded() hands to the hook on every later unshard (:211-217); at this
+            # point no all-gather has run and the metadata is still None, as in the reference
+            self._all_gather_output = unsharded_tensor
+            unsharded_tensor, _ = self._sharded_local_tensor.fsdp_post_all_gather(
+                (unsharded_tensor,), self._extensions_data.all_gather_metadata, self.param_dtype or self.orig_dtype
+            )
         self.unsharded_param = nn.Parameter(unsharded_tensor, requires_grad=self.requires_grad)
         self.unsharded_param._yafsdp_param = weakref.ref(self)
         if self.requires_grad:
@@ -136,16 +203,41 @@ class YaFSDPParam:
             self._unsharded_accumulated_grad = None
 
     def set_all_gather_input(self) -> None:
-        """Hook of ya_fsdp/_param.py:281-291 for tensor subclasses with
-        ``fsdp_pre_all_gather``; plain tensors have nothing to do."""
+        """ya_fsdp/_param.py:281-291: a tensor subclass with ``fsdp_pre_all_gather`` produces its own all-gather
+        input (an fp8 cast, say) and the metadata its ``fsdp_post_all_gather`` will want; the input is copied into
+        this parameter's fragment of the flat all-gather input.  Plain tensors have nothing to do."""
         if self.sharded_state != ShardedState.SHARDED:
             raise AssertionError(f"Expects to be in SHARDED, not {self.sharded_state}")
+        if self._extensions_data is None:
+            return
+        all_gather_inputs, self._extensions_data.all_gather_metadata = self._sharded_local_tensor.fsdp_pre_all_gather(
+            self.shard_mesh_from_root
+        )
+        (all_gather_input,) = all_gather_inputs
+        dst = self._all_gather_input
+        if all_gather_input.numel() != dst.numel():
+            raise AssertionError(
+                f"fsdp_pre_all_gather of {self._param_fqn} returned {all_gather_input.numel()} elements for a "
+                f"fragment of {dst.numel()}"
+            )
+        if dst.numel() > 0:
+            from . import _native
+
+            _native.flat_copy(dst, all_gather_input.detach().contiguous().view(-1))
 
     def to_sharded(self) -> None:
         self._setattr_on_modules(self.sharded_param)
         self.sharded_state = ShardedState.SHARDED
 
     def to_unsharded(self) -> None:
+        """ya_fsdp/_param.py:237-257."""
+        if self._extensions_data is not None and self._extensions_data.all_gather_metadata is not None:
+            # refresh what the subclass derives from this all-gather's metadata (quantisation scales, say) on the
+            # existing unsharded tensor; its data already is the gathered buffer
+            self._sharded_local_tensor.fsdp_post_all_gather(
+                (self._all_gather_output,), self._extensions_data.all_gather_metadata,
+                self.param_dtype or self.orig_dtype, out=self.unsharded_param,
+            )
         self._setattr_on_modules(self.unsharded_param)
         self.sharded_state = ShardedState.UNSHARDED
 
@@ -166,7 +258,12 @@ class YaFSDPParam:
             return
         new_param = getattr(info.module, info.param_name)
         new_local = local_tensor(new_param.detach())
-        if new_local.data_ptr() != self._sharded_param_data.data_ptr() and self.sharded_numel > 0:
+        if self._sharded_local is not self._sharded_param_data:
+            # a tensor subclass: its own copy_ knows where the values go (self._sharded_param_data.copy_(...), :348)
+            if new_local is not self._sharded_local and self.sharded_numel > 0:
+                with torch.no_grad():
+                    self._sharded_local.copy_(new_local)
+        elif new_local.data_ptr() != self._sharded_param_data.data_ptr() and self.sharded_numel > 0:
             from . import _native
 
             if new_local.device != self._sharded_param_data.device or new_local.numel() != self.sharded_numel:
@@ -175,7 +272,7 @@ class YaFSDPParam:
                 )
             _native.flat_copy(self._sharded_param_data, new_local.contiguous().view(-1))
         self.sharded_param = nn.Parameter(
-            self.to_sharded_dtensor(self._sharded_param_data), requires_grad=self.sharded_param.requires_grad
+            self.to_sharded_dtensor(self._sharded_local), requires_grad=self.sharded_param.requires_grad
         )
         self.sharded_param._yafsdp_param = weakref.ref(self)
         self._setattr_on_modules(self.sharded_param)

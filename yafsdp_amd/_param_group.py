@@ -116,8 +116,6 @@ class YaFSDPParamGroup:
         if device.type != "cuda":
             raise RuntimeError(f"the buffer path runs on the GPU only, got device {device}")
         device = resolve_device(device)
-        if mp_policy.all_gather_dtype_to_param_cls:
-            raise NotImplementedError("per-class all-gather dtypes (tensor-subclass extensions) are not part of this build")
         names = list(names) if names is not None else [f"param{i}" for i in range(len(params))]
         self.modules = tuple(modules)
         infos = _get_param_module_infos(list(params), self.modules) if self.modules else [None] * len(params)
@@ -148,42 +146,71 @@ class YaFSDPParamGroup:
         self.grad_buffer_ctx = (
             YaFSDPBufferContext(YaFSDPBufferContext.BufferType.REDUCE_SCATTER) if param_group_requires_grad else None
         )
-        # one all-gather dtype class (key None), kept as dicts like the reference's
-        self._all_gather_dtype_to_fsdp_params: dict[torch.dtype | None, list[YaFSDPParam]] = {None: self.fsdp_params}
+        # all-gather dtype classes (ya_fsdp/_param_group.py:194-227): key None holds the ordinary parameters, whose
+        # all-gather dtype is the group's parameter dtype; every entry of the policy's all_gather_dtype_to_param_cls
+        # holds the parameters that are instances of that tensor subclass.  Each class has flat buffers, a layout
+        # and a table of its own; empty classes are dropped.
+        cls_map = mp_policy.all_gather_dtype_to_param_cls or {}
+        classes: dict[torch.dtype | None, list[YaFSDPParam]] = {
+            None: [p for p in self.fsdp_params if not any(isinstance(p.param_data, c) for c in cls_map.values())]
+        }
+        for all_gather_dtype, param_cls in cls_map.items():
+            classes[all_gather_dtype] = [p for p in self.fsdp_params if isinstance(p.param_data, param_cls)]
+        self._all_gather_dtype_to_fsdp_params: dict[torch.dtype | None, list[YaFSDPParam]] = {
+            dtype: params for dtype, params in classes.items() if params
+        }
+        if sum(map(len, self._all_gather_dtype_to_fsdp_params.values())) != len(self.fsdp_params):
+            raise AssertionError("a parameter is an instance of more than one class of all_gather_dtype_to_param_cls")
         self._all_gather_input_set_dtypes: set[torch.dtype | None] = set()
 
         world_size, rank = mesh_info.shard_mesh_size, mesh_info.shard_mesh_rank
-        numels = [p._orig_size.numel() for p in self.fsdp_params]
-        self.layout: ShardLayout = make_layout(numels, world_size, self.shard_alignment)  # :245-265
-        self._unsharded_param_numels = {None: numels}
-        self.padded_unsharded_param_numel = {None: self.layout.padded_unsharded_numel}
-        self._padded_sharded_param_numel = {None: self.layout.padded_sharded_numel}
-        shard = torch.zeros(self.layout.padded_sharded_numel, dtype=self.orig_dtype, device=device)
-        self._padded_sharded_param_data = {None: shard}
-        self._padded_sharded_param_grad = {None: torch.zeros_like(shard) if param_group_requires_grad else None}
-        sharded_numels = self.layout.sharded_numels(rank)  # :354-358, closed form
-        global_offsets = self.layout.global_offsets(rank)  # :359-377
-        per_rank = self.layout.per_rank_sharded_numels()  # :347-353
-        self._sharded_param_numels = {None: sharded_numels}
-        # flatten + shard (:300-339) without the full-size temporary: copy only the
-        # fragment of each parameter that this rank owns
-        pos = 0
-        grad_shard = self._padded_sharded_param_grad[None]
-        with torch.no_grad():
-            for fsdp_param, n, go, sn in zip(self.fsdp_params, sharded_numels, global_offsets, per_rank):
-                frag = shard[pos : pos + n]
-                if n > 0:
-                    _native.flat_copy(frag, fsdp_param.param_data.detach().view(-1)[go : go + n])
-                fsdp_param.init_sharded_param(
-                    frag, grad_shard[pos : pos + n] if grad_shard is not None else None, global_offset=go,
-                    shard_numels=sn,
-                )  # :379-406
-                pos += n
+        self.layouts: dict[torch.dtype | None, ShardLayout] = {}
+        self._unsharded_param_numels: dict[torch.dtype | None, list[int]] = {}
+        self.padded_unsharded_param_numel: dict[torch.dtype | None, int] = {}
+        self._padded_sharded_param_numel: dict[torch.dtype | None, int] = {}
+        self._padded_sharded_param_data: dict[torch.dtype | None, torch.Tensor] = {}
+        self._padded_sharded_param_grad: dict[torch.dtype | None, torch.Tensor | None] = {}
+        self._sharded_param_numels: dict[torch.dtype | None, list[int]] = {}
+        for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+            numels = [p._orig_size.numel() for p in fsdp_params]
+            layout = make_layout(numels, world_size, self.shard_alignment)  # :245-265
+            self.layouts[all_gather_dtype] = layout
+            self._unsharded_param_numels[all_gather_dtype] = numels
+            self.padded_unsharded_param_numel[all_gather_dtype] = layout.padded_unsharded_numel
+            self._padded_sharded_param_numel[all_gather_dtype] = layout.padded_sharded_numel
+            shard = torch.zeros(layout.padded_sharded_numel, dtype=self.orig_dtype, device=device)
+            self._padded_sharded_param_data[all_gather_dtype] = shard
+            grad_shard = torch.zeros_like(shard) if param_group_requires_grad else None
+            self._padded_sharded_param_grad[all_gather_dtype] = grad_shard
+            sharded_numels = layout.sharded_numels(rank)  # :354-358, closed form
+            global_offsets = layout.global_offsets(rank)  # :359-377
+            per_rank = layout.per_rank_sharded_numels()  # :347-353
+            self._sharded_param_numels[all_gather_dtype] = sharded_numels
+            # flatten + shard (:300-339) without the full-size temporary: copy only the
+            # fragment of each parameter that this rank owns
+            pos = 0
+            with torch.no_grad():
+                for fsdp_param, n, go, sn in zip(fsdp_params, sharded_numels, global_offsets, per_rank):
+                    frag = shard[pos : pos + n]
+                    if n > 0:
+                        src = fsdp_param.param_data.detach().view(-1)[go : go + n]
+                        if type(src) is torch.Tensor:
+                            _native.flat_copy(frag, src)
+                        else:
+                            # a tensor subclass: only its own dispatch knows how its values become a plain tensor
+                            # (unsharded_param_data.copy_(fsdp_param.param_data.view(-1)), :324)
+                            frag.copy_(src)
+                    fsdp_param.init_sharded_param(
+                        frag, grad_shard[pos : pos + n] if grad_shard is not None else None, global_offset=go,
+                        shard_numels=sn,
+                    )  # :379-406
+                    pos += n
         for index, fsdp_param in enumerate(self.fsdp_params):
             fsdp_param._param_group_ref = weakref.ref(self)
             fsdp_param._index_in_group = index
-        self._table: _native.TensorTable | None = None
-        self._fragment_table: _native.TensorTable | None = None  # this rank's fragments of the gradient shard
+        self._tables: dict[torch.dtype | None, _native.TensorTable] = {}
+        # this rank's fragments of each class's gradient shard (built on first use, ya_fsdp/_collectives.py:191-214)
+        self._fragment_tables: dict[torch.dtype | None, _native.TensorTable] = {}
         self._state_dict_hook_handles: list = []
         # version of the master shard at which a fused optimizer step last wrote the
         # all-gather input (None: never); see all_gather
@@ -221,31 +248,82 @@ class YaFSDPParamGroup:
     def reduce_scatter_dtype(self) -> torch.dtype:
         return self.reduce_dtype or self.param_dtype or self.orig_dtype
 
+    def _ag_dtype(self, all_gather_dtype: torch.dtype | None) -> torch.dtype:
+        """Element type of a class's all-gather input and gathered buffer (ya_fsdp/_param_group.py:420)."""
+        return all_gather_dtype or self.param_dtype or self.orig_dtype
+
+    # the default class (ordinary parameters), for callers that deal with one class only
+    @property
+    def has_extension_classes(self) -> bool:
+        return any(dtype is not None for dtype in self._all_gather_dtype_to_fsdp_params)
+
+    def _default_class(self, what: str) -> None:
+        if None not in self._all_gather_dtype_to_fsdp_params:
+            raise NotImplementedError(
+                f"{what}: every parameter of {self} belongs to a tensor-subclass all-gather dtype class "
+                f"({list(self._all_gather_dtype_to_fsdp_params)}); use the per-class dictionaries"
+            )
+
+    @property
+    def layout(self) -> ShardLayout:
+        self._default_class("layout")
+        return self.layouts[None]
+
+    @property
+    def _table(self) -> "_native.TensorTable | None":
+        return self._tables.get(None)
+
+    @property
+    def _fragment_table(self) -> "_native.TensorTable | None":
+        return self._fragment_tables.get(None)
+
+    def data_buffer_bytes_by_dtype(self) -> dict[torch.dtype | None, int]:
+        """Bytes of the gathered buffer of every all-gather dtype class (ya_fsdp/_state.py:234-251)."""
+        return {
+            dtype: numel * self._ag_dtype(dtype).itemsize for dtype, numel in self.padded_unsharded_param_numel.items()
+        }
+
+    def grad_buffer_bytes_by_dtype(self) -> dict[torch.dtype | None, int]:
+        """Bytes of the reduce buffer of every all-gather dtype class (ya_fsdp/_state.py:265-284)."""
+        return {
+            dtype: numel * self.reduce_scatter_dtype.itemsize
+            for dtype, numel in self.padded_unsharded_param_numel.items()
+        }
+
     def data_buffer_bytes(self) -> int:
-        return self.layout.padded_unsharded_numel * self.all_gather_dtype.itemsize
+        self._default_class("data_buffer_bytes")
+        return self.data_buffer_bytes_by_dtype()[None]
 
     def grad_buffer_bytes(self) -> int:
-        return self.layout.padded_unsharded_numel * self.reduce_scatter_dtype.itemsize
+        self._default_class("grad_buffer_bytes")
+        return self.grad_buffer_bytes_by_dtype()[None]
 
     def _init_unsharded_params(self) -> None:
         """ya_fsdp/_param_group.py:409-457: typed views of the shared byte buffers,
         split into per-parameter views (the zero-copy copy-out)."""
-        t_pad, total = self.layout.padded_unsharded_numel, self.layout.total_numel
-        numels = self._unsharded_param_numels[None]
-        ag = self.data_buffer_ctx.buffers[None].narrow(0, 0, self.data_buffer_bytes()).view(self.all_gather_dtype)
-        self._all_gather_output = {None: ag}
-        if self.grad_buffer_ctx is not None:
-            rs = self.grad_buffer_ctx.buffers[None].narrow(0, 0, self.grad_buffer_bytes()).view(
-                self.reduce_scatter_dtype
+        self._all_gather_output = {}
+        self._reduce_scatter_input = {}
+        data_bytes, grad_bytes = self.data_buffer_bytes_by_dtype(), self.grad_buffer_bytes_by_dtype()
+        for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+            layout = self.layouts[all_gather_dtype]
+            t_pad, total = layout.padded_unsharded_numel, layout.total_numel
+            numels = self._unsharded_param_numels[all_gather_dtype]
+            ag = self.data_buffer_ctx.buffers[all_gather_dtype].narrow(0, 0, data_bytes[all_gather_dtype]).view(
+                self._ag_dtype(all_gather_dtype)
             )
-        else:
-            rs = None
-        self._reduce_scatter_input = {None: rs}
-        assert ag.numel() == t_pad
-        ag_views = ag[:total].split(numels)
-        rs_views = rs[:total].split(numels) if rs is not None else (None,) * len(numels)
-        for fsdp_param, v, g in zip(self.fsdp_params, ag_views, rs_views):
-            fsdp_param.init_unsharded_param(v, g)
+            self._all_gather_output[all_gather_dtype] = ag
+            if self.grad_buffer_ctx is not None:
+                rs = self.grad_buffer_ctx.buffers[all_gather_dtype].narrow(0, 0, grad_bytes[all_gather_dtype]).view(
+                    self.reduce_scatter_dtype
+                )
+            else:
+                rs = None
+            self._reduce_scatter_input[all_gather_dtype] = rs
+            assert ag.numel() == t_pad
+            ag_views = ag[:total].split(numels)
+            rs_views = rs[:total].split(numels) if rs is not None else (None,) * len(numels)
+            for fsdp_param, v, g in zip(fsdp_params, ag_views, rs_views):
+                fsdp_param.init_unsharded_param(v, g)
 
     def _validate_no_meta_params(self) -> None:
         """ya_fsdp/_param_group.py:939-951."""
@@ -264,33 +342,39 @@ class YaFSDPParamGroup:
         """ya_fsdp/_param_group.py:487-547 (idempotent)."""
         if not hasattr(self.comm_ctx, "all_gather_stream"):
             self.comm_ctx.lazy_init(self.device)
-        if None not in self.data_buffer_ctx.buffers:
+        if any(dtype not in self.data_buffer_ctx.buffers for dtype in self._all_gather_dtype_to_fsdp_params):
             raise RuntimeError(
                 "the data buffer of this group is not allocated: call init_shared_state(groups, device) first"
             )
         self._validate_no_meta_params()  # :491
         self._register_state_dict_hooks()  # :492
         self._init_unsharded_params()
-        shard = self._padded_sharded_param_data[None]
-        sharded_numels = self._sharded_param_numels[None]
-        n_local = sum(sharded_numels)
-        ag_in = shard if self.param_dtype is None else torch.zeros_like(shard, dtype=self.param_dtype)  # :502-508
-        self._all_gather_input = {None: ag_in}
-        for fsdp_param, frag in zip(self.fsdp_params, ag_in[:n_local].split(sharded_numels)):
-            fsdp_param.init_all_gather_input(frag)
+        self._all_gather_input = {}
         self._reduce_scatter_output = {}
-        if self.grad_buffer_ctx is not None:
-            rs = self._reduce_scatter_input[None]
-            s = self.layout.padded_sharded_numel
-            r = self.mesh_info.shard_mesh_rank
-            rs_out = rs[r * s : (r + 1) * s]  # chunk(W)[r], :531-535
-            self._reduce_scatter_output[None] = rs_out
-            for fsdp_param, frag in zip(self.fsdp_params, rs_out[:n_local].split(sharded_numels)):
-                fsdp_param.init_reduce_scatter_output(frag)
-        if self._table is None:
-            self._table = _native.TensorTable(
-                self._unsharded_param_numels[None], self.layout.padded_unsharded_numel, self.device
-            )
+        for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+            shard = self._padded_sharded_param_data[all_gather_dtype]
+            sharded_numels = self._sharded_param_numels[all_gather_dtype]
+            n_local = sum(sharded_numels)
+            if all_gather_dtype is None and self.param_dtype is None:
+                ag_in = shard  # :502-505
+            else:
+                ag_in = torch.zeros_like(shard, dtype=all_gather_dtype or self.param_dtype)  # :506-508
+            self._all_gather_input[all_gather_dtype] = ag_in
+            for fsdp_param, frag in zip(fsdp_params, ag_in[:n_local].split(sharded_numels)):
+                fsdp_param.init_all_gather_input(frag)
+            if self.grad_buffer_ctx is not None:
+                rs = self._reduce_scatter_input[all_gather_dtype]
+                s = self.layouts[all_gather_dtype].padded_sharded_numel
+                r = self.mesh_info.shard_mesh_rank
+                rs_out = rs[r * s : (r + 1) * s]  # chunk(W)[r], :531-535
+                self._reduce_scatter_output[all_gather_dtype] = rs_out
+                for fsdp_param, frag in zip(fsdp_params, rs_out[:n_local].split(sharded_numels)):
+                    fsdp_param.init_reduce_scatter_output(frag)
+            if all_gather_dtype not in self._tables:
+                self._tables[all_gather_dtype] = _native.TensorTable(
+                    self._unsharded_param_numels[all_gather_dtype],
+                    self.layouts[all_gather_dtype].padded_unsharded_numel, self.device,
+                )
 
     # ------------------------------------------------------------------- runtime --
     @property
@@ -422,37 +506,44 @@ class YaFSDPParamGroup:
                 current_stream.wait_event(release_event)
                 grad_buffer_ctx.release_event = None
             grad_buffer_ctx.owner = self
-        predivide_fused = False
+        predivide_fused: dict[torch.dtype | None, bool] = {}
         reduced_in_one_launch = False
         with profiler_range(self._with_fqn("FSDP::post_backward_accumulate")):
-            grads: list[torch.Tensor | None] = []
-            modes: list[int] = []
-            for fsdp_param in self.fsdp_params:
-                has_grad = fsdp_param.requires_grad and fsdp_param.unsharded_param.grad is not None
-                if has_grad and fsdp_param.unsharded_accumulated_grad is None:
-                    grads.append(fsdp_param.unsharded_grad_data)
-                    modes.append(MODE_COPY)  # _foreach_copy_, :693-700
-                    fsdp_param.unsharded_param.grad = None
-                    fsdp_param.unsharded_accumulated_grad = fsdp_param._unsharded_accumulated_grad
-                elif has_grad:
-                    grads.append(fsdp_param.unsharded_grad_data)
-                    modes.append(MODE_ADD)  # _foreach_add_, :701-708
-                    fsdp_param.unsharded_param.grad = None
-                else:
-                    grads.append(None)
-                    modes.append(MODE_SKIP)
-            if any(m != MODE_SKIP for m in modes):
-                assert grad_buffer_ctx is not None and self._table is not None
+            single_class = len(self._all_gather_dtype_to_fsdp_params) == 1
+            for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+                grads: list[torch.Tensor | None] = []
+                modes: list[int] = []
+                for fsdp_param in fsdp_params:
+                    has_grad = fsdp_param.requires_grad and fsdp_param.unsharded_param.grad is not None
+                    if has_grad and fsdp_param.unsharded_accumulated_grad is None:
+                        grads.append(fsdp_param.unsharded_grad_data)
+                        modes.append(MODE_COPY)  # _foreach_copy_, :693-700
+                        fsdp_param.unsharded_param.grad = None
+                        fsdp_param.unsharded_accumulated_grad = fsdp_param._unsharded_accumulated_grad
+                    elif has_grad:
+                        grads.append(fsdp_param.unsharded_grad_data)
+                        modes.append(MODE_ADD)  # _foreach_add_, :701-708
+                        fsdp_param.unsharded_param.grad = None
+                    else:
+                        grads.append(None)
+                        modes.append(MODE_SKIP)
+                if not any(m != MODE_SKIP for m in modes):
+                    continue
+                assert grad_buffer_ctx is not None and all_gather_dtype in self._tables
                 pre = None
                 if self.reduce_grads:
                     pre, _, _, _ = _get_gradient_divide_factors(
                         self._reduce_scatter_process_group, self.reduce_scatter_dtype, self.gradient_divide_factor,
                         self.force_sum_reduction_for_comms,
                     )
-                    predivide_fused = True
-                    reduced_in_one_launch = self._reduce_in_one_launch(grads, modes)
+                    predivide_fused[all_gather_dtype] = True
+                    if single_class and all_gather_dtype is None:
+                        reduced_in_one_launch = self._reduce_in_one_launch(grads, modes)
                 if not reduced_in_one_launch:
-                    foreach_reduce_copy_in(self, self._table, self._reduce_scatter_input[None], grads, modes, pre)
+                    foreach_reduce_copy_in(
+                        self, self._tables[all_gather_dtype], self._reduce_scatter_input[all_gather_dtype], grads,
+                        modes, pre,
+                    )
         fsdp_params_with_grad_per_dtype: dict[torch.dtype | None, list[YaFSDPParam]] = {}
         with profiler_range(self._with_fqn("YaFSDP::post_backward_reshard")):
             if not self.reduce_grads:
@@ -485,6 +576,8 @@ class YaFSDPParamGroup:
             return
         with profiler_range(self._with_fqn("YaFSDP::post_backward_reduce")):
             for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+                if not fsdp_params_with_grad_per_dtype[all_gather_dtype]:
+                    continue  # nothing of this class took part in the pass: its reduce buffer holds no gradient
                 self._post_reduce_event = reduce_scatter(
                     fsdp_params,
                     fsdp_params_with_grad_per_dtype[all_gather_dtype],
@@ -500,7 +593,7 @@ class YaFSDPParamGroup:
                     self.force_sum_reduction_for_comms,
                     self.mp_policy.bit32_acc_for_bit16_reduce_scatter,
                     None,
-                    predivide_fused=predivide_fused,
+                    predivide_fused=predivide_fused.get(all_gather_dtype, False),
                 )
         grad_buffer_ctx.release_event = self._post_reduce_event
         grad_buffer_ctx.owner = None
@@ -516,7 +609,7 @@ class YaFSDPParamGroup:
         if group.size() != 1 or self._grad_sumsq_slot is not None:
             return False
         if list(self._all_gather_dtype_to_fsdp_params) != [None] or self._table is None:
-            return False
+            return False  # one launch per group: only for a group with the default class alone
         need = [p for p in self.fsdp_params if p.sharded_param.requires_grad]
         in_sharded = (
             (self.reduce_dtype is None and self.param_dtype is None) or self.reduce_dtype == self.orig_dtype
@@ -549,6 +642,15 @@ class YaFSDPParamGroup:
             grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes,
             pre_factor=pre, post_factor=post, custom_divisor=custom,
         )
+
+    def _fragment_table_for(self, grad_shard: torch.Tensor, numels: "list[int]") -> "_native.TensorTable":
+        """Table over one class's gradient shard whose tensors are this rank's fragments (for the mixed copy /
+        accumulate case of ya_fsdp/_collectives.py:191-214); built on first use."""
+        key = next(k for k, v in self._padded_sharded_param_grad.items() if v is grad_shard)
+        table = self._fragment_tables.get(key)
+        if table is None:
+            table = self._fragment_tables[key] = _native.TensorTable(numels, grad_shard.numel(), grad_shard.device)
+        return table
 
     def finalize_backward(self) -> None:
         """ya_fsdp/_param_group.py:773-783."""
@@ -601,6 +703,8 @@ class YaFSDPParamGroup:
         launch).  The group's own unsharded parameters are zero-copy views
         (``_init_unsharded_params``); this is for consumers that need their own
         storage.  Runs on the current stream; call after ``wait_for_unshard``."""
+        if self.has_extension_classes:
+            raise NotImplementedError("copy_out_materialize serves groups with the default all-gather dtype class only")
         assert self._table is not None, "lazy_init() first"
         self._table.scatter_out(self._all_gather_output[None], [o.view(-1) if o is not None else None for o in outs])
 
@@ -718,14 +822,16 @@ def init_shared_state(
         for i, g in enumerate(groups):
             users[i % n].append(g)
         for ctx, gs in zip(ctxs, users):
-            ctx.lazy_init({None: max(size_of(g) for g in gs)}, device)
+            sizes = [size_of(g) for g in gs]  # bytes per all-gather dtype class
+            dtypes = {dtype for per_dtype in sizes for dtype in per_dtype}
+            ctx.lazy_init({dtype: max(per_dtype.get(dtype, 0) for per_dtype in sizes) for dtype in dtypes}, device)
             for g in gs:
                 setattr(g, attr, ctx)
 
-    assign(list(param_groups), "data_buffer_ctx", num_data_buffers, lambda g: g.data_buffer_bytes())
+    assign(list(param_groups), "data_buffer_ctx", num_data_buffers, lambda g: g.data_buffer_bytes_by_dtype())
     assign(
         [g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx", num_grad_buffers,
-        lambda g: g.grad_buffer_bytes(),
+        lambda g: g.grad_buffer_bytes_by_dtype(),
     )
     for g in param_groups:
         g.comm_ctx = comm_ctx

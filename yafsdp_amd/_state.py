@@ -197,20 +197,23 @@ class YaFSDPState(_State):
                 for i, g in enumerate(groups):
                     users[i % n].append(g)
             for ctx, gs in zip(ctxs, users):
-                ctx.lazy_init({None: max(size_of(g) for g in gs)}, self._device)
+                sizes = [size_of(g) for g in gs]  # bytes per all-gather dtype class (:234-251, :265-284)
+                dtypes = {dtype for per_dtype in sizes for dtype in per_dtype}
+                ctx.lazy_init({dtype: max(per_dtype.get(dtype, 0) for per_dtype in sizes) for dtype in dtypes},
+                              self._device)
                 for g in gs:
                     setattr(g, attr, ctx)
             return users
 
         data_users = assign(param_groups, "data_buffer_ctx", None if no_reshard_after_forward else 2,
-                            lambda g: g.data_buffer_bytes(), param_group_to_data_buffer_ctx_idx)
+                            lambda g: g.data_buffer_bytes_by_dtype(), param_group_to_data_buffer_ctx_idx)
         for state_groups in data_users:
             last = state_groups[-1]
             owner_state = next(s for s in self._state_ctx.all_states if s._fsdp_param_group is last)
             if owner_state._auto_reshard_after_forward:
                 last.reshard_after_forward = False  # ya_fsdp/_state.py:256-260
         assign([g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx",
-               None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes(),
+               None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes_by_dtype(),
                param_group_to_grad_buffer_ctx_idx)
 
     def validate_shared_state(self) -> None:

@@ -73,6 +73,14 @@ def local_tensor(t: torch.Tensor) -> torch.Tensor:
     return t._local_tensor if isinstance(t, RaggedShardDTensor) else t
 
 
+def plain_tensor(t: torch.Tensor) -> torch.Tensor:
+    """The plain tensor at the bottom of a local fragment: a tensor-subclass parameter is sharded as an instance of
+    its subclass whose first inner tensor is the fragment of the flat shard (ya_fsdp/_param.py:145-152)."""
+    while type(t) not in (torch.Tensor, torch.nn.Parameter) and hasattr(t, "__tensor_flatten__"):
+        t = getattr(t, t.__tensor_flatten__()[0][0])
+    return t
+
+
 def _locals(ts: Sequence[torch.Tensor]) -> list[torch.Tensor]:
     return [local_tensor(t) for t in ts]
 
@@ -244,11 +252,12 @@ class RaggedShardDTensor(torch.Tensor):
 
         placement = self._spec.placements[0]
         shard_numels = placement.shard_numels
-        full = self._local_tensor.new_empty(sum(shard_numels))
+        own = plain_tensor(self._local_tensor)
+        full = own.new_empty(sum(shard_numels))
         rank = self._spec.mesh.shard_mesh_rank
         pieces = full.split(list(shard_numels))
         if len(shard_numels) == 1:
-            locals_by_rank = [self._local_tensor]
+            locals_by_rank = [own]
         else:
             owner = self._spec.owner() if self._spec.owner is not None else None
             peers = getattr(owner, "_logical_peers", None)
@@ -265,9 +274,9 @@ class RaggedShardDTensor(torch.Tensor):
                 if peer is None:
                     raise RuntimeError(f"logical rank {k} of this parameter no longer exists")
                 if k == rank:
-                    locals_by_rank.append(self._local_tensor)
+                    locals_by_rank.append(own)
                 elif self._spec.kind == "grad":
-                    locals_by_rank.append(peer.sharded_param_grad._local_tensor)
+                    locals_by_rank.append(plain_tensor(peer.sharded_param_grad._local_tensor))
                 else:
                     locals_by_rank.append(peer._sharded_param_data)
         for piece, src in zip(pieces, locals_by_rank):

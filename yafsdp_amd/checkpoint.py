@@ -198,9 +198,19 @@ class RaggedShardLoadPlanner(_load_planner_base()):  # type: ignore[misc]
             self.state_dict = real
 
 
+def _one_class(group: YaFSDPParamGroup) -> None:
+    if group.has_extension_classes:
+        raise NotImplementedError(
+            f"{group} has tensor-subclass all-gather dtype classes (all_gather_dtype_to_param_cls), each with a flat "
+            "shard of its own: the whole-group helpers cover groups with the default class only; "
+            "sharded_state_dict, full_state_dict and the sharded parameters' own checkpoint hooks work per parameter"
+        )
+
+
 def group_meta_info(group: YaFSDPParamGroup) -> dict[str, list]:
     """The per-module record the legacy wrapper keeps in its state dict
     (ya_fsdp/ya_fsdp.py:236-245), for one group."""
+    _one_class(group)
     return {
         "shard_boundaries": list(group.layout.rank_range(group.mesh_info.shard_mesh_rank)),
         "padded_numel": group.layout.padded_unsharded_numel,
@@ -211,6 +221,8 @@ def group_meta_info(group: YaFSDPParamGroup) -> dict[str, list]:
 
 
 def _check_ranks(groups: Sequence[YaFSDPParamGroup]) -> None:
+    for g in groups:
+        _one_class(g)
     w = groups[0].layout.world_size
     if len(groups) != w:
         raise ValueError(f"need the groups of all {w} ranks, got {len(groups)}")

@@ -53,6 +53,24 @@ def fsdp_param_groups(modules: nn.Module | Iterable[nn.Module]) -> list[YaFSDPPa
     return groups
 
 
+def _flat_groups(modules: nn.Module | Iterable[nn.Module]) -> list[YaFSDPParamGroup]:
+    """``fsdp_param_groups`` for the passes of this module, which run over ONE flat shard per group: a group whose
+    policy gives tensor-subclass parameters an all-gather dtype class of their own has several."""
+    groups = fsdp_param_groups(modules)
+    for g in groups:
+        _require_one_class(g)
+    return groups
+
+
+def _require_one_class(group: YaFSDPParamGroup) -> None:
+    if group.has_extension_classes:
+        raise NotImplementedError(
+            f"{group} has tensor-subclass all-gather dtype classes (all_gather_dtype_to_param_cls): the flat "
+            "optimizer-side passes cover groups with the default class only; torch.optim and "
+            "torch.nn.utils.clip_grad_norm_ work on its sharded parameters"
+        )
+
+
 def _owner(param: torch.Tensor) -> YaFSDPParam | None:
     ref = getattr(param, "_yafsdp_param", None)
     return ref() if ref is not None else None
@@ -141,7 +159,7 @@ def enable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
     the reduce (seen through the shard's version counter), or one of this
     module's own passes that rewrites gradients (scaling, zero-fill).  Kernels
     launched on the gradient shard through ``_native`` directly are not seen."""
-    groups = [g for g in fsdp_param_groups(modules) if g._padded_sharded_param_grad[None] is not None]
+    groups = [g for g in _flat_groups(modules) if g._padded_sharded_param_grad[None] is not None]
     if not groups:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
     device = groups[0].device
@@ -191,7 +209,7 @@ def grad_clip_coef(
     buffer and must be ordered on one stream."""
     if norm_type not in (2, 2.0):
         raise NotImplementedError("only the 2-norm is implemented (ya_fsdp/ya_fsdp.py:544)")
-    groups = [g for g in fsdp_param_groups(modules) if g._padded_sharded_param_grad[None] is not None]
+    groups = [g for g in _flat_groups(modules) if g._padded_sharded_param_grad[None] is not None]
     if not groups:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
     device = groups[0].device
@@ -237,7 +255,7 @@ def clip_grad_norm_(
     traffic when nothing is clipped (coefficient exactly 1)."""
     total_norm, coef = grad_clip_coef(modules, max_norm, norm_type)
     coef = coef.view(1)
-    for group in fsdp_param_groups(modules):
+    for group in _flat_groups(modules):
         grad_shard = group._padded_sharded_param_grad[None]
         if grad_shard is None:
             continue
@@ -249,7 +267,7 @@ def clip_grad_norm_(
 
 def zero_grad(modules: nn.Module | Iterable[nn.Module]) -> None:
     """``zero_grad(set_to_none=False)``: one fill per group over its flat gradient shard."""
-    for group in fsdp_param_groups(modules):
+    for group in _flat_groups(modules):
         grad_shard = group._padded_sharded_param_grad[None]
         if grad_shard is not None:
             group._grad_sumsq_token = None
@@ -265,6 +283,7 @@ class _Unit:
         self.params = params
         self.indices = indices  # position of each parameter in group.fsdp_params
         if group is not None:
+            _require_one_class(group)
             shard = group._padded_sharded_param_data[None]
             if shard.dtype != torch.float32:
                 raise TypeError(f"FlatAdamW needs float32 master shards, got {shard.dtype} in {group}")
