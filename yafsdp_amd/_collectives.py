@@ -76,9 +76,9 @@ def all_gather(
     all_gather_dtype: torch.dtype | None,
     yccl_handle: Optional[Any],
 ) -> AllGatherResult:
-    """ya_fsdp/_collectives.py:31-76."""
-    if yccl_handle is not None:
-        raise NotImplementedError("YCCL handles are not part of this build")
+    """ya_fsdp/_collectives.py:31-76.  ``yccl_handle``: a communication library that owns the all-gather input
+    and the gathered buffer of this class and performs the exchange itself (``all_gather(input, output)`` on bf16
+    views of both, :67-70); the copy-in into its input buffer stays here."""
     with torch.cuda.stream(all_gather_stream):
         if all_gather_dtype is None:
             if (
@@ -99,17 +99,21 @@ def all_gather(
         if all_gather_dtype not in param_group._all_gather_input_set_dtypes:
             for fsdp_param in fsdp_params:
                 fsdp_param.set_all_gather_input()
-            if all_gather_dtype is None and param_dtype is not None:
-                # copy-in: cast the master shard (:53-54) and, in the same pass over it, place the result where
-                # the all-gather would (:56-58, :60-65); the version counter of the destination is untouched
-                # because no autograd op is involved
-                if all(t.data_ptr() % 16 == 0 for t in (slot, all_gather_input, padded_sharded_param_data)):
+            if all_gather_dtype is None and (param_dtype is not None or yccl_handle is not None):
+                # copy-in: cast the master shard (:53-54; into a handle's buffer also without a cast, :50-52) and,
+                # in the same pass over it, place the result where the all-gather would (:56-58, :60-65); the
+                # version counter of the destination is untouched because no autograd op is involved
+                if yccl_handle is not None and world_size > 1:
+                    _native.flat_copy(all_gather_input, padded_sharded_param_data)  # the handle places it
+                elif all(t.data_ptr() % 16 == 0 for t in (slot, all_gather_input, padded_sharded_param_data)):
                     _native.flat_copy_fanout([all_gather_input, slot], padded_sharded_param_data)
                     placed = True
                 else:
                     _native.flat_copy(all_gather_input, padded_sharded_param_data)
             param_group._all_gather_input_set_dtypes.add(all_gather_dtype)
-        if not placed:
+        if yccl_handle is not None and world_size > 1:
+            yccl_handle.all_gather(all_gather_input.view(torch.bfloat16), all_gather_output.view(torch.bfloat16))  # :67-70
+        elif not placed:
             # size-1 group (:56-58), or this rank's share of all_gather_into_tensor (:60-65)
             _native.flat_copy(slot, all_gather_input)
         all_gather_work = None
@@ -169,8 +173,9 @@ def reduce_scatter(
     ``predivide_fused``: the caller already applied the pre-divide inside the
     reduce copy-in launch (``foreach_reduce_copy_in``), so it is skipped here.
     """
-    if yccl_handle is not None:
-        raise NotImplementedError("YCCL handles are not part of this build")
+    # ``yccl_handle``: the communication library that owns the reduce buffer reduces it in place
+    # (``reduce_scatter(buffer)`` on its bf16 view, :163-164: a sum, which is why the divide factors then put the
+    # whole division after it, :229-230); this rank's chunk of the buffer holds the result afterwards.
     # bit32_acc_for_bit16_reduce_scatter only reaches the collective (acc_type=, :157-161) and is unused for a
     # group of size 1 (:140-150).  Here this rank's chunk is the only contribution to its reduce-scatter output,
     # and a binary32 sum of one 16-bit value rounds back to that value, so the flag changes nothing; the sum over
@@ -212,6 +217,8 @@ def reduce_scatter(
         else:
             # this rank's share of reduce_scatter_tensor (:152-162): its chunk, divided as the
             # collective would have (AVG: by the group size; pre-multiplied sum: by the factor)
+            if yccl_handle is not None:
+                yccl_handle.reduce_scatter(padded_unsharded_param_grad.view(torch.bfloat16))  # :163-164
             if reduce_scatter_op == "AVG":
                 collective_divide = float(world_size)
             elif reduce_scatter_op == "PREMUL_SUM":

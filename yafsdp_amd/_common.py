@@ -36,6 +36,14 @@ class LogicalShardGroup:
     def __repr__(self) -> str:
         return f"LogicalShardGroup(size={self._size}, rank={self._rank})"
 
+    # two logical groups of equal size and rank are the same group (every fully_shard call builds its own
+    # object), so dictionaries keyed by "the process group" work as they do with real process groups
+    def __eq__(self, other: object) -> bool:
+        return isinstance(other, LogicalShardGroup) and (self._size, self._rank) == (other._size, other._rank)
+
+    def __hash__(self) -> int:
+        return hash((LogicalShardGroup, self._size, self._rank))
+
 
 @dataclass
 class FSDPMeshInfo:

@@ -66,20 +66,52 @@ class YaFSDPBufferContext:
     def __init__(self, buffer_type: "YaFSDPBufferContext.BufferType"):
         self._buffer_type = buffer_type
         self.buffers: dict[torch.dtype | None, torch.Tensor] = {}
+        self.yccl_handles: dict[torch.dtype | None, Any] = {}
         self.owner: YaFSDPParamGroup | None = None
         self.release_event: torch.cuda.Event | None = None
 
-    def lazy_init(self, sizes_by_dtype: "dict[torch.dtype | None, int]", device: torch.device) -> None:
-        # byte buffers allocated as bf16 and re-viewed, as at :53-69; zero-filled
-        # so that pad lanes are defined from the first use on
-        self.buffers = {
-            dtype: torch.zeros(
-                (size_in_bytes + 1) // torch.bfloat16.itemsize, dtype=torch.bfloat16, device=device
-            ).view(torch.uint8)
-            for dtype, size_in_bytes in sizes_by_dtype.items()
-        }
+    def lazy_init(
+        self,
+        sizes_by_dtype: "dict[torch.dtype | None, int]",
+        device: torch.device,
+        yccl_handles: "dict[torch.dtype | None, Any] | None" = None,
+    ) -> None:
+        """Byte buffers allocated as bf16 and re-viewed, as at :53-69.  A communication handle registered for a
+        dtype class owns that class's buffer (``add_all_gather_output_buffer`` / ``add_reduce_scatter_buffer``,
+        each returning a bf16 tensor of the requested length).  All buffers start zero-filled so that pad lanes
+        are defined from the first use on."""
+        if yccl_handles is None:
+            yccl_handles = dict.fromkeys(sizes_by_dtype)
+        self.yccl_handles = yccl_handles
+        buffer_method = {
+            self.BufferType.ALL_GATHER: "add_all_gather_output_buffer",
+            self.BufferType.REDUCE_SCATTER: "add_reduce_scatter_buffer",
+        }[self._buffer_type]
+        self.buffers = {}
+        for dtype, size_in_bytes in sizes_by_dtype.items():
+            numel = (size_in_bytes + 1) // torch.bfloat16.itemsize
+            if (handle := yccl_handles.get(dtype)) is None:
+                buffer = torch.zeros(numel, dtype=torch.bfloat16, device=device)
+            else:
+                buffer = getattr(handle, buffer_method)(numel)
+                _check_handle_buffer(buffer, numel, device, buffer_method)
+                if numel > 0:
+                    _native.flat_fill(buffer, 0.0)
+            self.buffers[dtype] = buffer.view(torch.uint8)
         self.owner = None
         self.release_event = None
+
+
+def _check_handle_buffer(buffer: Any, numel: int, device: torch.device, method: str) -> None:
+    if (
+        not isinstance(buffer, torch.Tensor) or buffer.dtype != torch.bfloat16 or buffer.numel() != numel
+        or buffer.device != device or not buffer.is_contiguous()
+    ):
+        raise TypeError(
+            f"{method}({numel}) of the communication handle must return a contiguous bfloat16 tensor of {numel} "
+            f"elements on {device}, got {type(buffer).__name__}"
+            + (f" {buffer.dtype} {tuple(buffer.shape)} on {buffer.device}" if isinstance(buffer, torch.Tensor) else "")
+        )
 
 
 class YaFSDPCommContext:
@@ -355,7 +387,17 @@ class YaFSDPParamGroup:
             shard = self._padded_sharded_param_data[all_gather_dtype]
             sharded_numels = self._sharded_param_numels[all_gather_dtype]
             n_local = sum(sharded_numels)
-            if all_gather_dtype is None and self.param_dtype is None:
+            yccl_handle = self.data_buffer_ctx.yccl_handles.get(all_gather_dtype)
+            if yccl_handle is not None:
+                # the communication library owns the buffer it gathers from (:510-519)
+                ag_dtype = self._ag_dtype(all_gather_dtype)
+                numel = shard.numel() * ag_dtype.itemsize // torch.bfloat16.itemsize
+                buffer = yccl_handle.add_all_gather_input_buffer(numel)
+                _check_handle_buffer(buffer, numel, self.device, "add_all_gather_input_buffer")
+                if numel > 0:
+                    _native.flat_fill(buffer, 0.0)
+                ag_in = buffer.view(ag_dtype)
+            elif all_gather_dtype is None and self.param_dtype is None:
                 ag_in = shard  # :502-505
             else:
                 ag_in = torch.zeros_like(shard, dtype=all_gather_dtype or self.param_dtype)  # :506-508
@@ -416,7 +458,7 @@ class YaFSDPParamGroup:
                     self.device,
                     self.param_dtype,
                     all_gather_dtype,
-                    None,
+                    self.data_buffer_ctx.yccl_handles.get(all_gather_dtype),
                 )
 
     def wait_for_unshard(self) -> AllGatherResult | None:
@@ -535,6 +577,7 @@ class YaFSDPParamGroup:
                     pre, _, _, _ = _get_gradient_divide_factors(
                         self._reduce_scatter_process_group, self.reduce_scatter_dtype, self.gradient_divide_factor,
                         self.force_sum_reduction_for_comms,
+                        yccl_handle=grad_buffer_ctx.yccl_handles.get(all_gather_dtype),
                     )
                     predivide_fused[all_gather_dtype] = True
                     if single_class and all_gather_dtype is None:
@@ -592,7 +635,7 @@ class YaFSDPParamGroup:
                     self.gradient_divide_factor,
                     self.force_sum_reduction_for_comms,
                     self.mp_policy.bit32_acc_for_bit16_reduce_scatter,
-                    None,
+                    grad_buffer_ctx.yccl_handles.get(all_gather_dtype),
                     predivide_fused=predivide_fused.get(all_gather_dtype, False),
                 )
         grad_buffer_ctx.release_event = self._post_reduce_event
@@ -610,6 +653,8 @@ class YaFSDPParamGroup:
             return False
         if list(self._all_gather_dtype_to_fsdp_params) != [None] or self._table is None:
             return False  # one launch per group: only for a group with the default class alone
+        if self.grad_buffer_ctx is None or self.grad_buffer_ctx.yccl_handles.get(None) is not None:
+            return False  # a communication handle owns the reduce: the general route calls it
         need = [p for p in self.fsdp_params if p.sharded_param.requires_grad]
         in_sharded = (
             (self.reduce_dtype is None and self.param_dtype is None) or self.reduce_dtype == self.orig_dtype
@@ -799,14 +844,15 @@ class RegisterPostBackwardFunction(torch.autograd.Function):
 
 def init_shared_state(
     param_groups: Sequence[YaFSDPParamGroup], device: torch.device, num_data_buffers: int | None = 2,
-    num_grad_buffers: int | None = 1,
+    num_grad_buffers: int | None = 1, yccl_handle: Any | None = None,
 ) -> None:
     """Buffer assignment of ya_fsdp/_state.py:200-288 and :617-678 for groups
     that share one shard group: one communication context, ``num_data_buffers``
     data buffers handed out round-robin in group order, ``num_grad_buffers``
     gradient buffers; each buffer is as large as the largest group using it.
-    ``None`` gives every group its own buffer.  Ends with ``lazy_init`` of each
-    group."""
+    ``None`` gives every group its own buffer.  ``yccl_handle``: a communication
+    library object that owns all those buffers and performs the exchanges (see
+    ``YaFSDPBufferContext.lazy_init``).  Ends with ``lazy_init`` of each group."""
     device = torch.device(device)
     if not param_groups:
         return
@@ -824,7 +870,8 @@ def init_shared_state(
         for ctx, gs in zip(ctxs, users):
             sizes = [size_of(g) for g in gs]  # bytes per all-gather dtype class
             dtypes = {dtype for per_dtype in sizes for dtype in per_dtype}
-            ctx.lazy_init({dtype: max(per_dtype.get(dtype, 0) for per_dtype in sizes) for dtype in dtypes}, device)
+            ctx.lazy_init({dtype: max(per_dtype.get(dtype, 0) for per_dtype in sizes) for dtype in dtypes}, device,
+                          yccl_handles=dict.fromkeys(dtypes, yccl_handle))
             for g in gs:
                 setattr(g, attr, ctx)
 

@@ -121,6 +121,10 @@ class YaFSDPState(_State):
         allow_no_grad_reduce: bool = False,
         param_group_to_data_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
         param_group_to_grad_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
+        yccl_handle: Any | None = None,
+        process_group_to_yccl_handle: "dict[Any, Any] | None" = None,
+        data_buffer_ctx_idx_to_yccl_handle: "dict[int, Any] | None" = None,
+        grad_buffer_ctx_idx_to_yccl_handle: "dict[int, Any] | None" = None,
     ) -> None:
         """ya_fsdp/_state.py:127-175.  ``allow_no_grad_reduce`` gives every group
         its own gradient buffer, which gradient accumulation without
@@ -128,7 +132,13 @@ class YaFSDPState(_State):
         The two maps replace the round-robin buffer assignment: group -> index
         (in module order) of the group whose buffer context it uses; as in the
         reference (:645-660) a map is only accepted where the default would give
-        every group its own buffer."""
+        every group its own buffer.  The handle arguments name the communication
+        library object (duck-typed: ``add_all_gather_input_buffer``,
+        ``add_all_gather_output_buffer``, ``add_reduce_scatter_buffer``,
+        ``all_gather``, ``reduce_scatter``, ``process_profiling_events``) that owns
+        the buffers of a buffer context and performs its exchanges: one for all
+        contexts, one per shard process group (here: per logical mesh), or one
+        per buffer-context index (:663-677)."""
         if self._is_root is not None:
             return
         self._is_root = True
@@ -151,7 +161,8 @@ class YaFSDPState(_State):
             visited_states.add(state)
         self._init_fqns()
         self._init_shared_state(allow_no_grad_reduce, param_group_to_data_buffer_ctx_idx,
-                                param_group_to_grad_buffer_ctx_idx)
+                                param_group_to_grad_buffer_ctx_idx, yccl_handle, process_group_to_yccl_handle,
+                                data_buffer_ctx_idx_to_yccl_handle, grad_buffer_ctx_idx_to_yccl_handle)
         self.validate_shared_state()
         for state in self._state_ctx.all_states:
             if state._fsdp_param_group:
@@ -162,6 +173,10 @@ class YaFSDPState(_State):
         allow_no_grad_reduce: bool = False,
         param_group_to_data_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
         param_group_to_grad_buffer_ctx_idx: "dict[YaFSDPParamGroup, int] | None" = None,
+        yccl_handle: Any | None = None,
+        process_group_to_yccl_handle: "dict[Any, Any] | None" = None,
+        data_buffer_ctx_idx_to_yccl_handle: "dict[int, Any] | None" = None,
+        grad_buffer_ctx_idx_to_yccl_handle: "dict[int, Any] | None" = None,
     ) -> None:
         """ya_fsdp/_state.py:177-288 and :617-678: one communication context;
         two data buffers handed out round-robin in module order and one gradient
@@ -178,35 +193,44 @@ class YaFSDPState(_State):
             return
         no_reshard_after_forward = all(not g.reshard_after_forward for g in param_groups)
 
-        def assign(groups, attr, count, size_of, ctx_idx=None):
+        def assign(groups, attr, count, size_of, ctx_idx=None, idx_to_handle=None):
             if not groups:
                 return []
             if ctx_idx is not None:
                 assert count is None  # ya_fsdp/_state.py:659-660
-                ctxs, users = [], []
+                ctxs, users, idxs = [], [], []
                 for g in groups:  # buffer contexts in order of first use (:661-669)
                     ctx = getattr(groups[ctx_idx[g]], attr)
                     if not any(ctx is c for c in ctxs):
                         ctxs.append(ctx)
                         users.append([])
+                        idxs.append(ctx_idx[g])
                     users[next(i for i, c in enumerate(ctxs) if c is ctx)].append(g)
             else:
                 n = len(groups) if count is None else min(count, len(groups))
                 ctxs = [getattr(groups[i], attr) for i in range(n)]
                 users = [[] for _ in range(n)]
+                idxs = list(range(n))
                 for i, g in enumerate(groups):
                     users[i % n].append(g)
-            for ctx, gs in zip(ctxs, users):
+            for ctx, gs, idx in zip(ctxs, users, idxs):
                 sizes = [size_of(g) for g in gs]  # bytes per all-gather dtype class (:234-251, :265-284)
                 dtypes = {dtype for per_dtype in sizes for dtype in per_dtype}
+                if idx_to_handle is not None:  # :668-677, in the reference's order of precedence
+                    handle = idx_to_handle[idx]
+                elif process_group_to_yccl_handle is not None:
+                    handle = process_group_to_yccl_handle[gs[-1].mesh_info.shard_process_group]
+                else:
+                    handle = yccl_handle
                 ctx.lazy_init({dtype: max(per_dtype.get(dtype, 0) for per_dtype in sizes) for dtype in dtypes},
-                              self._device)
+                              self._device, yccl_handles=dict.fromkeys(dtypes, handle))
                 for g in gs:
                     setattr(g, attr, ctx)
             return users
 
         data_users = assign(param_groups, "data_buffer_ctx", None if no_reshard_after_forward else 2,
-                            lambda g: g.data_buffer_bytes_by_dtype(), param_group_to_data_buffer_ctx_idx)
+                            lambda g: g.data_buffer_bytes_by_dtype(), param_group_to_data_buffer_ctx_idx,
+                            data_buffer_ctx_idx_to_yccl_handle)
         for state_groups in data_users:
             last = state_groups[-1]
             owner_state = next(s for s in self._state_ctx.all_states if s._fsdp_param_group is last)
@@ -214,7 +238,7 @@ class YaFSDPState(_State):
                 last.reshard_after_forward = False  # ya_fsdp/_state.py:256-260
         assign([g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx",
                None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes_by_dtype(),
-               param_group_to_grad_buffer_ctx_idx)
+               param_group_to_grad_buffer_ctx_idx, grad_buffer_ctx_idx_to_yccl_handle)
 
     def validate_shared_state(self) -> None:
         """ya_fsdp/_state.py:290-414: enough buffers for overlap; at most one
@@ -358,6 +382,12 @@ class YaFSDPState(_State):
                     group._training_state = TrainingState.IDLE
                 if self._state_ctx.is_last_backward:
                     state._finalize_backward()
+                if group is not None:  # :517-529
+                    ctxs = [group.data_buffer_ctx] + ([group.grad_buffer_ctx] if group.grad_buffer_ctx else [])
+                    for ctx in ctxs:
+                        for handle in ctx.yccl_handles.values():
+                            if handle is not None:
+                                handle.process_profiling_events()
             if self._state_ctx.is_last_backward:
                 self._comm_ctx.post_forward_order.clear()
             self._state_ctx.post_backward_final_callback_queued = False
