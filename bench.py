@@ -1715,6 +1715,12 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             ("all_gather_size1_copy", lambda: _native.flat_copy(d_gathered_b, d_gathered), 2 * t_pad * 2),
             ("divide_in_place", lambda: _native.flat_div(d_rs_b, 2.0), 2 * t_pad * rsz),
         ]
+        # a 1-byte all-gather dtype class of the same layer (tensor-subclass parameters with an int8 / fp8 all-gather,
+        # ya_fsdp/_param.py:281-291, ya_fsdp/_collectives.py:56-58): T_pad bytes copied between odd byte addresses
+        d_bytes_src = d_gathered.view(torch.uint8)[1 : 1 + t_pad]
+        d_bytes_dst = d_gathered_b.view(torch.uint8)[3 : 3 + t_pad]
+        variant_ops.append(("all_gather_1byte_dtype_odd_addresses", lambda: _native.flat_copy(d_bytes_dst, d_bytes_src),
+                            2 * t_pad))
         evict = [f for _, f, _ in ops]
         own_evict = {}
         if has_copy_in and not fused:

@@ -262,6 +262,20 @@ int main(void) {
   HIP(hipMemcpy(h_o16, d_o16, (size_t)s * 2, hipMemcpyDeviceToHost));
   if (!same("adamw bf16 copy-in", h_o16, h_o16_want, (size_t)s * 2)) return 1;
 
+  /* opaque bytes at odd addresses on both sides (1-byte all-gather dtypes): d_p's bytes, shifted by 3, into
+   * d_m's, shifted by 5; the bytes around the destination range stay as they are */
+  {
+    const size_t n_bytes = (size_t)s * 4 - 64 - 7;
+    unsigned char* h_dst = malloc((size_t)s * 4);
+    HIP(hipMemcpy(h_dst, d_m, (size_t)s * 4, hipMemcpyDeviceToHost));
+    memcpy(h_dst + 5, (const unsigned char*)h_p + 3, n_bytes);
+    YA(yafsdp_flat_copy_bytes((char*)d_m + 5, (const char*)d_p + 3, (int64_t)n_bytes, stream));
+    HIP(hipStreamSynchronize(stream));
+    HIP(hipMemcpy(h_tmp, d_m, (size_t)s * 4, hipMemcpyDeviceToHost));
+    if (!same("byte copy at odd addresses", h_tmp, h_dst, (size_t)s * 4)) return 1;
+    free(h_dst);
+  }
+
   YA(yafsdp_binding_destroy(binding));
   YA(yafsdp_table_destroy(table));
   printf("PASS\n");

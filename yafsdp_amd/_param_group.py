@@ -537,8 +537,8 @@ class YaFSDPParamGroup:
             if default_prefetch:
                 self._backward_prefetch()
 
-    def post_backward(self) -> None:
-        """ya_fsdp/_param_group.py:655-771."""
+    def post_backward(self, *unused: Any) -> None:
+        """ya_fsdp/_param_group.py:655-771.  Safe to call when the group took no part in the backward."""
         self._training_state = TrainingState.POST_BACKWARD
         current_stream = torch.cuda.current_stream(self.device)
         if (grad_buffer_ctx := self.grad_buffer_ctx) is not None:
