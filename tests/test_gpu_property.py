@@ -370,3 +370,87 @@ def test_param_group_any_layout(shapes, w, r_frac, align, policy, iterations, se
             if owns[i]:
                 assert_bits_equal(got[pos : pos + n], want[pos : pos + n], f"gradient fragment {i}, iteration {it}")
             pos += n
+
+
+@settings(max_examples=30 * SCALE, **COMMON)
+@given(spec=st.lists(st.tuples(shape_st, st.booleans()), min_size=1, max_size=7), w=st.integers(1, 5),
+       r_frac=st.floats(0, 0.999), align=st.sampled_from([1, 2, 8, 16]), iterations=st.integers(1, 3),
+       seed=st.integers(0, 2**20))
+def test_param_group_with_all_gather_dtype_classes(spec, w, r_frac, align, iterations, seed):
+    """A group whose parameters are split at random between the default class and a tensor-subclass class with an
+    int8 all-gather (ya_fsdp/_param_group.py:194-227): per class the all-gather input, this rank's slot of the
+    gathered buffer and the gradient shard over a few iterations with missing gradients, against the reference's op
+    sequence on CPU tensors."""
+    import torch.nn as nn
+    from ext_subclasses import Int8Master, quantize
+    from test_gpu_param_group import BF16_MP, CpuGroup
+
+    from yafsdp_amd import FSDPMeshInfo, MixedPrecisionPolicy
+    from yafsdp_amd._param_group import YaFSDPParamGroup, init_shared_state
+
+    r = int(r_frac * w)
+    print("classes", spec, w, r, align, iterations, seed, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    values = [torch.randn(s, generator=g) * 0.08 for s, _ in spec]
+    dev_params = [nn.Parameter(Int8Master(v.to(DEV))) if ext else v.to(DEV).requires_grad_(True)
+                  for v, (_, ext) in zip(values, spec)]
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, all_gather_dtype_to_param_cls={torch.int8: Int8Master})
+    group = YaFSDPParamGroup(dev_params, FSDPMeshInfo(w, r), DEV, mp, align)
+    init_shared_state([group], DEV)
+    keys = {None: [i for i, (_, e) in enumerate(spec) if not e], torch.int8: [i for i, (_, e) in enumerate(spec) if e]}
+    keys = {k: idx for k, idx in keys.items() if idx}
+    assert list(group._all_gather_dtype_to_fsdp_params) == list(keys)
+    refs = {k: CpuGroup([values[i] for i in idx], w, r, align, BF16_MP) for k, idx in keys.items()}
+    post = float(w) if w > 1 else None
+    rng = np.random.default_rng(seed)
+    owns = [False] * len(spec)
+    for it in range(iterations):
+        group.pre_forward(); group.post_forward(); group.pre_backward()
+        torch.cuda.synchronize()
+        for k, ref in refs.items():
+            n_local = ref.lay.sharded_numels(r)
+            if k is None:
+                torch_ops.copy_in(ref.ag_in, ref.shard)
+                want_in = ref.ag_in
+            else:
+                want_in = torch.zeros(ref.lay.padded_sharded_numel, dtype=torch.int8)
+                for dst, frag in zip(want_in[: sum(n_local)].split(n_local), ref.shard[: sum(n_local)].split(n_local)):
+                    torch_ops.extension_copy_in(dst, quantize(frag))
+            got_in, got_out = group._all_gather_input[k].cpu(), group._all_gather_output[k].cpu()
+            s_ = ref.lay.padded_sharded_numel
+            assert torch.equal(got_in.view(torch.uint8), want_in.view(torch.uint8)), (k, "all-gather input")
+            assert torch.equal(got_out[r * s_ : (r + 1) * s_].view(torch.uint8), got_in.view(torch.uint8)), (k, "slot")
+        gg = torch.Generator().manual_seed(seed + 1 + it)
+        grads = [(torch.randn(s, generator=gg) * 1e-3).bfloat16() for s, _ in spec]
+        present = rng.random(len(spec)) < 0.8
+        if not present.any():
+            present[int(rng.integers(0, len(spec)))] = True
+        grads = [x if p else None for x, p in zip(grads, present)]
+        for fp, x in zip(group.fsdp_params, grads):
+            fp.unsharded_param.grad = None if x is None else x.to(DEV)
+        group.post_backward()
+        group.finalize_backward()
+        torch.cuda.synchronize()
+        for k, ref in refs.items():
+            mine = [grads[i] for i in keys[k]]
+            mine_owns = [owns[i] for i in keys[k]]
+            if all(x is None for x in mine):
+                continue  # the class took no part in this pass: its gradient shard is untouched
+            ref.accumulate(mine, [False] * len(mine))
+            with_grad = [j for j, x in enumerate(mine) if x is not None]
+            if all(not mine_owns[j] for j in with_grad) and len(with_grad) == len(mine):
+                ref.reduce(None, post, "copy")
+            elif all(mine_owns[j] for j in with_grad) and len(with_grad) == len(mine):
+                ref.reduce(None, post, "add")
+            else:
+                ref.reduce(None, post, "mixed", [None if x is None else mine_owns[j] for j, x in enumerate(mine)])
+        for i, x in enumerate(grads):
+            if x is not None:
+                owns[i] = True
+        for k, ref in refs.items():
+            got, want = group._padded_sharded_param_grad[k], ref.grad_shard
+            pos = 0
+            for j, n in enumerate(ref.lay.sharded_numels(r)):
+                if owns[keys[k][j]]:
+                    assert_bits_equal(got[pos : pos + n], want[pos : pos + n], f"class {k} fragment {j}, iteration {it}")
+                pos += n
