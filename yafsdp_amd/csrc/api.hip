@@ -336,7 +336,7 @@ int yafsdp_binding_create(yafsdp_table* table, const void* const* tensor_ptrs, c
   b->table = table;
   b->tensor_dtype = tensor_dtype;
   const int n = table->n_tensors;
-  if (n <= kSmallMax) {
+  if (n <= kSmallRoute) {
     fill_small(table, tensor_ptrs, mode, &b->small);
   } else {
     const size_t bytes = size_t(n) * (sizeof(void*) + sizeof(uint32_t));
@@ -391,7 +391,7 @@ int yafsdp_gather_in_bound(yafsdp_binding* binding, void* flat, int flat_dtype, 
   scale_plan(pre_factor, &scale, &k);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int grid = grid_for(table_blocks(table->n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  if (table->n_tensors <= kSmallMax)
+  if (table->n_tensors <= kSmallRoute)
     return int(launch_gather<SmallMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->small, flat,
                                         table->padded, table->n_tiles, k, zero_pad ? 1 : 0, grid, s));
   return int(launch_gather<LargeMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->large, flat,
@@ -411,7 +411,7 @@ int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat
   if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int grid = grid_for(table_blocks(table->n_slots), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  if (table->n_tensors <= kSmallMax)
+  if (table->n_tensors <= kSmallRoute)
     return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->small, flat,
                                          table->total, table->n_slots, grid, s));
   return int(launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->large, flat,
@@ -868,7 +868,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     if ((e = hipGetDevice(&t->device)) != hipSuccess) break;
     if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_offsets), t->offsets.size() * sizeof(int64_t))) != hipSuccess) break;
     if ((e = hipMemcpy(t->d_offsets, t->offsets.data(), t->offsets.size() * sizeof(int64_t), hipMemcpyHostToDevice)) != hipSuccess) break;
-    if (n_tensors > kSmallMax && n_tiles > 0) {
+    if (n_tensors > kSmallRoute && n_tiles > 0) {
       // per tile: first tensor whose end lies beyond the tile's first element
       tiles.resize(size_t(n_tiles));
       int p = 0;
@@ -891,7 +891,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
     }
     if (t->slot_start[n_tensors] > int64_t(INT32_MAX) - 4096) { rc = YAFSDP_ERR_INVALID_ARGUMENT; break; }
     t->n_slots = int32_t(t->slot_start[n_tensors]);
-    if (n_tensors > kSmallMax && t->n_slots > 0) {
+    if (n_tensors > kSmallRoute && t->n_slots > 0) {
       tiles.resize(size_t(t->n_slots));
       for (int p = 0; p < n_tensors; p++) {
         for (int64_t k = t->slot_start[p]; k < t->slot_start[p + 1]; k++) {
@@ -904,7 +904,7 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
       if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_slots), tiles.size() * sizeof(TileRec))) != hipSuccess) break;
       if ((e = hipMemcpy(t->d_slots, tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
     }
-    if (n_tensors > kSmallMax) {
+    if (n_tensors > kSmallRoute) {
       t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
       t->scratch.assign(t->stage_bytes, 0);
       for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
@@ -966,7 +966,7 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   if (rc != YAFSDP_OK) return rc;
   const int n_tiles = table->n_tiles;
   const int grid = grid_for(table_blocks(n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  if (table->n_tensors <= kSmallMax) {
+  if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     fill_small(table, tensor_ptrs, mode, &meta);
     return int(launch_gather<SmallMeta>(table->block, tensor_dtype, flat_dtype, scale, meta, flat, table->padded,
@@ -1018,7 +1018,7 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   if (grid == 0) return YAFSDP_OK;
   if (grid > int64_t(INT32_MAX) - 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (table->n_tensors <= kSmallMax) {
+  if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     static const void* const kNoPtrs[kSmallMax] = {};
     fill_small(table, table->total > 0 ? ptrs : kNoPtrs, mode, &meta);
@@ -1073,7 +1073,7 @@ int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_
   if (rc != YAFSDP_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  if (table->n_tensors <= kSmallMax) {
+  if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     fill_small(table, tensor_ptrs, mode, &meta);
     return int(launch_gather_post<SmallMeta>(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard,
@@ -1108,7 +1108,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   if (rc != YAFSDP_OK) return rc;
   const int n_tiles = table->n_slots;
   const int grid = grid_for(table_blocks(n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
-  if (table->n_tensors <= kSmallMax) {
+  if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     fill_small(table, ptrs, mode, &meta);
     return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,

@@ -339,7 +339,10 @@ __device__ __forceinline__ float gather_elem(float s, float d_old, float k) {
   else if constexpr (MODE == MODE_ADD) y = __fadd_rn(d_old, s);
   else y = d_old;
   if constexpr (SCALE != SCALE_NONE) {
-    if constexpr (MODE != MODE_SKIP) y = round_to<D>(y);
+    // the copy / add materialises in D before the divide reads it.  A copied value that D represents exactly
+    // (same dtype, or binary32 as the destination) needs no rounding instruction.
+    constexpr bool kExactCopy = MODE == MODE_COPY && (same_t<S, D>::value || same_t<D, F32>::value);
+    if constexpr (MODE != MODE_SKIP && !kExactCopy) y = round_to<D>(y);
     y = apply_scale<SCALE>(y, k);
   }
   return y;  // caller rounds to D on store

@@ -44,6 +44,14 @@
 namespace yafsdp {
 
 constexpr int kSmallMax = 16;
+// tables with at most this many tensors take the SmallMeta route (at most kSmallMax: the arrays' size).  Sending
+// a 9-tensor layer through per-tile records instead (-DYAFSDP_SMALL_ROUTE=8) measured 1 us slower per table kernel
+// and 13 us slower per step (the staging of pointers).
+#ifndef YAFSDP_SMALL_ROUTE
+#define YAFSDP_SMALL_ROUTE 16
+#endif
+constexpr int kSmallRoute = YAFSDP_SMALL_ROUTE;
+static_assert(kSmallRoute >= 0 && kSmallRoute <= kSmallMax, "SmallMeta holds at most kSmallMax tensors");
 enum : int { MODE_ZERO = 3 };  // internal: fill with zeros (pad lanes)
 
 struct TileRec {
@@ -56,6 +64,8 @@ struct TileLookup {
   int first;
   bool full;
   int64_t delta;
+  const void* base;  // tensor `first` (unspecified for a tile that starts in the pad)
+  int mode;          // its mode
 };
 
 struct ScatterLookup {
@@ -84,13 +94,22 @@ struct SmallMeta {
   }
 
   __device__ __forceinline__ TileLookup lookup(int tile, int64_t t0, int64_t tile_elems) const {
+    // tile_start is ascending: the last i with tile_start[i] <= tile is the tensor (a chain of scalar selects)
     int p = 0;
 #pragma unroll
-    for (int i = 1; i <= kSmallMax; i++) p += (tile_start[i] <= tile) ? 1 : 0;
+    for (int i = 1; i <= kSmallMax; i++) p = (tile_start[i] <= tile) ? i : p;
     TileLookup r;
     r.first = p;
+    // the three loads that depend on p leave together, before anything branches on their results
+    const int pc = p < kSmallMax ? p : kSmallMax - 1;
     const int64_t o0 = off[p];
-    const int64_t o1 = off[p < kSmallMax ? p + 1 : kSmallMax];
+    const int64_t o1 = off[pc + 1];
+    r.base = ptr[pc];
+    // (the empty statement reads the three values here, so that the compiler cannot sink each load to the branch
+    // that first uses it, where it would wait for them one after the other; they are inputs only, which keeps
+    // the pointer's address space known: global loads, not flat ones)
+    asm volatile("" ::"s"(o0), "s"(o1), "s"(r.base));
+    r.mode = int((modes >> (2 * pc)) & 3u);
     r.full = p < n_tensors && (o1 - t0 >= tile_elems);
     r.delta = t0 - o0;
     return r;
@@ -115,6 +134,9 @@ struct LargeMeta {
     r.first = t[tile].first;
     r.full = t[tile].full != 0;
     r.delta = t[tile].delta;
+    const int pc = r.first < n_tensors ? r.first : (n_tensors > 0 ? n_tensors - 1 : 0);
+    r.base = n_tensors > 0 ? tensor(pc) : nullptr;
+    r.mode = n_tensors > 0 ? mode(pc) : 0;
     return r;
   }
   __device__ __forceinline__ ScatterLookup lookup_scatter(int tile) const {
@@ -276,16 +298,19 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
   constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
   constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
   const int n_blocks = (n_tiles + kWin - 1) / kWin * kWin;
-  for (int b = blockIdx.x; b < n_blocks; b += gridDim.x) {
+  // (a loop that tests at its end: the first tile's lookup then does not wait for n_tiles to arrive before its
+  // own loads leave; a workgroup beyond the last tile finds tile >= n_tiles below)
+  int b = blockIdx.x;
+  do {
     const int tile = tile_of_block<kX, kWin>(b);
-    if (tile >= n_tiles) continue;
     const int64_t t0 = int64_t(tile) * kTile;
     const int64_t t1 = (t0 + kTile < padded) ? t0 + kTile : padded;
     const TileLookup rec = meta.lookup(tile, t0, kTile);
+    if (tile >= n_tiles) continue;
     int p = rec.first;
     if (rec.full) {  // the whole tile lies inside tensor p
-      const int mode = meta.mode(p);
-      const char* src = reinterpret_cast<const char*>(meta.tensor(p)) + rec.delta * S::kSize;
+      const int mode = rec.mode;
+      const char* src = reinterpret_cast<const char*>(rec.base) + rec.delta * S::kSize;
       char* dst = fbase + t0 * D::kSize;
       if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, STP>(dst, src, k);
       else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, STP>(dst, src, k);
@@ -313,7 +338,7 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
       pos = e;
       if (e == o1) ++p;
     }
-  }
+  } while ((b += gridDim.x) < n_blocks);
 }
 
 // ---------------------------------------------------------------- scatter-out --
