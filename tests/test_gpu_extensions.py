@@ -244,3 +244,35 @@ def test_training_with_int8_all_gather_matches_a_hand_written_loop():
         assert isinstance(wp._local_tensor, Int8Master)
         assert_bits_equal(wp._local_tensor._data.view(w.shape), w.cpu(), "weight master")
         assert_bits_equal(l.bias._local_tensor.view(b.shape), b.cpu(), "bias master")
+
+
+def test_checkpoint_and_full_tensor_of_extension_parameters(tmp_path):
+    """The sharded parameter of a tensor-subclass class wraps an ``Int8Master`` around its fragment of the flat master
+    shard; ``full_tensor()`` and the ``torch.distributed.checkpoint`` hooks deal in the plain master values."""
+    import torch.distributed.checkpoint as dcp
+
+    from yafsdp_amd import RaggedShardDTensor, fully_shard
+    from yafsdp_amd.checkpoint import RaggedShardLoadPlanner
+
+    def build(seed):
+        gen = torch.Generator().manual_seed(seed)
+        layer = QLinear(24, 40, gen)
+        values = (layer.weight.detach()._data.clone(), layer.bias.detach().clone())
+        return fully_shard(layer, mesh=(1, 0), mp_policy=INT8_MP), values
+
+    model, (w, b) = build(21)
+    assert isinstance(model.weight, RaggedShardDTensor) and isinstance(model.weight._local_tensor, Int8Master)
+    full = model.weight.full_tensor()
+    assert type(full) is torch.Tensor and full.shape == w.shape
+    assert_bits_equal(full, w.cpu(), "full_tensor of the extension parameter")
+    dcp.save(model.state_dict(), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True)
+    other, (w2, _) = build(22)
+    assert not torch.equal(w2, w)
+    dcp.load(other.state_dict(), checkpoint_id=str(tmp_path / "ckpt"), no_dist=True, planner=RaggedShardLoadPlanner())
+    torch.cuda.synchronize()
+    assert_bits_equal(other.weight._local_tensor._data.view(w.shape), w.cpu(), "loaded weight master")
+    assert_bits_equal(other.bias._local_tensor.view(b.shape), b.cpu(), "loaded bias master")
+    # and the loaded masters are what the next all-gather quantises
+    x = torch.randn(4, 24, generator=torch.Generator().manual_seed(1)).to(DEV).bfloat16()
+    want = F.linear(x, dequantize(quantize(w), STEP, torch.bfloat16), b.bfloat16())
+    assert_bits_equal(other(x), want.cpu(), "forward after loading")

@@ -391,6 +391,11 @@ class YaFSDPParamGroup:
             if yccl_handle is not None:
                 # the communication library owns the buffer it gathers from (:510-519)
                 ag_dtype = self._ag_dtype(all_gather_dtype)
+                if shard.numel() * ag_dtype.itemsize % torch.bfloat16.itemsize:
+                    raise ValueError(
+                        f"a communication handle exchanges bfloat16 elements, but the {ag_dtype} shard of {self} has "
+                        f"{shard.numel()} elements: use an even shard_alignment"
+                    )
                 numel = shard.numel() * ag_dtype.itemsize // torch.bfloat16.itemsize
                 buffer = yccl_handle.add_all_gather_input_buffer(numel)
                 _check_handle_buffer(buffer, numel, self.device, "add_all_gather_input_buffer")

@@ -307,7 +307,7 @@ class RaggedShardDTensor(torch.Tensor):
                 type=WriteItemType.SHARD,
                 tensor_data=TensorWriteData(
                     chunk=ChunkStorageMetadata(offsets=offsets, sizes=sizes),
-                    properties=TensorProperties.create_from_tensor(self._local_tensor),
+                    properties=TensorProperties.create_from_tensor(plain_tensor(self._local_tensor)),
                     size=torch.Size((reduce(operator.mul, self.size(), 1),)),
                 ),
             )
@@ -320,7 +320,8 @@ class RaggedShardDTensor(torch.Tensor):
         return [ChunkStorageMetadata(offsets=offsets, sizes=sizes)]
 
     def __get_tensor_shard__(self, index: int) -> torch.Tensor:
-        return self._local_tensor
+        # the plain fragment of the flat shard: what a tensor-subclass parameter wraps is written as its values
+        return plain_tensor(self._local_tensor)
 
 
 def _locals_any(args: Sequence[Any]) -> list[Any]:
