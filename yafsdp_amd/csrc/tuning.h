@@ -43,7 +43,10 @@ constexpr int kFlatStorePolicy = YAFSDP_FLAT_STP;
 // (All-zero buffers run up to 10 % faster than any other content on this memory
 // system and must not be used for tuning.)
 constexpr int kTableBlockSmall = 64;
-constexpr int kTableBlockLarge = 128;
+#ifndef YAFSDP_TABLE_BLOCK_LARGE
+#define YAFSDP_TABLE_BLOCK_LARGE 128
+#endif
+constexpr int kTableBlockLarge = YAFSDP_TABLE_BLOCK_LARGE;
 constexpr int kTableLargeThresholdLog2 = 28;  // padded size above 2^28 elements: the larger workgroup
 #ifndef YAFSDP_TABLE_U
 #define YAFSDP_TABLE_U 2
