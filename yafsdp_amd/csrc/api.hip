@@ -126,7 +126,10 @@ int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const vo
     const bool in_place = d0 == s0 && item_size(dst_dt) == item_size(src_dt);
     if (!in_place && d0 < s1 && s0 < d1) return YAFSDP_ERR_INVALID_ARGUMENT;
   }
-  int64_t head = ((16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15) / item_size(dst_dt);
+  // leading elements up to the destination's next 128-byte line (at most 63, fewer than a workgroup has lanes):
+  // tiles are whole lines from there on, so no two workgroups write into one cache line
+  static_assert(kFlatBlock >= 64, "workgroup 0 peels up to 63 leading elements, one per lane");
+  int64_t head = ((128 - (reinterpret_cast<uintptr_t>(dst) & 127)) & 127) / item_size(dst_dt);
   if (head > n) head = n;
   const int64_t units = (n - head) >> 3;
   const int64_t tile = int64_t(kFlatBlock) * kFlatUnroll;
@@ -708,7 +711,10 @@ int yafsdp_flat_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* st
     return flat_launch(DT_BF16, DT_BF16, SCALE_NONE, false, dst, src, n_bytes >> 1, 1.0f,
                        static_cast<hipStream_t>(stream));
   if (d0 < s0 + uintptr_t(n_bytes) && s0 < d0 + uintptr_t(n_bytes)) return YAFSDP_ERR_INVALID_ARGUMENT;  // overlap
-  int64_t head = int64_t((16 - (d0 & 15)) & 15);
+  // up to the destination's next 128-byte line, so that no two workgroups write into one cache line (tiles are a
+  // whole number of lines from there on): with 16-byte alignment only, every tile boundary split a line, and the
+  // counters showed 3 % more bytes written than the copy holds
+  int64_t head = int64_t((128 - (d0 & 127)) & 127);
   if (head > n_bytes) head = n_bytes;
   const int64_t n_tiles = (((n_bytes - head) >> 4) + kFlatBlock - 1) / kFlatBlock;
   int device = 0;

@@ -10,9 +10,11 @@
 //  * pairs with an fp32 side: quad arrangement (see elem.hip.h): every wave64
 //    access is a contiguous 1 KiB (fp32) or 512 B (2-byte) span.
 // All loads of a lane are issued before its first store.  The destination is
-// 16-byte aligned for the tile loop (the host peels up to 7 leading elements,
-// handled by workgroup 0 together with the tail); the source may sit at any
-// element-aligned address.
+// aligned for the tile loop: the host peels the leading elements up to its next
+// 128-byte line (fewer than 64; 16-byte alignment is what the kernel needs, the
+// line keeps two workgroups from writing into one cache line), handled by
+// workgroup 0 together with the tail; the source may sit at any element-aligned
+// address.
 #pragma once
 #include "elem.hip.h"
 #include "tuning.h"
@@ -149,8 +151,8 @@ flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned l
 // ---- opaque bytes ------------------------------------------------------------
 // dst[0:n] = src[0:n] for byte ranges at ANY byte address: the same-dtype copy of
 // 1-byte element types (fp8, int8, uint8), whose ragged per-parameter fragments
-// start and end at odd addresses.  `head` (0..15) leading bytes bring dst to a
-// 16-byte boundary; the body is 16-byte vectors, one per lane and tile (aligned
+// start and end at odd addresses.  `head` (0..127, at most BLOCK) leading bytes bring dst
+// to a 128-byte line; the body is 16-byte vectors, one per lane and tile (aligned
 // stores; the loads sit at whatever byte alignment the two addresses leave, which
 // the hardware serves natively like the element-aligned loads of the other
 // kernels); workgroup 0 also copies the head and the up to 15 trailing bytes.
@@ -159,6 +161,7 @@ typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
 template <int BLOCK, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 bytes_kernel(void* dst, const void* src, int64_t n, int head) {
+  static_assert(BLOCK >= 128, "workgroup 0 copies up to 127 leading bytes, one per lane");
   const int tid = threadIdx.x;
   const int64_t n_vecs = (n - head) >> 4;
   const int64_t body_end = head + (n_vecs << 4);

@@ -39,7 +39,7 @@ inline hipError_t launch_kernel(void (*kernel)(Params...), int grid, int block, 
 // dst[i] = post_elem(src[i], dst[i]); scale is SCALE_NONE / SCALE_MUL / SCALE_DIV
 hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,
                        float k, int grid, hipStream_t stream);
-// dst[0:n] = src[0:n], opaque bytes at any byte address; head: bytes up to dst's first 16-byte boundary
+// dst[0:n] = src[0:n], opaque bytes at any byte address; head: bytes up to dst's first 128-byte line (< workgroup size)
 hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int grid, hipStream_t stream);
 // the same pass, also writing partials[0:grid] = per-workgroup sums of squares of the stored values (postsumsq.hip);
 // grid must equal the number of tiles
