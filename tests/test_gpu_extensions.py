@@ -276,3 +276,56 @@ def test_checkpoint_and_full_tensor_of_extension_parameters(tmp_path):
     x = torch.randn(4, 24, generator=torch.Generator().manual_seed(1)).to(DEV).bfloat16()
     want = F.linear(x, dequantize(quantize(w), STEP, torch.bfloat16), b.bfloat16())
     assert_bits_equal(other(x), want.cpu(), "forward after loading")
+
+
+def test_flat_optimizer_passes_cover_every_all_gather_dtype_class():
+    """``grad_clip_coef`` / ``clip_grad_norm_`` / ``zero_grad`` / ``FlatAdamW`` run over the flat shards of both
+    classes of a group (ordinary parameters and the int8 all-gather class); the fused copy-in serves the default
+    class only, the subclass quantises its own masters in the next forward.  Against the C oracle per flat shard."""
+    from oracle import cref
+    from yafsdp_amd import fully_shard
+    from yafsdp_amd.optim import FlatAdamW, clip_grad_norm_, enable_fused_grad_norm, fsdp_param_groups, zero_grad
+
+    gen = torch.Generator().manual_seed(31)
+    layer = fully_shard(QLinear(24, 40, gen), mesh=(1, 0), mp_policy=INT8_MP)
+    (group,) = fsdp_param_groups(layer)
+    assert list(group._padded_sharded_param_grad) == [None, torch.int8]
+    with pytest.raises(NotImplementedError, match="default class only"):
+        enable_fused_grad_norm(layer)
+    opt = FlatAdamW(layer.parameters(), lr=1e-2, betas=(0.9, 0.95), weight_decay=0.1)
+    x = torch.randn(16, 24, generator=gen).to(DEV).bfloat16()
+    (layer(x).float().pow(2).mean() * 30.0).backward()
+    keys = [None, torch.int8]
+    masters = {k: group._padded_sharded_param_data[k].detach().cpu().clone() for k in keys}
+    grads = {k: group._padded_sharded_param_grad[k].detach().cpu().clone() for k in keys}
+    assert all(float(grads[k].abs().max()) > 0 for k in keys)
+    # clipping over both shards
+    max_norm = 1e-2
+    norm, coef = cref.clip_coef(sum(cref.sumsq(grads[k]) for k in keys), max_norm)
+    got = clip_grad_norm_(layer, max_norm)
+    assert abs(got.item() - norm) <= 6e-8 * norm and coef < 1.0
+    for k in keys:
+        cref.flat_scale(grads[k], coef)
+        assert_bits_equal(group._padded_sharded_param_grad[k], grads[k], f"clipped gradient shard {k}")
+    # one AdamW step per flat shard; only the default class gets its 16-bit all-gather input written
+    opt.step()
+    torch.cuda.synchronize()
+    for k in keys:
+        n = masters[k].numel()
+        out16 = torch.zeros(n, dtype=torch.bfloat16) if k is None else None
+        cref.adamw_step(masters[k], grads[k], torch.zeros(n), torch.zeros(n), out16, lr=1e-2, beta1=0.9, beta2=0.95,
+                        eps=1e-8, weight_decay=0.1, step=1)
+        assert_bits_equal(group._padded_sharded_param_data[k], masters[k], f"master shard {k} after the step")
+        if k is None:
+            assert_bits_equal(group._all_gather_input[None], out16, "fused copy-in of the default class")
+    assert group._all_gather_input_set_dtypes == {None}
+    for p in layer.parameters():
+        st = opt.state[p]
+        assert st["exp_avg"].shape == p.shape and float(st["exp_avg"]._local_tensor.abs().max()) > 0
+    # the next forward quantises the updated masters itself
+    want = F.linear(x, dequantize(quantize(masters[torch.int8][: 40 * 24].view(40, 24)), STEP, torch.bfloat16).to(DEV),
+                    masters[None][:40].bfloat16().to(DEV)).cpu()
+    assert_bits_equal(layer(x), want, "forward after the step")
+    zero_grad(layer)
+    for k in keys:
+        assert float(group._padded_sharded_param_grad[k].abs().max()) == 0.0

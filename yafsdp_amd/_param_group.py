@@ -240,6 +240,10 @@ class YaFSDPParamGroup:
         for index, fsdp_param in enumerate(self.fsdp_params):
             fsdp_param._param_group_ref = weakref.ref(self)
             fsdp_param._index_in_group = index
+        for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
+            for index, fsdp_param in enumerate(fsdp_params):
+                fsdp_param._all_gather_class = all_gather_dtype
+                fsdp_param._index_in_class = index
         self._tables: dict[torch.dtype | None, _native.TensorTable] = {}
         # this rank's fragments of each class's gradient shard (built on first use, ya_fsdp/_collectives.py:191-214)
         self._fragment_tables: dict[torch.dtype | None, _native.TensorTable] = {}

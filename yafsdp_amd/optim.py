@@ -53,21 +53,20 @@ def fsdp_param_groups(modules: nn.Module | Iterable[nn.Module]) -> list[YaFSDPPa
     return groups
 
 
-def _flat_groups(modules: nn.Module | Iterable[nn.Module]) -> list[YaFSDPParamGroup]:
-    """``fsdp_param_groups`` for the passes of this module, which run over ONE flat shard per group: a group whose
-    policy gives tensor-subclass parameters an all-gather dtype class of their own has several."""
-    groups = fsdp_param_groups(modules)
-    for g in groups:
-        _require_one_class(g)
-    return groups
+def _grad_classes(modules: nn.Module | Iterable[nn.Module]) -> "list[tuple[YaFSDPParamGroup, Any]]":
+    """Every flat gradient shard under ``modules``: one per parameter group and all-gather dtype class of it (key
+    ``None``: the ordinary parameters; a dtype: the tensor-subclass parameters that are all-gathered in it,
+    ya_fsdp/_param_group.py:194-227), in module order."""
+    return [(g, key) for g in fsdp_param_groups(modules) for key, shard in g._padded_sharded_param_grad.items()
+            if shard is not None]
 
 
 def _require_one_class(group: YaFSDPParamGroup) -> None:
     if group.has_extension_classes:
         raise NotImplementedError(
-            f"{group} has tensor-subclass all-gather dtype classes (all_gather_dtype_to_param_cls): the flat "
-            "optimizer-side passes cover groups with the default class only; torch.optim and "
-            "torch.nn.utils.clip_grad_norm_ work on its sharded parameters"
+            f"{group} has tensor-subclass all-gather dtype classes (all_gather_dtype_to_param_cls): the gradient "
+            "norm fused into the post-reduce covers groups with the default class only; grad_clip_coef, "
+            "clip_grad_norm_, zero_grad and FlatAdamW work on every class"
         )
 
 
@@ -87,26 +86,27 @@ def _merge(ranges: list[tuple[int, int]]) -> list[tuple[int, int]]:
     return out
 
 
-def _fragment_offsets(group: YaFSDPParamGroup) -> list[int]:
+def _fragment_offsets(group: YaFSDPParamGroup, key: Any = None) -> list[int]:
     offsets = [0]
-    for n in group._sharded_param_numels[None]:
+    for n in group._sharded_param_numels[key]:
         offsets.append(offsets[-1] + n)
     return offsets
 
 
-def _grad_ranges(group: YaFSDPParamGroup, indices: Sequence[int] | None = None) -> list[tuple[int, int]]:
-    """Ranges of the group's flat gradient shard that hold a gradient: the
-    fragments of the parameters whose ``.grad`` is set.  A gradient tensor that
-    is not the group's own view (assigned by the user) is copied into it first.
+def _grad_ranges(group: YaFSDPParamGroup, indices: Sequence[int] | None = None, key: Any = None) -> list[tuple[int, int]]:
+    """Ranges of one flat gradient shard of the group (class ``key``) that hold a gradient: the
+    fragments of the parameters whose ``.grad`` is set (``indices``: positions in the class's parameter list).
+    A gradient tensor that is not the group's own view (assigned by the user) is copied into it first.
     When every fragment has one, the range extends over the pad lanes (zeros)."""
-    grad_shard = group._padded_sharded_param_grad[None]
+    grad_shard = group._padded_sharded_param_grad[key]
     if grad_shard is None:
         return []
-    offsets = _fragment_offsets(group)
+    fsdp_params = group._all_gather_dtype_to_fsdp_params[key]
+    offsets = _fragment_offsets(group, key)
     ranges = []
-    complete = indices is None or len(indices) == len(group.fsdp_params)
-    for i in range(len(group.fsdp_params)) if indices is None else indices:
-        fsdp_param = group.fsdp_params[i]
+    complete = indices is None or len(indices) == len(fsdp_params)
+    for i in range(len(fsdp_params)) if indices is None else indices:
+        fsdp_param = fsdp_params[i]
         grad = fsdp_param.sharded_param.grad if fsdp_param.requires_grad else None
         if grad is None:
             if offsets[i + 1] > offsets[i]:
@@ -159,7 +159,10 @@ def enable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
     the reduce (seen through the shard's version counter), or one of this
     module's own passes that rewrites gradients (scaling, zero-fill).  Kernels
     launched on the gradient shard through ``_native`` directly are not seen."""
-    groups = [g for g in _flat_groups(modules) if g._padded_sharded_param_grad[None] is not None]
+    groups = fsdp_param_groups(modules)
+    for g in groups:
+        _require_one_class(g)
+    groups = [g for g in groups if g._padded_sharded_param_grad[None] is not None]
     if not groups:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
     device = groups[0].device
@@ -209,12 +212,13 @@ def grad_clip_coef(
     buffer and must be ordered on one stream."""
     if norm_type not in (2, 2.0):
         raise NotImplementedError("only the 2-norm is implemented (ya_fsdp/ya_fsdp.py:544)")
-    groups = [g for g in _flat_groups(modules) if g._padded_sharded_param_grad[None] is not None]
-    if not groups:
+    classes = _grad_classes(modules)
+    if not classes:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
+    groups = [g for g, _ in classes]
     device = groups[0].device
     norm_and_coef = torch.empty(2, dtype=torch.float32, device=device)
-    fused = _fused_partials(groups)
+    fused = _fused_partials(groups) if all(key is None for _, key in classes) else None
     if fused is not None:
         # sums left by the post-reduce where they still describe the gradients; a read pass into the group's own
         # slot (zeroed first: it may write fewer sums than the slot holds) where they do not
@@ -237,7 +241,7 @@ def grad_clip_coef(
         else:
             _native.clip_coef_from_partials(fused, fused.numel(), max_norm, norm_and_coef)
         return norm_and_coef[0], norm_and_coef[1]
-    work = [(g._padded_sharded_param_grad[None], lo, hi) for g in groups for lo, hi in _grad_ranges(g)]
+    work = [(g._padded_sharded_param_grad[key], lo, hi) for g, key in classes for lo, hi in _grad_ranges(g, None, key)]
     partials = _ClipState.get(device).reserve(max(len(work), 1))
     count = 0
     for grad_shard, lo, hi in work:
@@ -255,36 +259,32 @@ def clip_grad_norm_(
     traffic when nothing is clipped (coefficient exactly 1)."""
     total_norm, coef = grad_clip_coef(modules, max_norm, norm_type)
     coef = coef.view(1)
-    for group in _flat_groups(modules):
-        grad_shard = group._padded_sharded_param_grad[None]
-        if grad_shard is None:
-            continue
+    for group, key in _grad_classes(modules):
+        grad_shard = group._padded_sharded_param_grad[key]
         group._grad_sumsq_token = None  # the gradients are rewritten
-        for lo, hi in _grad_ranges(group):
+        for lo, hi in _grad_ranges(group, None, key):
             _native.flat_scale(grad_shard[lo:hi], coef)
     return total_norm
 
 
 def zero_grad(modules: nn.Module | Iterable[nn.Module]) -> None:
     """``zero_grad(set_to_none=False)``: one fill per group over its flat gradient shard."""
-    for group in _flat_groups(modules):
-        grad_shard = group._padded_sharded_param_grad[None]
-        if grad_shard is not None:
-            group._grad_sumsq_token = None
-            _native.flat_fill(grad_shard, 0.0)
+    for group, key in _grad_classes(modules):
+        group._grad_sumsq_token = None
+        _native.flat_fill(group._padded_sharded_param_grad[key], 0.0)
 
 
 class _Unit:
     """The parameters of one optimizer param group that live in one flat shard
     (an fsdp parameter group), or one plain tensor outside any group."""
 
-    def __init__(self, group: YaFSDPParamGroup | None, params: list[torch.Tensor], indices: list[int]):
+    def __init__(self, group: YaFSDPParamGroup | None, params: list[torch.Tensor], indices: list[int], key: Any = None):
         self.group = group
+        self.key = key  # all-gather dtype class of the group whose flat shard this is
         self.params = params
-        self.indices = indices  # position of each parameter in group.fsdp_params
+        self.indices = indices  # position of each parameter in the class's parameter list
         if group is not None:
-            _require_one_class(group)
-            shard = group._padded_sharded_param_data[None]
+            shard = group._padded_sharded_param_data[key]
             if shard.dtype != torch.float32:
                 raise TypeError(f"FlatAdamW needs float32 master shards, got {shard.dtype} in {group}")
             self.numel = shard.numel()
@@ -305,12 +305,12 @@ class _Unit:
         p = self.params[k]
         if self.group is None:
             return flat.view(p.shape)
-        return self.group.fsdp_params[self.indices[k]].to_sharded_dtensor(flat, kind="")
+        return self.group._all_gather_dtype_to_fsdp_params[self.key][self.indices[k]].to_sharded_dtensor(flat, kind="")
 
     def fragment(self, k: int) -> tuple[int, int]:
         if self.group is None:
             return 0, self.numel
-        offsets = _fragment_offsets(self.group)
+        offsets = _fragment_offsets(self.group, self.key)
         i = self.indices[k]
         return offsets[i], offsets[i + 1]
 
@@ -360,7 +360,7 @@ class FlatAdamW(torch.optim.Optimizer):
         units = self._units.get(key)
         if units is not None and sum(len(u.params) for u in units) == len(pg["params"]):
             return units
-        by_group: dict[int, tuple[YaFSDPParamGroup, list[torch.Tensor], list[int]]] = {}
+        by_shard: dict[tuple[int, Any], tuple[YaFSDPParamGroup, Any, list[torch.Tensor], list[int]]] = {}
         units = []
         for p in pg["params"]:
             owner = _owner(p)
@@ -368,12 +368,13 @@ class FlatAdamW(torch.optim.Optimizer):
             if group is None:
                 units.append(_Unit(None, [p], [0]))
                 continue
-            entry = by_group.setdefault(id(group), (group, [], []))
-            entry[1].append(p)
-            entry[2].append(owner._index_in_group)
-        for group, ps, idx in by_group.values():
+            cls_key = owner._all_gather_class
+            entry = by_shard.setdefault((id(group), cls_key), (group, cls_key, [], []))
+            entry[2].append(p)
+            entry[3].append(owner._index_in_class)
+        for group, cls_key, ps, idx in by_shard.values():
             order = sorted(range(len(ps)), key=lambda k: idx[k])
-            units.append(_Unit(group, [ps[k] for k in order], [idx[k] for k in order]))
+            units.append(_Unit(group, [ps[k] for k in order], [idx[k] for k in order], cls_key))
         for unit in units:
             for k, p in enumerate(unit.params):
                 lo, hi = unit.fragment(k)
@@ -418,12 +419,14 @@ class FlatAdamW(torch.optim.Optimizer):
             _native.adamw_step(p.view(-1), grad.view(-1), unit.exp_avg, unit.exp_avg_sq, None,
                                step=unit.steps[0], grad_scale=grad_scale, zero_grad=zero_grad, **hyper)
             return
-        shard = group._padded_sharded_param_data[None]
-        grad_shard = group._padded_sharded_param_grad[None]
+        key = unit.key
+        shard = group._padded_sharded_param_data[key]
+        grad_shard = group._padded_sharded_param_grad[key]
         if grad_shard is None:
             return
+        class_params = group._all_gather_dtype_to_fsdp_params[key]
         # launches: maximal runs of fragments that have a gradient and share a step count
-        ranges = _grad_ranges(group, unit.indices)
+        ranges = _grad_ranges(group, unit.indices, key)
         whole = ranges == [(0, shard.numel())]
         with_grad = [k for k, p in enumerate(unit.params) if p.grad is not None]
         if not with_grad:
@@ -434,7 +437,8 @@ class FlatAdamW(torch.optim.Optimizer):
         # the fused copy-in needs the whole shard rewritten in this pass; otherwise the
         # next forward casts the shard itself, as it does in the reference
         out16 = None
-        if (self.fuse_copy_in and whole and uniform and len(unit.indices) == len(group.fsdp_params)
+        # (a tensor-subclass class produces its all-gather input itself, through fsdp_pre_all_gather)
+        if (self.fuse_copy_in and key is None and whole and uniform and len(unit.indices) == len(class_params)
                 and group.param_dtype is not None and hasattr(group, "_all_gather_input") and group.is_sharded):
             out16 = group._all_gather_input[None]
         if whole and uniform:
@@ -458,7 +462,7 @@ class FlatAdamW(torch.optim.Optimizer):
             )
         if out16 is not None:
             # the next unshard finds its all-gather input ready (ya_fsdp/_collectives.py:47-55)
-            for fsdp_param in group.fsdp_params:
+            for fsdp_param in class_params:
                 fsdp_param.set_all_gather_input()
             group._all_gather_input_set_dtypes.add(None)
             group._copy_in_shard_version = shard._version
