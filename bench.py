@@ -1573,7 +1573,10 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     # the line): the step is driven from the host, a region lasts a few milliseconds, and one stall of the host or
     # the machine inside it (seen once in about twenty runs: 25 ms of idle GPU in a 16-ms region, with every
     # sampled kernel at its normal duration) would otherwise decide the figure.
-    dom_index = [n for n, _, _ in ops].index(dominant)  # most bytes, fused arithmetic
+    # the kernel `roofline` reports: the reduce copy-in, the launch with the path's arithmetic fused in (cast, divide,
+    # pad fill) and the lowest fraction of the step's launches (the shared copy-in + copy-out launch moves more bytes
+    # at a higher rate; every launch is in `kernels`)
+    dom_index = [n for n, _, _ in ops].index(dominant)
     # on every 4th step of the timed region (of a long region: on 16 steps spread evenly; attaching the pair costs
     # host time that a launch-bound workload would see) the dominant kernel's dispatch carries a pair of HIP events
     # (attached to the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
