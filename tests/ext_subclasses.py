@@ -74,7 +74,7 @@ class Int8Master(torch.Tensor):
 
         out = func(*unwrap(args), **{k: unwrap(v) for k, v in kwargs.items()})
         if func in _STRUCTURAL:
-            return Int8Master(out)
+            return cls(out)
         if isinstance(out, torch.Tensor) and args and isinstance(args[0], Int8Master) and out is args[0]._data:
             return args[0]  # an in-place op returns what it was called on
         return out

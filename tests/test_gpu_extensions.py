@@ -329,3 +329,33 @@ def test_flat_optimizer_passes_cover_every_all_gather_dtype_class():
     zero_grad(layer)
     for k in keys:
         assert float(group._padded_sharded_param_grad[k].abs().max()) == 0.0
+
+
+def test_malformed_extensions_are_refused_with_a_message():
+    from yafsdp_amd._param_group import YaFSDPParamGroup, init_shared_state
+
+    class PlainNewZeros(Int8Master):
+        """``new_zeros`` falls back to a plain tensor: the sharded parameter would lose the hooks."""
+
+        @classmethod
+        def __torch_dispatch__(cls, func, types, args=(), kwargs=None):
+            if func == torch.ops.aten.new_zeros.default:
+                return func(args[0]._data, *args[1:], **(kwargs or {}))
+            return super().__torch_dispatch__(func, types, args, kwargs)
+
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, all_gather_dtype_to_param_cls={torch.int8: PlainNewZeros})
+    p = nn.Parameter(PlainNewZeros(torch.zeros(32, device=DEV)))
+    with pytest.raises(AssertionError, match="new_zeros returned a plain tensor"):
+        YaFSDPParamGroup([p], FSDPMeshInfo(1, 0), DEV, mp, 8)
+
+    class ShortInput(Int8Master):
+        """``fsdp_pre_all_gather`` returns fewer elements than the fragment holds."""
+
+        def fsdp_pre_all_gather(self, mesh):
+            return (quantize(self._data)[:-1],), (STEP,)
+
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, all_gather_dtype_to_param_cls={torch.int8: ShortInput})
+    group = YaFSDPParamGroup([nn.Parameter(ShortInput(torch.ones(32, device=DEV)))], FSDPMeshInfo(1, 0), DEV, mp, 8)
+    init_shared_state([group], DEV)
+    with pytest.raises(AssertionError, match="returned 31 elements for a fragment of 32"):
+        group.pre_forward()
