@@ -1317,6 +1317,8 @@ def main() -> int:
                                                  "fully-shard-trainer-w1"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
+    ap.add_argument("--no-stream-plan", action="store_true",
+                    help="skip the leg that runs the step on the reference's two streams")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the step from a HIP graph (outside the timed region)")
     ap.add_argument("--no-torch-gpu", action="store_true",
@@ -1645,6 +1647,60 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                      "frac_of_hbm_peak": round(bytes_per_step * n_sus / s_dt / 1e9 / HBM_PEAK_GBS, 4)}
         log(f"sustained: {n_sus} steps in {s_dt:.2f}s, {sustained['value']} GB/s")
 
+    # ---- the same launches on the streams the reference puts them on (outside the timed region): copy-in and
+    # copy-out on the side stream that serves all-gather and reduce-scatter (ya_fsdp/_collectives.py:46,
+    # ya_fsdp/_param_group.py:80-88), the reduce copy-in on the compute stream (ya_fsdp/_param_group.py:669-708), the
+    # post-reduce on the side stream once the compute stream has got there (ya_fsdp/_collectives.py:110-111).  The
+    # timed region above keeps one stream, where the kernels' own durations add up to the step; here independent
+    # kernels overlap their ramps and drains.
+    reference_streams = None
+    if not args.no_stream_plan:
+        try:
+            main_stream, side_stream = torch.cuda.current_stream(dev), torch.cuda.Stream(device=dev)
+
+            def reference_step():
+                done = None
+                for name, fn, _ in ops:
+                    if name.startswith("reduce_copy_in"):
+                        fn()
+                        done = main_stream.record_event()
+                    else:
+                        with torch.cuda.stream(side_stream):
+                            if name == "post_reduce" and done is not None:
+                                side_stream.wait_event(done)
+                            fn()
+
+            n_ref = max(steps, 200)
+            side_stream.wait_stream(main_stream)
+            for _ in range(warmup):
+                reference_step()
+            main_stream.wait_stream(side_stream)
+            torch.cuda.synchronize()
+            r0 = time.perf_counter()
+            for _ in range(n_ref):
+                reference_step()
+            main_stream.wait_stream(side_stream)
+            torch.cuda.synchronize()
+            r_dt = (time.perf_counter() - r0) / n_ref
+            reference_streams = {
+                "plan": "copy-in + copy-out and post-reduce on a side stream, reduce copy-in on the compute stream",
+                "steps": n_ref, "ms_per_step": round(r_dt * 1e3, 4), "value": round(bytes_per_step / r_dt / 1e9, 1),
+                "unit": "GB/s", "frac_of_hbm_peak": round(bytes_per_step / r_dt / 1e9 / HBM_PEAK_GBS, 4)}
+            log(f"the reference's stream placement: {reference_streams['ms_per_step']} ms per step, "
+                f"{reference_streams['value']} GB/s")
+            if not args.no_parity and cpu_state is not None:
+                # the overlapped launches left the same bits (the gradient shard has accumulated many passes:
+                # compare the buffers that every pass rewrites)
+                ok = same(d_ag_in, cpu_state["ag_in"]) and same(d_rs, cpu_state["rs"])
+                ok = ok and all(same(a, b) for a, b in zip(d_outs, cpu_state["outs"]))
+                if not ok:
+                    raise ParityError(f"{workload}: results of the two-stream step differ from the oracle")
+        except ParityError:
+            raise
+        except Exception as exc:  # an optional leg must not cost the measurement above
+            log(f"stream placement leg skipped: {type(exc).__name__}: {exc}")
+            reference_streams = None
+
     # ---- the same step captured into a HIP graph and replayed (outside the timed region): both sides of the table
     # are bound, so the captured launches carry no per-call host work and no staging copy
     graph_replay = None
@@ -1880,6 +1936,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         "torch_gpu_baseline": torch_gpu,
         "graph_replay": graph_replay,
         "sustained": sustained,
+        "reference_stream_placement": reference_streams,
         "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
         "kernels": kernels,
         "kernel_variants": variants,
