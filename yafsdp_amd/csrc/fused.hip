@@ -10,7 +10,7 @@ namespace {
 template <class META, class M, class P, int BLOCK, int US>
 hipError_t unshard_go(const META& meta, const void* gathered, int n_slots, void* ag_in, const void* master, int64_t n,
                       int head, int n_flat_blocks, int grid, hipStream_t stream) {
-  return launch_kernel(unshard_kernel<META, M, P, BLOCK, kFusedFlatUnroll, US, kTableNtLoad, kFlatStorePolicy,
+  return launch_kernel(unshard_kernel<META, M, P, BLOCK, kFusedFlatUnroll, US, scatter_nt_load(US), kFlatStorePolicy,
                                       kScatterStorePolicy>,
                        grid, BLOCK, stream, meta, gathered, n_slots, ag_in, master, n, head, n_flat_blocks);
 }

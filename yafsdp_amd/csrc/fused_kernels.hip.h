@@ -36,7 +36,7 @@ unshard_kernel(META meta, const void* gathered, int n_slots, void* ag_in, const 
                int n_flat_blocks) {
   const int b = blockIdx.x;
   if (b < n_flat_blocks) {
-    flat_body<M, P, SCALE_NONE, false, BLOCK, UF, NTL, STP_FLAT>(ag_in, master, n, head, 1.0f, b, n_flat_blocks);
+    flat_body<M, P, SCALE_NONE, false, BLOCK, UF, kFlatNtLoad, STP_FLAT>(ag_in, master, n, head, 1.0f, b, n_flat_blocks);
   } else {
     scatter_body<META, P, P, BLOCK, US, NTL, STP_SCATTER>(meta, gathered, n_slots, b - n_flat_blocks,
                                                               int(gridDim.x) - n_flat_blocks);

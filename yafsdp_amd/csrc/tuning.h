@@ -76,6 +76,19 @@ constexpr int kScatterShortUnroll = 1;
 constexpr int kTableXcd = YAFSDP_TABLE_XCD;
 constexpr int kTableXcdRun = YAFSDP_TABLE_XCD_RUN;
 constexpr bool kTableNtLoad = YAFSDP_TABLE_NTL;
+// scatter-out reads the flat buffer.  On the short tile (every tensor starts on a cache line of the flat buffer)
+// each line is read once and the loads are non-temporal like everywhere else.  On the long tile the tensors sit at
+// odd offsets, every tile shares its first and last line with a neighbour, and ordinary loads let the L2 keep that
+// line for the other one: copy-out of a 573-tensor table as a launch of its own 108.6 -> 104.1 us (step +0.5 %); in
+// the shared launch of a 1427-tensor table the step is level.  Ordinary loads in gather-in as well move time from
+// one kernel of the step to the next without shortening the step (1427 tensors: copy-out 237 -> 232 us, reduce
+// copy-in 230 -> 236 us), so gather-in keeps non-temporal loads.
+#ifndef YAFSDP_SCATTER_LONG_NTL
+#define YAFSDP_SCATTER_LONG_NTL false
+#endif
+constexpr bool scatter_nt_load(int unroll) {
+  return unroll == 1 ? bool(YAFSDP_TABLE_NTL) : bool(YAFSDP_SCATTER_LONG_NTL);
+}
 #ifndef YAFSDP_GATHER_STP
 #define YAFSDP_GATHER_STP YAFSDP_TABLE_STP
 #endif
