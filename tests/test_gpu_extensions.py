@@ -359,3 +359,28 @@ def test_malformed_extensions_are_refused_with_a_message():
     init_shared_state([group], DEV)
     with pytest.raises(AssertionError, match="returned 31 elements for a fragment of 32"):
         group.pre_forward()
+
+
+def test_full_tensors_reassembles_every_class_from_all_logical_ranks():
+    """``checkpoint.full_tensors`` over the W logical ranks of one group: every parameter of both classes comes back
+    whole, as plain master values, in the group's parameter order; ``load_full_tensors`` puts them back."""
+    from yafsdp_amd.checkpoint import full_tensors, load_full_tensors
+
+    w = 3
+    ranks = [_make(MIXED, w, r, 8)[0] for r in range(w)]
+    for r, g in enumerate(ranks):
+        for i, fp in enumerate(g.fsdp_params):
+            fp._param_fqn = f"p{i}"
+    values = _values(MIXED, 3)
+    got = full_tensors(ranks)
+    assert list(got) == [f"p{i}" for i in range(len(MIXED))]
+    for i, v in enumerate(values):
+        assert type(got[f"p{i}"]) is torch.Tensor and got[f"p{i}"].shape == v.shape
+        assert_bits_equal(got[f"p{i}"], v, f"full parameter {i}")
+    # other values go in through load_full_tensors, rank by rank, and come back
+    g = torch.Generator().manual_seed(77)
+    new = {f"p{i}": torch.randn(s, generator=g).to(DEV) for i, (s, _) in enumerate(MIXED)}
+    load_full_tensors(ranks, new)
+    again = full_tensors(ranks)
+    for k, v in new.items():
+        assert_bits_equal(again[k], v.cpu(), f"reloaded {k}")

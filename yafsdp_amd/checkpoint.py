@@ -202,8 +202,8 @@ def _one_class(group: YaFSDPParamGroup) -> None:
     if group.has_extension_classes:
         raise NotImplementedError(
             f"{group} has tensor-subclass all-gather dtype classes (all_gather_dtype_to_param_cls), each with a flat "
-            "shard of its own: the whole-group helpers cover groups with the default class only; "
-            "sharded_state_dict, full_state_dict and the sharded parameters' own checkpoint hooks work per parameter"
+            "shard of its own: the legacy per-group record describes one flat buffer; full_tensors, "
+            "sharded_state_dict, full_state_dict and the sharded parameters' own checkpoint hooks serve every class"
         )
 
 
@@ -221,13 +221,11 @@ def group_meta_info(group: YaFSDPParamGroup) -> dict[str, list]:
 
 
 def _check_ranks(groups: Sequence[YaFSDPParamGroup]) -> None:
-    for g in groups:
-        _one_class(g)
-    w = groups[0].layout.world_size
+    w = groups[0].mesh_info.shard_mesh_size
     if len(groups) != w:
         raise ValueError(f"need the groups of all {w} ranks, got {len(groups)}")
     for r, g in enumerate(groups):
-        if g.layout != groups[0].layout or g.mesh_info.shard_mesh_rank != r:
+        if g.layouts != groups[0].layouts or g.mesh_info.shard_mesh_rank != r:
             raise ValueError("groups must be the same parameter group on ranks 0..W-1, in rank order")
 
 
@@ -235,31 +233,36 @@ def full_tensors(
     rank_groups: Sequence[YaFSDPParamGroup], out: Mapping[str, torch.Tensor] | None = None
 ) -> dict[str, torch.Tensor]:
     """``full_tensor()`` of every parameter of a group (ya_fsdp/_tensor.py:345-363)
-    from the flat master shards of all its ranks: W ``flat_copy`` launches into a
-    flat buffer, one ``scatter_out`` launch into the full parameters.  ``out``
-    may provide destination tensors (master dtype, contiguous) by fqn."""
+    from the flat master shards of all its ranks: per all-gather dtype class of
+    the group W ``flat_copy`` launches into a flat buffer and one ``scatter_out``
+    launch into the full parameters (plain tensors of the master values, also
+    for tensor-subclass parameters).  ``out`` may provide destination tensors
+    (master dtype, contiguous) by fqn."""
     _check_ranks(rank_groups)
     g0 = rank_groups[0]
-    lay = g0.layout
-    s = lay.padded_sharded_numel
     dtype, device = g0.orig_dtype, g0.device
-    flat = torch.empty(lay.padded_unsharded_numel, dtype=dtype, device=device)
-    for r, g in enumerate(rank_groups):
-        _native.flat_copy(flat[r * s : (r + 1) * s], g._padded_sharded_param_data[None])
-    result, dsts = {}, []
-    for fsdp_param in g0.fsdp_params:
-        fqn = fsdp_param._param_fqn
-        t = out[fqn] if out is not None and fqn in out else torch.empty(fsdp_param._orig_size, dtype=dtype, device=device)
-        if t.dtype != dtype or tuple(t.shape) != tuple(fsdp_param._orig_size) or not t.is_contiguous():
-            raise ValueError(f"{fqn}: destination must be a contiguous {dtype} tensor of shape {tuple(fsdp_param._orig_size)}")
-        result[fqn] = t
-        dsts.append(t.view(-1))
-    table = _native.TensorTable([d.numel() for d in dsts], lay.padded_unsharded_numel, device)
-    try:
-        table.scatter_out(flat, dsts)
-    finally:
-        table.close()
-    return result
+    result = {}
+    for key, fsdp_params in g0._all_gather_dtype_to_fsdp_params.items():
+        lay = g0.layouts[key]
+        s = lay.padded_sharded_numel
+        flat = torch.empty(lay.padded_unsharded_numel, dtype=dtype, device=device)
+        for r, g in enumerate(rank_groups):
+            _native.flat_copy(flat[r * s : (r + 1) * s], g._padded_sharded_param_data[key])
+        dsts = []
+        for fsdp_param in fsdp_params:
+            fqn = fsdp_param._param_fqn
+            t = out[fqn] if out is not None and fqn in out else torch.empty(fsdp_param._orig_size, dtype=dtype, device=device)
+            if t.dtype != dtype or tuple(t.shape) != tuple(fsdp_param._orig_size) or not t.is_contiguous():
+                raise ValueError(f"{fqn}: destination must be a contiguous {dtype} tensor of shape {tuple(fsdp_param._orig_size)}")
+            result[fqn] = t
+            dsts.append(t.view(-1))
+        table = _native.TensorTable([d.numel() for d in dsts], lay.padded_unsharded_numel, device)
+        try:
+            table.scatter_out(flat, dsts)
+        finally:
+            table.close()
+    # in the group's parameter order, whatever the classes
+    return {p._param_fqn: result[p._param_fqn] for p in g0.fsdp_params}
 
 
 def load_full_tensors(groups: YaFSDPParamGroup | Iterable[YaFSDPParamGroup], full: Mapping[str, torch.Tensor]) -> None:
