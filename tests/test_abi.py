@@ -26,7 +26,7 @@ def test_library_exports_every_symbol():
 
     for name in _declared_functions():
         assert hasattr(_native.lib, name), name
-    assert _native.lib.yafsdp_version() == 1000
+    assert _native.lib.yafsdp_version() == 1001  # 1.1: yafsdp_flat_copy_bytes
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
 
@@ -58,6 +58,13 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_flat_copy(0x10000, 1, 0x10000, 0, 64, None) == -1          # same base, 2-byte over 4-byte elements
     assert L.yafsdp_post_reduce(0x10000, 0, 0x100f0, 1, 64, 0.0, 1, None) == -1  # chunk inside the shard
     assert L.yafsdp_flat_copy(0x10000, 1, 0x10000, 1, 64, None) == 0           # self-copy: nothing to do
+    # opaque bytes: same rules at byte granularity
+    assert L.yafsdp_flat_copy_bytes(None, None, -1, None) == -1
+    assert L.yafsdp_flat_copy_bytes(None, None, 8, None) == -1
+    assert L.yafsdp_flat_copy_bytes(None, None, 0, None) == 0
+    assert L.yafsdp_flat_copy_bytes(0x10001, 0x10001, 63, None) == 0             # self-copy
+    assert L.yafsdp_flat_copy_bytes(0x10001, 0x10004, 63, None) == -1            # odd addresses, overlapping
+    assert L.yafsdp_flat_copy_bytes(0x10000, 0x10008, 64, None) == -1            # even addresses, overlapping
     # element counts that cannot be a real buffer are refused at table creation
     import ctypes
 

@@ -298,7 +298,7 @@ int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
 
 extern "C" {
 
-int yafsdp_version(void) { return 1000; }
+int yafsdp_version(void) { return 1001; }
 
 const char* yafsdp_error_string(int code) {
   switch (code) {
