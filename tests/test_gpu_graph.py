@@ -170,3 +170,37 @@ def test_captured_optimizer_side_replays_match_eager():
         assert_bits_equal(captured["out16"], eager["out16"], f"out16, replay {it}")
         assert torch.equal(captured["nc"], eager["nc"]), it
     del graph
+
+
+def test_captured_byte_copy_replays_match_eager():
+    """The byte copy of a 1-byte all-gather dtype (odd addresses, head and tail bytes) is kernel launches only:
+    captured once, replayed with new contents at the same addresses, with eager work in between."""
+    from yafsdp_amd import _native
+
+    n = 300_007
+    g = torch.Generator(device=DEV).manual_seed(5)
+    src_buf = torch.randint(0, 256, (n + 16,), device=DEV, dtype=torch.uint8, generator=g)
+    dst_buf = torch.zeros(n + 32, dtype=torch.uint8, device=DEV)
+    src, dst = src_buf[3 : 3 + n].view(torch.int8), dst_buf[5 : 5 + n].view(torch.int8)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _native.flat_copy(dst, src)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _native.flat_copy(dst, src)
+    for it in range(4):
+        src_buf.copy_(torch.randint(0, 256, (n + 16,), device=DEV, dtype=torch.uint8, generator=g))
+        dst_buf.fill_(0xEE)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = torch.full((n + 32,), 0xEE, dtype=torch.uint8)
+        want[5 : 5 + n] = src_buf[3 : 3 + n].cpu()
+        assert torch.equal(dst_buf.cpu(), want), f"replay {it}"
+        # eager work between the replays
+        eager = torch.zeros(n, dtype=torch.int8, device=DEV)
+        _native.flat_copy(eager, src)
+        assert torch.equal(eager.cpu(), src.cpu())
