@@ -56,7 +56,7 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 
 # HBM bytes per launch of the dominant kernel (gather_in_kernel), from two rocprofv3 --pmc runs
 # (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
-# (factors 1.99990 and 1.00000): (213040.75 * 1.99990 + 426103.375 * 1.00000) KiB.
+# (factors 1.99986 and 1.00000): (213067.8 * 1.99986 + 426086.1 * 1.00000) KiB.
 # Summary and commands: profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.  None = not measured.
 # "llama3-8b-layer-w8-optim": adamw_kernel, (213045.6 * 1.99946 + 372753.5 * 0.99996) KiB, scaled by the plain
 # fp32 copy of the same run; profiles/bench_llama3-8b-layer-w8-optim_hbm_traffic.md.
@@ -68,7 +68,7 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 # "tiny-layer-w1": gather_post_kernel, (9309.25 * 1.99322 + 18534.0) KiB, below the algorithmic bytes of the two
 # kernels it replaces because the reduce buffer is not read back;
 # all three in profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.
-MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872615800, "llama3-8b-layer-w8-optim": 817_885_000,
+MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_645_400, "llama3-8b-layer-w8-optim": 817_885_000,
                           "ragged-stress-w256": 1_505_902_865, "llama3-70b-layer-w64": 3_422_785_664,
                           "ragged-stress-w256-bf16-masters": 1_014_344_628, "tiny-layer-w1": 37_979_573}
 
@@ -1319,6 +1319,8 @@ def main() -> int:
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
     ap.add_argument("--no-stream-plan", action="store_true",
                     help="skip the leg that runs the step on the reference's two streams")
+    ap.add_argument("--no-store-policy-ab", action="store_true",
+                    help="skip the leg that runs the step with the reduce copy-in's write-through tail switched off")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the step from a HIP graph (outside the timed region)")
     ap.add_argument("--no-torch-gpu", action="store_true",
@@ -1647,6 +1649,34 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                      "frac_of_hbm_peak": round(bytes_per_step * n_sus / s_dt / 1e9 / HBM_PEAK_GBS, 4)}
         log(f"sustained: {n_sus} steps in {s_dt:.2f}s, {sustained['value']} GB/s")
 
+    # ---- the same step with the reduce copy-in's write-through tail switched off (outside the timed region): the
+    # library's default writes the end of the reduce buffer through the L2s, which shortens that kernel and leaves
+    # the write-back to overlap what follows; this leg shows what the choice is worth on this workload
+    tail_off = None
+    if not args.no_store_policy_ab:
+        tail_mb = _native.get_option(_native.OPT_GATHER_TAIL_MB)
+        _native.set_option(_native.OPT_GATHER_TAIL_MB, 0)
+        try:
+            n_ab = max(steps, 100)
+            for _ in range(max(1, warmup)):
+                step()
+            torch.cuda.synchronize()
+            a0 = time.perf_counter()
+            for _ in range(n_ab):
+                for fn in fns:
+                    fn()
+            torch.cuda.synchronize()
+            a_dt = (time.perf_counter() - a0) / n_ab
+        finally:
+            _native.set_option(_native.OPT_GATHER_TAIL_MB, tail_mb)
+        for _ in range(max(1, warmup)):  # the legs below start from the default policy's steady state
+            step()
+        torch.cuda.synchronize()
+        tail_off = {"steps": n_ab, "ms_per_step": round(a_dt * 1e3, 4), "value": round(bytes_per_step / a_dt / 1e9, 1),
+                    "unit": "GB/s", "default_tail_mb": tail_mb}
+        log(f"reduce copy-in without its write-through tail: {tail_off['ms_per_step']} ms per step, "
+            f"{tail_off['value']} GB/s (default: last {tail_mb} MB write through)")
+
     # ---- the same launches on the streams the reference puts them on (outside the timed region): copy-in and
     # copy-out on the side stream that serves all-gather and reduce-scatter (ya_fsdp/_collectives.py:46,
     # ya_fsdp/_param_group.py:80-88), the reduce copy-in on the compute stream (ya_fsdp/_param_group.py:669-708), the
@@ -1801,6 +1831,8 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         variant_ops.append(("all_gather_1byte_dtype_odd_addresses", lambda: _native.flat_copy(d_bytes_dst, d_bytes_src),
                             2 * t_pad))
         evict = [f for _, f, _ in ops]
+        last = max(i for i, (name, _, _) in enumerate(ops) if "copy_out" in name)  # the launch that holds copy-out
+        evict_rotated = evict[last + 1:] + evict[:last + 1]
         own_evict = {}
         if has_copy_in and not fused:
             # copy-in and copy-out as ONE launch (two independent jobs in one grid); compare with the sum of the
@@ -1818,7 +1850,10 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             own_evict["copy_in_alone"] = own_evict["copy_out_alone"] = evict[1:]
         for name, fn, nbytes in variant_ops:
             fn()
-            times = time_alone(fn, own_evict.get(name, evict[:2]), reps=10)
+            # (a whole step runs before each sample, rotated so that it ends with the copy-out launch: the caches
+            # are evicted, and the sample does not start behind a kernel that writes through, whose last megabytes
+            # are still on their way to memory when it completes and cost whatever follows 3-5 us)
+            times = time_alone(fn, own_evict.get(name, evict_rotated), reps=10)
             med = statistics.median(times)
             variants[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
                               "GBps": round(nbytes / med / 1e3, 1),
@@ -1937,6 +1972,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         "graph_replay": graph_replay,
         "sustained": sustained,
         "reference_stream_placement": reference_streams,
+        "reduce_copy_in_without_write_through_tail": tail_off,
         "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
         "kernels": kernels,
         "kernel_variants": variants,

@@ -384,10 +384,16 @@ typedef enum yafsdp_option {
   YAFSDP_OPT_TABLE_BLOCKS_PER_CU = 1, /* same for gather-in / scatter-out */
   YAFSDP_OPT_TABLE_LARGE_LOG2 = 2,    /* 0..62: tables created from now on whose padded size exceeds
                                          2^value elements run two waves per workgroup instead of one */
-  YAFSDP_OPT_SCATTER_TILE = 3         /* tile of yafsdp_scatter_out for tables created from now on: 0 = from the
+  YAFSDP_OPT_SCATTER_TILE = 3,        /* tile of yafsdp_scatter_out for tables created from now on: 0 = from the
                                          layout (short 512-element tiles when every tensor starts on a 128-byte
                                          line of the flat buffer, the gather-in tile otherwise), 1 = always
                                          short, 2 = never short */
+  YAFSDP_OPT_GATHER_TAIL_MB = 4       /* 0..2^20, default 96: yafsdp_gather_in / yafsdp_gather_in_bound write the last
+                                         `value` megabytes of the flat buffer through the L2s instead of leaving
+                                         them there as dirty lines (a store-policy choice; the bytes written are
+                                         the same).  The kernel then ends sooner; the write-back it no longer waits
+                                         for overlaps whatever runs next, which pays for it only if it saturates
+                                         the memory itself.  0 = off */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);

@@ -1,6 +1,7 @@
 """The C-ABI library loads without a GPU and exports every symbol that
 include/yafsdp_hip.h declares (no compute calls here)."""
 
+import ctypes
 import os
 import re
 
@@ -26,7 +27,7 @@ def test_library_exports_every_symbol():
 
     for name in _declared_functions():
         assert hasattr(_native.lib, name), name
-    assert _native.lib.yafsdp_version() == 1001  # 1.1: yafsdp_flat_copy_bytes
+    assert _native.lib.yafsdp_version() == 1002  # 1.1: yafsdp_flat_copy_bytes; 1.2: YAFSDP_OPT_GATHER_TAIL_MB
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
 
@@ -51,6 +52,12 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_set_option(2, 28) == 0
     assert L.yafsdp_set_option(3, 3) == -1
     assert L.yafsdp_set_option(3, 0) == 0
+    assert L.yafsdp_set_option(4, -1) == -1
+    assert L.yafsdp_set_option(4, (1 << 20) + 1) == -1
+    tail = ctypes.c_int(-1)
+    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 96
+    assert L.yafsdp_set_option(4, 0) == 0 and L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 0
+    assert L.yafsdp_set_option(4, 96) == 0
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
     # operands that overlap without being the same buffer are refused (addresses are never dereferenced here)
@@ -66,7 +73,6 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_flat_copy_bytes(0x10001, 0x10004, 63, None) == -1            # odd addresses, overlapping
     assert L.yafsdp_flat_copy_bytes(0x10000, 0x10008, 64, None) == -1            # even addresses, overlapping
     # element counts that cannot be a real buffer are refused at table creation
-    import ctypes
 
     import numpy as np
 

@@ -195,6 +195,31 @@ TABLE_CASES = [
                                            (torch.float32, torch.float32)])
 @pytest.mark.parametrize("pre", [None, 8.0, 3.0])
 def test_gather_in(nat, table_workgroup, case, grad_dt, rs_dt, pre):
+    _check_gather_in(nat, case, grad_dt, rs_dt, pre)
+
+
+@pytest.mark.parametrize("tail_mb", [0, 1, 3])
+@pytest.mark.parametrize("large_log2", [None, 0])
+@pytest.mark.parametrize("grad_dt,rs_dt,pre", [(torch.bfloat16, torch.bfloat16, None),
+                                               (torch.float32, torch.bfloat16, 8.0),
+                                               (torch.bfloat16, torch.float32, 3.0)])
+def test_gather_in_with_the_write_through_boundary_inside_the_buffer(nat, tail_mb, large_log2, grad_dt, rs_dt, pre):
+    """The last megabytes of the flat buffer are stored with another cache policy than the rest (0: none are; the
+    default is larger than any buffer of these tests, so everywhere else all tiles are).  Same bytes either way."""
+    default_tail = nat.get_option(nat.OPT_GATHER_TAIL_MB)
+    default_log2 = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
+    nat.set_option(nat.OPT_GATHER_TAIL_MB, tail_mb)
+    if large_log2 is not None:
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, large_log2)
+    try:
+        for case in [(40, 19, False, 513), (33, 14, True, 9), (9, 21, False, 17)]:
+            _check_gather_in(nat, case, grad_dt, rs_dt, pre)
+    finally:
+        nat.set_option(nat.OPT_GATHER_TAIL_MB, default_tail)
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default_log2)
+
+
+def _check_gather_in(nat, case, grad_dt, rs_dt, pre):
     p, max_log2, with_empty, pad = case
     rng = np.random.default_rng(p * 1000 + pad)
     g = torch.Generator().manual_seed(104 + p)

@@ -26,6 +26,7 @@ namespace {
 std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
 std::atomic<int> g_table_blocks_per_cu{kTableBlocksPerCu};
 std::atomic<int> g_table_large_log2{kTableLargeThresholdLog2};
+std::atomic<int> g_gather_tail_mb{kGatherTailWriteThroughMb};
 std::atomic<int> g_scatter_tile_mode{0};
 
 constexpr int kMaxDevices = 64;
@@ -190,6 +191,13 @@ struct yafsdp_binding {
 
 namespace {
 
+// first gather-in tile that writes through: the last YAFSDP_OPT_GATHER_TAIL_MB megabytes of the flat buffer
+int gather_wt_from(const yafsdp_table* t, int flat_dtype) {
+  const int64_t tile_bytes = t->tile_elems * item_size(flat_dtype);
+  const int64_t tail = (int64_t(g_gather_tail_mb.load(std::memory_order_relaxed)) << 20) / tile_bytes;
+  return tail >= t->n_tiles ? 0 : int(t->n_tiles - tail);
+}
+
 void table_free(yafsdp_table* t) {
   if (t == nullptr) return;
   if (t->d_offsets) (void)hipFree(t->d_offsets);
@@ -298,7 +306,7 @@ int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
 
 extern "C" {
 
-int yafsdp_version(void) { return 1001; }
+int yafsdp_version(void) { return 1002; }
 
 const char* yafsdp_error_string(int code) {
   switch (code) {
@@ -396,9 +404,11 @@ int yafsdp_gather_in_bound(yafsdp_binding* binding, void* flat, int flat_dtype, 
   const int grid = grid_for(table_blocks(table->n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallRoute)
     return int(launch_gather<SmallMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->small, flat,
-                                        table->padded, table->n_tiles, k, zero_pad ? 1 : 0, grid, s));
+                                        table->padded, table->n_tiles, k, zero_pad ? 1 : 0, gather_wt_from(table, flat_dtype),
+                                        grid, s));
   return int(launch_gather<LargeMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->large, flat,
-                                      table->padded, table->n_tiles, k, zero_pad ? 1 : 0, grid, s));
+                                      table->padded, table->n_tiles, k, zero_pad ? 1 : 0,
+                                      gather_wt_from(table, flat_dtype), grid, s));
 }
 
 int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat_dtype, void* stream) {
@@ -449,6 +459,11 @@ int yafsdp_set_option(int option, int value) {
     g_table_large_log2.store(value);
     return YAFSDP_OK;
   }
+  if (option == YAFSDP_OPT_GATHER_TAIL_MB) {
+    if (value < 0 || value > (1 << 20)) return YAFSDP_ERR_INVALID_ARGUMENT;
+    g_gather_tail_mb.store(value);
+    return YAFSDP_OK;
+  }
   if (option == YAFSDP_OPT_SCATTER_TILE) {
     if (value < 0 || value > 2) return YAFSDP_ERR_INVALID_ARGUMENT;
     g_scatter_tile_mode.store(value);
@@ -469,6 +484,7 @@ int yafsdp_get_option(int option, int* value) {
     case YAFSDP_OPT_TABLE_BLOCKS_PER_CU: *value = g_table_blocks_per_cu.load(); return YAFSDP_OK;
     case YAFSDP_OPT_TABLE_LARGE_LOG2: *value = g_table_large_log2.load(); return YAFSDP_OK;
     case YAFSDP_OPT_SCATTER_TILE: *value = g_scatter_tile_mode.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_GATHER_TAIL_MB: *value = g_gather_tail_mb.load(); return YAFSDP_OK;
   }
   return YAFSDP_ERR_INVALID_ARGUMENT;
 }
@@ -976,7 +992,7 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
     SmallMeta meta;
     fill_small(table, tensor_ptrs, mode, &meta);
     return int(launch_gather<SmallMeta>(table->block, tensor_dtype, flat_dtype, scale, meta, flat, table->padded,
-                                        n_tiles, k, zero_pad ? 1 : 0, grid, s));
+                                        n_tiles, k, zero_pad ? 1 : 0, gather_wt_from(table, flat_dtype), grid, s));
   }
   std::lock_guard<std::mutex> lock(table->mu);
   LargeMeta meta;
@@ -984,7 +1000,7 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   rc = stage_large(table, tensor_ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
   e = launch_gather<LargeMeta>(table->block, tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
-                               zero_pad ? 1 : 0, grid, s);
+                               zero_pad ? 1 : 0, gather_wt_from(table, flat_dtype), grid, s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }

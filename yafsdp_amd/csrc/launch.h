@@ -48,10 +48,12 @@ hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc,
 
 // META is SmallMeta or LargeMeta (explicitly instantiated in gather.hip / scatter.hip);
 // `block` is the workgroup size the table was built for (kTableBlockSmall or kTableBlockLarge); for launch_scatter
-// it is the table's scatter shape packed as workgroup size * 16 + units per lane
+// it is the table's scatter shape packed as workgroup size * 16 + units per lane.  launch_gather: full tiles from
+// tile `wt_from` on write through (n_tiles: none do)
 template <class META>
 hipError_t launch_gather(int block, int tensor_dt, int flat_dt, int scale, const META& meta, void* flat,
-                         int64_t padded, int n_tiles, float k, int pad_zero, int grid, hipStream_t stream);
+                         int64_t padded, int n_tiles, float k, int pad_zero, int wt_from, int grid,
+                         hipStream_t stream);
 template <class META>
 hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total,
                           int n_tiles, int grid, hipStream_t stream);

@@ -287,10 +287,11 @@ __device__ __forceinline__ int tile_of_block(int b) {
 
 // S: tensor dtype, D: flat buffer dtype.  pad_zero != 0 writes zeros to
 // [total, padded); otherwise pad lanes only see the divide (as in the
-// reference, whose pad content is whatever the buffer held).
+// reference, whose pad content is whatever the buffer held).  Full tiles
+// from tile wt_from on store write-through when STP is ST_NT.
 template <class META, class S, class D, int SCALE, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
-gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero) {
+gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero, int wt_from) {
   if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
@@ -312,6 +313,12 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
       const int mode = rec.mode;
       const char* src = reinterpret_cast<const char*>(rec.base) + rec.delta * S::kSize;
       char* dst = fbase + t0 * D::kSize;
+      if (STP == ST_NT && tile >= wt_from) {  // the end of the buffer writes through (see tuning.h)
+        if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, ST_WT>(dst, src, k);
+        else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, ST_WT>(dst, src, k);
+        else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, ST_WT>(dst, src, k);
+        continue;
+      }
       if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, STP>(dst, src, k);
       else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, STP>(dst, src, k);
       else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, STP>(dst, src, k);

@@ -95,6 +95,19 @@ constexpr bool scatter_nt_load(int unroll) {
 #ifndef YAFSDP_SCATTER_STP
 #define YAFSDP_SCATTER_STP YAFSDP_TABLE_STP
 #endif
+// The table kernels store non-temporal: the L2s keep the written lines and evict them as they fill.  A kernel that
+// ends with its L2s full of dirty lines pays for their write-back before it completes, so the tiles at the END of
+// the buffer write through instead (as the flat kernels do everywhere): the kernel ends with clean L2s, and what
+// it pushed to the memory side is little enough for the memory-side cache to hold it without the next kernel
+// paying for it.  Llama-3-8B layer, 436-MB reduce buffer, bytes written through at the end -> reduce copy-in /
+// step: 0 -> 136.2 us / 0.3283 ms; 64 MB 132.9 / 0.3250; 80 MB 132.3 / 0.3246; 96 MB 131.3 / 0.3237;
+// 112 MB 130.9 / 0.3251; 128 MB: step 0.3334 ms (the post-reduce kernel after it 40 -> 44.6 us).  Only the gather-in
+// kernels do this: the same tail on scatter-out (32 to 160 MB) made the step 2.5 to 3.8 % slower (copy-in-and-
+// copy-out 154.7 -> 156-158 us, and the two kernels after it slower as well).
+#ifndef YAFSDP_GATHER_TAIL_WT_MB
+#define YAFSDP_GATHER_TAIL_WT_MB 96
+#endif
+constexpr int kGatherTailWriteThroughMb = YAFSDP_GATHER_TAIL_WT_MB;  // default of YAFSDP_OPT_GATHER_TAIL_MB
 constexpr int kGatherStorePolicy = YAFSDP_GATHER_STP;
 constexpr int kScatterStorePolicy = YAFSDP_SCATTER_STP;
 inline int table_block_for(long long padded_elems, int threshold_log2) {
