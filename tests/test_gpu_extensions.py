@@ -278,20 +278,68 @@ def test_checkpoint_and_full_tensor_of_extension_parameters(tmp_path):
     assert_bits_equal(other(x), want.cpu(), "forward after loading")
 
 
+@pytest.mark.parametrize("world", [(1, 0), (2, 1)])
+def test_grad_norm_fused_into_the_post_reduce_of_every_all_gather_dtype_class(world):
+    """``enable_fused_grad_norm`` gives every class of a group its own slot of partial sums: after a backward pass the
+    clip coefficient needs no read pass over either gradient shard, and equals the one computed by reading them."""
+    from oracle import cref
+    from yafsdp_amd import _native, fully_shard
+    from yafsdp_amd.optim import disable_fused_grad_norm, enable_fused_grad_norm, fsdp_param_groups, grad_clip_coef
+
+    gen = torch.Generator().manual_seed(37)
+    layer = fully_shard(QLinear(24, 40, gen), mesh=world, mp_policy=INT8_MP)
+    (group,) = fsdp_param_groups(layer)
+    x = torch.randn(16, 24, generator=gen).to(DEV).bfloat16()
+    (layer(x).float().pow(2).mean() * 30.0).backward()  # the gradient shards exist from here on
+    enable_fused_grad_norm(layer)
+    keys = [None, torch.int8]
+    assert list(group._grad_sumsq_slot) == keys
+    layer.zero_grad(set_to_none=True)
+    (layer(x).float().pow(2).mean() * 30.0).backward()
+    for k in keys:
+        assert group._grad_sumsq_token.get(k) == group._padded_sharded_param_grad[k]._version
+    calls = {"read": 0}
+    real = _native.sumsq_partials
+
+    def counting(*a, **kw):
+        calls["read"] += 1
+        return real(*a, **kw)
+
+    _native.sumsq_partials = counting
+    try:
+        norm_fused, coef_fused = grad_clip_coef(layer, 1e-3)
+        assert calls["read"] == 0  # every sum came from a post-reduce
+        # a gradient rewritten behind the library's back (a torch op bumps the shard's version): that class alone
+        # is read again
+        group._padded_sharded_param_grad[torch.int8].mul_(1.0)
+        norm_mixed, _ = grad_clip_coef(layer, 1e-3)
+        assert calls["read"] == 1
+        disable_fused_grad_norm(layer)
+        assert not group._grad_sumsq_slot and group._grad_sumsq_partials is None
+        norm_read, coef_read = grad_clip_coef(layer, 1e-3)
+        assert calls["read"] == 3
+    finally:
+        _native.sumsq_partials = real
+    want, want_coef = cref.clip_coef(
+        sum(cref.sumsq(group._padded_sharded_param_grad[k].detach().cpu()) for k in keys), 1e-3)
+    assert want > 0 and want_coef < 1.0
+    for got in (norm_fused, norm_mixed, norm_read):
+        assert abs(got.item() - want) <= 2e-7 * want
+    assert abs(coef_fused.item() - want_coef) <= 2e-7 * want_coef
+
+
 def test_flat_optimizer_passes_cover_every_all_gather_dtype_class():
     """``grad_clip_coef`` / ``clip_grad_norm_`` / ``zero_grad`` / ``FlatAdamW`` run over the flat shards of both
     classes of a group (ordinary parameters and the int8 all-gather class); the fused copy-in serves the default
     class only, the subclass quantises its own masters in the next forward.  Against the C oracle per flat shard."""
     from oracle import cref
     from yafsdp_amd import fully_shard
-    from yafsdp_amd.optim import FlatAdamW, clip_grad_norm_, enable_fused_grad_norm, fsdp_param_groups, zero_grad
+    from yafsdp_amd.optim import FlatAdamW, clip_grad_norm_, fsdp_param_groups, zero_grad
 
     gen = torch.Generator().manual_seed(31)
     layer = fully_shard(QLinear(24, 40, gen), mesh=(1, 0), mp_policy=INT8_MP)
     (group,) = fsdp_param_groups(layer)
     assert list(group._padded_sharded_param_grad) == [None, torch.int8]
-    with pytest.raises(NotImplementedError, match="default class only"):
-        enable_fused_grad_norm(layer)
     opt = FlatAdamW(layer.parameters(), lr=1e-2, betas=(0.9, 0.95), weight_decay=0.1)
     x = torch.randn(16, 24, generator=gen).to(DEV).bfloat16()
     (layer(x).float().pow(2).mean() * 30.0).backward()

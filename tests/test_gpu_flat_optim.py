@@ -281,7 +281,7 @@ def test_fused_grad_norm_matches_the_read_pass():
     _native.sumsq_partials = counting
     try:
         model(x).float().pow(2).mean().backward()
-        assert all(g._grad_sumsq_token is not None for g in groups)
+        assert all(g._grad_sumsq_token.get(None) is not None for g in groups)
         norm_fused, coef_fused = grad_clip_coef(model, 1e-3)
         assert calls["read"] == 0                      # every sum came from the post-reduce
         disable_fused_grad_norm(model)
@@ -363,7 +363,7 @@ def test_fused_grad_norm_falls_back_when_the_reduce_writes_the_shard_directly():
     enable_fused_grad_norm(model)
     model.zero_grad(set_to_none=True)
     model(x).pow(2).mean().backward()
-    assert all(g._grad_sumsq_token is None for g in fsdp_param_groups(model))
+    assert all(g._grad_sumsq_token.get(None) is None for g in fsdp_param_groups(model))
     norm_a, _ = grad_clip_coef(model, 1.0)
     disable_fused_grad_norm(model)
     norm_b, _ = grad_clip_coef(model, 1.0)
@@ -395,7 +395,7 @@ def test_fused_grad_norm_small_group_with_a_frozen_parameter_in_the_middle():
     assert group._padded_sharded_param_grad[None].numel() <= 4096
     enable_fused_grad_norm(model)
     try:
-        assert group._grad_sumsq_slot[1] - group._grad_sumsq_slot[0] >= 2
+        assert group._grad_sumsq_slot[None][1] - group._grad_sumsq_slot[None][0] >= 2
         model.zero_grad(set_to_none=True)
         model(x).float().pow(2).mean().backward()
         norm_fused, coef_fused = grad_clip_coef(model, 1e-3)   # two ranges: read pass into the group's slot

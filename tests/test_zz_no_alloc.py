@@ -2,6 +2,7 @@
 (``yafsdp_flat_sumsq`` with a caller-provided workspace), called through the C ABI."""
 
 import ctypes
+import gc
 
 import pytest
 import torch
@@ -23,11 +24,17 @@ def _sumsq_pair(lib, src, accumulate, start):
                                nbytes, stream)
     assert rc == 0, lib.yafsdp_error_string(rc)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated(DEV)
-    rc = lib.yafsdp_flat_sumsq_static(src.data_ptr(), dt, src.numel(), got.data_ptr(), int(accumulate), stream)
-    assert rc == 0, lib.yafsdp_error_string(rc)
-    torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated(DEV) == before
+    # (no garbage of earlier tests may be collected, and its device memory returned, between the two readings)
+    gc.collect()
+    gc.disable()
+    try:
+        before = torch.cuda.memory_allocated(DEV)
+        rc = lib.yafsdp_flat_sumsq_static(src.data_ptr(), dt, src.numel(), got.data_ptr(), int(accumulate), stream)
+        assert rc == 0, lib.yafsdp_error_string(rc)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated(DEV) == before
+    finally:
+        gc.enable()
     return want, got
 
 

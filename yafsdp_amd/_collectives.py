@@ -236,11 +236,12 @@ def reduce_scatter(
         param_group = group_ref() if group_ref is not None else None
         # every parameter of the group gets a gradient in this pass: the whole shard is meaningful afterwards
         whole = len(fsdp_params_with_grad) == len(fsdp_params)
+        cls_key = getattr(fsdp_params[0], "_all_gather_class", None) if fsdp_params else None
         if param_group is not None:
-            param_group._grad_sumsq_token = None
+            param_group._grad_sumsq_token.pop(cls_key, None)
         if world_size > 1 and reduce_in_sharded:
             # the collective would have written straight into the shard (:124-125)
-            _post_reduce(param_group, whole, padded_sharded_param_grad, chunk, post, False)
+            _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, chunk, post, False)
         elif world_size == 1 and reduce_in_sharded:
             _div_if_needed(padded_sharded_param_grad, post)
         else:
@@ -248,9 +249,9 @@ def reduce_scatter(
             without_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is None]
             with_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is not None]
             if len(without_sharded_grad) == len(fsdp_params_which_require_grad):
-                _post_reduce(param_group, whole, padded_sharded_param_grad, output_tensor, post, False)  # :185
+                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, False)  # :185
             elif len(with_sharded_grad) == len(fsdp_params_which_require_grad):
-                _post_reduce(param_group, whole, padded_sharded_param_grad, output_tensor, post, True)  # :189
+                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, True)  # :189
             else:
                 with_ids = {id(p) for p in with_sharded_grad}
                 without_ids = {id(p) for p in without_sharded_grad}
@@ -275,13 +276,14 @@ def reduce_scatter(
 
 
 def _post_reduce(
-    param_group: "YaFSDPParamGroup | None", whole: bool, shard: torch.Tensor, chunk: torch.Tensor,
+    param_group: "YaFSDPParamGroup | None", cls_key: Any, whole: bool, shard: torch.Tensor, chunk: torch.Tensor,
     post: float | None, accumulate: bool,
 ) -> None:
-    """``post_reduce``; for a group with a slot for partial sums of squares
-    (``optim.enable_fused_grad_norm``) and a pass that gives every parameter
-    its gradient, the variant that also leaves the squared norm of the shard."""
-    slot = param_group._grad_sumsq_slot if param_group is not None else None
+    """``post_reduce`` of one all-gather dtype class of a group; for a class
+    with a slot for partial sums of squares (``optim.enable_fused_grad_norm``)
+    and a pass that gives every parameter of it its gradient, the variant that
+    also leaves the squared norm of the shard."""
+    slot = param_group._grad_sumsq_slot.get(cls_key) if param_group is not None else None
     if slot is None or not whole:
         _native.post_reduce(shard, chunk, post, accumulate)
         return
@@ -289,7 +291,7 @@ def _post_reduce(
     end = _native.post_reduce_sumsq(shard, chunk, post, accumulate, param_group._grad_sumsq_partials[:hi], lo)
     if end < hi:  # the slot is added up as a whole: entries a read pass may have left beyond these sums go
         param_group._grad_sumsq_partials[end:hi].zero_()
-    param_group._grad_sumsq_token = shard._version
+    param_group._grad_sumsq_token[cls_key] = shard._version
 
 
 def _get_gradient_divide_factors(

@@ -251,11 +251,12 @@ class YaFSDPParamGroup:
         # version of the master shard at which a fused optimizer step last wrote the
         # all-gather input (None: never); see all_gather
         self._copy_in_shard_version: int | None = None
-        # gradient norm fused into the post-reduce (optim.enable_fused_grad_norm): float64 buffer of partial sums,
-        # this group's slice of it, and the version of the gradient shard those sums describe
+        # gradient norm fused into the post-reduce (optim.enable_fused_grad_norm): float64 buffer of partial sums and,
+        # per all-gather dtype class, the class's slice of it and the version of the class's gradient shard those
+        # sums describe (no entry / None: they describe nothing)
         self._grad_sumsq_partials: torch.Tensor | None = None
-        self._grad_sumsq_slot: tuple[int, int] | None = None
-        self._grad_sumsq_token: int | None = None
+        self._grad_sumsq_slot: dict[Any, tuple[int, int]] = {}
+        self._grad_sumsq_token: dict[Any, int | None] = {}
 
     # ------------------------------------------------------------ initialisation --
     def _init_mp_dtypes(self) -> None:
@@ -658,7 +659,7 @@ class YaFSDPParamGroup:
         and the same contents of the reduce buffer afterwards.  Returns False, having launched nothing, for every
         other case; the caller then takes the general route."""
         group = self._reduce_scatter_process_group
-        if group.size() != 1 or self._grad_sumsq_slot is not None:
+        if group.size() != 1 or self._grad_sumsq_slot:
             return False
         if list(self._all_gather_dtype_to_fsdp_params) != [None] or self._table is None:
             return False  # one launch per group: only for a group with the default class alone
@@ -691,7 +692,7 @@ class YaFSDPParamGroup:
             return False
         if not _native.all_contiguous(grads):
             grads = [g if g is None or g.is_contiguous() else g.contiguous() for g in grads]
-        self._grad_sumsq_token = None
+        self._grad_sumsq_token.pop(None, None)
         return self._table.gather_in_post_reduce(
             grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes,
             pre_factor=pre, post_factor=post, custom_divisor=custom,

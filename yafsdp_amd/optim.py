@@ -61,15 +61,6 @@ def _grad_classes(modules: nn.Module | Iterable[nn.Module]) -> "list[tuple[YaFSD
             if shard is not None]
 
 
-def _require_one_class(group: YaFSDPParamGroup) -> None:
-    if group.has_extension_classes:
-        raise NotImplementedError(
-            f"{group} has tensor-subclass all-gather dtype classes (all_gather_dtype_to_param_cls): the gradient "
-            "norm fused into the post-reduce covers groups with the default class only; grad_clip_coef, "
-            "clip_grad_norm_, zero_grad and FlatAdamW work on every class"
-        )
-
-
 def _owner(param: torch.Tensor) -> YaFSDPParam | None:
     ref = getattr(param, "_yafsdp_param", None)
     return ref() if ref is not None else None
@@ -150,8 +141,8 @@ class _ClipState:
 
 def enable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
     """From now on the post-reduce of every ``fully_shard`` group under
-    ``modules`` also leaves the partial sums of squares of the gradient shard it
-    writes (``yafsdp_post_reduce_sumsq``), and ``grad_clip_coef`` /
+    ``modules`` (one per all-gather dtype class of the group) also leaves the
+    partial sums of squares of the gradient shard it writes (``yafsdp_post_reduce_sumsq``), and ``grad_clip_coef`` /
     ``clip_grad_norm_`` over the same ``modules`` add those up instead of
     reading the shards again: 4 bytes per element less per step.  A group
     falls back to the read pass whenever its sums do not describe its current
@@ -159,45 +150,43 @@ def enable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
     the reduce (seen through the shard's version counter), or one of this
     module's own passes that rewrites gradients (scaling, zero-fill).  Kernels
     launched on the gradient shard through ``_native`` directly are not seen."""
-    groups = fsdp_param_groups(modules)
-    for g in groups:
-        _require_one_class(g)
-    groups = [g for g in groups if g._padded_sharded_param_grad[None] is not None]
-    if not groups:
+    classes = _grad_classes(modules)
+    if not classes:
         raise ValueError("no fully_shard parameter group with gradients under the given modules")
-    device = groups[0].device
+    disable_fused_grad_norm(modules)
+    device = classes[0][0].device
     slots, total = [], 0
-    for g in groups:
+    for g, key in classes:
         # one partial sum per tile of the post-reduce; the read pass that replaces it when the sums are stale writes
-        # at least one per gradient range, and a group has at most as many ranges as parameters
-        n = max(_native.post_reduce_sumsq_count(g._padded_sharded_param_grad[None].numel()), len(g.fsdp_params), 1)
+        # at least one per gradient range, and a class has at most as many ranges as parameters
+        n_params = len(g._all_gather_dtype_to_fsdp_params[key])
+        n = max(_native.post_reduce_sumsq_count(g._padded_sharded_param_grad[key].numel()), n_params, 1)
         slots.append((total, total + n))
         total += n
     partials = torch.zeros(total, dtype=torch.float64, device=device)
-    for g, slot in zip(groups, slots):
-        g._grad_sumsq_partials, g._grad_sumsq_slot, g._grad_sumsq_token = partials, slot, None
+    for (g, key), slot in zip(classes, slots):
+        g._grad_sumsq_partials = partials
+        g._grad_sumsq_slot[key] = slot
 
 
 def disable_fused_grad_norm(modules: nn.Module | Iterable[nn.Module]) -> None:
     for g in fsdp_param_groups(modules):
-        g._grad_sumsq_partials, g._grad_sumsq_slot, g._grad_sumsq_token = None, None, None
+        g._grad_sumsq_partials = None
+        g._grad_sumsq_slot.clear()
+        g._grad_sumsq_token.clear()
 
 
-def _invalidate_grad_sumsq(groups: Iterable[YaFSDPParamGroup]) -> None:
-    for g in groups:
-        g._grad_sumsq_token = None
-
-
-def _fused_partials(groups: Sequence[YaFSDPParamGroup]) -> torch.Tensor | None:
-    """The shared buffer of partial sums if exactly these groups fill it, slot after slot."""
-    partials = groups[0]._grad_sumsq_partials
+def _fused_partials(classes: "Sequence[tuple[YaFSDPParamGroup, Any]]") -> torch.Tensor | None:
+    """The shared buffer of partial sums if exactly these gradient shards fill it, slot after slot."""
+    partials = classes[0][0]._grad_sumsq_partials
     if partials is None:
         return None
     end = 0
-    for g in groups:
-        if g._grad_sumsq_partials is not partials or g._grad_sumsq_slot is None or g._grad_sumsq_slot[0] != end:
+    for g, key in classes:
+        slot = g._grad_sumsq_slot.get(key)
+        if g._grad_sumsq_partials is not partials or slot is None or slot[0] != end:
             return None
-        end = g._grad_sumsq_slot[1]
+        end = slot[1]
     return partials if end == partials.numel() else None
 
 
@@ -218,22 +207,22 @@ def grad_clip_coef(
     groups = [g for g, _ in classes]
     device = groups[0].device
     norm_and_coef = torch.empty(2, dtype=torch.float32, device=device)
-    fused = _fused_partials(groups) if all(key is None for _, key in classes) else None
+    fused = _fused_partials(classes)
     if fused is not None:
-        # sums left by the post-reduce where they still describe the gradients; a read pass into the group's own
+        # sums left by the post-reduce where they still describe the gradients; a read pass into the class's own
         # slot (zeroed first: it may write fewer sums than the slot holds) where they do not
-        for g in groups:
-            grad_shard = g._padded_sharded_param_grad[None]
-            ranges = _grad_ranges(g)
-            if ranges == [(0, grad_shard.numel())] and g._grad_sumsq_token == grad_shard._version:
+        for g, key in classes:
+            grad_shard = g._padded_sharded_param_grad[key]
+            ranges = _grad_ranges(g, None, key)
+            if ranges == [(0, grad_shard.numel())] and g._grad_sumsq_token.get(key) == grad_shard._version:
                 continue
-            lo, hi = g._grad_sumsq_slot
+            lo, hi = g._grad_sumsq_slot[key]
             fused[lo:hi].zero_()
             pos = lo
             for k, (a, b) in enumerate(ranges):
                 # leave one entry for each range still to come (the slot holds at least one per parameter)
                 pos = _native.sumsq_partials(grad_shard[a:b], fused[: hi - (len(ranges) - 1 - k)], pos)
-            g._grad_sumsq_token = None
+            g._grad_sumsq_token.pop(key, None)
         if fused.numel() > 4 * _native.SUMSQ_MAX_PARTIALS:  # long array: many workgroups first, then one
             scratch = _ClipState.get(device).reserve(1 + fused.numel() // (4096 * _native.SUMSQ_MAX_PARTIALS))
             count = _native.sumsq_reduce_partials(fused, fused.numel(), scratch)
@@ -261,7 +250,7 @@ def clip_grad_norm_(
     coef = coef.view(1)
     for group, key in _grad_classes(modules):
         grad_shard = group._padded_sharded_param_grad[key]
-        group._grad_sumsq_token = None  # the gradients are rewritten
+        group._grad_sumsq_token.pop(key, None)  # the gradients are rewritten
         for lo, hi in _grad_ranges(group, None, key):
             _native.flat_scale(grad_shard[lo:hi], coef)
     return total_norm
@@ -270,7 +259,7 @@ def clip_grad_norm_(
 def zero_grad(modules: nn.Module | Iterable[nn.Module]) -> None:
     """``zero_grad(set_to_none=False)``: one fill per group over its flat gradient shard."""
     for group, key in _grad_classes(modules):
-        group._grad_sumsq_token = None
+        group._grad_sumsq_token.pop(key, None)
         _native.flat_fill(group._padded_sharded_param_grad[key], 0.0)
 
 
@@ -453,7 +442,7 @@ class FlatAdamW(torch.optim.Optimizer):
                     else:
                         runs.append((lo, hi, unit.steps[k]))
         if zero_grad:
-            group._grad_sumsq_token = None  # the gradients are rewritten
+            group._grad_sumsq_token.pop(key, None)  # the gradients are rewritten
         for lo, hi, step in runs:
             _native.adamw_step(
                 shard[lo:hi], grad_shard[lo:hi], unit.exp_avg[lo:hi], unit.exp_avg_sq[lo:hi],
