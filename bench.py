@@ -378,6 +378,8 @@ def run_full_model(args, as_record: bool = False):
         del before
 
     reps = max(1, args.steps // 10)
+    if as_record:  # a leg of the default line: bounded
+        reps = min(reps, 5)
     caps = (4096, 16, 8, 4, 2, 1) if args.sweep_grid_cap else (4096,)
     gemm_shapes = [("4096x4096x4096", (4096, 4096, 4096)), ("llama-mlp-up 4096x4096x14336", (4096, 4096, 14336)),
                    ("llama-mlp-down 4096x14336x4096", (4096, 14336, 4096))]
@@ -1306,8 +1308,8 @@ def run_ceilings(args) -> int:
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--regions", type=int, default=3,
                     help="how many times the timed region (warm-up + exactly --steps steps) is run; the median is reported")
     ap.add_argument("--workload", default="llama3-8b-layer-w8",
