@@ -1350,6 +1350,9 @@ def main() -> int:
     ap.add_argument("--table-large-log2", type=int, default=None, metavar="N",
                     help="tables with more than 2^N padded elements run two waves per workgroup instead of one "
                          "(the library's launch-shape option; default: the library's own threshold)")
+    ap.add_argument("--gather-tail-mb", type=int, default=None, metavar="N",
+                    help="megabytes at the end of the reduce buffer that the reduce copy-in stores write-through "
+                         "(the library's store-policy option; default: the library's own, 96; 0 = none)")
     ap.add_argument("--analyze-trace", metavar="CSV", default=None,
                     help="llama3-8b-full-w8 only: no GPU work; summarise the kernel-trace CSV that rocprofv3 wrote for "
                          "`--workload llama3-8b-full-w8 --steps 10 --no-parity` (GEMM resource columns, concurrency)")
@@ -1432,6 +1435,8 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     torch.cuda.set_device(dev)
     if args.table_large_log2 is not None:
         _native.set_option(_native.OPT_TABLE_LARGE_LOG2, args.table_large_log2)
+    if args.gather_tail_mb is not None:
+        _native.set_option(_native.OPT_GATHER_TAIL_MB, args.gather_tail_mb)
     # master / compute / reduce dtypes of the group: fp32 masters with bf16 compute and reduce, except the stress
     # test's second group (bf16 masters: no copy-in cast, fp32 reduce buffer, bf16 gradient shard)
     master_dt, rs_dt = torch.float32, torch.bfloat16
