@@ -391,9 +391,10 @@ typedef enum yafsdp_option {
   YAFSDP_OPT_GATHER_TAIL_MB = 4       /* 0..2^20, default 96: yafsdp_gather_in / yafsdp_gather_in_bound write the last
                                          `value` megabytes of the flat buffer through the L2s instead of leaving
                                          them there as dirty lines (a store-policy choice; the bytes written are
-                                         the same).  The kernel then ends sooner; the write-back it no longer waits
-                                         for overlaps whatever runs next, which pays for it only if it saturates
-                                         the memory itself.  0 = off */
+                                         the same).  The memory-side cache absorbs them and drains them after the
+                                         kernel has completed: the kernel ends sooner, and whatever runs next pays
+                                         for the drain only if it saturates the memory itself from its first
+                                         microsecond.  0 = off */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);

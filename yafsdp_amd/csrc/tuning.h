@@ -95,15 +95,18 @@ constexpr bool scatter_nt_load(int unroll) {
 #ifndef YAFSDP_SCATTER_STP
 #define YAFSDP_SCATTER_STP YAFSDP_TABLE_STP
 #endif
-// The table kernels store non-temporal: the L2s keep the written lines and evict them as they fill.  A kernel that
-// ends with its L2s full of dirty lines pays for their write-back before it completes, so the tiles at the END of
-// the buffer write through instead (as the flat kernels do everywhere): the kernel ends with clean L2s, and what
-// it pushed to the memory side is little enough for the memory-side cache to hold it without the next kernel
-// paying for it.  Llama-3-8B layer, 436-MB reduce buffer, bytes written through at the end -> reduce copy-in /
-// step: 0 -> 136.2 us / 0.3283 ms; 64 MB 132.9 / 0.3250; 80 MB 132.3 / 0.3246; 96 MB 131.3 / 0.3237;
-// 112 MB 130.9 / 0.3251; 128 MB: step 0.3334 ms (the post-reduce kernel after it 40 -> 44.6 us).  Only the gather-in
-// kernels do this: the same tail on scatter-out (32 to 160 MB) made the step 2.5 to 3.8 % slower (copy-in-and-
-// copy-out 154.7 -> 156-158 us, and the two kernels after it slower as well).
+// The table kernels store non-temporal: the L2s keep the written lines and evict them as they fill.  The gather-in
+// tiles at the END of the buffer write through instead (as the flat kernels do everywhere).  Two things follow.  The
+// kernel ends with clean L2s: its closing write-back finds no dirty line (40 thousand otherwise).  And the memory-side
+// cache takes the written-through lines faster than DRAM takes evicted ones, as long as it has room for them, and
+// drains them after the kernel has completed, in time that the memory would otherwise spend idle between two kernels
+// (drain of one, ramp of the next).  The gain is linear in the tail: Llama-3-8B layer, 436-MB reduce buffer, bytes
+// written through at the end -> reduce copy-in / step: 0 -> 136.2 us / 0.3263 ms; 16 MB 134.8 / 0.3253;
+// 32 MB 135.1 / 0.3245; 48 MB 133.7 / 0.3242; 64 MB 133.3 / 0.3233; 96 MB 131.5 / 0.3219; another box: 0 -> 136.2 /
+// 0.3283; 96 MB 131.3 / 0.3237; 112 MB 130.9 / 0.3251; 128 MB: step 0.3334 ms (the post-reduce kernel after it 40 ->
+// 44.6 us): beyond about half of the 256-MB memory-side cache the kernel after it pays more than was gained.  Only
+// the gather-in kernels do this: the same tail on scatter-out (32 to 160 MB) made the step 2.5 to 3.8 % slower
+// (copy-in-and-copy-out 154.7 -> 156-158 us, and the two kernels after it slower as well).
 #ifndef YAFSDP_GATHER_TAIL_WT_MB
 #define YAFSDP_GATHER_TAIL_WT_MB 96
 #endif
