@@ -1962,6 +1962,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                    "copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
                    "post-reduce chunk += gradient shard (master dtype) [S]",
             "launches_per_step": [n for n, _, _ in ops],
+            "reduce_copy_in_write_through_tail_mb": _native.get_option(_native.OPT_GATHER_TAIL_MB),
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "parity": parity,
