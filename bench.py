@@ -1322,7 +1322,8 @@ def main() -> int:
     ap.add_argument("--no-stream-plan", action="store_true",
                     help="skip the leg that runs the step on the reference's two streams")
     ap.add_argument("--no-store-policy-ab", action="store_true",
-                    help="skip the leg that runs the step with the reduce copy-in's write-through tail switched off")
+                    help="skip the leg that runs the step with the write-through tails of copy-out and reduce copy-in "
+                         "switched off")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the step from a HIP graph (outside the timed region)")
     ap.add_argument("--no-torch-gpu", action="store_true",
@@ -1352,7 +1353,10 @@ def main() -> int:
                          "(the library's launch-shape option; default: the library's own threshold)")
     ap.add_argument("--gather-tail-mb", type=int, default=None, metavar="N",
                     help="megabytes at the end of the reduce buffer that the reduce copy-in stores write-through "
-                         "(the library's store-policy option; default: the library's own, 96; 0 = none)")
+                         "(the library's store-policy option; default: the library's own, 56; 0 = none)")
+    ap.add_argument("--scatter-tail-mb", type=int, default=None, metavar="N",
+                    help="the same for the last megabytes of tensors that copy-out writes (default: the library's "
+                         "own, 32; 0 = none)")
     ap.add_argument("--analyze-trace", metavar="CSV", default=None,
                     help="llama3-8b-full-w8 only: no GPU work; summarise the kernel-trace CSV that rocprofv3 wrote for "
                          "`--workload llama3-8b-full-w8 --steps 10 --no-parity` (GEMM resource columns, concurrency)")
@@ -1437,6 +1441,8 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         _native.set_option(_native.OPT_TABLE_LARGE_LOG2, args.table_large_log2)
     if args.gather_tail_mb is not None:
         _native.set_option(_native.OPT_GATHER_TAIL_MB, args.gather_tail_mb)
+    if args.scatter_tail_mb is not None:
+        _native.set_option(_native.OPT_SCATTER_TAIL_MB, args.scatter_tail_mb)
     # master / compute / reduce dtypes of the group: fp32 masters with bf16 compute and reduce, except the stress
     # test's second group (bf16 masters: no copy-in cast, fp32 reduce buffer, bf16 gradient shard)
     master_dt, rs_dt = torch.float32, torch.bfloat16
@@ -1656,15 +1662,18 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                      "frac_of_hbm_peak": round(bytes_per_step * n_sus / s_dt / 1e9 / HBM_PEAK_GBS, 4)}
         log(f"sustained: {n_sus} steps in {s_dt:.2f}s, {sustained['value']} GB/s")
 
-    # ---- the same step with the reduce copy-in's write-through tail switched off (outside the timed region): the
-    # library's default writes the end of the reduce buffer through the L2s, which shortens that kernel and leaves
-    # the write-back to overlap what follows; this leg shows what the choice is worth on this workload
+    # ---- the same step with the write-through tails of copy-out and reduce copy-in switched off (outside the timed
+    # region): the library's default writes the end of each of the two big outputs through the L2s, which shortens
+    # those kernels and leaves the write-back to overlap what follows; this leg shows what the choice is worth on this
+    # workload
     tail_off = None
     if not args.no_store_policy_ab:
         tail_mb = _native.get_option(_native.OPT_GATHER_TAIL_MB)
+        scatter_tail_mb = _native.get_option(_native.OPT_SCATTER_TAIL_MB)
         _native.set_option(_native.OPT_GATHER_TAIL_MB, 0)
+        _native.set_option(_native.OPT_SCATTER_TAIL_MB, 0)
         try:
-            n_ab = max(steps, 100)
+            n_ab = max(steps, 1000)  # long enough for its closing synchronisation not to show (compare: sustained)
             for _ in range(max(1, warmup)):
                 step()
             torch.cuda.synchronize()
@@ -1676,13 +1685,14 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             a_dt = (time.perf_counter() - a0) / n_ab
         finally:
             _native.set_option(_native.OPT_GATHER_TAIL_MB, tail_mb)
+            _native.set_option(_native.OPT_SCATTER_TAIL_MB, scatter_tail_mb)
         for _ in range(max(1, warmup)):  # the legs below start from the default policy's steady state
             step()
         torch.cuda.synchronize()
         tail_off = {"steps": n_ab, "ms_per_step": round(a_dt * 1e3, 4), "value": round(bytes_per_step / a_dt / 1e9, 1),
-                    "unit": "GB/s", "default_tail_mb": tail_mb}
-        log(f"reduce copy-in without its write-through tail: {tail_off['ms_per_step']} ms per step, "
-            f"{tail_off['value']} GB/s (default: last {tail_mb} MB write through)")
+                    "unit": "GB/s", "default_scatter_tail_mb": scatter_tail_mb, "default_gather_tail_mb": tail_mb}
+        log(f"without the write-through tails: {tail_off['ms_per_step']} ms per step, {tail_off['value']} GB/s "
+            f"(default: last {scatter_tail_mb} MB of copy-out and last {tail_mb} MB of reduce copy-in write through)")
 
     # ---- the same launches on the streams the reference puts them on (outside the timed region): copy-in and
     # copy-out on the side stream that serves all-gather and reduce-scatter (ya_fsdp/_collectives.py:46,
@@ -1782,12 +1792,25 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             graph_replay = None
 
     # ---- per-kernel table (outside the timed region): each op's dispatch timed on its own
-    def time_alone(fn, others, reps=20):
+    tail_options = (_native.OPT_SCATTER_TAIL_MB, _native.OPT_GATHER_TAIL_MB)
+
+    def time_alone(fn, others, reps=20, plain_evictors=False):
+        """Durations of `fn`'s own dispatch, each right behind the launches `others`.  plain_evictors: those run with
+        their write-through tails off, so that the sample does not inherit the megabytes which they would leave in
+        the memory-side cache for later write-back."""
         times = []
+        tails = [_native.get_option(o) for o in tail_options]
         for _ in range(reps):
             a, b = _event_pair()
-            for f in others:  # evict: the other ops stream 1-2 GB through the caches
-                f()
+            if plain_evictors:
+                for o in tail_options:
+                    _native.set_option(o, 0)
+            try:
+                for f in others:  # evict: the other ops stream 1-2 GB through the caches
+                    f()
+            finally:
+                for o, v in zip(tail_options, tails):
+                    _native.set_option(o, v)
             _native.time_next_launch(a, b)
             fn()
             torch.cuda.synchronize()
@@ -1838,8 +1861,6 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         variant_ops.append(("all_gather_1byte_dtype_odd_addresses", lambda: _native.flat_copy(d_bytes_dst, d_bytes_src),
                             2 * t_pad))
         evict = [f for _, f, _ in ops]
-        last = max(i for i, (name, _, _) in enumerate(ops) if "copy_out" in name)  # the launch that holds copy-out
-        evict_rotated = evict[last + 1:] + evict[:last + 1]
         own_evict = {}
         if has_copy_in and not fused:
             # copy-in and copy-out as ONE launch (two independent jobs in one grid); compare with the sum of the
@@ -1857,14 +1878,19 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             own_evict["copy_in_alone"] = own_evict["copy_out_alone"] = evict[1:]
         for name, fn, nbytes in variant_ops:
             fn()
-            # (a whole step runs before each sample, rotated so that it ends with the copy-out launch: the caches
-            # are evicted, and the sample does not start behind a kernel that writes through, whose last megabytes
-            # are still on their way to memory when it completes and cost whatever follows 3-5 us)
-            times = time_alone(fn, own_evict.get(name, evict_rotated), reps=10)
+            # (the step's first two launches run before each sample, so the caches hold nothing of the sample's
+            # operands.  These forms are not part of the timed step: us_median rates the kernel by itself, behind
+            # evicting launches with their write-through tails off, which leave little in the memory-side cache for
+            # the sample to write back; us_median_behind_step is the same sample behind the same launches as the
+            # library runs them by default.)
+            evictors = own_evict.get(name, evict[:2])
+            times = time_alone(fn, evictors, reps=10, plain_evictors=True)
+            behind = statistics.median(time_alone(fn, evictors, reps=10))
             med = statistics.median(times)
             variants[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
                               "GBps": round(nbytes / med / 1e3, 1),
-                              "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+                              "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
+                              "us_median_behind_step": round(behind, 2)}
             log(f"  {name:26s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s")
         del d_shard_b, d_gathered_b, d_rs_b
     except Exception as exc:  # an optional leg must not cost the measurement above
@@ -1962,6 +1988,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                    "copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
                    "post-reduce chunk += gradient shard (master dtype) [S]",
             "launches_per_step": [n for n, _, _ in ops],
+            "copy_out_write_through_tail_mb": _native.get_option(_native.OPT_SCATTER_TAIL_MB),
             "reduce_copy_in_write_through_tail_mb": _native.get_option(_native.OPT_GATHER_TAIL_MB),
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
@@ -1980,7 +2007,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         "graph_replay": graph_replay,
         "sustained": sustained,
         "reference_stream_placement": reference_streams,
-        "reduce_copy_in_without_write_through_tail": tail_off,
+        "without_write_through_tails": tail_off,
         "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
         "kernels": kernels,
         "kernel_variants": variants,

@@ -27,7 +27,7 @@ def test_library_exports_every_symbol():
 
     for name in _declared_functions():
         assert hasattr(_native.lib, name), name
-    assert _native.lib.yafsdp_version() == 1002  # 1.1: yafsdp_flat_copy_bytes; 1.2: YAFSDP_OPT_GATHER_TAIL_MB
+    assert _native.lib.yafsdp_version() == 1003  # 1.1: yafsdp_flat_copy_bytes; 1.2, 1.3: the two write-through tail options
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
 
@@ -55,9 +55,14 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_set_option(4, -1) == -1
     assert L.yafsdp_set_option(4, (1 << 20) + 1) == -1
     tail = ctypes.c_int(-1)
-    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 96
+    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 56
     assert L.yafsdp_set_option(4, 0) == 0 and L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 0
-    assert L.yafsdp_set_option(4, 96) == 0
+    assert L.yafsdp_set_option(4, 56) == 0
+    assert L.yafsdp_set_option(5, -1) == -1
+    assert L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 32
+    assert L.yafsdp_set_option(5, 7) == 0 and L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 7
+    assert L.yafsdp_set_option(5, 32) == 0
+    assert L.yafsdp_set_option(6, 1) == -1
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
     # operands that overlap without being the same buffer are refused (addresses are never dereferenced here)

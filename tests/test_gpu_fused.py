@@ -112,6 +112,27 @@ def test_copy_in_scatter_out(nat, case, master_dt, param_dt, shard_n):
     table.close()
 
 
+@pytest.mark.parametrize("tail_mb", [0, 1, 3])
+@pytest.mark.parametrize("two_waves", [False, True])
+@pytest.mark.parametrize("master_dt,param_dt", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)])
+def test_copy_out_with_the_write_through_boundary_inside_the_tensors(nat, tail_mb, two_waves, master_dt, param_dt):
+    """The tile slots of the last megabytes of tensors are stored with another cache policy than the rest (0: none
+    are; the default is larger than all tensors of the other tests together, so there all are), in the shared launch
+    and in scatter-out as a launch of its own.  Same bytes either way."""
+    default_tail = nat.get_option(nat.OPT_SCATTER_TAIL_MB)
+    default_log2 = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
+    nat.set_option(nat.OPT_SCATTER_TAIL_MB, tail_mb)
+    if two_waves:
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0)
+    try:
+        for case in [(7, 19, False, 513, False), (9, 17, False, 64, True), (33, 14, True, 9, False),
+                     (5, 21, False, 0, True)]:
+            test_copy_in_scatter_out(nat, case, master_dt, param_dt, 4099)
+    finally:
+        nat.set_option(nat.OPT_SCATTER_TAIL_MB, default_tail)
+        nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default_log2)
+
+
 def test_copy_in_scatter_out_declines_and_errors(nat):
     flat = torch.ones(16, dtype=torch.bfloat16, device=DEV)
     ag = torch.zeros(8, dtype=torch.bfloat16, device=DEV)

@@ -32,7 +32,8 @@ except ImportError:  # not built: the Python checks below do the same work, slow
 
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MODE_SKIP, MODE_COPY, MODE_ADD = 0, 1, 2
-OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU, OPT_TABLE_LARGE_LOG2, OPT_SCATTER_TILE, OPT_GATHER_TAIL_MB = 0, 1, 2, 3, 4
+OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU, OPT_TABLE_LARGE_LOG2, OPT_SCATTER_TILE = 0, 1, 2, 3
+OPT_GATHER_TAIL_MB, OPT_SCATTER_TAIL_MB = 4, 5
 
 # every symbol include/yafsdp_hip.h declares
 EXPORTED_SYMBOLS = (

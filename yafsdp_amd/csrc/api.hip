@@ -27,6 +27,7 @@ std::atomic<int> g_flat_blocks_per_cu{kFlatBlocksPerCu};
 std::atomic<int> g_table_blocks_per_cu{kTableBlocksPerCu};
 std::atomic<int> g_table_large_log2{kTableLargeThresholdLog2};
 std::atomic<int> g_gather_tail_mb{kGatherTailWriteThroughMb};
+std::atomic<int> g_scatter_tail_mb{kScatterTailWriteThroughMb};
 std::atomic<int> g_scatter_tile_mode{0};
 
 constexpr int kMaxDevices = 64;
@@ -194,8 +195,17 @@ namespace {
 // first gather-in tile that writes through: the last YAFSDP_OPT_GATHER_TAIL_MB megabytes of the flat buffer
 int gather_wt_from(const yafsdp_table* t, int flat_dtype) {
   const int64_t tile_bytes = t->tile_elems * item_size(flat_dtype);
+  if (tile_bytes <= 0) return 0;
   const int64_t tail = (int64_t(g_gather_tail_mb.load(std::memory_order_relaxed)) << 20) / tile_bytes;
   return tail >= t->n_tiles ? 0 : int(t->n_tiles - tail);
+}
+
+// first scatter-out tile slot that writes through: the slots of the last YAFSDP_OPT_SCATTER_TAIL_MB megabytes of tensors
+int scatter_wt_from(const yafsdp_table* t, int tensor_dtype) {
+  const int64_t slot_bytes = t->slot_elems * item_size(tensor_dtype);
+  if (slot_bytes <= 0) return 0;  // a table without elements launches nothing
+  const int64_t tail = (int64_t(g_scatter_tail_mb.load(std::memory_order_relaxed)) << 20) / slot_bytes;
+  return tail >= t->n_slots ? 0 : int(t->n_slots - tail);
 }
 
 void table_free(yafsdp_table* t) {
@@ -306,7 +316,7 @@ int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
 
 extern "C" {
 
-int yafsdp_version(void) { return 1002; }
+int yafsdp_version(void) { return 1003; }
 
 const char* yafsdp_error_string(int code) {
   switch (code) {
@@ -426,9 +436,11 @@ int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat
   const int grid = grid_for(table_blocks(table->n_slots), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallRoute)
     return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->small, flat,
-                                         table->total, table->n_slots, grid, s));
+                                         table->total, table->n_slots, scatter_wt_from(table, binding->tensor_dtype),
+                                         grid, s));
   return int(launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->large, flat,
-                                       table->total, table->n_slots, grid, s));
+                                       table->total, table->n_slots, scatter_wt_from(table, binding->tensor_dtype),
+                                       grid, s));
 }
 
 int yafsdp_time_next_launch(void* start_event, void* stop_event) {
@@ -459,9 +471,9 @@ int yafsdp_set_option(int option, int value) {
     g_table_large_log2.store(value);
     return YAFSDP_OK;
   }
-  if (option == YAFSDP_OPT_GATHER_TAIL_MB) {
+  if (option == YAFSDP_OPT_GATHER_TAIL_MB || option == YAFSDP_OPT_SCATTER_TAIL_MB) {
     if (value < 0 || value > (1 << 20)) return YAFSDP_ERR_INVALID_ARGUMENT;
-    g_gather_tail_mb.store(value);
+    (option == YAFSDP_OPT_GATHER_TAIL_MB ? g_gather_tail_mb : g_scatter_tail_mb).store(value);
     return YAFSDP_OK;
   }
   if (option == YAFSDP_OPT_SCATTER_TILE) {
@@ -485,6 +497,7 @@ int yafsdp_get_option(int option, int* value) {
     case YAFSDP_OPT_TABLE_LARGE_LOG2: *value = g_table_large_log2.load(); return YAFSDP_OK;
     case YAFSDP_OPT_SCATTER_TILE: *value = g_scatter_tile_mode.load(); return YAFSDP_OK;
     case YAFSDP_OPT_GATHER_TAIL_MB: *value = g_gather_tail_mb.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_SCATTER_TAIL_MB: *value = g_scatter_tail_mb.load(); return YAFSDP_OK;
   }
   return YAFSDP_ERR_INVALID_ARGUMENT;
 }
@@ -1040,12 +1053,13 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   if (grid == 0) return YAFSDP_OK;
   if (grid > int64_t(INT32_MAX) - 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int wt_from = scatter_wt_from(table, flat_dtype);  // the tensors have the gathered buffer's dtype here
   if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     static const void* const kNoPtrs[kSmallMax] = {};
     fill_small(table, table->total > 0 ? ptrs : kNoPtrs, mode, &meta);
     return int(launch_unshard<SmallMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots),
-                                         ag_in, master, n, int(head), int(n_flat_blocks), int(grid), s));
+                                         wt_from, ag_in, master, n, int(head), int(n_flat_blocks), int(grid), s));
   }
   if (table->total == 0)  // nothing to split: the cast alone
     return flat_launch(master_dtype, flat_dtype, SCALE_NONE, false, ag_in, master, n, 1.0f, s);
@@ -1054,8 +1068,8 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   int slot = -1;
   const int rc = stage_large(table, ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
-  e = launch_unshard<LargeMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots), ag_in, master,
-                                n, int(head), int(n_flat_blocks), int(grid), s);
+  e = launch_unshard<LargeMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots), wt_from, ag_in,
+                                master, n, int(head), int(n_flat_blocks), int(grid), s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }
@@ -1134,14 +1148,15 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
     SmallMeta meta;
     fill_small(table, ptrs, mode, &meta);
     return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,
-                                         grid, s));
+                                         scatter_wt_from(table, tensor_dtype), grid, s));
   }
   std::lock_guard<std::mutex> lock(table->mu);
   LargeMeta meta;
   int slot = -1;
   rc = stage_large(table, ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
-  e = launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles, grid, s);
+  e = launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,
+                                scatter_wt_from(table, tensor_dtype), grid, s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }

@@ -5,7 +5,8 @@
 //    input) and the materialising copy-out of a gathered buffer as ONE grid.
 //    The two jobs do not depend on each other (the copy-out reads a gathered
 //    buffer that is already complete); the first `n_flat_blocks` workgroups
-//    run the flat pass, the others the scatter-out tile slots.
+//    run the flat pass, the others the scatter-out tile slots (full tiles
+//    of the slots from `wt_from` on store write-through, see tuning.h).
 //
 //  * gather_post_kernel: reduce copy-in and post-reduce as one pass, for a
 //    shard group of size ONE.  There the rank's chunk of the reduce buffer IS
@@ -32,13 +33,13 @@ namespace yafsdp {
 // M: master dtype, P: dtype of the all-gather input, of the gathered buffer and of the tensors.
 template <class META, class M, class P, int BLOCK, int UF, int US, bool NTL, int STP_FLAT, int STP_SCATTER>
 __global__ void __launch_bounds__(BLOCK)
-unshard_kernel(META meta, const void* gathered, int n_slots, void* ag_in, const void* master, int64_t n, int head,
-               int n_flat_blocks) {
+unshard_kernel(META meta, const void* gathered, int n_slots, int wt_from, void* ag_in, const void* master, int64_t n,
+               int head, int n_flat_blocks) {
   const int b = blockIdx.x;
   if (b < n_flat_blocks) {
     flat_body<M, P, SCALE_NONE, false, BLOCK, UF, kFlatNtLoad, STP_FLAT>(ag_in, master, n, head, 1.0f, b, n_flat_blocks);
   } else {
-    scatter_body<META, P, P, BLOCK, US, NTL, STP_SCATTER>(meta, gathered, n_slots, b - n_flat_blocks,
+    scatter_body<META, P, P, BLOCK, US, NTL, STP_SCATTER>(meta, gathered, n_slots, wt_from, b - n_flat_blocks,
                                                               int(gridDim.x) - n_flat_blocks);
   }
 }

@@ -48,15 +48,15 @@ hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc,
 
 // META is SmallMeta or LargeMeta (explicitly instantiated in gather.hip / scatter.hip);
 // `block` is the workgroup size the table was built for (kTableBlockSmall or kTableBlockLarge); for launch_scatter
-// it is the table's scatter shape packed as workgroup size * 16 + units per lane.  launch_gather: full tiles from
-// tile `wt_from` on write through (n_tiles: none do)
+// it is the table's scatter shape packed as workgroup size * 16 + units per lane.  Full tiles from tile (gather-in)
+// or tile slot (scatter-out, launch_unshard) `wt_from` on write through (n_tiles: none do)
 template <class META>
 hipError_t launch_gather(int block, int tensor_dt, int flat_dt, int scale, const META& meta, void* flat,
                          int64_t padded, int n_tiles, float k, int pad_zero, int wt_from, int grid,
                          hipStream_t stream);
 template <class META>
 hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& meta, const void* flat, int64_t total,
-                          int n_tiles, int grid, hipStream_t stream);
+                          int n_tiles, int wt_from, int grid, hipStream_t stream);
 
 // the two fused launches (fused.hip).  launch_unshard: the first n_flat_blocks workgroups of the grid cast
 // master[0:n] into ag_in (tiles of workgroup size * kFusedFlatUnroll units), the others run the scatter-out tile
@@ -65,8 +65,8 @@ hipError_t launch_scatter(int block, int flat_dt, int tensor_dt, const META& met
 constexpr int kFusedFlatUnroll = 2;
 template <class META>
 hipError_t launch_unshard(int scatter_shape, int master_dt, int param_dt, const META& meta, const void* gathered,
-                          int n_slots, void* ag_in, const void* master, int64_t n, int head, int n_flat_blocks,
-                          int grid, hipStream_t stream);
+                          int n_slots, int wt_from, void* ag_in, const void* master, int64_t n, int head,
+                          int n_flat_blocks, int grid, hipStream_t stream);
 // reduce copy-in + post-reduce of a size-1 shard group; `block`: the table's gather-in workgroup size
 // The divides of the reduce step, applied by that kernel at run time (wave-uniform branches; a shard group of size
 // one has none unless the caller set a custom factor or reduces in fp16 with one):

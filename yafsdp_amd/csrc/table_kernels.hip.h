@@ -399,10 +399,12 @@ __device__ __forceinline__ void scatter_segment(char* dst, const char* src, int6
 }
 
 // S: flat buffer dtype, D: tensor dtype.  Tensors with mode 0 are not written;
-// pad lanes of the flat buffer are never read.  n_tiles counts tile slots.  `block` of `n_blocks`: the workgroup's
-// place in the grid of scatter_out_kernel, or in the part of a larger grid that serves this job.
+// pad lanes of the flat buffer are never read.  n_tiles counts tile slots; full tiles of the slots from wt_from on
+// store write-through when STP is ST_NT.  `block` of `n_blocks`: the workgroup's place in the grid of
+// scatter_out_kernel, or in the part of a larger grid that serves this job.
 template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
-__device__ __forceinline__ void scatter_body(const META& meta, const void* flat, int n_tiles, int block, int n_blocks) {
+__device__ __forceinline__ void scatter_body(const META& meta, const void* flat, int n_tiles, int wt_from, int block,
+                                             int n_blocks) {
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   constexpr int64_t kLineElems = 128 / D::kSize;
@@ -428,17 +430,21 @@ __device__ __forceinline__ void scatter_body(const META& meta, const void* flat,
     if (lo >= hi) continue;
     char* dst = tbase + lo * D::kSize;
     const char* src = fbase + (o0 + lo) * S::kSize;
-    if (hi - lo == kTile) scatter_full_tile<S, D, BLOCK, U, NTL, STP>(dst, src);
-    else scatter_segment<S, D, BLOCK, NTL, NTS>(dst, src, hi - lo);
+    if (hi - lo == kTile) {
+      if (STP == ST_NT && tile >= wt_from) scatter_full_tile<S, D, BLOCK, U, NTL, ST_WT>(dst, src);
+      else scatter_full_tile<S, D, BLOCK, U, NTL, STP>(dst, src);
+    } else {
+      scatter_segment<S, D, BLOCK, NTL, NTS>(dst, src, hi - lo);
+    }
   }
 }
 
 template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
-scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles) {
+scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles, int wt_from) {
   if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   (void)total;
-  scatter_body<META, S, D, BLOCK, U, NTL, STP>(meta, flat, n_tiles, int(blockIdx.x), int(gridDim.x));
+  scatter_body<META, S, D, BLOCK, U, NTL, STP>(meta, flat, n_tiles, wt_from, int(blockIdx.x), int(gridDim.x));
 }
 
 }  // namespace yafsdp

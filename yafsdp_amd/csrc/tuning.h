@@ -95,22 +95,29 @@ constexpr bool scatter_nt_load(int unroll) {
 #ifndef YAFSDP_SCATTER_STP
 #define YAFSDP_SCATTER_STP YAFSDP_TABLE_STP
 #endif
-// The table kernels store non-temporal: the L2s keep the written lines and evict them as they fill.  The gather-in
-// tiles at the END of the buffer write through instead (as the flat kernels do everywhere).  Two things follow.  The
+// The table kernels store non-temporal: the L2s keep the written lines and evict them as they fill.  The tiles at
+// the END of a launch's output write through instead (as the flat kernels do everywhere): the last megabytes of the
+// flat buffer in gather-in, the tile slots of the last megabytes of tensors in scatter-out.  Two things follow.  The
 // kernel ends with clean L2s: its closing write-back finds no dirty line (40 thousand otherwise).  And the memory-side
 // cache takes the written-through lines faster than DRAM takes evicted ones, as long as it has room for them, and
-// drains them after the kernel has completed, in time that the memory would otherwise spend idle between two kernels
-// (drain of one, ramp of the next).  The gain is linear in the tail: Llama-3-8B layer, 436-MB reduce buffer, bytes
-// written through at the end -> reduce copy-in / step: 0 -> 136.2 us / 0.3263 ms; 16 MB 134.8 / 0.3253;
-// 32 MB 135.1 / 0.3245; 48 MB 133.7 / 0.3242; 64 MB 133.3 / 0.3233; 96 MB 131.5 / 0.3219; another box: 0 -> 136.2 /
-// 0.3283; 96 MB 131.3 / 0.3237; 112 MB 130.9 / 0.3251; 128 MB: step 0.3334 ms (the post-reduce kernel after it 40 ->
-// 44.6 us): beyond about half of the 256-MB memory-side cache the kernel after it pays more than was gained.  Only
-// the gather-in kernels do this: the same tail on scatter-out (32 to 160 MB) made the step 2.5 to 3.8 % slower
-// (copy-in-and-copy-out 154.7 -> 156-158 us, and the two kernels after it slower as well).
+// writes them back when later traffic evicts them, partly in time that the memory would otherwise spend idle between
+// two kernels (drain of one, ramp of the next).  The gain is linear in the tail up to a budget that consecutive kernels share:
+// about 100 MB of write-through data in flight; beyond it the kernels that follow pay more than was gained.
+// Llama-3-8B layer (copy-in + copy-out, reduce copy-in, post-reduce; ms per step), scatter tail / gather tail in MB:
+// 0 / 0 0.3274; 0 / 48 0.3249; 0 / 64 0.3239; 0 / 96 0.3226; 0 / 128 0.3334; 32 / 0 0.3232; 24 / 56 0.3205;
+// 32 / 48 0.3205; 32 / 56 0.3200; 32 / 64 0.3200; 32 / 72 0.3216; 32 / 96 0.3295; 40 / 56 0.3202; 40 / 64 0.3218.
+// 70B layer: 0 / 0 1.0827; 0 / 96 1.0775; 32 / 56 1.0685.  Back to back with a kernel that saturates the memory from
+// its first microsecond the deferred write-back is not free: the two ragged groups at a shard group of 256 (4-us
+// post-reduce, so the next copy-out follows the reduce copy-in at once) 0 / 0 0.4741 and 0.2716; 32 / 0 0.4741 and
+// 0.2728; 32 / 56 0.4765 and 0.2765; 0 / 96 0.4776 and 0.2770.
 #ifndef YAFSDP_GATHER_TAIL_WT_MB
-#define YAFSDP_GATHER_TAIL_WT_MB 96
+#define YAFSDP_GATHER_TAIL_WT_MB 56
 #endif
-constexpr int kGatherTailWriteThroughMb = YAFSDP_GATHER_TAIL_WT_MB;  // default of YAFSDP_OPT_GATHER_TAIL_MB
+#ifndef YAFSDP_SCATTER_TAIL_WT_MB
+#define YAFSDP_SCATTER_TAIL_WT_MB 32
+#endif
+constexpr int kGatherTailWriteThroughMb = YAFSDP_GATHER_TAIL_WT_MB;    // default of YAFSDP_OPT_GATHER_TAIL_MB
+constexpr int kScatterTailWriteThroughMb = YAFSDP_SCATTER_TAIL_WT_MB;  // default of YAFSDP_OPT_SCATTER_TAIL_MB
 constexpr int kGatherStorePolicy = YAFSDP_GATHER_STP;
 constexpr int kScatterStorePolicy = YAFSDP_SCATTER_STP;
 inline int table_block_for(long long padded_elems, int threshold_log2) {
