@@ -1324,6 +1324,8 @@ def main() -> int:
     ap.add_argument("--no-store-policy-ab", action="store_true",
                     help="skip the leg that runs the step with the write-through tails of copy-out and reduce copy-in "
                          "switched off")
+    ap.add_argument("--no-rotating-sets", action="store_true",
+                    help="skip the leg that alternates the step between two sets of buffers")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the step from a HIP graph (outside the timed region)")
     ap.add_argument("--no-torch-gpu", action="store_true",
@@ -1357,6 +1359,10 @@ def main() -> int:
     ap.add_argument("--scatter-tail-mb", type=int, default=None, metavar="N",
                     help="the same for the last megabytes of tensors that copy-out writes (default: the library's "
                          "own, 32; 0 = none)")
+    ap.add_argument("--flat-tail-mb", type=int, default=None, metavar="N",
+                    help="the same for the flat kernels (copy-in, post-reduce), which write through everywhere by "
+                         "default; 0 = they store everything non-temporal")
+    ap.add_argument("--post-reduce-tail-mb", type=int, default=None, metavar="N", help="the same for the post-reduce")
     ap.add_argument("--analyze-trace", metavar="CSV", default=None,
                     help="llama3-8b-full-w8 only: no GPU work; summarise the kernel-trace CSV that rocprofv3 wrote for "
                          "`--workload llama3-8b-full-w8 --steps 10 --no-parity` (GEMM resource columns, concurrency)")
@@ -1374,6 +1380,14 @@ def main() -> int:
     if not torch.cuda.is_available():
         log("bench.py: no GPU visible; the buffer path has no CPU implementation to measure.")
         return 3
+    from yafsdp_amd import _native
+
+    for value, option in ((args.gather_tail_mb, _native.OPT_GATHER_TAIL_MB),
+                          (args.scatter_tail_mb, _native.OPT_SCATTER_TAIL_MB),
+                          (args.flat_tail_mb, _native.OPT_FLAT_TAIL_MB),
+                          (args.post_reduce_tail_mb, _native.OPT_POST_REDUCE_TAIL_MB)):
+        if value is not None:  # the library's store-policy options, for every workload
+            _native.set_option(option, value)
     if args.workload == "llama3-8b-full-w8":
         return run_full_model(args)
     if args.workload.endswith("-optim"):
@@ -1439,10 +1453,6 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     torch.cuda.set_device(dev)
     if args.table_large_log2 is not None:
         _native.set_option(_native.OPT_TABLE_LARGE_LOG2, args.table_large_log2)
-    if args.gather_tail_mb is not None:
-        _native.set_option(_native.OPT_GATHER_TAIL_MB, args.gather_tail_mb)
-    if args.scatter_tail_mb is not None:
-        _native.set_option(_native.OPT_SCATTER_TAIL_MB, args.scatter_tail_mb)
     # master / compute / reduce dtypes of the group: fp32 masters with bf16 compute and reduce, except the stress
     # test's second group (bf16 masters: no copy-in cast, fp32 reduce buffer, bf16 gradient shard)
     master_dt, rs_dt = torch.float32, torch.bfloat16
@@ -1693,6 +1703,75 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                     "unit": "GB/s", "default_scatter_tail_mb": scatter_tail_mb, "default_gather_tail_mb": tail_mb}
         log(f"without the write-through tails: {tail_off['ms_per_step']} ms per step, {tail_off['value']} GB/s "
             f"(default: last {scatter_tail_mb} MB of copy-out and last {tail_mb} MB of reduce copy-in write through)")
+
+    # ---- the same step alternating between TWO sets of buffers (outside the timed region), as the reference's
+    # parameter groups alternate between two shared gathered buffers and two shared reduce buffers
+    # (ya_fsdp/_state.py:636-652).  The timed region above rewrites ONE set step after step, so whatever its kernels
+    # leave in the 256-MB memory-side cache (written-through lines above all) is still there when the next step
+    # reads or overwrites the same addresses; with two sets 2.2 GB of other traffic lie between two visits.
+    rotating = None
+    if not args.no_rotating_sets:
+        try:
+            second = {
+                "master": d_master.clone(), "ag_in": torch.empty_like(d_ag_in), "gathered": d_gathered.clone(),
+                "outs": [torch.empty_like(x) for x in d_outs], "grads": [x.clone() for x in d_grads],
+                "rs": torch.zeros_like(d_rs), "shard": d_shard.clone(),
+            }
+            chunk2 = second["rs"][r * s : (r + 1) * s]
+
+            def step_second():
+                if fused and w == 1:
+                    ok = table.copy_in_scatter_out(second["gathered"], second["outs"], second["ag_in"], second["master"])
+                    ok = ok and table.gather_in_post_reduce(second["grads"], second["rs"], second["shard"], True)
+                    if not ok:
+                        raise RuntimeError("shared launch declined")
+                    return
+                if fused:
+                    if not table.copy_in_scatter_out(second["gathered"], second["outs"], second["ag_in"],
+                                                     second["master"]):
+                        raise RuntimeError("copy_in_scatter_out declined")
+                else:
+                    if has_copy_in:
+                        _native.flat_copy(second["ag_in"], second["master"])
+                    table.scatter_out(second["gathered"], second["outs"])
+                table.gather_in(second["grads"], second["rs"], None, pre, True)
+                _native.post_reduce(second["shard"], chunk2, None, True)
+
+            def alternating_ms_per_step(n_pairs):
+                for _ in range(max(1, warmup // 2)):
+                    step()
+                    step_second()
+                torch.cuda.synchronize()
+                q0 = time.perf_counter()
+                for _ in range(n_pairs):
+                    step()
+                    step_second()
+                torch.cuda.synchronize()
+                return (time.perf_counter() - q0) / (2 * n_pairs) * 1e3
+
+            n_pairs = max(steps, 1000) // 2
+            rot_ms = alternating_ms_per_step(n_pairs)
+            tails = [_native.get_option(o) for o in (_native.OPT_SCATTER_TAIL_MB, _native.OPT_GATHER_TAIL_MB)]
+            try:
+                _native.set_option(_native.OPT_SCATTER_TAIL_MB, 0)
+                _native.set_option(_native.OPT_GATHER_TAIL_MB, 0)
+                rot_plain_ms = alternating_ms_per_step(n_pairs)
+            finally:
+                _native.set_option(_native.OPT_SCATTER_TAIL_MB, tails[0])
+                _native.set_option(_native.OPT_GATHER_TAIL_MB, tails[1])
+            for _ in range(max(1, warmup)):  # the legs below start from the single set's steady state
+                step()
+            torch.cuda.synchronize()
+            rotating = {"sets": 2, "steps": 2 * n_pairs, "ms_per_step": round(rot_ms, 4),
+                        "value": round(bytes_per_step / rot_ms / 1e6, 1), "unit": "GB/s",
+                        "frac_of_hbm_peak": round(bytes_per_step / rot_ms / 1e6 / HBM_PEAK_GBS, 4),
+                        "without_write_through_tails_ms_per_step": round(rot_plain_ms, 4)}
+            log(f"two buffer sets in rotation: {rotating['ms_per_step']} ms per step, {rotating['value']} GB/s "
+                f"({rotating['without_write_through_tails_ms_per_step']} ms with the write-through tails off)")
+            del second, chunk2
+        except Exception as exc:  # an optional leg must not cost the measurement above
+            log(f"rotating-sets leg skipped: {type(exc).__name__}: {exc}")
+            rotating = None
 
     # ---- the same launches on the streams the reference puts them on (outside the timed region): copy-in and
     # copy-out on the side stream that serves all-gather and reduce-scatter (ya_fsdp/_collectives.py:46,
@@ -2008,6 +2087,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         "sustained": sustained,
         "reference_stream_placement": reference_streams,
         "without_write_through_tails": tail_off,
+        "two_buffer_sets_in_rotation": rotating,
         "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
         "kernels": kernels,
         "kernel_variants": variants,

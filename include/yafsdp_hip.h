@@ -395,11 +395,16 @@ typedef enum yafsdp_option {
                                          later: the kernel ends sooner, and whatever runs next pays for the
                                          write-back only if it saturates the memory itself from its first
                                          microsecond.  0 = off */
-  YAFSDP_OPT_SCATTER_TAIL_MB = 5      /* 0..2^20, default 32: the same for the tile slots of the last `value`
+  YAFSDP_OPT_SCATTER_TAIL_MB = 5,     /* 0..2^20, default 32: the same for the tile slots of the last `value`
                                          megabytes of tensors in yafsdp_scatter_out / yafsdp_scatter_out_bound /
                                          yafsdp_copy_in_scatter_out.  Consecutive kernels share one budget of
                                          write-through data in flight (about 100 MB on MI355X, the flat kernels'
                                          stores included): raise one option and lower the other */
+  YAFSDP_OPT_FLAT_TAIL_MB = 6,        /* 0..2^20, default 2^20 (everything): the same for yafsdp_flat_copy,
+                                         yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
+                                         yafsdp_copy_in_scatter_out, which write through everywhere by default;
+                                         0 = they store everything non-temporal */
+  YAFSDP_OPT_POST_REDUCE_TAIL_MB = 7  /* the same for yafsdp_post_reduce / yafsdp_post_reduce_fragments */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);

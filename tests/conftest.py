@@ -21,3 +21,14 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _library_default_store_policy(request):
+    """fully_shard picks the library's store policy from the number of parameter groups (process-wide options): every
+    GPU test starts from the library's own defaults, whatever model the test before it built."""
+    if "gpu" in request.keywords:
+        from yafsdp_amd import _native
+
+        _native.set_store_policy("single_set")
+    yield

@@ -27,7 +27,7 @@ def test_library_exports_every_symbol():
 
     for name in _declared_functions():
         assert hasattr(_native.lib, name), name
-    assert _native.lib.yafsdp_version() == 1003  # 1.1: yafsdp_flat_copy_bytes; 1.2, 1.3: the two write-through tail options
+    assert _native.lib.yafsdp_version() == 1005  # 1.1: yafsdp_flat_copy_bytes; 1.2-1.5: the four write-through tail options
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
 
@@ -62,7 +62,13 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 32
     assert L.yafsdp_set_option(5, 7) == 0 and L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 7
     assert L.yafsdp_set_option(5, 32) == 0
-    assert L.yafsdp_set_option(6, 1) == -1
+    assert L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 1 << 20
+    assert L.yafsdp_set_option(6, 0) == 0 and L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 0
+    assert L.yafsdp_set_option(6, 1 << 20) == 0
+    assert L.yafsdp_get_option(7, ctypes.byref(tail)) == 0 and tail.value == 1 << 20
+    assert L.yafsdp_set_option(7, 5) == 0 and L.yafsdp_get_option(7, ctypes.byref(tail)) == 0 and tail.value == 5
+    assert L.yafsdp_set_option(7, 1 << 20) == 0
+    assert L.yafsdp_set_option(8, 1) == -1
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
     # operands that overlap without being the same buffer are refused (addresses are never dereferenced here)
@@ -96,3 +102,23 @@ def test_no_product_module_imports_the_oracle():
                 src = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", src, flags=re.M), f
                 assert "libbufpath_ref" not in src, f
+
+
+def test_store_policies_set_the_four_tail_options():
+    import pytest
+
+    from yafsdp_amd import _native
+
+    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"] == (1 << 20, 1 << 20, 32, 56)
+    try:
+        _native.set_store_policy("rotating_sets")
+        assert _native.get_store_policy() == (0, 0, 0, 128)
+        assert _native.get_option(_native.OPT_GATHER_TAIL_MB) == 128
+        _native.set_store_policy((5, 6, 7, 8))
+        assert _native.get_store_policy() == (5, 6, 7, 8)
+        with pytest.raises(KeyError):
+            _native.set_store_policy("no_such_policy")
+        with pytest.raises(ValueError):
+            _native.set_store_policy((1, 2, 3))
+    finally:
+        _native.set_store_policy("single_set")

@@ -647,3 +647,27 @@ def test_torch_adamw_and_clip_grad_norm_on_the_sharded_parameters(impl):
         for q, t in zip(twin_model.parameters(), twins):
             q.copy_(t.view(q.shape))
     assert torch.equal(y, twin_model.to(torch.bfloat16)(xs[0].to(torch.bfloat16)))
+
+
+def test_store_policy_follows_the_number_of_parameter_groups(monkeypatch):
+    """Which stores write through is a process-wide choice of the library; fully_shard makes it when the root is
+    initialised: several groups take turns on the shared buffers (little of what one writes is still cached when its
+    buffer comes round again), a single group rewrites its own.  Either way the same bits (every other test)."""
+    from yafsdp_amd import _native, fully_shard
+
+    x = torch.randn(4, 128, device=DEV)
+    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"]  # the library's defaults
+    model = _wrap(_make(61), mp_policy=MP)  # four groups
+    model(x).float().pow(2).mean().backward()
+    assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"]
+    single = fully_shard(Block(128, 256).to(DEV), mp_policy=MP)  # one group
+    single(x).float().pow(2).mean().backward()
+    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"]
+    # the environment can fix the policy or leave the options alone
+    monkeypatch.setenv("YAFSDP_STORE_POLICY", "keep")
+    _native.set_store_policy((1, 2, 3, 4))
+    _wrap(_make(62), mp_policy=MP)(x).float().pow(2).mean().backward()
+    assert _native.get_store_policy() == (1, 2, 3, 4)
+    monkeypatch.setenv("YAFSDP_STORE_POLICY", "rotating_sets")
+    fully_shard(Block(128, 256).to(DEV), mp_policy=MP)(x).float().pow(2).mean().backward()
+    assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"]

@@ -120,16 +120,19 @@ def test_copy_out_with_the_write_through_boundary_inside_the_tensors(nat, tail_m
     are; the default is larger than all tensors of the other tests together, so there all are), in the shared launch
     and in scatter-out as a launch of its own.  Same bytes either way."""
     default_tail = nat.get_option(nat.OPT_SCATTER_TAIL_MB)
+    default_flat_tail = nat.get_option(nat.OPT_FLAT_TAIL_MB)
     default_log2 = nat.get_option(nat.OPT_TABLE_LARGE_LOG2)
     nat.set_option(nat.OPT_SCATTER_TAIL_MB, tail_mb)
+    nat.set_option(nat.OPT_FLAT_TAIL_MB, tail_mb)  # the cast part of the shared launch: the same kind of boundary
     if two_waves:
         nat.set_option(nat.OPT_TABLE_LARGE_LOG2, 0)
     try:
-        for case in [(7, 19, False, 513, False), (9, 17, False, 64, True), (33, 14, True, 9, False),
-                     (5, 21, False, 0, True)]:
-            test_copy_in_scatter_out(nat, case, master_dt, param_dt, 4099)
+        for case, shard_n in [((7, 19, False, 513, False), 1_300_001), ((9, 17, False, 64, True), 4099),
+                              ((33, 14, True, 9, False), 4099), ((5, 21, False, 0, True), 2_000_003)]:
+            test_copy_in_scatter_out(nat, case, master_dt, param_dt, shard_n)
     finally:
         nat.set_option(nat.OPT_SCATTER_TAIL_MB, default_tail)
+        nat.set_option(nat.OPT_FLAT_TAIL_MB, default_flat_tail)
         nat.set_option(nat.OPT_TABLE_LARGE_LOG2, default_log2)
 
 

@@ -140,6 +140,45 @@ def test_post_reduce(nat, shard_dt, chunk_dt, post, acc):
         assert_bits_equal(got, want, "post_reduce")
 
 
+@pytest.mark.parametrize("tail_mb", [0, 1, 3])
+def test_flat_kernels_with_the_write_through_boundary_inside_the_buffer(nat, tail_mb):
+    """The flat kernels write through everywhere by default; with a tail option below the size of the output the
+    tiles before the last megabytes store non-temporal instead (0: all of them).  Same bytes either way."""
+    g = torch.Generator().manual_seed(131)
+    n = 1_500_003  # 3 MB of bf16, 6 MB of fp32
+    defaults = (nat.get_option(nat.OPT_FLAT_TAIL_MB), nat.get_option(nat.OPT_POST_REDUCE_TAIL_MB))
+    nat.set_option(nat.OPT_FLAT_TAIL_MB, tail_mb)
+    nat.set_option(nat.OPT_POST_REDUCE_TAIL_MB, tail_mb)
+    try:
+        for src_dt, dst_dt in [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32),
+                               (torch.bfloat16, torch.bfloat16)]:
+            _say("flat_copy with tail", tail_mb, src_dt, dst_dt)
+            src = mixed_values(g, n + 1, src_dt)
+            want = torch.full((n + 11,), 3.0, dtype=dst_dt)
+            torch_ops.copy_in(want[3 : 3 + n], src[1:])
+            got = torch.full((n + 11,), 3.0, dtype=dst_dt, device=DEV)
+            nat.flat_copy(got[3 : 3 + n], src.to(DEV)[1:])
+            assert_bits_equal(got, want, "flat_copy")
+        buf = mixed_values(g, n, torch.bfloat16)
+        want = buf.clone()
+        torch_ops.div_if_needed(want, 8.0)
+        got = buf.to(DEV)
+        nat.flat_div(got, 8.0)
+        assert_bits_equal(got, want, "flat_div")
+        for acc in (False, True):
+            _say("post_reduce with tail", tail_mb, acc)
+            chunk = mixed_values(g, n, torch.bfloat16, std=1e-3)
+            shard0 = mixed_values(g, n, torch.float32, std=1e-4)
+            want = shard0.clone()
+            torch_ops.reduce_scatter_local(want, chunk.clone(), 1, 0, None, 8.0, "add" if acc else "copy")
+            got = shard0.to(DEV)
+            nat.post_reduce(got, chunk.to(DEV), 8.0, acc)
+            assert_bits_equal(got, want, "post_reduce")
+    finally:
+        nat.set_option(nat.OPT_FLAT_TAIL_MB, defaults[0])
+        nat.set_option(nat.OPT_POST_REDUCE_TAIL_MB, defaults[1])
+
+
 @pytest.mark.parametrize("shard_dt,chunk_dt", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32)])
 @pytest.mark.parametrize("post", [None, 8.0])
 def test_post_reduce_fragments(nat, shard_dt, chunk_dt, post):

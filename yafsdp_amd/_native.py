@@ -33,7 +33,7 @@ except ImportError:  # not built: the Python checks below do the same work, slow
 DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
 MODE_SKIP, MODE_COPY, MODE_ADD = 0, 1, 2
 OPT_FLAT_BLOCKS_PER_CU, OPT_TABLE_BLOCKS_PER_CU, OPT_TABLE_LARGE_LOG2, OPT_SCATTER_TILE = 0, 1, 2, 3
-OPT_GATHER_TAIL_MB, OPT_SCATTER_TAIL_MB = 4, 5
+OPT_GATHER_TAIL_MB, OPT_SCATTER_TAIL_MB, OPT_FLAT_TAIL_MB, OPT_POST_REDUCE_TAIL_MB = 4, 5, 6, 7
 
 # every symbol include/yafsdp_hip.h declares
 EXPORTED_SYMBOLS = (
@@ -878,3 +878,32 @@ def get_option(option: int) -> int:
     v = ctypes.c_int()
     _check(lib.yafsdp_get_option(int(option), ctypes.byref(v)), "yafsdp_get_option")
     return v.value
+
+
+# Store policies: how many megabytes at the END of each kind of kernel's output are stored write-through (the rest
+# non-temporal), as (flat copies / casts / divides, post-reduce, scatter-out, gather-in).  Written-through lines
+# stay in the 256-MB memory-side cache until later traffic evicts them, so the right amount depends on when the
+# written buffers are touched again:
+#   "single_set"     one set of buffers rewritten step after step (one parameter group; a loop over one layer): the
+#                    flat kernels write through everywhere and the two table kernels their last 32 / 56 MB; the next
+#                    step finds much of it still cached.  The library's own defaults.
+#   "rotating_sets"  several parameter groups taking turns on shared buffers (ya_fsdp/_state.py:636-652), gigabytes
+#                    of other traffic between two visits: write-through data only defers its write-back, which
+#                    pays up to about 128 MB per step (half of the cache) and costs beyond; the reduce copy-in takes
+#                    that budget whatever the shard size, everything else stores non-temporal.
+_EVERYTHING = 1 << 20
+STORE_POLICIES = {"single_set": (_EVERYTHING, _EVERYTHING, 32, 56), "rotating_sets": (0, 0, 0, 128)}
+_STORE_POLICY_OPTIONS = (OPT_FLAT_TAIL_MB, OPT_POST_REDUCE_TAIL_MB, OPT_SCATTER_TAIL_MB, OPT_GATHER_TAIL_MB)
+
+
+def set_store_policy(policy: "str | tuple[int, int, int, int]") -> None:
+    """Process-wide, like the options it sets; takes effect with the next launch."""
+    values = STORE_POLICIES[policy] if isinstance(policy, str) else tuple(policy)
+    if len(values) != len(_STORE_POLICY_OPTIONS):
+        raise ValueError(f"a store policy has {len(_STORE_POLICY_OPTIONS)} entries, got {values}")
+    for option, value in zip(_STORE_POLICY_OPTIONS, values):
+        set_option(option, value)
+
+
+def get_store_policy() -> "tuple[int, int, int, int]":
+    return tuple(get_option(option) for option in _STORE_POLICY_OPTIONS)

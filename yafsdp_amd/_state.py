@@ -7,6 +7,7 @@ from __future__ import annotations
 
 import functools
 import logging
+import os
 from typing import Any
 
 import torch
@@ -16,6 +17,7 @@ from torch.distributed._composable_state import _get_module_state, _insert_modul
 from torch.distributed.utils import _apply_to_tensors, _to_kwargs
 from torch.utils._pytree import tree_flatten
 
+from . import _native
 from ._api import MixedPrecisionPolicy
 from ._common import TrainingState, profiler_range
 from ._param_group import YaFSDPCommContext, YaFSDPParamGroup
@@ -191,6 +193,13 @@ class YaFSDPState(_State):
         param_groups = [s._fsdp_param_group for s in self._state_ctx.all_states if s._fsdp_param_group is not None]
         if not param_groups:
             return
+        # which stores write through depends on how soon the written buffers come round again, and this is where
+        # that is known: several groups take turns on the shared buffers, a single group rewrites its own
+        policy = os.environ.get("YAFSDP_STORE_POLICY", "auto")
+        if policy == "auto":
+            policy = "rotating_sets" if len(param_groups) > 1 else "single_set"
+        if policy != "keep":
+            _native.set_store_policy(policy)
         no_reshard_after_forward = all(not g.reshard_after_forward for g in param_groups)
 
         def assign(groups, attr, count, size_of, ctx_idx=None, idx_to_handle=None):

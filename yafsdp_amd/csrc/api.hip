@@ -28,6 +28,8 @@ std::atomic<int> g_table_blocks_per_cu{kTableBlocksPerCu};
 std::atomic<int> g_table_large_log2{kTableLargeThresholdLog2};
 std::atomic<int> g_gather_tail_mb{kGatherTailWriteThroughMb};
 std::atomic<int> g_scatter_tail_mb{kScatterTailWriteThroughMb};
+std::atomic<int> g_flat_tail_mb{kFlatTailWriteThroughMb};
+std::atomic<int> g_post_reduce_tail_mb{kPostReduceTailWriteThroughMb};
 std::atomic<int> g_scatter_tile_mode{0};
 
 constexpr int kMaxDevices = 64;
@@ -116,8 +118,17 @@ int64_t table_blocks(int64_t n_tiles) {
   return (n_tiles + win - 1) / win * win;
 }
 
+// first tile of a flat pass that writes through: the last tail_mb megabytes of its output (tile_units: 8-element
+// units per tile; tail_mb: YAFSDP_OPT_FLAT_TAIL_MB, or YAFSDP_OPT_POST_REDUCE_TAIL_MB for the post-reduce)
+int flat_wt_from(int64_t n_tiles, int64_t tile_units, int dst_dt, const std::atomic<int>& tail_mb) {
+  const int64_t tile_bytes = tile_units * 8 * item_size(dst_dt);
+  const int64_t tail = (int64_t(tail_mb.load(std::memory_order_relaxed)) << 20) / tile_bytes;
+  const int64_t from = tail >= n_tiles ? 0 : n_tiles - tail;
+  return from > INT32_MAX ? INT32_MAX : int(from);
+}
+
 int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, float k,
-                hipStream_t stream) {
+                hipStream_t stream, const std::atomic<int>& tail_mb = g_flat_tail_mb) {
   if (n == 0) return YAFSDP_OK;
   if (!aligned_to(dst, item_size(dst_dt)) || !aligned_to(src, item_size(src_dt))) return YAFSDP_ERR_MISALIGNED;
   {
@@ -140,7 +151,9 @@ int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const vo
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return int(e);
   const int grid = grid_for(n_tiles, g_flat_blocks_per_cu.load(std::memory_order_relaxed), device);
-  e = launch_flat(src_dt, dst_dt, scale, acc, dst, src, n, int(head), k, grid, stream);
+  e = launch_flat(src_dt, dst_dt, scale, acc, dst, src, n, int(head), k, flat_wt_from(n_tiles, tile, dst_dt, tail_mb),
+                  grid,
+                  stream);
   return int(e);
 }
 
@@ -316,7 +329,7 @@ int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
 
 extern "C" {
 
-int yafsdp_version(void) { return 1003; }
+int yafsdp_version(void) { return 1005; }
 
 const char* yafsdp_error_string(int code) {
   switch (code) {
@@ -471,9 +484,12 @@ int yafsdp_set_option(int option, int value) {
     g_table_large_log2.store(value);
     return YAFSDP_OK;
   }
-  if (option == YAFSDP_OPT_GATHER_TAIL_MB || option == YAFSDP_OPT_SCATTER_TAIL_MB) {
+  if (option == YAFSDP_OPT_GATHER_TAIL_MB || option == YAFSDP_OPT_SCATTER_TAIL_MB ||
+      option == YAFSDP_OPT_FLAT_TAIL_MB || option == YAFSDP_OPT_POST_REDUCE_TAIL_MB) {
     if (value < 0 || value > (1 << 20)) return YAFSDP_ERR_INVALID_ARGUMENT;
-    (option == YAFSDP_OPT_GATHER_TAIL_MB ? g_gather_tail_mb : g_scatter_tail_mb).store(value);
+    (option == YAFSDP_OPT_GATHER_TAIL_MB ? g_gather_tail_mb
+     : option == YAFSDP_OPT_SCATTER_TAIL_MB ? g_scatter_tail_mb
+     : option == YAFSDP_OPT_FLAT_TAIL_MB ? g_flat_tail_mb : g_post_reduce_tail_mb).store(value);
     return YAFSDP_OK;
   }
   if (option == YAFSDP_OPT_SCATTER_TILE) {
@@ -498,6 +514,8 @@ int yafsdp_get_option(int option, int* value) {
     case YAFSDP_OPT_SCATTER_TILE: *value = g_scatter_tile_mode.load(); return YAFSDP_OK;
     case YAFSDP_OPT_GATHER_TAIL_MB: *value = g_gather_tail_mb.load(); return YAFSDP_OK;
     case YAFSDP_OPT_SCATTER_TAIL_MB: *value = g_scatter_tail_mb.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_FLAT_TAIL_MB: *value = g_flat_tail_mb.load(); return YAFSDP_OK;
+    case YAFSDP_OPT_POST_REDUCE_TAIL_MB: *value = g_post_reduce_tail_mb.load(); return YAFSDP_OK;
   }
   return YAFSDP_ERR_INVALID_ARGUMENT;
 }
@@ -790,7 +808,7 @@ int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chun
     if (scale == SCALE_NONE) return YAFSDP_OK;
   }
   return flat_launch(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, chunk, n, k,
-                     static_cast<hipStream_t>(stream));
+                     static_cast<hipStream_t>(stream), g_post_reduce_tail_mb);
 }
 
 int64_t yafsdp_post_reduce_sumsq_count(int64_t n) {
@@ -857,7 +875,7 @@ int yafsdp_post_reduce_fragments(void* shard, int shard_dtype, const void* chunk
       char* d = static_cast<char*>(shard) + pos * item_size(shard_dtype);
       const char* s = static_cast<const char*>(chunk) + pos * item_size(chunk_dtype);
       int rc = flat_launch(chunk_dtype, shard_dtype, scale, m == MODE_ADD, d, s, run, k,
-                           static_cast<hipStream_t>(stream));
+                           static_cast<hipStream_t>(stream), g_post_reduce_tail_mb);
       if (rc != YAFSDP_OK) return rc;
     }
     pos += run;
@@ -1054,12 +1072,14 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   if (grid > int64_t(INT32_MAX) - 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int wt_from = scatter_wt_from(table, flat_dtype);  // the tensors have the gathered buffer's dtype here
+  const int cast_wt_from = flat_wt_from(n_flat_blocks, flat_tile, flat_dtype, g_flat_tail_mb);  // one tile per workgroup of the cast
   if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     static const void* const kNoPtrs[kSmallMax] = {};
     fill_small(table, table->total > 0 ? ptrs : kNoPtrs, mode, &meta);
     return int(launch_unshard<SmallMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots),
-                                         wt_from, ag_in, master, n, int(head), int(n_flat_blocks), int(grid), s));
+                                         wt_from, ag_in, master, n, int(head), int(n_flat_blocks), cast_wt_from,
+                                         int(grid), s));
   }
   if (table->total == 0)  // nothing to split: the cast alone
     return flat_launch(master_dtype, flat_dtype, SCALE_NONE, false, ag_in, master, n, 1.0f, s);
@@ -1069,7 +1089,7 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   const int rc = stage_large(table, ptrs, mode, &meta, &slot, s);
   if (rc != YAFSDP_OK) return rc;
   e = launch_unshard<LargeMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots), wt_from, ag_in,
-                                master, n, int(head), int(n_flat_blocks), int(grid), s);
+                                master, n, int(head), int(n_flat_blocks), cast_wt_from, int(grid), s);
   if (e != hipSuccess) return int(e);
   return finish_large(table, slot, s);
 }

@@ -100,10 +100,11 @@ __device__ __forceinline__ void flat_full_tile(char* dst, const char* src, float
 // wall-clock count at its start and, after its stores have been acknowledged,
 // at its end into trace[2 b], trace[2 b + 1].
 // The flat pass as seen by workgroup `block` of `n_blocks` (the whole grid of flat_kernel, or the part of a
-// larger grid that serves this job).
+// larger grid that serves this job).  With STP = ST_WT the full tiles before tile `wt_from` store non-temporal
+// instead (0: every tile writes through).
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __device__ __forceinline__ void flat_body(void* dst, const void* src, int64_t n, int head, float k, int block,
-                                          int n_blocks) {
+                                          int n_blocks, int wt_from) {
   const int tid = threadIdx.x;
   const int64_t n_units = (n - head) >> 3;
   const int64_t body_end = head + (n_units << 3);
@@ -119,8 +120,12 @@ __device__ __forceinline__ void flat_body(void* dst, const void* src, int64_t n,
   const int64_t n_tiles = (n_units + kTile - 1) / kTile;
   for (int64_t tile = block; tile < n_tiles; tile += n_blocks) {
     if (tile * kTile + kTile <= n_units) {
-      flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dbase + tile * kTile * (8 * D::kSize),
-                                                           sbase + tile * kTile * (8 * S::kSize), k);
+      if (STP == ST_WT && tile < wt_from)  // before the write-through part of the output (see tuning.h)
+        flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, ST_NT>(dbase + tile * kTile * (8 * D::kSize),
+                                                               sbase + tile * kTile * (8 * S::kSize), k);
+      else
+        flat_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dbase + tile * kTile * (8 * D::kSize),
+                                                             sbase + tile * kTile * (8 * S::kSize), k);
     } else {  // last, partial tile
       for (int64_t u = tile * kTile + tid; u < n_units; u += BLOCK) {
         Unit<S> s = load_unit<S, NTL>(sbase + u * (8 * S::kSize));
@@ -134,11 +139,11 @@ __device__ __forceinline__ void flat_body(void* dst, const void* src, int64_t n,
 
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
-flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned long long* trace) {
+flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned long long* trace, int wt_from) {
   if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   unsigned long long t_start = 0;
   if (trace != nullptr) t_start = wall_clock64();
-  flat_body<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dst, src, n, head, k, int(blockIdx.x), int(gridDim.x));
+  flat_body<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dst, src, n, head, k, int(blockIdx.x), int(gridDim.x), wt_from);
   if (trace != nullptr) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every load has arrived, every store is acknowledged
     if (threadIdx.x == 0) {

@@ -9,32 +9,32 @@ namespace {
 // ---- copy-in + copy-out -----------------------------------------------------------------------------------------
 template <class META, class M, class P, int BLOCK, int US>
 hipError_t unshard_go(const META& meta, const void* gathered, int n_slots, int wt_from, void* ag_in, const void* master, int64_t n,
-                      int head, int n_flat_blocks, int grid, hipStream_t stream) {
+                      int head, int n_flat_blocks, int flat_wt_from, int grid, hipStream_t stream) {
   return launch_kernel(unshard_kernel<META, M, P, BLOCK, kFusedFlatUnroll, US, scatter_nt_load(US), kFlatStorePolicy,
                                       kScatterStorePolicy>,
-                       grid, BLOCK, stream, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks);
+                       grid, BLOCK, stream, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from);
 }
 
 // the three scatter-out shapes a table can have (scatter_shape_for)
 template <class META, class M, class P>
 hipError_t unshard_by_shape(int shape, const META& meta, const void* gathered, int n_slots, int wt_from, void* ag_in,
-                            const void* master, int64_t n, int head, int n_flat_blocks, int grid, hipStream_t stream) {
+                            const void* master, int64_t n, int head, int n_flat_blocks, int flat_wt_from, int grid, hipStream_t stream) {
   if (shape == kTableBlockSmall * 16 + kScatterShortUnroll)
-    return unshard_go<META, M, P, kTableBlockSmall, kScatterShortUnroll>(meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
+    return unshard_go<META, M, P, kTableBlockSmall, kScatterShortUnroll>(meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
   if (shape == kTableBlockSmall * 16 + kGatherUnroll)
-    return unshard_go<META, M, P, kTableBlockSmall, kGatherUnroll>(meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
+    return unshard_go<META, M, P, kTableBlockSmall, kGatherUnroll>(meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
   if (shape == kTableBlockLarge * 16 + kGatherUnroll)
-    return unshard_go<META, M, P, kTableBlockLarge, kGatherUnroll>(meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
+    return unshard_go<META, M, P, kTableBlockLarge, kGatherUnroll>(meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
   return hipErrorInvalidValue;
 }
 
 template <class META, class M>
 hipError_t unshard_by_param(int p_dt, int shape, const META& meta, const void* gathered, int n_slots, int wt_from, void* ag_in,
-                            const void* master, int64_t n, int head, int n_flat_blocks, int grid, hipStream_t stream) {
+                            const void* master, int64_t n, int head, int n_flat_blocks, int flat_wt_from, int grid, hipStream_t stream) {
   switch (p_dt) {
-    case DT_F32: return unshard_by_shape<META, M, F32>(shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
-    case DT_BF16: return unshard_by_shape<META, M, BF16>(shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
-    case DT_F16: return unshard_by_shape<META, M, F16>(shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
+    case DT_F32: return unshard_by_shape<META, M, F32>(shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
+    case DT_BF16: return unshard_by_shape<META, M, BF16>(shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
+    case DT_F16: return unshard_by_shape<META, M, F16>(shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -87,11 +87,11 @@ bool fused_reduce_supports(int tensor_dt, int flat_dt) { return flat_dt == tenso
 template <class META>
 hipError_t launch_unshard(int scatter_shape, int master_dt, int param_dt, const META& meta, const void* gathered,
                           int n_slots, int wt_from, void* ag_in, const void* master, int64_t n, int head, int n_flat_blocks,
-                          int grid, hipStream_t stream) {
+                          int flat_wt_from, int grid, hipStream_t stream) {
   switch (master_dt) {
-    case DT_F32: return unshard_by_param<META, F32>(param_dt, scatter_shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
-    case DT_BF16: return unshard_by_param<META, BF16>(param_dt, scatter_shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
-    case DT_F16: return unshard_by_param<META, F16>(param_dt, scatter_shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, grid, stream);
+    case DT_F32: return unshard_by_param<META, F32>(param_dt, scatter_shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
+    case DT_BF16: return unshard_by_param<META, BF16>(param_dt, scatter_shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
+    case DT_F16: return unshard_by_param<META, F16>(param_dt, scatter_shape, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from, grid, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -109,9 +109,9 @@ hipError_t launch_gather_post(int block, int tensor_dt, int flat_dt, int shard_d
 }
 
 template hipError_t launch_unshard<SmallMeta>(int, int, int, const SmallMeta&, const void*, int, int, void*, const void*,
-                                              int64_t, int, int, int, hipStream_t);
+                                              int64_t, int, int, int, int, hipStream_t);
 template hipError_t launch_unshard<LargeMeta>(int, int, int, const LargeMeta&, const void*, int, int, void*, const void*,
-                                              int64_t, int, int, int, hipStream_t);
+                                              int64_t, int, int, int, int, hipStream_t);
 template hipError_t launch_gather_post<SmallMeta>(int, int, int, int, const SmallMeta&, void*, void*, int64_t, int, int,
                                                   int, const ReduceDivides&, int, hipStream_t);
 template hipError_t launch_gather_post<LargeMeta>(int, int, int, int, const LargeMeta&, void*, void*, int64_t, int, int,

@@ -34,10 +34,11 @@ namespace yafsdp {
 template <class META, class M, class P, int BLOCK, int UF, int US, bool NTL, int STP_FLAT, int STP_SCATTER>
 __global__ void __launch_bounds__(BLOCK)
 unshard_kernel(META meta, const void* gathered, int n_slots, int wt_from, void* ag_in, const void* master, int64_t n,
-               int head, int n_flat_blocks) {
+               int head, int n_flat_blocks, int flat_wt_from) {
   const int b = blockIdx.x;
   if (b < n_flat_blocks) {
-    flat_body<M, P, SCALE_NONE, false, BLOCK, UF, kFlatNtLoad, STP_FLAT>(ag_in, master, n, head, 1.0f, b, n_flat_blocks);
+    flat_body<M, P, SCALE_NONE, false, BLOCK, UF, kFlatNtLoad, STP_FLAT>(ag_in, master, n, head, 1.0f, b, n_flat_blocks,
+                                                                       flat_wt_from);
   } else {
     scatter_body<META, P, P, BLOCK, US, NTL, STP_SCATTER>(meta, gathered, n_slots, wt_from, b - n_flat_blocks,
                                                               int(gridDim.x) - n_flat_blocks);

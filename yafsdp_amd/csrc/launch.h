@@ -37,8 +37,9 @@ inline hipError_t launch_kernel(void (*kernel)(Params...), int grid, int block, 
 }
 
 // dst[i] = post_elem(src[i], dst[i]); scale is SCALE_NONE / SCALE_MUL / SCALE_DIV
+// (full tiles before tile `wt_from` store non-temporal, the others write through)
 hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,
-                       float k, int grid, hipStream_t stream);
+                       float k, int wt_from, int grid, hipStream_t stream);
 // dst[0:n] = src[0:n], opaque bytes at any byte address; head: bytes up to dst's first 128-byte line (< workgroup size)
 hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int grid, hipStream_t stream);
 // the same pass, also writing partials[0:grid] = per-workgroup sums of squares of the stored values (postsumsq.hip);
@@ -66,7 +67,7 @@ constexpr int kFusedFlatUnroll = 2;
 template <class META>
 hipError_t launch_unshard(int scatter_shape, int master_dt, int param_dt, const META& meta, const void* gathered,
                           int n_slots, int wt_from, void* ag_in, const void* master, int64_t n, int head,
-                          int n_flat_blocks, int grid, hipStream_t stream);
+                          int n_flat_blocks, int flat_wt_from, int grid, hipStream_t stream);
 // reduce copy-in + post-reduce of a size-1 shard group; `block`: the table's gather-in workgroup size
 // The divides of the reduce step, applied by that kernel at run time (wave-uniform branches; a shard group of size
 // one has none unless the caller set a custom factor or reduces in fp16 with one):

@@ -118,6 +118,16 @@ constexpr bool scatter_nt_load(int unroll) {
 #endif
 constexpr int kGatherTailWriteThroughMb = YAFSDP_GATHER_TAIL_WT_MB;    // default of YAFSDP_OPT_GATHER_TAIL_MB
 constexpr int kScatterTailWriteThroughMb = YAFSDP_SCATTER_TAIL_WT_MB;  // default of YAFSDP_OPT_SCATTER_TAIL_MB
+// The flat kernels write through everywhere by default (the option counts megabytes at the end of their output
+// like the two above; 2^20 covers any buffer, 0 stores everything non-temporal).
+#ifndef YAFSDP_FLAT_TAIL_WT_MB
+#define YAFSDP_FLAT_TAIL_WT_MB (1 << 20)
+#endif
+constexpr int kFlatTailWriteThroughMb = YAFSDP_FLAT_TAIL_WT_MB;  // default of YAFSDP_OPT_FLAT_TAIL_MB
+#ifndef YAFSDP_POST_REDUCE_TAIL_WT_MB
+#define YAFSDP_POST_REDUCE_TAIL_WT_MB (1 << 20)
+#endif
+constexpr int kPostReduceTailWriteThroughMb = YAFSDP_POST_REDUCE_TAIL_WT_MB;  // of YAFSDP_OPT_POST_REDUCE_TAIL_MB
 constexpr int kGatherStorePolicy = YAFSDP_GATHER_STP;
 constexpr int kScatterStorePolicy = YAFSDP_SCATTER_STP;
 inline int table_block_for(long long padded_elems, int threshold_log2) {
