@@ -1389,6 +1389,9 @@ def main() -> int:
         if value is not None:  # the library's store-policy options, for every workload
             _native.set_option(option, value)
     if args.workload == "llama3-8b-full-w8":
+        if all(v is None for v in (args.gather_tail_mb, args.scatter_tail_mb, args.flat_tail_mb,
+                                   args.post_reduce_tail_mb)):
+            _native.set_store_policy("rotating_sets")  # 35 groups on shared buffers: what fully_shard selects
         return run_full_model(args)
     if args.workload.endswith("-optim"):
         return run_optim(args)
@@ -1413,7 +1416,12 @@ def main() -> int:
                 log(f"config {wl}: {out['configs'][wl]['value']} GB/s, {time.perf_counter() - t0:.1f}s wall")
             # the full-model pass next to GEMMs on a second stream (its own oracle check of an overlapped pass)
             t0 = time.perf_counter()
-            rec = run_full_model(args, as_record=True)
+            in_force = _native.get_store_policy()
+            _native.set_store_policy("rotating_sets")  # 35 groups on shared buffers: what fully_shard selects
+            try:
+                rec = run_full_model(args, as_record=True)
+            finally:
+                _native.set_store_policy(in_force)
             if not isinstance(rec, dict):
                 raise ParityError("llama3-8b-full-w8: the overlapped pass differs from the oracle")
             out["configs"]["llama3-8b-full-w8"] = rec
@@ -1749,25 +1757,32 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                 torch.cuda.synchronize()
                 return (time.perf_counter() - q0) / (2 * n_pairs) * 1e3
 
+            # under the store policy in force (the library's default unless options were given), under the policy
+            # that fully_shard selects for several parameter groups, and with every store non-temporal
             n_pairs = max(steps, 1000) // 2
+            in_force = _native.get_store_policy()
             rot_ms = alternating_ms_per_step(n_pairs)
-            tails = [_native.get_option(o) for o in (_native.OPT_SCATTER_TAIL_MB, _native.OPT_GATHER_TAIL_MB)]
             try:
-                _native.set_option(_native.OPT_SCATTER_TAIL_MB, 0)
-                _native.set_option(_native.OPT_GATHER_TAIL_MB, 0)
+                _native.set_store_policy("rotating_sets")
+                rot_policy_ms = alternating_ms_per_step(n_pairs)
+                _native.set_store_policy((0, 0, 0, 0))
                 rot_plain_ms = alternating_ms_per_step(n_pairs)
             finally:
-                _native.set_option(_native.OPT_SCATTER_TAIL_MB, tails[0])
-                _native.set_option(_native.OPT_GATHER_TAIL_MB, tails[1])
+                _native.set_store_policy(in_force)
             for _ in range(max(1, warmup)):  # the legs below start from the single set's steady state
                 step()
             torch.cuda.synchronize()
-            rotating = {"sets": 2, "steps": 2 * n_pairs, "ms_per_step": round(rot_ms, 4),
-                        "value": round(bytes_per_step / rot_ms / 1e6, 1), "unit": "GB/s",
-                        "frac_of_hbm_peak": round(bytes_per_step / rot_ms / 1e6 / HBM_PEAK_GBS, 4),
-                        "without_write_through_tails_ms_per_step": round(rot_plain_ms, 4)}
-            log(f"two buffer sets in rotation: {rotating['ms_per_step']} ms per step, {rotating['value']} GB/s "
-                f"({rotating['without_write_through_tails_ms_per_step']} ms with the write-through tails off)")
+
+            def rate(ms):
+                return {"ms_per_step": round(ms, 4), "value": round(bytes_per_step / ms / 1e6, 1), "unit": "GB/s",
+                        "frac_of_hbm_peak": round(bytes_per_step / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+            rotating = {"sets": 2, "steps": 2 * n_pairs, "store_policy_in_force": list(in_force), **rate(rot_ms),
+                        "store_policy_rotating_sets": rate(rot_policy_ms),
+                        "all_stores_non_temporal": rate(rot_plain_ms)}
+            log(f"two buffer sets in rotation: {rotating['ms_per_step']} ms per step, {rotating['value']} GB/s; "
+                f"under the rotating-sets store policy {rot_policy_ms:.4f} ms, all stores non-temporal "
+                f"{rot_plain_ms:.4f} ms")
             del second, chunk2
         except Exception as exc:  # an optional leg must not cost the measurement above
             log(f"rotating-sets leg skipped: {type(exc).__name__}: {exc}")
@@ -2067,8 +2082,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                    "copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
                    "post-reduce chunk += gradient shard (master dtype) [S]",
             "launches_per_step": [n for n, _, _ in ops],
-            "copy_out_write_through_tail_mb": _native.get_option(_native.OPT_SCATTER_TAIL_MB),
-            "reduce_copy_in_write_through_tail_mb": _native.get_option(_native.OPT_GATHER_TAIL_MB),
+            "store_policy_mb_flat_postreduce_scatter_gather": list(_native.get_store_policy()),
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
         "parity": parity,

@@ -95,21 +95,27 @@ constexpr bool scatter_nt_load(int unroll) {
 #ifndef YAFSDP_SCATTER_STP
 #define YAFSDP_SCATTER_STP YAFSDP_TABLE_STP
 #endif
-// The table kernels store non-temporal: the L2s keep the written lines and evict them as they fill.  The tiles at
-// the END of a launch's output write through instead (as the flat kernels do everywhere): the last megabytes of the
-// flat buffer in gather-in, the tile slots of the last megabytes of tensors in scatter-out.  Two things follow.  The
-// kernel ends with clean L2s: its closing write-back finds no dirty line (40 thousand otherwise).  And the memory-side
-// cache takes the written-through lines faster than DRAM takes evicted ones, as long as it has room for them, and
-// writes them back when later traffic evicts them, partly in time that the memory would otherwise spend idle between
-// two kernels (drain of one, ramp of the next).  The gain is linear in the tail up to a budget that consecutive kernels share:
-// about 100 MB of write-through data in flight; beyond it the kernels that follow pay more than was gained.
-// Llama-3-8B layer (copy-in + copy-out, reduce copy-in, post-reduce; ms per step), scatter tail / gather tail in MB:
-// 0 / 0 0.3274; 0 / 48 0.3249; 0 / 64 0.3239; 0 / 96 0.3226; 0 / 128 0.3334; 32 / 0 0.3232; 24 / 56 0.3205;
-// 32 / 48 0.3205; 32 / 56 0.3200; 32 / 64 0.3200; 32 / 72 0.3216; 32 / 96 0.3295; 40 / 56 0.3202; 40 / 64 0.3218.
-// 70B layer: 0 / 0 1.0827; 0 / 96 1.0775; 32 / 56 1.0685.  Back to back with a kernel that saturates the memory from
-// its first microsecond the deferred write-back is not free: the two ragged groups at a shard group of 256 (4-us
-// post-reduce, so the next copy-out follows the reduce copy-in at once) 0 / 0 0.4741 and 0.2716; 32 / 0 0.4741 and
-// 0.2728; 32 / 56 0.4765 and 0.2765; 0 / 96 0.4776 and 0.2770.
+// Store policy.  A kernel stores non-temporal (the L2s keep the written lines and evict them as they fill) or
+// write-through (the lines go to the memory side as they are produced and stay in
+// its 256-MB cache until later traffic evicts them).  Which megabytes of a kernel's output write through is a
+// run-time choice per kind of kernel: always the END of the output (the last tiles of the flat buffer in gather-in,
+// the tile slots of the last tensors in scatter-out, the last tiles of a flat pass), because a kernel whose last
+// stores wrote through ends with clean L2s (its closing write-back finds no dirty line, 40 thousand otherwise).
+// What write-through data is worth depends on when the written buffers are touched again:
+//  * One set of buffers rewritten step after step (a loop over one layer; a model with one parameter group): the next
+//    step finds much of what wrote through still cached, reads it from there or overwrites it before it ever reached
+//    DRAM.  Llama-3-8B layer, ms per step, megabytes of (flat kernels, post-reduce, scatter-out tail, gather-in
+//    tail): (all, all, 0, 0) 0.3272; (all, all, 0, 96) 0.3226; (all, all, 32, 56) 0.3200-0.3240; (all, all, 32, 96)
+//    0.3295; (0, 0, 0, 0) 0.3309; (0, 0, 0, 128) 0.3268.  These are the defaults below.
+//  * Two or more sets of buffers in rotation (parameter groups taking turns on shared buffers, gigabytes of other
+//    traffic between two visits): write-through data only defers its write-back into time the memory would spend
+//    idle around kernel boundaries, which pays up to about 128 MB per step (half of the cache) and costs beyond.
+//    Same layer, two sets alternating: (0, 0, 0, 0) 0.3317; (all, all, 0, 0) 0.3331; (all, all, 32, 56) 0.3329;
+//    (0, all, 0, 16) 0.3282; (all, 0, 0, 64) 0.3272; (0, 0, 32, 96) 0.3272; (0, 0, 0, 128) 0.3268; (0, 0, 64, 96)
+//    0.3328.  Who gets the budget matters little; the reduce copy-in takes it whatever the shard size in the policy
+//    that the fully_shard layer selects for models with several parameter groups (options at run time).
+// An AdamW pass with a write-through tail gains 6 % when it visits the same shard again and again and loses 2 % over
+// four shards in rotation (each is visited once per optimizer step): the optimizer kernels store non-temporal.
 #ifndef YAFSDP_GATHER_TAIL_WT_MB
 #define YAFSDP_GATHER_TAIL_WT_MB 56
 #endif
