@@ -405,13 +405,13 @@ typedef enum yafsdp_option {
                                          yafsdp_copy_in_scatter_out, which write through everywhere by default;
                                          0 = they store everything non-temporal */
   YAFSDP_OPT_POST_REDUCE_TAIL_MB = 7  /* the same for yafsdp_post_reduce / yafsdp_post_reduce_fragments.
-                                         The defaults of options 4-7 suit a caller that rewrites ONE set of buffers
-                                         step after step (the next step finds what wrote through still cached).
-                                         A caller whose kernels take turns on several sets of buffers, as the
-                                         parameter groups of a model do, is served best by 0 / 0 / 0 / 128 for
-                                         options 6 / 7 / 5 / 4: write-through data then only defers its
-                                         write-back, which pays up to half of the 256-MB memory-side cache per
-                                         step */
+                                         Written-through lines pay if they are still in the 256-MB memory-side
+                                         cache when their buffer is read or written again, and cost if they are
+                                         evicted in the middle of other kernels.  The defaults of options 4-7 suit
+                                         a caller that rewrites ONE set of buffers step after step.  A caller whose
+                                         parameter groups take turns on shared buffers, with one gradient buffer
+                                         for all groups as in the reference, is served best by 0 / 0 / 0 / 128 for
+                                         options 6 / 7 / 5 / 4 (the end of the buffer that comes round soonest) */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);

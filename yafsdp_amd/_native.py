@@ -882,15 +882,15 @@ def get_option(option: int) -> int:
 
 # Store policies: how many megabytes at the END of each kind of kernel's output are stored write-through (the rest
 # non-temporal), as (flat copies / casts / divides, post-reduce, scatter-out, gather-in).  Written-through lines
-# stay in the 256-MB memory-side cache until later traffic evicts them, so the right amount depends on when the
-# written buffers are touched again:
+# stay in the 256-MB memory-side cache until later traffic evicts them; they pay if they are still there when their
+# buffer is touched again (a read is served from the cache, a write overwrites them before they reached DRAM) and
+# cost if they are evicted in the middle of other kernels:
 #   "single_set"     one set of buffers rewritten step after step (one parameter group; a loop over one layer): the
-#                    flat kernels write through everywhere and the two table kernels their last 32 / 56 MB; the next
-#                    step finds much of it still cached.  The library's own defaults.
-#   "rotating_sets"  several parameter groups taking turns on shared buffers (ya_fsdp/_state.py:636-652), gigabytes
-#                    of other traffic between two visits: write-through data only defers its write-back, which
-#                    pays up to about 128 MB per step (half of the cache) and costs beyond; the reduce copy-in takes
-#                    that budget whatever the shard size, everything else stores non-temporal.
+#                    flat kernels write through everywhere and the two table kernels their last 32 / 56 MB.  The
+#                    library's own defaults.
+#   "rotating_sets"  several parameter groups taking turns on shared buffers (ya_fsdp/_state.py:636-652): the one
+#                    gradient buffer that all groups share comes round soonest, so the reduce copy-in writes its
+#                    last 128 MB through and everything else stores non-temporal.
 _EVERYTHING = 1 << 20
 STORE_POLICIES = {"single_set": (_EVERYTHING, _EVERYTHING, 32, 56), "rotating_sets": (0, 0, 0, 128)}
 _STORE_POLICY_OPTIONS = (OPT_FLAT_TAIL_MB, OPT_POST_REDUCE_TAIL_MB, OPT_SCATTER_TAIL_MB, OPT_GATHER_TAIL_MB)

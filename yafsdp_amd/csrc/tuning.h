@@ -101,19 +101,22 @@ constexpr bool scatter_nt_load(int unroll) {
 // run-time choice per kind of kernel: always the END of the output (the last tiles of the flat buffer in gather-in,
 // the tile slots of the last tensors in scatter-out, the last tiles of a flat pass), because a kernel whose last
 // stores wrote through ends with clean L2s (its closing write-back finds no dirty line, 40 thousand otherwise).
-// What write-through data is worth depends on when the written buffers are touched again:
-//  * One set of buffers rewritten step after step (a loop over one layer; a model with one parameter group): the next
-//    step finds much of what wrote through still cached, reads it from there or overwrites it before it ever reached
-//    DRAM.  Llama-3-8B layer, ms per step, megabytes of (flat kernels, post-reduce, scatter-out tail, gather-in
-//    tail): (all, all, 0, 0) 0.3272; (all, all, 0, 96) 0.3226; (all, all, 32, 56) 0.3200-0.3240; (all, all, 32, 96)
-//    0.3295; (0, 0, 0, 0) 0.3309; (0, 0, 0, 128) 0.3268.  These are the defaults below.
-//  * Two or more sets of buffers in rotation (parameter groups taking turns on shared buffers, gigabytes of other
-//    traffic between two visits): write-through data only defers its write-back into time the memory would spend
-//    idle around kernel boundaries, which pays up to about 128 MB per step (half of the cache) and costs beyond.
-//    Same layer, two sets alternating: (0, 0, 0, 0) 0.3317; (all, all, 0, 0) 0.3331; (all, all, 32, 56) 0.3329;
-//    (0, all, 0, 16) 0.3282; (all, 0, 0, 64) 0.3272; (0, 0, 32, 96) 0.3272; (0, 0, 0, 128) 0.3268; (0, 0, 64, 96)
-//    0.3328.  Who gets the budget matters little; the reduce copy-in takes it whatever the shard size in the policy
-//    that the fully_shard layer selects for models with several parameter groups (options at run time).
+// What write-through data is worth depends on whether it is still in that cache when its buffer is touched again:
+// a later read is then served from there, and a later write overwrites it before it ever reached DRAM.
+//  * One set of buffers rewritten step after step (a loop over one layer; a model with one parameter group): much of
+//    what wrote through is found again.  Llama-3-8B layer, ms per step, megabytes of (flat kernels, post-reduce,
+//    scatter-out tail, gather-in tail): (all, all, 0, 0) 0.3272; (all, all, 0, 96) 0.3226; (all, all, 32, 56)
+//    0.3200-0.3240; (all, all, 32, 96) 0.3295; (0, 0, 0, 0) 0.3309; (0, 0, 0, 128) 0.3268.  These are the defaults below.
+//  * K sets of buffers taking turns, 2.2 GB of other traffic between two visits of a set: a set's written-through end
+//    survives until its next visit if K of them fit the cache together, and costs (evictions of dirty lines in the
+//    middle of other kernels) if they do not.  Gather-in tail alone, everything else non-temporal, same layer:
+//    K=2: 0 MB 0.3317, 96 MB 0.3285, 128 MB 0.3277, 144 MB 0.3321; K=3: 0 MB 0.3323, 64 MB 0.3299, 85 MB 0.3294,
+//    128 MB 0.3340; K=4: 0 MB 0.3339, 64 MB 0.3320, 85 MB 0.3359.  With the defaults above: K=2 0.3329, K=3 0.3346,
+//    K=4 0.3354 (write-through everywhere in the flat kernels already overfills the cache).  The reference shares ONE
+//    gradient buffer among all parameter groups (and two gathered buffers), so the reduce buffer's end is what comes
+//    round soonest: the policy that the fully_shard layer selects for models with several groups writes the last
+//    128 MB of the reduce buffer through and nothing else (options at run time), which is also what a full pass over
+//    35 groups measures as best, alone and next to GEMMs.
 // An AdamW pass with a write-through tail gains 6 % when it visits the same shard again and again and loses 2 % over
 // four shards in rotation (each is visited once per optimizer step): the optimizer kernels store non-temporal.
 #ifndef YAFSDP_GATHER_TAIL_WT_MB
