@@ -1355,10 +1355,10 @@ def main() -> int:
                          "(the library's launch-shape option; default: the library's own threshold)")
     ap.add_argument("--gather-tail-mb", type=int, default=None, metavar="N",
                     help="megabytes at the end of the reduce buffer that the reduce copy-in stores write-through "
-                         "(the library's store-policy option; default: the library's own, 56; 0 = none)")
+                         "(the library's store-policy option; default: the library's own, 96; 0 = none)")
     ap.add_argument("--scatter-tail-mb", type=int, default=None, metavar="N",
                     help="the same for the last megabytes of tensors that copy-out writes (default: the library's "
-                         "own, 32; 0 = none)")
+                         "own, 0 = none)")
     ap.add_argument("--flat-tail-mb", type=int, default=None, metavar="N",
                     help="the same for the flat kernels (copy-in, post-reduce), which write through everywhere by "
                          "default; 0 = they store everything non-temporal")

@@ -388,18 +388,18 @@ typedef enum yafsdp_option {
                                          layout (short 512-element tiles when every tensor starts on a 128-byte
                                          line of the flat buffer, the gather-in tile otherwise), 1 = always
                                          short, 2 = never short */
-  YAFSDP_OPT_GATHER_TAIL_MB = 4,      /* 0..2^20, default 56: yafsdp_gather_in / yafsdp_gather_in_bound write the last
+  YAFSDP_OPT_GATHER_TAIL_MB = 4,      /* 0..2^20, default 96: yafsdp_gather_in / yafsdp_gather_in_bound write the last
                                          `value` megabytes of the flat buffer through the L2s instead of leaving
                                          them there as dirty lines (a store-policy choice; the bytes written are
                                          the same).  The memory-side cache absorbs them and writes them back
                                          later: the kernel ends sooner, and whatever runs next pays for the
                                          write-back only if it saturates the memory itself from its first
                                          microsecond.  0 = off */
-  YAFSDP_OPT_SCATTER_TAIL_MB = 5,     /* 0..2^20, default 32: the same for the tile slots of the last `value`
+  YAFSDP_OPT_SCATTER_TAIL_MB = 5,     /* 0..2^20, default 0: the same for the tile slots of the last `value`
                                          megabytes of tensors in yafsdp_scatter_out / yafsdp_scatter_out_bound /
-                                         yafsdp_copy_in_scatter_out.  Consecutive kernels share one budget of
-                                         write-through data in flight (about 100 MB on MI355X, the flat kernels'
-                                         stores included): raise one option and lower the other */
+                                         yafsdp_copy_in_scatter_out.  What one kernel wrote through the next
+                                         may have to evict: with 32 here and 56 for the reduce copy-in a step of
+                                         the two is 0.8 % shorter and the reduce copy-in itself 3 % longer */
   YAFSDP_OPT_FLAT_TAIL_MB = 6,        /* 0..2^20, default 2^20 (everything): the same for yafsdp_flat_copy,
                                          yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
                                          yafsdp_copy_in_scatter_out, which write through everywhere by default;

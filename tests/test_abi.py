@@ -55,13 +55,13 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_set_option(4, -1) == -1
     assert L.yafsdp_set_option(4, (1 << 20) + 1) == -1
     tail = ctypes.c_int(-1)
-    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 56
+    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 96
     assert L.yafsdp_set_option(4, 0) == 0 and L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 0
-    assert L.yafsdp_set_option(4, 56) == 0
+    assert L.yafsdp_set_option(4, 96) == 0
     assert L.yafsdp_set_option(5, -1) == -1
-    assert L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 32
+    assert L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 0
     assert L.yafsdp_set_option(5, 7) == 0 and L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 7
-    assert L.yafsdp_set_option(5, 32) == 0
+    assert L.yafsdp_set_option(5, 0) == 0
     assert L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 1 << 20
     assert L.yafsdp_set_option(6, 0) == 0 and L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 0
     assert L.yafsdp_set_option(6, 1 << 20) == 0
@@ -109,7 +109,7 @@ def test_store_policies_set_the_four_tail_options():
 
     from yafsdp_amd import _native
 
-    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"] == (1 << 20, 1 << 20, 32, 56)
+    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"] == (1 << 20, 1 << 20, 0, 96)
     try:
         _native.set_store_policy("rotating_sets")
         assert _native.get_store_policy() == (0, 0, 0, 128)

@@ -886,13 +886,13 @@ def get_option(option: int) -> int:
 # buffer is touched again (a read is served from the cache, a write overwrites them before they reached DRAM) and
 # cost if they are evicted in the middle of other kernels:
 #   "single_set"     one set of buffers rewritten step after step (one parameter group; a loop over one layer): the
-#                    flat kernels write through everywhere and the two table kernels their last 32 / 56 MB.  The
+#                    flat kernels write through everywhere and the reduce copy-in its last 96 MB.  The
 #                    library's own defaults.
 #   "rotating_sets"  several parameter groups taking turns on shared buffers (ya_fsdp/_state.py:636-652): the one
 #                    gradient buffer that all groups share comes round soonest, so the reduce copy-in writes its
 #                    last 128 MB through and everything else stores non-temporal.
 _EVERYTHING = 1 << 20
-STORE_POLICIES = {"single_set": (_EVERYTHING, _EVERYTHING, 32, 56), "rotating_sets": (0, 0, 0, 128)}
+STORE_POLICIES = {"single_set": (_EVERYTHING, _EVERYTHING, 0, 96), "rotating_sets": (0, 0, 0, 128)}
 _STORE_POLICY_OPTIONS = (OPT_FLAT_TAIL_MB, OPT_POST_REDUCE_TAIL_MB, OPT_SCATTER_TAIL_MB, OPT_GATHER_TAIL_MB)
 
 

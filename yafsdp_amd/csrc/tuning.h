@@ -105,13 +105,15 @@ constexpr bool scatter_nt_load(int unroll) {
 // a later read is then served from there, and a later write overwrites it before it ever reached DRAM.
 //  * One set of buffers rewritten step after step (a loop over one layer; a model with one parameter group): much of
 //    what wrote through is found again.  Llama-3-8B layer, ms per step, megabytes of (flat kernels, post-reduce,
-//    scatter-out tail, gather-in tail): (all, all, 0, 0) 0.3272; (all, all, 0, 96) 0.3226; (all, all, 32, 56)
-//    0.3200-0.3240; (all, all, 32, 96) 0.3295; (0, 0, 0, 0) 0.3309; (0, 0, 0, 128) 0.3268.  These are the defaults below.
+//    scatter-out tail, gather-in tail): (all, all, 0, 0) 0.3272; (all, all, 0, 64) 0.3239; (all, all, 0, 96) 0.3226,
+//    the defaults below; (all, all, 0, 128) 0.3334; (all, all, 32, 56) 0.3200, but the reduce copy-in itself then
+//    runs 135 us instead of 131.5 (it pays for the copy-out's lines); (all, all, 32, 96) 0.3295; (0, 0, 0, 0) 0.3309;
+//    (0, 0, 0, 128) 0.3268.
 //  * K sets of buffers taking turns, 2.2 GB of other traffic between two visits of a set: a set's written-through end
 //    survives until its next visit if K of them fit the cache together, and costs (evictions of dirty lines in the
 //    middle of other kernels) if they do not.  Gather-in tail alone, everything else non-temporal, same layer:
 //    K=2: 0 MB 0.3317, 96 MB 0.3285, 128 MB 0.3277, 144 MB 0.3321; K=3: 0 MB 0.3323, 64 MB 0.3299, 85 MB 0.3294,
-//    128 MB 0.3340; K=4: 0 MB 0.3339, 64 MB 0.3320, 85 MB 0.3359.  With the defaults above: K=2 0.3329, K=3 0.3346,
+//    128 MB 0.3340; K=4: 0 MB 0.3339, 64 MB 0.3320, 85 MB 0.3359.  With (all, all, 32, 56): K=2 0.3329, K=3 0.3346,
 //    K=4 0.3354 (write-through everywhere in the flat kernels already overfills the cache).  The reference shares ONE
 //    gradient buffer among all parameter groups (and two gathered buffers), so the reduce buffer's end is what comes
 //    round soonest: the policy that the fully_shard layer selects for models with several groups writes the last
@@ -120,10 +122,10 @@ constexpr bool scatter_nt_load(int unroll) {
 // An AdamW pass with a write-through tail gains 6 % when it visits the same shard again and again and loses 2 % over
 // four shards in rotation (each is visited once per optimizer step): the optimizer kernels store non-temporal.
 #ifndef YAFSDP_GATHER_TAIL_WT_MB
-#define YAFSDP_GATHER_TAIL_WT_MB 56
+#define YAFSDP_GATHER_TAIL_WT_MB 96
 #endif
 #ifndef YAFSDP_SCATTER_TAIL_WT_MB
-#define YAFSDP_SCATTER_TAIL_WT_MB 32
+#define YAFSDP_SCATTER_TAIL_WT_MB 0
 #endif
 constexpr int kGatherTailWriteThroughMb = YAFSDP_GATHER_TAIL_WT_MB;    // default of YAFSDP_OPT_GATHER_TAIL_MB
 constexpr int kScatterTailWriteThroughMb = YAFSDP_SCATTER_TAIL_WT_MB;  // default of YAFSDP_OPT_SCATTER_TAIL_MB
