@@ -27,6 +27,9 @@ def test_library_exports_every_symbol():
 
     for name in _declared_functions():
         assert hasattr(_native.lib, name), name
+    import __graft_entry__
+
+    assert _native.lib.yafsdp_version() // 1000 == __graft_entry__.ABI_MAJOR  # what build() checks
     assert _native.lib.yafsdp_version() == 1005  # 1.1: yafsdp_flat_copy_bytes; 1.2-1.5: the four write-through tail options
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
