@@ -660,6 +660,10 @@ def test_store_policy_follows_the_number_of_parameter_groups(monkeypatch):
     model = _wrap(_make(61), mp_policy=MP)  # four groups
     model(x).float().pow(2).mean().backward()
     assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"]
+    # a gradient buffer per group (gradient accumulation without reduction): four buffers take turns
+    model = _wrap(_make(63), mp_policy=MP)
+    model._get_fsdp_state()._lazy_init(allow_no_grad_reduce=True)
+    assert _native.get_store_policy() == (0, 0, 0, 64)
     single = fully_shard(Block(128, 256).to(DEV), mp_policy=MP)  # one group
     single(x).float().pow(2).mean().backward()
     assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"]

@@ -193,13 +193,6 @@ class YaFSDPState(_State):
         param_groups = [s._fsdp_param_group for s in self._state_ctx.all_states if s._fsdp_param_group is not None]
         if not param_groups:
             return
-        # which stores write through depends on how soon the written buffers come round again, and this is where
-        # that is known: several groups take turns on the shared buffers, a single group rewrites its own
-        policy = os.environ.get("YAFSDP_STORE_POLICY", "auto")
-        if policy == "auto":
-            policy = "rotating_sets" if len(param_groups) > 1 else "single_set"
-        if policy != "keep":
-            _native.set_store_policy(policy)
         no_reshard_after_forward = all(not g.reshard_after_forward for g in param_groups)
 
         def assign(groups, attr, count, size_of, ctx_idx=None, idx_to_handle=None):
@@ -245,9 +238,23 @@ class YaFSDPState(_State):
             owner_state = next(s for s in self._state_ctx.all_states if s._fsdp_param_group is last)
             if owner_state._auto_reshard_after_forward:
                 last.reshard_after_forward = False  # ya_fsdp/_state.py:256-260
-        assign([g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx",
-               None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes_by_dtype(),
-               param_group_to_grad_buffer_ctx_idx, grad_buffer_ctx_idx_to_yccl_handle)
+        grad_users = assign([g for g in param_groups if g.grad_buffer_ctx is not None], "grad_buffer_ctx",
+                            None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes_by_dtype(),
+                            param_group_to_grad_buffer_ctx_idx, grad_buffer_ctx_idx_to_yccl_handle)
+        # Which stores write through (and so stay in the 256-MB memory-side cache) depends on how soon the written
+        # buffers come round again, and this is where that is known.  A single group rewrites its own buffers step
+        # after step.  Several groups take turns: the gradient buffers come round soonest (one for all groups by
+        # default), and the written-through end of each survives until its next visit if all of them fit the cache
+        # together (measured with 2, 3 and 4 buffers in rotation: 128, 85, 64 MB each).
+        policy = os.environ.get("YAFSDP_STORE_POLICY", "auto")
+        if policy == "auto":
+            if len(param_groups) == 1:
+                policy = "single_set"
+            else:
+                tail_mb = min(128, 256 // max(1, len(grad_users)))
+                policy = (0, 0, 0, tail_mb if tail_mb >= 32 else 0)
+        if policy != "keep":
+            _native.set_store_policy(policy)
 
     def validate_shared_state(self) -> None:
         """ya_fsdp/_state.py:290-414: enough buffers for overlap; at most one
