@@ -404,7 +404,8 @@ typedef enum yafsdp_option {
                                          yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
                                          yafsdp_copy_in_scatter_out, which write through everywhere by default;
                                          0 = they store everything non-temporal */
-  YAFSDP_OPT_POST_REDUCE_TAIL_MB = 7  /* the same for yafsdp_post_reduce / yafsdp_post_reduce_fragments.
+  YAFSDP_OPT_POST_REDUCE_TAIL_MB = 7  /* the same for yafsdp_post_reduce / yafsdp_post_reduce_sumsq /
+                                         yafsdp_post_reduce_fragments.
                                          Written-through lines pay if they are still in the 256-MB memory-side
                                          cache when their buffer is read or written again, and cost if they are
                                          evicted in the middle of other kernels.  The defaults of options 4-7 suit

@@ -299,6 +299,18 @@ def test_post_reduce_sumsq(nat, shard_dt, chunk_dt, post, acc):
         assert torch.allclose(av, bv, rtol=2e-7, atol=0.0), (av, bv)
 
 
+@pytest.mark.parametrize("tail_mb", [0, 1, 3])
+def test_post_reduce_sumsq_with_the_write_through_boundary_inside_the_shard(nat, tail_mb):
+    """The same pass with only the last megabytes of the shard stored write-through (0: none): same shard, same sums."""
+    default = nat.get_option(nat.OPT_POST_REDUCE_TAIL_MB)
+    nat.set_option(nat.OPT_POST_REDUCE_TAIL_MB, tail_mb)
+    try:
+        test_post_reduce_sumsq(nat, torch.float32, torch.bfloat16, 8.0, True)
+        test_post_reduce_sumsq(nat, torch.bfloat16, torch.float32, None, False)
+    finally:
+        nat.set_option(nat.OPT_POST_REDUCE_TAIL_MB, default)
+
+
 def test_post_reduce_sumsq_special_values_and_errors(nat):
     # a NaN or an infinity in the result makes the norm non-finite, as torch's norm would
     chunk = torch.tensor([1.0, float("inf"), 2.0, 3.0, 0.5, 0.25, 7.0, 8.0, 9.0], device=DEV).bfloat16()

@@ -843,7 +843,9 @@ int yafsdp_post_reduce_sumsq(void* shard, int shard_dtype, const void* chunk, in
   float k;
   scale_plan(post_factor, &scale, &k);
   const hipError_t e = launch_post_reduce_sumsq(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, chunk, n, head,
-                                                k, partials, int(n_tiles), static_cast<hipStream_t>(stream));
+                                                k, partials,
+                                                flat_wt_from(n_tiles, tile, shard_dtype, g_post_reduce_tail_mb),
+                                                int(n_tiles), static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return int(e);
   *n_written = n_tiles;
   return YAFSDP_OK;

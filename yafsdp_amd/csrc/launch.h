@@ -45,7 +45,7 @@ hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int gri
 // the same pass, also writing partials[0:grid] = per-workgroup sums of squares of the stored values (postsumsq.hip);
 // grid must equal the number of tiles
 hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n,
-                                    int head, float k, double* partials, int grid, hipStream_t stream);
+                                    int head, float k, double* partials, int wt_from, int grid, hipStream_t stream);
 
 // META is SmallMeta or LargeMeta (explicitly instantiated in gather.hip / scatter.hip);
 // `block` is the workgroup size the table was built for (kTableBlockSmall or kTableBlockLarge); for launch_scatter

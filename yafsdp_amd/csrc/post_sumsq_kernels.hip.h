@@ -49,9 +49,50 @@ __device__ __forceinline__ double post_scalar_sumsq(void* dst, const void* src, 
   return double(stored) * double(stored);
 }
 
+// One full tile of the pass: stores with policy STP, adds the squares of what it stored to acc0 / acc1.
+template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
+__device__ __forceinline__ void post_sumsq_full_tile(char* dt, const char* st, float k, double& acc0, double& acc1) {
+  const TileStore<D, STP> out(dt, BLOCK * U * 8 * D::kSize);
+  if constexpr (wide_pair<S, D>::value) {
+    Quad<S> s[2 * U];
+    Quad<D> d[2 * U];
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(st + quad_elem<BLOCK, U>(q) * S::kSize);
+    if constexpr (ACC) {
+#pragma unroll
+      for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dt + quad_elem<BLOCK, U>(q) * D::kSize);
+    }
+#pragma unroll
+    for (int q = 0; q < 2 * U; q++) {
+      const Quad<D> r = flat_quad<S, D, SCALE, ACC>(s[q], d[q], k);
+      store_quad_at<D, STP>(out, quad_elem<BLOCK, U>(q) * D::kSize, r);
+      if (q & 1) acc1 = quad_sumsq<D>(r, acc1);
+      else acc0 = quad_sumsq<D>(r, acc0);
+    }
+  } else {
+    Unit<S> s[U];
+    Unit<D> d[U];
+#pragma unroll
+    for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(st + unit_index<BLOCK, U>(j) * (8 * S::kSize));
+    if constexpr (ACC) {
+#pragma unroll
+      for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dt + unit_index<BLOCK, U>(j) * (8 * D::kSize));
+    }
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      const Unit<D> r = flat_unit<S, D, SCALE, ACC>(s[j], d[j], k);
+      store_unit_at<D, STP>(out, unit_index<BLOCK, U>(j) * (8 * D::kSize), r);
+      if (j & 1) acc1 = unit_sumsq<D>(r, acc1);
+      else acc0 = unit_sumsq<D>(r, acc0);
+    }
+  }
+}
+
+// With STP = ST_WT the full tiles before tile `wt_from` store non-temporal instead (0: every tile writes through),
+// as in flat_kernel.
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
-post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float k, double* partials) {
+post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float k, double* partials, int wt_from) {
   __shared__ double lds[BLOCK / 64];
   constexpr bool NTS = (STP == ST_NT);  // the partial last tile keeps ordinary global stores
   const int tid = threadIdx.x;
@@ -72,40 +113,10 @@ post_reduce_sumsq_kernel(void* dst, const void* src, int64_t n, int head, float 
     char* dt = dbase + tile * kTile * (8 * D::kSize);
     const char* st = sbase + tile * kTile * (8 * S::kSize);
     if (tile * kTile + kTile <= n_units) {
-      const TileStore<D, STP> out(dt, BLOCK * U * 8 * D::kSize);
-      if constexpr (wide_pair<S, D>::value) {
-        Quad<S> s[2 * U];
-        Quad<D> d[2 * U];
-#pragma unroll
-        for (int q = 0; q < 2 * U; q++) s[q] = load_quad<S, NTL>(st + quad_elem<BLOCK, U>(q) * S::kSize);
-        if constexpr (ACC) {
-#pragma unroll
-          for (int q = 0; q < 2 * U; q++) d[q] = load_quad<D, NTL>(dt + quad_elem<BLOCK, U>(q) * D::kSize);
-        }
-#pragma unroll
-        for (int q = 0; q < 2 * U; q++) {
-          const Quad<D> r = flat_quad<S, D, SCALE, ACC>(s[q], d[q], k);
-          store_quad_at<D, STP>(out, quad_elem<BLOCK, U>(q) * D::kSize, r);
-          if (q & 1) acc1 = quad_sumsq<D>(r, acc1);
-          else acc0 = quad_sumsq<D>(r, acc0);
-        }
-      } else {
-        Unit<S> s[U];
-        Unit<D> d[U];
-#pragma unroll
-        for (int j = 0; j < U; j++) s[j] = load_unit<S, NTL>(st + unit_index<BLOCK, U>(j) * (8 * S::kSize));
-        if constexpr (ACC) {
-#pragma unroll
-          for (int j = 0; j < U; j++) d[j] = load_unit<D, NTL>(dt + unit_index<BLOCK, U>(j) * (8 * D::kSize));
-        }
-#pragma unroll
-        for (int j = 0; j < U; j++) {
-          const Unit<D> r = flat_unit<S, D, SCALE, ACC>(s[j], d[j], k);
-          store_unit_at<D, STP>(out, unit_index<BLOCK, U>(j) * (8 * D::kSize), r);
-          if (j & 1) acc1 = unit_sumsq<D>(r, acc1);
-          else acc0 = unit_sumsq<D>(r, acc0);
-        }
-      }
+      if (STP == ST_WT && tile < wt_from)
+        post_sumsq_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, ST_NT>(dt, st, k, acc0, acc1);
+      else
+        post_sumsq_full_tile<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dt, st, k, acc0, acc1);
     } else {  // last, partial tile
       for (int64_t u = tile * kTile + tid; u < n_units; u += BLOCK) {
         Unit<S> s = load_unit<S, NTL>(sbase + u * (8 * S::kSize));

@@ -8,33 +8,33 @@ namespace yafsdp {
 namespace {
 
 template <class S, class D, int SCALE, bool ACC>
-hipError_t go(void* dst, const void* src, int64_t n, int head, float k, double* partials, int grid,
-              hipStream_t stream) {
+hipError_t go(void* dst, const void* src, int64_t n, int head, float k, double* partials, int wt_from,
+              int grid, hipStream_t stream) {
   return launch_kernel(post_reduce_sumsq_kernel<S, D, SCALE, ACC, kPostSumsqBlock, kPostSumsqUnroll, kFlatNtLoad, kFlatStorePolicy>,
-                       grid, kPostSumsqBlock, stream, dst, src, n, head, k, partials);
+                       grid, kPostSumsqBlock, stream, dst, src, n, head, k, partials, wt_from);
 }
 
 template <class S, class D>
 hipError_t by_op(int scale, bool acc, void* dst, const void* src, int64_t n, int head, float k, double* partials,
-                 int grid, hipStream_t stream) {
+                 int wt_from, int grid, hipStream_t stream) {
   switch (scale * 2 + (acc ? 1 : 0)) {
-    case 0: return go<S, D, SCALE_NONE, false>(dst, src, n, head, k, partials, grid, stream);
-    case 1: return go<S, D, SCALE_NONE, true>(dst, src, n, head, k, partials, grid, stream);
-    case 2: return go<S, D, SCALE_MUL, false>(dst, src, n, head, k, partials, grid, stream);
-    case 3: return go<S, D, SCALE_MUL, true>(dst, src, n, head, k, partials, grid, stream);
-    case 4: return go<S, D, SCALE_DIV, false>(dst, src, n, head, k, partials, grid, stream);
-    case 5: return go<S, D, SCALE_DIV, true>(dst, src, n, head, k, partials, grid, stream);
+    case 0: return go<S, D, SCALE_NONE, false>(dst, src, n, head, k, partials, wt_from, grid, stream);
+    case 1: return go<S, D, SCALE_NONE, true>(dst, src, n, head, k, partials, wt_from, grid, stream);
+    case 2: return go<S, D, SCALE_MUL, false>(dst, src, n, head, k, partials, wt_from, grid, stream);
+    case 3: return go<S, D, SCALE_MUL, true>(dst, src, n, head, k, partials, wt_from, grid, stream);
+    case 4: return go<S, D, SCALE_DIV, false>(dst, src, n, head, k, partials, wt_from, grid, stream);
+    case 5: return go<S, D, SCALE_DIV, true>(dst, src, n, head, k, partials, wt_from, grid, stream);
   }
   return hipErrorInvalidValue;
 }
 
 template <class S>
 hipError_t by_dst(int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head, float k,
-                  double* partials, int grid, hipStream_t stream) {
+                  double* partials, int wt_from, int grid, hipStream_t stream) {
   switch (dst_dt) {
-    case DT_F32: return by_op<S, F32>(scale, acc, dst, src, n, head, k, partials, grid, stream);
-    case DT_BF16: return by_op<S, BF16>(scale, acc, dst, src, n, head, k, partials, grid, stream);
-    case DT_F16: return by_op<S, F16>(scale, acc, dst, src, n, head, k, partials, grid, stream);
+    case DT_F32: return by_op<S, F32>(scale, acc, dst, src, n, head, k, partials, wt_from, grid, stream);
+    case DT_BF16: return by_op<S, BF16>(scale, acc, dst, src, n, head, k, partials, wt_from, grid, stream);
+    case DT_F16: return by_op<S, F16>(scale, acc, dst, src, n, head, k, partials, wt_from, grid, stream);
   }
   return hipErrorInvalidValue;
 }
@@ -42,11 +42,11 @@ hipError_t by_dst(int dst_dt, int scale, bool acc, void* dst, const void* src, i
 }  // namespace
 
 hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n,
-                                    int head, float k, double* partials, int grid, hipStream_t stream) {
+                                    int head, float k, double* partials, int wt_from, int grid, hipStream_t stream) {
   switch (src_dt) {
-    case DT_F32: return by_dst<F32>(dst_dt, scale, acc, dst, src, n, head, k, partials, grid, stream);
-    case DT_BF16: return by_dst<BF16>(dst_dt, scale, acc, dst, src, n, head, k, partials, grid, stream);
-    case DT_F16: return by_dst<F16>(dst_dt, scale, acc, dst, src, n, head, k, partials, grid, stream);
+    case DT_F32: return by_dst<F32>(dst_dt, scale, acc, dst, src, n, head, k, partials, wt_from, grid, stream);
+    case DT_BF16: return by_dst<BF16>(dst_dt, scale, acc, dst, src, n, head, k, partials, wt_from, grid, stream);
+    case DT_F16: return by_dst<F16>(dst_dt, scale, acc, dst, src, n, head, k, partials, wt_from, grid, stream);
   }
   return hipErrorInvalidValue;
 }
