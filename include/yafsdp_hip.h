@@ -401,7 +401,7 @@ typedef enum yafsdp_option {
                                          may have to evict: with 32 here and 56 for the reduce copy-in a step of
                                          the two is 0.8 % shorter and the reduce copy-in itself 3 % longer */
   YAFSDP_OPT_FLAT_TAIL_MB = 6,        /* 0..2^20, default 2^20 (everything): the same for yafsdp_flat_copy,
-                                         yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
+                                         yafsdp_flat_copy_bytes, yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
                                          yafsdp_copy_in_scatter_out, which write through everywhere by default;
                                          0 = they store everything non-temporal */
   YAFSDP_OPT_POST_REDUCE_TAIL_MB = 7  /* the same for yafsdp_post_reduce / yafsdp_post_reduce_sumsq /

@@ -159,6 +159,11 @@ def test_flat_kernels_with_the_write_through_boundary_inside_the_buffer(nat, tai
             got = torch.full((n + 11,), 3.0, dtype=dst_dt, device=DEV)
             nat.flat_copy(got[3 : 3 + n], src.to(DEV)[1:])
             assert_bits_equal(got, want, "flat_copy")
+        raw = torch.randint(0, 256, (4 * n + 8,), generator=g, dtype=torch.uint8)  # 6 MB between odd byte addresses
+        got = torch.zeros(4 * n + 8, dtype=torch.uint8, device=DEV)
+        nat.flat_copy(got[3 : 3 + 4 * n], raw.to(DEV)[1 : 1 + 4 * n])
+        assert torch.equal(got[3 : 3 + 4 * n].cpu(), raw[1 : 1 + 4 * n]) and int(got[:3].max()) == 0
+        assert int(got[3 + 4 * n :].max()) == 0
         buf = mixed_values(g, n, torch.bfloat16)
         want = buf.clone()
         torch_ops.div_if_needed(want, 8.0)

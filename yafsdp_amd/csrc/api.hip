@@ -768,7 +768,11 @@ int yafsdp_flat_copy_bytes(void* dst, const void* src, int64_t n_bytes, void* st
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return int(e);
   const int grid = grid_for(n_tiles, g_flat_blocks_per_cu.load(std::memory_order_relaxed), device);
-  return int(launch_bytes(dst, src, n_bytes, int(head), grid, static_cast<hipStream_t>(stream)));
+  // (a tile is one 16-byte vector per lane)
+  const int64_t tail_tiles = (int64_t(g_flat_tail_mb.load(std::memory_order_relaxed)) << 20) / (int64_t(kFlatBlock) * 16);
+  const int64_t wt_from = tail_tiles >= n_tiles ? 0 : n_tiles - tail_tiles;
+  return int(launch_bytes(dst, src, n_bytes, int(head), wt_from > INT32_MAX ? INT32_MAX : int(wt_from), grid,
+                          static_cast<hipStream_t>(stream)));
 }
 
 int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream) {

@@ -62,9 +62,9 @@ hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, c
   return hipErrorInvalidValue;
 }
 
-hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int grid, hipStream_t stream) {
+hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int wt_from, int grid, hipStream_t stream) {
   return launch_kernel(bytes_kernel<kFlatBlock, kFlatNtLoad, kFlatStorePolicy>, grid, kFlatBlock, stream, dst, src, n,
-                       head);
+                       head, wt_from);
 }
 
 }  // namespace yafsdp

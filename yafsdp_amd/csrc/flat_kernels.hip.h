@@ -165,7 +165,7 @@ typedef u32x4 u32x4_a1 __attribute__((aligned(1)));
 
 template <int BLOCK, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
-bytes_kernel(void* dst, const void* src, int64_t n, int head) {
+bytes_kernel(void* dst, const void* src, int64_t n, int head, int wt_from) {
   static_assert(BLOCK >= 128, "workgroup 0 copies up to 127 leading bytes, one per lane");
   const int tid = threadIdx.x;
   const int64_t n_vecs = (n - head) >> 4;
@@ -184,12 +184,17 @@ bytes_kernel(void* dst, const void* src, int64_t n, int head) {
   for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
     const int64_t v = tile * BLOCK + tid;
     if (tile * BLOCK + BLOCK <= n_vecs) {
-      const TileStore<BF16, STP> out(dbase + tile * BLOCK * 16, BLOCK * 16);
       const u32x4_a1* q = reinterpret_cast<const u32x4_a1*>(sbase + v * 16);
       u32x4 x;
       if constexpr (NTL) x = __builtin_nontemporal_load(q);
       else x = *q;
-      out.vec(tid * 16, x);
+      if (STP == ST_WT && tile < wt_from) {  // before the write-through part of the output, as in flat_body
+        const TileStore<BF16, ST_NT> out(dbase + tile * BLOCK * 16, BLOCK * 16);
+        out.vec(tid * 16, x);
+      } else {
+        const TileStore<BF16, STP> out(dbase + tile * BLOCK * 16, BLOCK * 16);
+        out.vec(tid * 16, x);
+      }
     } else if (v < n_vecs) {  // last, partial tile
       const u32x4 x = *reinterpret_cast<const u32x4_a1*>(sbase + v * 16);
       *reinterpret_cast<u32x4*>(dbase + v * 16) = x;

@@ -41,7 +41,7 @@ inline hipError_t launch_kernel(void (*kernel)(Params...), int grid, int block, 
 hipError_t launch_flat(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n, int head,
                        float k, int wt_from, int grid, hipStream_t stream);
 // dst[0:n] = src[0:n], opaque bytes at any byte address; head: bytes up to dst's first 128-byte line (< workgroup size)
-hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int grid, hipStream_t stream);
+hipError_t launch_bytes(void* dst, const void* src, int64_t n, int head, int wt_from, int grid, hipStream_t stream);
 // the same pass, also writing partials[0:grid] = per-workgroup sums of squares of the stored values (postsumsq.hip);
 // grid must equal the number of tiles
 hipError_t launch_post_reduce_sumsq(int src_dt, int dst_dt, int scale, bool acc, void* dst, const void* src, int64_t n,
