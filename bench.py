@@ -1326,6 +1326,8 @@ def main() -> int:
                          "switched off")
     ap.add_argument("--no-rotating-sets", action="store_true",
                     help="skip the leg that alternates the step between two sets of buffers")
+    ap.add_argument("--rotating-sets", type=int, default=2, metavar="K",
+                    help="number of buffer sets of that leg (each set of the default workload is 2 GB)")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the leg that replays the step from a HIP graph (outside the timed region)")
     ap.add_argument("--no-torch-gpu", action="store_true",
@@ -1720,46 +1722,51 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     rotating = None
     if not args.no_rotating_sets:
         try:
-            second = {
-                "master": d_master.clone(), "ag_in": torch.empty_like(d_ag_in), "gathered": d_gathered.clone(),
-                "outs": [torch.empty_like(x) for x in d_outs], "grads": [x.clone() for x in d_grads],
-                "rs": torch.zeros_like(d_rs), "shard": d_shard.clone(),
-            }
-            chunk2 = second["rs"][r * s : (r + 1) * s]
+            n_sets = max(2, args.rotating_sets)
 
-            def step_second():
+            def more_buffers():
+                d = {"master": d_master.clone(), "ag_in": torch.empty_like(d_ag_in), "gathered": d_gathered.clone(),
+                     "outs": [torch.empty_like(x) for x in d_outs], "grads": [x.clone() for x in d_grads],
+                     "rs": torch.zeros_like(d_rs), "shard": d_shard.clone()}
+                d["chunk"] = d["rs"][r * s : (r + 1) * s]
+                return d
+
+            others = [more_buffers() for _ in range(n_sets - 1)]
+
+            def step_on(d):
                 if fused and w == 1:
-                    ok = table.copy_in_scatter_out(second["gathered"], second["outs"], second["ag_in"], second["master"])
-                    ok = ok and table.gather_in_post_reduce(second["grads"], second["rs"], second["shard"], True)
+                    ok = table.copy_in_scatter_out(d["gathered"], d["outs"], d["ag_in"], d["master"])
+                    ok = ok and table.gather_in_post_reduce(d["grads"], d["rs"], d["shard"], True)
                     if not ok:
                         raise RuntimeError("shared launch declined")
                     return
                 if fused:
-                    if not table.copy_in_scatter_out(second["gathered"], second["outs"], second["ag_in"],
-                                                     second["master"]):
+                    if not table.copy_in_scatter_out(d["gathered"], d["outs"], d["ag_in"], d["master"]):
                         raise RuntimeError("copy_in_scatter_out declined")
                 else:
                     if has_copy_in:
-                        _native.flat_copy(second["ag_in"], second["master"])
-                    table.scatter_out(second["gathered"], second["outs"])
-                table.gather_in(second["grads"], second["rs"], None, pre, True)
-                _native.post_reduce(second["shard"], chunk2, None, True)
+                        _native.flat_copy(d["ag_in"], d["master"])
+                    table.scatter_out(d["gathered"], d["outs"])
+                table.gather_in(d["grads"], d["rs"], None, pre, True)
+                _native.post_reduce(d["shard"], d["chunk"], None, True)
 
-            def alternating_ms_per_step(n_pairs):
-                for _ in range(max(1, warmup // 2)):
+            def alternating_ms_per_step(n_rounds):
+                for _ in range(max(1, warmup // n_sets)):
                     step()
-                    step_second()
+                    for d in others:
+                        step_on(d)
                 torch.cuda.synchronize()
                 q0 = time.perf_counter()
-                for _ in range(n_pairs):
+                for _ in range(n_rounds):
                     step()
-                    step_second()
+                    for d in others:
+                        step_on(d)
                 torch.cuda.synchronize()
-                return (time.perf_counter() - q0) / (2 * n_pairs) * 1e3
+                return (time.perf_counter() - q0) / (n_sets * n_rounds) * 1e3
 
             # under the store policy in force (the library's default unless options were given), under the policy
             # that fully_shard selects for several parameter groups, and with every store non-temporal
-            n_pairs = max(steps, 1000) // 2
+            n_pairs = max(steps, 1000) // n_sets
             in_force = _native.get_store_policy()
             rot_ms = alternating_ms_per_step(n_pairs)
             try:
@@ -1777,13 +1784,13 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
                 return {"ms_per_step": round(ms, 4), "value": round(bytes_per_step / ms / 1e6, 1), "unit": "GB/s",
                         "frac_of_hbm_peak": round(bytes_per_step / ms / 1e6 / HBM_PEAK_GBS, 4)}
 
-            rotating = {"sets": 2, "steps": 2 * n_pairs, "store_policy_in_force": list(in_force), **rate(rot_ms),
+            rotating = {"sets": n_sets, "steps": n_sets * n_pairs, "store_policy_in_force": list(in_force), **rate(rot_ms),
                         "store_policy_rotating_sets": rate(rot_policy_ms),
                         "all_stores_non_temporal": rate(rot_plain_ms)}
-            log(f"two buffer sets in rotation: {rotating['ms_per_step']} ms per step, {rotating['value']} GB/s; "
+            log(f"{n_sets} buffer sets in rotation: {rotating['ms_per_step']} ms per step, {rotating['value']} GB/s; "
                 f"under the rotating-sets store policy {rot_policy_ms:.4f} ms, all stores non-temporal "
                 f"{rot_plain_ms:.4f} ms")
-            del second, chunk2
+            del others
         except Exception as exc:  # an optional leg must not cost the measurement above
             log(f"rotating-sets leg skipped: {type(exc).__name__}: {exc}")
             rotating = None
@@ -2101,7 +2108,7 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         "sustained": sustained,
         "reference_stream_placement": reference_streams,
         "without_write_through_tails": tail_off,
-        "two_buffer_sets_in_rotation": rotating,
+        "buffer_sets_in_rotation": rotating,
         "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
         "kernels": kernels,
         "kernel_variants": variants,
