@@ -39,11 +39,20 @@ def _view_at(x: torch.Tensor, offset: int, fill: float = 3.0) -> tuple[torch.Ten
     return buf, view
 
 
+tables = st.lists(st.one_of(st.just(0), st.integers(1, 40), st.integers(1, 6000)), min_size=1, max_size=40)
+# which stores write through (flat kernels, post-reduce, scatter-out tail, gather-in tail, in megabytes from the end
+# of the output): the tables here are smaller than a megabyte, so every kind of kernel runs either all write-through
+# or all non-temporal
+ALL_MB = 1 << 20
+policies = st.sampled_from([(ALL_MB, ALL_MB, 0, 96), (0, 0, 0, 128), (0, 0, 0, 0), (ALL_MB, ALL_MB, ALL_MB, ALL_MB)])
+
+
 @settings(max_examples=120 * SCALE, **COMMON)
 @given(src_dt=st.sampled_from(DTYPES), dst_dt=st.sampled_from(DTYPES), n=st.integers(0, 70_000),
        s_off=st.integers(0, 8), d_off=st.integers(0, 8), factor=st.sampled_from(FACTORS), acc=st.booleans(),
-       seed=st.integers(0, 2**20))
-def test_post_reduce_any_shape(nat, src_dt, dst_dt, n, s_off, d_off, factor, acc, seed):
+       seed=st.integers(0, 2**20), policy=policies)
+def test_post_reduce_any_shape(nat, src_dt, dst_dt, n, s_off, d_off, factor, acc, seed, policy):
+    nat.set_store_policy(policy)
     print("post_reduce", src_dt, dst_dt, n, s_off, d_off, factor, acc, seed, flush=True)
     g = torch.Generator().manual_seed(seed)
     chunk = mixed_values(g, n, src_dt, 1e-3)
@@ -58,13 +67,13 @@ def test_post_reduce_any_shape(nat, src_dt, dst_dt, n, s_off, d_off, factor, acc
     assert float(guard.min()) == 3.0 and float(guard.max()) == 3.0
 
 
-tables = st.lists(st.one_of(st.just(0), st.integers(1, 40), st.integers(1, 6000)), min_size=1, max_size=40)
 
 
 @settings(max_examples=80 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), grad_dt=st.sampled_from(DTYPES), rs_dt=st.sampled_from(DTYPES),
-       pre=st.sampled_from(FACTORS), two_waves=st.booleans(), zero_pad=st.booleans(), seed=st.integers(0, 2**20))
-def test_gather_in_any_table(nat, numels, pad, grad_dt, rs_dt, pre, two_waves, zero_pad, seed):
+       pre=st.sampled_from(FACTORS), two_waves=st.booleans(), zero_pad=st.booleans(), seed=st.integers(0, 2**20), policy=policies)
+def test_gather_in_any_table(nat, numels, pad, grad_dt, rs_dt, pre, two_waves, zero_pad, seed, policy):
+    nat.set_store_policy(policy)
     print("gather_in", numels, pad, grad_dt, rs_dt, pre, two_waves, zero_pad, seed, flush=True)
     rng = np.random.default_rng(seed)
     g = torch.Generator().manual_seed(seed)
@@ -99,8 +108,9 @@ def test_gather_in_any_table(nat, numels, pad, grad_dt, rs_dt, pre, two_waves, z
 
 @settings(max_examples=80 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), flat_dt=st.sampled_from(DTYPES), out_dt=st.sampled_from(DTYPES),
-       two_waves=st.booleans(), bound=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2))
-def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bound, seed, tile_mode):
+       two_waves=st.booleans(), bound=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2), policy=policies)
+def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bound, seed, tile_mode, policy):
+    nat.set_store_policy(policy)
     print("scatter_out", numels, pad, flat_dt, out_dt, two_waves, bound, seed, tile_mode, flush=True)
     rng = np.random.default_rng(seed)
     g = torch.Generator().manual_seed(seed)
@@ -136,8 +146,9 @@ def test_scatter_out_any_table(nat, numels, pad, flat_dt, out_dt, two_waves, bou
 
 @settings(max_examples=80 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), master_dt=st.sampled_from(DTYPES), param_dt=st.sampled_from(DTYPES),
-       shard_n=st.integers(0, 9000), two_waves=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2))
-def test_copy_in_scatter_out_any_table(nat, numels, pad, master_dt, param_dt, shard_n, two_waves, seed, tile_mode):
+       shard_n=st.integers(0, 9000), two_waves=st.booleans(), seed=st.integers(0, 2**20), tile_mode=st.integers(0, 2), policy=policies)
+def test_copy_in_scatter_out_any_table(nat, numels, pad, master_dt, param_dt, shard_n, two_waves, seed, tile_mode, policy):
+    nat.set_store_policy(policy)
     """Copy-in and copy-out as one launch: both halves with their guard lanes against the oracle."""
     print("copy_in_scatter_out", numels, pad, master_dt, param_dt, shard_n, two_waves, seed, tile_mode, flush=True)
     rng = np.random.default_rng(seed)
@@ -176,8 +187,9 @@ def test_copy_in_scatter_out_any_table(nat, numels, pad, master_dt, param_dt, sh
 @settings(max_examples=100 * SCALE, **COMMON)
 @given(numels=tables, pad=st.integers(0, 700), grad_dt=st.sampled_from(DTYPES), wide_buffer=st.booleans(),
        shard_dt=st.sampled_from(DTYPES), acc=st.booleans(), two_waves=st.booleans(), zero_pad=st.booleans(),
-       seed=st.integers(0, 2**20))
-def test_gather_in_post_reduce_any_table(nat, numels, pad, grad_dt, wide_buffer, shard_dt, acc, two_waves, zero_pad, seed):
+       seed=st.integers(0, 2**20), policy=policies)
+def test_gather_in_post_reduce_any_table(nat, numels, pad, grad_dt, wide_buffer, shard_dt, acc, two_waves, zero_pad, seed, policy):
+    nat.set_store_policy(policy)
     """Reduce copy-in and post-reduce of a size-one group as one launch: the reduce buffer (guard lanes included)
     and the gradient shard against the reference's op sequence."""
     rs_dt = torch.float32 if wide_buffer else grad_dt
@@ -222,8 +234,9 @@ def test_gather_in_post_reduce_any_table(nat, numels, pad, grad_dt, wide_buffer,
        beta1=st.sampled_from([0.9, 0.5, 0.3, 0.0]), beta2=st.sampled_from([0.95, 0.999, 0.5]),
        wd=st.sampled_from([0.0, 0.1, 1e-2]), lr=st.sampled_from([3e-4, 1e-2, 0.0]), step=st.integers(1, 2000),
        out_dt=st.sampled_from([None, torch.bfloat16, torch.float16]), gscale=st.sampled_from([None, 0.5, 0.19153, 1.0]),
-       zero_grad=st.booleans(), seed=st.integers(0, 2**20))
-def test_adamw_any_shape(nat, n, off, decoupled, beta1, beta2, wd, lr, step, out_dt, gscale, zero_grad, seed):
+       zero_grad=st.booleans(), seed=st.integers(0, 2**20), policy=policies)
+def test_adamw_any_shape(nat, n, off, decoupled, beta1, beta2, wd, lr, step, out_dt, gscale, zero_grad, seed, policy):
+    nat.set_store_policy(policy)
     from oracle import cref
 
     print("adamw", n, off, decoupled, beta1, beta2, wd, lr, step, out_dt, gscale, zero_grad, seed, flush=True)
@@ -252,8 +265,9 @@ def test_adamw_any_shape(nat, n, off, decoupled, beta1, beta2, wd, lr, step, out
 
 @settings(max_examples=60 * SCALE, **COMMON)
 @given(dt=st.sampled_from(DTYPES), n=st.integers(0, 300_000), off=st.integers(0, 8),
-       coef=st.sampled_from([1.0, 0.5, 0.19153, 3.0]), seed=st.integers(0, 2**20))
-def test_sumsq_fill_scale_any_shape(nat, dt, n, off, coef, seed):
+       coef=st.sampled_from([1.0, 0.5, 0.19153, 3.0]), seed=st.integers(0, 2**20), policy=policies)
+def test_sumsq_fill_scale_any_shape(nat, dt, n, off, coef, seed, policy):
+    nat.set_store_policy(policy)
     import math
 
     from oracle import cref
@@ -279,8 +293,9 @@ def test_sumsq_fill_scale_any_shape(nat, dt, n, off, coef, seed):
 
 @settings(max_examples=60 * SCALE, **COMMON)
 @given(src_dt=st.sampled_from(DTYPES), dst_dt=st.sampled_from(DTYPES), n=st.integers(0, 60_000),
-       k=st.integers(1, 16), seed=st.integers(0, 2**20))
-def test_fanout_any_shape(nat, src_dt, dst_dt, n, k, seed):
+       k=st.integers(1, 16), seed=st.integers(0, 2**20), policy=policies)
+def test_fanout_any_shape(nat, src_dt, dst_dt, n, k, seed, policy):
+    nat.set_store_policy(policy)
     print("fanout", src_dt, dst_dt, n, k, seed, flush=True)
     g = torch.Generator().manual_seed(seed)
     src = mixed_values(g, n, src_dt)
@@ -294,8 +309,9 @@ def test_fanout_any_shape(nat, src_dt, dst_dt, n, k, seed):
 
 @settings(max_examples=60 * SCALE, **COMMON)
 @given(chunk_dt=st.sampled_from(DTYPES), shard_dt=st.sampled_from(DTYPES), n=st.integers(0, 60_000),
-       k=st.integers(1, 16), post=st.sampled_from(FACTORS), acc=st.booleans(), seed=st.integers(0, 2**20))
-def test_fanin_any_shape(nat, chunk_dt, shard_dt, n, k, post, acc, seed):
+       k=st.integers(1, 16), post=st.sampled_from(FACTORS), acc=st.booleans(), seed=st.integers(0, 2**20), policy=policies)
+def test_fanin_any_shape(nat, chunk_dt, shard_dt, n, k, post, acc, seed, policy):
+    nat.set_store_policy(policy)
     print("fanin", chunk_dt, shard_dt, n, k, post, acc, seed, flush=True)
     g = torch.Generator().manual_seed(seed)
     chunks = [mixed_values(g, n, chunk_dt, 1e-3).roll(i) for i in range(k)]
