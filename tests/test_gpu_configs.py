@@ -52,8 +52,17 @@ def nat():
     return _native
 
 
-def test_config2_llama8b_layer_w8(nat):
-    print("config 2", flush=True)
+@pytest.fixture(params=["single_set", "rotating_sets", "tails_on_both_table_kernels"])
+def store_policy(request, nat):
+    """Which stores write through: at these sizes the boundary between the two kinds of stores lies inside the
+    buffers (the conftest fixture restores the library's defaults before the next test)."""
+    named = {"tails_on_both_table_kernels": (1 << 20, 1 << 20, 32, 56)}
+    nat.set_store_policy(named.get(request.param, request.param))
+    return request.param
+
+
+def test_config2_llama8b_layer_w8(nat, store_policy):
+    print("config 2", store_policy, flush=True)
     numels = [_numel(s) for s in LLAMA8B]
     w = 8
     lay = make_layout(numels, w, 512)
@@ -173,7 +182,7 @@ def _stress_numels(seed=1005, p=2000):
 
 
 @pytest.mark.parametrize("which", ["fp32-masters/bf16-compute", "bf16-masters/fp32-reduce"])
-def test_config5_ragged_stress_w256(nat, which):
+def test_config5_ragged_stress_w256(nat, which, store_policy):
     print("config 5", which, flush=True)
     all_numels, is_fp32 = _stress_numels()
     if which.startswith("fp32"):
