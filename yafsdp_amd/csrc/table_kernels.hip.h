@@ -277,6 +277,14 @@ __device__ __forceinline__ void gather_segment(char* dst, const char* src, int64
 }
 
 // Tile handled by workgroup b: b itself, or the XCD-aware permutation inside windows of kWin tiles.
+// a full tile of gather-in under the (wave-uniform) mode of its tensor; a skipped tensor's lanes still see the divide
+template <class S, class D, int SCALE, int BLOCK, int U, bool NTL, int STP>
+__device__ __forceinline__ void gather_full_tile_by_mode(int mode, char* dst, const char* src, float k) {
+  if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, STP>(dst, src, k);
+  else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, STP>(dst, src, k);
+  else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, STP>(dst, src, k);
+}
+
 template <int kX, int kWin>
 __device__ __forceinline__ int tile_of_block(int b) {
   if constexpr (kX == 1) return b;
@@ -313,15 +321,10 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
       const int mode = rec.mode;
       const char* src = reinterpret_cast<const char*>(rec.base) + rec.delta * S::kSize;
       char* dst = fbase + t0 * D::kSize;
-      if (STP == ST_NT && tile >= wt_from) {  // the end of the buffer writes through (see tuning.h)
-        if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, ST_WT>(dst, src, k);
-        else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, ST_WT>(dst, src, k);
-        else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, ST_WT>(dst, src, k);
-        continue;
-      }
-      if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, STP>(dst, src, k);
-      else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, STP>(dst, src, k);
-      else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, STP>(dst, src, k);
+      if (STP == ST_NT && tile >= wt_from)  // the end of the buffer writes through (see tuning.h)
+        gather_full_tile_by_mode<S, D, SCALE, BLOCK, U, NTL, ST_WT>(mode, dst, src, k);
+      else
+        gather_full_tile_by_mode<S, D, SCALE, BLOCK, U, NTL, STP>(mode, dst, src, k);
       continue;
     }
     int64_t pos = t0;
