@@ -76,15 +76,16 @@ constexpr int kScatterShortUnroll = 1;
 constexpr int kTableXcd = YAFSDP_TABLE_XCD;
 constexpr int kTableXcdRun = YAFSDP_TABLE_XCD_RUN;
 constexpr bool kTableNtLoad = YAFSDP_TABLE_NTL;
-// scatter-out reads the flat buffer.  On the short tile (every tensor starts on a cache line of the flat buffer)
-// each line is read once and the loads are non-temporal like everywhere else.  On the long tile the tensors sit at
-// odd offsets, every tile shares its first and last line with a neighbour, and ordinary loads let the L2 keep that
-// line for the other one: copy-out of a 573-tensor table as a launch of its own 108.6 -> 104.1 us (step +0.5 %); in
-// the shared launch of a 1427-tensor table the step is level.  Ordinary loads in gather-in as well move time from
-// one kernel of the step to the next without shortening the step (1427 tensors: copy-out 237 -> 232 us, reduce
-// copy-in 230 -> 236 us), so gather-in keeps non-temporal loads.
+// scatter-out reads the flat buffer with non-temporal loads on both tile shapes, like every other kernel.  On the
+// long tile (tensors at odd offsets: every tile shares its first and last line with a neighbour) ordinary loads let
+// the L2 keep the shared line and are 0.5-0.7 % faster by themselves (573-tensor table, copy-out as a launch of its
+// own 107 -> 105 us), but what they read also passes through the memory-side cache and evicts the written-through
+// end of the reduce buffer that the store policy below keeps there: with that tail the step of the 573-tensor group
+// takes 0.2773 ms with ordinary loads and 0.2685 ms with non-temporal ones (0.2718 without any tail), that of the
+// 1427-tensor group 0.4778 and 0.4727 ms (0.4742).  Ordinary loads in gather-in move time from one kernel of the step
+// to the next without shortening the step (1427 tensors: copy-out 237 -> 232 us, reduce copy-in 230 -> 236 us).
 #ifndef YAFSDP_SCATTER_LONG_NTL
-#define YAFSDP_SCATTER_LONG_NTL false
+#define YAFSDP_SCATTER_LONG_NTL true
 #endif
 constexpr bool scatter_nt_load(int unroll) {
   return unroll == 1 ? bool(YAFSDP_TABLE_NTL) : bool(YAFSDP_SCATTER_LONG_NTL);
