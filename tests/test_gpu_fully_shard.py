@@ -675,3 +675,6 @@ def test_store_policy_follows_the_number_of_parameter_groups(monkeypatch):
     monkeypatch.setenv("YAFSDP_STORE_POLICY", "rotating_sets")
     fully_shard(Block(128, 256).to(DEV), mp_policy=MP)(x).float().pow(2).mean().backward()
     assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"]
+    monkeypatch.setenv("YAFSDP_STORE_POLICY", "fastest")
+    with pytest.raises(ValueError, match="YAFSDP_STORE_POLICY"):
+        fully_shard(Block(128, 256).to(DEV), mp_policy=MP)(x)

@@ -247,6 +247,10 @@ class YaFSDPState(_State):
         # default), and the written-through end of each survives until its next visit if all of them fit the cache
         # together (measured with 2, 3 and 4 buffers in rotation: 128, 85, 64 MB each).
         policy = os.environ.get("YAFSDP_STORE_POLICY", "auto")
+        if policy not in ("auto", "keep", *_native.STORE_POLICIES):
+            raise ValueError(
+                f"YAFSDP_STORE_POLICY={policy!r}: expected auto, keep or one of {sorted(_native.STORE_POLICIES)}"
+            )
         if policy == "auto":
             if len(param_groups) == 1:
                 policy = "single_set"
