@@ -110,6 +110,22 @@ int yafsdp_flat_div_copy(void* dst, int dst_dtype, const void* src, int src_dtyp
 int yafsdp_post_reduce(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
                        double post_factor, int accumulate, void* stream);
 
+/* This rank's share of a reduce-scatter whose reduction scales inside the collective
+ * (ya_fsdp/_collectives.py:243-249: ReduceOp.AVG, or _make_nccl_premul_sum(1 / factor), handed to
+ * dist.reduce_scatter_tensor at :152-162).  The collective library defines both as a PRE-MULTIPLIED sum
+ * (ncclRedOpCreatePreMulSum; ncclAvg on floating-point data uses the scalar 1 / nRanks): the scalar is converted to
+ * the data type, and every rank's element is multiplied by it and rounded to the data type before the sum.  It
+ * is not a division: x * round(1 / f) and x / f differ when f is no power of two.
+ *   k = round_dtype(float(scalar))
+ *   yafsdp_flat_premul:         buf[i] = round_dtype(buf[i] * k)                       (in place)
+ *   yafsdp_post_reduce_premul:  t = round_chunk_dtype(chunk[i] * k);
+ *                               shard[i] = round_shard_dtype(accumulate ? shard[i] + t : t)
+ * i.e. the collective's share fused with padded_sharded_param_grad.copy_ (:185) / .add_ (:189); the chunk is not
+ * written.  Any finite scalar is applied (there is no "> 1" rule inside the collective). */
+int yafsdp_flat_premul(void* buf, int dtype, int64_t n, double scalar, void* stream);
+int yafsdp_post_reduce_premul(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
+                              double scalar, int accumulate, void* stream);
+
 /* yafsdp_post_reduce that also returns the sum of squares of the shard it
  * writes, as per-workgroup partial sums in binary64 (squares of binary32
  * numbers are exact there): the gradient norm of clip_grad_norm_
@@ -378,7 +394,7 @@ int yafsdp_time_next_launch(void* start_event, void* stop_event);
  * grid size if it exceeded `capacity` (then nothing is traced).  Consumed by one launch; NULL disarms. */
 int yafsdp_trace_next_flat_launch(uint64_t* trace, int64_t capacity, int64_t* n_workgroups);
 
-/* Launch-shape knobs (process-wide, for measurement): */
+/* Launch-shape and store-policy options (process-wide): */
 typedef enum yafsdp_option {
   YAFSDP_OPT_FLAT_BLOCKS_PER_CU = 0,  /* workgroups per compute unit of the flat kernels' grid */
   YAFSDP_OPT_TABLE_BLOCKS_PER_CU = 1, /* same for gather-in / scatter-out */
@@ -388,34 +404,40 @@ typedef enum yafsdp_option {
                                          layout (short 512-element tiles when every tensor starts on a 128-byte
                                          line of the flat buffer, the gather-in tile otherwise), 1 = always
                                          short, 2 = never short */
-  YAFSDP_OPT_GATHER_TAIL_MB = 4,      /* 0..2^20, default 96: yafsdp_gather_in / yafsdp_gather_in_bound write the last
+  YAFSDP_OPT_GATHER_TAIL_MB = 4,      /* 0..2^20, default 64: yafsdp_gather_in / yafsdp_gather_in_bound write the last
                                          `value` megabytes of the flat buffer through the L2s instead of leaving
                                          them there as dirty lines (a store-policy choice; the bytes written are
                                          the same).  The memory-side cache absorbs them and writes them back
-                                         later: the kernel ends sooner, and whatever runs next pays for the
-                                         write-back only if it saturates the memory itself from its first
-                                         microsecond.  0 = off */
+                                         later: the kernel ends with clean L2s, and the lines are still in that
+                                         256-MB cache when the buffer is read again soon.  0 = off */
   YAFSDP_OPT_SCATTER_TAIL_MB = 5,     /* 0..2^20, default 0: the same for the tile slots of the last `value`
                                          megabytes of tensors in yafsdp_scatter_out / yafsdp_scatter_out_bound /
-                                         yafsdp_copy_in_scatter_out.  What one kernel wrote through the next
-                                         may have to evict: with 32 here and 56 for the reduce copy-in a step of
-                                         the two is 0.8 % shorter and the reduce copy-in itself 3 % longer */
-  YAFSDP_OPT_FLAT_TAIL_MB = 6,        /* 0..2^20, default 2^20 (everything): the same for yafsdp_flat_copy,
-                                         yafsdp_flat_copy_bytes, yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
-                                         yafsdp_copy_in_scatter_out, which write through everywhere by default;
-                                         0 = they store everything non-temporal */
+                                         yafsdp_copy_in_scatter_out */
+  YAFSDP_OPT_FLAT_TAIL_MB = 6,        /* 0..2^20, default 0: the same for yafsdp_flat_copy, yafsdp_flat_copy_bytes,
+                                         yafsdp_flat_div, yafsdp_flat_div_copy and the cast part of
+                                         yafsdp_copy_in_scatter_out; 2^20 = they write through everywhere */
   YAFSDP_OPT_POST_REDUCE_TAIL_MB = 7  /* the same for yafsdp_post_reduce / yafsdp_post_reduce_sumsq /
                                          yafsdp_post_reduce_fragments.
                                          Written-through lines pay if they are still in the 256-MB memory-side
                                          cache when their buffer is read or written again, and cost if they are
-                                         evicted in the middle of other kernels.  The defaults of options 4-7 suit
-                                         a caller that rewrites ONE set of buffers step after step.  A caller whose
-                                         parameter groups take turns on shared buffers, with one gradient buffer
-                                         for all groups as in the reference, is served best by 0 / 0 / 0 / 128 for
-                                         options 6 / 7 / 5 / 4 (the end of the buffer that comes round soonest) */
+                                         evicted in the middle of other kernels.  The defaults of options 4-7
+                                         (64 / 0 / 0 / 0) are cache-neutral: they suit parameter groups that take
+                                         turns on shared buffers (up to four reduce buffers in rotation; with ONE
+                                         gradient buffer for all groups, as in the reference, 128 for option 4 is
+                                         better still).  A caller that rewrites ONE set of buffers in a loop gains
+                                         2-4 % from 96 / 0 / 2^20 / 2^20 (the loop then finds its own output in
+                                         that cache, which a training run does not) */
 } yafsdp_option;
 int yafsdp_set_option(int option, int value);
 int yafsdp_get_option(int option, int* value);
+/* The same two store-policy options for ONE table (YAFSDP_OPT_GATHER_TAIL_MB, YAFSDP_OPT_SCATTER_TAIL_MB; every
+ * other option is refused): the table's own value, 0..2^20, takes precedence over the process-wide one in every
+ * call on this table; -1 (the state a table is created in) follows the process-wide option again.  How soon a
+ * flat buffer comes round again is a property of the parameter group that owns it (how many gradient buffers its
+ * model rotates through), not of the process: two models in one process keep their own settings this way.
+ * No counterpart in the reference (its ops take no cache policy). */
+int yafsdp_table_set_option(yafsdp_table* table, int option, int value);
+int yafsdp_table_get_option(const yafsdp_table* table, int option, int* value);
 
 #ifdef __cplusplus
 }

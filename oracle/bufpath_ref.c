@@ -115,6 +115,20 @@ void ref_flat_div(void* buf, int dt, int64_t n, double factor) {
   for (int64_t i = 0; i < n; i++) store_f(buf, dt, i, load_f(buf, dt, i) / f);
 }
 
+/* One rank's contribution to a reduce-scatter whose reduction is a pre-multiplied
+ * sum (ya_fsdp/_collectives.py:243-249, 152-162: ReduceOp.AVG or
+ * _make_nccl_premul_sum(1 / factor) handed to dist.reduce_scatter_tensor).  The
+ * collective library (NCCL / RCCL, not part of the reference's tree) defines the
+ * op as: the scalar is converted to the data type, every rank's input element is
+ * multiplied by it and the product rounded to the data type BEFORE the sum
+ * (ncclRedOpCreatePreMulSum); ncclAvg on floating-point data is that op with the
+ * scalar 1/nRanks.  Not a division: for a factor that is no power of two
+ * x * round(1/f) and x / f differ. */
+void ref_flat_premul(void* buf, int dt, int64_t n, double scalar) {
+  const float k = round_to(dt, (float)scalar);
+  for (int64_t i = 0; i < n; i++) store_f(buf, dt, i, load_f(buf, dt, i) * k);
+}
+
 /* chunk.div_(post) [rounds to the chunk dtype]; then shard.copy_(chunk) or
  * shard.add_(chunk) [binary32 add, rounds to the shard dtype]. The chunk itself
  * is left unmodified here (it is scratch in the reference after this point). */

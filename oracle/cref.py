@@ -35,6 +35,8 @@ def lib() -> ctypes.CDLL:
         L.ref_flat_copy.argtypes = [vp, i32, vp, i32, i64]
         L.ref_flat_div.restype = None
         L.ref_flat_div.argtypes = [vp, i32, i64, dbl]
+        L.ref_flat_premul.restype = None
+        L.ref_flat_premul.argtypes = [vp, i32, i64, dbl]
         L.ref_post_reduce.restype = None
         L.ref_post_reduce.argtypes = [vp, i32, vp, i32, i64, dbl, i32]
         L.ref_gather_in.restype = None
@@ -68,6 +70,11 @@ def flat_div(buf: torch.Tensor, factor: float | None) -> None:
     if factor is None:
         return
     lib().ref_flat_div(buf.data_ptr(), DT[buf.dtype], buf.numel(), float(factor))
+
+
+def flat_premul(buf: torch.Tensor, scalar: float) -> None:
+    _check(buf)
+    lib().ref_flat_premul(buf.data_ptr(), DT[buf.dtype], buf.numel(), float(scalar))
 
 
 def post_reduce(shard: torch.Tensor, chunk: torch.Tensor, post: float | None, accumulate: bool) -> None:

@@ -114,6 +114,35 @@ def get_gradient_divide_factors(
     return pre_factor, post_factor, "SUM", None
 
 
+def reduce_scatter_one_rank_share(
+    output_tensor: torch.Tensor, op: str, world_size: int, premul: float | None = None
+) -> None:
+    """What ``dist.reduce_scatter_tensor(output, input, op=...)`` (ya_fsdp/_collectives.py:152-162) does to ONE
+    rank's contribution, for the three ops ``_get_gradient_divide_factors`` can return (:243-249, 267), applied in
+    place to this rank's chunk (the only contribution there is on one GPU).
+
+    The arithmetic lives in the collective library (NCCL, RCCL on ROCm; a dependency of torch, not part of the
+    reference's tree and not pinned by it).  Its published definition: ``ncclRedOpCreatePreMulSum(scalar)`` converts
+    the scalar to the data type, multiplies every rank's input element by it and rounds the product to the data
+    type *before* the sum; ``ncclAvg`` on floating-point data is that same op with the scalar ``1 / nRanks``
+    (integers: sum, then divide); ``ncclSum`` leaves a single contribution as it is.  torch hands
+    ``_make_nccl_premul_sum(1 / factor)`` over as that scalar cast to the tensor's dtype.  So neither op divides:
+    for a group size or factor that is no power of two ``x * round(1 / f)`` differs from ``x / f``."""
+    if op == "SUM":
+        return
+    if op == "AVG":
+        scalar = 1.0 / world_size
+    elif op == "PREMUL_SUM":
+        assert premul is not None
+        scalar = premul
+    else:
+        raise ValueError(op)
+    # binary64 -> binary32 -> data type, then an elementwise product of two tensors of that type (computed in
+    # binary32, where the product of two 16-bit values is exact, and rounded once to the data type)
+    k = torch.tensor(scalar, dtype=torch.float64).to(torch.float32).to(output_tensor.dtype)
+    output_tensor.mul_(torch.full_like(output_tensor, k.item()))
+
+
 def reduce_scatter_local(
     padded_sharded_param_grad: torch.Tensor,
     padded_unsharded_param_grad: torch.Tensor,
@@ -124,6 +153,7 @@ def reduce_scatter_local(
     mode: str,
     sharded_numels: Sequence[int] | None = None,
     fragment_has_sharded_grad: Sequence[bool | None] | None = None,
+    collective: "tuple[str, float | None] | None" = None,
 ) -> torch.Tensor:
     """ya_fsdp/_collectives.py:124-214 for the branch that goes through the
     reduce buffer (``reduce_in_sharded`` false), with the inter-GPU collective
@@ -132,9 +162,12 @@ def reduce_scatter_local(
 
     ``mode``: "copy" (:185), "add" (:189) or "mixed" (:191-214).  For "mixed",
     ``fragment_has_sharded_grad[p]`` is True (accumulate), False (copy) or None
-    (parameter produced no gradient: fragment untouched)."""
+    (parameter produced no gradient: fragment untouched).  ``collective``: ``(op, premul)`` of the reduce-scatter
+    (``reduce_scatter_one_rank_share``); None leaves the chunk as it is (a sum of one contribution)."""
     div_if_needed(padded_unsharded_param_grad, predivide_factor)  # :139
     output_tensor = padded_unsharded_param_grad.chunk(world_size)[rank]  # :127-129
+    if collective is not None:
+        reduce_scatter_one_rank_share(output_tensor, collective[0], world_size, collective[1])  # :152-162
     div_if_needed(output_tensor, postdivide_factor)  # :165
     if mode == "copy":
         padded_sharded_param_grad.copy_(output_tensor)  # :185

@@ -25,10 +25,10 @@ def pytest_collection_modifyitems(config, items):
 
 @pytest.fixture(autouse=True)
 def _library_default_store_policy(request):
-    """fully_shard picks the library's store policy from the number of parameter groups (process-wide options): every
-    GPU test starts from the library's own defaults, whatever model the test before it built."""
+    """Tests set the library's process-wide store-policy options: every GPU test starts from the library's own
+    defaults, whatever the test before it chose."""
     if "gpu" in request.keywords:
         from yafsdp_amd import _native
 
-        _native.set_store_policy("single_set")
+        _native.set_store_policy("rotating_sets")
     yield

@@ -30,7 +30,7 @@ def test_library_exports_every_symbol():
     import __graft_entry__
 
     assert _native.lib.yafsdp_version() // 1000 == __graft_entry__.ABI_MAJOR  # what build() checks
-    assert _native.lib.yafsdp_version() == 1005  # 1.1: yafsdp_flat_copy_bytes; 1.2-1.5: the four write-through tail options
+    assert _native.lib.yafsdp_version() == 1006  # 1.1: yafsdp_flat_copy_bytes; 1.2-1.5: the four write-through tail options; 1.6: per-table tails, pre-multiplied share
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
 
@@ -49,6 +49,13 @@ def test_argument_validation_without_gpu():
     # empty ranges are fine whatever their pointers (torch hands out null for empty tensors)
     assert L.yafsdp_post_reduce(None, 1, None, 0, 0, 8.0, 1, None) == 0
     assert L.yafsdp_flat_div_copy(None, 1, None, 0, 0, 3.0, None) == 0
+    assert L.yafsdp_flat_premul(None, 1, 0, 1.0 / 3, None) == 0
+    assert L.yafsdp_flat_premul(None, 7, 0, 0.5, None) == -2
+    assert L.yafsdp_flat_premul(None, 1, 4, 0.5, None) == -1
+    assert L.yafsdp_flat_premul(None, 1, 0, float("inf"), None) == -1  # no finite scalar in the data type
+    assert L.yafsdp_post_reduce_premul(None, 0, None, 1, 0, 0.2, 1, None) == 0
+    assert L.yafsdp_post_reduce_premul(None, 0, None, 1, 4, 0.2, 1, None) == -1
+    assert L.yafsdp_table_set_option(None, 4, 64) == -1
     assert L.yafsdp_set_option(99, 1) == -1
     assert L.yafsdp_set_option(0, 0) == -1
     assert L.yafsdp_set_option(2, 63) == -1
@@ -58,19 +65,19 @@ def test_argument_validation_without_gpu():
     assert L.yafsdp_set_option(4, -1) == -1
     assert L.yafsdp_set_option(4, (1 << 20) + 1) == -1
     tail = ctypes.c_int(-1)
-    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 96
+    assert L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 64
     assert L.yafsdp_set_option(4, 0) == 0 and L.yafsdp_get_option(4, ctypes.byref(tail)) == 0 and tail.value == 0
-    assert L.yafsdp_set_option(4, 96) == 0
+    assert L.yafsdp_set_option(4, 64) == 0
     assert L.yafsdp_set_option(5, -1) == -1
     assert L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 0
     assert L.yafsdp_set_option(5, 7) == 0 and L.yafsdp_get_option(5, ctypes.byref(tail)) == 0 and tail.value == 7
     assert L.yafsdp_set_option(5, 0) == 0
-    assert L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 1 << 20
-    assert L.yafsdp_set_option(6, 0) == 0 and L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 0
-    assert L.yafsdp_set_option(6, 1 << 20) == 0
-    assert L.yafsdp_get_option(7, ctypes.byref(tail)) == 0 and tail.value == 1 << 20
+    assert L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 0
+    assert L.yafsdp_set_option(6, 1 << 20) == 0 and L.yafsdp_get_option(6, ctypes.byref(tail)) == 0 and tail.value == 1 << 20
+    assert L.yafsdp_set_option(6, 0) == 0
+    assert L.yafsdp_get_option(7, ctypes.byref(tail)) == 0 and tail.value == 0
     assert L.yafsdp_set_option(7, 5) == 0 and L.yafsdp_get_option(7, ctypes.byref(tail)) == 0 and tail.value == 5
-    assert L.yafsdp_set_option(7, 1 << 20) == 0
+    assert L.yafsdp_set_option(7, 0) == 0
     assert L.yafsdp_set_option(8, 1) == -1
     assert L.yafsdp_gather_in(None, None, None, 0, None, 0, 0.0, 1, None) == -1
     assert L.yafsdp_table_destroy(None) == 0
@@ -112,11 +119,12 @@ def test_store_policies_set_the_four_tail_options():
 
     from yafsdp_amd import _native
 
-    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"] == (1 << 20, 1 << 20, 0, 96)
+    # the library's own defaults are the cache-neutral policy; the one tuned to a loop over one buffer set is opt-in
+    assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"] == (0, 0, 0, 64)
     try:
-        _native.set_store_policy("rotating_sets")
-        assert _native.get_store_policy() == (0, 0, 0, 128)
-        assert _native.get_option(_native.OPT_GATHER_TAIL_MB) == 128
+        _native.set_store_policy("single_set")
+        assert _native.get_store_policy() == (1 << 20, 1 << 20, 0, 96)
+        assert _native.get_option(_native.OPT_GATHER_TAIL_MB) == 96
         _native.set_store_policy((5, 6, 7, 8))
         assert _native.get_store_policy() == (5, 6, 7, 8)
         with pytest.raises(KeyError):
@@ -124,4 +132,4 @@ def test_store_policies_set_the_four_tail_options():
         with pytest.raises(ValueError):
             _native.set_store_policy((1, 2, 3))
     finally:
-        _native.set_store_policy("single_set")
+        _native.set_store_policy("rotating_sets")

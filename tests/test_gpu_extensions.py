@@ -140,12 +140,13 @@ def test_classes_unshard_and_reduce(w, r, align):
         group.post_backward()
         group.finalize_backward()
         torch.cuda.synchronize()
-        # bf16 reduce: the division by W happens "inside the collective"; on one GPU a post-divide of the rank's chunk
-        post = float(w) if w > 1 else None
+        # bf16 reduce: ReduceOp.AVG, i.e. the collective multiplies every contribution by 1 / W rounded to bf16
+        collective = ("AVG", None) if w > 1 else None
         for key, ref in ((None, plain), (torch.int8, ext)):
             mine = [gr for gr, (_, e) in zip(grads, MIXED) if e == (key is not None)]
             torch_ops.reduce_copy_in(ref.rs_views, mine, False)
-            torch_ops.reduce_scatter_local(ref.grad_shard, ref.rs, w, r, None, post, "copy" if step == 0 else "add")
+            torch_ops.reduce_scatter_local(ref.grad_shard, ref.rs, w, r, None, None, "copy" if step == 0 else "add",
+                                           collective=collective)
             assert_bits_equal(group._padded_sharded_param_grad[key], ref.grad_shard, f"gradient shard {key} pass {step}")
         for fp in group.fsdp_params:
             assert fp.sharded_param.grad is fp.sharded_param_grad

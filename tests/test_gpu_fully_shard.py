@@ -649,32 +649,42 @@ def test_torch_adamw_and_clip_grad_norm_on_the_sharded_parameters(impl):
     assert torch.equal(y, twin_model.to(torch.bfloat16)(xs[0].to(torch.bfloat16)))
 
 
-def test_store_policy_follows_the_number_of_parameter_groups(monkeypatch):
-    """Which stores write through is a process-wide choice of the library; fully_shard makes it when the root is
-    initialised: several groups take turns on the shared buffers (little of what one writes is still cached when its
-    buffer comes round again), a single group rewrites its own.  Either way the same bits (every other test)."""
+def test_store_policy_follows_the_number_of_gradient_buffers(monkeypatch):
+    """How much of a reduce buffer's end is stored write-through is chosen per parameter group when the root is
+    initialised, from the number of gradient buffers that take turns (the tables of the group carry it); the
+    process-wide options are the application's and stay as they are.  Either way the same bits (every other test)."""
     from yafsdp_amd import _native, fully_shard
 
+    def tails(model):
+        out = set()
+        for state in model._get_fsdp_state()._state_ctx.all_states:
+            if (group := state._fsdp_param_group) is not None:
+                out |= {t.get_option(_native.OPT_GATHER_TAIL_MB) for t in group._tables.values()}
+        return out
+
     x = torch.randn(4, 128, device=DEV)
-    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"]  # the library's defaults
-    model = _wrap(_make(61), mp_policy=MP)  # four groups
+    defaults = _native.get_store_policy()
+    assert defaults == _native.STORE_POLICIES["rotating_sets"]  # the library's defaults
+    model = _wrap(_make(61), mp_policy=MP)  # four groups, one gradient buffer
     model(x).float().pow(2).mean().backward()
-    assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"]
+    assert tails(model) == {128} and _native.get_store_policy() == defaults
     # a gradient buffer per group (gradient accumulation without reduction): four buffers take turns
-    model = _wrap(_make(63), mp_policy=MP)
-    model._get_fsdp_state()._lazy_init(allow_no_grad_reduce=True)
-    assert _native.get_store_policy() == (0, 0, 0, 64)
+    many = _wrap(_make(63), mp_policy=MP)
+    many._get_fsdp_state()._lazy_init(allow_no_grad_reduce=True)
+    many(x).float().pow(2).mean().backward()
+    assert tails(many) == {64} and tails(model) == {128}  # two models in one process keep their own
     single = fully_shard(Block(128, 256).to(DEV), mp_policy=MP)  # one group
     single(x).float().pow(2).mean().backward()
-    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"]
-    # the environment can fix the policy or leave the options alone
+    assert tails(single) == {128} and _native.get_store_policy() == defaults
+    # the environment can leave everything alone, or make an explicit process-wide choice
     monkeypatch.setenv("YAFSDP_STORE_POLICY", "keep")
     _native.set_store_policy((1, 2, 3, 4))
-    _wrap(_make(62), mp_policy=MP)(x).float().pow(2).mean().backward()
-    assert _native.get_store_policy() == (1, 2, 3, 4)
-    monkeypatch.setenv("YAFSDP_STORE_POLICY", "rotating_sets")
+    kept = _wrap(_make(62), mp_policy=MP)
+    kept(x).float().pow(2).mean().backward()
+    assert _native.get_store_policy() == (1, 2, 3, 4) and tails(kept) == {-1}
+    monkeypatch.setenv("YAFSDP_STORE_POLICY", "single_set")
     fully_shard(Block(128, 256).to(DEV), mp_policy=MP)(x).float().pow(2).mean().backward()
-    assert _native.get_store_policy() == _native.STORE_POLICIES["rotating_sets"]
+    assert _native.get_store_policy() == _native.STORE_POLICIES["single_set"]
     monkeypatch.setenv("YAFSDP_STORE_POLICY", "fastest")
     with pytest.raises(ValueError, match="YAFSDP_STORE_POLICY"):
         fully_shard(Block(128, 256).to(DEV), mp_policy=MP)(x)

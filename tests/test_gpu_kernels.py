@@ -140,6 +140,80 @@ def test_post_reduce(nat, shard_dt, chunk_dt, post, acc):
         assert_bits_equal(got, want, "post_reduce")
 
 
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("scalar", [1 / 3, 1 / 5, 1 / 6, 1 / 8, 0.5, 1.0, 2.0, 1 / 1000, 1 / 7])
+def test_flat_premul(nat, dt, scalar):
+    """One rank's share of the collective's pre-multiplied sum, in place."""
+    g = torch.Generator().manual_seed(141)
+    for n, off in [(4099, 0), (20_000, 3)]:
+        _say("flat_premul", dt, scalar, n, off)
+        x = mixed_values(g, n + off, dt, std=1e-3)
+        want = x.clone()
+        torch_ops.reduce_scatter_one_rank_share(want[off:], "PREMUL_SUM", 8, scalar)
+        got = x.to(DEV)
+        nat.flat_premul(got[off:], scalar)
+        assert_bits_equal(got, want, f"premul {dt} {scalar}")
+
+
+@pytest.mark.parametrize("shard_dt", DTYPES)
+@pytest.mark.parametrize("chunk_dt", DTYPES)
+@pytest.mark.parametrize("op,w,factor", [("AVG", 3, None), ("AVG", 6, None), ("AVG", 8, None), ("PREMUL_SUM", 8, 3.0),
+                                         ("PREMUL_SUM", 6, 5.0)])
+@pytest.mark.parametrize("acc", [False, True])
+def test_post_reduce_premul(nat, shard_dt, chunk_dt, op, w, factor, acc):
+    g = torch.Generator().manual_seed(142)
+    premul = None if factor is None else 1 / factor
+    for n, off in [(5, 0), (8192 * 2 + 11, 0), (30_001, 1)]:
+        _say("post_reduce_premul", shard_dt, chunk_dt, op, w, factor, acc, n, off)
+        chunk = mixed_values(g, n + off, chunk_dt, std=1e-3)
+        shard0 = mixed_values(g, n + off, shard_dt, std=1e-4).flip(0).contiguous()
+        want = shard0.clone()
+        torch_ops.reduce_scatter_local(want[off:], chunk.clone()[off:], 1, 0, None, None, "add" if acc else "copy",
+                                       collective=(op, premul) if op == "PREMUL_SUM" else None)
+        if op == "AVG":  # (the oracle's AVG takes the scalar from the group size: restate it with that size)
+            want = shard0.clone()
+            scaled = chunk.clone()
+            torch_ops.reduce_scatter_one_rank_share(scaled[off:], "AVG", w)
+            torch_ops.reduce_scatter_local(want[off:], scaled[off:], 1, 0, None, None, "add" if acc else "copy")
+        got = shard0.to(DEV)
+        d_chunk = chunk.to(DEV)
+        nat.post_reduce_premul(got[off:], d_chunk[off:], 1.0 / w if op == "AVG" else premul, acc)
+        assert_bits_equal(got, want, "post_reduce_premul")
+        assert_bits_equal(d_chunk, chunk, "the chunk is not written")
+
+
+def test_per_table_write_through_tail(nat):
+    """A table's own tail option takes precedence over the process-wide one, changes no byte, and -1 hands the
+    choice back."""
+    g = torch.Generator().manual_seed(143)
+    numels = [300_001, 7, 1_200_000, 65]
+    t = sum(numels)
+    t_pad = t + 183
+    grads = [mixed_values(g, n, torch.bfloat16, std=1e-3) for n in numels]
+    want = torch.zeros(t_pad, dtype=torch.bfloat16)
+    torch_ops.reduce_copy_in(list(want[:t].split(numels)), grads, False)
+    torch_ops.div_if_needed(want, 8.0)
+    table = nat.TensorTable(numels, t_pad, DEV)
+    d_grads = [x.to(DEV) for x in grads]
+    assert table.get_option(nat.OPT_GATHER_TAIL_MB) == -1 and table.get_option(nat.OPT_SCATTER_TAIL_MB) == -1
+    for mb in (0, 1, 2, 1 << 20, -1):  # 3 MB of output: the boundary lies inside the buffer for 1 and 2
+        _say("per-table gather tail", mb)
+        table.set_option(nat.OPT_GATHER_TAIL_MB, mb)
+        assert table.get_option(nat.OPT_GATHER_TAIL_MB) == mb
+        got = torch.full((t_pad,), 9.0, dtype=torch.bfloat16, device=DEV)
+        table.gather_in(d_grads, got, None, 8.0, True)
+        assert_bits_equal(got, want, f"gather_in with a table tail of {mb} MB")
+        table.set_option(nat.OPT_SCATTER_TAIL_MB, mb)
+        outs = [torch.empty(n, dtype=torch.bfloat16, device=DEV) for n in numels]
+        table.scatter_out(got, outs)
+        for a, b in zip(outs, want[:t].split(numels)):
+            assert_bits_equal(a, b, f"scatter_out with a table tail of {mb} MB")
+    with pytest.raises(RuntimeError):
+        table.set_option(nat.OPT_FLAT_TAIL_MB, 1)  # only the two table kernels' tails are per table
+    assert nat.get_store_policy() == nat.STORE_POLICIES["rotating_sets"]  # the process-wide options were not touched
+    table.close()
+
+
 @pytest.mark.parametrize("tail_mb", [0, 1, 3])
 def test_flat_kernels_with_the_write_through_boundary_inside_the_buffer(nat, tail_mb):
     """The flat kernels write through everywhere by default; with a tail option below the size of the output the

@@ -82,9 +82,10 @@ class CpuGroup:
         torch_ops.reduce_copy_in([self.rs_views[i] for i in cp], [grads[i] for i in cp], False)
         torch_ops.reduce_copy_in([self.rs_views[i] for i in ad], [grads[i] for i in ad], True)
 
-    def reduce(self, pre, post, mode, has=None):
+    def reduce(self, pre, post, mode, has=None, collective=None):
         torch_ops.reduce_scatter_local(
-            self.grad_shard, self.rs, self.w, self.r, pre, post, mode, self.lay.sharded_numels(self.r), has
+            self.grad_shard, self.rs, self.w, self.r, pre, post, mode, self.lay.sharded_numels(self.r), has,
+            collective=collective,
         )
 
 
@@ -144,23 +145,66 @@ def test_backward_reduce_copy_then_accumulate(shapes, w, r, align, force_sum):
     group, cpu_params = _make_group(shapes, w, r, align, BF16_MP)
     group.force_sum_reduction_for_comms = force_sum
     ref = CpuGroup(cpu_params, w, r, align, BF16_MP)
-    # bf16 reduce: (None, None, AVG) -> the division by W happens "inside the collective";
-    # force_sum -> (None, W, SUM).  On one GPU both are a post-divide by W of the rank's chunk.
-    post = float(w) if w > 1 else None
+    # bf16 reduce: (None, None, AVG) -> the scaling by 1/W happens inside the collective (a pre-multiplied sum);
+    # force_sum -> (None, W, SUM): a post-divide by W of the rank's chunk.
+    post = float(w) if w > 1 and force_sum else None
+    collective = ("AVG", None) if w > 1 and not force_sum else None
     for it in range(2):
         group.pre_forward(); group.post_forward(); group.pre_backward()
         ref.unshard(first_of_iteration=True)
         grads = _grads(shapes, torch.bfloat16, 10 + it)
         _run_backward(group, ref, grads)
-        ref.reduce(None, post, "copy" if it == 0 else "add")
+        ref.reduce(None, post, "copy" if it == 0 else "add", collective=collective)
         group.finalize_backward()
         torch.cuda.synchronize()
-        if post is None:  # with a post-divide the reference also rewrites its (scratch) chunk in place
+        if post is None and collective is None:  # otherwise the reference also rewrites its (scratch) chunk in place
             assert_bits_equal(group._reduce_scatter_input[None], ref.rs, "reduce buffer")
         assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, f"grad shard after backward {it}")
         for fp in group.fsdp_params:
             assert fp.sharded_param.grad is fp.sharded_param_grad
         assert group.grad_buffer_ctx.owner is None and group._training_state.name == "IDLE"
+
+
+@pytest.mark.parametrize("w,r", [(3, 1), (6, 5), (8, 3)])
+@pytest.mark.parametrize("factor", [None, 3.0, 5.0, "w"])
+@pytest.mark.parametrize("reduce_dtype", [torch.bfloat16, torch.float32])
+def test_collective_scaling_at_group_sizes_above_one(w, r, factor, reduce_dtype):
+    """ya_fsdp/_collectives.py:243-249 for a bf16 / fp32 reduce without forced sum: no factor or factor == W ->
+    ReduceOp.AVG, any other factor -> _make_nccl_premul_sum(1 / factor).  Both scale every contribution inside the
+    collective by the reciprocal ROUNDED TO THE REDUCE DTYPE (a product, not a division: W = 3, 6 and factors 3, 5
+    tell the two apart).  First backward copies into the gradient shard, second accumulates, third leaves two
+    parameters without gradient (fragment-wise path, which reads the chunk the collective left)."""
+    shapes, align = ODD_SHAPES, 8
+    mp = MixedPrecisionPolicy(param_dtype=torch.bfloat16, reduce_dtype=reduce_dtype)
+    group, cpu_params = _make_group(shapes, w, r, align, mp)
+    f = float(w) if factor == "w" else factor
+    group.gradient_divide_factor = f
+    ref = CpuGroup(cpu_params, w, r, align, mp)
+    pre, post, op, premul = torch_ops.get_gradient_divide_factors(w, reduce_dtype, f, False)
+    assert (pre, post) == (None, None) and op == ("AVG" if f in (None, float(w)) else "PREMUL_SUM")
+    for it in range(3):
+        group.pre_forward(); group.post_forward(); group.pre_backward()
+        grads = _grads(shapes, torch.bfloat16, 90 + it)
+        if it == 2:
+            grads[0] = None; grads[6] = None
+        _run_backward(group, ref, grads)
+        if it < 2:
+            ref.reduce(None, None, "copy" if it == 0 else "add", collective=(op, premul))
+        else:
+            ref.reduce(None, None, "mixed", [None if g is None else True for g in grads], collective=(op, premul))
+        group.finalize_backward()
+        torch.cuda.synchronize()
+        assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, f"grad shard after backward {it}")
+    # the fragment-wise path leaves the collective's result in this rank's chunk, as the reference does (compared on
+    # the fragments whose parameters had a gradient: the others hold leftovers of earlier passes, which the
+    # reference scales once more in place and the fused launches of the earlier passes never wrote back)
+    s = ref.lay.padded_sharded_numel
+    mine, theirs = group._reduce_scatter_input[None][r * s : (r + 1) * s], ref.rs[r * s : (r + 1) * s]
+    pos = 0
+    for n, g_ in zip(ref.lay.sharded_numels(r), grads):
+        if g_ is not None:
+            assert_bits_equal(mine[pos : pos + n], theirs[pos : pos + n], "chunk fragment")
+        pos += n
 
 
 def test_bit32_acc_flag_leaves_the_one_contribution_result_unchanged():
@@ -174,7 +218,7 @@ def test_bit32_acc_flag_leaves_the_one_contribution_result_unchanged():
     group.pre_forward(); group.post_forward(); group.pre_backward()
     ref.unshard()
     _run_backward(group, ref, _grads(ODD_SHAPES, torch.bfloat16, 77))
-    ref.reduce(None, float(w), "copy")
+    ref.reduce(None, None, "copy", collective=("AVG", None))
     group.finalize_backward()
     torch.cuda.synchronize()
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
@@ -191,7 +235,7 @@ def test_gradient_accumulation_without_sync_uses_add():
     _run_backward(group, ref, _grads(shapes, torch.bfloat16, 21), reduce=False)   # add, no reduce
     group.pre_backward()
     _run_backward(group, ref, _grads(shapes, torch.bfloat16, 22), reduce=True)    # add, then reduce
-    ref.reduce(None, float(w), "copy")
+    ref.reduce(None, None, "copy", collective=("AVG", None))
     group.finalize_backward()
     torch.cuda.synchronize()
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
@@ -307,14 +351,14 @@ def test_mixed_params_with_and_without_sharded_grad(monkeypatch):
     g1[1] = None; g1[4] = None                      # two params get no gradient in the first backward
     _run_backward(group, ref, g1)
     has = [None if g is None else False for g in g1]
-    ref.reduce(None, float(w), "mixed", has)        # partial first reduction goes through the fragment path
+    ref.reduce(None, None, "mixed", has, collective=("AVG", None))        # partial first reduction goes through the fragment path
     group.finalize_backward()
     group.pre_forward(); group.post_forward(); group.pre_backward()
     ref.unshard()
     g2 = _grads(shapes, torch.bfloat16, 31)
     _run_backward(group, ref, g2)
     has2 = [g is not None for g in g1]              # params that already own a sharded grad accumulate
-    ref.reduce(None, float(w), "mixed", has2)
+    ref.reduce(None, None, "mixed", has2, collective=("AVG", None))
     group.finalize_backward()
     torch.cuda.synchronize()
     assert_bits_equal(group._padded_sharded_param_grad[None], ref.grad_shard, "grad shard")
@@ -348,7 +392,7 @@ def test_bf16_masters_fp32_reduce():
     for it in range(2):
         group.pre_forward(); group.post_forward(); group.pre_backward()
         _run_backward(group, ref, _grads(shapes, torch.bfloat16, 50 + it))
-        ref.reduce(None, float(w), "copy" if it == 0 else "add")
+        ref.reduce(None, None, "copy" if it == 0 else "add", collective=("AVG", None))
         group.finalize_backward()
     torch.cuda.synchronize()
     assert group._padded_sharded_param_grad[None].dtype == torch.bfloat16

@@ -349,8 +349,10 @@ def test_param_group_any_layout(shapes, w, r_frac, align, policy, iterations, se
         while w % pre == 0 and w / pre > pre:
             pre *= 2
         pre, post = float(pre), float(w / pre)
-    else:                 # AVG inside the collective: this rank's share is its chunk divided by W
-        pre, post = None, (float(w) if w > 1 else None)
+        collective = None
+    else:                 # AVG inside the collective: this rank's share is its chunk times 1 / W rounded to the dtype
+        pre, post = None, None
+        collective = ("AVG", None) if w > 1 else None
     group, cpu_params = _make_group(shapes, w, r, align, mp, seed=seed % 1000)
     ref = CpuGroup(cpu_params, w, r, align, mp)
     rng = np.random.default_rng(seed)
@@ -369,11 +371,12 @@ def test_param_group_any_layout(shapes, w, r_frac, align, policy, iterations, se
         _run_backward(group, ref, grads)
         with_grad = [i for i, x in enumerate(grads) if x is not None]
         if all(not owns[i] for i in with_grad) and len(with_grad) == len(shapes):
-            ref.reduce(pre, post, "copy")
+            ref.reduce(pre, post, "copy", collective=collective)
         elif all(owns[i] for i in with_grad) and len(with_grad) == len(shapes):
-            ref.reduce(pre, post, "add")
+            ref.reduce(pre, post, "add", collective=collective)
         else:
-            ref.reduce(pre, post, "mixed", [None if x is None else owns[i] for i, x in enumerate(grads)])
+            ref.reduce(pre, post, "mixed", [None if x is None else owns[i] for i, x in enumerate(grads)],
+                       collective=collective)
         for i in with_grad:
             owns[i] = True
         group.finalize_backward()
@@ -417,7 +420,7 @@ def test_param_group_with_all_gather_dtype_classes(spec, w, r_frac, align, itera
     keys = {k: idx for k, idx in keys.items() if idx}
     assert list(group._all_gather_dtype_to_fsdp_params) == list(keys)
     refs = {k: CpuGroup([values[i] for i in idx], w, r, align, BF16_MP) for k, idx in keys.items()}
-    post = float(w) if w > 1 else None
+    collective = ("AVG", None) if w > 1 else None  # bf16 reduce: the collective scales by 1 / W rounded to bf16
     rng = np.random.default_rng(seed)
     owns = [False] * len(spec)
     for it in range(iterations):
@@ -455,11 +458,12 @@ def test_param_group_with_all_gather_dtype_classes(spec, w, r_frac, align, itera
             ref.accumulate(mine, [False] * len(mine))
             with_grad = [j for j, x in enumerate(mine) if x is not None]
             if all(not mine_owns[j] for j in with_grad) and len(with_grad) == len(mine):
-                ref.reduce(None, post, "copy")
+                ref.reduce(None, None, "copy", collective=collective)
             elif all(mine_owns[j] for j in with_grad) and len(with_grad) == len(mine):
-                ref.reduce(None, post, "add")
+                ref.reduce(None, None, "add", collective=collective)
             else:
-                ref.reduce(None, post, "mixed", [None if x is None else mine_owns[j] for j, x in enumerate(mine)])
+                ref.reduce(None, None, "mixed", [None if x is None else mine_owns[j] for j, x in enumerate(mine)],
+                           collective=collective)
         for i, x in enumerate(grads):
             if x is not None:
                 owns[i] = True

@@ -197,3 +197,86 @@ def test_mixed_fragments():
     want[7:127] = q[7:127].float()
     assert_bits_equal(shard, want, "mixed")
     assert_bits_equal(shard[127:], shard0[127:], "untouched fragments and pad")
+
+
+# ---- the collective's own scaling for group sizes above one (ya_fsdp/_collectives.py:243-249, 152-162) ----------
+def _scalar_in(dt, scalar):
+    """The pre-multiplier as the collective sees it: binary64 -> binary32 -> data type (by integer arithmetic for
+    bf16, numpy for fp16), as a binary64 number."""
+    f = np.float32(scalar)
+    if dt == torch.float32:
+        return float(f)
+    if dt == torch.float16:
+        return float(np.float16(f))
+    bits = _bf16_closed_form(np.array([f], dtype=np.float32).view(np.uint32))
+    return float((bits.astype(np.uint32) << 16).view(np.float32)[0])
+
+
+def test_premul_scalars_hand_checked():
+    # 1/3 = 0.0101010101...b: binary32 0x3EAAAAAB (rounded up), bf16 0x3EAB, fp16 0x3555
+    assert np.array([_scalar_in(torch.float32, 1 / 3)], dtype=np.float32).view(np.uint32)[0] == 0x3EAAAAAB
+    assert _scalar_in(torch.bfloat16, 1 / 3) == 0.333984375        # 0x3EAB
+    assert _scalar_in(torch.float16, 1 / 3) == 0.333251953125      # 0x3555
+    for dt, three_thirds in ((torch.bfloat16, 1.0), (torch.float16, 1.0), (torch.float32, 1.0)):
+        # 3 * round(1/3) lies within half an ulp of 1 in all three types
+        x = torch.tensor([1.0, 3.0, -3.0, 0.0], dtype=dt)
+        torch_ops.reduce_scatter_one_rank_share(x, "AVG", 3)
+        assert x.double().tolist() == [_scalar_in(dt, 1 / 3), three_thirds, -three_thirds, 0.0]
+    # a case where multiplying by the rounded reciprocal and dividing part ways, by hand:
+    # bf16 7.0 * 0.333984375 = 2.337890625 -> between 2.328125 (0x4015) and 2.34375 (0x4016), nearer the latter;
+    # 7 / 3 = 2.3333... -> nearer 2.328125
+    x = torch.tensor([7.0], dtype=torch.bfloat16)
+    torch_ops.reduce_scatter_one_rank_share(x, "PREMUL_SUM", 8, 1 / 3)
+    assert x.item() == 2.34375 and (torch.tensor([7.0], dtype=torch.bfloat16) / 3).item() == 2.328125
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("op,w,factor", [("AVG", 3, None), ("AVG", 6, None), ("AVG", 8, None), ("AVG", 7, None),
+                                         ("PREMUL_SUM", 8, 3.0), ("PREMUL_SUM", 6, 5.0), ("PREMUL_SUM", 3, 0.5),
+                                         ("PREMUL_SUM", 4, 1000.0), ("SUM", 8, None)])
+def test_one_rank_share_of_the_collective_is_a_rounded_product(dt, op, w, factor):
+    g = torch.Generator().manual_seed(17)
+    x = mixed_values(g, 1 << 15, dt, std=1e-3)
+    premul = None if factor is None else 1 / factor  # what _make_nccl_premul_sum receives (:249)
+    a = x.clone()
+    torch_ops.reduce_scatter_one_rank_share(a, op, w, premul)
+    if op == "SUM":
+        assert_bits_equal(a, x, "a sum of one contribution")
+        return
+    scalar = 1.0 / w if op == "AVG" else premul
+    b = x.clone()
+    cref.flat_premul(b, scalar)
+    assert_bits_equal(a, b, "pre-multiplied share: torch vs C")
+    # independent: the binary64 product of two binary32 numbers is exact (48 <= 53 bits), so rounding it once to
+    # binary32 gives the correctly rounded binary32 product; for the 16-bit types that product is already exact in
+    # binary32 and the one rounding is the cast to the type
+    k = _scalar_in(dt, scalar)
+    want = (x.double() * k).float().to(dt)
+    finite = torch.isfinite(x.float()) & torch.isfinite(want.float())
+    assert_bits_equal(a[finite], want[finite], "pre-multiplied share vs float64")
+    # and it is NOT the division that a sum followed by "/ factor" would give, unless the factor is a power of two
+    f = float(w) if op == "AVG" else factor
+    d = x.clone()
+    d.div_(f)
+    differs = int(((a.view(torch.int16 if dt != torch.float32 else torch.int32)
+                    != d.view(torch.int16 if dt != torch.float32 else torch.int32)) & finite).sum())
+    if f in (0.5, 8.0):
+        assert differs == 0
+    else:
+        assert differs > 100, (op, w, factor, differs)
+
+
+def test_reduce_scatter_local_applies_the_collective_between_the_two_divides():
+    """pre-divide (:139) on the whole buffer, the collective's share (:152-162) and the post-divide (:165) on the
+    chunk, then the accumulation (:189): every step rounds to the reduce dtype."""
+    g = torch.Generator().manual_seed(19)
+    w, r, s = 3, 1, 1 << 12
+    rs = mixed_values(g, w * s, torch.bfloat16, std=1e-3, specials=False)
+    shard0 = mixed_values(g, s, torch.float32, std=1e-4, specials=False)
+    shard, buf = shard0.clone(), rs.clone()
+    out = torch_ops.reduce_scatter_local(shard, buf, w, r, None, None, "add", collective=("AVG", None))
+    k = _scalar_in(torch.bfloat16, 1 / 3)
+    chunk = (rs[r * s : (r + 1) * s].double() * k).float().to(torch.bfloat16)
+    assert_bits_equal(out, chunk, "the chunk after the collective")
+    assert_bits_equal(shard, (shard0.double() + chunk.double()).float(), "gradient shard")
+    assert_bits_equal(buf[:s], rs[:s], "other ranks' chunks are left alone")

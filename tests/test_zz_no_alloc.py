@@ -28,11 +28,15 @@ def _sumsq_pair(lib, src, accumulate, start):
     gc.collect()
     gc.disable()
     try:
+        # the driver's own count of free device memory sees a hipMalloc inside the library; torch's statistics
+        # (its caching allocator's) would not
+        before_free, _ = torch.cuda.mem_get_info(DEV)
         before = torch.cuda.memory_allocated(DEV)
         rc = lib.yafsdp_flat_sumsq_static(src.data_ptr(), dt, src.numel(), got.data_ptr(), int(accumulate), stream)
         assert rc == 0, lib.yafsdp_error_string(rc)
         torch.cuda.synchronize()
         assert torch.cuda.memory_allocated(DEV) == before
+        assert torch.cuda.mem_get_info(DEV)[0] == before_free
     finally:
         gc.enable()
     return want, got
@@ -46,6 +50,10 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
     big = (torch.randn(3_000_001, generator=g) * 1e-2).to(DEV)
     small = (torch.randn(70_003, generator=g) * 3.0).bfloat16().to(DEV)
     with torch.cuda.device(DEV):
+        # the first call on a device performs the set-up (the scratch's address is looked up): before the
+        # readings of free memory below, which the first use of a code object may move
+        assert lib.yafsdp_flat_sumsq_static(None, 0, 0, None, 0, None) == 0
+        _sumsq_pair(lib, small[:64], False, 0.0)
         # two calls in a row, the second with a smaller input of another dtype: whatever the first call left in
         # the shared scratch must not leak into the second
         want, got = _sumsq_pair(lib, big, False, 123.0)
@@ -59,6 +67,11 @@ def test_static_scratch_entry_point_matches_the_workspace_one():
         assert torch.equal(want.view(torch.int64), got.view(torch.int64))
         want, got = _sumsq_pair(lib, small[:5], True, 0.5)
         assert torch.equal(want.view(torch.int64), got.view(torch.int64))
+        # nothing to add: the output becomes 0, or keeps its value when accumulating, from both entry points
+        want, got = _sumsq_pair(lib, small[:0], False, 7.0)
+        assert float(want) == 0.0 and float(got) == 0.0
+        want, got = _sumsq_pair(lib, small[:0], True, 7.0)
+        assert float(want) == 7.0 and float(got) == 7.0
 
 
 def test_static_scratch_entry_point_limits():

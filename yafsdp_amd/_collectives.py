@@ -194,7 +194,7 @@ def reduce_scatter(
         )  # :112-123
         shard_numel = padded_unsharded_param_grad.numel() // world_size
         chunk = padded_unsharded_param_grad[rank * shard_numel : (rank + 1) * shard_numel]  # :127-129
-        predivide_factor, postdivide_factor, reduce_scatter_op, premul = _get_gradient_divide_factors(
+        predivide_factor, postdivide_factor, reduce_scatter_op, premul_scalar = _get_gradient_divide_factors(
             reduce_scatter_group,
             reduce_dtype or param_dtype or orig_dtype,
             gradient_divide_factor,
@@ -213,25 +213,26 @@ def reduce_scatter(
             elif reduce_in_sharded:
                 _native.flat_copy(output_tensor, padded_unsharded_param_grad)  # :150
             # else: output aliases the reduce buffer, copy_ onto itself is a no-op (:150)
-            collective_divide = None
+            premul = None
         else:
-            # this rank's share of reduce_scatter_tensor (:152-162): its chunk, divided as the
-            # collective would have (AVG: by the group size; pre-multiplied sum: by the factor)
+            # this rank's share of reduce_scatter_tensor (:152-162): its chunk, scaled as the collective scales
+            # every contribution.  AVG and the pre-multiplied sum are one op in the collective library
+            # (ncclRedOpCreatePreMulSum; ncclAvg on floating-point data uses 1 / nRanks): the scalar is converted to
+            # the data type and each contribution is multiplied by it, rounded, before the sum - a product with the
+            # rounded reciprocal, not a division (they differ unless the factor is a power of two).
             if yccl_handle is not None:
                 yccl_handle.reduce_scatter(padded_unsharded_param_grad.view(torch.bfloat16))  # :163-164
             if reduce_scatter_op == "AVG":
-                collective_divide = float(world_size)
+                premul = 1.0 / world_size
             elif reduce_scatter_op == "PREMUL_SUM":
-                collective_divide = float(gradient_divide_factor)
+                premul = premul_scalar  # 1 / gradient_divide_factor, :249
             else:
-                collective_divide = None
-            if collective_divide is not None and collective_divide <= 1 and collective_divide != 1:
-                # a pre-multiplier >= 1 is outside the "> 1" rule of the fused divide: apply it on its own
-                _native.flat_div_copy(chunk, chunk, collective_divide)
-                collective_divide = None
+                premul = None
             output_tensor = chunk
-        # post-divide (:165) fused with the copy / accumulate into the gradient shard (:166-214)
-        post = postdivide_factor if collective_divide is None else collective_divide
+        # post-divide (:165), or the collective's own scaling, fused with the copy / accumulate into the gradient
+        # shard (:166-214); the reference never has both (a scaling collective comes with postdivide_factor None)
+        post = postdivide_factor
+        assert premul is None or post is None
         group_ref = getattr(fsdp_params[0], "_param_group_ref", None) if fsdp_params else None
         param_group = group_ref() if group_ref is not None else None
         # every parameter of the group gets a gradient in this pass: the whole shard is meaningful afterwards
@@ -241,7 +242,7 @@ def reduce_scatter(
             param_group._grad_sumsq_token.pop(cls_key, None)
         if world_size > 1 and reduce_in_sharded:
             # the collective would have written straight into the shard (:124-125)
-            _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, chunk, post, False)
+            _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, chunk, post, False, premul)
         elif world_size == 1 and reduce_in_sharded:
             _div_if_needed(padded_sharded_param_grad, post)
         else:
@@ -249,9 +250,9 @@ def reduce_scatter(
             without_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is None]
             with_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is not None]
             if len(without_sharded_grad) == len(fsdp_params_which_require_grad):
-                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, False)  # :185
+                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, False, premul)  # :185
             elif len(with_sharded_grad) == len(fsdp_params_which_require_grad):
-                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, True)  # :189
+                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, True, premul)  # :189
             else:
                 with_ids = {id(p) for p in with_sharded_grad}
                 without_ids = {id(p) for p in without_sharded_grad}
@@ -260,6 +261,8 @@ def reduce_scatter(
                     for p in fsdp_params
                 ]
                 numels = [p.sharded_numel for p in fsdp_params]
+                if premul is not None:
+                    _native.flat_premul(output_tensor, premul)  # the collective leaves its result in the chunk
                 if param_group is None:
                     _native.post_reduce_fragments(padded_sharded_param_grad, output_tensor, numels, modes, post)
                 else:
@@ -277,16 +280,22 @@ def reduce_scatter(
 
 def _post_reduce(
     param_group: "YaFSDPParamGroup | None", cls_key: Any, whole: bool, shard: torch.Tensor, chunk: torch.Tensor,
-    post: float | None, accumulate: bool,
+    post: float | None, accumulate: bool, premul: float | None = None,
 ) -> None:
     """``post_reduce`` of one all-gather dtype class of a group; for a class
     with a slot for partial sums of squares (``optim.enable_fused_grad_norm``)
     and a pass that gives every parameter of it its gradient, the variant that
-    also leaves the squared norm of the shard."""
+    also leaves the squared norm of the shard.  ``premul``: the scalar of a
+    collective that scales inside the reduction (then there is no post-divide)."""
     slot = param_group._grad_sumsq_slot.get(cls_key) if param_group is not None else None
     if slot is None or not whole:
-        _native.post_reduce(shard, chunk, post, accumulate)
+        if premul is not None:
+            _native.post_reduce_premul(shard, chunk, premul, accumulate)
+        else:
+            _native.post_reduce(shard, chunk, post, accumulate)
         return
+    if premul is not None:
+        _native.flat_premul(chunk, premul)
     lo, hi = slot
     end = _native.post_reduce_sumsq(shard, chunk, post, accumulate, param_group._grad_sumsq_partials[:hi], lo)
     if end < hi:  # the slot is added up as a whole: entries a read pass may have left beyond these sums go

@@ -44,6 +44,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_flat_div",
     "yafsdp_flat_div_copy",
     "yafsdp_post_reduce",
+    "yafsdp_flat_premul",
+    "yafsdp_post_reduce_premul",
     "yafsdp_post_reduce_sumsq_count",
     "yafsdp_post_reduce_sumsq",
     "yafsdp_post_reduce_fragments",
@@ -75,6 +77,8 @@ EXPORTED_SYMBOLS = (
     "yafsdp_trace_next_flat_launch",
     "yafsdp_set_option",
     "yafsdp_get_option",
+    "yafsdp_table_set_option",
+    "yafsdp_table_get_option",
 )
 
 
@@ -100,6 +104,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_flat_div_copy.argtypes = [vp, i32, vp, i32, i64, dbl, vp]
     lib.yafsdp_post_reduce.restype = i32
     lib.yafsdp_post_reduce.argtypes = [vp, i32, vp, i32, i64, dbl, i32, vp]
+    lib.yafsdp_flat_premul.restype = i32
+    lib.yafsdp_flat_premul.argtypes = [vp, i32, i64, dbl, vp]
+    lib.yafsdp_post_reduce_premul.restype = i32
+    lib.yafsdp_post_reduce_premul.argtypes = [vp, i32, vp, i32, i64, dbl, i32, vp]
     lib.yafsdp_post_reduce_sumsq_count.restype = i64
     lib.yafsdp_post_reduce_sumsq_count.argtypes = [i64]
     lib.yafsdp_post_reduce_sumsq.restype = i32
@@ -162,6 +170,10 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_set_option.argtypes = [i32, i32]
     lib.yafsdp_get_option.restype = i32
     lib.yafsdp_get_option.argtypes = [i32, ctypes.POINTER(i32)]
+    lib.yafsdp_table_set_option.restype = i32
+    lib.yafsdp_table_set_option.argtypes = [vp, i32, i32]
+    lib.yafsdp_table_get_option.restype = i32
+    lib.yafsdp_table_get_option.argtypes = [vp, i32, ctypes.POINTER(i32)]
     return lib
 
 
@@ -280,6 +292,33 @@ def post_reduce(shard: torch.Tensor, chunk: torch.Tensor, post_factor: float | N
         )
 
 
+def flat_premul(buf: torch.Tensor, scalar: float) -> None:
+    """``buf *= dtype(scalar)`` in place, rounded to the dtype: one rank's share of a pre-multiplied sum (what the
+    collective's AVG / ``_make_nccl_premul_sum`` reduction does to every contribution before adding them up)."""
+    _flat_arg(buf, "buf")
+    with _on(buf.device):
+        _check(
+            lib.yafsdp_flat_premul(buf.data_ptr(), _dt(buf), buf.numel(), float(scalar), _stream(buf)),
+            "yafsdp_flat_premul",
+        )
+
+
+def post_reduce_premul(shard: torch.Tensor, chunk: torch.Tensor, scalar: float, accumulate: bool) -> None:
+    """``post_reduce`` whose chunk first takes the collective's pre-multiplication (``flat_premul``) instead of a
+    post-divide; the chunk itself is not written."""
+    _flat_arg(shard, "shard"), _flat_arg(chunk, "chunk")
+    if shard.numel() != chunk.numel():
+        raise ValueError(f"numel mismatch: {shard.numel()} vs {chunk.numel()}")
+    with _on(shard.device):
+        _check(
+            lib.yafsdp_post_reduce_premul(
+                shard.data_ptr(), _dt(shard), chunk.data_ptr(), _dt(chunk), shard.numel(),
+                float(scalar), int(bool(accumulate)), _stream(shard),
+            ),
+            "yafsdp_post_reduce_premul",
+        )
+
+
 def post_reduce_sumsq_count(numel: int) -> int:
     """Partial sums ``post_reduce_sumsq`` writes at most for a shard of ``numel`` elements."""
     return int(lib.yafsdp_post_reduce_sumsq_count(int(numel)))
@@ -385,6 +424,17 @@ class TensorTable:
         h, self._handle = getattr(self, "_handle", None), None
         if h:
             lib.yafsdp_table_destroy(h)
+
+    def set_option(self, option: int, value: int) -> None:
+        """This table's own write-through tail (``OPT_GATHER_TAIL_MB`` / ``OPT_SCATTER_TAIL_MB``) in megabytes; it
+        takes precedence over the process-wide option in every call on this table.  -1: follow the process-wide
+        option again."""
+        _check(lib.yafsdp_table_set_option(self._handle, int(option), int(value)), "yafsdp_table_set_option")
+
+    def get_option(self, option: int) -> int:
+        v = ctypes.c_int()
+        _check(lib.yafsdp_table_get_option(self._handle, int(option), ctypes.byref(v)), "yafsdp_table_get_option")
+        return v.value
 
     def bind(self, tensors: Sequence[torch.Tensor | None], modes: Sequence[int] | None = None) -> "TensorBinding":
         """Fix the tensor side for many calls (see ``TensorBinding``)."""
@@ -885,14 +935,15 @@ def get_option(option: int) -> int:
 # stay in the 256-MB memory-side cache until later traffic evicts them; they pay if they are still there when their
 # buffer is touched again (a read is served from the cache, a write overwrites them before they reached DRAM) and
 # cost if they are evicted in the middle of other kernels:
-#   "single_set"     one set of buffers rewritten step after step (one parameter group; a loop over one layer): the
-#                    flat kernels write through everywhere and the reduce copy-in its last 96 MB.  The
-#                    library's own defaults.
-#   "rotating_sets"  several parameter groups taking turns on shared buffers (ya_fsdp/_state.py:636-652): the one
-#                    gradient buffer that all groups share comes round soonest, so the reduce copy-in writes its
-#                    last 128 MB through and everything else stores non-temporal.
+#   "rotating_sets"  the library's own defaults, cache-neutral: parameter groups taking turns on shared buffers
+#                    (ya_fsdp/_state.py:636-652), up to four reduce buffers in rotation.  Only the reduce copy-in
+#                    writes its last 64 MB through (the gradient buffers come round soonest); `fully_shard` sizes
+#                    that tail per group from the number of gradient buffers of its model (``TensorTable.set_option``).
+#   "single_set"     opt-in: one set of buffers rewritten step after step (a loop over one layer).  The flat kernels
+#                    write through everywhere and the reduce copy-in its last 96 MB, and the loop finds its own
+#                    output in that cache, which a training run over many groups does not.
 _EVERYTHING = 1 << 20
-STORE_POLICIES = {"single_set": (_EVERYTHING, _EVERYTHING, 0, 96), "rotating_sets": (0, 0, 0, 128)}
+STORE_POLICIES = {"rotating_sets": (0, 0, 0, 64), "single_set": (_EVERYTHING, _EVERYTHING, 0, 96)}
 _STORE_POLICY_OPTIONS = (OPT_FLAT_TAIL_MB, OPT_POST_REDUCE_TAIL_MB, OPT_SCATTER_TAIL_MB, OPT_GATHER_TAIL_MB)
 
 

@@ -245,6 +245,7 @@ class YaFSDPParamGroup:
                 fsdp_param._all_gather_class = all_gather_dtype
                 fsdp_param._index_in_class = index
         self._tables: dict[torch.dtype | None, _native.TensorTable] = {}
+        self._gather_tail_mb: int | None = None  # set_gather_tail_mb; None: the library's process-wide option
         # this rank's fragments of each class's gradient shard (built on first use, ya_fsdp/_collectives.py:191-214)
         self._fragment_tables: dict[torch.dtype | None, _native.TensorTable] = {}
         self._state_dict_hook_handles: list = []
@@ -305,6 +306,14 @@ class YaFSDPParamGroup:
     def layout(self) -> ShardLayout:
         self._default_class("layout")
         return self.layouts[None]
+
+    def set_gather_tail_mb(self, megabytes: int | None) -> None:
+        """How many megabytes at the end of this group's reduce buffer the reduce copy-in stores write-through (they
+        then sit in the memory-side cache when the post-reduce or the next group's reduce copy-in comes to the same
+        buffer).  A store-policy choice that changes no result; None follows the library's process-wide option."""
+        self._gather_tail_mb = megabytes
+        for table in self._tables.values():
+            table.set_option(_native.OPT_GATHER_TAIL_MB, -1 if megabytes is None else megabytes)
 
     @property
     def _table(self) -> "_native.TensorTable | None":
@@ -427,6 +436,8 @@ class YaFSDPParamGroup:
                     self._unsharded_param_numels[all_gather_dtype],
                     self.layouts[all_gather_dtype].padded_unsharded_numel, self.device,
                 )
+                if self._gather_tail_mb is not None:
+                    self._tables[all_gather_dtype].set_option(_native.OPT_GATHER_TAIL_MB, self._gather_tail_mb)
 
     # ------------------------------------------------------------------- runtime --
     @property

@@ -242,23 +242,22 @@ class YaFSDPState(_State):
                             None if allow_no_grad_reduce else 1, lambda g: g.grad_buffer_bytes_by_dtype(),
                             param_group_to_grad_buffer_ctx_idx, grad_buffer_ctx_idx_to_yccl_handle)
         # Which stores write through (and so stay in the 256-MB memory-side cache) depends on how soon the written
-        # buffers come round again, and this is where that is known.  A single group rewrites its own buffers step
-        # after step.  Several groups take turns: the gradient buffers come round soonest (one for all groups by
-        # default), and the written-through end of each survives until its next visit if all of them fit the cache
-        # together (measured with 2, 3 and 4 buffers in rotation: 128, 85, 64 MB each).
+        # buffers come round again, and this is where that is known: the gradient buffers come round soonest (one
+        # for all groups by default), and the written-through end of each survives until its next visit if all of
+        # them fit that cache together (measured with 1, 2, 3 and 4 buffers in rotation: 128, 128, 85, 64 MB each).
+        # The choice is made per group (its tables carry it), so two models in one process keep their own; the
+        # process-wide options stay what the application set them to.
         policy = os.environ.get("YAFSDP_STORE_POLICY", "auto")
         if policy not in ("auto", "keep", *_native.STORE_POLICIES):
             raise ValueError(
                 f"YAFSDP_STORE_POLICY={policy!r}: expected auto, keep or one of {sorted(_native.STORE_POLICIES)}"
             )
         if policy == "auto":
-            if len(param_groups) == 1:
-                policy = "single_set"
-            else:
-                tail_mb = min(128, 256 // max(1, len(grad_users)))
-                policy = (0, 0, 0, tail_mb if tail_mb >= 32 else 0)
-        if policy != "keep":
-            _native.set_store_policy(policy)
+            tail_mb = min(128, 256 // max(1, len(grad_users)))
+            for g in param_groups:
+                g.set_gather_tail_mb(tail_mb if tail_mb >= 32 else 0)
+        elif policy != "keep":
+            _native.set_store_policy(policy)  # an explicit, process-wide choice of the application
 
     def validate_shared_state(self) -> None:
         """ya_fsdp/_state.py:290-414: enough buffers for overlap; at most one

@@ -106,16 +106,30 @@ bool scale_plan_any(double divisor, int* scale, float* k) {
   return true;
 }
 
+// The scalar of a pre-multiplied sum as the collective applies it: converted to the data type (through binary32,
+// round to nearest even), here as the binary32 number of that value.  A product with it is one exact binary32
+// multiply for the 16-bit types (8 x 8 or 11 x 11 significand bits) and one rounded multiply for binary32.
+bool premul_plan(double scalar, int dtype, int* scale, float* k) {
+  float f = static_cast<float>(scalar);
+  if (dtype == DT_BF16) {
+    uint32_t bits;
+    std::memcpy(&bits, &f, 4);
+    if ((bits & 0x7FFFFFFFu) > 0x7F800000u) return false;
+    bits = ((bits + 0x7FFFu + ((bits >> 16) & 1u)) >> 16) << 16;
+    std::memcpy(&f, &bits, 4);
+  } else if (dtype == DT_F16) {
+    f = static_cast<float>(static_cast<_Float16>(f));
+  }
+  if (!std::isfinite(f)) return false;
+  *scale = f == 1.0f ? SCALE_NONE : SCALE_MUL;
+  *k = f;
+  return true;
+}
+
 int grid_for(int64_t n_tiles, int blocks_per_cu, int device) {
   int64_t cap = int64_t(cu_count(device)) * (blocks_per_cu > 0 ? blocks_per_cu : 1);
   int64_t g = n_tiles < cap ? n_tiles : cap;
   return g < 1 ? 1 : int(g);
-}
-
-// workgroups a table kernel needs for n tiles (see kTableXcd)
-int64_t table_blocks(int64_t n_tiles) {
-  constexpr int64_t win = kTableXcd > 0 ? int64_t(kTableXcd) * kTableXcdRun : 1;
-  return (n_tiles + win - 1) / win * win;
 }
 
 // first tile of a flat pass that writes through: the last tail_mb megabytes of its output (tile_units: 8-element
@@ -131,6 +145,13 @@ int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const vo
                 hipStream_t stream, const std::atomic<int>& tail_mb = g_flat_tail_mb) {
   if (n == 0) return YAFSDP_OK;
   if (!aligned_to(dst, item_size(dst_dt)) || !aligned_to(src, item_size(src_dt))) return YAFSDP_ERR_MISALIGNED;
+  if (src_dt == dst_dt && scale == SCALE_NONE && !acc && src_dt != DT_BF16) {
+    // a same-dtype copy moves bytes, whatever they encode: it runs as the copy of 2-byte units, whose lanes each own
+    // 16 consecutive bytes (872 MB of binary32: 82 % of peak as 2-byte units against 77 % in the arrangement that
+    // the casts between binary32 and a 2-byte dtype use)
+    n = n * item_size(src_dt) / 2;
+    src_dt = dst_dt = DT_BF16;
+  }
   {
     // in place (same address, same element size) is fine: every element is read before it is written by the
     // same lane; any other overlap of the two byte ranges has no defined result (torch's copy_ refuses it too)
@@ -191,6 +212,9 @@ struct yafsdp_table {
   std::vector<char> scratch;        // host: the arrays of the current call in staging format
   int next = 0;
   std::mutex mu;
+  // yafsdp_table_set_option: this table's own write-through tails, -1 = the process-wide option
+  std::atomic<int> gather_tail_mb{-1};
+  std::atomic<int> scatter_tail_mb{-1};
 };
 
 // The tensor side of a table fixed for many calls: validated once, and for
@@ -209,7 +233,9 @@ namespace {
 int gather_wt_from(const yafsdp_table* t, int flat_dtype) {
   const int64_t tile_bytes = t->tile_elems * item_size(flat_dtype);
   if (tile_bytes <= 0) return 0;
-  const int64_t tail = (int64_t(g_gather_tail_mb.load(std::memory_order_relaxed)) << 20) / tile_bytes;
+  int mb = t->gather_tail_mb.load(std::memory_order_relaxed);
+  if (mb < 0) mb = g_gather_tail_mb.load(std::memory_order_relaxed);
+  const int64_t tail = (int64_t(mb) << 20) / tile_bytes;
   return tail >= t->n_tiles ? 0 : int(t->n_tiles - tail);
 }
 
@@ -217,7 +243,9 @@ int gather_wt_from(const yafsdp_table* t, int flat_dtype) {
 int scatter_wt_from(const yafsdp_table* t, int tensor_dtype) {
   const int64_t slot_bytes = t->slot_elems * item_size(tensor_dtype);
   if (slot_bytes <= 0) return 0;  // a table without elements launches nothing
-  const int64_t tail = (int64_t(g_scatter_tail_mb.load(std::memory_order_relaxed)) << 20) / slot_bytes;
+  int mb = t->scatter_tail_mb.load(std::memory_order_relaxed);
+  if (mb < 0) mb = g_scatter_tail_mb.load(std::memory_order_relaxed);
+  const int64_t tail = (int64_t(mb) << 20) / slot_bytes;
   return tail >= t->n_slots ? 0 : int(t->n_slots - tail);
 }
 
@@ -283,9 +311,11 @@ int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, L
     if (t->filled[i] && std::memcmp(t->h_stage[i], cur, used) == 0) { s = i; break; }
   }
   if (s >= 0) {
-    // same arrays as an earlier call: the device copy is reused.  A kernel on another stream than the one the
-    // copy was enqueued on is ordered behind it (on the device; the host does not wait).
-    if (t->ev_pending[s] && t->staged_on[s] != stream) {
+    // same arrays as an earlier call: the device copy is reused.  This call's kernel is ordered behind the slot's
+    // last reader, whichever stream that ran on (on the device; the host does not wait; a wait for an event of the
+    // same stream costs nothing), so the event that this call records afterwards covers every earlier reader and
+    // the copy before them.
+    if (t->ev_pending[s]) {
       hipError_t e = hipStreamWaitEvent(stream, t->ev[s], 0);
       if (e != hipSuccess) return int(e);
     }
@@ -325,11 +355,19 @@ int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
   return YAFSDP_OK;
 }
 
+// The launch after stage_large failed: the slot's content is no longer offered for reuse, and the slot stays
+// ordered behind whatever stage_large enqueued (the event is recorded all the same).  Returns `launch_error`.
+int abandon_large(yafsdp_table* t, int slot, hipStream_t stream, hipError_t launch_error) {
+  t->filled[slot] = false;
+  if (hipEventRecord(t->ev[slot], stream) == hipSuccess) t->ev_pending[slot] = true;
+  return int(launch_error);
+}
+
 }  // namespace
 
 extern "C" {
 
-int yafsdp_version(void) { return 1005; }
+int yafsdp_version(void) { return 1006; }
 
 const char* yafsdp_error_string(int code) {
   switch (code) {
@@ -424,7 +462,7 @@ int yafsdp_gather_in_bound(yafsdp_binding* binding, void* flat, int flat_dtype, 
   float k;
   scale_plan(pre_factor, &scale, &k);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int grid = grid_for(table_blocks(table->n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table->n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallRoute)
     return int(launch_gather<SmallMeta>(table->block, binding->tensor_dtype, flat_dtype, scale, binding->small, flat,
                                         table->padded, table->n_tiles, k, zero_pad ? 1 : 0, gather_wt_from(table, flat_dtype),
@@ -446,7 +484,7 @@ int yafsdp_scatter_out_bound(yafsdp_binding* binding, const void* flat, int flat
   if (e != hipSuccess) return int(e);
   if (device != table->device) return YAFSDP_ERR_WRONG_DEVICE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int grid = grid_for(table_blocks(table->n_slots), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(table->n_slots, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallRoute)
     return int(launch_scatter<SmallMeta>(table->scatter_shape, flat_dtype, binding->tensor_dtype, binding->small, flat,
                                          table->total, table->n_slots, scatter_wt_from(table, binding->tensor_dtype),
@@ -503,6 +541,22 @@ int yafsdp_set_option(int option, int value) {
     case YAFSDP_OPT_TABLE_BLOCKS_PER_CU: g_table_blocks_per_cu.store(value); return YAFSDP_OK;
   }
   return YAFSDP_ERR_INVALID_ARGUMENT;
+}
+
+int yafsdp_table_set_option(yafsdp_table* table, int option, int value) {
+  if (table == nullptr || value < -1 || value > (1 << 20)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (option == YAFSDP_OPT_GATHER_TAIL_MB) table->gather_tail_mb.store(value);
+  else if (option == YAFSDP_OPT_SCATTER_TAIL_MB) table->scatter_tail_mb.store(value);
+  else return YAFSDP_ERR_INVALID_ARGUMENT;
+  return YAFSDP_OK;
+}
+
+int yafsdp_table_get_option(const yafsdp_table* table, int option, int* value) {
+  if (table == nullptr || value == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (option == YAFSDP_OPT_GATHER_TAIL_MB) *value = table->gather_tail_mb.load();
+  else if (option == YAFSDP_OPT_SCATTER_TAIL_MB) *value = table->scatter_tail_mb.load();
+  else return YAFSDP_ERR_INVALID_ARGUMENT;
+  return YAFSDP_OK;
 }
 
 int yafsdp_get_option(int option, int* value) {
@@ -645,7 +699,13 @@ int yafsdp_flat_sumsq_static(const void* src, int dtype, int64_t n, double* sums
   double* scratch = nullptr;
   const int rc0 = sumsq_static_scratch(&scratch);  // set-up on the first call on this device
   if (rc0 != YAFSDP_OK) return rc0;
-  if (n == 0) return YAFSDP_OK;  // a call that only performs the set-up
+  if (n == 0) {
+    // nothing to add: like yafsdp_flat_sumsq, *sumsq becomes 0 unless it accumulates (a call with a null `sumsq`
+    // only performs the set-up)
+    if (sumsq == nullptr) return YAFSDP_OK;
+    if (!aligned_to(sumsq, 8)) return YAFSDP_ERR_MISALIGNED;
+    return int(launch_sumsq_finish(scratch, 0, sumsq, accumulate ? 1 : 0, 0.0f, nullptr, static_cast<hipStream_t>(stream)));
+  }
   // every partial sum the finishing launch reads is written by the launch before it: nothing has to start at zero
   int64_t count = 0;
   const int rc = yafsdp_sumsq_partials(src, dtype, n, scratch, kSumsqMaxPartials, &count, stream);
@@ -783,6 +843,32 @@ int yafsdp_flat_div(void* buf, int dtype, int64_t n, double factor, void* stream
   scale_plan(factor, &scale, &k);
   if (scale == SCALE_NONE) return YAFSDP_OK;
   return flat_launch(dtype, dtype, scale, false, buf, buf, n, k, static_cast<hipStream_t>(stream));
+}
+
+int yafsdp_flat_premul(void* buf, int dtype, int64_t n, double scalar, void* stream) {
+  if (!valid_dtype(dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && buf == nullptr)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  if (!premul_plan(scalar, dtype, &scale, &k)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (scale == SCALE_NONE || n == 0) return YAFSDP_OK;
+  return flat_launch(dtype, dtype, scale, false, buf, buf, n, k, static_cast<hipStream_t>(stream));
+}
+
+int yafsdp_post_reduce_premul(void* shard, int shard_dtype, const void* chunk, int chunk_dtype, int64_t n,
+                              double scalar, int accumulate, void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  if (n < 0 || (n > 0 && (shard == nullptr || chunk == nullptr))) return YAFSDP_ERR_INVALID_ARGUMENT;
+  int scale;
+  float k;
+  if (!premul_plan(scalar, chunk_dtype, &scale, &k)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (n == 0) return YAFSDP_OK;
+  if (shard == chunk) {  // the collective wrote into the shard itself: only its scaling is left
+    if (shard_dtype != chunk_dtype || accumulate) return YAFSDP_ERR_INVALID_ARGUMENT;
+    if (scale == SCALE_NONE) return YAFSDP_OK;
+  }
+  return flat_launch(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, chunk, n, k,
+                     static_cast<hipStream_t>(stream), g_post_reduce_tail_mb);
 }
 
 int yafsdp_flat_div_copy(void* dst, int dst_dtype, const void* src, int src_dtype, int64_t n, double divisor,
@@ -1024,7 +1110,7 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   int rc = check_dyn(table, tensor_ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
   const int n_tiles = table->n_tiles;
-  const int grid = grid_for(table_blocks(n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     fill_small(table, tensor_ptrs, mode, &meta);
@@ -1038,7 +1124,7 @@ int yafsdp_gather_in(yafsdp_table* table, const void* const* tensor_ptrs, const 
   if (rc != YAFSDP_OK) return rc;
   e = launch_gather<LargeMeta>(table->block, tensor_dtype, flat_dtype, scale, meta, flat, table->padded, n_tiles, k,
                                zero_pad ? 1 : 0, gather_wt_from(table, flat_dtype), grid, s);
-  if (e != hipSuccess) return int(e);
+  if (e != hipSuccess) return abandon_large(table, slot, s, e);
   return finish_large(table, slot, s);
 }
 
@@ -1073,7 +1159,7 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   int64_t n_flat_blocks = n > 0 ? (((n - head) >> 3) + flat_tile - 1) / flat_tile : 0;
   if (n > 0 && n_flat_blocks < 1) n_flat_blocks = 1;  // workgroup 0 of the flat job peels head and tail
   const int64_t n_slots = table->total > 0 ? table->n_slots : 0;
-  const int64_t grid = n_flat_blocks + table_blocks(n_slots);
+  const int64_t grid = n_flat_blocks + n_slots;
   if (grid == 0) return YAFSDP_OK;
   if (grid > int64_t(INT32_MAX) - 4096) return YAFSDP_ERR_INVALID_ARGUMENT;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1096,7 +1182,7 @@ int yafsdp_copy_in_scatter_out(yafsdp_table* table, const void* flat, int flat_d
   if (rc != YAFSDP_OK) return rc;
   e = launch_unshard<LargeMeta>(table->scatter_shape, master_dtype, flat_dtype, meta, flat, int(n_slots), wt_from, ag_in,
                                 master, n, int(head), int(n_flat_blocks), cast_wt_from, int(grid), s);
-  if (e != hipSuccess) return int(e);
+  if (e != hipSuccess) return abandon_large(table, slot, s, e);
   return finish_large(table, slot, s);
 }
 
@@ -1149,7 +1235,7 @@ int yafsdp_gather_in_post_reduce(yafsdp_table* table, const void* const* tensor_
   if (rc != YAFSDP_OK) return rc;
   e = launch_gather_post<LargeMeta>(table->block, tensor_dtype, flat_dtype, shard_dtype, meta, flat, shard,
                                     table->padded, table->n_tiles, zero_pad ? 1 : 0, accumulate ? 1 : 0, dv, grid, s);
-  if (e != hipSuccess) return int(e);
+  if (e != hipSuccess) return abandon_large(table, slot, s, e);
   return finish_large(table, slot, s);
 }
 
@@ -1169,7 +1255,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   int rc = check_dyn(table, ptrs, mode, item_size(tensor_dtype));
   if (rc != YAFSDP_OK) return rc;
   const int n_tiles = table->n_slots;
-  const int grid = grid_for(table_blocks(n_tiles), g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
+  const int grid = grid_for(n_tiles, g_table_blocks_per_cu.load(std::memory_order_relaxed), device);
   if (table->n_tensors <= kSmallRoute) {
     SmallMeta meta;
     fill_small(table, ptrs, mode, &meta);
@@ -1183,7 +1269,7 @@ int yafsdp_scatter_out(yafsdp_table* table, const void* flat, int flat_dtype, vo
   if (rc != YAFSDP_OK) return rc;
   e = launch_scatter<LargeMeta>(table->scatter_shape, flat_dtype, tensor_dtype, meta, flat, table->total, n_tiles,
                                 scatter_wt_from(table, tensor_dtype), grid, s);
-  if (e != hipSuccess) return int(e);
+  if (e != hipSuccess) return abandon_large(table, slot, s, e);
   return finish_large(table, slot, s);
 }
 

@@ -140,7 +140,6 @@ __device__ __forceinline__ void flat_body(void* dst, const void* src, int64_t n,
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 flat_kernel(void* dst, const void* src, int64_t n, int head, float k, unsigned long long* trace, int wt_from) {
-  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   unsigned long long t_start = 0;
   if (trace != nullptr) t_start = wall_clock64();
   flat_body<S, D, SCALE, ACC, BLOCK, U, NTL, STP>(dst, src, n, head, k, int(blockIdx.x), int(gridDim.x), wt_from);

@@ -10,7 +10,7 @@ namespace {
 template <class META, class M, class P, int BLOCK, int US>
 hipError_t unshard_go(const META& meta, const void* gathered, int n_slots, int wt_from, void* ag_in, const void* master, int64_t n,
                       int head, int n_flat_blocks, int flat_wt_from, int grid, hipStream_t stream) {
-  return launch_kernel(unshard_kernel<META, M, P, BLOCK, kFusedFlatUnroll, US, scatter_nt_load(US), kFlatStorePolicy,
+  return launch_kernel(unshard_kernel<META, M, P, BLOCK, kFusedFlatUnroll, US, kTableNtLoad, kFlatStorePolicy,
                                       kScatterStorePolicy>,
                        grid, BLOCK, stream, meta, gathered, n_slots, wt_from, ag_in, master, n, head, n_flat_blocks, flat_wt_from);
 }

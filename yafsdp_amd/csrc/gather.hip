@@ -47,6 +47,8 @@ hipError_t by_flat(int block, int flat_dt, int scale, const META& meta, void* fl
 template <class META>
 hipError_t launch_gather(int block, int tensor_dt, int flat_dt, int scale, const META& meta, void* flat,
                          int64_t padded, int n_tiles, float k, int pad_zero, int wt_from, int grid, hipStream_t stream) {
+  // the kernel looks its first tile up before it tests the tile count: every workgroup must own a tile
+  if (n_tiles < 1 || grid < 1 || grid > n_tiles) return hipErrorInvalidValue;
   switch (tensor_dt) {
     case DT_F32: return by_flat<META, F32>(block, flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, wt_from, grid, stream);
     case DT_BF16: return by_flat<META, BF16>(block, flat_dt, scale, meta, flat, padded, n_tiles, k, pad_zero, wt_from, grid, stream);

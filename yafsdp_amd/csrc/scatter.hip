@@ -7,7 +7,7 @@ namespace {
 
 template <class META, class S, class D, int BLOCK, int U>
 hipError_t go(const META& meta, const void* flat, int64_t total, int n_tiles, int wt_from, int grid, hipStream_t stream) {
-  return launch_kernel(scatter_out_kernel<META, S, D, BLOCK, U, scatter_nt_load(U), kScatterStorePolicy>, grid, BLOCK,
+  return launch_kernel(scatter_out_kernel<META, S, D, BLOCK, U, kTableNtLoad, kScatterStorePolicy>, grid, BLOCK,
                        stream, meta, flat, total, n_tiles, wt_from);
 }
 

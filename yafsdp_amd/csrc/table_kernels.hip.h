@@ -45,12 +45,9 @@ namespace yafsdp {
 
 constexpr int kSmallMax = 16;
 // tables with at most this many tensors take the SmallMeta route (at most kSmallMax: the arrays' size).  Sending
-// a 9-tensor layer through per-tile records instead (-DYAFSDP_SMALL_ROUTE=8) measured 1 us slower per table kernel
-// and 13 us slower per step (the staging of pointers).
-#ifndef YAFSDP_SMALL_ROUTE
-#define YAFSDP_SMALL_ROUTE 16
-#endif
-constexpr int kSmallRoute = YAFSDP_SMALL_ROUTE;
+// a 9-tensor layer through per-tile records instead measured 1 us slower per table kernel and 13 us slower per
+// step (the staging of pointers).
+constexpr int kSmallRoute = 16;
 static_assert(kSmallRoute >= 0 && kSmallRoute <= kSmallMax, "SmallMeta holds at most kSmallMax tensors");
 enum : int { MODE_ZERO = 3 };  // internal: fill with zeros (pad lanes)
 
@@ -276,21 +273,12 @@ __device__ __forceinline__ void gather_segment(char* dst, const char* src, int64
   }
 }
 
-// Tile handled by workgroup b: b itself, or the XCD-aware permutation inside windows of kWin tiles.
 // a full tile of gather-in under the (wave-uniform) mode of its tensor; a skipped tensor's lanes still see the divide
 template <class S, class D, int SCALE, int BLOCK, int U, bool NTL, int STP>
 __device__ __forceinline__ void gather_full_tile_by_mode(int mode, char* dst, const char* src, float k) {
   if (mode == MODE_COPY) gather_full_tile<S, D, SCALE, MODE_COPY, BLOCK, U, NTL, STP>(dst, src, k);
   else if (mode == MODE_ADD) gather_full_tile<S, D, SCALE, MODE_ADD, BLOCK, U, NTL, STP>(dst, src, k);
   else if (SCALE != SCALE_NONE) gather_full_tile<S, D, SCALE, MODE_SKIP, BLOCK, U, NTL, STP>(dst, src, k);
-}
-
-template <int kX, int kWin>
-__device__ __forceinline__ int tile_of_block(int b) {
-  if constexpr (kX == 1) return b;
-  constexpr int kRun = kWin / kX;
-  const int w = b / kWin, r = b % kWin;
-  return w * kWin + (r % kX) * kRun + r / kX;
 }
 
 // S: tensor dtype, D: flat buffer dtype.  pad_zero != 0 writes zeros to
@@ -300,22 +288,17 @@ __device__ __forceinline__ int tile_of_block(int b) {
 template <class META, class S, class D, int SCALE, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, int pad_zero, int wt_from) {
-  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   constexpr int64_t kTile = int64_t(BLOCK) * U * 8;
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   char* fbase = reinterpret_cast<char*>(flat);
-  constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
-  constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
-  const int n_blocks = (n_tiles + kWin - 1) / kWin * kWin;
-  // (a loop that tests at its end: the first tile's lookup then does not wait for n_tiles to arrive before its
-  // own loads leave; a workgroup beyond the last tile finds tile >= n_tiles below)
-  int b = blockIdx.x;
+  // Workgroup b handles tile b (the host launches at most n_tiles workgroups and at least one when n_tiles > 0).
+  // A loop that tests at its end: the first tile's lookup then does not wait for n_tiles to arrive before its own
+  // loads leave.
+  int tile = blockIdx.x;
   do {
-    const int tile = tile_of_block<kX, kWin>(b);
     const int64_t t0 = int64_t(tile) * kTile;
     const int64_t t1 = (t0 + kTile < padded) ? t0 + kTile : padded;
     const TileLookup rec = meta.lookup(tile, t0, kTile);
-    if (tile >= n_tiles) continue;
     int p = rec.first;
     if (rec.full) {  // the whole tile lies inside tensor p
       const int mode = rec.mode;
@@ -348,7 +331,7 @@ gather_in_kernel(META meta, void* flat, int64_t padded, int n_tiles, float k, in
       pos = e;
       if (e == o1) ++p;
     }
-  } while ((b += gridDim.x) < n_blocks);
+  } while ((tile += gridDim.x) < n_tiles);
 }
 
 // ---------------------------------------------------------------- scatter-out --
@@ -412,12 +395,7 @@ __device__ __forceinline__ void scatter_body(const META& meta, const void* flat,
   constexpr bool NTS = (STP == ST_NT);  // ragged segments keep ordinary global stores
   constexpr int64_t kLineElems = 128 / D::kSize;
   const char* fbase = reinterpret_cast<const char*>(flat);
-  constexpr int kX = kTableXcd > 0 ? kTableXcd : 1;  // 1: workgroup b handles tile b
-  constexpr int kWin = kX * (kTableXcd > 0 ? kTableXcdRun : 1);
-  const int n_rounded = (n_tiles + kWin - 1) / kWin * kWin;
-  for (int b = block; b < n_rounded; b += n_blocks) {
-    const int tile = tile_of_block<kX, kWin>(b);
-    if (tile >= n_tiles) continue;
+  for (int tile = block; tile < n_tiles; tile += n_blocks) {
     const ScatterLookup rec = meta.lookup_scatter(tile);
     const int p = rec.tensor;
     if (p >= meta.n_tensors) continue;
@@ -445,7 +423,6 @@ __device__ __forceinline__ void scatter_body(const META& meta, const void* flat,
 template <class META, class S, class D, int BLOCK, int U, bool NTL, int STP>
 __global__ void __launch_bounds__(BLOCK)
 scatter_out_kernel(META meta, const void* flat, int64_t total, int n_tiles, int wt_from) {
-  if constexpr (kWavePrio > 0) __builtin_amdgcn_s_setprio(kWavePrio);
   (void)total;
   scatter_body<META, S, D, BLOCK, U, NTL, STP>(meta, flat, n_tiles, wt_from, int(blockIdx.x), int(gridDim.x));
 }
