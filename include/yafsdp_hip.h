@@ -386,6 +386,18 @@ int yafsdp_adamw_step(float* param, float* grad, float* exp_avg, float* exp_avg_
  * launch several kernels); NULL, NULL disarms. */
 int yafsdp_time_next_launch(void* start_event, void* stop_event);
 
+/* The next kernel this thread launches through the library records `event` (a hipEvent_t; timing may be disabled)
+ * when it completes, as hipEventRecord(event, stream) right after the call would, but on the kernel's own
+ * dispatch (hipExtLaunchKernel): no marker packet follows the kernel in its queue.  A marker between two kernels
+ * of one stream was measured at 6.5 us of idle GPU, a kernel -> event -> wait -> kernel hop between two streams at
+ * 11.4 us; the reference records one event per all-gather and two per reduce (ya_fsdp/_collectives.py:73-76,
+ * 215; ya_fsdp/_param_group.py:595-606, 757-769).  Consumed by ONE launch (the first, for an entry point that
+ * launches several kernels: use it with single-launch calls).  A call that launches nothing (an empty range)
+ * leaves the event armed: yafsdp_complete_next_launch_pending() then returns 1 and the caller records the event
+ * itself after disarming with NULL.  No counterpart in the reference (torch records events as queue markers). */
+int yafsdp_complete_next_launch(void* event);
+int yafsdp_complete_next_launch_pending(void);
+
 /* Measurement hook: per-workgroup timeline of the next kernel that this thread launches through
  * yafsdp_flat_copy / yafsdp_flat_div / yafsdp_flat_div_copy / yafsdp_post_reduce.  Workgroup b of that launch
  * stores the GPU's 100 MHz wall-clock count at its start into trace[2 b] and, once its loads have arrived and its

@@ -542,3 +542,43 @@ def test_table_with_the_maximum_number_of_tensors(nat):
     table.scatter_out(flat, list(out.split(numels)))
     assert_bits_equal(out, flat[:t].cpu().bfloat16(), "scatter_out, 65,534 tensors")
     table.close()
+
+
+def test_completion_event_recorded_by_the_launch_itself(nat):
+    """``launch_recording``: the kernel's own dispatch records the event.  Another stream that waits for the event
+    sees the kernel's output (new data every round, so a missed dependency shows as stale values), the host can
+    synchronise on it, and a call that launches nothing still leaves the event recorded."""
+    g = torch.Generator().manual_seed(151)
+    n = 8_000_000
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    event = torch.cuda.Event()
+    src = torch.empty(n, dtype=torch.float32, device=DEV)
+    mid = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    out = torch.zeros(n, dtype=torch.bfloat16, device=DEV)
+    main = torch.cuda.current_stream()
+    for round_ in range(6):
+        _say("completion event round", round_)
+        x = torch.randn(n, generator=g) * 0.02 + round_
+        src.copy_(x.to(DEV))
+        a.wait_stream(main)
+        with torch.cuda.stream(a):
+            got = nat.launch_recording(event, lambda: nat.flat_copy(mid, src), a)
+            assert got is event
+        with torch.cuda.stream(b):
+            b.wait_event(event)
+            nat.flat_copy(out, mid)
+        main.wait_stream(b)
+        assert_bits_equal(out, x.bfloat16(), f"round {round_}")
+        b.wait_stream(main)
+        a.wait_stream(main)  # the next round's src.copy_ must not overtake this round's reads
+    with torch.cuda.stream(a):
+        src.fill_(3.0)
+        nat.launch_recording(event, lambda: nat.flat_copy(mid, src), a)
+    event.synchronize()  # the host waits for the kernel through the same event
+    assert event.query() and float(mid[n - 1]) == 3.0 and float(mid[0]) == 3.0
+    # nothing to launch: the event is recorded the ordinary way, and nothing stays armed for a later launch
+    fresh = torch.cuda.Event()
+    with torch.cuda.stream(a):
+        nat.launch_recording(fresh, lambda: nat.flat_copy(mid[:0], src[:0]), a)
+    fresh.synchronize()
+    assert fresh.query() and nat.lib.yafsdp_complete_next_launch_pending() == 0

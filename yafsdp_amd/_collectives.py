@@ -96,6 +96,15 @@ def all_gather(
         rank = all_gather_group.rank()
         slot = all_gather_output if world_size == 1 else all_gather_output[rank * shard_numel : (rank + 1) * shard_numel]
         placed = False
+        all_gather_event = None
+
+        def last(launch):
+            """The final launch of this all-gather records the event that its consumers wait for."""
+            nonlocal all_gather_event
+            all_gather_event = _native.launch_recording(
+                param_group.completion_event(("all_gather", all_gather_dtype)), launch, all_gather_stream
+            )
+
         if all_gather_dtype not in param_group._all_gather_input_set_dtypes:
             for fsdp_param in fsdp_params:
                 fsdp_param.set_all_gather_input()
@@ -106,7 +115,7 @@ def all_gather(
                 if yccl_handle is not None and world_size > 1:
                     _native.flat_copy(all_gather_input, padded_sharded_param_data)  # the handle places it
                 elif all(t.data_ptr() % 16 == 0 for t in (slot, all_gather_input, padded_sharded_param_data)):
-                    _native.flat_copy_fanout([all_gather_input, slot], padded_sharded_param_data)
+                    last(lambda: _native.flat_copy_fanout([all_gather_input, slot], padded_sharded_param_data))
                     placed = True
                 else:
                     _native.flat_copy(all_gather_input, padded_sharded_param_data)
@@ -115,9 +124,10 @@ def all_gather(
             yccl_handle.all_gather(all_gather_input.view(torch.bfloat16), all_gather_output.view(torch.bfloat16))  # :67-70
         elif not placed:
             # size-1 group (:56-58), or this rank's share of all_gather_into_tensor (:60-65)
-            _native.flat_copy(slot, all_gather_input)
+            last(lambda: _native.flat_copy(slot, all_gather_input))
         all_gather_work = None
-        all_gather_event = all_gather_stream.record_event()
+        if all_gather_event is None:
+            all_gather_event = all_gather_stream.record_event()
     return AllGatherResult(all_gather_event, all_gather_work)
 
 
@@ -167,11 +177,15 @@ def reduce_scatter(
     yccl_handle: Optional[Any],
     *,
     predivide_fused: bool = False,
+    ready_event: "torch.cuda.Event | None" = None,
 ) -> torch.cuda.Event:
     """ya_fsdp/_collectives.py:93-218.
 
     ``predivide_fused``: the caller already applied the pre-divide inside the
     reduce copy-in launch (``foreach_reduce_copy_in``), so it is skipped here.
+    ``ready_event``: recorded on the current stream when the reduce buffer was
+    complete; the reduce-scatter stream then waits for it instead of for the
+    whole current stream (:110-111).
     """
     # ``yccl_handle``: the communication library that owns the reduce buffer reduces it in place
     # (``reduce_scatter(buffer)`` on its bf16 view, :163-164: a sum, which is why the divide factors then put the
@@ -180,7 +194,11 @@ def reduce_scatter(
     # group of size 1 (:140-150).  Here this rank's chunk is the only contribution to its reduce-scatter output,
     # and a binary32 sum of one 16-bit value rounds back to that value, so the flag changes nothing; the sum over
     # several contributions in binary32 is ``post_reduce_fanin``.
-    reduce_scatter_stream.wait_stream(torch.cuda.current_stream(padded_sharded_param_grad.device))
+    if ready_event is not None:
+        reduce_scatter_stream.wait_event(ready_event)
+    else:
+        reduce_scatter_stream.wait_stream(torch.cuda.current_stream(padded_sharded_param_grad.device))
+    post_reduce_event = None
     with torch.cuda.stream(reduce_scatter_stream):
         world_size, rank = reduce_scatter_group.size(), reduce_scatter_group.rank()
         reduce_in_sharded = (
@@ -242,7 +260,8 @@ def reduce_scatter(
             param_group._grad_sumsq_token.pop(cls_key, None)
         if world_size > 1 and reduce_in_sharded:
             # the collective would have written straight into the shard (:124-125)
-            _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, chunk, post, False, premul)
+            post_reduce_event = _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, chunk, post,
+                                             False, premul, reduce_scatter_stream)
         elif world_size == 1 and reduce_in_sharded:
             _div_if_needed(padded_sharded_param_grad, post)
         else:
@@ -250,9 +269,11 @@ def reduce_scatter(
             without_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is None]
             with_sharded_grad = [p for p in fsdp_params_with_grad if p.sharded_param.grad is not None]
             if len(without_sharded_grad) == len(fsdp_params_which_require_grad):
-                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, False, premul)  # :185
+                post_reduce_event = _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor,
+                                                 post, False, premul, reduce_scatter_stream)  # :185
             elif len(with_sharded_grad) == len(fsdp_params_which_require_grad):
-                _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor, post, True, premul)  # :189
+                post_reduce_event = _post_reduce(param_group, cls_key, whole, padded_sharded_param_grad, output_tensor,
+                                                 post, True, premul, reduce_scatter_stream)  # :189
             else:
                 with_ids = {id(p) for p in with_sharded_grad}
                 without_ids = {id(p) for p in without_sharded_grad}
@@ -272,7 +293,8 @@ def reduce_scatter(
                     table = param_group._fragment_table_for(padded_sharded_param_grad, numels)
                     fragments = list(output_tensor[: sum(numels)].split(numels))
                     table.gather_in(fragments, padded_sharded_param_grad, modes, None, zero_pad=False)
-        post_reduce_event = reduce_scatter_stream.record_event()
+        if post_reduce_event is None:
+            post_reduce_event = reduce_scatter_stream.record_event()
         for fsdp_param in fsdp_params_with_grad:
             fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad  # :216-217
         return post_reduce_event
@@ -280,20 +302,27 @@ def reduce_scatter(
 
 def _post_reduce(
     param_group: "YaFSDPParamGroup | None", cls_key: Any, whole: bool, shard: torch.Tensor, chunk: torch.Tensor,
-    post: float | None, accumulate: bool, premul: float | None = None,
-) -> None:
+    post: float | None, accumulate: bool, premul: float | None = None, stream: "torch.cuda.Stream | None" = None,
+) -> "torch.cuda.Event | None":
     """``post_reduce`` of one all-gather dtype class of a group; for a class
     with a slot for partial sums of squares (``optim.enable_fused_grad_norm``)
     and a pass that gives every parameter of it its gradient, the variant that
     also leaves the squared norm of the shard.  ``premul``: the scalar of a
-    collective that scales inside the reduction (then there is no post-divide)."""
+    collective that scales inside the reduction (then there is no post-divide).
+    Returns the event that the (one) launch recorded on its own dispatch, or
+    None when the caller has to record one behind what was launched."""
     slot = param_group._grad_sumsq_slot.get(cls_key) if param_group is not None else None
     if slot is None or not whole:
-        if premul is not None:
-            _native.post_reduce_premul(shard, chunk, premul, accumulate)
-        else:
-            _native.post_reduce(shard, chunk, post, accumulate)
-        return
+        def launch():
+            if premul is not None:
+                _native.post_reduce_premul(shard, chunk, premul, accumulate)
+            else:
+                _native.post_reduce(shard, chunk, post, accumulate)
+
+        if param_group is None or stream is None:
+            launch()
+            return None
+        return _native.launch_recording(param_group.completion_event(("post_reduce", cls_key)), launch, stream)
     if premul is not None:
         _native.flat_premul(chunk, premul)
     lo, hi = slot
@@ -301,6 +330,7 @@ def _post_reduce(
     if end < hi:  # the slot is added up as a whole: entries a read pass may have left beyond these sums go
         param_group._grad_sumsq_partials[end:hi].zero_()
     param_group._grad_sumsq_token[cls_key] = shard._version
+    return None
 
 
 def _get_gradient_divide_factors(

@@ -246,6 +246,9 @@ class YaFSDPParamGroup:
                 fsdp_param._index_in_class = index
         self._tables: dict[torch.dtype | None, _native.TensorTable] = {}
         self._gather_tail_mb: int | None = None  # set_gather_tail_mb; None: the library's process-wide option
+        # events that a kernel of the path records on its own dispatch (_native.launch_recording), kept per purpose:
+        # each is only ever recorded on one stream, so a later record implies every earlier one
+        self._completion_events: dict[Any, torch.cuda.Event] = {}
         # this rank's fragments of each class's gradient shard (built on first use, ya_fsdp/_collectives.py:191-214)
         self._fragment_tables: dict[torch.dtype | None, _native.TensorTable] = {}
         self._state_dict_hook_handles: list = []
@@ -306,6 +309,13 @@ class YaFSDPParamGroup:
     def layout(self) -> ShardLayout:
         self._default_class("layout")
         return self.layouts[None]
+
+    def completion_event(self, purpose: Any) -> torch.cuda.Event:
+        """The group's event for ``purpose`` (a hashable name), created on first use."""
+        event = self._completion_events.get(purpose)
+        if event is None:
+            event = self._completion_events[purpose] = torch.cuda.Event()
+        return event
 
     def set_gather_tail_mb(self, megabytes: int | None) -> None:
         """How many megabytes at the end of this group's reduce buffer the reduce copy-in stores write-through (they
@@ -570,6 +580,7 @@ class YaFSDPParamGroup:
                 grad_buffer_ctx.release_event = None
             grad_buffer_ctx.owner = self
         predivide_fused: dict[torch.dtype | None, bool] = {}
+        copy_in_events: dict[torch.dtype | None, torch.cuda.Event] = {}
         reduced_in_one_launch = False
         with profiler_range(self._with_fqn("FSDP::post_backward_accumulate")):
             single_class = len(self._all_gather_dtype_to_fsdp_params) == 1
@@ -603,7 +614,18 @@ class YaFSDPParamGroup:
                     predivide_fused[all_gather_dtype] = True
                     if single_class and all_gather_dtype is None:
                         reduced_in_one_launch = self._reduce_in_one_launch(grads, modes)
-                if not reduced_in_one_launch:
+                if not reduced_in_one_launch and self.reduce_grads:
+                    # the launch records its own completion: the reduce-scatter stream waits for that event instead
+                    # of a marker placed behind the kernel in the compute stream's queue
+                    copy_in_events[all_gather_dtype] = _native.launch_recording(
+                        self.completion_event(("reduce_copy_in", all_gather_dtype)),
+                        lambda: foreach_reduce_copy_in(
+                            self, self._tables[all_gather_dtype], self._reduce_scatter_input[all_gather_dtype],
+                            grads, modes, pre,
+                        ),
+                        current_stream,
+                    )
+                elif not reduced_in_one_launch:
                     foreach_reduce_copy_in(
                         self, self._tables[all_gather_dtype], self._reduce_scatter_input[all_gather_dtype], grads,
                         modes, pre,
@@ -632,7 +654,7 @@ class YaFSDPParamGroup:
         if reduced_in_one_launch:
             # the gradient shard is already written, on this stream (ya_fsdp/_collectives.py:216-217 for the rest)
             with profiler_range(self._with_fqn("YaFSDP::post_backward_reduce")):
-                self._post_reduce_event = current_stream.record_event()
+                self._post_reduce_event = self.completion_event("reduce_in_one_launch")  # recorded by that launch
                 for fsdp_param in fsdp_params_with_grad_per_dtype[None]:
                     fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad
             grad_buffer_ctx.release_event = self._post_reduce_event
@@ -658,6 +680,7 @@ class YaFSDPParamGroup:
                     self.mp_policy.bit32_acc_for_bit16_reduce_scatter,
                     grad_buffer_ctx.yccl_handles.get(all_gather_dtype),
                     predivide_fused=predivide_fused.get(all_gather_dtype, False),
+                    ready_event=copy_in_events.get(all_gather_dtype),
                 )
         grad_buffer_ctx.release_event = self._post_reduce_event
         grad_buffer_ctx.owner = None
@@ -704,10 +727,16 @@ class YaFSDPParamGroup:
         if not _native.all_contiguous(grads):
             grads = [g if g is None or g.is_contiguous() else g.contiguous() for g in grads]
         self._grad_sumsq_token.pop(None, None)
-        return self._table.gather_in_post_reduce(
-            grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes,
-            pre_factor=pre, post_factor=post, custom_divisor=custom,
+        served = []
+        _native.launch_recording(
+            self.completion_event("reduce_in_one_launch"),
+            lambda: served.append(self._table.gather_in_post_reduce(
+                grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes,
+                pre_factor=pre, post_factor=post, custom_divisor=custom,
+            )),
+            torch.cuda.current_stream(self.device),
         )
+        return bool(served and served[0])
 
     def _fragment_table_for(self, grad_shard: torch.Tensor, numels: "list[int]") -> "_native.TensorTable":
         """Table over one class's gradient shard whose tensors are this rank's fragments (for the mixed copy /

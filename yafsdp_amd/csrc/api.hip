@@ -501,6 +501,14 @@ int yafsdp_time_next_launch(void* start_event, void* stop_event) {
   return YAFSDP_OK;
 }
 
+int yafsdp_complete_next_launch(void* event) {
+  tl_timed_launch.start = nullptr;
+  tl_timed_launch.stop = static_cast<hipEvent_t>(event);
+  return YAFSDP_OK;
+}
+
+int yafsdp_complete_next_launch_pending(void) { return tl_timed_launch.stop != nullptr ? 1 : 0; }
+
 int yafsdp_trace_next_flat_launch(uint64_t* trace, int64_t capacity, int64_t* n_workgroups) {
   if (trace == nullptr) {  // disarm
     tl_timed_launch.trace = nullptr;

@@ -9,10 +9,10 @@
 
 namespace yafsdp {
 
-// Measurement hook: when a start/stop event pair has been armed on this thread
-// (yafsdp_time_next_launch), the next kernel launched through the library is
-// dispatched with the events attached to that dispatch, so that they carry the
-// kernel's own begin and end timestamps (no launch gap in between).
+// When a start/stop event pair has been armed on this thread (yafsdp_time_next_launch), or a completion event
+// alone (yafsdp_complete_next_launch), the next kernel launched through the library is dispatched with the events
+// attached to that dispatch: they carry the kernel's own begin and end (no launch gap in between, and no packet
+// of their own in the queue, which an event recorded after the kernel costs).
 struct TimedLaunch {
   hipEvent_t start = nullptr, stop = nullptr;
   // per-workgroup timeline of the next flat kernel (yafsdp_trace_next_flat_launch): device buffer of 2 * capacity
@@ -26,7 +26,7 @@ extern thread_local TimedLaunch tl_timed_launch;
 template <class... Params, class... Args>
 inline hipError_t launch_kernel(void (*kernel)(Params...), int grid, int block, hipStream_t stream, Args... args) {
   TimedLaunch& t = tl_timed_launch;
-  if (t.start != nullptr) {
+  if (t.start != nullptr || t.stop != nullptr) {
     const hipEvent_t a = t.start, b = t.stop;
     t.start = t.stop = nullptr;
     hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, stream, a, b, 0, static_cast<Params>(args)...);
