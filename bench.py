@@ -68,6 +68,12 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 # "tiny-layer-w1": gather_post_kernel, (9309.25 * 1.99322 + 18534.0) KiB, below the algorithmic bytes of the two
 # kernels it replaces because the reduce buffer is not read back;
 # all three in profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.
+# Megabytes a GEMM stand-in of the full-model workload moves between the L2s and the memory side per launch
+# (TCC_EA0_RDREQ x 128 B + TCC_EA0_WRREQ x 64 B of the hipBLASLt kernel alone; profiles/bench_llama3-8b-full-w8_overlap.md),
+# and the rate at which a copy kernel of the path moves its bytes when it has the memory side to itself.
+GEMM_MEMORY_SIDE_MB = {"4096x4096x4096": 453.4 + 33.6, "llama-mlp-up 4096x4096x14336": 755.4 + 117.4,
+                       "llama-mlp-down 4096x14336x4096": 755.4 + 33.6}
+COPY_RATE_MB_PER_MS = 6550.0
 MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_645_400, "llama3-8b-layer-w8-optim": 817_885_000,
                           "ragged-stress-w256": 1_505_902_865, "llama3-70b-layer-w64": 3_422_785_664,
                           "ragged-stress-w256-bf16-masters": 1_014_344_628, "tiny-layer-w1": 37_979_573}
@@ -232,6 +238,10 @@ def run_full_model(args, as_record: bool = False):
                 "outs": [[torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels] for _ in range(2)],
                 "rs": torch.zeros(t_pad, dtype=torch.bfloat16, device=dev),
             }
+            # what fully_shard gives the tables of groups that share ONE gradient buffer (unless options were given)
+            if all(v is None for v in (args.gather_tail_mb, args.scatter_tail_mb, args.flat_tail_mb,
+                                       args.post_reduce_tail_mb)):
+                shape_res[key]["table"].set_option(_native.OPT_GATHER_TAIL_MB, 128)
         s_ = lay.padded_sharded_numel
         groups.append({
             "name": name, "res": shape_res[key], "lay": lay,
@@ -257,11 +267,11 @@ def run_full_model(args, as_record: bool = False):
     def gemm():
         torch.matmul(gemm_state["a"], gemm_state["b"], out=gemm_state["c"])
 
-    def unshard(i):  # copy-in + copy-out of group i (current stream)
+    def unshard(i):  # copy-in + copy-out of group i as one launch (current stream)
         g = groups[i]
         res = g["res"]
-        _native.flat_copy(g["ag_in"], g["master"])
-        res["table"].scatter_out(res["gathered"][i % 2], res["outs"][i % 2])
+        if not res["table"].copy_in_scatter_out(res["gathered"][i % 2], res["outs"][i % 2], g["ag_in"], g["master"]):
+            raise RuntimeError("copy_in_scatter_out declined")
 
     def reduce_in(i):
         g = groups[i]
@@ -273,21 +283,23 @@ def run_full_model(args, as_record: bool = False):
         _native.post_reduce(g["shard"], g["res"]["rs"][r * s_ : (r + 1) * s_], None, True)
 
     n = len(groups)
+    # the events of the hand-offs between the two streams are recorded by the kernels' own dispatches
+    # (_native.launch_recording): one event per group and purpose, each only ever recorded on one stream
+    ev_ready = [torch.cuda.Event() for _ in range(n)]   # copy-in + copy-out of group i done (side stream)
+    ev_done = [torch.cuda.Event() for _ in range(n)]    # reduce copy-in of group i done (compute stream)
+    ev_freed = [torch.cuda.Event() for _ in range(n)]   # post-reduce of group i done: its reduce buffer is free
 
     def step(copies=True, gemms=True, gather_on_side=False):
         # forward
-        ready = [None] * n
         if copies:
             with torch.cuda.stream(side):
-                unshard(0)
-                ready[0] = side.record_event()
+                _native.launch_recording(ev_ready[0], lambda: unshard(0), side)
         for i in range(n):
             if copies and i + 1 < n:
                 with torch.cuda.stream(side):  # prefetch the next group while this one computes
-                    unshard(i + 1)
-                    ready[i + 1] = side.record_event()
+                    _native.launch_recording(ev_ready[i + 1], lambda: unshard(i + 1), side)
             if copies:
-                main.wait_event(ready[i])
+                main.wait_event(ev_ready[i])
             if gemms:
                 gemm()
         # backward, reverse order
@@ -300,18 +312,18 @@ def run_full_model(args, as_record: bool = False):
                 key = id(groups[i]["res"])
                 if key in freed:
                     main.wait_event(freed[key])   # a shared gradient buffer is released by the post-reduce before
-                reduce_in(i)                      # compute stream, like the reference's foreach calls
-                done = main.record_event()
-                with torch.cuda.stream(side):     # reduce-scatter stream: waits for the compute stream
-                    side.wait_event(done)
-                    post(i)
-                    freed[key] = side.record_event()
+                # compute stream, like the reference's foreach calls
+                _native.launch_recording(ev_done[i], lambda: reduce_in(i), main)
+                with torch.cuda.stream(side):     # reduce-scatter stream: waits for the reduce copy-in
+                    side.wait_event(ev_done[i])
+                    freed[key] = _native.launch_recording(ev_freed[i], lambda: post(i), side)
             elif copies:
-                # not the reference's plan: the reduce copy-in leaves the compute stream as well (the side stream
-                # waits for the gradients, then runs both kernels; its own order keeps the shared buffer safe)
-                done = main.record_event()
+                # not the reference's plan (the library's opt-in, set_reduce_copy_in_on_side_stream): the reduce
+                # copy-in leaves the compute stream as well; the side stream waits for the gradients, then runs both
+                # kernels back to back, and its own order keeps the shared buffer safe
                 with torch.cuda.stream(side):
-                    side.wait_event(done)
+                    if gemms:
+                        side.wait_event(main.record_event())
                     reduce_in(i)
                     post(i)
 
@@ -390,6 +402,11 @@ def run_full_model(args, as_record: bool = False):
     t_unshard, t_gather, t_post = timed_loop(unshard, reps), timed_loop(reduce_in, reps), timed_loop(post, reps)
     log(f"  copies by kind, alone: copy-in + copy-out {t_unshard:.3f} ms, reduce copy-in {t_gather:.3f} ms, "
         f"post-reduce {t_post:.3f} ms per pass over {n} groups")
+    # copies alone under both stream plans (no GEMMs): the reference's (reduce copy-in on the compute stream, every
+    # hand-off between the two streams an event) and the library's opt-in (reduce copy-in on the side stream too)
+    t_copy_ref, t_copy_side = timed(True, False, reps), timed(True, False, reps, gather_on_side=True)
+    log(f"  copies alone as the pass runs them: {t_copy_ref:.3f} ms under the reference's stream plan, "
+        f"{t_copy_side:.3f} ms with the reduce copy-in on the side stream")
     for gname, (m_, k_, n_) in gemm_shapes:
         set_gemm(m_, k_, n_)
         t_gemm = timed(False, True, reps)
@@ -397,7 +414,7 @@ def run_full_model(args, as_record: bool = False):
         for bpc in caps:  # grid cap of the copy kernels in workgroups per compute unit
             _native.set_option(_native.OPT_FLAT_BLOCKS_PER_CU, bpc)
             _native.set_option(_native.OPT_TABLE_BLOCKS_PER_CU, bpc)
-            tc = timed(True, False, reps)
+            tc = t_copy_ref if bpc == 4096 else timed(True, False, reps)
             tb = timed(True, True, reps)
             sweep[bpc] = {"ms_copies_alone": round(tc, 3), "ms_overlapped": round(tb, 3),
                           "overlap_efficiency": round(max(tc, t_gemm) / tb, 4)}
@@ -412,12 +429,27 @@ def run_full_model(args, as_record: bool = False):
         # on the compute stream (ya_fsdp/_param_group.py:669-708), in line with the GEMMs, and only the
         # post-reduce is on the side stream
         critical = max(t_gemm / 3.0, t_unshard) + t_unshard / n + t_gemm * 2.0 / 3.0 + t_gather + t_post / n
+        # ... and what the memory system allows: a GEMM is not a pure matrix-core kernel, its tiles refetch the
+        # operands from the memory side (GEMM_MEMORY_SIDE_MB per launch, from the L2's counters), and a copy kernel
+        # saturates the memory side by itself.  While both run they share it, so a stretch of the pass in which
+        # copies of duration c (alone) and GEMMs of duration g (alone, moving m megabytes) overlap takes at least
+        # max(g, c + m / copy rate); stretches on one stream only take their own time.
+        mem_ms_per_gemm = GEMM_MEMORY_SIDE_MB[gname] / COPY_RATE_MB_PER_MS
+        g1 = t_gemm / (3.0 * n)  # one GEMM
+        fwd = n * max(g1, t_unshard / n + mem_ms_per_gemm) + t_unshard / n
+        bwd_ref = n * max(2 * g1, t_post / n + 2 * mem_ms_per_gemm) + t_gather + t_post / n
+        bwd_side = n * max(2 * g1, (t_gather + t_post) / n + 2 * mem_ms_per_gemm) + (t_gather + t_post) / n
+        model_ref, model_side = fwd + bwd_ref, fwd + bwd_side
         t_alt = timed(True, True, reps, gather_on_side=True)
-        log(f"  {gname}: critical path of the reference's stream plan {critical:.3f} ms; with the reduce copy-in on "
-            f"the side stream as well: overlapped {t_alt:.3f} ms")
+        log(f"  {gname}: critical path of the reference's stream plan {critical:.3f} ms, shared-memory-side model "
+            f"{model_ref:.3f} ms; with the reduce copy-in on the side stream as well: overlapped {t_alt:.3f} ms "
+            f"(model {model_side:.3f} ms)")
         per_gemm[gname] = {
             "critical_path_ms": round(critical, 4), "efficiency_vs_critical_path": round(critical / t_both, 4),
+            "memory_side_model_ms": round(model_ref, 4), "efficiency_vs_memory_side_model": round(model_ref / t_both, 4),
             "ms_overlapped_reduce_copy_in_on_side_stream": round(t_alt, 4),
+            "memory_side_model_ms_reduce_copy_in_on_side_stream": round(model_side, 4),
+            "efficiency_vs_memory_side_model_reduce_copy_in_on_side_stream": round(model_side / t_alt, 4),
             "ms_copies_alone": round(t_copy, 4), "ms_gemms_alone": round(t_gemm, 4), "ms_overlapped": round(t_both, 4),
             "overlap_efficiency": round(max(t_copy, t_gemm) / t_both, 4),
             "hidden_fraction": round((t_copy + t_gemm - t_both) / min(t_copy, t_gemm), 4),
@@ -441,8 +473,7 @@ def run_full_model(args, as_record: bool = False):
     li = 5
     lay = groups[li]["lay"]
     t_, tp, s_ = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
-    per = [("copy_in", lambda: _native.flat_copy(groups[li]["ag_in"], groups[li]["master"]), s_ * 6),
-           ("copy_out", lambda: groups[li]["res"]["table"].scatter_out(groups[li]["res"]["gathered"][1], groups[li]["res"]["outs"][1]), 4 * t_),
+    per = [("copy_in_and_copy_out", lambda: unshard(li), s_ * 6 + 4 * t_),
            ("reduce_copy_in", lambda: reduce_in(li), 4 * t_ + 2 * (tp - t_)),
            ("post_reduce", lambda: post(li), s_ * 10)]
     for name, fn, nbytes in per:
@@ -468,6 +499,9 @@ def run_full_model(args, as_record: bool = False):
         "ms_copies_by_kind_alone": {"copy_in_and_copy_out": round(t_unshard, 4), "reduce_copy_in": round(t_gather, 4),
                                     "post_reduce": round(t_post, 4)},
         "gemm_shapes": per_gemm, "copy_GBps_alone": round(bytes_step / t_copy / 1e6, 1),
+        "ms_copies_alone_reduce_copy_in_on_side_stream": round(t_copy_side, 4),
+        "copy_GBps_alone_reduce_copy_in_on_side_stream": round(bytes_step / t_copy_side / 1e6, 1),
+        "copy_GBps_by_kind": round(bytes_step / (t_unshard + t_gather + t_post) / 1e6, 1),
         "copy_GBps_overlapped_lower_bound": round(bytes_step / t_both / 1e6, 1), "bytes_per_step": bytes_step,
         "kernels": kernels,
     }
@@ -480,9 +514,14 @@ def run_full_model(args, as_record: bool = False):
             "value": out["value"], "unit": out["unit"], "parity": parity, "ms_overlapped": out["ms_overlapped"],
             "ms_copies_alone": out["ms_copies_alone"], "ms_gemms_alone": out["ms_gemms_alone"],
             "copy_GBps_alone": out["copy_GBps_alone"], "groups": n, "logical_world_size": w, "passes_timed": reps,
+            "copy_GBps_alone_reduce_copy_in_on_side_stream": out["copy_GBps_alone_reduce_copy_in_on_side_stream"],
+            "copy_GBps_by_kind": out["copy_GBps_by_kind"], "ms_copies_by_kind_alone": out["ms_copies_by_kind_alone"],
             "gemm_shapes": {k: {a_: b_ for a_, b_ in v.items()
                                 if a_ in ("ms_gemms_alone", "ms_overlapped", "overlap_efficiency",
-                                          "efficiency_vs_critical_path", "critical_path_ms")}
+                                          "efficiency_vs_critical_path", "critical_path_ms", "memory_side_model_ms",
+                                          "efficiency_vs_memory_side_model",
+                                          "ms_overlapped_reduce_copy_in_on_side_stream",
+                                          "efficiency_vs_memory_side_model_reduce_copy_in_on_side_stream")}
                             for k, v in per_gemm.items()},
         }
     print(json.dumps(out), flush=True)
@@ -1319,17 +1358,21 @@ def main() -> int:
                                                  "fully-shard-trainer-w1"])
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--no-parity", action="store_true", help="skip the in-run bit-exactness check against the oracle")
-    ap.add_argument("--no-stream-plan", action="store_true",
-                    help="skip the leg that runs the step on the reference's two streams")
-    ap.add_argument("--no-store-policy-ab", action="store_true",
-                    help="skip the leg that runs the step with the write-through tails of copy-out and reduce copy-in "
-                         "switched off")
-    ap.add_argument("--no-rotating-sets", action="store_true",
-                    help="skip the leg that alternates the step between two sets of buffers")
-    ap.add_argument("--rotating-sets", type=int, default=2, metavar="K",
-                    help="number of buffer sets of that leg (each set of the default workload is 2 GB)")
-    ap.add_argument("--no-graph", action="store_true",
-                    help="skip the leg that replays the step from a HIP graph (outside the timed region)")
+    ap.add_argument("--buffer-sets", "--rotating-sets", type=int, default=4, metavar="K", dest="buffer_sets",
+                    help="sets of buffers that take turns in the timed region (step k runs on set k mod K; each set of "
+                         "the default workload is 2 GB).  1: one set rewritten step after step, which finds its own "
+                         "output in the memory-side cache")
+    ap.add_argument("--stream-plan", action="store_true",
+                    help="add the leg that runs the step on the reference's two streams")
+    ap.add_argument("--store-policy-ab", action="store_true",
+                    help="add the leg that repeats the rotating loop under other store policies")
+    ap.add_argument("--graph", action="store_true",
+                    help="add the leg that replays the rotating steps from HIP graphs")
+    ap.add_argument("--variants", action="store_true",
+                    help="add the table of the other forms of the same kernels (accumulating reduce copy-in, "
+                         "post-reduce as a copy, same-dtype copies, in-place divide, each launch alone)")
+    for old in ("--no-stream-plan", "--no-store-policy-ab", "--no-rotating-sets", "--no-graph"):
+        ap.add_argument(old, action="store_true", help=argparse.SUPPRESS)  # these legs are off unless asked for
     ap.add_argument("--no-torch-gpu", action="store_true",
                     help="skip the leg that times the reference's torch ops on the GPU (outside the timed region)")
     ap.add_argument("--sweep-grid-cap", action="store_true",
@@ -1349,21 +1392,20 @@ def main() -> int:
     ap.add_argument("--no-configs", action="store_true",
                     help="default workload only: skip the `configs` block (the other configurations of the path, each "
                          "with its own oracle check, about a minute in total)")
-    ap.add_argument("--sustained-seconds", type=float, default=1.5,
-                    help="length of the sustained leg: back-to-back steps of the workload for at least this long "
-                         "(0 disables it)")
+    ap.add_argument("--sustained-seconds", type=float, default=0.0,
+                    help="add a sustained leg: back-to-back rotating steps of the workload for at least this long")
     ap.add_argument("--table-large-log2", type=int, default=None, metavar="N",
                     help="tables with more than 2^N padded elements run two waves per workgroup instead of one "
                          "(the library's launch-shape option; default: the library's own threshold)")
     ap.add_argument("--gather-tail-mb", type=int, default=None, metavar="N",
                     help="megabytes at the end of the reduce buffer that the reduce copy-in stores write-through "
-                         "(the library's store-policy option; default: the library's own, 96; 0 = none)")
+                         "(the library's store-policy option; default: the library's own, 64; 0 = none)")
     ap.add_argument("--scatter-tail-mb", type=int, default=None, metavar="N",
                     help="the same for the last megabytes of tensors that copy-out writes (default: the library's "
                          "own, 0 = none)")
     ap.add_argument("--flat-tail-mb", type=int, default=None, metavar="N",
-                    help="the same for the flat kernels (copy-in, post-reduce), which write through everywhere by "
-                         "default; 0 = they store everything non-temporal")
+                    help="the same for the flat kernels (copy-in, flat copies and divides; default 0: they store "
+                         "everything non-temporal; 1048576 = write-through everywhere)")
     ap.add_argument("--post-reduce-tail-mb", type=int, default=None, metavar="N", help="the same for the post-reduce")
     ap.add_argument("--analyze-trace", metavar="CSV", default=None,
                     help="llama3-8b-full-w8 only: no GPU work; summarise the kernel-trace CSV that rocprofv3 wrote for "
@@ -1391,9 +1433,6 @@ def main() -> int:
         if value is not None:  # the library's store-policy options, for every workload
             _native.set_option(option, value)
     if args.workload == "llama3-8b-full-w8":
-        if all(v is None for v in (args.gather_tail_mb, args.scatter_tail_mb, args.flat_tail_mb,
-                                   args.post_reduce_tail_mb)):
-            _native.set_store_policy("rotating_sets")  # 35 groups on shared buffers: what fully_shard selects
         return run_full_model(args)
     if args.workload.endswith("-optim"):
         return run_optim(args)
@@ -1418,12 +1457,7 @@ def main() -> int:
                 log(f"config {wl}: {out['configs'][wl]['value']} GB/s, {time.perf_counter() - t0:.1f}s wall")
             # the full-model pass next to GEMMs on a second stream (its own oracle check of an overlapped pass)
             t0 = time.perf_counter()
-            in_force = _native.get_store_policy()
-            _native.set_store_policy("rotating_sets")  # 35 groups on shared buffers: what fully_shard selects
-            try:
-                rec = run_full_model(args, as_record=True)
-            finally:
-                _native.set_store_policy(in_force)
+            rec = run_full_model(args, as_record=True)
             if not isinstance(rec, dict):
                 raise ParityError("llama3-8b-full-w8: the overlapped pass differs from the oracle")
             out["configs"]["llama3-8b-full-w8"] = rec
@@ -1451,9 +1485,10 @@ def cpu_model() -> str:
 
 def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -> dict:
     """One parameter group's pass (copy-in, copy-out, reduce copy-in, post-reduce) on synthetic inputs of the named
-    workload: parity against the oracle, `warmup` untimed and `steps` timed passes.  `full` adds the per-kernel
-    tables, the sustained leg, graph replay and the baselines; without it only the timed passes and the parity
-    check run, and a compact record comes back."""
+    workload, over ``--buffer-sets`` sets of buffers taking turns (step k runs on set k mod K): parity of every set
+    against the oracle, `warmup` untimed and `steps` timed passes.  `full` adds the per-kernel table, the one-set
+    loop and the baselines (and the legs asked for by flags); without it only the timed passes and the parity check
+    run, and a compact record comes back."""
     import torch
 
     from yafsdp_amd import _native
@@ -1479,7 +1514,9 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     lay = make_layout(numels, w, align)
     t, t_pad, s = lay.total_numel, lay.padded_unsharded_numel, lay.padded_sharded_numel
     pre = float(w) if w > 1 else None
-    log(f"workload {workload}: P={len(numels)} T={t} T_pad={t_pad} S={s} W={w} rank={r} pre-divide={pre}")
+    n_sets = max(1, args.buffer_sets)
+    log(f"workload {workload}: P={len(numels)} T={t} T_pad={t_pad} S={s} W={w} rank={r} pre-divide={pre}, "
+        f"{n_sets} buffer set(s) in rotation")
 
     # ---- synthetic inputs, generated on the CPU so that the oracle sees the same bits
     g = torch.Generator().manual_seed(seed)
@@ -1496,75 +1533,86 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     shard0 = (torch.randn(s, generator=g) * 1e-4).to(master_dt)  # existing gradient shard (master dtype)
     log(f"inputs generated in {time.perf_counter() - t0:.1f}s")
 
-    d_master = master.to(dev)
-    d_gathered = gathered.to(dev)
-    d_grads = [x.to(dev) for x in grads]
-    d_ag_in = torch.zeros(s, dtype=torch.bfloat16, device=dev)
-    d_outs = [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels]
-    d_rs = torch.zeros(t_pad, dtype=rs_dt, device=dev)
-    d_shard = shard0.to(dev)
-    d_chunk = d_rs[r * s : (r + 1) * s]
     table = _native.TensorTable(numels, t_pad, dev)
-    # the copy-out destinations persist across steps: their side of the table is bound once.  Gradients are fresh
-    # allocations of autograd in a training step, so the reduce copy-in passes its pointers on every call.
-    out_binding = table.bind(d_outs)
 
-    def op_copy_in():
-        _native.flat_copy(d_ag_in, d_master)
+    # ---- K sets of buffers: the first from the host inputs, the others device copies of it at their own addresses.
+    # A training run never comes back to a buffer before gigabytes of other traffic have passed (the reference's
+    # groups take turns on two gathered buffers and one reduce buffer, ya_fsdp/_state.py:636-652): with ONE set
+    # rewritten step after step a kernel finds what the step before left in the 256-MB memory-side cache, which
+    # flatters it.  The timed region therefore rotates over K sets (2 GB each for the default workload).
+    def first_set():
+        d = {"master": master.to(dev), "gathered": gathered.to(dev), "grads": [x.to(dev) for x in grads],
+             "ag_in": torch.zeros(s, dtype=torch.bfloat16, device=dev),
+             "outs": [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels],
+             "rs": torch.zeros(t_pad, dtype=rs_dt, device=dev), "shard": shard0.to(dev)}
+        return d
 
-    def op_copy_out():
-        out_binding.scatter_out(d_gathered)
+    def another_set(d0):
+        return {"master": d0["master"].clone(), "gathered": d0["gathered"].clone(),
+                "grads": [x.clone() for x in d0["grads"]], "ag_in": torch.zeros_like(d0["ag_in"]),
+                "outs": [torch.empty_like(x) for x in d0["outs"]], "rs": torch.zeros_like(d0["rs"]),
+                "shard": shard0.to(dev)}
 
-    def op_reduce_copy_in():
-        table.gather_in(d_grads, d_rs, None, pre, True)
+    sets = [first_set()]
+    for _ in range(n_sets - 1):
+        sets.append(another_set(sets[0]))
+    fused_unshard = has_copy_in and not args.no_fused
+    fused_reduce = w == 1 and has_copy_in and not args.no_fused
+    for d in sets:
+        d["chunk"] = d["rs"][r * s : (r + 1) * s]
+        # the copy-out destinations persist across steps: their side of the table is bound once.  Gradients are
+        # fresh allocations of autograd in a training step, so the reduce copy-in passes its pointers on every call.
+        d["out_binding"] = table.bind(d["outs"])
 
-    def op_post_reduce():
-        _native.post_reduce(d_shard, d_chunk, None, True)
+    copy_in_bytes, copy_out_bytes = s * (msz + 2), 2 * t * 2
+    gather_bytes, post_bytes = t * (2 + rsz) + (t_pad - t) * rsz, s * (rsz + 2 * msz)
 
-    ops = [
-        ("copy_in", op_copy_in, s * (msz + 2)),
-        ("copy_out", op_copy_out, 2 * t * 2),
-        ("reduce_copy_in", op_reduce_copy_in, t * (2 + rsz) + (t_pad - t) * rsz),
-        ("post_reduce", op_post_reduce, s * (rsz + 2 * msz)),
-    ]
-    if not has_copy_in:  # the all-gather input aliases the master shard (ya_fsdp/_param_group.py:502-505)
-        ops = ops[1:]
-    bytes_per_step = sum(b for _, _, b in ops)  # what the reference's four ops move, however many launches do it
-    dominant = "reduce_copy_in"
-    fused = False
-    if w == 1 and has_copy_in and not args.no_fused:
-        # a shard group of size one: copy-in + copy-out as one launch, reduce copy-in + post-reduce as one launch
-        # (nothing happens between the two halves of either pair, ya_fsdp/_collectives.py:140-150)
-        def op_unshard():
-            if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
+    def ops_of(d):
+        """(name, launch, algorithmic bytes) of one step on buffer set d."""
+        def unshard():
+            if not table.copy_in_scatter_out(d["gathered"], d["outs"], d["ag_in"], d["master"]):
                 raise RuntimeError("copy_in_scatter_out declined")
 
-        def op_reduce():
-            if not table.gather_in_post_reduce(d_grads, d_rs, d_shard, True):
+        def reduce_one_launch():
+            if not table.gather_in_post_reduce(d["grads"], d["rs"], d["shard"], True):
                 raise RuntimeError("gather_in_post_reduce declined")
 
-        ops = [
-            ("copy_in_and_copy_out", op_unshard, ops[0][2] + ops[1][2]),
-            ("reduce_copy_in_and_post_reduce", op_reduce, ops[2][2] + ops[3][2]),
-        ]
-        dominant, fused = "reduce_copy_in_and_post_reduce", True
-    elif has_copy_in and not args.no_fused:
-        # any group size: copy-in and copy-out as one grid (both sit back to back on the all-gather stream in the
-        # reference, ya_fsdp/_collectives.py:46-58 and ya_fsdp/_param_group.py:581-594)
-        def op_unshard_w():
-            if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
-                raise RuntimeError("copy_in_scatter_out declined")
+        ops = []
+        if fused_unshard:
+            # copy-in and copy-out as one grid (both sit back to back on the all-gather stream in the reference,
+            # ya_fsdp/_collectives.py:46-58 and ya_fsdp/_param_group.py:581-594)
+            ops.append(("copy_in_and_copy_out", unshard, copy_in_bytes + copy_out_bytes))
+        else:
+            if has_copy_in:  # otherwise the all-gather input aliases the master shard (ya_fsdp/_param_group.py:502-505)
+                ops.append(("copy_in", lambda: _native.flat_copy(d["ag_in"], d["master"]), copy_in_bytes))
+            ops.append(("copy_out", lambda: d["out_binding"].scatter_out(d["gathered"]), copy_out_bytes))
+        if fused_reduce:
+            # a shard group of size one: nothing happens between reduce copy-in and post-reduce
+            # (ya_fsdp/_collectives.py:140-150), one launch does both
+            ops.append(("reduce_copy_in_and_post_reduce", reduce_one_launch, gather_bytes + post_bytes))
+        else:
+            ops.append(("reduce_copy_in", lambda: table.gather_in(d["grads"], d["rs"], None, pre, True), gather_bytes))
+            ops.append(("post_reduce", lambda: _native.post_reduce(d["shard"], d["chunk"], None, True), post_bytes))
+        return ops
 
-        ops = [("copy_in_and_copy_out", op_unshard_w, ops[0][2] + ops[1][2])] + ops[2:]
-        fused = True
+    set_ops = [ops_of(d) for d in sets]
+    set_fns = [[fn for _, fn, _ in ops] for ops in set_ops]
+    op_names = [n for n, _, _ in set_ops[0]]
+    op_bytes = [b for _, _, b in set_ops[0]]
+    # what the reference's four ops move, however many launches do it
+    bytes_per_step = (copy_in_bytes if has_copy_in else 0) + copy_out_bytes + gather_bytes + post_bytes
+    dominant = "reduce_copy_in_and_post_reduce" if fused_reduce else "reduce_copy_in"
+    dom_index = op_names.index(dominant)
 
-    def step():
-        for _, fn, _ in ops:
+    def step(k=0):
+        for fn in set_fns[k % n_sets]:
             fn()
 
-    # ---- parity of one pass against the oracle (same run, same inputs)
+    # ---- parity of one pass on EVERY buffer set (same run, same inputs): the first set against the oracle on the
+    # host, the others against the first on the device (they hold copies of the same inputs)
     parity = "skipped"
     cpu_state = None
+    cpu_step = None
     if not args.no_parity:
         from oracle import torch_ops
 
@@ -1584,59 +1632,69 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             "shard": shard0.clone(),
         }
         cpu_step(cpu_state)
-        step()
+        for k in range(n_sets):
+            step(k)
         torch.cuda.synchronize()
 
-        def same(a, b):
-            iv = torch.int32 if a.dtype == torch.float32 else torch.int16
-            return torch.equal(a.cpu().view(iv), b.view(iv))
+        def bits(a):
+            return a.view(torch.int32 if a.dtype == torch.float32 else torch.int16)
 
-        ok = same(d_ag_in, cpu_state["ag_in"]) and same(d_rs, cpu_state["rs"]) and same(d_shard, cpu_state["shard"])  # noqa: E501 (d_ag_in stays zero on both sides without a copy-in)
-        ok = ok and all(same(a, b) for a, b in zip(d_outs, cpu_state["outs"]))
+        def same(a, b):
+            return torch.equal(bits(a.cpu()), bits(b))
+
+        d0 = sets[0]
+        ok = same(d0["ag_in"], cpu_state["ag_in"]) and same(d0["rs"], cpu_state["rs"]) and same(d0["shard"], cpu_state["shard"])  # noqa: E501 (ag_in stays zero on both sides without a copy-in)
+        ok = ok and all(same(a, b) for a, b in zip(d0["outs"], cpu_state["outs"]))
+        for d in sets[1:]:
+            ok = ok and all(torch.equal(bits(d[key]), bits(d0[key])) for key in ("ag_in", "rs", "shard"))
+            ok = ok and all(torch.equal(bits(a), bits(b)) for a, b in zip(d["outs"], d0["outs"]))
         parity = "bit-exact" if ok else "MISMATCH"
-        log("parity vs oracle:", parity)
+        log(f"parity vs oracle ({n_sets} buffer sets):", parity)
         if not ok:
             raise ParityError(f"{workload}: GPU results differ from the oracle")
 
     if args.calibrate_copy > 0:
         d_copy = torch.empty(t_pad, dtype=torch.bfloat16, device=dev)
         for _ in range(args.calibrate_copy):
-            _native.flat_copy(d_copy, d_gathered)
+            _native.flat_copy(d_copy, sets[0]["gathered"])
         torch.cuda.synchronize()
         del d_copy
 
-    # ---- timed region: `warmup` untimed steps, then exactly `steps` steps between two synchronisations.  The region
-    # is run --regions times (3 unless told otherwise) and the MEDIAN region is the one reported (all are listed in
-    # the line): the step is driven from the host, a region lasts a few milliseconds, and one stall of the host or
-    # the machine inside it (seen once in about twenty runs: 25 ms of idle GPU in a 16-ms region, with every
-    # sampled kernel at its normal duration) would otherwise decide the figure.
-    # the kernel `roofline` reports: the reduce copy-in, the launch with the path's arithmetic fused in (cast, divide,
-    # pad fill) and the lowest fraction of the step's launches (the shared copy-in + copy-out launch moves more bytes
-    # at a higher rate; every launch is in `kernels`)
-    dom_index = [n for n, _, _ in ops].index(dominant)
-    # on every 4th step of the timed region (of a long region: on 16 steps spread evenly; attaching the pair costs
-    # host time that a launch-bound workload would see) the dominant kernel's dispatch carries a pair of HIP events
-    # (attached to the dispatch itself: kernel begin and end on the stream it runs on, no launch gap inside the pair)
+    # ---- timed region: `warmup` untimed steps, then exactly `steps` steps between two synchronisations, step k on
+    # buffer set k mod K.  The region is run --regions times (3 unless told otherwise) and the MEDIAN region is the
+    # one reported (all are listed in the line): the step is driven from the host, a region lasts a few
+    # milliseconds, and one stall of the host or the machine inside it (seen once in about twenty runs: 25 ms of
+    # idle GPU in a 16-ms region, with every sampled kernel at its normal duration) would otherwise decide the figure.
+    # The kernel `roofline` reports is the reduce copy-in, the launch with the path's arithmetic fused in (cast,
+    # divide, pad fill) and the lowest fraction of the step's launches (every launch is in `kernels`).  On every 4th
+    # step of the timed region (of a long region: on 16 steps spread evenly; attaching the pair costs host time that
+    # a launch-bound workload would see) its dispatch carries a pair of HIP events (attached to the dispatch itself:
+    # kernel begin and end on the stream it runs on, no launch gap inside the pair).
     every = max(4, -(-steps // (16 if full else 4)))  # the compact records of the other configurations: 4 samples
+    if n_sets > 1 and every % n_sets == 0:
+        every += 1  # the samples then fall on every buffer set in turn
     sampled = [k for k in range(steps) if k % every == 0]
-    fns = [fn for _, fn, _ in ops]
 
-    def timed_region():
+    def timed_region(first=0, rotate=True):
+        def fns_of(k):
+            return set_fns[(first + k) % n_sets] if rotate else set_fns[first]
+
         for w_ in range(warmup):
             if w_ == 0:  # the event-carrying dispatch path runs once before anything is timed
                 prime = _event_pair()
-                for i, fn in enumerate(fns):
+                for i, fn in enumerate(fns_of(w_)):
                     if i == dom_index:
                         _native.time_next_launch(*prime)
                     fn()
                 continue
-            step()
+            for fn in fns_of(w_):
+                fn()
         torch.cuda.synchronize()
         ev = {k: _event_pair() for k in sampled}
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for k in range(steps):
-            for i, fn in enumerate(fns):
+            for i, fn in enumerate(fns_of(warmup + k)):
                 if i == dom_index and k in ev:
                     _native.time_next_launch(*ev[k])
                 fn()
@@ -1650,359 +1708,247 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
     ms_per_step = elapsed * 1e3 / steps
     value = bytes_per_step * steps / elapsed / 1e9
     dom_avg_us = sum(dom_us) / len(dom_us)
-    dom_bytes = ops[dom_index][2]
+    dom_bytes = op_bytes[dom_index]
     achieved = dom_bytes / dom_avg_us / 1e3
 
-    if not full:
-        out_binding.close()
+    def close_all():
+        for d in sets:
+            d["out_binding"].close()
         table.close()
+
+    def rate(ms):
+        return {"ms_per_step": round(ms, 4), "value": round(bytes_per_step / ms / 1e6, 1), "unit": "GB/s",
+                "frac_of_hbm_peak": round(bytes_per_step / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    if not full:
+        close_all()
         return {
             "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms_per_step, 4), "steps": steps,
             "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4), "parity": parity, "bytes_per_step": bytes_per_step,
             "params": len(numels), "padded_numel": t_pad, "shard_numel": s, "logical_world_size": w,
+            "buffer_sets": n_sets,
             "dominant_kernel_us": round(dom_avg_us, 2), "dominant_kernel_GBps": round(achieved, 1),
-            "launches_per_step": len(ops), "dominant_kernel": dominant,
+            "launches_per_step": len(op_names), "dominant_kernel": dominant,
             "timed_regions_ms_per_step": region_ms_per_step,
         }
 
-    # ---- sustained leg: back-to-back steps for at least --sustained-seconds (outside the timed region above; the
-    # same eager calls, long enough for clocks and the memory system to settle)
+    # ---- ONE buffer set rewritten step after step (outside the timed region): the loop finds part of its own output
+    # in the memory-side cache, so this is NOT a rate a training run sees.  Under the library's defaults, and under
+    # the opt-in policy tuned to exactly this loop ("single_set": write-through everywhere in the flat kernels and a
+    # 96-MB tail of the reduce buffer).
+    one_set = None
+    if n_sets > 1:
+        one_ms = timed_region(rotate=False)[0] * 1e3 / steps
+        in_force = _native.get_store_policy()
+        try:
+            _native.set_store_policy("single_set")
+            tuned_ms = timed_region(rotate=False)[0] * 1e3 / steps
+        finally:
+            _native.set_store_policy(in_force)
+        one_set = {"note": "cache-assisted: one buffer set rewritten step after step finds its own output in the "
+                           "256-MB memory-side cache; not the headline",
+                   "steps": steps, **rate(one_ms), "store_policy_single_set": rate(tuned_ms)}
+        log(f"one buffer set (cache-assisted): {one_set['ms_per_step']} ms per step, {one_set['value']} GB/s; under "
+            f"the single_set store policy {tuned_ms:.4f} ms")
+        for k in range(max(1, warmup)):  # the legs below start from the rotation's steady state
+            step(k)
+        torch.cuda.synchronize()
+
+    # ---- sustained leg (--sustained-seconds): back-to-back rotating steps for at least that long
     sustained = None
     if args.sustained_seconds > 0:
         n_sus = max(steps, int(args.sustained_seconds / (ms_per_step * 1e-3)) + 1)
         torch.cuda.synchronize()
         s0 = time.perf_counter()
-        for _ in range(n_sus):
-            for fn in fns:
+        for k in range(n_sus):
+            for fn in set_fns[k % n_sets]:
                 fn()
         torch.cuda.synchronize()
         s_dt = time.perf_counter() - s0
-        sustained = {"steps": n_sus, "seconds": round(s_dt, 3), "ms_per_step": round(s_dt * 1e3 / n_sus, 4),
-                     "value": round(bytes_per_step * n_sus / s_dt / 1e9, 1), "unit": "GB/s",
-                     "frac_of_hbm_peak": round(bytes_per_step * n_sus / s_dt / 1e9 / HBM_PEAK_GBS, 4)}
+        sustained = {"steps": n_sus, "seconds": round(s_dt, 3), **rate(s_dt * 1e3 / n_sus)}
         log(f"sustained: {n_sus} steps in {s_dt:.2f}s, {sustained['value']} GB/s")
 
-    # ---- the same step with the write-through tails of copy-out and reduce copy-in switched off (outside the timed
-    # region): the library's default writes the end of each of the two big outputs through the L2s, which shortens
-    # those kernels and leaves the write-back to overlap what follows; this leg shows what the choice is worth on this
-    # workload
-    tail_off = None
-    if not args.no_store_policy_ab:
-        tail_mb = _native.get_option(_native.OPT_GATHER_TAIL_MB)
-        scatter_tail_mb = _native.get_option(_native.OPT_SCATTER_TAIL_MB)
-        _native.set_option(_native.OPT_GATHER_TAIL_MB, 0)
-        _native.set_option(_native.OPT_SCATTER_TAIL_MB, 0)
+    # ---- store policies in rotation (--store-policy-ab): the same rotating loop under other tail settings
+    policy_ab = None
+    if args.store_policy_ab:
+        policy_ab = {}
+        in_force = _native.get_store_policy()
         try:
-            n_ab = max(steps, 1000)  # long enough for its closing synchronisation not to show (compare: sustained)
-            for _ in range(max(1, warmup)):
-                step()
-            torch.cuda.synchronize()
-            a0 = time.perf_counter()
-            for _ in range(n_ab):
-                for fn in fns:
-                    fn()
-            torch.cuda.synchronize()
-            a_dt = (time.perf_counter() - a0) / n_ab
+            for name, pol in (("all_stores_non_temporal", (0, 0, 0, 0)), ("gather_tail_128", (0, 0, 0, 128)),
+                              ("single_set", "single_set")):
+                _native.set_store_policy(pol)
+                policy_ab[name] = rate(timed_region()[0] * 1e3 / steps)
         finally:
-            _native.set_option(_native.OPT_GATHER_TAIL_MB, tail_mb)
-            _native.set_option(_native.OPT_SCATTER_TAIL_MB, scatter_tail_mb)
-        for _ in range(max(1, warmup)):  # the legs below start from the default policy's steady state
-            step()
-        torch.cuda.synchronize()
-        tail_off = {"steps": n_ab, "ms_per_step": round(a_dt * 1e3, 4), "value": round(bytes_per_step / a_dt / 1e9, 1),
-                    "unit": "GB/s", "default_scatter_tail_mb": scatter_tail_mb, "default_gather_tail_mb": tail_mb}
-        log(f"without the write-through tails: {tail_off['ms_per_step']} ms per step, {tail_off['value']} GB/s "
-            f"(default: last {scatter_tail_mb} MB of copy-out and last {tail_mb} MB of reduce copy-in write through)")
+            _native.set_store_policy(in_force)
+        policy_ab["in_force"] = {"policy": list(in_force), **rate(ms_per_step)}
+        log("store policies in rotation: " + ", ".join(f"{k} {v['ms_per_step']} ms" for k, v in policy_ab.items()))
 
-    # ---- the same step alternating between TWO sets of buffers (outside the timed region), as the reference's
-    # parameter groups alternate between two shared gathered buffers and two shared reduce buffers
-    # (ya_fsdp/_state.py:636-652).  The timed region above rewrites ONE set step after step, so whatever its kernels
-    # leave in the 256-MB memory-side cache (written-through lines above all) is still there when the next step
-    # reads or overwrites the same addresses; with two sets 2.2 GB of other traffic lie between two visits.
-    rotating = None
-    if not args.no_rotating_sets:
-        try:
-            n_sets = max(2, args.rotating_sets)
-
-            def more_buffers():
-                d = {"master": d_master.clone(), "ag_in": torch.empty_like(d_ag_in), "gathered": d_gathered.clone(),
-                     "outs": [torch.empty_like(x) for x in d_outs], "grads": [x.clone() for x in d_grads],
-                     "rs": torch.zeros_like(d_rs), "shard": d_shard.clone()}
-                d["chunk"] = d["rs"][r * s : (r + 1) * s]
-                return d
-
-            others = [more_buffers() for _ in range(n_sets - 1)]
-
-            def step_on(d):
-                if fused and w == 1:
-                    ok = table.copy_in_scatter_out(d["gathered"], d["outs"], d["ag_in"], d["master"])
-                    ok = ok and table.gather_in_post_reduce(d["grads"], d["rs"], d["shard"], True)
-                    if not ok:
-                        raise RuntimeError("shared launch declined")
-                    return
-                if fused:
-                    if not table.copy_in_scatter_out(d["gathered"], d["outs"], d["ag_in"], d["master"]):
-                        raise RuntimeError("copy_in_scatter_out declined")
-                else:
-                    if has_copy_in:
-                        _native.flat_copy(d["ag_in"], d["master"])
-                    table.scatter_out(d["gathered"], d["outs"])
-                table.gather_in(d["grads"], d["rs"], None, pre, True)
-                _native.post_reduce(d["shard"], d["chunk"], None, True)
-
-            def alternating_ms_per_step(n_rounds):
-                for _ in range(max(1, warmup // n_sets)):
-                    step()
-                    for d in others:
-                        step_on(d)
-                torch.cuda.synchronize()
-                q0 = time.perf_counter()
-                for _ in range(n_rounds):
-                    step()
-                    for d in others:
-                        step_on(d)
-                torch.cuda.synchronize()
-                return (time.perf_counter() - q0) / (n_sets * n_rounds) * 1e3
-
-            # under the store policy in force (the library's default unless options were given), under the policy
-            # that fully_shard selects for several parameter groups, and with every store non-temporal
-            n_pairs = max(steps, 1000) // n_sets
-            in_force = _native.get_store_policy()
-            rot_ms = alternating_ms_per_step(n_pairs)
-            try:
-                _native.set_store_policy("rotating_sets")
-                rot_policy_ms = alternating_ms_per_step(n_pairs)
-                _native.set_store_policy((0, 0, 0, 0))
-                rot_plain_ms = alternating_ms_per_step(n_pairs)
-            finally:
-                _native.set_store_policy(in_force)
-            for _ in range(max(1, warmup)):  # the legs below start from the single set's steady state
-                step()
-            torch.cuda.synchronize()
-
-            def rate(ms):
-                return {"ms_per_step": round(ms, 4), "value": round(bytes_per_step / ms / 1e6, 1), "unit": "GB/s",
-                        "frac_of_hbm_peak": round(bytes_per_step / ms / 1e6 / HBM_PEAK_GBS, 4)}
-
-            rotating = {"sets": n_sets, "steps": n_sets * n_pairs, "store_policy_in_force": list(in_force), **rate(rot_ms),
-                        "store_policy_rotating_sets": rate(rot_policy_ms),
-                        "all_stores_non_temporal": rate(rot_plain_ms)}
-            log(f"{n_sets} buffer sets in rotation: {rotating['ms_per_step']} ms per step, {rotating['value']} GB/s; "
-                f"under the rotating-sets store policy {rot_policy_ms:.4f} ms, all stores non-temporal "
-                f"{rot_plain_ms:.4f} ms")
-            del others
-        except Exception as exc:  # an optional leg must not cost the measurement above
-            log(f"rotating-sets leg skipped: {type(exc).__name__}: {exc}")
-            rotating = None
-
-    # ---- the same launches on the streams the reference puts them on (outside the timed region): copy-in and
-    # copy-out on the side stream that serves all-gather and reduce-scatter (ya_fsdp/_collectives.py:46,
+    # ---- the same launches on the streams the reference puts them on (--stream-plan): copy-in and copy-out on the
+    # side stream that serves all-gather and reduce-scatter (ya_fsdp/_collectives.py:46,
     # ya_fsdp/_param_group.py:80-88), the reduce copy-in on the compute stream (ya_fsdp/_param_group.py:669-708), the
-    # post-reduce on the side stream once the compute stream has got there (ya_fsdp/_collectives.py:110-111).  The
-    # timed region above keeps one stream, where the kernels' own durations add up to the step; here independent
-    # kernels overlap their ramps and drains.
+    # post-reduce on the side stream once the compute stream has got there (ya_fsdp/_collectives.py:110-111).
     reference_streams = None
-    if not args.no_stream_plan:
-        try:
-            main_stream, side_stream = torch.cuda.current_stream(dev), torch.cuda.Stream(device=dev)
+    if args.stream_plan:
+        main_stream, side_stream = torch.cuda.current_stream(dev), torch.cuda.Stream(device=dev)
 
-            def reference_step():
-                done = None
-                for name, fn, _ in ops:
-                    if name.startswith("reduce_copy_in"):
+        def reference_step(k):
+            done = None
+            for name, fn in zip(op_names, set_fns[k % n_sets]):
+                if name.startswith("reduce_copy_in"):
+                    fn()
+                    done = main_stream.record_event()
+                else:
+                    with torch.cuda.stream(side_stream):
+                        if name == "post_reduce" and done is not None:
+                            side_stream.wait_event(done)
                         fn()
-                        done = main_stream.record_event()
-                    else:
-                        with torch.cuda.stream(side_stream):
-                            if name == "post_reduce" and done is not None:
-                                side_stream.wait_event(done)
-                            fn()
 
-            n_ref = max(steps, 200)
-            side_stream.wait_stream(main_stream)
-            for _ in range(warmup):
-                reference_step()
-            main_stream.wait_stream(side_stream)
-            torch.cuda.synchronize()
-            r0 = time.perf_counter()
-            for _ in range(n_ref):
-                reference_step()
-            main_stream.wait_stream(side_stream)
-            torch.cuda.synchronize()
-            r_dt = (time.perf_counter() - r0) / n_ref
-            reference_streams = {
-                "plan": "copy-in + copy-out and post-reduce on a side stream, reduce copy-in on the compute stream",
-                "steps": n_ref, "ms_per_step": round(r_dt * 1e3, 4), "value": round(bytes_per_step / r_dt / 1e9, 1),
-                "unit": "GB/s", "frac_of_hbm_peak": round(bytes_per_step / r_dt / 1e9 / HBM_PEAK_GBS, 4)}
-            log(f"the reference's stream placement: {reference_streams['ms_per_step']} ms per step, "
-                f"{reference_streams['value']} GB/s")
-            if not args.no_parity and cpu_state is not None:
-                # the overlapped launches left the same bits (the gradient shard has accumulated many passes:
-                # compare the buffers that every pass rewrites)
-                ok = same(d_ag_in, cpu_state["ag_in"]) and same(d_rs, cpu_state["rs"])
-                ok = ok and all(same(a, b) for a, b in zip(d_outs, cpu_state["outs"]))
-                if not ok:
-                    raise ParityError(f"{workload}: results of the two-stream step differ from the oracle")
-        except ParityError:
-            raise
-        except Exception as exc:  # an optional leg must not cost the measurement above
-            log(f"stream placement leg skipped: {type(exc).__name__}: {exc}")
-            reference_streams = None
+        n_ref = max(steps, 200)
+        side_stream.wait_stream(main_stream)
+        for k in range(warmup):
+            reference_step(k)
+        main_stream.wait_stream(side_stream)
+        torch.cuda.synchronize()
+        r0 = time.perf_counter()
+        for k in range(n_ref):
+            reference_step(k)
+        main_stream.wait_stream(side_stream)
+        torch.cuda.synchronize()
+        r_dt = (time.perf_counter() - r0) / n_ref
+        reference_streams = {
+            "plan": "copy-in + copy-out and post-reduce on a side stream, reduce copy-in on the compute stream",
+            "steps": n_ref, **rate(r_dt * 1e3)}
+        log(f"the reference's stream placement: {reference_streams['ms_per_step']} ms per step, "
+            f"{reference_streams['value']} GB/s")
+        if not args.no_parity and cpu_state is not None:
+            # the overlapped launches left the same bits (the gradient shard has accumulated many passes:
+            # compare the buffers that every pass rewrites)
+            d0 = sets[0]
+            ok = same(d0["ag_in"], cpu_state["ag_in"]) and same(d0["rs"], cpu_state["rs"])
+            ok = ok and all(same(a, b) for a, b in zip(d0["outs"], cpu_state["outs"]))
+            if not ok:
+                raise ParityError(f"{workload}: results of the two-stream step differ from the oracle")
 
-    # ---- the same step captured into a HIP graph and replayed (outside the timed region): both sides of the table
-    # are bound, so the captured launches carry no per-call host work and no staging copy
+    # ---- the rotating steps captured into HIP graphs and replayed (--graph): one graph of K steps (one per buffer
+    # set) and one of 4 K steps; both sides of the table are bound, so the captured launches carry no per-call host
+    # work and no staging copy.  A graph launch has a fixed cost of its own (a few microseconds of idle GPU at its
+    # start and end), which the longer graph spreads over four times as many steps.
     graph_replay = None
-    if not args.no_graph:
-        try:
-            grad_binding = table.bind(d_grads)
+    if args.graph:
+        grad_bindings = [table.bind(d["grads"]) for d in sets]
 
-            def bound_step():
-                if fused and len(numels) <= 16:  # small tables carry their pointers as kernel arguments
-                    for f in fns:
-                        f()
-                    return
-                if has_copy_in:
-                    _native.flat_copy(d_ag_in, d_master)
-                out_binding.scatter_out(d_gathered)
-                grad_binding.gather_in(d_rs, pre, True)
-                _native.post_reduce(d_shard, d_chunk, None, True)
+        def bound_step(k):
+            d, gb = sets[k % n_sets], grad_bindings[k % n_sets]
+            if fused_unshard and len(numels) <= 16:  # small tables carry their pointers as kernel arguments
+                for f in set_fns[k % n_sets]:
+                    f()
+                return
+            if has_copy_in:
+                _native.flat_copy(d["ag_in"], d["master"])
+            d["out_binding"].scatter_out(d["gathered"])
+            gb.gather_in(d["rs"], pre, True)
+            _native.post_reduce(d["shard"], d["chunk"], None, True)
 
+        graph_replay = {}
+        for rounds in (1, 4):
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                bound_step()
+                for k in range(n_sets):
+                    bound_step(k)
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                bound_step()
+                for k in range(rounds * n_sets):
+                    bound_step(k)
             for _ in range(3):
                 graph.replay()
             torch.cuda.synchronize()
+            n_rep = max(1, steps // (rounds * n_sets))
             g0 = time.perf_counter()
-            for _ in range(steps):
+            for _ in range(n_rep):
                 graph.replay()
             torch.cuda.synchronize()
-            g_dt = (time.perf_counter() - g0) / steps
-            graph_replay = {"ms_per_step": round(g_dt * 1e3, 4), "value": round(bytes_per_step / g_dt / 1e9, 1), "unit": "GB/s"}
-            log(f"HIP graph replay of the step: {graph_replay['ms_per_step']} ms, {graph_replay['value']} GB/s")
+            g_dt = (time.perf_counter() - g0) / (n_rep * rounds * n_sets)
+            graph_replay[f"{rounds * n_sets}_steps_per_graph"] = rate(g_dt * 1e3)
             del graph
-            grad_binding.close()
-        except Exception as exc:  # an optional leg must not cost the measurement above
-            log(f"HIP graph leg skipped: {type(exc).__name__}: {exc}")
-            graph_replay = None
+        for gb in grad_bindings:
+            gb.close()
+        log("HIP graph replay: " + ", ".join(f"{k}: {v['ms_per_step']} ms per step" for k, v in graph_replay.items()))
 
-    # ---- per-kernel table (outside the timed region): each op's dispatch timed on its own
-    tail_options = (_native.OPT_SCATTER_TAIL_MB, _native.OPT_GATHER_TAIL_MB)
-
-    def time_alone(fn, others, reps=20, plain_evictors=False):
-        """Durations of `fn`'s own dispatch, each right behind the launches `others`.  plain_evictors: those run with
-        their write-through tails off, so that the sample does not inherit the megabytes which they would leave in
-        the memory-side cache for later write-back."""
-        times = []
-        tails = [_native.get_option(o) for o in tail_options]
-        for _ in range(reps):
+    # ---- per-kernel table (outside the timed region): every launch of 4 K rotating steps carries an event pair on
+    # its own dispatch, so each kernel is rated as it runs inside the rotation
+    samples = {n: [] for n in op_names}
+    pairs = []
+    for k in range(4 * n_sets):
+        for name, fn in zip(op_names, set_fns[k % n_sets]):
             a, b = _event_pair()
-            if plain_evictors:
-                for o in tail_options:
-                    _native.set_option(o, 0)
-            try:
-                for f in others:  # evict: the other ops stream 1-2 GB through the caches
-                    f()
-            finally:
-                for o, v in zip(tail_options, tails):
-                    _native.set_option(o, v)
             _native.time_next_launch(a, b)
             fn()
-            torch.cuda.synchronize()
-            times.append(a.elapsed_time(b) * 1e3)
-        return times
-
+            pairs.append((name, a, b))
+    torch.cuda.synchronize()
+    for name, a, b in pairs:
+        samples[name].append(a.elapsed_time(b) * 1e3)
     kernels = {}
-    for i, (name, fn, nbytes) in enumerate(ops):
-        # the rest of the step runs before it, in step order, so the op sees the caches as it does inside a step
-        times = time_alone(fn, [f for _, f, _ in ops[i + 1:] + ops[:i]])
-        med = statistics.median(times)
-        warm = []  # same op back to back: whatever fits stays in the 256 MB memory-side cache
-        for _ in range(20):
-            a, b = _event_pair()
-            fn()
-            _native.time_next_launch(a, b)
-            fn()
-            torch.cuda.synchronize()
-            warm.append(a.elapsed_time(b) * 1e3)
+    for name, nbytes in zip(op_names, op_bytes):
+        med = statistics.median(samples[name])
         kernels[name] = {
-            "bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
+            "bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(samples[name]), 2),
             "GBps": round(nbytes / med / 1e3, 1), "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
-            "us_median_back_to_back": round(statistics.median(warm), 2),
+            "launches_timed": len(samples[name]),
         }
-        log(f"  {name:15s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s "
+        log(f"  {name:30s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s "
             f"({100 * nbytes / med / 1e3 / HBM_PEAK_GBS:.1f}% of peak)")
 
-    # ---- the other forms of the same kernels (ya_fsdp/_param_group.py:701-708, ya_fsdp/_collectives.py:56-58, 139,
-    # 185): gradient accumulation into the reduce buffer, the first reduce of an iteration (copy instead of add),
-    # the all-gather of a size-1 group, and the pre-divide as a pass of its own
-    variants = {}
-    try:
-        d_shard_b = torch.empty_like(d_shard)
-        d_gathered_b = torch.empty_like(d_gathered)
-        d_rs_b = torch.zeros_like(d_rs)
+    # ---- the other forms of the same kernels (--variants; ya_fsdp/_param_group.py:701-708,
+    # ya_fsdp/_collectives.py:56-58, 139, 185): gradient accumulation into the reduce buffer, the first reduce of an
+    # iteration (copy instead of add), the all-gather of a size-1 group, the pre-divide as a pass of its own, a
+    # same-dtype fp32 copy, and a 1-byte all-gather dtype class between odd byte addresses.  Each is timed on its own
+    # dispatch right behind one step on another buffer set (2 GB of other traffic).
+    variants = None
+    if args.variants:
+        d0 = sets[0]
+        d_shard_b = torch.empty_like(d0["shard"])
+        d_gathered_b = torch.empty_like(d0["gathered"])
+        d_rs_b = torch.zeros_like(d0["rs"])
+        d_f32_src = torch.randn(t_pad // 2, device=dev)
+        d_f32_dst = torch.empty_like(d_f32_src)
         add_modes = [_native.MODE_ADD] * len(numels)
-        variant_ops = [
-            ("reduce_copy_in_accumulate", lambda: table.gather_in(d_grads, d_rs_b, add_modes, None, True),
-             t * (2 + 2 * rsz) + (t_pad - t) * rsz),
-            ("post_reduce_copy", lambda: _native.post_reduce(d_shard_b, d_chunk, None, False), s * (rsz + msz)),
-            ("all_gather_size1_copy", lambda: _native.flat_copy(d_gathered_b, d_gathered), 2 * t_pad * 2),
-            ("divide_in_place", lambda: _native.flat_div(d_rs_b, 2.0), 2 * t_pad * rsz),
-        ]
-        # a 1-byte all-gather dtype class of the same layer (tensor-subclass parameters with an int8 / fp8 all-gather,
-        # ya_fsdp/_param.py:281-291, ya_fsdp/_collectives.py:56-58): T_pad bytes copied between odd byte addresses
-        d_bytes_src = d_gathered.view(torch.uint8)[1 : 1 + t_pad]
+        d_bytes_src = d0["gathered"].view(torch.uint8)[1 : 1 + t_pad]
         d_bytes_dst = d_gathered_b.view(torch.uint8)[3 : 3 + t_pad]
-        variant_ops.append(("all_gather_1byte_dtype_odd_addresses", lambda: _native.flat_copy(d_bytes_dst, d_bytes_src),
-                            2 * t_pad))
-        evict = [f for _, f, _ in ops]
-        own_evict = {}
-        if has_copy_in and not fused:
-            # copy-in and copy-out as ONE launch (two independent jobs in one grid); compare with the sum of the
-            # two rows of the per-kernel table.  Evicted by the two reduce-side ops.
-            def one_launch_unshard():
-                if not table.copy_in_scatter_out(d_gathered, d_outs, d_ag_in, d_master):
-                    raise RuntimeError("copy_in_scatter_out declined")
-
-            variant_ops.append(("copy_in_and_copy_out_one_launch", one_launch_unshard, s * (msz + 2) + 2 * t * 2))
-            own_evict["copy_in_and_copy_out_one_launch"] = evict[2:]
-        elif fused and w > 1:
-            # the step runs copy-in and copy-out as one launch: here each as a launch of its own
-            variant_ops.append(("copy_in_alone", op_copy_in, s * (msz + 2)))
-            variant_ops.append(("copy_out_alone", op_copy_out, 2 * t * 2))
-            own_evict["copy_in_alone"] = own_evict["copy_out_alone"] = evict[1:]
+        variant_ops = [
+            ("reduce_copy_in_accumulate", lambda: table.gather_in(d0["grads"], d_rs_b, add_modes, None, True),
+             t * (2 + 2 * rsz) + (t_pad - t) * rsz),
+            ("post_reduce_copy", lambda: _native.post_reduce(d_shard_b, d0["chunk"], None, False), s * (rsz + msz)),
+            ("all_gather_size1_copy", lambda: _native.flat_copy(d_gathered_b, d0["gathered"]), 2 * t_pad * 2),
+            ("divide_in_place", lambda: _native.flat_div(d_rs_b, 2.0), 2 * t_pad * rsz),
+            ("same_dtype_fp32_copy", lambda: _native.flat_copy(d_f32_dst, d_f32_src), 2 * (t_pad // 2) * 4),
+            ("all_gather_1byte_dtype_odd_addresses", lambda: _native.flat_copy(d_bytes_dst, d_bytes_src), 2 * t_pad),
+            ("copy_in_alone", lambda: _native.flat_copy(d0["ag_in"], d0["master"]), copy_in_bytes),
+            ("copy_out_alone", lambda: d0["out_binding"].scatter_out(d0["gathered"]), copy_out_bytes),
+        ]
+        variants = {}
         for name, fn, nbytes in variant_ops:
             fn()
-            # (the step's first two launches run before each sample, so the caches hold nothing of the sample's
-            # operands.  These forms are not part of the timed step: us_median rates the kernel by itself, behind
-            # evicting launches with their write-through tails off, which leave little in the memory-side cache for
-            # the sample to write back; us_median_behind_step is the same sample behind the same launches as the
-            # library runs them by default.)
-            evictors = own_evict.get(name, evict[:2])
-            times = time_alone(fn, evictors, reps=10, plain_evictors=True)
-            behind = statistics.median(time_alone(fn, evictors, reps=10))
+            times = []
+            for _ in range(10):
+                step(1)  # evict: a whole step on another buffer set
+                a, b = _event_pair()
+                _native.time_next_launch(a, b)
+                fn()
+                torch.cuda.synchronize()
+                times.append(a.elapsed_time(b) * 1e3)
             med = statistics.median(times)
             variants[name] = {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(min(times), 2),
                               "GBps": round(nbytes / med / 1e3, 1),
-                              "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4),
-                              "us_median_behind_step": round(behind, 2)}
-            log(f"  {name:26s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s")
-        del d_shard_b, d_gathered_b, d_rs_b
-    except Exception as exc:  # an optional leg must not cost the measurement above
-        log(f"variant table skipped: {type(exc).__name__}: {exc}")
-        variants = None
+                              "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+            log(f"  {name:38s} {nbytes / 1e6:8.1f} MB  median {med:7.1f} us  {nbytes / med / 1e3:7.1f} GB/s")
+        del d_shard_b, d_gathered_b, d_rs_b, d_f32_src, d_f32_dst
 
     # ---- CPU baseline: the oracle (reference torch-op sequence) on the host cores
     cpu_baseline = None
     if args.cpu_seconds > 0 and cpu_state is not None:
-        from oracle import torch_ops  # noqa: F811
-
         cores = os.cpu_count() or 1
         torch.set_num_threads(cores)  # every host core the box shows
         for _ in range(3):            # warm-up passes (page faults, thread pool start-up), not timed
@@ -2026,45 +1972,37 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
         log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads ({reps} passes)")
 
     # ---- the same torch-op sequence on the GPU (torch's own ROCm kernels): what the reference runs on this
-    # hardware today.  Outside the timed region; reported next to the CPU baseline, not a target.
+    # hardware today, over the same K buffer sets in rotation.  Outside the timed region; reported next to the CPU
+    # baseline, not a target.
     torch_gpu = None
     if cpu_state is not None and not args.no_torch_gpu:
-        try:
-            from oracle import torch_ops  # noqa: F811
+        from oracle import torch_ops  # noqa: F811
 
-            g_rs = torch.zeros(t_pad, dtype=rs_dt, device=dev)
-            g_state = {
-                "ag_in": torch.zeros(s, dtype=torch.bfloat16, device=dev),
-                "outs": [torch.empty(n, dtype=torch.bfloat16, device=dev) for n in numels],
-                "rs": g_rs, "rs_views": list(g_rs[:t].split(numels)), "shard": shard0.to(dev),
-            }
+        def gpu_torch_step(d):
+            if has_copy_in:
+                torch_ops.copy_in(d["ag_in"], d["master"])
+            torch_ops.copy_out_materialize(d["gathered"], numels, d["outs"])
+            torch_ops.reduce_copy_in(d["rs_views"], d["grads"], False)
+            torch_ops.reduce_scatter_local(d["shard"], d["rs"], w, r, pre, None, "add")
 
-            def gpu_torch_step(st):
-                if has_copy_in:
-                    torch_ops.copy_in(st["ag_in"], d_master)
-                torch_ops.copy_out_materialize(d_gathered, numels, st["outs"])
-                torch_ops.reduce_copy_in(st["rs_views"], d_grads, False)
-                torch_ops.reduce_scatter_local(st["shard"], st["rs"], w, r, pre, None, "add")
-
-            for _ in range(3):
-                gpu_torch_step(g_state)
-            torch.cuda.synchronize()
-            reps = 20
-            c0 = time.perf_counter()
-            for _ in range(reps):
-                gpu_torch_step(g_state)
-            torch.cuda.synchronize()
-            dt = (time.perf_counter() - c0) / reps
-            torch_gpu = {
-                "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
-                "sample": f"{reps} passes of the reference's torch ops (copy_, split + copy_, _foreach_copy_, div_, add_) on "
-                          f"device tensors with torch {torch.__version__}, same inputs, rated with the same algorithmic bytes",
-            }
-            log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
-            del g_state, g_rs
-        except Exception as exc:  # an optional leg must not cost the measurement above
-            log(f"torch-on-GPU leg skipped: {type(exc).__name__}: {exc}")
-            torch_gpu = None
+        for d in sets:
+            d["rs_views"] = list(d["rs"][:t].split(numels))
+        for k in range(n_sets):
+            gpu_torch_step(sets[k])
+        torch.cuda.synchronize()
+        reps = 5 * n_sets
+        c0 = time.perf_counter()
+        for k in range(reps):
+            gpu_torch_step(sets[k % n_sets])
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - c0) / reps
+        torch_gpu = {
+            "value": round(bytes_per_step / dt / 1e9, 1), "unit": "GB/s", "ms_per_step": round(dt * 1e3, 4),
+            "sample": f"{reps} passes of the reference's torch ops (copy_, split + copy_, _foreach_copy_, div_, add_) on "
+                      f"device tensors with torch {torch.__version__}, same inputs and buffer sets, rated with the "
+                      f"same algorithmic bytes",
+        }
+        log(f"torch ops on the GPU: {torch_gpu['value']} GB/s, {torch_gpu['ms_per_step']} ms per step")
 
     out = {
         "metric": "HBM GB/s + % of peak for copy-in/out+grad-reduce, Llama-3-8B layer @W=8",
@@ -2084,11 +2022,12 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             "workload": workload, "params": len(numels), "total_numel": t, "padded_numel": t_pad,
             "shard_numel": s, "logical_world_size": w, "rank": r, "shard_alignment": align,
             "predivide": pre, "bytes_per_step": bytes_per_step,
+            "buffer_sets": n_sets,  # step k of the timed region runs on buffer set k mod buffer_sets
             "master_dtype": str(master_dt).replace("torch.", ""), "reduce_dtype": str(rs_dt).replace("torch.", ""),
             "ops": ("copy-in master->bf16 [S]; " if has_copy_in else "") +
                    "copy-out bf16 flat->tensors [T]; reduce copy-in bf16 grads->flat /W [T_pad]; "
                    "post-reduce chunk += gradient shard (master dtype) [S]",
-            "launches_per_step": [n for n, _, _ in ops],
+            "launches_per_step": op_names,
             "store_policy_mb_flat_postreduce_scatter_gather": list(_native.get_store_policy()),
         },
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
@@ -2101,20 +2040,19 @@ def run_layer(args, workload: str, steps: int, warmup: int, full: bool = True) -
             "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(workload),
             "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_avg_us, 2), "launches_timed": len(dom_us),
+            "sampled_in": f"the timed region ({n_sets} buffer sets in rotation)",
         },
         "cpu_baseline": cpu_baseline,
         "torch_gpu_baseline": torch_gpu,
-        "graph_replay": graph_replay,
-        "sustained": sustained,
-        "reference_stream_placement": reference_streams,
-        "without_write_through_tails": tail_off,
-        "buffer_sets_in_rotation": rotating,
-        "step_us_minus_isolated_kernel_us": round(ms_per_step * 1e3 - sum(k["us_median"] for k in kernels.values()), 2),
+        "one_buffer_set": one_set,
         "kernels": kernels,
-        "kernel_variants": variants,
     }
-    out_binding.close()
-    table.close()
+    for key, leg in (("sustained", sustained), ("store_policies_in_rotation", policy_ab),
+                     ("reference_stream_placement", reference_streams), ("graph_replay", graph_replay),
+                     ("kernel_variants", variants)):
+        if leg is not None:
+            out[key] = leg
+    close_all()
     return out
 
 

@@ -400,6 +400,14 @@ def test_setters_that_must_not_change_the_numbers():
     blocks[1].set_modules_to_backward_prefetch([blocks[0]])
     _assert_same_masters(_train(model, xs, 0.05), want)
 
+    # the library's own opt-in: reduce copy-in on the reduce-scatter stream (real autograd gradients here, freed
+    # right after the launch that reads them on the other stream)
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    model.set_reduce_copy_in_on_side_stream(True)
+    groups = [g for m in model._fsdp_modules(True) if (g := m._get_fsdp_state()._fsdp_param_group) is not None]
+    assert groups and all(g.reduce_copy_in_on_side_stream for g in groups)
+    _assert_same_masters(_train(model, xs, 0.05), want)
+
 
 
 def test_parameters_kept_unsharded_between_micro_batches():

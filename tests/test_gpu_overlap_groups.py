@@ -24,8 +24,9 @@ GROUP_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("w,r", [(4, 2), (1, 0)])
-def test_groups_sharing_buffers_under_concurrent_gemms(w, r):
+@pytest.mark.parametrize("w,r", [(4, 2), (1, 0), (3, 1)])
+@pytest.mark.parametrize("copy_in_on_side_stream", [False, True])
+def test_groups_sharing_buffers_under_concurrent_gemms(w, r, copy_in_on_side_stream):
     from yafsdp_amd._param_group import YaFSDPParamGroup, init_shared_state
 
     align = 512
@@ -35,6 +36,9 @@ def test_groups_sharing_buffers_under_concurrent_gemms(w, r):
         dev_params = [p.to(DEV).requires_grad_(True) for p in cpu_params]
         groups.append(YaFSDPParamGroup(dev_params, FSDPMeshInfo(w, r), DEV, BF16_MP, align))
         refs.append(CpuGroup(cpu_params, w, r, align, BF16_MP))
+    for g in groups:
+        # the opt-in stream plan: reduce copy-in on the reduce-scatter stream, right in front of the post-reduce
+        g.reduce_copy_in_on_side_stream = copy_in_on_side_stream
     init_shared_state(groups, DEV)  # 2 data buffers handed out round-robin, 1 gradient buffer
     assert len({id(g.data_buffer_ctx) for g in groups}) == 2 and len({id(g.grad_buffer_ctx) for g in groups}) == 1
     n = len(groups)
@@ -46,7 +50,7 @@ def test_groups_sharing_buffers_under_concurrent_gemms(w, r):
         for _ in range(k):
             torch.matmul(a, b, out=c)
 
-    post = float(w) if w > 1 else None
+    collective = ("AVG", None) if w > 1 else None  # bf16 reduce: the collective scales by 1 / W rounded to bf16
     for it in range(2):
         print("iteration", it, "w", w, flush=True)
         snaps = [None] * n
@@ -78,7 +82,7 @@ def test_groups_sharing_buffers_under_concurrent_gemms(w, r):
         torch.cuda.synchronize()
         for i, (g, ref) in enumerate(zip(groups, refs)):
             ref.unshard(first_of_iteration=True)
-            ref.reduce(None, post, "copy" if it == 0 else "add")
+            ref.reduce(None, None, "copy" if it == 0 else "add", collective=collective)
             assert_bits_equal(snaps[i][1], ref.ag_in, f"iteration {it} group {i}: all-gather input")
             assert_bits_equal(snaps[i][0], ref.ag_in, f"iteration {it} group {i}: this rank's slot of the gathered buffer")
             assert_bits_equal(g._padded_sharded_param_grad[None], ref.grad_shard, f"iteration {it} group {i}: grad shard")

@@ -169,6 +169,10 @@ class YaFSDPParamGroup:
         self.force_sum_reduction_for_comms: bool = False
         self.unshard_async_op: bool = False
         self.unshard_in_backward: bool = True
+        # opt-in, not the reference's plan (ya_fsdp/_param_group.py:669-708 runs the foreach calls on the compute
+        # stream): the reduce copy-in of a pass that reduces runs on the reduce-scatter stream as well, right in
+        # front of the post-reduce, and the compute stream goes on with the next group's backward at once
+        self.reduce_copy_in_on_side_stream: bool = False
         self._all_gather_result: AllGatherResult | None = None
         self._post_reduce_event: torch.cuda.Event | None = None
 
@@ -571,7 +575,13 @@ class YaFSDPParamGroup:
     def post_backward(self, *unused: Any) -> None:
         """ya_fsdp/_param_group.py:655-771.  Safe to call when the group took no part in the backward."""
         self._training_state = TrainingState.POST_BACKWARD
-        current_stream = torch.cuda.current_stream(self.device)
+        compute_stream = torch.cuda.current_stream(self.device)
+        # the stream that writes the reduce buffer: the compute stream as in the reference, or (opt-in, for a pass
+        # that reduces) the reduce-scatter stream once the compute stream has produced this group's gradients
+        on_side = self.reduce_copy_in_on_side_stream and self.reduce_grads and self.grad_buffer_ctx is not None
+        current_stream = self.comm_ctx.reduce_scatter_stream if on_side else compute_stream
+        if on_side:
+            current_stream.wait_stream(compute_stream)
         if (grad_buffer_ctx := self.grad_buffer_ctx) is not None:
             if (owner := grad_buffer_ctx.owner) is not None and owner is not self:
                 raise RuntimeError(f"{self} tried to acquire its gradient buffer, but it is in use by {owner}.")
@@ -582,7 +592,9 @@ class YaFSDPParamGroup:
         predivide_fused: dict[torch.dtype | None, bool] = {}
         copy_in_events: dict[torch.dtype | None, torch.cuda.Event] = {}
         reduced_in_one_launch = False
-        with profiler_range(self._with_fqn("FSDP::post_backward_accumulate")):
+        with profiler_range(self._with_fqn("FSDP::post_backward_accumulate")), (
+            torch.cuda.stream(current_stream) if on_side else contextlib.nullcontext()
+        ):
             single_class = len(self._all_gather_dtype_to_fsdp_params) == 1
             for all_gather_dtype, fsdp_params in self._all_gather_dtype_to_fsdp_params.items():
                 grads: list[torch.Tensor | None] = []
@@ -603,6 +615,10 @@ class YaFSDPParamGroup:
                         modes.append(MODE_SKIP)
                 if not any(m != MODE_SKIP for m in modes):
                     continue
+                if on_side:
+                    for grad in grads:  # allocated on the compute stream, read on this one
+                        if grad is not None:
+                            grad.record_stream(current_stream)
                 assert grad_buffer_ctx is not None and all_gather_dtype in self._tables
                 pre = None
                 if self.reduce_grads:
@@ -613,12 +629,12 @@ class YaFSDPParamGroup:
                     )
                     predivide_fused[all_gather_dtype] = True
                     if single_class and all_gather_dtype is None:
-                        reduced_in_one_launch = self._reduce_in_one_launch(grads, modes)
+                        reduced_in_one_launch = self._reduce_in_one_launch(grads, modes, current_stream, on_side)
                 if not reduced_in_one_launch and self.reduce_grads:
                     # the launch records its own completion: the reduce-scatter stream waits for that event instead
                     # of a marker placed behind the kernel in the compute stream's queue
                     copy_in_events[all_gather_dtype] = _native.launch_recording(
-                        self.completion_event(("reduce_copy_in", all_gather_dtype)),
+                        self.completion_event(("reduce_copy_in", all_gather_dtype, on_side)),
                         lambda: foreach_reduce_copy_in(
                             self, self._tables[all_gather_dtype], self._reduce_scatter_input[all_gather_dtype],
                             grads, modes, pre,
@@ -654,7 +670,7 @@ class YaFSDPParamGroup:
         if reduced_in_one_launch:
             # the gradient shard is already written, on this stream (ya_fsdp/_collectives.py:216-217 for the rest)
             with profiler_range(self._with_fqn("YaFSDP::post_backward_reduce")):
-                self._post_reduce_event = self.completion_event("reduce_in_one_launch")  # recorded by that launch
+                self._post_reduce_event = self.completion_event(("reduce_in_one_launch", on_side))  # recorded by that launch
                 for fsdp_param in fsdp_params_with_grad_per_dtype[None]:
                     fsdp_param.sharded_param.grad = fsdp_param.sharded_param_grad
             grad_buffer_ctx.release_event = self._post_reduce_event
@@ -685,7 +701,8 @@ class YaFSDPParamGroup:
         grad_buffer_ctx.release_event = self._post_reduce_event
         grad_buffer_ctx.owner = None
 
-    def _reduce_in_one_launch(self, grads: "list[torch.Tensor | None]", modes: "list[int]") -> bool:
+    def _reduce_in_one_launch(self, grads: "list[torch.Tensor | None]", modes: "list[int]",
+                              stream: "torch.cuda.Stream", on_side: bool = False) -> bool:
         """A shard group of size ONE whose gradients pass through the reduce buffer: the rank's chunk is the whole
         buffer and the "reduce-scatter" copies it onto itself (ya_fsdp/_collectives.py:140-150), so the reduce
         copy-in (ya_fsdp/_param_group.py:693-708), the divides (:139, :146-148, :165) and the copy or accumulation
@@ -729,12 +746,12 @@ class YaFSDPParamGroup:
         self._grad_sumsq_token.pop(None, None)
         served = []
         _native.launch_recording(
-            self.completion_event("reduce_in_one_launch"),
+            self.completion_event(("reduce_in_one_launch", on_side)),
             lambda: served.append(self._table.gather_in_post_reduce(
                 grads, self._reduce_scatter_input[None], shard, n_acc > 0, modes,
                 pre_factor=pre, post_factor=post, custom_divisor=custom,
             )),
-            torch.cuda.current_stream(self.device),
+            stream,
         )
         return bool(served and served[0])
 
