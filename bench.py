@@ -1329,6 +1329,36 @@ def run_ceilings(args) -> int:
     kernels["torch_copy_bf16"] = {"bytes": n * 4, "us_median": round(med, 2), "us_min": round(min(times), 2),
                                   "GBps": round(n * 4 / med / 1e3, 1), "frac_of_peak": round(n * 4 / med / 1e3 / HBM_PEAK_GBS, 4)}
     log(f"  {'torch_copy_bf16':24s} {n * 4 / 1e6:8.1f} MB  median {med:7.1f} us  {n * 4 / med / 1e3:7.1f} GB/s")
+    # ---- what a 1:1 copy SUSTAINS: 40 copies back to back over four source / destination pairs (3.5 GB of
+    # buffers in rotation), timed from the first kernel's begin to the last one's end.  A single dispatch timed by
+    # itself flatters write-through stores (the kernel ends while the memory-side cache still holds its output,
+    # and the next kernel pays for the write-back) and penalises non-temporal ones (the kernel's end waits for the
+    # L2s' dirty lines); a train of copies counts every byte of every policy once.
+    pairs = [(torch.empty_like(a), a.clone()) for _ in range(4)]
+    for label, tail in (("non_temporal_stores", 0), ("write_through_stores", 1 << 20)):
+        saved = _native.get_option(_native.OPT_FLAT_TAIL_MB)
+        _native.set_option(_native.OPT_FLAT_TAIL_MB, tail)
+        try:
+            rates = []
+            for _ in range(5):
+                for dst_, src_ in pairs:
+                    _native.flat_copy(dst_, src_)
+                x, y = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                x.record()
+                for k in range(40):
+                    _native.flat_copy(*pairs[k % 4])
+                y.record()
+                torch.cuda.synchronize()
+                rates.append(40 * n * 4 / (x.elapsed_time(y) * 1e3) / 1e3)
+        finally:
+            _native.set_option(_native.OPT_FLAT_TAIL_MB, saved)
+        med = statistics.median(rates)
+        kernels[f"copy_bf16_train_of_40_over_4_buffer_pairs_{label}"] = {
+            "bytes": n * 4, "us_median": round(n * 4 / med / 1e3, 2), "GBps": round(med, 1),
+            "frac_of_peak": round(med / HBM_PEAK_GBS, 4)}
+        log(f"  train of 40 copies, {label}: {med:7.1f} GB/s ({100 * med / HBM_PEAK_GBS:.1f}% of peak)")
+    del pairs
+    stream_mixes = _stream_mix_ceilings(torch, _native, dev, lambda: _native.flat_copy(big2, big), max(args.steps, 10))
     best = kernels["copy_bf16_to_bf16"]
     out_line = {
         "metric": "HBM GB/s of plain streaming kernels (read-only, write-only, 1:1 copy) at the headline buffer size",
@@ -1338,10 +1368,115 @@ def run_ceilings(args) -> int:
         "config": {"workload": args.workload, "elements": n},
         "roofline": {"bound": "hbm", "kernel": "flat_kernel (bf16 -> bf16 copy)", "achieved": best["GBps"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": best["frac_of_peak"], "traffic": None},
-        "cpu_baseline": None, "kernels": kernels,
+        "cpu_baseline": None, "kernels": kernels, "stream_mixes": stream_mixes,
     }
     print(json.dumps(out_line), flush=True)
     return 0
+
+
+def _stream_mix_ceilings(torch, _native, dev, evict, reps):
+    """What a single pass over SEVERAL arrays at once reaches on this memory system: the measurement-only mover of
+    yafsdp_amd/csrc/ceilings.hip (no arithmetic to speak of) with the stream mixes of the optimizer-side kernels, over
+    workgroup shapes, with the arrays at their natural addresses and skewed against each other; next to it the
+    library's own kernel of each mix on the same arrays.  One rank's shard of the Llama-3-8B layer (27.3 M elements)."""
+    import ctypes
+
+    path = os.path.join(ROOT, "yafsdp_amd", "libyafsdp_ceilings.so")
+    if not os.path.exists(path):
+        log(f"stream-mix ceilings skipped: {path} is not built (python -m yafsdp_amd._build)")
+        return None
+    lib = ctypes.CDLL(path)
+    vp = ctypes.c_void_p
+    lib.ceil_stream_mix.restype = ctypes.c_int
+    lib.ceil_stream_mix.argtypes = [ctypes.c_int] * 5 + [vp, vp, vp, ctypes.c_int64, vp, vp, vp]
+    n = 26_624 * 1024  # 27,262,976 elements: whole tiles for every shape below
+    gen = torch.Generator(device=dev).manual_seed(11)
+    stream = vp(torch.cuda.current_stream(dev).cuda_stream)
+
+    def arrays(count, skew_bytes):
+        """`count` binary32 arrays of n elements cut from one allocation, array k shifted by k * skew_bytes."""
+        stride = n * 4 + skew_bytes
+        pool = torch.empty((count * stride + 256) // 4, dtype=torch.float32, device=dev)
+        pool.copy_(torch.randn(pool.numel(), device=dev, generator=gen) * 0.02)
+        return pool, [pool[(k * stride) // 4 : (k * stride) // 4 + n] for k in range(count)]
+
+    def ptrs(tensors):
+        return (vp * max(1, len(tensors)))(*[t.data_ptr() for t in tensors]) if tensors else (vp * 1)()
+
+    def timed(fn_with_events):
+        times = []
+        for _ in range(reps):
+            evict()
+            a, b = _event_pair()
+            fn_with_events(a, b)
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b) * 1e3)
+        return statistics.median(times), min(times)
+
+    def mover(nr, nw32, nw16, block, unroll, reads, w32, w16):
+        def run(a, b):
+            rc = lib.ceil_stream_mix(nr, nw32, nw16, block, unroll, ptrs(reads), ptrs(w32), ptrs(w16), n, stream,
+                                     vp(a.cuda_event), vp(b.cuda_event))
+            if rc != 0:
+                raise RuntimeError(f"ceil_stream_mix({nr},{nw32},{nw16},{block},{unroll}) returned {rc}")
+        return run
+
+    def row(us, nbytes):
+        med, lo = us
+        return {"bytes": nbytes, "us_median": round(med, 2), "us_min": round(lo, 2), "GBps": round(nbytes / med / 1e3, 1),
+                "frac_of_peak": round(nbytes / med / 1e3 / HBM_PEAK_GBS, 4)}
+
+    out = {}
+    shapes = [(64, 1), (64, 2), (64, 4), (128, 1), (128, 2), (128, 4), (256, 1), (256, 2), (256, 4), (512, 1), (512, 2),
+              (1024, 1)]
+    # ---- the fused AdamW mix: p, g, m, v read; p, m, v (binary32) and the 2-byte all-gather input written
+    adam_bytes = n * 30
+    for skew in (0, 4096 + 256, 1 << 20):
+        pool, (p_, g_, m_, v_) = arrays(4, skew)
+        out16 = torch.empty(n, dtype=torch.bfloat16, device=dev)
+        table = {}
+        for block, unroll in shapes:
+            table[f"{block}x{unroll}"] = row(timed(mover(4, 3, 1, block, unroll, [p_, g_, m_, v_], [p_, m_, v_], [out16])),
+                                             adam_bytes)
+        best = max(table, key=lambda k: table[k]["GBps"])
+
+        def adam(a, b):
+            _native.time_next_launch(a, b)
+            _native.adamw_step(p_, g_, m_, v_, out16, lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=3)
+
+        out[f"adamw_mix_4r_3w32_1w16_skew_{skew}"] = {"mover_by_shape": table, "mover_best_shape": best,
+                                                      "mover_best": table[best], "library_adamw_kernel": row(timed(adam), adam_bytes)}
+        log(f"  AdamW mix (16 B read, 14 B written per element), arrays skewed by {skew} B: mover best {best} "
+            f"{table[best]['GBps']} GB/s ({table[best]['us_median']} us), library kernel "
+            f"{out[f'adamw_mix_4r_3w32_1w16_skew_{skew}']['library_adamw_kernel']['GBps']} GB/s")
+        del pool, p_, g_, m_, v_, out16
+    # ---- one array read and written in place (the scaling pass), and one read / another written
+    pool, (x_, y_) = arrays(2, 0)
+    coef = torch.tensor([0.5], device=dev)
+    table = {f"{b_}x{u_}": row(timed(mover(1, 1, 0, b_, u_, [x_], [x_], [])), n * 8) for b_, u_ in shapes}
+    best = max(table, key=lambda k: table[k]["GBps"])
+
+    def scale(a, b):
+        _native.time_next_launch(a, b)
+        _native.flat_scale(x_, coef)
+
+    out["in_place_1r_1w32"] = {"mover_by_shape": table, "mover_best_shape": best, "mover_best": table[best],
+                               "library_scale_kernel": row(timed(scale), n * 8)}
+    log(f"  in-place mix (4 B read, 4 B written): mover best {best} {table[best]['GBps']} GB/s, library scale kernel "
+        f"{out['in_place_1r_1w32']['library_scale_kernel']['GBps']} GB/s")
+    table = {f"{b_}x{u_}": row(timed(mover(1, 0, 0, b_, u_, [x_], [], [])), n * 4) for b_, u_ in shapes}
+    best = max(table, key=lambda k: table[k]["GBps"])
+    partials = torch.empty(_native.SUMSQ_MAX_PARTIALS, dtype=torch.float64, device=dev)
+
+    def sumsq(a, b):
+        _native.time_next_launch(a, b)
+        _native.sumsq_partials(x_, partials, 0)
+
+    out["read_only_1r"] = {"mover_by_shape": table, "mover_best_shape": best, "mover_best": table[best],
+                           "library_sumsq_kernel": row(timed(sumsq), n * 4)}
+    log(f"  read-only, 109 MB: mover best {best} {table[best]['GBps']} GB/s, library sum-of-squares kernel "
+        f"{out['read_only_1r']['library_sumsq_kernel']['GBps']} GB/s")
+    return out
 
 
 def main() -> int:

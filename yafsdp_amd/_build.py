@@ -63,6 +63,23 @@ def build(force: bool = True, jobs: int = 8) -> str:
     return OUT
 
 
+CEILINGS_OUT = os.path.join(HERE, "libyafsdp_ceilings.so")
+
+
+def build_ceilings(force: bool = True) -> str:
+    """Compile the measurement-only stream-mix mover (``csrc/ceilings.hip``) into a library of its own; only the
+    benchmark's hbm-ceilings workload loads it."""
+    src = os.path.join(CSRC, "ceilings.hip")
+    if not force and os.path.exists(CEILINGS_OUT) and os.path.getmtime(CEILINGS_OUT) >= os.path.getmtime(src):
+        return CEILINGS_OUT
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", src, "-o", CEILINGS_OUT]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        noise = "is not a recognized feature for this target"
+        raise RuntimeError("hipcc failed on ceilings.hip:\n" + "\n".join(l for l in r.stderr.splitlines() if noise not in l))
+    return CEILINGS_OUT
+
+
 TENSORLIST_SRC = os.path.join(CSRC, "tensorlist.cpp")
 TENSORLIST_OUT = os.path.join(HERE, "_tensorlist.so")
 
@@ -94,3 +111,4 @@ def build_tensorlist(force: bool = True) -> str:
 if __name__ == "__main__":
     print(build())
     print(build_tensorlist())
+    print(build_ceilings())
