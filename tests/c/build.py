@@ -27,5 +27,16 @@ def build() -> str:
     return OUT
 
 
+RING_OUT = os.path.join(HERE, "stage_ring_check")
+
+
+def build_stage_ring_check() -> str:
+    """Host-only simulation of the staging slots' state machine (``yafsdp_amd/csrc/stage_ring.h``): g++, no HIP."""
+    cmd = ["g++", "-O1", "-std=c++17", "-Wall", os.path.join(HERE, "stage_ring_check.cpp"), "-o", RING_OUT]
+    subprocess.run(cmd, check=True)
+    return RING_OUT
+
+
 if __name__ == "__main__":
     print(build())
+    print(build_stage_ring_check())

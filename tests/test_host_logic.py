@@ -53,3 +53,21 @@ def test_sizes_to_slices_docstring_example():
     assert sizes_to_slices([20, 20, 30]) == [slice(0, 20, None), slice(20, 40, None), slice(40, 70, None)]
     assert sizes_to_slices([]) == []
     assert sizes_to_slices([0, 3, 0]) == [slice(0, 0), slice(0, 3), slice(3, 3)]
+
+
+def test_staging_slot_state_machine_against_a_simulated_runtime():
+    """``yafsdp_amd/csrc/stage_ring.h`` (the slots that carry per-call pointer arrays to the table kernels) driven by
+    a simulated runtime on the host: random streams, repeated and fresh tensor sets, failed copies and launches,
+    partial completion; every kernel must be ordered behind the copy it reads and no copy may overtake a queued
+    reader (tests/c/stage_ring_check.cpp)."""
+    import importlib.util
+    import os
+    import subprocess
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c")
+    spec = importlib.util.spec_from_file_location("c_build", os.path.join(here, "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    binary = mod.build_stage_ring_check()
+    r = subprocess.run([binary], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and r.stdout.strip().endswith("PASS"), r.stdout[-2000:] + r.stderr[-2000:]

@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libyafsdp_hip.so")
 SOURCES = ["api.hip", "flat.hip", "gather.hip", "scatter.hip", "optim.hip", "fan.hip", "postsumsq.hip", "fused.hip"]
 HEADERS = ["elem.hip.h", "flat_kernels.hip.h", "table_kernels.hip.h", "optim_kernels.hip.h", "fan_kernels.hip.h",
-           "post_sumsq_kernels.hip.h", "fused_kernels.hip.h", "launch.h", "tuning.h"]
+           "post_sumsq_kernels.hip.h", "fused_kernels.hip.h", "launch.h", "stage_ring.h", "tuning.h"]
 ARCH = "gfx950"
 
 # -ffp-contract=off: every multiply and add of the path rounds on its own, as

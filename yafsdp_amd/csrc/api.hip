@@ -10,6 +10,7 @@
 
 #include "../../include/yafsdp_hip.h"
 #include "launch.h"
+#include "stage_ring.h"
 #include "tuning.h"
 
 using namespace yafsdp;
@@ -180,6 +181,19 @@ int flat_launch(int src_dt, int dst_dt, int scale, bool acc, void* dst, const vo
 
 }  // namespace
 
+// The HIP side of the staging slots' state machine.
+struct HipRuntime {
+  typedef hipStream_t Stream;
+  typedef hipEvent_t Event;
+  static constexpr int kNotReady = int(hipErrorNotReady);
+  int stream_wait_event(Stream s, Event e) { return int(hipStreamWaitEvent(s, e, 0)); }
+  int event_query(Event e) { return int(hipEventQuery(e)); }
+  int memcpy_h2d_async(void* dst, const void* src, size_t n, Stream s) {
+    return int(hipMemcpyAsync(dst, src, n, hipMemcpyHostToDevice, s));
+  }
+  int event_record(Event e, Stream s) { return int(hipEventRecord(e, s)); }
+};
+
 struct yafsdp_table {
   int device = 0;
   int32_t n_tensors = 0;
@@ -197,20 +211,9 @@ struct yafsdp_table {
   std::vector<int64_t> slot_start;  // host, n_tensors + 1
   int32_t n_slots = 0;
   TileRec* d_slots = nullptr;    // only for tables with more than kSmallMax tensors
-  // staging slots for the per-call pointer/mode arrays of tables with more than kSmallMax tensors: pinned host
-  // slot -> device slot.  A slot keeps what was staged into it, so a call whose arrays equal a slot's content
-  // (the caching allocator hands autograd the same addresses step after step) reuses the device copy without
-  // copying again.  ev[s] marks the end of the last kernel that reads slot s.
-  static constexpr int kRing = 8;
-  size_t stage_bytes = 0;
-  char* h_stage[kRing] = {};
-  char* d_stage[kRing] = {};
-  hipEvent_t ev[kRing] = {};
-  bool ev_pending[kRing] = {};
-  bool filled[kRing] = {};          // h_stage[s] / d_stage[s] hold a staged set
-  hipStream_t staged_on[kRing] = {};  // stream the copy into d_stage[s] was enqueued on
+  // staging slots for the per-call pointer / mode arrays of tables with more than kSmallMax tensors (stage_ring.h)
+  StageRing<HipRuntime> ring;
   std::vector<char> scratch;        // host: the arrays of the current call in staging format
-  int next = 0;
   std::mutex mu;
   // yafsdp_table_set_option: this table's own write-through tails, -1 = the process-wide option
   std::atomic<int> gather_tail_mb{-1};
@@ -254,10 +257,10 @@ void table_free(yafsdp_table* t) {
   if (t->d_offsets) (void)hipFree(t->d_offsets);
   if (t->d_tiles) (void)hipFree(t->d_tiles);
   if (t->d_slots) (void)hipFree(t->d_slots);
-  for (int i = 0; i < yafsdp_table::kRing; i++) {
-    if (t->ev[i]) (void)hipEventDestroy(t->ev[i]);
-    if (t->h_stage[i]) (void)hipHostFree(t->h_stage[i]);
-    if (t->d_stage[i]) (void)hipFree(t->d_stage[i]);
+  for (int i = 0; i < t->ring.kRing; i++) {
+    if (t->ring.ev[i]) (void)hipEventDestroy(t->ring.ev[i]);
+    if (t->ring.h_stage[i]) (void)hipHostFree(t->ring.h_stage[i]);
+    if (t->ring.d_stage[i]) (void)hipFree(t->ring.d_stage[i]);
   }
   delete t;
 }
@@ -306,61 +309,30 @@ int stage_large(yafsdp_table* t, const void* const* ptrs, const uint8_t* mode, L
   uint32_t* cm = reinterpret_cast<uint32_t*>(cur + size_t(n) * sizeof(void*));
   for (int p = 0; p < n; p++) cm[p] = mode ? mode[p] : uint32_t(MODE_COPY);
   const size_t used = size_t(n) * (sizeof(void*) + sizeof(uint32_t));
+  HipRuntime rt;
   int s = -1;
-  for (int i = 0; i < yafsdp_table::kRing; i++) {
-    if (t->filled[i] && std::memcmp(t->h_stage[i], cur, used) == 0) { s = i; break; }
-  }
-  if (s >= 0) {
-    // same arrays as an earlier call: the device copy is reused.  This call's kernel is ordered behind the slot's
-    // last reader, whichever stream that ran on (on the device; the host does not wait; a wait for an event of the
-    // same stream costs nothing), so the event that this call records afterwards covers every earlier reader and
-    // the copy before them.
-    if (t->ev_pending[s]) {
-      hipError_t e = hipStreamWaitEvent(stream, t->ev[s], 0);
-      if (e != hipSuccess) return int(e);
-    }
-  } else {
-    for (int k = 0; k < yafsdp_table::kRing && s < 0; k++) {
-      const int i = (t->next + k) % yafsdp_table::kRing;
-      if (t->ev_pending[i]) {
-        const hipError_t q = hipEventQuery(t->ev[i]);
-        if (q == hipErrorNotReady) continue;  // its last kernel (and the copy before it) is still in flight
-        if (q != hipSuccess) return int(q);
-        t->ev_pending[i] = false;
-      }
-      s = i;
-    }
-    if (s < 0) return YAFSDP_ERR_BUSY;
-    t->next = (s + 1) % yafsdp_table::kRing;
-    std::memcpy(t->h_stage[s], cur, used);
-    t->filled[s] = true;
-    t->staged_on[s] = stream;
-    hipError_t e = hipMemcpyAsync(t->d_stage[s], t->h_stage[s], t->stage_bytes, hipMemcpyHostToDevice, stream);
-    if (e != hipSuccess) { t->filled[s] = false; return int(e); }
-  }
+  const int rc = t->ring.acquire(rt, cur, used, stream, YAFSDP_ERR_BUSY, &s);
+  if (rc != 0) return rc;
   m->offsets = t->d_offsets;
   m->tiles = t->d_tiles;
   m->slots = t->d_slots;
-  m->ptrs = reinterpret_cast<const void* const*>(t->d_stage[s]);
-  m->modes_ = reinterpret_cast<const uint32_t*>(t->d_stage[s] + size_t(n) * sizeof(void*));
+  m->ptrs = reinterpret_cast<const void* const*>(t->ring.d_stage[s]);
+  m->modes_ = reinterpret_cast<const uint32_t*>(t->ring.d_stage[s] + size_t(n) * sizeof(void*));
   m->n_tensors = n;
   *slot = s;
   return YAFSDP_OK;
 }
 
 int finish_large(yafsdp_table* t, int slot, hipStream_t stream) {
-  hipError_t e = hipEventRecord(t->ev[slot], stream);
-  if (e != hipSuccess) return int(e);
-  t->ev_pending[slot] = true;
-  return YAFSDP_OK;
+  HipRuntime rt;
+  return t->ring.finish(rt, slot, stream);
 }
 
 // The launch after stage_large failed: the slot's content is no longer offered for reuse, and the slot stays
 // ordered behind whatever stage_large enqueued (the event is recorded all the same).  Returns `launch_error`.
 int abandon_large(yafsdp_table* t, int slot, hipStream_t stream, hipError_t launch_error) {
-  t->filled[slot] = false;
-  if (hipEventRecord(t->ev[slot], stream) == hipSuccess) t->ev_pending[slot] = true;
-  return int(launch_error);
+  HipRuntime rt;
+  return t->ring.abandon(rt, slot, stream, int(launch_error));
 }
 
 }  // namespace
@@ -1058,12 +1030,13 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
       if ((e = hipMemcpy(t->d_slots, tiles.data(), tiles.size() * sizeof(TileRec), hipMemcpyHostToDevice)) != hipSuccess) break;
     }
     if (n_tensors > kSmallRoute) {
-      t->stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
-      t->scratch.assign(t->stage_bytes, 0);
-      for (int i = 0; i < yafsdp_table::kRing && e == hipSuccess; i++) {
-        if ((e = hipHostMalloc(reinterpret_cast<void**>(&t->h_stage[i]), t->stage_bytes, hipHostMallocDefault)) != hipSuccess) break;
-        if ((e = hipMalloc(reinterpret_cast<void**>(&t->d_stage[i]), t->stage_bytes)) != hipSuccess) break;
-        if ((e = hipEventCreateWithFlags(&t->ev[i], hipEventDisableTiming)) != hipSuccess) break;
+      const size_t stage_bytes = (size_t(n_tensors) * (sizeof(void*) + sizeof(uint32_t)) + 15) & ~size_t(15);
+      t->ring.stage_bytes = stage_bytes;
+      t->scratch.assign(stage_bytes, 0);
+      for (int i = 0; i < t->ring.kRing && e == hipSuccess; i++) {
+        if ((e = hipHostMalloc(reinterpret_cast<void**>(&t->ring.h_stage[i]), stage_bytes, hipHostMallocDefault)) != hipSuccess) break;
+        if ((e = hipMalloc(reinterpret_cast<void**>(&t->ring.d_stage[i]), stage_bytes)) != hipSuccess) break;
+        if ((e = hipEventCreateWithFlags(&t->ring.ev[i], hipEventDisableTiming)) != hipSuccess) break;
       }
     }
   } while (false);
@@ -1082,9 +1055,9 @@ int yafsdp_table_create(int n_tensors, const int64_t* numels, int64_t padded_num
 int yafsdp_table_destroy(yafsdp_table* table) {
   if (table == nullptr) return YAFSDP_OK;
   int rc = YAFSDP_OK;
-  for (int i = 0; i < yafsdp_table::kRing; i++) {
-    if (table->ev_pending[i]) {
-      hipError_t e = hipEventSynchronize(table->ev[i]);
+  for (int i = 0; i < table->ring.kRing; i++) {
+    if (table->ring.ev_pending[i]) {
+      hipError_t e = hipEventSynchronize(table->ring.ev[i]);
       if (e != hipSuccess) rc = int(e);
     }
   }
