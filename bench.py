@@ -55,8 +55,8 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
     return [(n,) for n, f in zip(numels, is_fp32_master) if f == fp32_masters]
 
 # HBM bytes per launch of the dominant kernel (gather_in_kernel), from two rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE), each scaled by the reading of a plain copy of known size in the same run
-# (factors 1.99986 and 1.00000): (213067.8 * 1.99986 + 426086.1 * 1.00000) KiB.
+# (FETCH_SIZE, WRITE_SIZE) of the default command (four buffer sets in rotation), each scaled by the reading of a
+# plain copy of known size (factors 1.99986 and 1.00000): (213073.8 * 1.99986 + 426081.6 * 1.00000) KiB.
 # Summary and commands: profiles/bench_llama3-8b-layer-w8_hbm_traffic.md.  None = not measured.
 # "llama3-8b-layer-w8-optim": adamw_kernel, (213045.6 * 1.99946 + 372753.5 * 0.99996) KiB, scaled by the plain
 # fp32 copy of the same run; profiles/bench_llama3-8b-layer-w8-optim_hbm_traffic.md.
@@ -71,10 +71,10 @@ def _ragged_stress_shapes(seed=1005, p=2000, fp32_masters=True):
 # Megabytes a GEMM stand-in of the full-model workload moves between the L2s and the memory side per launch
 # (TCC_EA0_RDREQ x 128 B + TCC_EA0_WRREQ x 64 B of the hipBLASLt kernel alone; profiles/bench_llama3-8b-full-w8_overlap.md),
 # and the rate at which a copy kernel of the path moves its bytes when it has the memory side to itself.
-GEMM_MEMORY_SIDE_MB = {"4096x4096x4096": 453.4 + 33.6, "llama-mlp-up 4096x4096x14336": 755.4 + 117.4,
-                       "llama-mlp-down 4096x14336x4096": 755.4 + 33.6}
+GEMM_MEMORY_SIDE_MB = {"4096x4096x4096": 201.8 + 33.6, "llama-mlp-up 4096x4096x14336": 755.4 + 117.4,
+                       "llama-mlp-down 4096x14336x4096": 705.1 + 33.6}
 COPY_RATE_MB_PER_MS = 6550.0
-MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_645_400, "llama3-8b-layer-w8-optim": 817_885_000,
+MEASURED_TRAFFIC_BYTES = {"llama3-8b-layer-w8": 872_652_200, "llama3-8b-layer-w8-optim": 817_885_000,
                           "ragged-stress-w256": 1_505_902_865, "llama3-70b-layer-w64": 3_422_785_664,
                           "ragged-stress-w256-bf16-masters": 1_014_344_628, "tiny-layer-w1": 37_979_573}
 
@@ -193,6 +193,43 @@ def analyze_overlap_trace(path: str) -> int:
     return 0
 
 
+def analyze_gaps(path: str) -> int:
+    """Reads the kernel trace (CSV) of ``--workload llama3-8b-full-w8 --copies-only`` and prints, per phase (the
+    phases are fenced by kernels that are not the library's), how long the GPU idles between consecutive kernels of the
+    path, by kind of pair: next kernel's begin minus this kernel's end."""
+    import csv
+
+    def kind(name):
+        for key, k in (("unshard_kernel", "copy-in + copy-out"), ("gather_in_kernel", "reduce copy-in"),
+                       ("flat_kernel<yafsdp::BF16", "post-reduce")):
+            if key in name:
+                return k
+        return None
+
+    rows = sorted(csv.DictReader(open(path)), key=lambda r: int(r["Start_Timestamp"]))
+    phases, cur = [], []
+    for r in rows:
+        k = kind(r["Kernel_Name"])
+        if k is None:
+            if cur:
+                phases.append(cur)
+            cur = []
+        else:
+            cur.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), k))
+    if cur:
+        phases.append(cur)
+    for p in (p for p in phases if len(p) >= 200):
+        busy, span = sum(e - s_ for s_, e, _ in p), p[-1][1] - p[0][0]
+        print(f"phase of {len(p)} kernels: {span / 1e6:.3f} ms from first begin to last end, kernels themselves "
+              f"{busy / 1e6:.3f} ms")
+        gaps = {}
+        for a, b in zip(p, p[1:]):
+            gaps.setdefault((a[2], b[2]), []).append(b[0] - a[1])
+        for (a, b), v in sorted(gaps.items()):
+            print(f"    {a:>20s} -> {b:<20s} n={len(v):4d}  median gap {statistics.median(v) / 1e3:7.2f} us")
+    return 0
+
+
 def run_full_model(args, as_record: bool = False):
     """Full Llama-3-8B per-rank pass at logical W=8 on one GPU: embedding, 32 decoder layers, lm_head and
     the final norm as 35 parameter groups.  Forward: copy-in + copy-out of group i+1 run on a side stream while a
@@ -289,15 +326,24 @@ def run_full_model(args, as_record: bool = False):
     ev_done = [torch.cuda.Event() for _ in range(n)]    # reduce copy-in of group i done (compute stream)
     ev_freed = [torch.cuda.Event() for _ in range(n)]   # post-reduce of group i done: its reduce buffer is free
 
-    def step(copies=True, gemms=True, gather_on_side=False):
+    def recording(event, launch, stream, markers):
+        """`launch` on `stream` with `event` recorded at its end: by the kernel's own dispatch, or (markers) the
+        ordinary way, by a marker packet behind it."""
+        if markers:
+            launch()
+            event.record(stream)
+            return event
+        return _native.launch_recording(event, launch, stream)
+
+    def step(copies=True, gemms=True, gather_on_side=False, markers=False, backward_on_one_stream=False):
         # forward
         if copies:
             with torch.cuda.stream(side):
-                _native.launch_recording(ev_ready[0], lambda: unshard(0), side)
+                recording(ev_ready[0], lambda: unshard(0), side, markers)
         for i in range(n):
             if copies and i + 1 < n:
                 with torch.cuda.stream(side):  # prefetch the next group while this one computes
-                    _native.launch_recording(ev_ready[i + 1], lambda: unshard(i + 1), side)
+                    recording(ev_ready[i + 1], lambda: unshard(i + 1), side, markers)
             if copies:
                 main.wait_event(ev_ready[i])
             if gemms:
@@ -308,15 +354,21 @@ def run_full_model(args, as_record: bool = False):
             if gemms:
                 gemm()
                 gemm()
-            if copies and not gather_on_side:
+            if copies and backward_on_one_stream:
+                # (measurement only: no hand-off between streams in the backward half)
+                if i == n - 1:
+                    main.wait_stream(side)
+                reduce_in(i)
+                post(i)
+            elif copies and not gather_on_side:
                 key = id(groups[i]["res"])
                 if key in freed:
                     main.wait_event(freed[key])   # a shared gradient buffer is released by the post-reduce before
                 # compute stream, like the reference's foreach calls
-                _native.launch_recording(ev_done[i], lambda: reduce_in(i), main)
+                recording(ev_done[i], lambda: reduce_in(i), main, markers)
                 with torch.cuda.stream(side):     # reduce-scatter stream: waits for the reduce copy-in
                     side.wait_event(ev_done[i])
-                    freed[key] = _native.launch_recording(ev_freed[i], lambda: post(i), side)
+                    freed[key] = recording(ev_freed[i], lambda: post(i), side, markers)
             elif copies:
                 # not the reference's plan (the library's opt-in, set_reduce_copy_in_on_side_stream): the reduce
                 # copy-in leaves the compute stream as well; the side stream waits for the gradients, then runs both
@@ -327,15 +379,32 @@ def run_full_model(args, as_record: bool = False):
                     reduce_in(i)
                     post(i)
 
-    def timed(copies, gemms, reps, gather_on_side=False):
+    def timed(copies, gemms, reps, gather_on_side=False, **how):
         for _ in range(2):
-            step(copies, gemms, gather_on_side)
+            step(copies, gemms, gather_on_side, **how)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(reps):
-            step(copies, gemms, gather_on_side)
+            step(copies, gemms, gather_on_side, **how)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / reps * 1e3
+
+    if args.copies_only:
+        # the copies-only pass under four ways of handing work between the two streams, each phase fenced by a small
+        # torch fill kernel so that a kernel trace of this run can be cut into phases (--analyze-gaps)
+        out = {}
+        for name, how in (("reference_plan_marker_events", dict(markers=True)),
+                          ("reference_plan_kernel_recorded_events", dict()),
+                          ("reduce_copy_in_on_side_stream", dict(gather_on_side=True)),
+                          ("backward_half_on_one_stream", dict(backward_on_one_stream=True))):
+            torch.cuda.synchronize()
+            torch.zeros(12345, device=dev)
+            out[name] = round(timed(True, False, max(1, args.steps // 10), **how), 4)
+            log(f"  copies only, {name}: {out[name]} ms per pass")
+        torch.zeros(12345, device=dev)
+        torch.cuda.synchronize()
+        print(json.dumps({"workload": "llama3-8b-full-w8", "copies_only_ms_per_pass": out}), flush=True)
+        return 0
 
     def timed_loop(fn, reps):
         """ms per pass of fn(i) over all groups, back to back on the current stream."""
@@ -1542,6 +1611,12 @@ def main() -> int:
                     help="the same for the flat kernels (copy-in, flat copies and divides; default 0: they store "
                          "everything non-temporal; 1048576 = write-through everywhere)")
     ap.add_argument("--post-reduce-tail-mb", type=int, default=None, metavar="N", help="the same for the post-reduce")
+    ap.add_argument("--copies-only", action="store_true",
+                    help="llama3-8b-full-w8 only: run just the copies-only pass under four ways of handing work "
+                         "between the two streams (for a kernel trace)")
+    ap.add_argument("--analyze-gaps", metavar="CSV", default=None,
+                    help="no GPU work; summarise the idle time between consecutive kernels in the kernel-trace CSV that "
+                         "rocprofv3 wrote for `--workload llama3-8b-full-w8 --copies-only --no-parity`")
     ap.add_argument("--analyze-trace", metavar="CSV", default=None,
                     help="llama3-8b-full-w8 only: no GPU work; summarise the kernel-trace CSV that rocprofv3 wrote for "
                          "`--workload llama3-8b-full-w8 --steps 10 --no-parity` (GEMM resource columns, concurrency)")
@@ -1549,6 +1624,8 @@ def main() -> int:
 
     if args.analyze_trace:
         return analyze_overlap_trace(args.analyze_trace)
+    if args.analyze_gaps:
+        return analyze_gaps(args.analyze_gaps)
     if args.gpus != 1:
         log(f"bench.py: this build runs on ONE GPU (the logical world size is a layout parameter); "
             f"--gpus {args.gpus} is not supported.")
