@@ -214,10 +214,10 @@ def test_per_table_write_through_tail(nat):
     table.close()
 
 
-@pytest.mark.parametrize("tail_mb", [0, 1, 3])
+@pytest.mark.parametrize("tail_mb", [0, 1, 3, 1 << 20])
 def test_flat_kernels_with_the_write_through_boundary_inside_the_buffer(nat, tail_mb):
-    """The flat kernels write through everywhere by default; with a tail option below the size of the output the
-    tiles before the last megabytes store non-temporal instead (0: all of them).  Same bytes either way."""
+    """The flat kernels store non-temporal by default (tail option 0); with a tail option below the size of the output
+    the last megabytes are stored write-through instead (2^20: everything).  Same bytes either way."""
     g = torch.Generator().manual_seed(131)
     n = 1_500_003  # 3 MB of bf16, 6 MB of fp32
     defaults = (nat.get_option(nat.OPT_FLAT_TAIL_MB), nat.get_option(nat.OPT_POST_REDUCE_TAIL_MB))
