@@ -356,3 +356,36 @@ def test_sumsq_reduce_partials(nat):
     with pytest.raises(RuntimeError, match="invalid argument"):
         nat.sumsq_reduce_partials(torch.zeros(10000, dtype=torch.float64, device=DEV), 10000,
                                   torch.zeros(2, dtype=torch.float64, device=DEV))
+
+
+@pytest.mark.parametrize("impl", ["fused", "foreach"])
+def test_adamw_against_torch_optim_on_the_gpu(nat, impl):
+    """What the reference itself would run on this GPU: torch.optim.AdamW(fused=True | foreach=True) on device
+    tensors (ya_fsdp/_tensor.py:269-312 forwards those ops to the local fragments).  torch's GPU kernels are compiled
+    with multiply-add contraction and evaluate the update in their own operation order, so they differ from torch's
+    CPU kernels (which the oracle follows bit for bit in the moments) in the last bits; this test states how far the
+    fused kernel here is from them after each of five steps, in binary32 ulps of max(|value|, floor) with the floors
+    at each quantity's typical size (1e-4, 1e-8, 1e-3: a moment that cancels to almost nothing would otherwise
+    dominate a relative measure).  Measured: foreach 0 / 2.9 / 9.1 ulps (exp_avg / exp_avg_sq / parameters), fused
+    4.8 / 4.0 / 13.2; asserted with a margin of about two."""
+    n = 300_000
+    gen = torch.Generator().manual_seed(207)
+    p0 = torch.randn(n, generator=gen) * 0.02
+    param = torch.nn.Parameter(p0.to(DEV))
+    hp = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.1)
+    opt = torch.optim.AdamW([param], fused=(impl == "fused"), foreach=(impl == "foreach"), **hp)
+    dp, dm, dv = p0.to(DEV), torch.zeros(n, device=DEV), torch.zeros(n, device=DEV)
+    worst = {"exp_avg": 0.0, "exp_avg_sq": 0.0, "param": 0.0}
+    for step in range(1, 6):
+        grad = (torch.randn(n, generator=gen) * 1e-3).to(DEV)
+        param.grad = grad.clone()
+        opt.step()
+        nat.adamw_step(dp, grad, dm, dv, None, lr=1e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1, step=step)
+        st = opt.state[param]
+        for name, mine, theirs, floor in (("exp_avg", dm, st["exp_avg"], 1e-4), ("exp_avg_sq", dv, st["exp_avg_sq"], 1e-8),
+                                          ("param", dp, param.detach(), 1e-3)):
+            scale = torch.maximum(theirs.abs().double(), torch.full_like(theirs, floor, dtype=torch.float64))
+            ulps = float(((mine.double() - theirs.double()).abs() / (scale * 2.0**-23)).max())
+            worst[name] = max(worst[name], ulps)
+    print("fused AdamW here vs torch.optim on the GPU,", impl, "- worst difference in ulps:", worst, flush=True)
+    assert worst["exp_avg"] <= 8.0 and worst["exp_avg_sq"] <= 8.0 and worst["param"] <= 32.0, worst
