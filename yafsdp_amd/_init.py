@@ -55,23 +55,15 @@ def _get_managed_modules(root_modules: tuple, get_state, ignored_params: set | N
 
 
 def _ignore_module(module: nn.Module, ignored_params: set, decision: dict) -> bool:
-    """ya_fsdp/_init.py:79-108: a module is ignored only if all its parameters
-    and all its children are."""
-    if module in decision:
-        return decision[module]
-    if len(list(module.buffers(recurse=False))) > 0:
-        decision[module] = False
-        return False
-    for _, param in module.named_parameters(recurse=False):
-        if param not in ignored_params:
-            decision[module] = False
-            return False
-    for child in module.children():
-        if not _ignore_module(child, ignored_params, decision):
-            decision[module] = False
-            return False
-    decision[module] = True
-    return True
+    """A module drops out of the managed set only if it owns no buffer, every parameter it owns is ignored and
+    every child drops out too (the rule of ya_fsdp/_init.py:79-108); ``decision`` memoises per module."""
+    if module not in decision:
+        decision[module] = (
+            next(iter(module.buffers(recurse=False)), None) is None
+            and all(param in ignored_params for param in module.parameters(recurse=False))
+            and all(_ignore_module(child, ignored_params, decision) for child in module.children())
+        )
+    return decision[module]
 
 
 def _adjust_managed_modules(modules: list[nn.Module], ignored_params: set) -> list[nn.Module]:
@@ -80,29 +72,22 @@ def _adjust_managed_modules(modules: list[nn.Module], ignored_params: set) -> li
 
 
 def _get_managed_states(modules: list[nn.Module], ignored_params: set | None = None):
-    """ya_fsdp/_init.py:164-189."""
-    params: list[nn.Parameter] = []
-    buffers: list[torch.Tensor] = []
-    visited_params: set[nn.Parameter] = set()
-    visited_buffers: set[torch.Tensor] = set()
-    ignored_params = ignored_params or set()
+    """The parameters and buffers that the given modules own directly, each object once, in module order
+    (what ya_fsdp/_init.py:164-189 collects).  A 0-d parameter cannot be split along dim 0 and is refused."""
+    skip = ignored_params or set()
+    params: dict[nn.Parameter, None] = {}  # insertion-ordered, keyed by identity (a tensor hashes by id)
+    buffers: dict[torch.Tensor, None] = {}
     for module in modules:
         for name, param in module.named_parameters(recurse=False):
-            if param in ignored_params:
+            if param in skip or param in params:
                 continue
-            if param not in visited_params:
-                if len(param.shape) == 0:
-                    raise ValueError(
-                        "fully_shard doesn't support scalar parameters. "
-                        f"Change {name} to a 1D tensor with numel equal to 1."
-                    )
-                params.append(param)
-                visited_params.add(param)
-        for buffer in module.buffers(recurse=False):
-            if buffer not in visited_buffers:
-                buffers.append(buffer)
-                visited_buffers.add(buffer)
-    return params, buffers
+            if param.dim() == 0:
+                raise ValueError(
+                    f"fully_shard doesn't support scalar parameters. Change {name} to a 1D tensor with numel equal to 1."
+                )
+            params[param] = None
+        buffers.update(dict.fromkeys(module.buffers(recurse=False)))
+    return list(params), list(buffers)
 
 
 def _move_states_to_device(params, buffers, device: torch.device) -> None:

@@ -344,72 +344,100 @@ class YaFSDPState(_State):
                 group._module_fqn = module_name if group._module_fqn is None else f"{group._module_fqn}, {module_name}"
 
     # -------------------------------------------------------------------- hooks --
+    # Order of events in one iteration, which is the reference's (ya_fsdp/_state.py:443-565): forward pre-hook
+    # (root bookkeeping, input casts, the group's unshard, explicit prefetches) -> module forward -> forward
+    # post-hook (the group's reshard, tensor hooks on the outputs) -> those tensor hooks during backward (the
+    # group's unshard for backward, explicit prefetches) -> one callback at the end of backward that settles
+    # every group.  A forward that runs INSIDE backward (activation recomputation) finds the state in
+    # PRE_BACKWARD and passes through both forward hooks untouched.
+    def _recomputing_in_backward(self) -> bool:
+        return self._training_state == TrainingState.PRE_BACKWARD
+
+    def _cast_floating_point(self, tree: Any, dtype: torch.dtype, label: str) -> Any:
+        with profiler_range(label):
+            return _apply_to_tensors(functools.partial(_cast_fp_tensor, dtype), tree)
+
+    @staticmethod
+    def _prefetch(states: "list[YaFSDPState]", phase: str) -> None:
+        for other in states:
+            if other._fsdp_param_group is not None:
+                YaFSDPParamGroup._prefetch_unshard(other._fsdp_param_group, phase)
+
     def _pre_forward(self, module: nn.Module, args: tuple, kwargs: dict) -> tuple[tuple, dict]:
-        """ya_fsdp/_state.py:443-468."""
-        if self._training_state == TrainingState.PRE_BACKWARD:
+        if self._recomputing_in_backward():
             return args, kwargs
         self._training_state = TrainingState.FORWARD
         args, kwargs = self._root_pre_forward(module, args, kwargs)
-        if self._mp_policy.cast_forward_inputs and self._mp_policy.param_dtype:
-            with profiler_range("YaFSDP::cast_forward_inputs"):
-                cast_fn = functools.partial(_cast_fp_tensor, self._mp_policy.param_dtype)
-                args, kwargs = _apply_to_tensors(cast_fn, args), _apply_to_tensors(cast_fn, kwargs)
+        policy = self._mp_policy
+        if policy.cast_forward_inputs and policy.param_dtype:
+            args, kwargs = self._cast_floating_point((args, kwargs), policy.param_dtype, "YaFSDP::cast_forward_inputs")
         if self._fsdp_param_group:
             args, kwargs = self._fsdp_param_group.pre_forward(module, args, kwargs)
-        for fsdp_state in self._states_to_forward_prefetch:
-            if (target := fsdp_state._fsdp_param_group) is not None:
-                YaFSDPParamGroup._prefetch_unshard(target, "forward")
+        self._prefetch(self._states_to_forward_prefetch, "forward")
         return args, kwargs
 
     def _post_forward(self, module: nn.Module, input: Any, output: Any) -> Any:
-        """ya_fsdp/_state.py:470-488."""
-        if self._training_state == TrainingState.PRE_BACKWARD:
+        if self._recomputing_in_backward():
             return output
         if self._fsdp_param_group:
             output = self._fsdp_param_group.post_forward(module, input, output)
-        output = self._register_pre_backward_hook(output)
+        self._hook_outputs_for_backward(output)
         self._training_state = TrainingState.IDLE
-        if self._state_ctx.iter_forward_root is self:
-            self._state_ctx.iter_forward_root = None
-        if self._mp_policy.output_dtype is not None:
-            with profiler_range("YaFSDP::cast_forward_outputs"):
-                output = _apply_to_tensors(functools.partial(_cast_fp_tensor, self._mp_policy.output_dtype), output)
+        ctx = self._state_ctx
+        if ctx.iter_forward_root is self:  # the outermost forward of this iteration has returned
+            ctx.iter_forward_root = None
+        if (dtype := self._mp_policy.output_dtype) is not None:
+            output = self._cast_floating_point(output, dtype, "YaFSDP::cast_forward_outputs")
         return output
 
+    def _hook_outputs_for_backward(self, output: Any) -> None:
+        """Every output tensor that takes part in autograd announces this module's backward
+        (ya_fsdp/_state.py:549-556); under ``no_grad`` there is no backward to announce."""
+        if not torch.is_grad_enabled():
+            return
+        for leaf in tree_flatten(output)[0]:
+            if torch.is_tensor(leaf) and leaf.requires_grad:
+                leaf.register_hook(self._pre_backward)
+
     def _pre_backward(self, grad: torch.Tensor) -> torch.Tensor:
-        """ya_fsdp/_state.py:490-499."""
         self._training_state = TrainingState.PRE_BACKWARD
-        self._register_root_post_backward_final_callback()
+        self._queue_end_of_backward()
+        explicit = self._states_to_backward_prefetch
         if self._fsdp_param_group:
-            default_prefetch = len(self._states_to_backward_prefetch) == 0
-            self._fsdp_param_group.pre_backward(default_prefetch)
-        for fsdp_state in self._states_to_backward_prefetch:
-            if (target := fsdp_state._fsdp_param_group) is not None:
-                YaFSDPParamGroup._prefetch_unshard(target, "backward")
+            # without an explicit list the group prefetches its predecessor in forward order itself
+            self._fsdp_param_group.pre_backward(not explicit)
+        self._prefetch(explicit, "backward")
         return grad
 
+    def _queue_end_of_backward(self) -> None:
+        """The first module to enter backward queues the end-of-backward callback on the autograd engine, once
+        per backward pass (ya_fsdp/_state.py:558-565)."""
+        ctx = self._state_ctx
+        if not ctx.post_backward_final_callback_queued:
+            ctx.post_backward_final_callback_queued = True
+            Variable._execution_engine.queue_callback(self._root_post_backward_final_callback)
+
     def _root_post_backward_final_callback(self) -> None:
-        """ya_fsdp/_state.py:501-532."""
+        """End of a backward pass (ya_fsdp/_state.py:501-532): groups whose post-backward node never ran are
+        reduced now, every state returns to IDLE, and after the last backward of an iteration the groups wait for
+        their reductions and the recorded forward order is dropped."""
+        ctx = self._state_ctx
+        last = ctx.is_last_backward
         with profiler_range("YaFSDP::root_post_backward_callback"):
-            for state in self._state_ctx.all_states:
+            for state in ctx.all_states:
                 group = state._fsdp_param_group
-                if group and group._training_state != TrainingState.POST_BACKWARD:
-                    # forward inputs did not require gradient: the autograd node did not run
-                    group.post_backward()
+                if group is not None and group._training_state != TrainingState.POST_BACKWARD:
+                    group.post_backward()  # its forward inputs did not require gradient: no autograd node fired
                 state._training_state = TrainingState.IDLE
-                if group:
+                if group is not None:
                     group._training_state = TrainingState.IDLE
-                if self._state_ctx.is_last_backward:
+                if last:
                     state._finalize_backward()
-                if group is not None:  # :517-529
-                    ctxs = [group.data_buffer_ctx] + ([group.grad_buffer_ctx] if group.grad_buffer_ctx else [])
-                    for ctx in ctxs:
-                        for handle in ctx.yccl_handles.values():
-                            if handle is not None:
-                                handle.process_profiling_events()
-            if self._state_ctx.is_last_backward:
+                if group is not None:
+                    _flush_profiling_events(group)
+            if last:
                 self._comm_ctx.post_forward_order.clear()
-            self._state_ctx.post_backward_final_callback_queued = False
+            ctx.post_backward_final_callback_queued = False
 
     def _finalize_backward(self) -> None:
         if self._modules_to_run_forward:  # ya_fsdp/_state.py:534-546
@@ -422,22 +450,16 @@ class YaFSDPState(_State):
         if self._fsdp_param_group:
             self._fsdp_param_group.finalize_backward()
 
-    def _register_pre_backward_hook(self, output: Any) -> Any:
-        """ya_fsdp/_state.py:549-556."""
-        if not torch.is_grad_enabled():
-            return output
-        flat_outputs, _ = tree_flatten(output)
-        for t in flat_outputs:
-            if torch.is_tensor(t) and t.requires_grad:
-                t.register_hook(self._pre_backward)
-        return output
 
-    def _register_root_post_backward_final_callback(self) -> None:
-        """ya_fsdp/_state.py:558-565."""
-        if self._state_ctx.post_backward_final_callback_queued:
-            return
-        self._state_ctx.post_backward_final_callback_queued = True
-        Variable._execution_engine.queue_callback(self._root_post_backward_final_callback)
+def _flush_profiling_events(group: YaFSDPParamGroup) -> None:
+    """Communication-library handles attached to the group's buffers turn the events they recorded during the
+    pass into profiler ranges (ya_fsdp/_state.py:517-529)."""
+    for buffer_ctx in (group.data_buffer_ctx, group.grad_buffer_ctx):
+        if buffer_ctx is None:
+            continue
+        for handle in buffer_ctx.yccl_handles.values():
+            if handle is not None:
+                handle.process_profiling_events()
 
 
 def _get_module_fsdp_state(module: nn.Module) -> YaFSDPState | None:

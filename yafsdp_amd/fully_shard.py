@@ -33,42 +33,54 @@ def fully_shard(
     shard_alignment: int = 8,
     device: torch.device | str | None = None,
 ) -> "YaFSDPModule | list[YaFSDPModule]":
-    """ya_fsdp/fully_shard.py:67-129.  A list of modules forms ONE parameter group
-    whose parameters are gathered before the first of them runs forward and
-    released after the last one has (ya_fsdp/_state.py:575-613)."""
+    """Same keyword contract and return value as ya_fsdp/fully_shard.py:67-129.  A list of modules forms ONE
+    parameter group whose parameters are gathered before the first of them runs forward and released after the
+    last one has (ya_fsdp/_state.py:575-613).  ``reshard_after_forward=None`` means "True, and let the root decide
+    which groups may stay unsharded"."""
+    roots = _group_roots(module)
+    state = YaFSDPState()
+    state.init(roots, resolve_device(device), mp_policy, reshard_after_forward is not None)
+    managed = _get_managed_modules(roots, _get_module_fsdp_state, ignored_params)
+    params, buffers = _get_managed_states(managed, ignored_params)
+    _move_states_to_device(params, buffers, state._device)
+    if params:
+        state._fsdp_param_group = group = YaFSDPParamGroup(
+            params, mesh_info_from(mesh), state._device, mp_policy, shard_alignment,
+            names=_param_names(roots, params), modules=roots,
+        )
+        group.reshard_after_forward = reshard_after_forward is None or bool(reshard_after_forward)
+    for root in roots:
+        root.__class__ = _sharded_class_of(type(root))
+    return module  # type: ignore[return-value]
+
+
+def _group_roots(module: Any) -> tuple:
+    """What one ``fully_shard`` call wraps: the module itself, or the members of a list that are not inside
+    another member.  Containers without a forward and modules that are wrapped already are refused, as in
+    ya_fsdp/fully_shard.py:77-80 and torch's ``contract``."""
     if isinstance(module, (nn.ModuleList, nn.ModuleDict)):
         raise ValueError(f"fully_shard does not support containers that do not implement forward: {module}")
-    arg_module = module
     if isinstance(module, nn.Module):
-        modules = (module,)
+        roots = (module,)
     else:
-        modules = tuple(_get_root_modules(list(module)))
-        if not modules or not all(isinstance(m, nn.Module) for m in modules):
+        members = list(module)
+        if not members or not all(isinstance(m, nn.Module) for m in members):
             raise ValueError("fully_shard expects a module or a non-empty list of modules")
-    for m in modules:
-        if _get_module_fsdp_state(m) is not None:
-            raise AssertionError(f"fully_shard has already been applied to {type(m).__name__}")
-    mesh_info = mesh_info_from(mesh)
-    device = resolve_device(device)
-    auto_reshard_after_forward = reshard_after_forward is not None
-    state = YaFSDPState()
-    state.init(modules, device, mp_policy, auto_reshard_after_forward)
-    managed_modules = _get_managed_modules(modules, _get_module_fsdp_state, ignored_params)
-    params, buffers = _get_managed_states(managed_modules, ignored_params)
-    _move_states_to_device(params, buffers, device)
-    if params:
-        names = _param_names(modules, params)
-        group = YaFSDPParamGroup(params, mesh_info, device, mp_policy, shard_alignment, names=names, modules=modules)
-        group.reshard_after_forward = True if reshard_after_forward is None else bool(reshard_after_forward)
-        state._fsdp_param_group = group
-    for m in modules:
-        cls = m.__class__
-        new_cls = cls_to_fsdp_cls.get(cls)
-        if not new_cls:
-            new_cls = type(f"YaFSDP{cls.__name__}", (YaFSDPModule, cls), {"__deepcopy__": _unimplemented_deepcopy})
-            cls_to_fsdp_cls[cls] = new_cls
-        m.__class__ = new_cls
-    return arg_module  # type: ignore[return-value]
+        roots = tuple(_get_root_modules(members))
+    for root in roots:
+        if _get_module_fsdp_state(root) is not None:
+            raise AssertionError(f"fully_shard has already been applied to {type(root).__name__}")
+    return roots
+
+
+def _sharded_class_of(cls: type) -> type:
+    """``YaFSDP<Cls>``: the module's own class with ``YaFSDPModule`` in front of it in the method resolution order,
+    made once per class (ya_fsdp/fully_shard.py:119-127)."""
+    if cls not in cls_to_fsdp_cls:
+        cls_to_fsdp_cls[cls] = type(
+            f"YaFSDP{cls.__name__}", (YaFSDPModule, cls), {"__deepcopy__": _unimplemented_deepcopy}
+        )
+    return cls_to_fsdp_cls[cls]
 
 
 def _get_root_modules(modules: list) -> list:
@@ -99,21 +111,49 @@ def _unimplemented_deepcopy(*args: Any, **kwargs: Any) -> NoReturn:
 
 
 class YaFSDPModule:
-    """Methods added to a module by ``fully_shard`` (ya_fsdp/fully_shard.py:138-256)."""
+    """The methods a module gains from ``fully_shard`` (names, arguments and effects of
+    ya_fsdp/fully_shard.py:138-256).  Every setter is a write to the module's parameter group or to the state the
+    groups of one model share; those that change what a shared buffer must hold re-run the buffer validation once
+    the root has assigned buffers."""
 
     def __new__(cls, *args: Any, **kwargs: Any) -> Any:
-        orig_cls = cls.__mro__[2]
-        self = orig_cls.__new__(orig_cls, *args, **kwargs)
-        self.__init__(*args, **kwargs)
-        return self
+        # YaFSDP<Cls> -> YaFSDPModule -> Cls: constructing the swapped class constructs a plain Cls
+        plain = cls.__mro__[2]
+        obj = plain.__new__(plain, *args, **kwargs)
+        obj.__init__(*args, **kwargs)
+        return obj
 
+    # ---- lookups the methods share -------------------------------------------------------------
+    def _get_fsdp_state(self) -> YaFSDPState:
+        state = _get_module_fsdp_state(self)  # type: ignore[arg-type]
+        if state is None:
+            raise AssertionError(f"No YaFSDP state found on {self}")
+        return state
+
+    def _fsdp_modules(self, recurse: bool) -> "list[YaFSDPModule]":
+        """This module, or every wrapped module at or below it, in ``nn.Module.modules()`` order."""
+        candidates = self.modules() if recurse else (self,)  # type: ignore[attr-defined]
+        return [m for m in candidates if isinstance(m, YaFSDPModule)]
+
+    def _own_group(self) -> "YaFSDPParamGroup | None":
+        return self._get_fsdp_state()._fsdp_param_group
+
+    def _write_to_groups(self, recurse: bool, attr: str, value: Any, *, revalidate: bool = False) -> None:
+        for module in self._fsdp_modules(recurse):
+            state = module._get_fsdp_state()
+            if (group := state._fsdp_param_group) is None:
+                continue
+            setattr(group, attr, value)
+            if revalidate and state._is_root is not None:  # buffers are assigned: check they still suffice
+                state.validate_shared_state()
+
+    # ---- gathering and releasing by hand -------------------------------------------------------
     def reshard(self) -> None:
-        if group := self._get_fsdp_state()._fsdp_param_group:
+        if (group := self._own_group()) is not None:
             group.reshard()
 
     def unshard(self, async_op: bool = False) -> "UnshardHandle | None":
-        state = self._get_fsdp_state()
-        group = state._fsdp_param_group
+        group = self._own_group()
         if group is not None:
             group.unshard(async_op=async_op)
         handle = _UnshardHandleImpl(group)
@@ -122,56 +162,28 @@ class YaFSDPModule:
         handle.wait()
         return None
 
-    def set_is_last_backward(self, is_last_backward: bool) -> None:
-        self._get_fsdp_state()._state_ctx.is_last_backward = is_last_backward
-
+    # ---- per-group switches --------------------------------------------------------------------
     def set_requires_gradient_sync(self, requires_gradient_sync: bool, *, recurse: bool = True) -> None:
-        for module in self._fsdp_modules(recurse):
-            state = module._get_fsdp_state()
-            if group := state._fsdp_param_group:
-                group.reduce_grads = requires_gradient_sync
-                if state._is_root is not None:
-                    state.validate_shared_state()
+        self._write_to_groups(recurse, "reduce_grads", requires_gradient_sync, revalidate=True)
+
+    def set_reshard_after_backward(self, reshard_after_backward: bool, *, recurse: bool = True) -> None:
+        self._write_to_groups(recurse, "reshard_after_backward", reshard_after_backward, revalidate=True)
 
     def set_reshard_after_forward(self, reshard_after_forward: bool, recurse: bool = True) -> None:
         if not isinstance(reshard_after_forward, bool):
             raise ValueError(f"reshard_after_forward should be a bool, got {type(reshard_after_forward)}")
         for module in self._fsdp_modules(recurse):
-            state = module._get_fsdp_state()
-            state._auto_reshard_after_forward = False
-            if group := state._fsdp_param_group:
-                group.reshard_after_forward = reshard_after_forward
-
-    def set_reshard_after_backward(self, reshard_after_backward: bool, *, recurse: bool = True) -> None:
-        for module in self._fsdp_modules(recurse):
-            state = module._get_fsdp_state()
-            if group := state._fsdp_param_group:
-                group.reshard_after_backward = reshard_after_backward
-                if state._is_root is not None:
-                    state.validate_shared_state()
-
-    def set_modules_to_forward_prefetch(self, modules: "list[YaFSDPModule]") -> None:
-        _assert_all_fsdp_modules(modules)
-        self._get_fsdp_state()._states_to_forward_prefetch = [m._get_fsdp_state() for m in modules]
-
-    def set_modules_to_backward_prefetch(self, modules: "list[YaFSDPModule]") -> None:
-        _assert_all_fsdp_modules(modules)
-        self._get_fsdp_state()._states_to_backward_prefetch = [m._get_fsdp_state() for m in modules]
-
-    def set_post_optim_event(self, event: torch.cuda.Event) -> None:
-        self._get_fsdp_state()._state_ctx.post_optim_event = event
+            module._get_fsdp_state()._auto_reshard_after_forward = False  # an explicit choice: the root keeps it
+        self._write_to_groups(recurse, "reshard_after_forward", reshard_after_forward)
 
     def set_unshard_in_backward(self, unshard_in_backward: bool) -> None:
-        if (group := self._get_fsdp_state()._fsdp_param_group) is not None:
-            group.unshard_in_backward = unshard_in_backward
+        self._write_to_groups(False, "unshard_in_backward", unshard_in_backward)
 
     def set_gradient_divide_factor(self, factor: float) -> None:
-        if (group := self._get_fsdp_state()._fsdp_param_group) is not None:
-            group.gradient_divide_factor = factor
+        self._write_to_groups(False, "gradient_divide_factor", factor)
 
     def set_force_sum_reduction_for_comms(self, enable: bool) -> None:
-        if (group := self._get_fsdp_state()._fsdp_param_group) is not None:
-            group.force_sum_reduction_for_comms = enable
+        self._write_to_groups(False, "force_sum_reduction_for_comms", enable)
 
     def set_reduce_copy_in_on_side_stream(self, enable: bool, *, recurse: bool = True) -> None:
         """Not part of the reference's interface.  The reference flattens a group's gradients into the reduce buffer
@@ -180,50 +192,60 @@ class YaFSDPModule:
         front of the post-reduce, and the compute stream only hands the gradients over.  Same results (the
         kernels and their order on the reduce buffer do not change); measured 4-5 % faster on a full Llama-3-8B
         pass next to GEMMs."""
-        for module in self._fsdp_modules(recurse):
-            if group := module._get_fsdp_state()._fsdp_param_group:
-                group.reduce_copy_in_on_side_stream = bool(enable)
+        self._write_to_groups(recurse, "reduce_copy_in_on_side_stream", bool(enable))
 
-    def _fsdp_modules(self, recurse: bool) -> "list[YaFSDPModule]":
-        mods = list(self.modules()) if recurse else [self]  # type: ignore[attr-defined]
-        return [m for m in mods if isinstance(m, YaFSDPModule)]
+    # ---- state shared by the groups of one model -----------------------------------------------
+    def set_is_last_backward(self, is_last_backward: bool) -> None:
+        self._get_fsdp_state()._state_ctx.is_last_backward = is_last_backward
 
-    def _get_fsdp_state(self) -> YaFSDPState:
-        if (state := _get_module_fsdp_state(self)) is None:  # type: ignore[arg-type]
-            raise AssertionError(f"No YaFSDP state found on {self}")
-        return state
+    def set_post_optim_event(self, event: torch.cuda.Event) -> None:
+        self._get_fsdp_state()._state_ctx.post_optim_event = event
+
+    def set_modules_to_forward_prefetch(self, modules: "list[YaFSDPModule]") -> None:
+        self._get_fsdp_state()._states_to_forward_prefetch = _states_of(modules)
+
+    def set_modules_to_backward_prefetch(self, modules: "list[YaFSDPModule]") -> None:
+        self._get_fsdp_state()._states_to_backward_prefetch = _states_of(modules)
 
     def _apply(self, *args: Any, **kwargs: Any) -> Any:
-        """ya_fsdp/fully_shard.py:241-252."""
+        """``.to()`` / ``.float()`` / ``.cuda()`` act on the registered (sharded) parameters, after which each
+        parameter's shard bookkeeping is rebuilt from what ``nn.Module._apply`` left (ya_fsdp/fully_shard.py:241-252)."""
         self.reshard()
         ret = super()._apply(*args, **kwargs)  # type: ignore[misc]
-        if not (group := self._get_fsdp_state()._fsdp_param_group):
-            return ret
-        with torch.no_grad():
-            for fsdp_param in group.fsdp_params:
-                fsdp_param.reset_sharded_param()
+        if (group := self._own_group()) is not None:
+            with torch.no_grad():
+                for fsdp_param in group.fsdp_params:
+                    fsdp_param.reset_sharded_param()
         return ret
 
 
 class UnshardHandle:
+    """What ``unshard(async_op=True)`` returns: ``wait()`` makes the current stream wait for the gathered
+    parameters."""
+
     def wait(self) -> None:
         return
 
 
 class _UnshardHandleImpl(UnshardHandle):
     def __init__(self, fsdp_param_group: YaFSDPParamGroup | None):
-        self._fsdp_param_group = fsdp_param_group
+        self._fsdp_param_group = fsdp_param_group  # dropped at the first wait: a handle must not keep a group alive
         self._all_gather_result = None
 
     def wait(self) -> None:
-        if self._fsdp_param_group is not None:
-            self._all_gather_result = self._fsdp_param_group.wait_for_unshard()
-            self._fsdp_param_group = None
-        elif (result := self._all_gather_result) is not None:
-            result.wait()
+        group, self._fsdp_param_group = self._fsdp_param_group, None
+        if group is not None:
+            self._all_gather_result = group.wait_for_unshard()
+        elif self._all_gather_result is not None:
+            self._all_gather_result.wait()
 
 
 def _assert_all_fsdp_modules(modules) -> None:
     for module in modules:
         if not isinstance(module, YaFSDPModule):
             raise ValueError(f"Expects YaFSDPModule but got {type(module)}: {module}")
+
+
+def _states_of(modules) -> "list[YaFSDPState]":
+    _assert_all_fsdp_modules(modules)
+    return [module._get_fsdp_state() for module in modules]
