@@ -71,3 +71,35 @@ def test_staging_slot_state_machine_against_a_simulated_runtime():
     binary = mod.build_stage_ring_check()
     r = subprocess.run([binary], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and r.stdout.strip().endswith("PASS"), r.stdout[-2000:] + r.stderr[-2000:]
+
+
+def _run_bench(*flags):
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    bench = Path(__file__).resolve().parents[1] / "bench.py"
+    return subprocess.run([sys.executable, str(bench), *flags], capture_output=True, text=True, timeout=300)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every figure of this build is one GPU's: a request for more ends at once, with a message that says so and
+    without a result line on stdout."""
+    done = _run_bench("--gpus", "2", "--steps", "1", "--warmup", "0")
+    assert done.returncode != 0
+    assert "ONE GPU" in done.stderr + done.stdout
+    assert "{" not in done.stdout
+
+
+def test_bench_has_no_cpu_path_to_measure():
+    """Without a GPU the benchmark must not fall back to anything that runs on the host."""
+    import torch
+
+    if torch.cuda.is_available():
+        import pytest
+
+        pytest.skip("a GPU is visible")
+    done = _run_bench("--steps", "1", "--warmup", "0")
+    assert done.returncode != 0
+    assert "no GPU" in done.stderr + done.stdout
+    assert "{" not in done.stdout
