@@ -372,7 +372,7 @@ def _assert_same_masters(got, want):
         assert torch.equal(got[k].view(torch.int32), want[k].detach().view(torch.int32)), k
 
 
-def test_setters_that_must_not_change_the_numbers():
+def test_setters_that_must_not_change_the_numbers(monkeypatch):
     """ya_fsdp/fully_shard.py:138-239: keeping parameters unsharded after backward, forcing SUM (at world size 1
     no division either way, ya_fsdp/_collectives.py:221-267), a post-optimizer event for the all-gather stream to
     wait on, and explicit prefetch orders leave the training bit-identical."""
@@ -407,6 +407,17 @@ def test_setters_that_must_not_change_the_numbers():
     groups = [g for m in model._fsdp_modules(True) if (g := m._get_fsdp_state()._fsdp_param_group) is not None]
     assert groups and all(g.reduce_copy_in_on_side_stream for g in groups)
     _assert_same_masters(_train(model, xs, 0.05), want)
+
+    # the same through the environment, for a training script that cannot call the setter
+    monkeypatch.setenv("YAFSDP_REDUCE_COPY_IN_ON_SIDE_STREAM", "1")
+    model = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    monkeypatch.delenv("YAFSDP_REDUCE_COPY_IN_ON_SIDE_STREAM")
+    groups = [g for m in model._fsdp_modules(True) if (g := m._get_fsdp_state()._fsdp_param_group) is not None]
+    assert groups and all(g.reduce_copy_in_on_side_stream for g in groups)
+    _assert_same_masters(_train(model, xs, 0.05), want)
+    plain = _wrap(copy.deepcopy(model0), mp_policy=MP)
+    assert not any(g.reduce_copy_in_on_side_stream
+                   for m in plain._fsdp_modules(True) if (g := m._get_fsdp_state()._fsdp_param_group) is not None)
 
 
 

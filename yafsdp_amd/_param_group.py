@@ -32,6 +32,7 @@ import weakref
 
 import contextlib
 import logging
+import os
 from enum import Enum, auto
 from typing import Any, Generator, Sequence
 
@@ -171,8 +172,9 @@ class YaFSDPParamGroup:
         self.unshard_in_backward: bool = True
         # opt-in, not the reference's plan (ya_fsdp/_param_group.py:669-708 runs the foreach calls on the compute
         # stream): the reduce copy-in of a pass that reduces runs on the reduce-scatter stream as well, right in
-        # front of the post-reduce, and the compute stream goes on with the next group's backward at once
-        self.reduce_copy_in_on_side_stream: bool = False
+        # front of the post-reduce, and the compute stream goes on with the next group's backward at once.
+        # YAFSDP_REDUCE_COPY_IN_ON_SIDE_STREAM=1 turns it on for every group of a process whose code cannot change.
+        self.reduce_copy_in_on_side_stream: bool = os.environ.get("YAFSDP_REDUCE_COPY_IN_ON_SIDE_STREAM", "0") == "1"
         self._all_gather_result: AllGatherResult | None = None
         self._post_reduce_event: torch.cuda.Event | None = None
 
