@@ -268,6 +268,18 @@ int yafsdp_flat_copy_fanout(void* const* dsts, int n_dst, int dst_dtype, const v
 int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* chunks, int n_src, int chunk_dtype,
                              int64_t n, double post_factor, int accumulate, void* stream);
 
+/* The same for a collective that scales inside the reduction: ReduceOp.AVG, or
+ * the pre-multiplied sum the reference builds for a custom divide factor
+ * (ya_fsdp/_collectives.py:243-249).  The collective library multiplies every
+ * rank's element by the scalar converted to the chunk dtype, which rounds each
+ * product to that dtype, and adds the products:
+ *   term_k = round(chunk_k * round(scalar))       both roundings to the chunk dtype
+ *   sum    = term_0 + term_1 + ... in binary32, in index order
+ *   out    = round(sum) to the chunk dtype;   shard = out or shard + out
+ * With one chunk this is yafsdp_post_reduce_premul. */
+int yafsdp_post_reduce_fanin_premul(void* shard, int shard_dtype, const void* const* chunks, int n_src,
+                                    int chunk_dtype, int64_t n, double scalar, int accumulate, void* stream);
+
 /* The tensor side of a table fixed for many calls.  The reference's unsharded
  * parameters and gradient accumulators are views of pre-allocated buffers that
  * live as long as the group (ya_fsdp/_param_group.py:409-457), and consumers of

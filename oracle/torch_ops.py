@@ -312,15 +312,24 @@ def reduce_scatter_fanin(
     chunks: Sequence[torch.Tensor],
     postdivide_factor: float | None,
     accumulate: bool,
+    premul: float | None = None,
 ) -> None:
     """A reduce-scatter over the ranks' chunks with binary32 accumulation in rank
     order (``acc_type=torch.float32``, ya_fsdp/_collectives.py:157-161) whose output
     has the reduce dtype, then the post-divide (:165) and ``copy_`` / ``add_``
-    into the gradient shard (:185 / :189)."""
+    into the gradient shard (:185 / :189).  ``premul``: the collective scales
+    inside the reduction (``ReduceOp.AVG`` = 1 / ranks, or ``_make_nccl_premul_sum``,
+    :243-249) - the collective library converts the scalar to the data type and
+    multiplies every rank's element by it in that type before the sum."""
+    dtype = chunks[0].dtype
+    if premul is not None:
+        assert postdivide_factor is None
+        scalar = torch.tensor(premul, dtype=torch.float32).to(dtype)
+        chunks = [c * scalar for c in chunks]  # same-dtype tensor product: rounds to dtype
     acc = chunks[0].to(torch.float32).clone()
     for c in chunks[1:]:
         acc.add_(c.to(torch.float32))
-    output_tensor = acc.to(chunks[0].dtype)
+    output_tensor = acc.to(dtype)
     div_if_needed(output_tensor, postdivide_factor)
     if accumulate:
         padded_sharded_param_grad.add_(output_tensor)

@@ -30,7 +30,7 @@ def test_library_exports_every_symbol():
     import __graft_entry__
 
     assert _native.lib.yafsdp_version() // 1000 == __graft_entry__.ABI_MAJOR  # what build() checks
-    assert _native.lib.yafsdp_version() == 1006  # 1.1: yafsdp_flat_copy_bytes; 1.2-1.5: the four write-through tail options; 1.6: per-table tails, pre-multiplied share
+    assert _native.lib.yafsdp_version() == 1007  # 1.1: yafsdp_flat_copy_bytes; 1.2-1.5: the four write-through tail options; 1.6: per-table tails, pre-multiplied share; 1.7: pre-multiplied fan-in
     assert _native.error_string(0) == "success"
     assert "dtype" in _native.error_string(-2)
 

@@ -58,6 +58,42 @@ def test_reduce_fanin(nat, chunk_dt, shard_dt, post, acc, n_src):
         assert float(got[n:].float().min()) == 5.0 and float(got[n:].float().max()) == 5.0
 
 
+@pytest.mark.parametrize("chunk_dt,shard_dt", [(torch.bfloat16, torch.float32), (torch.float32, torch.float32),
+                                               (torch.float16, torch.float32), (torch.float32, torch.bfloat16),
+                                               (torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16)])
+@pytest.mark.parametrize("acc", [False, True])
+@pytest.mark.parametrize("n_src,scalar", [(1, 1 / 3), (3, 1 / 3), (6, 1 / 6), (8, 1 / 8), (16, 1 / 5.0), (2, 1.0)])
+def test_reduce_fanin_of_a_collective_that_scales_inside_the_reduction(nat, chunk_dt, shard_dt, acc, n_src, scalar):
+    """ReduceOp.AVG / the pre-multiplied sum (ya_fsdp/_collectives.py:243-249) over several ranks' chunks: each
+    element times the scalar in the chunk dtype, rounded, before the binary32 sum.  Specials included: a product
+    that overflows the chunk dtype becomes an infinity before the sum, as in the collective."""
+    g = torch.Generator().manual_seed(404 + n_src)
+    for n in SIZES:
+        print("fanin premul", chunk_dt, shard_dt, acc, n_src, scalar, n, flush=True)
+        chunks = [mixed_values(g, n, chunk_dt, 1e-3).roll(k) for k in range(n_src)]
+        shard = mixed_values(g, n, shard_dt, 1e-4).flip(0)
+        want = shard.clone()
+        torch_ops.reduce_scatter_fanin(want, [c.clone() for c in chunks], None, acc, premul=scalar)
+        got = torch.full((n + 8,), 5.0, dtype=shard_dt, device=DEV)
+        got[:n] = shard.to(DEV)
+        nat.post_reduce_fanin(got[:n], [c.to(DEV) for c in chunks], None, acc, premul=scalar)
+        assert_bits_equal(got[:n], want, f"pre-multiplied fan-in n={n}")
+        assert float(got[n:].float().min()) == 5.0 and float(got[n:].float().max()) == 5.0
+
+
+def test_one_chunk_premultiplied_fanin_is_the_one_rank_share(nat):
+    g = torch.Generator().manual_seed(405)
+    n = 50_001
+    chunk = mixed_values(g, n, torch.bfloat16, 1e-3).to(DEV)
+    shard = mixed_values(g, n, torch.float32, 1e-4).to(DEV)
+    a, b = shard.clone(), shard.clone()
+    nat.post_reduce_premul(a, chunk, 1 / 3, True)
+    nat.post_reduce_fanin(b, [chunk], None, True, premul=1 / 3)
+    assert_bits_equal(a, b.cpu(), "single chunk, pre-multiplied")
+    with pytest.raises(ValueError):
+        nat.post_reduce_fanin(b, [chunk], 3.0, True, premul=1 / 3)
+
+
 def test_one_chunk_fanin_is_post_reduce(nat):
     g = torch.Generator().manual_seed(403)
     n = 50_001

@@ -7,9 +7,10 @@ are done here by the test with the one-GPU kernels of those exchange points:
 
 * all-gather: rank r's gathered buffer receives the 16-bit all-gather input of every peer in its slot
   (``flat_copy``, what ``all_gather_into_tensor`` delivers, ya_fsdp/_collectives.py:60-65);
-* reduce-scatter: rank r's gradient shard receives the sum over all ranks' reduce buffers of chunk r, added in
-  binary32 in rank order, rounded to the reduce dtype, divided by W (``post_reduce_fanin``: ReduceOp.AVG with a
-  binary32 accumulator, ya_fsdp/_collectives.py:152-165, then :185).
+* reduce-scatter: rank r's gradient shard receives ``ReduceOp.AVG`` over all ranks' reduce buffers of chunk r as the
+  collective library defines it (a pre-multiplied sum: every rank's element times 1 / W in the reduce dtype, rounded,
+  then the sum), added in binary32 in rank order and rounded to the reduce dtype (``post_reduce_fanin(premul=)``:
+  ya_fsdp/_collectives.py:152-162 and :243-249 with a binary32 accumulator, then :185).
 
 The masters of all ranks, reassembled, must equal bit for bit those of one unsharded model trained by hand
 with the same arithmetic.  No second GPU, no process group, no peer mapping is involved."""
@@ -59,14 +60,14 @@ def _all_gather(ranks):
 
 
 def _reduce_scatter(ranks):
-    """Chunk r of every rank's reduce buffer, summed in binary32, rounded, averaged, into rank r's gradient shard."""
+    """Chunk r of every rank's reduce buffer, averaged as the collective does it, into rank r's gradient shard."""
     w = len(ranks)
     per_rank = [_groups(model) for model in ranks]
     for r in range(w):
         for g, group in enumerate(per_rank[r]):
             s = group.layout.padded_sharded_numel
             chunks = [per_rank[q][g]._reduce_scatter_input[None][r * s : (r + 1) * s] for q in range(w)]
-            _native.post_reduce_fanin(group._padded_sharded_param_grad[None], chunks, float(w), False)
+            _native.post_reduce_fanin(group._padded_sharded_param_grad[None], chunks, None, False, premul=1.0 / w)
             for fp in group.fsdp_params:
                 fp.sharded_param.grad = fp.sharded_param_grad      # ya_fsdp/_collectives.py:216-217
     for groups in per_rank:                                         # the reduce buffers are free again
@@ -77,11 +78,13 @@ def _reduce_scatter(ranks):
 
 
 def _reference(model0, batches, lr, w):
-    """One unsharded model, the same arithmetic by hand: bf16 gradients per micro-batch, summed over the ranks in
-    binary32 in rank order, rounded to bf16, divided by W in bf16, upcast into the fp32 gradient, SGD."""
+    """One unsharded model, the same arithmetic by hand: bf16 gradients per micro-batch, each multiplied by
+    bf16(1 / W) in bf16, summed over the ranks in binary32 in rank order, rounded to bf16, upcast into the fp32
+    gradient, SGD."""
     ref = copy.deepcopy(model0)
     masters = list(ref.parameters())
     opt = torch.optim.SGD(masters, lr=lr)
+    scalar = torch.tensor(1.0 / w, dtype=torch.float32).to(torch.bfloat16).to(DEV)
     for xs in batches:
         lowp = copy.deepcopy(ref).to(torch.bfloat16)
         sums = None
@@ -89,10 +92,10 @@ def _reference(model0, batches, lr, w):
             for p in lowp.parameters():
                 p.grad = None
             lowp(x.to(torch.bfloat16)).float().pow(2).mean().backward()
-            grads = [p.grad.float() for p in lowp.parameters()]
+            grads = [(p.grad * scalar).float() for p in lowp.parameters()]  # bf16 * bf16 -> bf16: one rounding
             sums = grads if sums is None else [a.add_(g) for a, g in zip(sums, grads)]
         for m, a in zip(masters, sums):
-            m.grad = a.bfloat16().div_(float(w)).float()
+            m.grad = a.bfloat16().float()
         opt.step()
         opt.zero_grad(set_to_none=True)
     return ref

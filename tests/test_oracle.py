@@ -266,6 +266,57 @@ def test_one_rank_share_of_the_collective_is_a_rounded_product(dt, op, w, factor
         assert differs > 100, (op, w, factor, differs)
 
 
+def test_fanin_with_premultiplied_contributions_hand_checked():
+    """Three ranks, bf16, AVG: every rank's element times bf16(1/3) = 0.333984375, rounded to bf16, then added in
+    binary32 in rank order and rounded to bf16 - not (a + b + c) / 3."""
+    # 7 * k = 2.337890625 -> 2.34375;  1 * k -> 0.333984375;  3 * k = 1.001953125 -> 1.0 (half an ulp of 1 is 0.00390625)
+    chunks = [torch.tensor([7.0, 1.0], dtype=torch.bfloat16), torch.tensor([1.0, 1.0], dtype=torch.bfloat16),
+              torch.tensor([3.0, 1.0], dtype=torch.bfloat16)]
+    shard = torch.zeros(2, dtype=torch.float32)
+    torch_ops.reduce_scatter_fanin(shard, chunks, None, False, premul=1 / 3)
+    # element 0: 2.34375 + 0.333984375 + 1.0 = 3.677734375 -> bf16 spacing 0.015625 at 2..4: 3.671875 | 3.6875, nearer 3.671875
+    # element 1: 3 * 0.333984375 = 1.001953125 -> 1.0
+    assert shard.tolist() == [3.671875, 1.0]
+    # the sum-then-divide form gives 11 / 3 = 3.6666 -> 3.671875 as well for element 0, but differs on, e.g., 7 alone:
+    lone = torch.zeros(1, dtype=torch.bfloat16)
+    torch_ops.reduce_scatter_fanin(lone, [torch.tensor([7.0], dtype=torch.bfloat16)], None, False, premul=1 / 3)
+    assert lone.item() == 2.34375
+    other = torch.zeros(1, dtype=torch.bfloat16)
+    torch_ops.reduce_scatter_fanin(other, [torch.tensor([7.0], dtype=torch.bfloat16)], 3.0, False)
+    assert other.item() == 2.328125
+
+
+@pytest.mark.parametrize("dt", DTYPES)
+@pytest.mark.parametrize("n_src,scalar", [(3, 1 / 3), (6, 1 / 6), (8, 1 / 8), (5, 1 / 3.0)])
+def test_fanin_with_premultiplied_contributions_vs_float64(dt, n_src, scalar):
+    """Independent restatement: term = the exact binary64 product rounded once to the data type (through binary32
+    for the 16-bit types, where it is exact); sum = binary32 additions in rank order, each the correctly rounded
+    binary64 sum of two binary32 numbers rounded once more to binary32 - which double rounding cannot change,
+    because 53 >= 2 * 24 + 2; output rounded to the data type; with one contribution it is the one-rank share."""
+    g = torch.Generator().manual_seed(23)
+    n = 1 << 14
+    chunks = [mixed_values(g, n, dt, std=1e-3, specials=False) for _ in range(n_src)]
+    k = _scalar_in(dt, scalar)
+    acc = None
+    for c in chunks:
+        term = (c.double() * k).float().to(dt).double()
+        acc = term if acc is None else (acc + term).float().double()
+    want = acc.float().to(dt)
+    for shard_dt in (torch.float32, dt):
+        got = torch.zeros(n, dtype=shard_dt)
+        torch_ops.reduce_scatter_fanin(got, [c.clone() for c in chunks], None, False, premul=scalar)
+        assert_bits_equal(got, want.to(shard_dt), "fan-in of pre-multiplied contributions vs float64")
+        base = mixed_values(g, n, shard_dt, std=1e-3, specials=False)
+        got = base.clone()
+        torch_ops.reduce_scatter_fanin(got, [c.clone() for c in chunks], None, True, premul=scalar)
+        assert_bits_equal(got, (base.double() + want.double()).float().to(shard_dt), "accumulating form")
+    one = chunks[0].clone()
+    torch_ops.reduce_scatter_one_rank_share(one, "PREMUL_SUM", n_src, scalar)
+    alone = torch.zeros(n, dtype=dt)
+    torch_ops.reduce_scatter_fanin(alone, [chunks[0].clone()], None, False, premul=scalar)
+    assert_bits_equal(alone, one, "one contribution = the one-rank share")
+
+
 def test_reduce_scatter_local_applies_the_collective_between_the_two_divides():
     """pre-divide (:139) on the whole buffer, the collective's share (:152-162) and the post-divide (:165) on the
     chunk, then the accumulation (:189): every step rounds to the reduce dtype."""

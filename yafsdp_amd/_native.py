@@ -58,6 +58,7 @@ EXPORTED_SYMBOLS = (
     "yafsdp_gather_in_post_reduce",
     "yafsdp_flat_copy_fanout",
     "yafsdp_post_reduce_fanin",
+    "yafsdp_post_reduce_fanin_premul",
     "yafsdp_binding_create",
     "yafsdp_binding_destroy",
     "yafsdp_gather_in_bound",
@@ -134,6 +135,8 @@ def _load() -> ctypes.CDLL:
     lib.yafsdp_flat_copy_fanout.argtypes = [vp, i32, i32, vp, i32, i64, vp]
     lib.yafsdp_post_reduce_fanin.restype = i32
     lib.yafsdp_post_reduce_fanin.argtypes = [vp, i32, vp, i32, i32, i64, dbl, i32, vp]
+    lib.yafsdp_post_reduce_fanin_premul.restype = i32
+    lib.yafsdp_post_reduce_fanin_premul.argtypes = [vp, i32, vp, i32, i32, i64, dbl, i32, vp]
     lib.yafsdp_binding_create.restype = i32
     lib.yafsdp_binding_create.argtypes = [vp, vp, vp, i32, ctypes.POINTER(vp)]
     lib.yafsdp_binding_destroy.restype = i32
@@ -629,26 +632,35 @@ def flat_copy_fanout(dsts: Sequence[torch.Tensor], src: torch.Tensor) -> None:
 
 
 def post_reduce_fanin(
-    shard: torch.Tensor, chunks: Sequence[torch.Tensor], post_factor: float | None, accumulate: bool
+    shard: torch.Tensor, chunks: Sequence[torch.Tensor], post_factor: float | None, accumulate: bool,
+    *, premul: float | None = None,
 ) -> None:
     """``shard (+)= div(round(sum of chunks in float32))``: the reduce-scatter of the ranks' chunks, the
-    post-divide and the accumulation into the gradient shard in one pass (at most 16 chunks)."""
+    post-divide and the accumulation into the gradient shard in one pass (at most 16 chunks).  ``premul``: the
+    scalar of a collective that scales inside the reduction (``ReduceOp.AVG``: 1 / ranks) - every chunk element is
+    multiplied by it, rounded to the chunk dtype, before the sum; there is no post-divide then."""
     _flat_arg(shard, "shard")
     if not chunks:
         raise ValueError("at least one chunk")
+    if premul is not None and post_factor is not None:
+        raise ValueError("a collective that scales inside the reduction has no post-divide")
     for c in chunks:
         _flat_arg(c, "chunk")
         if c.numel() != shard.numel() or c.dtype != chunks[0].dtype or c.device != shard.device:
             raise ValueError("chunks must match the shard's size and device and share a dtype")
     ptrs = (ctypes.c_void_p * len(chunks))(*[c.data_ptr() for c in chunks])
+    head = (shard.data_ptr(), _dt(shard), ptrs, len(chunks), _dt(chunks[0]), shard.numel())
     with _on(shard.device):
-        _check(
-            lib.yafsdp_post_reduce_fanin(
-                shard.data_ptr(), _dt(shard), ptrs, len(chunks), _dt(chunks[0]), shard.numel(), _factor(post_factor),
-                int(bool(accumulate)), _stream(shard),
-            ),
-            "yafsdp_post_reduce_fanin",
-        )
+        if premul is not None:
+            _check(
+                lib.yafsdp_post_reduce_fanin_premul(*head, float(premul), int(bool(accumulate)), _stream(shard)),
+                "yafsdp_post_reduce_fanin_premul",
+            )
+        else:
+            _check(
+                lib.yafsdp_post_reduce_fanin(*head, _factor(post_factor), int(bool(accumulate)), _stream(shard)),
+                "yafsdp_post_reduce_fanin",
+            )
 
 
 class TensorBinding:

@@ -339,7 +339,7 @@ int abandon_large(yafsdp_table* t, int slot, hipStream_t stream, hipError_t laun
 
 extern "C" {
 
-int yafsdp_version(void) { return 1006; }
+int yafsdp_version(void) { return 1007; }
 
 const char* yafsdp_error_string(int code) {
   switch (code) {
@@ -607,9 +607,9 @@ int yafsdp_flat_copy_fanout(void* const* dsts, int n_dst, int dst_dtype, const v
   return int(launch_fanout(src_dtype, dst_dtype, ptrs, src, n, grid, static_cast<hipStream_t>(stream)));
 }
 
-int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* chunks, int n_src, int chunk_dtype,
-                             int64_t n, double post_factor, int accumulate, void* stream) {
-  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+namespace {
+int fanin_launch(void* shard, int shard_dtype, const void* const* chunks, int n_src, int chunk_dtype, int64_t n,
+                 int scale, float k, int accumulate, void* stream) {
   if (n < 0 || n_src < 1 || n_src > kFanMax || chunks == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
   if (n == 0) return YAFSDP_OK;
   if (shard == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
@@ -617,17 +617,34 @@ int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* ch
   FanPtrs ptrs;
   std::memset(&ptrs, 0, sizeof(ptrs));
   ptrs.n = n_src;
-  for (int k = 0; k < n_src; k++) {
-    if (chunks[k] == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
-    if (!aligned_to(chunks[k], 16)) return YAFSDP_ERR_MISALIGNED;
-    ptrs.p[k] = const_cast<void*>(chunks[k]);
+  for (int c = 0; c < n_src; c++) {
+    if (chunks[c] == nullptr) return YAFSDP_ERR_INVALID_ARGUMENT;
+    if (!aligned_to(chunks[c], 16)) return YAFSDP_ERR_MISALIGNED;
+    ptrs.p[c] = const_cast<void*>(chunks[c]);
   }
-  int scale;
-  float k;
-  scale_plan(post_factor, &scale, &k);
   const int grid = opt_grid(n >> 2, kFanInBlock, kFanInUnroll, nullptr);
   return int(launch_fanin(chunk_dtype, shard_dtype, scale, accumulate != 0, shard, ptrs, n, k, grid,
                           static_cast<hipStream_t>(stream)));
+}
+}  // namespace
+
+int yafsdp_post_reduce_fanin(void* shard, int shard_dtype, const void* const* chunks, int n_src, int chunk_dtype,
+                             int64_t n, double post_factor, int accumulate, void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  int scale;
+  float k;
+  scale_plan(post_factor, &scale, &k);
+  return fanin_launch(shard, shard_dtype, chunks, n_src, chunk_dtype, n, scale, k, accumulate, stream);
+}
+
+int yafsdp_post_reduce_fanin_premul(void* shard, int shard_dtype, const void* const* chunks, int n_src,
+                                    int chunk_dtype, int64_t n, double scalar, int accumulate, void* stream) {
+  if (!valid_dtype(shard_dtype) || !valid_dtype(chunk_dtype)) return YAFSDP_ERR_UNSUPPORTED_DTYPE;
+  int scale;
+  float k;
+  if (!premul_plan(scalar, chunk_dtype, &scale, &k)) return YAFSDP_ERR_INVALID_ARGUMENT;
+  if (scale == SCALE_MUL) scale = SCALE_PREMUL;  // a scalar that rounds to 1 leaves the plain sum
+  return fanin_launch(shard, shard_dtype, chunks, n_src, chunk_dtype, n, scale, k, accumulate, stream);
 }
 
 int yafsdp_flat_fill(void* dst, int dtype, int64_t n, double value, void* stream) {

@@ -17,7 +17,8 @@ enum : int { DT_F32 = 0, DT_BF16 = 1, DT_F16 = 2 };
 // how a divide factor is applied: not at all, as an exact multiply by the
 // reciprocal (power-of-two factors only: same bits as a division), or as a
 // correctly rounded binary32 division.
-enum : int { SCALE_NONE = 0, SCALE_MUL = 1, SCALE_DIV = 2 };
+// SCALE_PREMUL exists for the fan-in only: every contribution is multiplied by k and rounded BEFORE the sum
+enum : int { SCALE_NONE = 0, SCALE_MUL = 1, SCALE_DIV = 2, SCALE_PREMUL = 3 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));

@@ -38,6 +38,8 @@ hipError_t fanin_by_op(int scale, bool acc, void* shard, const FanPtrs& chunks, 
     case 3: return fanin_go<S, D, SCALE_MUL, true>(shard, chunks, n, k, grid, stream);
     case 4: return fanin_go<S, D, SCALE_DIV, false>(shard, chunks, n, k, grid, stream);
     case 5: return fanin_go<S, D, SCALE_DIV, true>(shard, chunks, n, k, grid, stream);
+    case 6: return fanin_go<S, D, SCALE_PREMUL, false>(shard, chunks, n, k, grid, stream);
+    case 7: return fanin_go<S, D, SCALE_PREMUL, true>(shard, chunks, n, k, grid, stream);
   }
   return hipErrorInvalidValue;
 }

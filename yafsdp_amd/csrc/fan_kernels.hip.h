@@ -70,9 +70,21 @@ fanout_kernel(FanPtrs dsts, const void* src, int64_t n) {
 // reference, ya_fsdp/_collectives.py:157-161), the sum is rounded to the chunk
 // dtype as the collective's output tensor is, then post-divide (:165) and
 // copy_ / add_ into the gradient shard (:185 / :189).
+//
+// SCALE_PREMUL is the collective that scales inside the reduction (ReduceOp.AVG, or the pre-multiplied sum of
+// _make_nccl_premul_sum, :243-249): the collective library multiplies every rank's element by the scalar, both in
+// the chunk dtype, i.e. rounds each product to that dtype, and adds the products; there is no post-divide then.
 template <class S, class D, int SCALE, bool ACC>
 __device__ __forceinline__ float fanin_finish(float sum, float d_old, float k) {
-  return post_elem<S, D, SCALE, ACC>(round_to<S>(sum), d_old, k);
+  constexpr int kAfterSum = SCALE == SCALE_PREMUL ? SCALE_NONE : SCALE;
+  return post_elem<S, D, kAfterSum, ACC>(round_to<S>(sum), d_old, k);
+}
+
+// one rank's element as it enters the sum
+template <class S, int SCALE>
+__device__ __forceinline__ float fanin_term(float x, float k) {
+  if constexpr (SCALE == SCALE_PREMUL) return round_to<S>(apply_scale<SCALE_MUL>(x, k));
+  else return x;
 }
 
 template <class S, class D, int SCALE, bool ACC, int BLOCK, int U, bool NTL, bool NTS>
@@ -100,12 +112,14 @@ fanin_kernel(void* shard, FanPtrs chunks, int64_t n, float k) {
       float sum[4], fo[4] = {0.f, 0.f, 0.f, 0.f}, fy[4];
       unpack_quad<S>(x[0], sum);
 #pragma unroll
+      for (int e = 0; e < 4; e++) sum[e] = fanin_term<S, SCALE>(sum[e], k);
+#pragma unroll
       for (int c = 1; c < kFanMax; c++) {
         if (c < chunks.n) {
           float f[4];
           unpack_quad<S>(x[c], f);
 #pragma unroll
-          for (int e = 0; e < 4; e++) sum[e] = __fadd_rn(sum[e], f[e]);
+          for (int e = 0; e < 4; e++) sum[e] = __fadd_rn(sum[e], fanin_term<S, SCALE>(f[e], k));
         }
       }
       if constexpr (ACC) unpack_quad<D>(old, fo);
@@ -117,8 +131,9 @@ fanin_kernel(void* shard, FanPtrs chunks, int64_t n, float k) {
   if (blockIdx.x == 0) {
     const int64_t i = (n_quads << 2) + threadIdx.x;
     if (i < n) {
-      float sum = to_f32<S>(reinterpret_cast<const s_t*>(chunks.p[0])[i]);
-      for (int c = 1; c < chunks.n; c++) sum = __fadd_rn(sum, to_f32<S>(reinterpret_cast<const s_t*>(chunks.p[c])[i]));
+      float sum = fanin_term<S, SCALE>(to_f32<S>(reinterpret_cast<const s_t*>(chunks.p[0])[i]), k);
+      for (int c = 1; c < chunks.n; c++)
+        sum = __fadd_rn(sum, fanin_term<S, SCALE>(to_f32<S>(reinterpret_cast<const s_t*>(chunks.p[c])[i]), k));
       d_t* d = reinterpret_cast<d_t*>(shard) + i;
       float d_old = 0.f;
       if constexpr (ACC) d_old = to_f32<D>(*d);
