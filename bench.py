@@ -616,6 +616,7 @@ def run_full_model(args, as_record: bool = False):
             "ms_copies_alone": out["ms_copies_alone"], "ms_gemms_alone": out["ms_gemms_alone"],
             "copy_GBps_alone": out["copy_GBps_alone"], "groups": n, "logical_world_size": w, "passes_timed": reps,
             "copy_GBps_alone_reduce_copy_in_on_side_stream": out["copy_GBps_alone_reduce_copy_in_on_side_stream"],
+            "copy_GBps_alone_replayed_from_one_graph": out["copy_GBps_alone_replayed_from_one_graph"],
             "copy_GBps_by_kind": out["copy_GBps_by_kind"], "ms_copies_by_kind_alone": out["ms_copies_by_kind_alone"],
             "gemm_shapes": {k: {a_: b_ for a_, b_ in v.items()
                                 if a_ in ("ms_gemms_alone", "ms_overlapped", "overlap_efficiency",
