@@ -16,6 +16,7 @@
 /* oracle/bufpath_ref.c */
 void ref_flat_copy(void* dst, int dd, const void* src, int sd, int64_t n);
 void ref_post_reduce(void* shard, int sdt, const void* chunk, int cdt, int64_t n, double post, int accumulate);
+void ref_flat_premul(void* buf, int dt, int64_t n, double scalar);
 void ref_gather_in(int n_tensors, const void* const* tensors, const int64_t* offsets, const uint8_t* mode, int tdt,
                    void* flat, int fdt, int64_t t_pad, double pre, int zero_pad);
 void ref_scatter_out(int n_tensors, void* const* tensors, const int64_t* offsets, int tdt, const void* flat, int fdt);
@@ -211,6 +212,65 @@ int main(void) {
     free(h_twice); free(h_part);
     HIP(hipFree(d_shard2)); HIP(hipFree(d_part));
     memcpy(h_shard, h_shard_want, (size_t)s * 4);
+  }
+
+  /* ---- this rank's share of a reduce-scatter that scales inside the reduction (ReduceOp.AVG over 3 ranks): the
+   * bf16 chunk times bf16(1 / 3), rounded to bf16, accumulated into the fp32 shard - not a division by 3.  The
+   * completion event is recorded by the kernel's own dispatch instead of by a marker behind it. */
+  {
+    uint16_t* h_chunk = malloc((size_t)s * 2);
+    float* h_share_want = malloc((size_t)s * 4);
+    float* h_by_division = malloc((size_t)s * 4);
+    memcpy(h_chunk, h_grads[0], (size_t)s * 2);
+    memcpy(h_share_want, h_shard_want, (size_t)s * 4);
+    memcpy(h_by_division, h_shard_want, (size_t)s * 4);
+    ref_post_reduce(h_by_division, YAFSDP_F32, h_chunk, YAFSDP_BF16, s, 3.0, 1);
+    ref_flat_premul(h_chunk, YAFSDP_BF16, s, 1.0 / 3.0);
+    ref_post_reduce(h_share_want, YAFSDP_F32, h_chunk, YAFSDP_BF16, s, 0.0, 1);
+    float* d_share;
+    hipEvent_t done;
+    HIP(hipMalloc((void**)&d_share, (size_t)s * 4));
+    HIP(hipMemcpy(d_share, h_shard_want, (size_t)s * 4, hipMemcpyHostToDevice));
+    HIP(hipEventCreateWithFlags(&done, hipEventDisableTiming));
+    YA(yafsdp_complete_next_launch(done));
+    YA(yafsdp_post_reduce_premul(d_share, YAFSDP_F32, d_grads[0], YAFSDP_BF16, s, 1.0 / 3.0, 1, stream));
+    if (yafsdp_complete_next_launch_pending()) { printf("MISMATCH the launch left the completion event armed\n"); return 1; }
+    HIP(hipEventSynchronize(done));  /* the kernel has completed: no stream synchronisation needed */
+    HIP(hipMemcpy(h_shard, d_share, (size_t)s * 4, hipMemcpyDeviceToHost));
+    if (!same("post_reduce_premul bf16 * bf16(1/3) += f32, event from the dispatch", h_shard, h_share_want, (size_t)s * 4))
+      return 1;
+    int64_t differ = 0;
+    for (int64_t i = 0; i < s; i++) differ += memcmp(&h_share_want[i], &h_by_division[i], 4) != 0;
+    if (differ == 0) { printf("MISMATCH the scaled share equals a division by 3 everywhere\n"); return 1; }
+    printf("ok the share differs from a division by 3 on %lld of %lld elements\n", (long long)differ, (long long)s);
+    HIP(hipEventDestroy(done));
+    HIP(hipFree(d_share));
+    free(h_chunk); free(h_share_want); free(h_by_division);
+    memcpy(h_shard, h_shard_want, (size_t)s * 4);
+  }
+
+  /* ---- store policy of one table: the write-through tail is an option per table that follows the process-wide
+   * default until it is set; it
+   * changes no result */
+  {
+    int v = -2;
+    YA(yafsdp_table_get_option(table, YAFSDP_OPT_GATHER_TAIL_MB, &v));
+    if (v != -1) { printf("MISMATCH a new table's option reads %d, not -1 (follow the process)\n", v); return 1; }
+    YA(yafsdp_table_set_option(table, YAFSDP_OPT_GATHER_TAIL_MB, 1));
+    YA(yafsdp_table_get_option(table, YAFSDP_OPT_GATHER_TAIL_MB, &v));
+    if (v != 1) { printf("MISMATCH table option reads %d after setting 1\n", v); return 1; }
+    float* h_again = malloc((size_t)padded * 4);
+    for (int64_t i = 0; i < padded; i++) h_again[i] = next_float(1e-3f);
+    memcpy(h_want, h_again, (size_t)padded * 4);
+    ref_gather_in(P, (const void* const*)h_grads, offsets, modes, YAFSDP_BF16, h_want, YAFSDP_F32, padded, 8.0, 1);
+    HIP(hipMemcpy(d_flat, h_again, (size_t)padded * 4, hipMemcpyHostToDevice));
+    YA(yafsdp_gather_in(table, (const void* const*)d_grads, modes, YAFSDP_BF16, d_flat, YAFSDP_F32, 8.0, 1, stream));
+    HIP(hipStreamSynchronize(stream));
+    HIP(hipMemcpy(h_again, d_flat, (size_t)padded * 4, hipMemcpyDeviceToHost));
+    if (!same("gather_in with a 1-MB write-through tail on this table", h_again, h_want, (size_t)padded * 4)) return 1;
+    YA(yafsdp_table_set_option(table, YAFSDP_OPT_GATHER_TAIL_MB, -1));
+    printf("ok table option\n");
+    free(h_again);
   }
 
   /* ---- gradient norm, clip coefficient, fused AdamW with bf16 copy-in */
