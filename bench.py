@@ -820,6 +820,8 @@ def run_trainer(args) -> int:
     torch.cuda.set_device(dev)
     dim, ffn, heads, kv_heads, layers, seq = 4096, 14336, 32, 8, args.layers, args.seq_len
     hd = dim // heads
+    world = max(1, args.logical_world_size)
+    mesh = None if world == 1 else (world, world // 2)
 
     class RMSNorm(nn.Module):
         def __init__(self):
@@ -912,26 +914,29 @@ def run_trainer(args) -> int:
 
     results["compute_only_bf16"] = timed(floor_step, reps, warm, "compute_only_bf16")
 
-    # ---- hand-written mixed precision with torch ops
-    masters = [p.detach().clone().requires_grad_(True) for p in model0.parameters()]
-    lowp_params = list(lowp.parameters())
-    for m in masters:
-        m.grad = torch.zeros_like(m)
-    opt_t = torch.optim.AdamW(masters, fused=True, **hyper)
+    # ---- hand-written mixed precision with torch ops (the whole model's masters and optimizer state on this GPU:
+    # comparable with the wrapped loops at world size 1 only)
+    if world == 1:
+        masters = [p.detach().clone().requires_grad_(True) for p in model0.parameters()]
+        lowp_params = list(lowp.parameters())
+        for m in masters:
+            m.grad = torch.zeros_like(m)
+        opt_t = torch.optim.AdamW(masters, fused=True, **hyper)
 
-    def torch_step():
-        with torch.no_grad():
-            torch._foreach_copy_(lowp_params, masters)          # the cast the copy-in does
-        loss_of(lowp(x)).backward()
-        with torch.no_grad():
-            torch._foreach_copy_([m.grad for m in masters], [p.grad for p in lowp_params])  # bf16 -> fp32 gradients
-        for p in lowp_params:
-            p.grad = None
-        torch.nn.utils.clip_grad_norm_(masters, 1.0, foreach=True)
-        opt_t.step()
+        def torch_step():
+            with torch.no_grad():
+                torch._foreach_copy_(lowp_params, masters)          # the cast the copy-in does
+            loss_of(lowp(x)).backward()
+            with torch.no_grad():
+                torch._foreach_copy_([m.grad for m in masters], [p.grad for p in lowp_params])  # bf16 -> fp32 gradients
+            for p in lowp_params:
+                p.grad = None
+            torch.nn.utils.clip_grad_norm_(masters, 1.0, foreach=True)
+            opt_t.step()
 
-    results["torch_ops_by_hand"] = timed(torch_step, reps, warm, "torch_ops_by_hand")
-    del masters, opt_t, lowp, lowp_params
+        results["torch_ops_by_hand"] = timed(torch_step, reps, warm, "torch_ops_by_hand")
+        del masters, opt_t, lowp_params
+    del lowp
     torch.cuda.empty_cache()
 
     # ---- fully_shard, two optimizers
@@ -940,8 +945,18 @@ def run_trainer(args) -> int:
     def wrapped():
         m = copy.deepcopy(model0)
         for layer in m.layers:
-            fully_shard(layer, mp_policy=mp)
-        return fully_shard(m, mp_policy=mp)
+            fully_shard(layer, mesh=mesh, mp_policy=mp)
+        return fully_shard(m, mesh=mesh, mp_policy=mp)
+
+    def seed_peer_slots(m):
+        """At a logical world size above one nothing delivers the other ranks' slots of the gathered buffers; they
+        get weight-like values once (every later unshard rewrites this rank's slot only), so that the GEMMs run on
+        ordinary data."""
+        for mod in m._fsdp_modules(True):
+            group = mod._get_fsdp_state()._fsdp_param_group
+            if group is not None:
+                for gathered in group._all_gather_output.values():
+                    gathered.normal_(0.0, 0.02)
 
     for name in ("fully_shard_torch_adamw", "fully_shard_flat_adamw"):
         model = wrapped()
@@ -965,6 +980,9 @@ def run_trainer(args) -> int:
             # unless they are cleared, as with torch.optim
             opt.zero_grad(set_to_none=True)
 
+        if world > 1:
+            fs_step()  # lazy initialisation assigns the buffers
+            seed_peer_slots(model)
         results[name] = timed(fs_step, reps, warm, name)
         del model, params, opt
         torch.cuda.empty_cache()
@@ -973,11 +991,15 @@ def run_trainer(args) -> int:
         log(f"  {k_:28s} {v_:8.3f} ms / iteration (median; {spread[k_]})  ({seq / v_ * 1e3:9.0f} tokens/s)")
     best = results["fully_shard_flat_adamw"]
     out = {
-        "metric": f"training iteration at world size 1: {layers} Llama-3-8B decoder layers through fully_shard + flat AdamW",
+        "metric": (f"training iteration at world size 1: {layers} Llama-3-8B decoder layers through fully_shard + flat AdamW"
+                   if world == 1 else
+                   f"one rank's share of a training iteration at logical world size {world} (no exchanges between "
+                   f"ranks): {layers} Llama-3-8B decoder layers through fully_shard + flat AdamW"),
         "value": round(seq / best * 1e3, 1), "unit": "tokens/s", "n_gpus": 1, "steps": reps, "warmup": warm,
         "ms_per_step": round(best, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "fully-shard-trainer-w1", "layers": layers, "parameters": n_params, "tokens_per_step": seq,
+        "config": {"workload": "fully-shard-trainer-w1", "logical_world_size": world, "layers": layers,
+                   "parameters": n_params, "tokens_per_step": seq,
                    "master_dtype": "float32", "optimizer": "AdamW + gradient clipping"},
         "ms_per_iteration": {k_: round(v_, 4) for k_, v_ in results.items()},
         "ms_per_iteration_mean_min_max": spread,
@@ -1620,6 +1642,9 @@ def main() -> int:
                          "and the GEMMs on a stream limited to the others")
     ap.add_argument("--layers", type=int, default=4, help="fully-shard-trainer-w1 only: decoder layers")
     ap.add_argument("--seq-len", type=int, default=4096, help="fully-shard-trainer-w1 only: tokens per iteration")
+    ap.add_argument("--logical-world-size", type=int, default=1, metavar="W",
+                    help="fully-shard-trainer-w1 only: wrap with mesh=(W, W // 2), i.e. time one rank's share of a "
+                         "W-rank run (its shard of every group; the exchanges between ranks are not part of it)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="N",
                     help="also launch N plain bf16->bf16 flat copies of T_pad elements (a kernel of known traffic, "
                          "used to scale rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings); outside the timed region")
